@@ -1,0 +1,226 @@
+"""Op-library subset of the CPU oracle -- TEST INFRASTRUCTURE ONLY.
+
+Restates, on top of oracle/tile_oracle.py, the contractions that the reference
+op library emits for the operations on the hot path (plaidml/op/lib/ops.cc):
+
+  convolution   :879-1467 (NXC input, XCK filter; strides, dilations, autopad,
+                 explicit padding, group layouts NONE and IN_C with DEPTHWISE
+                 autogrouping), padding rule :347-382
+  pool          :2562-2703 (MAX / MIN / SUM / AVG, NXC)
+  dot           :1512-1561
+  mean          :1970-2003, sum / max via the same AggregationAxes :71-127
+  relu          :2705-2728 (plain form only)
+  softmax       :3049-3098 (last-axis form)
+  argmax        :505-521
+
+Nothing in the shipped package imports this module.
+"""
+import builtins
+
+from . import tile_oracle as E
+
+SAME_UPPER, SAME_LOWER, VALID, EXPLICIT = 'same_upper', 'same_lower', 'valid', 'explicit'
+
+
+def compute_padding_and_output_size(input_size, filter_size, stride, autopad, pad_lo=0, pad_hi=0,
+                                    dilation=1, data_dilation=1, use_ceil=False):
+    """plaidml/op/lib/ops.cc:347-382.  Integer division is C division of non-negative values."""
+    i_eff = data_dilation * (input_size - 1) + 1
+    f_eff = dilation * (filter_size - 1) + 1
+    ceil_term = stride - 1 if use_ceil else 0
+    if autopad == EXPLICIT:
+        return pad_lo, (i_eff + pad_lo + pad_hi - f_eff + stride + ceil_term) // stride
+    if autopad == VALID:
+        return 0, (i_eff - f_eff + stride + ceil_term) // stride
+    if autopad in (SAME_LOWER, SAME_UPPER):
+        out = (i_eff + stride - 1) // stride
+        lower = 1 if autopad == SAME_LOWER else 0
+        pad = (builtins.max(0, (out - 1) * stride + f_eff - i_eff) + lower) // 2
+        return pad, out
+    raise ValueError('Unexpected autopadding mode: %s' % autopad)
+
+
+def convolution(I, F, strides=None, dilations=None, data_dilations=None, autopad=SAME_UPPER,
+                manual_padding=None, depthwise=False, name='conv'):
+    """NXC input, XCK filter.  depthwise=True is GroupLayout IN_C + AutoGroupMode DEPTHWISE."""
+    rank = len(I.shape) - 2
+    strides = list(strides or [1] * rank)
+    dilations = list(dilations or [1] * rank)
+    data_dilations = list(data_dilations or [1] * rank)
+    manual_padding = list(manual_padding or [])
+    if len(manual_padding) == rank:
+        manual_padding = manual_padding + manual_padding  # symmetric shorthand
+    while len(manual_padding) < 2 * rank:
+        manual_padding.append(0)
+    if manual_padding and any(manual_padding) and autopad != EXPLICIT:
+        raise ValueError('Autopadding and manual padding both requested for single conv operation')
+    N, CI = I.shape[0], I.shape[-1]
+    xs = I.shape[1:-1]
+    ks = F.shape[:rank]
+    F_CI, F_CO = F.shape[rank], F.shape[rank + 1]
+    if F_CI != CI:
+        raise ValueError('bind dims mismatch: filter input channels %d != %d' % (F_CI, CI))
+    G = CI if depthwise else 1
+    CO = F_CO * G if depthwise else F_CO
+    n, co, ci, g = E.TensorIndexes(4)
+    x = E.TensorIndexes(rank)
+    k = E.TensorIndexes(rank)
+    pads, outs = [], []
+    for i in range(rank):
+        p, o = compute_padding_and_output_size(xs[i], ks[i], strides[i], autopad, manual_padding[i],
+                                               manual_padding[i + rank], dilations[i], data_dilations[i])
+        pads.append(p)
+        outs.append(o)
+    sp = [(strides[i] * x[i] + dilations[i] * k[i] - pads[i]) // data_dilations[i] for i in range(rank)]
+    cons = []
+    if depthwise:
+        i_c = (CI // G) * g + ci
+        f_ci, f_co = (CI // G) * g + ci, co
+        o_c = (CO // G) * g + co
+        cons.append(ci < CI // G)
+    else:
+        i_c, f_ci, f_co, o_c = ci, ci, co, co
+    c = E.Contraction(name).outShape([N] + outs + [CO]).outAccess([n] + x + [o_c])
+    c.sum(I[[n] + sp + [i_c]] * F[k + [f_ci, f_co]]).add_constraints(cons)
+    return c.build()
+
+
+def pool(I, mode, pool_size, strides, autopad=VALID, manual_padding=None, include_padding_in_avg=False,
+         use_ceil=False, name='pool'):
+    rank = len(pool_size)
+    manual_padding = list(manual_padding or [])
+    while len(manual_padding) < 2 * rank:
+        manual_padding.append(0)
+    N, C = I.shape[0], I.shape[-1]
+    X = I.shape[1:-1]
+    n, c = E.TensorIndexes(2)
+    x = E.TensorIndexes(rank)
+    k = E.TensorIndexes(rank)
+    o_dims, i_idxs, cons = [N], [n], []
+    for i in range(rank):
+        p, o = compute_padding_and_output_size(X[i], pool_size[i], strides[i], autopad, manual_padding[i],
+                                               manual_padding[rank + i], 1, 1, use_ceil)
+        o_dims.append(o)
+        i_idxs.append(strides[i] * x[i] + k[i] - p)
+        cons.append(k[i] < pool_size[i])
+    o_dims.append(C)
+    i_idxs.append(c)
+    o_idxs = [n] + x + [c]
+
+    def mk():
+        return E.Contraction(name).outShape(o_dims).outAccess(o_idxs).add_constraints(cons)
+
+    if mode == 'max':
+        return mk().max(I[i_idxs]).build()
+    if mode == 'min':
+        return mk().min(I[i_idxs]).build()
+    if mode == 'sum':
+        return mk().sum(I[i_idxs]).build()
+    if mode == 'avg':
+        O = mk().sum(I[i_idxs]).build()
+        if include_padding_in_avg:
+            total = 1
+            for s in pool_size:
+                total *= s
+            return O / total
+        one = E.cast(E.Constant(1), I.dt)
+        ones = E.Contraction(name).outShape(I.shape).outAccess(o_idxs).assign(one[()]).build()
+        count = mk().sum(ones[i_idxs]).build()
+        return O / count
+    raise ValueError('Unrecognized pool_mode in pool op')
+
+
+def dot(X, Y, name='dot'):
+    if X.dt != Y.dt:
+        raise ValueError('Invalid dtype in dot')
+    if len(X.shape) == 1 and len(Y.shape) == 1:
+        i, = E.TensorIndexes(1)
+        return E.Contraction(name).outShape(X.shape[0]).outAccess(i).sum(X[i] * Y[i]).build()
+    xi = E.TensorIndexes(len(X.shape))
+    yi = E.TensorIndexes(len(Y.shape))
+    z, = E.TensorIndexes(1)
+    xi[-1] = z
+    yi[-2] = z
+    o_dims = list(X.shape[:-1]) + list(Y.shape[:-2]) + [Y.shape[-1]]
+    o_idxs = xi[:-1] + yi[:-2] + [yi[-1]]
+    return E.Contraction(name).outShape(o_dims).outAccess(o_idxs).sum(X[xi] * Y[yi]).build()
+
+
+class _Axes:
+    """AggregationAxes, plaidml/op/lib/ops.cc:71-127."""
+
+    def __init__(self, shape, axes, keepdims):
+        nd = len(shape)
+        if axes is None:
+            axes = list(range(nd))
+        if isinstance(axes, int):
+            axes = [axes]
+        self.axes = sorted(set(a + nd if a < 0 else a for a in axes))
+        self.src_idxs = E.TensorIndexes(nd)
+        self.src_dims = list(shape)
+        self.reduce_idxs = [self.src_idxs[a] for a in self.axes]
+        self.reduce_dims = [shape[a] for a in self.axes]
+        if keepdims:
+            self.dst_idxs = list(self.src_idxs)
+            self.dst_dims = list(shape)
+            for a in self.axes:
+                self.dst_idxs[a] = E.TensorIndex()
+                self.dst_dims[a] = 1
+        else:
+            self.dst_idxs = [self.src_idxs[i] for i in range(nd) if i not in self.axes]
+            self.dst_dims = [shape[i] for i in range(nd) if i not in self.axes]
+
+
+def _reduce(I, axes, keepdims, agg, name):
+    a = _Axes(I.shape, axes, keepdims)
+    c = E.Contraction(name).outShape(a.dst_dims).outAccess(a.dst_idxs)
+    getattr(c, agg)(I[a.src_idxs])
+    return c.build(), a
+
+
+def sum(I, axes=None, keepdims=False):  # noqa: A001
+    return _reduce(I, axes, keepdims, 'sum', 'sum')[0]
+
+
+def max(I, axes=None, keepdims=False):  # noqa: A001
+    return _reduce(I, axes, keepdims, 'max', 'max')[0]
+
+
+def mean(I, axes=None, keepdims=False):
+    if len(I.shape) == 0 or (isinstance(axes, (list, tuple)) and len(axes) == 0):
+        return I
+    so, a = _reduce(I, axes, keepdims, 'sum', 'mean')
+    denom = 1
+    for ax in a.axes:
+        denom *= I.shape[ax]
+    return so / denom
+
+
+def relu(I):
+    return E.relu(I)
+
+
+def softmax(I, axis=-1, name='softmax'):
+    nd = len(I.shape)
+    if axis < 0:
+        axis += nd
+    if axis != nd - 1:
+        raise NotImplementedError('softmax over a non-trailing axis')
+    idxs = E.TensorIndexes(nd)
+    r_dims = list(I.shape)
+    r_idxs = list(idxs)
+    r_dims[axis] = 1
+    r_idxs[axis] = 0
+    M = E.Contraction(name).outShape(r_dims).outAccess(r_idxs).max(I[idxs]).build()
+    Ex = E.exp(I - M)
+    Nn = E.Contraction(name).outShape(r_dims).outAccess(r_idxs).sum(Ex[idxs]).build()
+    return Ex / Nn
+
+
+def argmax(I, axis=-1):
+    a = _Axes(I.shape, axis, False)
+    M = E.Contraction('argmax').outShape(a.dst_dims).outAccess(a.dst_idxs).max(I[a.src_idxs]).build()
+    IX = E.index(a.reduce_dims, 0)
+    AM = E.Contraction('argmax').outShape(a.dst_dims).outAccess(a.dst_idxs).max(
+        E.cond(I[a.src_idxs], M[a.dst_idxs], IX[a.reduce_idxs])).build()
+    return E.cast(AM, E.DType.UINT32)
