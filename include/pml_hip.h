@@ -1,0 +1,347 @@
+/*
+ * pml_hip.h -- C ABI of the gfx950 kernel library that sits beneath the `hip`
+ * runtime device, in the position the libxsmm shims occupy beneath `llvm_cpu`
+ * in the reference (pmlc/rt/xsmm.cc:17-890).
+ *
+ * Shape of the interface follows the reference's dispatch-once / invoke-many
+ * convention (pmlc/rt/xsmm.cc:17-56: `*_dispatch_*` returns an int64 handle at
+ * compile time, `*_invoke_*` takes the handle plus raw pointers at run time).
+ * Differences that the GPU forces: one invoke covers a whole contraction, not
+ * one cache tile; pointers are device pointers; invokes are stream-ordered.
+ *
+ * Every function returns 0 on success and a non-zero status on failure unless
+ * stated otherwise; pml_hip_last_error() gives the message for the calling
+ * thread.  Plain C types only.
+ */
+#ifndef PML_HIP_H_
+#define PML_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types.  Values equal plaidml_datatype (plaidml/core/ffi.h:139-156);
+ * bfloat16 is appended so that no existing value changes. */
+enum {
+  PML_HIP_BOOL = 4,
+  PML_HIP_I8 = 5,
+  PML_HIP_U8 = 6,
+  PML_HIP_I16 = 7,
+  PML_HIP_U16 = 8,
+  PML_HIP_I32 = 9,
+  PML_HIP_U32 = 10,
+  PML_HIP_I64 = 11,
+  PML_HIP_U64 = 12,
+  PML_HIP_F16 = 13,
+  PML_HIP_F32 = 14,
+  PML_HIP_F64 = 15,
+  PML_HIP_BF16 = 16
+};
+
+/* Aggregations and combinations of a contraction (pmlc/util/enums.td:9-33). */
+enum { PML_HIP_AGG_ASSIGN = 0, PML_HIP_AGG_ADD = 1, PML_HIP_AGG_MAX = 2, PML_HIP_AGG_MIN = 3, PML_HIP_AGG_MUL = 4 };
+enum { PML_HIP_COMBO_NONE = 0, PML_HIP_COMBO_ADD = 1, PML_HIP_COMBO_COND = 2, PML_HIP_COMBO_EQ = 3, PML_HIP_COMBO_MUL = 4 };
+
+typedef void* pml_hip_stream; /* a hipStream_t; NULL is the default stream */
+typedef void* pml_hip_event;  /* a hipEvent_t */
+
+/* ---- library, device, memory, streams ------------------------------------
+ * Counterpart of the process-level set-up the reference does in
+ * pmlc::rt::registerXsmm (pmlc/rt/xsmm.cc:863-890, libxsmm_init) and of the host
+ * buffers of pmlc/util/buffer.h:15-70, which here live in HBM. */
+int pml_hip_init(int device_ordinal);
+int pml_hip_device_count(void); /* number of devices, 0 if none; never fails */
+int pml_hip_device_name(char* buf, size_t buf_len);
+const char* pml_hip_last_error(void);
+
+int pml_hip_malloc(void** dptr, size_t nbytes);
+int pml_hip_free(void* dptr);
+int pml_hip_host_alloc(void** hptr, size_t nbytes); /* pinned host memory */
+int pml_hip_host_free(void* hptr);
+int pml_hip_memcpy_h2d(void* dst, const void* src, size_t nbytes, pml_hip_stream s);
+int pml_hip_memcpy_d2h(void* dst, const void* src, size_t nbytes, pml_hip_stream s);
+int pml_hip_memcpy_d2d(void* dst, const void* src, size_t nbytes, pml_hip_stream s);
+/* Fills with a 32-bit pattern using a kernel (safe to capture into a graph). */
+int pml_hip_fill_u32(void* dptr, uint32_t pattern, size_t n_words, pml_hip_stream s);
+
+int pml_hip_stream_create(pml_hip_stream* s);
+int pml_hip_stream_destroy(pml_hip_stream s);
+int pml_hip_stream_sync(pml_hip_stream s);
+int pml_hip_event_create(pml_hip_event* e);
+int pml_hip_event_destroy(pml_hip_event e);
+int pml_hip_event_record(pml_hip_event e, pml_hip_stream s);
+int pml_hip_event_sync(pml_hip_event e);
+int pml_hip_event_elapsed_ms(pml_hip_event start, pml_hip_event stop, float* ms);
+
+/* ---- fused elementwise tail ------------------------------------------------
+ * A chain of scalar operations applied to one running value per output
+ * element.  It plays the role of the bias / ReLU variants of the reference
+ * GEMM shims (plaidml_rt_xsmm_gemm_bias / _relu / _relu_beta1,
+ * pmlc/rt/xsmm.cc:58-233) and of the TPP unary / binary kernels
+ * (plaidml_rt_xsmm_unary_* :344-385, plaidml_rt_xsmm_binary_* :387-455), with the
+ * scalar semantics of pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:1227-1385.
+ * After each step the value is rounded to that step's result type. */
+enum {
+  PML_HIP_EPI_ADD = 1,  /* v = v + x */
+  PML_HIP_EPI_SUB,      /* v = v - x */
+  PML_HIP_EPI_RSUB,     /* v = x - v */
+  PML_HIP_EPI_MUL,      /* v = v * x */
+  PML_HIP_EPI_DIV,      /* v = v / x */
+  PML_HIP_EPI_RDIV,     /* v = x / v */
+  PML_HIP_EPI_MAX,      /* v = (v < x) ? x : v */
+  PML_HIP_EPI_MIN,      /* v = (v < x) ? v : x */
+  PML_HIP_EPI_RELU,     /* v = (v < 0) ? 0 : v */
+  PML_HIP_EPI_NEG,
+  PML_HIP_EPI_EXP,
+  PML_HIP_EPI_LOG,
+  PML_HIP_EPI_SQRT,
+  PML_HIP_EPI_TANH,
+  PML_HIP_EPI_FLOOR,
+  PML_HIP_EPI_CEIL,
+  PML_HIP_EPI_ROUND,    /* C roundf: half away from zero */
+  PML_HIP_EPI_CAST,     /* convert v to `dtype` (fp->int truncates toward zero) */
+  PML_HIP_EPI_STORE,    /* store v to extra output `operand` (index into the outs array) */
+  PML_HIP_EPI_CMP_LT,   /* v = (v < x), result BOOL */
+  PML_HIP_EPI_CMP_GT,
+  PML_HIP_EPI_CMP_LE,
+  PML_HIP_EPI_CMP_GE,
+  PML_HIP_EPI_CMP_EQ,
+  PML_HIP_EPI_CMP_NE,
+  PML_HIP_EPI_SIGMOID_UNUSED_
+};
+
+/* where the second operand x of a step comes from */
+enum {
+  PML_HIP_OPND_NONE = 0,
+  PML_HIP_OPND_IMM = 1,    /* the immediate `imm` (converted to the step's type) */
+  PML_HIP_OPND_TENSOR = 2  /* operands[`operand`], addressed by the per-call strides */
+};
+
+#define PML_HIP_MAX_EPI_OPS 12
+#define PML_HIP_MAX_EPI_OPERANDS 6
+#define PML_HIP_MAX_RANK 6
+
+typedef struct {
+  int32_t opcode;
+  int32_t dtype;        /* result element type of this step */
+  int32_t operand_kind; /* PML_HIP_OPND_* */
+  int32_t operand;      /* index into operands[] (TENSOR) or outs[] (STORE) */
+  double imm;
+} pml_hip_epi_op;
+
+typedef struct {
+  int32_t n_ops;
+  int32_t n_operands;
+  pml_hip_epi_op ops[PML_HIP_MAX_EPI_OPS];
+  /* element type of each tensor operand */
+  int32_t operand_dtype[PML_HIP_MAX_EPI_OPERANDS];
+  /* For a 2-D (rows x cols) output as produced by gemm / conv2d: element strides
+   * of each tensor operand along the row and the column of the output
+   * (0 = broadcast).  A per-channel bias is {0, 1}. */
+  int64_t operand_row_stride[PML_HIP_MAX_EPI_OPERANDS];
+  int64_t operand_col_stride[PML_HIP_MAX_EPI_OPERANDS];
+} pml_hip_epilogue;
+
+/* ---- dense contraction: GEMM ------------------------------------------------
+ * C[m,n] = tail( init[m,n] + sum_k A[m,k] * B[k,n] ), row-major with leading
+ * dimensions, one launch per contraction.
+ * Replaces plaidml_rt_xsmm_gemm_dispatch_f32 / _invoke_f32 and the bias / relu
+ * variants (pmlc/rt/xsmm.cc:17-233), and the strided batch-reduce
+ * plaidml_rt_xsmm_brgemm_* (:235-287).
+ *   in_dtype F32  -> fp32 MFMA, fp32 accumulate
+ *   in_dtype BF16 -> bf16 MFMA, fp32 accumulate, result rounded once to acc_dtype's storage
+ *   in_dtype I8   -> int8 MFMA, int32 accumulate (this is the `cast(A, INT32)` then
+ *                    contract pattern of plaidml/edsl/tests/edsl_test.cc:509-545 applied to int8)
+ * out_dtype is the element type of the contraction result (F32, BF16 or I32); the
+ * tail then runs on that value and the final value is stored to C in the type of
+ * the last step (or out_dtype when the tail is empty). */
+typedef struct {
+  int32_t in_dtype;
+  int32_t out_dtype;
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc;
+  /* optional initial value (AddInitPattern, pmlc/dialect/tile/transforms/algebraic_opt.cc:30-75):
+   * init_kind 0 = none, 1 = tensor addressed with init_row_stride / init_col_stride */
+  int32_t init_kind;
+  int32_t init_dtype;
+  int64_t init_row_stride, init_col_stride;
+  int32_t c_dtype; /* element type stored to C (type after the tail) */
+  int32_t reserved;
+  pml_hip_epilogue tail;
+} pml_hip_gemm_desc;
+
+int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* desc); /* 0 on failure */
+int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, const void* init,
+                        const void* const* operands, void* const* outs, pml_hip_stream s);
+
+/* ---- dense contraction: 2-D convolution, NHWC (x) HWCK ------------------------
+ * O[n,y,x,co] = tail( init + sum_{ky,kx,ci} I[n, sy*y + dy*ky - py, sx*x + dx*kx - px, ci] * F[ky,kx,ci,co] )
+ * over the taps that fall inside the input (out-of-range taps are not part of
+ * the index set: docs/usage/edsl_ops.rst:24-44).  The index formulas are the
+ * ones plaidml/op/lib/ops.cc:1342-1450 emits for NXC / XCK layouts.
+ * Replaces the offset batch-reduce shims plaidml_rt_xsmm_brgemm_offs_*
+ * (pmlc/rt/xsmm.cc:289-342,457-861).  The tail sees the output as a
+ * (n*oh*ow) x co matrix. */
+typedef struct {
+  int32_t in_dtype;
+  int32_t out_dtype;
+  int64_t n, h, w, ci;
+  int64_t kh, kw, co;
+  int64_t oh, ow;
+  int64_t stride_h, stride_w;
+  int64_t dil_h, dil_w;
+  int64_t pad_h, pad_w; /* pad_before */
+  int32_t init_kind;
+  int32_t init_dtype;
+  int64_t init_row_stride, init_col_stride;
+  int32_t c_dtype;
+  int32_t reserved;
+  pml_hip_epilogue tail;
+} pml_hip_conv2d_desc;
+
+int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* desc);
+int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, void* output, const void* init,
+                          const void* const* operands, void* const* outs, pml_hip_stream s);
+
+/* ---- depthwise 2-D convolution, NHWC, channel multiplier 1 --------------------
+ * O[n,y,x,c] = tail( sum_{ky,kx} I[n, sy*y + ky - py, sx*x + kx - px, c] * F[ky,kx,c,0] )
+ * (GroupLayout IN_C + AutoGroupMode DEPTHWISE, plaidml/op/lib/ops.cc:1034-1045,1380-1384).
+ * Bandwidth-bound; the reference runs it as scalar loops after
+ * linalgx-regulate-depthwise (pmlc/dialect/linalgx/transforms/regulate_depthwise.cc:22-60). */
+typedef struct {
+  int32_t dtype; /* F32 or BF16 */
+  int32_t reserved;
+  int64_t n, h, w, c;
+  int64_t kh, kw;
+  int64_t oh, ow;
+  int64_t stride_h, stride_w;
+  int64_t dil_h, dil_w;
+  int64_t pad_h, pad_w;
+  pml_hip_epilogue tail; /* rows = n*oh*ow, cols = c */
+} pml_hip_dwconv2d_desc;
+
+int64_t pml_hip_dwconv2d_dispatch(const pml_hip_dwconv2d_desc* desc);
+int pml_hip_dwconv2d_invoke(int64_t plan, const void* input, const void* filter, void* output,
+                            const void* const* operands, void* const* outs, pml_hip_stream s);
+
+/* ---- window reduction: 2-D pooling, NHWC --------------------------------------
+ * O[n,y,x,c] = agg_{ky<kh,kx<kw} I[n, sy*y + ky - py, sx*x + kx - px, c] over in-range taps
+ * (plaidml/op/lib/ops.cc:2562-2703).  With `with_index`, a second output receives
+ * max_{taps with I == O} (ky*kw + kx) as int32: the cond/max argmax pattern of
+ * plaidml/op/lib/ops.cc:505-521 restricted to the window (ties -> largest index;
+ * a NaN tap is never selected). */
+typedef struct {
+  int32_t dtype; /* F32 or BF16 */
+  int32_t agg;   /* PML_HIP_AGG_MAX / MIN / ADD */
+  int64_t n, h, w, c;
+  int64_t kh, kw;
+  int64_t oh, ow;
+  int64_t stride_h, stride_w;
+  int64_t pad_h, pad_w;
+  int32_t with_index;
+  int32_t reserved;
+} pml_hip_pool2d_desc;
+
+int64_t pml_hip_pool2d_dispatch(const pml_hip_pool2d_desc* desc);
+int pml_hip_pool2d_invoke(int64_t plan, const void* input, void* output, void* index_output, pml_hip_stream s);
+
+/* ---- standalone elementwise chain -----------------------------------------------
+ * out[i] = tail(in[i]) over an N-d output with broadcasting operands; the
+ * counterpart of plaidml_rt_xsmm_unary_* / _binary_* (pmlc/rt/xsmm.cc:344-455)
+ * with the broadcast rule of buildBroadcastMap
+ * (pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:443-472). */
+typedef struct {
+  int32_t rank;
+  int32_t in_dtype;
+  int32_t out_dtype;
+  int32_t reserved;
+  int64_t sizes[PML_HIP_MAX_RANK];     /* output sizes */
+  int64_t in_strides[PML_HIP_MAX_RANK]; /* element strides of the first input (0 = broadcast) */
+  int64_t operand_strides[PML_HIP_MAX_EPI_OPERANDS][PML_HIP_MAX_RANK];
+  pml_hip_epilogue tail; /* row/col strides unused here */
+} pml_hip_eltwise_desc;
+
+int64_t pml_hip_eltwise_dispatch(const pml_hip_eltwise_desc* desc);
+int pml_hip_eltwise_invoke(int64_t plan, const void* input, void* output, const void* const* operands,
+                           void* const* outs, pml_hip_stream s);
+
+/* three-input select(cond, t, f) with broadcasting (tile.select, SelectOp of
+ * pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:262-273) */
+typedef struct {
+  int32_t rank;
+  int32_t cond_dtype;
+  int32_t t_dtype, f_dtype, out_dtype;
+  int32_t reserved;
+  int64_t sizes[PML_HIP_MAX_RANK];
+  int64_t cond_strides[PML_HIP_MAX_RANK], t_strides[PML_HIP_MAX_RANK], f_strides[PML_HIP_MAX_RANK];
+} pml_hip_select_desc;
+int pml_hip_select(const pml_hip_select_desc* desc, const void* cond, const void* t, const void* f, void* out,
+                   pml_hip_stream s);
+
+/* index(dims, axis) (tile.index, IndexOpConversion tile_to_linalg.cc:863-): int32 iota along `axis` */
+int pml_hip_index(void* out, int32_t rank, const int64_t* sizes, int32_t axis, pml_hip_stream s);
+
+/* ---- any contraction ---------------------------------------------------------
+ * The loop-nest form a contraction takes after bounds computation: the
+ * `affine.parallel` + `pxa.load` + `pxa.reduce` nest of
+ * pmlc/conversion/linalg_to_pxa/linalg_to_pxa.cc:283-428 with residual
+ * constraints as `affine.if`.  One GPU thread (or one wavefront, for long
+ * reductions) owns one output element and walks the reduction box; used for
+ * every contraction no specialised kernel matches, so that every Tile program
+ * in scope runs on the device.
+ *
+ * Index variables are ordered output-first: the first n_out_idx variables
+ * enumerate distinct output elements (their ranges multiply to the number of
+ * threads), the remaining ones are reduced.  An access / constraint is a set of
+ * linear forms (sum_i coef[i]*idx[i] + c0) / den that must be an integer q with
+ * 0 <= q < size; a tuple failing any form is skipped. */
+#define PML_HIP_MAX_IDX 12
+#define PML_HIP_MAX_FORMS 32
+
+typedef struct {
+  int32_t coef[PML_HIP_MAX_IDX];
+  int32_t c0;
+  int32_t den;
+  int32_t operand; /* 0 = output, 1.. = source, -1 = explicit constraint */
+  int64_t size;
+  int64_t stride; /* flat element stride of this dimension in its operand */
+} pml_hip_form;
+
+typedef struct {
+  int32_t dtype;    /* element type of the result and of the arithmetic */
+  int32_t agg;
+  int32_t combo;
+  int32_t n_idx;
+  int32_t n_out_idx;
+  int32_t n_src;
+  int32_t n_forms;
+  int32_t cmp_dtype; /* COMBO_COND: element type the two comparands are compared in */
+  int32_t src_dtype[3];
+  int32_t has_init;  /* output buffer already holds the initial value; else the identity is used */
+  int64_t lo[PML_HIP_MAX_IDX], hi[PML_HIP_MAX_IDX]; /* inclusive box */
+  int64_t out_elems;
+  double identity_f;  /* initial value when has_init == 0, floating result types */
+  int64_t identity_i; /* same for integer result types (already narrowed to dtype) */
+  pml_hip_form forms[PML_HIP_MAX_FORMS];
+} pml_hip_contract_desc;
+
+int64_t pml_hip_contract_dispatch(const pml_hip_contract_desc* desc);
+int pml_hip_contract_invoke(int64_t plan, const void* const* srcs, void* out, pml_hip_stream s);
+
+/* sizeof() of a descriptor struct as this library was compiled, so that a foreign-language
+ * binding can verify its own layout: 0 epilogue, 1 gemm, 2 conv2d, 3 dwconv2d, 4 pool2d,
+ * 5 eltwise, 6 select, 7 contract, 8 form.  Returns 0 for an unknown id. */
+size_t pml_hip_struct_size(int which);
+
+/* Releases a plan returned by any *_dispatch. */
+int pml_hip_plan_free(int64_t plan);
+/* Writes a one-line description of the plan (kernel family, tile, grid) for plan dumps. */
+int pml_hip_plan_describe(int64_t plan, char* buf, size_t buf_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PML_HIP_H_ */

@@ -1,0 +1,92 @@
+// Internal: kernel argument blocks, plan records and launcher prototypes shared
+// by the C ABI (pml_hip.hip) and the kernel translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "pml_hip.h"
+
+namespace pml {
+
+enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2 };
+enum { TILE_128x128 = 0, TILE_128x64, TILE_256x64, TILE_64x64 };
+
+struct TailPtrs {
+  const void* operands[PML_HIP_MAX_EPI_OPERANDS];
+  void* outs[PML_HIP_MAX_EPI_OPERANDS];
+};
+
+// Arguments of the MFMA GEMM / implicit-GEMM kernel (passed by value).
+struct IgemmArgs {
+  int64_t M, N, K;
+  const void* A;
+  int64_t lda;
+  const void* Bt;  // [N][K], K contiguous
+  int64_t ldbt;
+  void* C;
+  int64_t ldc;
+  // convolution geometry (CONV instantiations only)
+  int H, W, CI, OH, OW, KH, KW, SH, SW, PH, PW, DH, DW;
+  // result type of the contraction, optional initial value
+  int out_dtype;
+  const void* init;
+  int init_dtype;
+  int64_t init_rs, init_cs;
+  // fast tail: 0 = interpret `tail`; 1 = (optional relu) then store as c_dtype
+  int tail_mode;
+  int tail_relu;
+  int c_dtype;
+  pml_hip_epilogue tail;
+  const void* operands[PML_HIP_MAX_EPI_OPERANDS];
+  void* outs[PML_HIP_MAX_EPI_OPERANDS];
+};
+
+hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
+hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int64_t N, int64_t ldb, int64_t ldbt,
+                          hipStream_t s);
+
+// generic kernels (generic.hip)
+struct ContractArgs {
+  pml_hip_contract_desc d;
+  const void* srcs[3];
+  void* out;
+};
+hipError_t contract_launch(const ContractArgs& a, hipStream_t s);
+
+struct EltwiseArgs {
+  pml_hip_eltwise_desc d;
+  const void* in;
+  void* out;
+  const void* operands[PML_HIP_MAX_EPI_OPERANDS];
+  void* outs[PML_HIP_MAX_EPI_OPERANDS];
+  int64_t total;
+  int wide;  // 1: some element type needs the (double, int64) interpreter
+};
+hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s);
+hipError_t select_launch(const pml_hip_select_desc& d, const void* c, const void* t, const void* f, void* out,
+                         hipStream_t s);
+hipError_t index_launch(void* out, int rank, const int64_t* sizes, int axis, hipStream_t s);
+hipError_t fill_u32_launch(void* p, uint32_t pattern, size_t n_words, hipStream_t s);
+
+// window kernels (window.hip)
+struct DwconvArgs {
+  pml_hip_dwconv2d_desc d;
+  const void* in;
+  const void* filter;
+  void* out;
+  const void* operands[PML_HIP_MAX_EPI_OPERANDS];
+  void* outs[PML_HIP_MAX_EPI_OPERANDS];
+};
+hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s);
+struct PoolArgs {
+  pml_hip_pool2d_desc d;
+  const void* in;
+  void* out;
+  void* idx;
+};
+hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s);
+
+}  // namespace pml

@@ -1,0 +1,656 @@
+// The C ABI of the kernel library (include/pml_hip.h): device set-up, memory,
+// streams and the dispatch / invoke pairs that select a tiling once and launch
+// it many times.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "device_common.h"
+#include "plans.h"
+
+namespace pml {
+namespace {
+
+thread_local std::string g_err;
+
+int fail(const std::string& msg) {
+  g_err = msg;
+  return 1;
+}
+int check(hipError_t e, const char* what) {
+  if (e == hipSuccess) return 0;
+  g_err = std::string(what) + ": " + hipGetErrorString(e);
+  return 1;
+}
+
+enum PlanKind { PLAN_GEMM = 1, PLAN_CONV, PLAN_DWCONV, PLAN_POOL, PLAN_ELTWISE, PLAN_CONTRACT };
+
+struct Plan {
+  int kind = 0;
+  int mfma_kind = 0;
+  int tile = 0;
+  pml_hip_gemm_desc gemm;
+  pml_hip_conv2d_desc conv;
+  pml_hip_dwconv2d_desc dw;
+  pml_hip_pool2d_desc pool;
+  pml_hip_eltwise_desc elt;
+  pml_hip_contract_desc con;
+  // packed right-hand side Bt[N][K]
+  void* bt = nullptr;
+  int64_t bt_ld = 0;
+  size_t bt_bytes = 0;
+  std::string text;
+  ~Plan() {
+    if (bt) (void)hipFree(bt);
+  }
+};
+
+int mfma_kind_of(int in_dtype) {
+  switch (in_dtype) {
+    case PML_HIP_F32: return KIND_F32;
+    case PML_HIP_BF16: return KIND_BF16;
+    case PML_HIP_I8: return KIND_I8;
+  }
+  return -1;
+}
+
+const char* tile_name(int t) {
+  switch (t) {
+    case TILE_128x128: return "128x128";
+    case TILE_128x64: return "128x64";
+    case TILE_256x64: return "256x64";
+    case TILE_64x64: return "64x64";
+  }
+  return "?";
+}
+
+// Stated tiling choice per shape class.  256 CUs want >= 256 workgroups in
+// flight (one wave of the grid); prefer the largest tile that still yields
+// about two workgroups per CU, and never a tile wider than N.
+int choose_tile(int64_t m, int64_t n) {
+  auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+  const int64_t want = 2 * 256;
+  if (n <= 64) {
+    if (tiles(256, 64) >= want) return TILE_256x64;
+    if (tiles(128, 64) >= 256) return TILE_128x64;
+    return TILE_64x64;
+  }
+  if (tiles(128, 128) >= want) return TILE_128x128;
+  if (tiles(128, 64) >= 256) return TILE_128x64;
+  return TILE_64x64;
+}
+
+// A tail that is only "relu?" can use the fast store path.
+void classify_tail(const pml_hip_epilogue& t, int out_dtype, int c_dtype, int* mode, int* relu) {
+  *mode = 0;
+  *relu = 0;
+  if (c_dtype != out_dtype) return;
+  if (t.n_ops == 0) {
+    *mode = 1;
+    return;
+  }
+  if (t.n_ops == 1 && t.ops[0].opcode == PML_HIP_EPI_RELU && t.ops[0].dtype == out_dtype) {
+    *mode = 1;
+    *relu = 1;
+  }
+}
+
+bool valid_tail(const pml_hip_epilogue& t) {
+  if (t.n_ops < 0 || t.n_ops > PML_HIP_MAX_EPI_OPS) return false;
+  if (t.n_operands < 0 || t.n_operands > PML_HIP_MAX_EPI_OPERANDS) return false;
+  for (int i = 0; i < t.n_ops; ++i) {
+    const pml_hip_epi_op& op = t.ops[i];
+    if (op.opcode < PML_HIP_EPI_ADD || op.opcode > PML_HIP_EPI_CMP_NE) return false;
+    if (op.operand_kind == PML_HIP_OPND_TENSOR && (op.operand < 0 || op.operand >= t.n_operands)) return false;
+    if (op.opcode == PML_HIP_EPI_STORE && (op.operand < 0 || op.operand >= PML_HIP_MAX_EPI_OPERANDS)) return false;
+    if (dt_size(op.dtype) == 8 && op.opcode != PML_HIP_EPI_STORE) return false;  // 64-bit steps: general path only
+  }
+  return true;
+}
+
+}  // namespace
+}  // namespace pml
+
+using namespace pml;
+
+extern "C" {
+
+const char* pml_hip_last_error(void) { return g_err.c_str(); }
+
+int pml_hip_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+int pml_hip_init(int device_ordinal) {
+  int n = pml_hip_device_count();
+  if (n <= 0) return fail("no HIP device is visible");
+  if (device_ordinal < 0 || device_ordinal >= n) return fail("device ordinal out of range");
+  return check(hipSetDevice(device_ordinal), "hipSetDevice");
+}
+
+int pml_hip_device_name(char* buf, size_t buf_len) {
+  if (!buf || buf_len == 0) return fail("null buffer");
+  int dev = 0;
+  if (check(hipGetDevice(&dev), "hipGetDevice")) return 1;
+  hipDeviceProp_t prop;
+  if (check(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties")) return 1;
+  std::snprintf(buf, buf_len, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+  return 0;
+}
+
+int pml_hip_malloc(void** dptr, size_t nbytes) {
+  if (!dptr) return fail("null out pointer");
+  *dptr = nullptr;
+  if (nbytes == 0) nbytes = 16;
+  return check(hipMalloc(dptr, nbytes), "hipMalloc");
+}
+int pml_hip_free(void* dptr) { return dptr ? check(hipFree(dptr), "hipFree") : 0; }
+int pml_hip_host_alloc(void** hptr, size_t nbytes) {
+  if (!hptr) return fail("null out pointer");
+  return check(hipHostMalloc(hptr, nbytes ? nbytes : 16, hipHostMallocDefault), "hipHostMalloc");
+}
+int pml_hip_host_free(void* hptr) { return hptr ? check(hipHostFree(hptr), "hipHostFree") : 0; }
+
+int pml_hip_memcpy_h2d(void* dst, const void* src, size_t nbytes, pml_hip_stream s) {
+  if (nbytes == 0) return 0;
+  if (check(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, (hipStream_t)s), "hipMemcpyAsync(h2d)")) return 1;
+  return check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize");
+}
+int pml_hip_memcpy_d2h(void* dst, const void* src, size_t nbytes, pml_hip_stream s) {
+  if (nbytes == 0) return 0;
+  if (check(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, (hipStream_t)s), "hipMemcpyAsync(d2h)")) return 1;
+  return check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize");
+}
+int pml_hip_memcpy_d2d(void* dst, const void* src, size_t nbytes, pml_hip_stream s) {
+  if (nbytes == 0) return 0;
+  return check(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, (hipStream_t)s), "hipMemcpyAsync(d2d)");
+}
+int pml_hip_fill_u32(void* dptr, uint32_t pattern, size_t n_words, pml_hip_stream s) {
+  return check(fill_u32_launch(dptr, pattern, n_words, (hipStream_t)s), "fill");
+}
+
+int pml_hip_stream_create(pml_hip_stream* s) {
+  hipStream_t st;
+  if (check(hipStreamCreate(&st), "hipStreamCreate")) return 1;
+  *s = (pml_hip_stream)st;
+  return 0;
+}
+int pml_hip_stream_destroy(pml_hip_stream s) { return check(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy"); }
+int pml_hip_stream_sync(pml_hip_stream s) { return check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize"); }
+int pml_hip_event_create(pml_hip_event* e) {
+  hipEvent_t ev;
+  if (check(hipEventCreate(&ev), "hipEventCreate")) return 1;
+  *e = (pml_hip_event)ev;
+  return 0;
+}
+int pml_hip_event_destroy(pml_hip_event e) { return check(hipEventDestroy((hipEvent_t)e), "hipEventDestroy"); }
+int pml_hip_event_record(pml_hip_event e, pml_hip_stream s) {
+  return check(hipEventRecord((hipEvent_t)e, (hipStream_t)s), "hipEventRecord");
+}
+int pml_hip_event_sync(pml_hip_event e) { return check(hipEventSynchronize((hipEvent_t)e), "hipEventSynchronize"); }
+int pml_hip_event_elapsed_ms(pml_hip_event start, pml_hip_event stop, float* ms) {
+  return check(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
+}
+
+// ---------------------------------------------------------------------------
+// GEMM
+// ---------------------------------------------------------------------------
+
+int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
+  if (!d) {
+    fail("null descriptor");
+    return 0;
+  }
+  const int kind = mfma_kind_of(d->in_dtype);
+  if (kind < 0) {
+    fail("gemm: in_dtype must be F32, BF16 or I8");
+    return 0;
+  }
+  const bool out_ok = (kind == KIND_I8) ? d->out_dtype == PML_HIP_I32
+                                        : (d->out_dtype == PML_HIP_F32 || (kind == KIND_BF16 && d->out_dtype == PML_HIP_BF16));
+  if (!out_ok) {
+    fail("gemm: out_dtype does not fit in_dtype");
+    return 0;
+  }
+  if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->lda < d->k || d->ldb < d->n || d->ldc < d->n) {
+    fail("gemm: bad sizes or leading dimensions");
+    return 0;
+  }
+  const int es = dt_size(d->in_dtype);
+  if ((d->k * es) % 16 != 0 || (d->lda * es) % 16 != 0) {
+    fail("gemm: K and lda must cover whole 16-byte vectors");
+    return 0;
+  }
+  if (!valid_tail(d->tail)) {
+    fail("gemm: malformed tail");
+    return 0;
+  }
+  Plan* p = new Plan();
+  p->kind = PLAN_GEMM;
+  p->mfma_kind = kind;
+  p->gemm = *d;
+  p->tile = choose_tile(d->m, d->n);
+  p->bt_ld = d->k;
+  p->bt_bytes = (size_t)d->n * d->k * es;
+  if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
+    delete p;
+    fail("gemm: cannot allocate the packed right-hand side");
+    return 0;
+  }
+  char buf[256];
+  std::snprintf(buf, sizeof buf, "gemm %s m=%lld n=%lld k=%lld tile=%s mfma=%s", d->in_dtype == PML_HIP_F32 ? "f32" : d->in_dtype == PML_HIP_BF16 ? "bf16" : "i8",
+                (long long)d->m, (long long)d->n, (long long)d->k, tile_name(p->tile),
+                kind == KIND_F32 ? "f32_32x32x2" : kind == KIND_BF16 ? "f32_32x32x16_bf16" : "i32_32x32x32_i8");
+  p->text = buf;
+  return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, const void* init,
+                        const void* const* operands, void* const* outs, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
+  const pml_hip_gemm_desc& d = p->gemm;
+  if (!a || !b || !c) return fail("gemm_invoke: null operand");
+  if (((uintptr_t)a & 15) != 0) return fail("gemm_invoke: A must be 16-byte aligned");
+  if (d.init_kind && !init) return fail("gemm_invoke: the plan expects an initial value");
+  const int es = dt_size(d.in_dtype);
+  if (check(transpose_pack(es, b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack")) return 1;
+  IgemmArgs g;
+  std::memset(&g, 0, sizeof g);
+  g.M = d.m;
+  g.N = d.n;
+  g.K = d.k;
+  g.A = a;
+  g.lda = d.lda;
+  g.Bt = p->bt;
+  g.ldbt = p->bt_ld;
+  g.C = c;
+  g.ldc = d.ldc;
+  g.out_dtype = d.out_dtype;
+  g.init = d.init_kind ? init : nullptr;
+  g.init_dtype = d.init_dtype;
+  g.init_rs = d.init_row_stride;
+  g.init_cs = d.init_col_stride;
+  g.c_dtype = d.c_dtype;
+  classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
+  g.tail = d.tail;
+  for (int i = 0; i < d.tail.n_operands; ++i) {
+    if (!operands || !operands[i]) return fail("gemm_invoke: missing tail operand");
+    g.operands[i] = operands[i];
+  }
+  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
+  for (int i = 0; i < d.tail.n_ops; ++i)
+    if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
+      return fail("gemm_invoke: missing extra output");
+  return check(igemm_launch(p->mfma_kind, p->tile, false, g, (hipStream_t)s), "igemm_launch");
+}
+
+// ---------------------------------------------------------------------------
+// conv2d
+// ---------------------------------------------------------------------------
+
+int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
+  if (!d) {
+    fail("null descriptor");
+    return 0;
+  }
+  const int kind = mfma_kind_of(d->in_dtype);
+  if (kind < 0) {
+    fail("conv2d: in_dtype must be F32, BF16 or I8");
+    return 0;
+  }
+  const bool out_ok = (kind == KIND_I8) ? d->out_dtype == PML_HIP_I32
+                                        : (d->out_dtype == PML_HIP_F32 || (kind == KIND_BF16 && d->out_dtype == PML_HIP_BF16));
+  if (!out_ok) {
+    fail("conv2d: out_dtype does not fit in_dtype");
+    return 0;
+  }
+  if (d->n <= 0 || d->h <= 0 || d->w <= 0 || d->ci <= 0 || d->co <= 0 || d->kh <= 0 || d->kw <= 0 || d->oh <= 0 ||
+      d->ow <= 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dil_h <= 0 || d->dil_w <= 0) {
+    fail("conv2d: bad geometry");
+    return 0;
+  }
+  const int es = dt_size(d->in_dtype);
+  if ((d->ci * es) % 16 != 0) {
+    fail("conv2d: input channels must cover whole 16-byte vectors");
+    return 0;
+  }
+  if (d->n * d->h * d->w * d->ci >= ((int64_t)1 << 40) || d->h * d->w > (1 << 30)) {
+    fail("conv2d: tensor too large");
+    return 0;
+  }
+  if (!valid_tail(d->tail)) {
+    fail("conv2d: malformed tail");
+    return 0;
+  }
+  Plan* p = new Plan();
+  p->kind = PLAN_CONV;
+  p->mfma_kind = kind;
+  p->conv = *d;
+  const int64_t M = d->n * d->oh * d->ow;
+  const int64_t K = d->kh * d->kw * d->ci;
+  p->tile = choose_tile(M, d->co);
+  p->bt_ld = K;
+  p->bt_bytes = (size_t)d->co * K * es;
+  if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
+    delete p;
+    fail("conv2d: cannot allocate the packed filter");
+    return 0;
+  }
+  char buf[256];
+  std::snprintf(buf, sizeof buf, "conv2d %s n=%lld %lldx%lldx%lld k=%lldx%lld co=%lld -> %lldx%lld (implicit gemm m=%lld n=%lld k=%lld) tile=%s",
+                d->in_dtype == PML_HIP_F32 ? "f32" : d->in_dtype == PML_HIP_BF16 ? "bf16" : "i8", (long long)d->n,
+                (long long)d->h, (long long)d->w, (long long)d->ci, (long long)d->kh, (long long)d->kw, (long long)d->co,
+                (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, tile_name(p->tile));
+  p->text = buf;
+  return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, void* output, const void* init,
+                          const void* const* operands, void* const* outs, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_CONV) return fail("conv2d_invoke: not a conv2d plan");
+  const pml_hip_conv2d_desc& d = p->conv;
+  if (!input || !filter || !output) return fail("conv2d_invoke: null operand");
+  if (((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
+  if (d.init_kind && !init) return fail("conv2d_invoke: the plan expects an initial value");
+  const int es = dt_size(d.in_dtype);
+  const int64_t K = d.kh * d.kw * d.ci;
+  // the HWCK filter is a row-major [K][CO] matrix
+  if (check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack")) return 1;
+  IgemmArgs g;
+  std::memset(&g, 0, sizeof g);
+  g.M = d.n * d.oh * d.ow;
+  g.N = d.co;
+  g.K = K;
+  g.A = input;
+  g.Bt = p->bt;
+  g.ldbt = p->bt_ld;
+  g.C = output;
+  g.ldc = d.co;
+  g.H = (int)d.h;
+  g.W = (int)d.w;
+  g.CI = (int)d.ci;
+  g.OH = (int)d.oh;
+  g.OW = (int)d.ow;
+  g.KH = (int)d.kh;
+  g.KW = (int)d.kw;
+  g.SH = (int)d.stride_h;
+  g.SW = (int)d.stride_w;
+  g.PH = (int)d.pad_h;
+  g.PW = (int)d.pad_w;
+  g.DH = (int)d.dil_h;
+  g.DW = (int)d.dil_w;
+  g.out_dtype = d.out_dtype;
+  g.init = d.init_kind ? init : nullptr;
+  g.init_dtype = d.init_dtype;
+  g.init_rs = d.init_row_stride;
+  g.init_cs = d.init_col_stride;
+  g.c_dtype = d.c_dtype;
+  classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
+  g.tail = d.tail;
+  for (int i = 0; i < d.tail.n_operands; ++i) {
+    if (!operands || !operands[i]) return fail("conv2d_invoke: missing tail operand");
+    g.operands[i] = operands[i];
+  }
+  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
+  for (int i = 0; i < d.tail.n_ops; ++i)
+    if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
+      return fail("conv2d_invoke: missing extra output");
+  return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
+}
+
+// ---------------------------------------------------------------------------
+// depthwise conv, pooling
+// ---------------------------------------------------------------------------
+
+int64_t pml_hip_dwconv2d_dispatch(const pml_hip_dwconv2d_desc* d) {
+  if (!d) {
+    fail("null descriptor");
+    return 0;
+  }
+  if (d->dtype != PML_HIP_F32 && d->dtype != PML_HIP_BF16) {
+    fail("dwconv2d: dtype must be F32 or BF16");
+    return 0;
+  }
+  const int V = 16 / dt_size(d->dtype);
+  if (d->c <= 0 || d->c % V != 0) {
+    fail("dwconv2d: channels must cover whole 16-byte vectors");
+    return 0;
+  }
+  if (d->n <= 0 || d->h <= 0 || d->w <= 0 || d->kh <= 0 || d->kw <= 0 || d->oh <= 0 || d->ow <= 0 ||
+      d->stride_h <= 0 || d->stride_w <= 0 || d->dil_h <= 0 || d->dil_w <= 0 || !valid_tail(d->tail)) {
+    fail("dwconv2d: bad geometry or tail");
+    return 0;
+  }
+  Plan* p = new Plan();
+  p->kind = PLAN_DWCONV;
+  p->dw = *d;
+  char buf[200];
+  std::snprintf(buf, sizeof buf, "dwconv2d %s n=%lld %lldx%lldx%lld k=%lldx%lld -> %lldx%lld (16B channel vectors)",
+                d->dtype == PML_HIP_F32 ? "f32" : "bf16", (long long)d->n, (long long)d->h, (long long)d->w,
+                (long long)d->c, (long long)d->kh, (long long)d->kw, (long long)d->oh, (long long)d->ow);
+  p->text = buf;
+  return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_dwconv2d_invoke(int64_t plan, const void* input, const void* filter, void* output,
+                            const void* const* operands, void* const* outs, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_DWCONV) return fail("dwconv2d_invoke: not a dwconv2d plan");
+  if (!input || !filter || !output) return fail("dwconv2d_invoke: null operand");
+  if ((((uintptr_t)input | (uintptr_t)filter | (uintptr_t)output) & 15) != 0)
+    return fail("dwconv2d_invoke: buffers must be 16-byte aligned");
+  DwconvArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.d = p->dw;
+  a.in = input;
+  a.filter = filter;
+  a.out = output;
+  for (int i = 0; i < a.d.tail.n_operands; ++i) {
+    if (!operands || !operands[i]) return fail("dwconv2d_invoke: missing tail operand");
+    a.operands[i] = operands[i];
+  }
+  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) a.outs[i] = outs ? outs[i] : nullptr;
+  return check(dwconv2d_launch(a, (hipStream_t)s), "dwconv2d_launch");
+}
+
+int64_t pml_hip_pool2d_dispatch(const pml_hip_pool2d_desc* d) {
+  if (!d) {
+    fail("null descriptor");
+    return 0;
+  }
+  if (d->dtype != PML_HIP_F32 && d->dtype != PML_HIP_BF16) {
+    fail("pool2d: dtype must be F32 or BF16");
+    return 0;
+  }
+  if (d->agg != PML_HIP_AGG_MAX && d->agg != PML_HIP_AGG_MIN && d->agg != PML_HIP_AGG_ADD) {
+    fail("pool2d: aggregation must be max, min or add");
+    return 0;
+  }
+  const int V = 16 / dt_size(d->dtype);
+  if (d->c <= 0 || d->c % V != 0 || d->n <= 0 || d->h <= 0 || d->w <= 0 || d->kh <= 0 || d->kw <= 0 || d->oh <= 0 ||
+      d->ow <= 0 || d->stride_h <= 0 || d->stride_w <= 0) {
+    fail("pool2d: bad geometry (channels must cover whole 16-byte vectors)");
+    return 0;
+  }
+  Plan* p = new Plan();
+  p->kind = PLAN_POOL;
+  p->pool = *d;
+  char buf[200];
+  std::snprintf(buf, sizeof buf, "pool2d %s agg=%d n=%lld %lldx%lldx%lld k=%lldx%lld -> %lldx%lld%s",
+                d->dtype == PML_HIP_F32 ? "f32" : "bf16", d->agg, (long long)d->n, (long long)d->h, (long long)d->w,
+                (long long)d->c, (long long)d->kh, (long long)d->kw, (long long)d->oh, (long long)d->ow,
+                d->with_index ? " +argmax" : "");
+  p->text = buf;
+  return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_pool2d_invoke(int64_t plan, const void* input, void* output, void* index_output, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_POOL) return fail("pool2d_invoke: not a pool2d plan");
+  if (!input || !output) return fail("pool2d_invoke: null operand");
+  if (p->pool.with_index && !index_output) return fail("pool2d_invoke: the plan expects an index output");
+  if ((((uintptr_t)input | (uintptr_t)output | (uintptr_t)index_output) & 15) != 0)
+    return fail("pool2d_invoke: buffers must be 16-byte aligned");
+  PoolArgs a;
+  a.d = p->pool;
+  a.in = input;
+  a.out = output;
+  a.idx = index_output;
+  return check(pool2d_launch(a, (hipStream_t)s), "pool2d_launch");
+}
+
+// ---------------------------------------------------------------------------
+// elementwise, select, index
+// ---------------------------------------------------------------------------
+
+int64_t pml_hip_eltwise_dispatch(const pml_hip_eltwise_desc* d) {
+  if (!d) {
+    fail("null descriptor");
+    return 0;
+  }
+  if (d->rank < 0 || d->rank > PML_HIP_MAX_RANK) {
+    fail("eltwise: rank out of range");
+    return 0;
+  }
+  const pml_hip_epilogue& t = d->tail;
+  if (t.n_ops < 0 || t.n_ops > PML_HIP_MAX_EPI_OPS || t.n_operands < 0 || t.n_operands > PML_HIP_MAX_EPI_OPERANDS) {
+    fail("eltwise: malformed tail");
+    return 0;
+  }
+  Plan* p = new Plan();
+  p->kind = PLAN_ELTWISE;
+  p->elt = *d;
+  p->text = "eltwise chain of " + std::to_string(t.n_ops) + " steps, rank " + std::to_string(d->rank);
+  return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_eltwise_invoke(int64_t plan, const void* input, void* output, const void* const* operands,
+                           void* const* outs, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_ELTWISE) return fail("eltwise_invoke: not an eltwise plan");
+  if (!input || !output) return fail("eltwise_invoke: null operand");
+  EltwiseArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.d = p->elt;
+  a.in = input;
+  a.out = output;
+  a.total = 1;
+  for (int r = 0; r < a.d.rank; ++r) a.total *= a.d.sizes[r];
+  bool wide = dt_size(a.d.in_dtype) == 8 || dt_size(a.d.out_dtype) == 8;
+  for (int i = 0; i < a.d.tail.n_operands; ++i) {
+    if (!operands || !operands[i]) return fail("eltwise_invoke: missing operand");
+    a.operands[i] = operands[i];
+    wide = wide || dt_size(a.d.tail.operand_dtype[i]) == 8;
+  }
+  for (int i = 0; i < a.d.tail.n_ops; ++i) wide = wide || dt_size(a.d.tail.ops[i].dtype) == 8;
+  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) a.outs[i] = outs ? outs[i] : nullptr;
+  a.wide = wide ? 1 : 0;
+  return check(eltwise_launch(a, (hipStream_t)s), "eltwise_launch");
+}
+
+int pml_hip_select(const pml_hip_select_desc* d, const void* cond, const void* t, const void* f, void* out,
+                   pml_hip_stream s) {
+  if (!d || !cond || !t || !f || !out) return fail("select: null argument");
+  if (d->rank < 0 || d->rank > PML_HIP_MAX_RANK) return fail("select: rank out of range");
+  return check(select_launch(*d, cond, t, f, out, (hipStream_t)s), "select_launch");
+}
+
+int pml_hip_index(void* out, int32_t rank, const int64_t* sizes, int32_t axis, pml_hip_stream s) {
+  if (!out || !sizes || rank <= 0 || axis < 0 || axis >= rank) return fail("index: bad argument");
+  return check(index_launch(out, rank, sizes, axis, (hipStream_t)s), "index_launch");
+}
+
+// ---------------------------------------------------------------------------
+// any contraction
+// ---------------------------------------------------------------------------
+
+int64_t pml_hip_contract_dispatch(const pml_hip_contract_desc* d) {
+  if (!d) {
+    fail("null descriptor");
+    return 0;
+  }
+  if (d->n_idx < 0 || d->n_idx > PML_HIP_MAX_IDX || d->n_out_idx < 0 || d->n_out_idx > d->n_idx || d->n_forms < 0 ||
+      d->n_forms > PML_HIP_MAX_FORMS || d->n_src < 1 || d->n_src > 3) {
+    fail("contract: descriptor out of range");
+    return 0;
+  }
+  int64_t outs = 1;
+  for (int v = 0; v < d->n_out_idx; ++v) {
+    if (d->hi[v] < d->lo[v]) {
+      outs = 0;
+      break;
+    }
+    outs *= d->hi[v] - d->lo[v] + 1;
+  }
+  if (outs != d->out_elems) {
+    fail("contract: out_elems does not match the output index ranges");
+    return 0;
+  }
+  for (int f = 0; f < d->n_forms; ++f) {
+    if (d->forms[f].den <= 0 || d->forms[f].operand < -1 || d->forms[f].operand > d->n_src) {
+      fail("contract: malformed form");
+      return 0;
+    }
+  }
+  if (d->combo == PML_HIP_COMBO_EQ) {
+    fail("contract: the eq combination is not supported");
+    return 0;
+  }
+  Plan* p = new Plan();
+  p->kind = PLAN_CONTRACT;
+  p->con = *d;
+  p->text = "contract (thread per output element) agg=" + std::to_string(d->agg) + " combo=" + std::to_string(d->combo) +
+            " idx=" + std::to_string(d->n_idx) + " outputs=" + std::to_string((long long)d->out_elems);
+  return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_contract_invoke(int64_t plan, const void* const* srcs, void* out, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_CONTRACT) return fail("contract_invoke: not a contract plan");
+  if (!srcs || !out) return fail("contract_invoke: null operand");
+  ContractArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.d = p->con;
+  for (int i = 0; i < a.d.n_src; ++i) {
+    if (!srcs[i]) return fail("contract_invoke: null source");
+    a.srcs[i] = srcs[i];
+  }
+  a.out = out;
+  return check(contract_launch(a, (hipStream_t)s), "contract_launch");
+}
+
+size_t pml_hip_struct_size(int which) {
+  switch (which) {
+    case 0: return sizeof(pml_hip_epilogue);
+    case 1: return sizeof(pml_hip_gemm_desc);
+    case 2: return sizeof(pml_hip_conv2d_desc);
+    case 3: return sizeof(pml_hip_dwconv2d_desc);
+    case 4: return sizeof(pml_hip_pool2d_desc);
+    case 5: return sizeof(pml_hip_eltwise_desc);
+    case 6: return sizeof(pml_hip_select_desc);
+    case 7: return sizeof(pml_hip_contract_desc);
+    case 8: return sizeof(pml_hip_form);
+  }
+  return 0;
+}
+
+int pml_hip_plan_free(int64_t plan) {
+  delete (Plan*)(intptr_t)plan;
+  return 0;
+}
+
+int pml_hip_plan_describe(int64_t plan, char* buf, size_t buf_len) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || !buf || buf_len == 0) return fail("plan_describe: bad argument");
+  std::snprintf(buf, buf_len, "%s", p->text.c_str());
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,202 @@
+// Bandwidth-bound window kernels over NHWC tensors: depthwise convolution and
+// pooling (with the optional window-argmax output).  One thread owns 16 bytes
+// of channels (8 bf16 / 4 fp32) of one output pixel; consecutive threads walk
+// the channel vectors of a pixel, then the next pixel, so every global access
+// of a wavefront is a run of contiguous 16-byte pieces.  The KHxKW taps of
+// neighbouring outputs overlap and are served by L1/L2, so HBM sees each input
+// byte about once.
+#include <hip/hip_runtime.h>
+
+#include "device_common.h"
+#include "plans.h"
+
+namespace pml {
+
+namespace {
+
+template <int ES>
+struct VecIO;
+template <>
+struct VecIO<2> {
+  static constexpr int V = 8;
+  __device__ static void load(const void* p, int64_t elem_off, float* f) {
+    i32x4_t raw = *(const i32x4_t*)((const uint16_t*)p + elem_off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(((uint32_t)raw[i]) << 16);
+      f[2 * i + 1] = __uint_as_float(((uint32_t)raw[i]) & 0xffff0000u);
+    }
+  }
+};
+template <>
+struct VecIO<4> {
+  static constexpr int V = 4;
+  __device__ static void load(const void* p, int64_t elem_off, float* f) {
+    f32x4_t raw = *(const f32x4_t*)((const float*)p + elem_off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = raw[i];
+  }
+};
+
+template <int ES>
+__global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t total_vecs) {
+  constexpr int V = VecIO<ES>::V;
+  const pml_hip_dwconv2d_desc& d = a.d;
+  const int dt = d.dtype;
+  const int64_t cvecs = d.c / V;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total_vecs; g += stride) {
+    const int64_t cv = g % cvecs;
+    const int64_t pix = g / cvecs;
+    const int ox = (int)(pix % d.ow);
+    const int64_t t = pix / d.ow;
+    const int oy = (int)(t % d.oh);
+    const int64_t n = t / d.oh;
+    const int64_t c0 = cv * V;
+    float acc[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
+    for (int ky = 0; ky < d.kh; ++ky) {
+      const int64_t iy = (int64_t)oy * d.stride_h + (int64_t)ky * d.dil_h - d.pad_h;
+      if (iy < 0 || iy >= d.h) continue;
+      for (int kx = 0; kx < d.kw; ++kx) {
+        const int64_t ix = (int64_t)ox * d.stride_w + (int64_t)kx * d.dil_w - d.pad_w;
+        if (ix < 0 || ix >= d.w) continue;
+        float x[V], w[V];
+        VecIO<ES>::load(a.in, ((n * d.h + iy) * d.w + ix) * d.c + c0, x);
+        VecIO<ES>::load(a.filter, ((int64_t)ky * d.kw + kx) * d.c + c0, w);
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] += x[i] * w[i];
+      }
+    }
+    const int64_t o0 = pix * d.c + c0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      Scalar<float, int> v;
+      v.i = 0;
+      v.f = round_float_to<float>(dt, acc[i]);
+      int cur = dt;
+      int64_t off[PML_HIP_MAX_EPI_OPERANDS];
+#pragma unroll
+      for (int q = 0; q < PML_HIP_MAX_EPI_OPERANDS; ++q)
+        off[q] = q < d.tail.n_operands ? pix * d.tail.operand_row_stride[q] + (c0 + i) * d.tail.operand_col_stride[q] : 0;
+      v = run_tail<float, int>(d.tail, v, &cur, a.operands, off, a.outs, o0 + i);
+      store_scalar<float, int>(a.out, o0 + i, cur, v);
+    }
+  }
+}
+
+template <int ES>
+__global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_vecs) {
+  constexpr int V = VecIO<ES>::V;
+  const pml_hip_pool2d_desc& d = a.d;
+  const int dt = d.dtype;
+  const int64_t cvecs = d.c / V;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total_vecs; g += stride) {
+    const int64_t cv = g % cvecs;
+    const int64_t pix = g / cvecs;
+    const int ox = (int)(pix % d.ow);
+    const int64_t t = pix / d.ow;
+    const int oy = (int)(t % d.oh);
+    const int64_t n = t / d.oh;
+    const int64_t c0 = cv * V;
+    float acc[V];
+    const float ident = d.agg == PML_HIP_AGG_MAX ? -INFINITY : (d.agg == PML_HIP_AGG_MIN ? INFINITY : 0.f);
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = ident;
+    for (int ky = 0; ky < d.kh; ++ky) {
+      const int64_t iy = (int64_t)oy * d.stride_h + ky - d.pad_h;
+      if (iy < 0 || iy >= d.h) continue;
+      for (int kx = 0; kx < d.kw; ++kx) {
+        const int64_t ix = (int64_t)ox * d.stride_w + kx - d.pad_w;
+        if (ix < 0 || ix >= d.w) continue;
+        float x[V];
+        VecIO<ES>::load(a.in, ((n * d.h + iy) * d.w + ix) * d.c + c0, x);
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          if (d.agg == PML_HIP_AGG_MAX)
+            acc[i] = (x[i] > acc[i]) ? x[i] : acc[i];
+          else if (d.agg == PML_HIP_AGG_MIN)
+            acc[i] = (x[i] < acc[i]) ? x[i] : acc[i];
+          else
+            acc[i] += x[i];
+        }
+      }
+    }
+    const int64_t o0 = pix * d.c + c0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      Scalar<float, int> v;
+      v.i = 0;
+      v.f = round_float_to<float>(dt, acc[i]);
+      acc[i] = v.f;
+      store_scalar<float, int>(a.out, o0 + i, dt, v);
+    }
+    if (d.with_index) {
+      // largest window index whose (in-range) tap equals the pooled value; 0 if none
+      int best[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) best[i] = 0;
+      for (int ky = 0; ky < d.kh; ++ky) {
+        const int64_t iy = (int64_t)oy * d.stride_h + ky - d.pad_h;
+        if (iy < 0 || iy >= d.h) continue;
+        for (int kx = 0; kx < d.kw; ++kx) {
+          const int64_t ix = (int64_t)ox * d.stride_w + kx - d.pad_w;
+          if (ix < 0 || ix >= d.w) continue;
+          float x[V];
+          VecIO<ES>::load(a.in, ((n * d.h + iy) * d.w + ix) * d.c + c0, x);
+          const int k = ky * (int)d.kw + kx;
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const int cand = (x[i] == acc[i]) ? k : 0;
+            best[i] = cand > best[i] ? cand : best[i];
+          }
+        }
+      }
+      int32_t* ip = (int32_t*)a.idx + o0;
+#pragma unroll
+      for (int i = 0; i < V; i += 4) {
+        i32x4_t w = {best[i], best[i + 1], best[i + 2], best[i + 3]};
+        *(i32x4_t*)(ip + i) = w;
+      }
+    }
+  }
+}
+
+inline unsigned grid_for(int64_t items) {
+  int64_t blocks = (items + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  const int64_t cap = 256 * 32;
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+}  // namespace
+
+hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
+  const pml_hip_dwconv2d_desc& d = a.d;
+  const int es = dt_size(d.dtype);
+  const int V = 16 / es;
+  const int64_t total = d.n * d.oh * d.ow * (d.c / V);
+  if (total == 0) return hipSuccess;
+  if (es == 2)
+    hipLaunchKernelGGL((dwconv2d_kernel<2>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  else
+    hipLaunchKernelGGL((dwconv2d_kernel<4>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  return hipGetLastError();
+}
+
+hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s) {
+  const pml_hip_pool2d_desc& d = a.d;
+  const int es = dt_size(d.dtype);
+  const int V = 16 / es;
+  const int64_t total = d.n * d.oh * d.ow * (d.c / V);
+  if (total == 0) return hipSuccess;
+  if (es == 2)
+    hipLaunchKernelGGL((pool2d_kernel<2>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  else
+    hipLaunchKernelGGL((pool2d_kernel<4>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  return hipGetLastError();
+}
+
+}  // namespace pml

@@ -1,0 +1,42 @@
+"""The C-ABI libraries load and export every symbol their headers declare (no GPU needed)."""
+import ctypes
+import os
+import re
+
+from plaidml_amd import hipkernels as hk
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared(header):
+    text = open(os.path.join(ROOT, 'include', header)).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(pml_hip_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_kernel_library_exports_every_declared_symbol():
+    names = declared('pml_hip.h')
+    assert len(names) >= 30
+    L = hk.lib()
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(hk.EXPORTS) == names
+
+
+def test_descriptor_layouts_match():
+    L = hk.lib()
+    for which, cls in enumerate([hk.Epilogue, hk.GemmDesc, hk.Conv2dDesc, hk.Dwconv2dDesc, hk.Pool2dDesc,
+                                 hk.EltwiseDesc, hk.SelectDesc, hk.ContractDesc, hk.Form]):
+        assert L.pml_hip_struct_size(which) == ctypes.sizeof(cls), cls.__name__
+
+
+def test_dispatch_rejects_bad_descriptors_without_a_gpu():
+    L = hk.lib()
+    d = hk.GemmDesc()
+    d.in_dtype, d.out_dtype = hk.F64, hk.F64
+    assert L.pml_hip_gemm_dispatch(ctypes.byref(d)) == 0
+    assert b'in_dtype' in L.pml_hip_last_error()
+    c = hk.Conv2dDesc()
+    c.in_dtype, c.out_dtype = hk.BF16, hk.BF16
+    assert L.pml_hip_conv2d_dispatch(ctypes.byref(c)) == 0
+    assert b'geometry' in L.pml_hip_last_error()

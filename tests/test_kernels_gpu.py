@@ -1,0 +1,286 @@
+"""Parity of the HIP kernel library (called through its C ABI) against the CPU oracle.
+
+Bars: bit-exact for int8 -> int32 and for index outputs; rtol 1e-3 for fp32;
+rtol 2e-2 for bf16 (both taken from the north-star statement of this build).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import tile_oracle as E
+from oracle import tile_oplib as op
+from plaidml_amd import hipkernels as hk
+
+pytestmark = pytest.mark.gpu
+
+D = E.DType
+FP32_RTOL, BF16_RTOL = 1e-3, 2e-2
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _device():
+    hk.init(0)
+    print('device:', hk.device_name(), flush=True)
+
+
+def bf16(a):
+    return E.bf16_bits(np.asarray(a, np.float32))
+
+
+def run_gemm(A, B, in_dt, out_dt, init=None, init_strides=(0, 0), init_dt=0, tail=None, operands=(), c_dt=None,
+             extra_out=None):
+    M, K = A.shape
+    _, N = B.shape
+    d = hk.GemmDesc()
+    d.in_dtype, d.out_dtype = in_dt, out_dt
+    d.m, d.n, d.k = M, N, K
+    d.lda, d.ldb, d.ldc = K, N, N
+    d.c_dtype = c_dt if c_dt is not None else out_dt
+    if init is not None:
+        d.init_kind, d.init_dtype = 1, init_dt
+        d.init_row_stride, d.init_col_stride = init_strides
+    if tail is not None:
+        d.tail = tail
+    plan = hk.lib().pml_hip_gemm_dispatch(ctypes.byref(d))
+    assert plan, hk.lib().pml_hip_last_error()
+    print('plan:', hk.describe(plan), flush=True)
+    dA, dB = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(B)
+    np_c = {hk.F32: np.float32, hk.BF16: np.uint16, hk.I32: np.int32, hk.I8: np.int8}[d.c_dtype]
+    dC = hk.DeviceBuffer(M * N * np.dtype(np_c).itemsize)
+    dI = hk.DeviceBuffer.from_numpy(init) if init is not None else None
+    dops = [hk.DeviceBuffer.from_numpy(o) for o in operands]
+    outs = []
+    dX = None
+    if extra_out is not None:
+        dX = hk.DeviceBuffer(M * N * np.dtype(extra_out).itemsize)
+        outs = [dX.ptr]
+    hk.check(hk.lib().pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, dI.ptr if dI else None,
+                                          hk.ptr_array([o.ptr for o in dops]), hk.ptr_array(outs), None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    C = dC.to_numpy(np_c, (M, N))
+    X = dX.to_numpy(extra_out, (M, N)) if dX else None
+    hk.lib().pml_hip_plan_free(plan)
+    return (C, X) if extra_out is not None else C
+
+
+@pytest.mark.parametrize('M,N,K', [(1024, 1024, 1024), (96, 80, 40), (8, 16, 32), (257, 130, 68)])
+def test_gemm_f32(M, N, K):
+    rng = np.random.default_rng(1)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    C = run_gemm(A, B, hk.F32, hk.F32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_allclose(C, ref, rtol=FP32_RTOL, atol=1e-4)
+
+
+def test_gemm_f32_matches_oracle_contraction():
+    rng = np.random.default_rng(2)
+    Av = rng.standard_normal((8, 32)).astype(np.float32)
+    Bv = rng.standard_normal((32, 16)).astype(np.float32)
+    A, B = E.Placeholder(D.FLOAT32, Av.shape), E.Placeholder(D.FLOAT32, Bv.shape)
+    i, j, k = E.TensorIndexes(3)
+    O = E.Contraction().outShape(8, 16).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    ref, = E.run(E.Program('dot', [A, B], [O]), [Av, Bv])
+    np.testing.assert_allclose(run_gemm(Av, Bv, hk.F32, hk.F32), ref, rtol=FP32_RTOL, atol=1e-5)
+
+
+@pytest.mark.parametrize('M,N,K', [(512, 512, 512), (100, 72, 48), (4096, 4096, 4096)])
+def test_gemm_i8_bit_exact(M, N, K):
+    rng = np.random.default_rng(4)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    C = run_gemm(A, B, hk.I8, hk.I32)
+    # |acc| <= K * 127^2 < 2^31, so the int32 result equals the exact integer product
+    if M * N * K <= 1 << 27:
+        ref = A.astype(np.int64) @ B.astype(np.int64)
+        np.testing.assert_array_equal(C, ref.astype(np.int32))
+    else:
+        # full size: exact check on sampled rows / columns, and the checksum identity sum_j C[i,j] = A[i,:] . rowsum(B)
+        rows = rng.choice(M, 24, replace=False)
+        ref = A[rows].astype(np.int64) @ B.astype(np.int64)
+        np.testing.assert_array_equal(C[rows], ref.astype(np.int32))
+        cols = rng.choice(N, 24, replace=False)
+        refc = A.astype(np.int64) @ B[:, cols].astype(np.int64)
+        np.testing.assert_array_equal(C[:, cols], refc.astype(np.int32))
+        lhs = C.astype(np.int64).sum(axis=1)
+        rhs = A.astype(np.int64) @ B.astype(np.int64).sum(axis=1)
+        np.testing.assert_array_equal(lhs, rhs)
+
+
+def test_gemm_i8_requantize_tail():
+    # C = A.B (si32, stored to the extra output); Q = cast(round(clip(cast(C, f32) * S[col], -127, 127)), si8)
+    rng = np.random.default_rng(5)
+    M, N, K = 128, 96, 64
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    S = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    tail = hk.make_tail(
+        ops=[(hk.EPI_STORE, hk.I32, 0, 0, 0.0), (hk.EPI_CAST, hk.F32, 0, 0, 0.0),
+             (hk.EPI_MUL, hk.F32, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_MAX, hk.F32, hk.OPND_IMM, 0, -127.0),
+             (hk.EPI_MIN, hk.F32, hk.OPND_IMM, 0, 127.0), (hk.EPI_ROUND, hk.F32, 0, 0, 0.0),
+             (hk.EPI_CAST, hk.I8, 0, 0, 0.0)],
+        operands=[(hk.F32, 0, 1)])
+    Q, C = run_gemm(A, B, hk.I8, hk.I32, tail=tail, operands=[S], c_dt=hk.I8, extra_out=np.int32)
+    ref = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.int32)
+    np.testing.assert_array_equal(C, ref)
+    # oracle program for the epilogue
+    Cp = E.Placeholder(D.INT32, ref.shape)
+    Sp = E.Placeholder(D.FLOAT32, [N])
+    x = E.cast(Cp, D.FLOAT32) * Sp
+    x = E.select(x < -127.0, E.cast(E.Constant(-127.0), D.FLOAT32), x)
+    x = E.select(x < 127.0, x, E.cast(E.Constant(127.0), D.FLOAT32))
+    Qo, = E.run(E.Program('q', [Cp, Sp], [E.cast(E.round(x), D.INT8)]), [ref, S])
+    np.testing.assert_array_equal(Q, Qo)
+
+
+@pytest.mark.parametrize('M,N,K', [(256, 256, 256), (72, 200, 136)])
+def test_gemm_bf16(M, N, K):
+    rng = np.random.default_rng(6)
+    A = E.round_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    B = E.round_bf16(rng.standard_normal((K, N)).astype(np.float32))
+    C = run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16)
+    ref = E.round_bf16((A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+    np.testing.assert_allclose(E.bf16_from_bits(C), ref, rtol=BF16_RTOL, atol=1e-2)
+
+
+def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bias=None, relu=False, tail=None,
+             operands=()):
+    N, H, W, CI = I.shape
+    KH, KW, _, CO = F.shape
+    ph, OH = op.compute_padding_and_output_size(H, KH, stride, autopad)
+    pw, OW = op.compute_padding_and_output_size(W, KW, stride, autopad)
+    d = hk.Conv2dDesc()
+    d.in_dtype, d.out_dtype, d.c_dtype = in_dt, out_dt, out_dt
+    d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, KH, KW, CO, OH, OW
+    d.stride_h = d.stride_w = stride
+    d.dil_h = d.dil_w = 1
+    d.pad_h, d.pad_w = ph, pw
+    if bias is not None:
+        d.init_kind, d.init_dtype = 1, out_dt
+        d.init_row_stride, d.init_col_stride = 0, 1
+    if tail is not None:
+        d.tail = tail
+    elif relu:
+        d.tail = hk.make_tail(ops=[(hk.EPI_RELU, out_dt, 0, 0, 0.0)])
+    plan = hk.lib().pml_hip_conv2d_dispatch(ctypes.byref(d))
+    assert plan, hk.lib().pml_hip_last_error()
+    print('plan:', hk.describe(plan), flush=True)
+    dI, dF = hk.DeviceBuffer.from_numpy(I), hk.DeviceBuffer.from_numpy(F)
+    np_c = {hk.F32: np.float32, hk.BF16: np.uint16, hk.I32: np.int32}[out_dt]
+    dO = hk.DeviceBuffer(N * OH * OW * CO * np.dtype(np_c).itemsize)
+    dB = hk.DeviceBuffer.from_numpy(bias) if bias is not None else None
+    dops = [hk.DeviceBuffer.from_numpy(o) for o in operands]
+    hk.check(hk.lib().pml_hip_conv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, dB.ptr if dB else None,
+                                            hk.ptr_array([o.ptr for o in dops]), hk.ptr_array([]), None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    out = dO.to_numpy(np_c, (N, OH, OW, CO))
+    hk.lib().pml_hip_plan_free(plan)
+    return out
+
+
+def oracle_conv(Iv, Fv, dt, stride, autopad, bias=None, relu=False):
+    I, F = E.Placeholder(dt, Iv.shape), E.Placeholder(dt, Fv.shape)
+    ins, vals = [I, F], [Iv, Fv]
+    O = op.convolution(I, F, strides=[stride, stride], autopad=autopad)
+    if bias is not None:
+        B = E.Placeholder(dt, bias.shape)
+        ins.append(B)
+        vals.append(bias)
+        O = O + B
+    if relu:
+        O = op.relu(O)
+    out, = E.run(E.Program('conv', ins, [O]), vals)
+    return out
+
+
+@pytest.mark.parametrize('shape,k,stride,autopad', [((2, 12, 12, 32), 3, 1, op.SAME_UPPER), ((1, 9, 11, 64), 3, 2, op.SAME_UPPER),
+                                                     ((2, 8, 8, 32), 1, 1, op.VALID), ((1, 14, 14, 32), 7, 2, op.SAME_UPPER)])
+def test_conv_f32(shape, k, stride, autopad):
+    rng = np.random.default_rng(7)
+    Iv = rng.standard_normal(shape).astype(np.float32)
+    Fv = (rng.standard_normal((k, k, shape[3], 48)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(48).astype(np.float32)
+    out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, autopad=autopad, bias=bias, relu=True)
+    ref = oracle_conv(Iv, Fv, D.FLOAT32, stride, autopad, bias, True)
+    np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4)
+
+
+@pytest.mark.parametrize('shape,k,stride,co', [((2, 14, 14, 64), 3, 1, 64), ((1, 10, 10, 128), 1, 2, 72), ((2, 7, 9, 64), 3, 2, 40)])
+def test_conv_bf16(shape, k, stride, co):
+    rng = np.random.default_rng(8)
+    Iv = E.round_bf16(rng.standard_normal(shape).astype(np.float32))
+    Fv = E.round_bf16((rng.standard_normal((k, k, shape[3], co)) * np.sqrt(2.0 / (k * k * shape[3]))).astype(np.float32))
+    bias = E.round_bf16(rng.standard_normal(co).astype(np.float32))
+    out = run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=stride, bias=bf16(bias), relu=True)
+    ref = oracle_conv(Iv, Fv, D.BFLOAT16, stride, op.SAME_UPPER, bias, True)
+    np.testing.assert_allclose(E.bf16_from_bits(out), ref, rtol=BF16_RTOL, atol=1e-2)
+
+
+def test_conv_bf16_full_size_properties():
+    # BASELINE configs[1] at full size: N128 56x56x64 (*) 3x3x64x64 SAME + bias + ReLU, bf16.
+    # Size-independent checks: (a) sampled output pixels against a float64 evaluation of the
+    # definition, (b) linearity in the filter: conv(I, F1 + F2) = conv(I, F1) + conv(I, F2) up to rounding.
+    rng = np.random.default_rng(2)
+    Iv = E.round_bf16(rng.standard_normal((128, 56, 56, 64)).astype(np.float32))
+    Fv = E.round_bf16((np.random.default_rng(3).standard_normal((3, 3, 64, 64)) * np.sqrt(2.0 / 576)).astype(np.float32))
+    bias = np.zeros(64, np.float32)
+    out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bf16(bias), relu=True))
+    assert out.shape == (128, 56, 56, 64) and (out >= 0).all()
+    Ip = np.pad(Iv.astype(np.float64), ((0, 0), (1, 1), (1, 1), (0, 0)))
+    F64 = Fv.astype(np.float64)
+    pts = [(0, 0, 0), (127, 55, 55), (5, 0, 55), (77, 55, 0)] + [tuple(rng.integers(0, s) for s in (128, 56, 56)) for _ in range(60)]
+    for n, y, x in pts:
+        win = Ip[n, y:y + 3, x:x + 3, :]
+        ref = np.maximum(np.einsum('abc,abcd->d', win, F64), 0)
+        np.testing.assert_allclose(out[n, y, x], ref, rtol=BF16_RTOL, atol=2e-2)
+
+
+def test_dwconv_pool_bf16():
+    rng = np.random.default_rng(9)
+    N, H, W, C = 2, 19, 19, 32
+    Iv = E.round_bf16(rng.standard_normal((N, H, W, C)).astype(np.float32))
+    Fv = E.round_bf16((rng.standard_normal((3, 3, C, 1)) * 0.3).astype(np.float32))
+    d = hk.Dwconv2dDesc()
+    d.dtype = hk.BF16
+    d.n, d.h, d.w, d.c, d.kh, d.kw, d.oh, d.ow = N, H, W, C, 3, 3, H, W
+    d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
+    d.pad_h = d.pad_w = 1
+    plan = hk.lib().pml_hip_dwconv2d_dispatch(ctypes.byref(d))
+    assert plan, hk.lib().pml_hip_last_error()
+    dI, dF = hk.DeviceBuffer.from_numpy(bf16(Iv)), hk.DeviceBuffer.from_numpy(bf16(Fv))
+    dO = hk.DeviceBuffer(N * H * W * C * 2)
+    hk.check(hk.lib().pml_hip_dwconv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, hk.ptr_array([]), hk.ptr_array([]), None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    out = E.bf16_from_bits(dO.to_numpy(np.uint16, (N, H, W, C)))
+    I, F = E.Placeholder(D.BFLOAT16, Iv.shape), E.Placeholder(D.BFLOAT16, Fv.shape)
+    ref, = E.run(E.Program('dw', [I, F], [op.convolution(I, F, depthwise=True)]), [Iv, Fv])
+    np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
+
+    # max-pool 3x3/2 SAME with window argmax; ties forced by quantising the input
+    Pv = E.round_bf16(np.round(Iv * 2) / 2)
+    p = hk.Pool2dDesc()
+    p.dtype, p.agg = hk.BF16, hk.AGG_MAX
+    p.n, p.h, p.w, p.c, p.kh, p.kw, p.oh, p.ow = N, H, W, C, 3, 3, 10, 10
+    p.stride_h = p.stride_w = 2
+    p.pad_h = p.pad_w = 1
+    p.with_index = 1
+    plan2 = hk.lib().pml_hip_pool2d_dispatch(ctypes.byref(p))
+    assert plan2, hk.lib().pml_hip_last_error()
+    dP = hk.DeviceBuffer.from_numpy(bf16(Pv))
+    dM, dX = hk.DeviceBuffer(N * 10 * 10 * C * 2), hk.DeviceBuffer(N * 10 * 10 * C * 4)
+    hk.check(hk.lib().pml_hip_pool2d_invoke(plan2, dP.ptr, dM.ptr, dX.ptr, None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    m = E.bf16_from_bits(dM.to_numpy(np.uint16, (N, 10, 10, C)))
+    ix = dX.to_numpy(np.int32, (N, 10, 10, C))
+    R = E.Placeholder(D.BFLOAT16, Pv.shape)
+    M = op.pool(R, 'max', [3, 3], [2, 2], autopad=op.SAME_UPPER)
+    n_, x0, x1, c, k0, k1 = E.TensorIndexes(6)
+    IX = E.index([3, 3], 0) * 3 + E.index([3, 3], 1)
+    AM = E.Contraction().outShape(M.shape).outAccess(n_, x0, x1, c).max(
+        E.cond(R[n_, 2 * x0 + k0 - 1, 2 * x1 + k1 - 1, c], M[n_, x0, x1, c], IX[k0, k1])).build()
+    mo, ao = E.run(E.Program('pool', [R], [M, AM]), [Pv])
+    np.testing.assert_array_equal(m, mo)
+    np.testing.assert_array_equal(ix, ao)
+    hk.lib().pml_hip_plan_free(plan)
+    hk.lib().pml_hip_plan_free(plan2)
