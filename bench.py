@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the Tile contraction hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): conv2d NHWC via the contraction
+  O[n,y,x,co] += I[n,y+ky-1,x+kx-1,ci] * F[ky,kx,ci,co]   (N128, 56x56x64, 3x3x64x64, stride 1, SAME)
+followed by the fused bias + ReLU tail, bf16 (fp32 accumulate).  One step = one pass over the
+batch: the filter re-layout kernel plus the implicit-GEMM kernel, inputs resident in HBM.
+
+Prints ONE JSON line.  `value` is TFLOP/s over the algorithmic FLOPs (2 x valid index tuples:
+SAME-padding taps that fall outside the image are not counted).  `roofline` describes the
+dominant kernel (the implicit-GEMM conv) timed alone with HIP events; `cpu_baseline` is the
+OpenMP restatement (oracle/cpu_baseline.c) on a bounded sample of the same workload.
+`extra` carries the other single-kernel configs for information only.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {'bf16': 2500.0, 'f32': 157.3, 'i8': 5000.0}  # dense MFMA TFLOP/s (TOP/s), MI355X
+HBM_PEAK_GBS = 8000.0
+
+
+def conv_plan(hk, in_dt, N, H, W, CI, CO, KH, KW, relu=True):
+    d = hk.Conv2dDesc()
+    d.in_dtype, d.out_dtype, d.c_dtype = in_dt, in_dt, in_dt
+    d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, KH, KW, CO, H, W
+    d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
+    d.pad_h, d.pad_w = (KH - 1) // 2, (KW - 1) // 2
+    d.init_kind, d.init_dtype = 1, in_dt
+    d.init_row_stride, d.init_col_stride = 0, 1
+    if relu:
+        d.tail = hk.make_tail(ops=[(hk.EPI_RELU, in_dt, 0, 0, 0.0)])
+    plan = hk.lib().pml_hip_conv2d_dispatch(ctypes.byref(d))
+    if not plan:
+        raise RuntimeError(hk.lib().pml_hip_last_error().decode())
+    return plan
+
+
+def time_loop(hk, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    t = hk.Timer()
+    wall0 = time.perf_counter()
+    t.start()
+    for _ in range(steps):
+        fn()
+    ms = t.stop()
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    wall = (time.perf_counter() - wall0) * 1e3
+    return ms / steps, wall / steps
+
+
+def valid_taps(size, k, pad):
+    return sum(1 for x in range(size) for t in range(k) if 0 <= x + t - pad < size)
+
+
+def cpu_baseline_conv(E, N_sample, H, W, CI, CO, seed_i, seed_f, flops_per_image):
+    lib = ctypes.CDLL(os.path.join(ROOT, 'oracle', 'libcpu_baseline.so'))
+    lib.cpu_baseline_threads.restype = ctypes.c_int
+    threads = lib.cpu_baseline_threads()
+    rng = np.random.default_rng(seed_i)
+    Iv = E.round_bf16(rng.standard_normal((N_sample, H, W, CI)).astype(np.float32))
+    Fv = E.round_bf16((np.random.default_rng(seed_f).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32))
+    bias = np.zeros(CO, np.float32)
+    out = np.empty((N_sample, H, W, CO), np.float32)
+    fp = ctypes.POINTER(ctypes.c_float)
+
+    def run():
+        lib.cpu_conv2d_nhwc_f32(Iv.ctypes.data_as(fp), Fv.ctypes.data_as(fp), bias.ctypes.data_as(fp),
+                                out.ctypes.data_as(fp), N_sample, H, W, CI, 3, 3, CO, H, W, 1, 1, 1)
+
+    run()  # warm-up
+    reps, total = 0, 0.0
+    while total < 10.0 and reps < 50:
+        t0 = time.perf_counter()
+        run()
+        total += time.perf_counter() - t0
+        reps += 1
+    sec = total / reps
+    return {
+        'value': round(flops_per_image * N_sample / sec / 1e12, 5), 'unit': 'TFLOP/s', 'cores': threads, 'kind': 'port',
+        'sample': '%d of 128 images of the same conv (fp32 arithmetic on bf16-valued inputs), %d runs, OMP_NUM_THREADS=%s'
+                  % (N_sample, reps, os.environ.get('OMP_NUM_THREADS', 'unset')),
+    }, E.round_bf16(out), Iv, Fv
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--no-extra', action='store_true')
+    ap.add_argument('--no-cpu', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from oracle import tile_oracle as E  # checker: used only for the cpu_baseline leg and the spot check
+    from plaidml_amd import hipkernels as hk
+
+    hk.init(0)
+    L = hk.lib()
+    N, H, W, CI, CO = 128, 56, 56, 64, 64
+    taps = valid_taps(H, 3, 1) * valid_taps(W, 3, 1)          # valid (y,ky) x (x,kx) pairs
+    flops = 2.0 * N * taps * CI * CO
+    flops_full_box = 2.0 * N * H * W * 9 * CI * CO
+    bytes_alg = (N * H * W * CI + N * H * W * CO) * 2 + 9 * CI * CO * 2 + CO * 2
+
+    rng = np.random.default_rng(2)
+    Iv = E.round_bf16(rng.standard_normal((N, H, W, CI)).astype(np.float32))
+    Fv = E.round_bf16((np.random.default_rng(3).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32))
+    dI = hk.DeviceBuffer.from_numpy(E.bf16_bits(Iv))
+    dF = hk.DeviceBuffer.from_numpy(E.bf16_bits(Fv))
+    dB = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.uint16))
+    dO = hk.DeviceBuffer(N * H * W * CO * 2)
+    plan = conv_plan(hk, hk.BF16, N, H, W, CI, CO, 3, 3)
+    none = hk.ptr_array([])
+
+    def step():
+        hk.check(L.pml_hip_conv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, dB.ptr, none, none, None))
+
+    def kernel_only():
+        hk.check(L.pml_hip_conv2d_invoke(plan, dI.ptr, None, dO.ptr, dB.ptr, none, none, None))
+
+    ms_step, wall_step = time_loop(hk, step, args.steps, args.warmup)
+    hk.check(L.pml_hip_conv2d_pack_filter(plan, dF.ptr, None))
+    ms_kernel, _ = time_loop(hk, kernel_only, args.steps, args.warmup)
+
+    result = {
+        'metric': 'contraction TFLOP/s & % MFMA peak (GEMM/conv); ResNet-50 b128 fwd img/s',
+        'value': round(flops / (ms_step * 1e-3) / 1e12, 3),
+        'unit': 'TFLOP/s',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(ms_step, 5),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16', 'data': 'synthetic',
+        'config': {'workload': 'configs[1]: conv2d NHWC N128 56x56x64 (*) 3x3x64x64 stride 1 SAME + bias + ReLU, bf16, fp32 accumulate',
+                   'plan': hk.describe(plan), 'device': hk.device_name(),
+                   'algorithmic_gflop': round(flops / 1e9, 3), 'full_box_gflop': round(flops_full_box / 1e9, 3),
+                   'host_wall_ms_per_step': round(wall_step, 5)},
+        'roofline': {'bound': 'mfma', 'achieved': round(flops / (ms_kernel * 1e-3) / 1e12, 3), 'peak': PEAK['bf16'],
+                     'unit': 'TFLOP/s', 'frac': round(flops / (ms_kernel * 1e-3) / 1e12 / PEAK['bf16'], 4),
+                     'traffic': None, 'kernel': 'igemm_kernel<bf16, conv>', 'kernel_ms': round(ms_kernel, 5),
+                     'hbm_GBps_at_algorithmic_bytes': round(bytes_alg / (ms_kernel * 1e-3) / 1e9, 1),
+                     'hbm_frac': round(bytes_alg / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+
+    # spot check of the timed output against the CPU baseline on the sampled images
+    if not args.no_cpu:
+        n_s = 4
+        cb, ref, _, _ = cpu_baseline_conv(E, n_s, H, W, CI, CO, 2, 3, flops / N)
+        got = E.bf16_from_bits(dO.to_numpy(np.uint16, (N, H, W, CO)))[:n_s]
+        if not np.allclose(got, ref, rtol=2e-2, atol=2e-2):
+            raise SystemExit('bench: GPU output disagrees with the CPU baseline on the sampled images')
+        result['cpu_baseline'] = cb
+    else:
+        result['cpu_baseline'] = None
+
+    if not args.no_extra:
+        extra = {}
+        # configs[1], fp32 variant
+        dI32 = hk.DeviceBuffer.from_numpy(Iv)
+        dF32 = hk.DeviceBuffer.from_numpy(Fv)
+        dB32 = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.float32))
+        dO32 = hk.DeviceBuffer(N * H * W * CO * 4)
+        p32 = conv_plan(hk, hk.F32, N, H, W, CI, CO, 3, 3)
+        ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_conv2d_invoke(p32, dI32.ptr, dF32.ptr, dO32.ptr, dB32.ptr, none, none, None)),
+                          max(5, args.steps // 5), 3)
+        extra['conv_f32_configs1'] = {'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2),
+                                      'frac_mfma_f32': round(flops / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(p32)}
+        for b in (dI32, dF32, dB32, dO32):
+            b.free()
+        # configs[0]: fp32 GEMM 1024^3
+        g = hk.GemmDesc()
+        g.in_dtype = g.out_dtype = g.c_dtype = hk.F32
+        g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 1024
+        pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+        A = np.random.default_rng(1).uniform(-1, 1, (1024, 1024)).astype(np.float32)
+        dA, dBm, dC = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(A.T.copy()), hk.DeviceBuffer(4 << 20)
+        ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dA.ptr, dBm.ptr, dC.ptr, None, none, none, None)), 50, 10)
+        extra['gemm_f32_1024_configs0'] = {'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2),
+                                           'frac_mfma_f32': round(2 * 1024 ** 3 / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(pg)}
+        # configs[2]: int8 GEMM 4096^3 -> int32
+        g = hk.GemmDesc()
+        g.in_dtype, g.out_dtype, g.c_dtype = hk.I8, hk.I32, hk.I32
+        g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 4096
+        pi = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+        Ai = np.random.default_rng(4).integers(-127, 128, (4096, 4096), dtype=np.int8)
+        dAi, dBi, dCi = hk.DeviceBuffer.from_numpy(Ai), hk.DeviceBuffer.from_numpy(Ai.T.copy()), hk.DeviceBuffer(4096 * 4096 * 4)
+        ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pi, dAi.ptr, dBi.ptr, dCi.ptr, None, none, none, None)), 20, 5)
+        extra['gemm_i8_4096_configs2'] = {'ms': round(ms, 4), 'TOP/s': round(2 * 4096 ** 3 / ms / 1e9, 2),
+                                          'frac_mfma_i8': round(2 * 4096 ** 3 / ms / 1e9 / PEAK['i8'], 4), 'plan': hk.describe(pi)}
+        result['extra'] = extra
+
+    print(json.dumps(result))
+
+
+if __name__ == '__main__':
+    main()

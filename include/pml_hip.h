@@ -176,6 +176,10 @@ typedef struct {
 int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* desc); /* 0 on failure */
 int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, const void* init,
                         const void* const* operands, void* const* outs, pml_hip_stream s);
+/* Right-hand sides that are constants of the program (weights) are re-laid-out once, the way the
+ * reference runs its `init` closure once when the executable is built
+ * (pmlc/rt/jit_executable.cc:404-418): after pack_b, invoke may be given b == NULL. */
+int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s);
 
 /* ---- dense contraction: 2-D convolution, NHWC (x) HWCK ------------------------
  * O[n,y,x,co] = tail( init + sum_{ky,kx,ci} I[n, sy*y + dy*ky - py, sx*x + dx*kx - px, ci] * F[ky,kx,ci,co] )
@@ -205,6 +209,8 @@ typedef struct {
 int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* desc);
 int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, void* output, const void* init,
                           const void* const* operands, void* const* outs, pml_hip_stream s);
+/* Same as pml_hip_gemm_pack_b for a constant filter: afterwards invoke may be given filter == NULL. */
+int pml_hip_conv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream s);
 
 /* ---- depthwise 2-D convolution, NHWC, channel multiplier 1 --------------------
  * O[n,y,x,c] = tail( sum_{ky,kx} I[n, sy*y + ky - py, sx*x + kx - px, c] * F[ky,kx,c,0] )

@@ -42,6 +42,7 @@ struct Plan {
   void* bt = nullptr;
   int64_t bt_ld = 0;
   size_t bt_bytes = 0;
+  bool packed = false;
   std::string text;
   ~Plan() {
     if (bt) (void)hipFree(bt);
@@ -255,11 +256,12 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
   const pml_hip_gemm_desc& d = p->gemm;
-  if (!a || !b || !c) return fail("gemm_invoke: null operand");
+  if (!a || !c) return fail("gemm_invoke: null operand");
+  if (!b && !p->packed) return fail("gemm_invoke: b is null and no packed right-hand side exists");
   if (((uintptr_t)a & 15) != 0) return fail("gemm_invoke: A must be 16-byte aligned");
   if (d.init_kind && !init) return fail("gemm_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
-  if (check(transpose_pack(es, b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack")) return 1;
+  if (b && check(transpose_pack(es, b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack")) return 1;
   IgemmArgs g;
   std::memset(&g, 0, sizeof g);
   g.M = d.m;
@@ -356,13 +358,15 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_CONV) return fail("conv2d_invoke: not a conv2d plan");
   const pml_hip_conv2d_desc& d = p->conv;
-  if (!input || !filter || !output) return fail("conv2d_invoke: null operand");
+  if (!input || !output) return fail("conv2d_invoke: null operand");
+  if (!filter && !p->packed) return fail("conv2d_invoke: filter is null and no packed filter exists");
   if (((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
   if (d.init_kind && !init) return fail("conv2d_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
   const int64_t K = d.kh * d.kw * d.ci;
   // the HWCK filter is a row-major [K][CO] matrix
-  if (check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack")) return 1;
+  if (filter && check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
+    return 1;
   IgemmArgs g;
   std::memset(&g, 0, sizeof g);
   g.M = d.n * d.oh * d.ow;
@@ -403,6 +407,27 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("conv2d_invoke: missing extra output");
   return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
+}
+
+int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_GEMM || !b) return fail("gemm_pack_b: bad argument");
+  const pml_hip_gemm_desc& d = p->gemm;
+  if (check(transpose_pack(dt_size(d.in_dtype), b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack"))
+    return 1;
+  p->packed = true;
+  return 0;
+}
+
+int pml_hip_conv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_CONV || !filter) return fail("conv2d_pack_filter: bad argument");
+  const pml_hip_conv2d_desc& d = p->conv;
+  const int64_t K = d.kh * d.kw * d.ci;
+  if (check(transpose_pack(dt_size(d.in_dtype), filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
+    return 1;
+  p->packed = true;
+  return 0;
 }
 
 // ---------------------------------------------------------------------------

@@ -31,7 +31,7 @@ EXPORTS = [
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
-    'pml_hip_plan_describe', 'pml_hip_struct_size',
+    'pml_hip_plan_describe', 'pml_hip_struct_size', 'pml_hip_gemm_pack_b', 'pml_hip_conv2d_pack_filter',
 ]
 
 i32, i64, f64 = ctypes.c_int32, ctypes.c_int64, ctypes.c_double
@@ -135,6 +135,8 @@ def lib():
         L.pml_hip_plan_free.argtypes = [ctypes.c_int64]
         L.pml_hip_plan_describe.argtypes = [ctypes.c_int64, ctypes.c_char_p, sz]
         L.pml_hip_struct_size.restype = sz
+        L.pml_hip_gemm_pack_b.argtypes = [ctypes.c_int64, vp, vp]
+        L.pml_hip_conv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
         _lib = L
     return _lib
 
