@@ -10,8 +10,10 @@
 //   int8: one  v_mfma_i32_32x32x32_i8
 //   fp32: four v_mfma_f32_32x32x2_f32   (the k order inside a block is permuted
 //         identically for A and Bt, which leaves the sum unchanged)
-// 256 threads = 4 wavefronts in a 2x2 grid; LDS is double-buffered and the next
-// slab travels global -> registers while the current one feeds the MFMAs.
+// 256 threads = 4 wavefronts; LDS is double-buffered and the next slab travels
+// global -> registers while the current one feeds the MFMAs.  After the K loop
+// the accumulator tile is staged through LDS so that the tail runs once per
+// element in row-major order and stores are contiguous 8/16-byte pieces.
 #include <hip/hip_runtime.h>
 
 #include "device_common.h"
@@ -27,8 +29,8 @@ hipError_t igemm_launch_kind_2(int cfg, bool conv, const IgemmArgs& a, hipStream
 
 namespace {
 
-constexpr int kSlabBytes = 128;                // bytes of K per LDS row
-constexpr int kRowStride = kSlabBytes + 16;    // padded LDS row (16B-slot skew: conflict-free b128 reads)
+constexpr int kSlabBytes = 128;              // bytes of K per LDS row
+constexpr int kRowStride = kSlabBytes + 16;  // padded LDS row (16B-slot skew: conflict-free b128 reads)
 constexpr int kThreads = 256;
 
 template <int KIND>
@@ -81,108 +83,24 @@ __device__ inline int xcd_remap(int bid, int nblocks) {
   return (bid % kXcds) * per + (bid / kXcds);
 }
 
-// Applies init + tail to one 32x32 accumulator block staged in LDS (row stride
-// 33 words) and stores it.  Lane l handles rows l/8 + 8*it, columns 4*(l%8)..+3.
-template <int KIND>
-__device__ __attribute__((noinline)) void tail_block(const IgemmArgs& p, const typename Acc<KIND>::scalar* patch,
-                                                     int64_t m_base, int64_t n_base, int lane) {
-  const int c4 = (lane & 7) * 4;
-  const int64_t n = n_base + c4;
-  if (n >= p.N) return;
-  const bool fast = p.tail_mode == 1 && n + 3 < p.N && (p.ldc & 3) == 0;
-  for (int it = 0; it < 4; ++it) {
-    const int row = it * 8 + (lane >> 3);
-    const int64_t m = m_base + row;
-    if (m >= p.M) continue;
-    if (fast) {
-      // (optional init) -> round to the result type -> (optional relu) -> one vector store
-      if (KIND == KIND_I8) {
-        i32x4_t v;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          int iv = (int)patch[row * 33 + c4 + q];
-          if (p.init) iv += load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype).i;
-          if (p.tail_relu) iv = iv < 0 ? 0 : iv;
-          v[q] = iv;
-        }
-        *(i32x4_t*)((int*)p.C + m * p.ldc + n) = v;
-      } else {
-        float f[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float fv = (float)patch[row * 33 + c4 + q];
-          if (p.init) fv += load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype).f;
-          f[q] = fv;
-        }
-        if (p.out_dtype == PML_HIP_BF16) {
-          uint16_t h[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            h[q] = f32_to_bf16_bits(f[q]);
-            if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
-          }
-          uint2 w = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
-          *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = w;
-        } else {
-          f32x4_t v;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] = (p.tail_relu && f[q] < 0.f) ? 0.f : f[q];
-          *(f32x4_t*)((float*)p.C + m * p.ldc + n) = v;
-        }
-      }
-      continue;
-    }
-    for (int q = 0; q < 4; ++q) {
-      if (n + q >= p.N) break;
-      Scalar<float, int> v;
-      v.f = 0;
-      v.i = 0;
-      int cur = p.out_dtype;
-      const int64_t nn = n + q;
-      if (KIND == KIND_I8) {
-        int iv = (int)patch[row * 33 + c4 + q];
-        if (p.init) iv += load_scalar<float, int>(p.init, m * p.init_rs + nn * p.init_cs, p.init_dtype).i;
-        v.i = iv;
-      } else {
-        float fv = (float)patch[row * 33 + c4 + q];
-        if (p.init) fv += load_scalar<float, int>(p.init, m * p.init_rs + nn * p.init_cs, p.init_dtype).f;
-        v.f = round_float_to<float>(cur, fv);
-      }
-      const int64_t o = m * p.ldc + nn;
-      if (p.tail_mode == 1) {
-        if (p.tail_relu) {
-          if (KIND == KIND_I8)
-            v.i = v.i < 0 ? 0 : v.i;
-          else
-            v.f = v.f < 0.f ? 0.f : v.f;
-        }
-      } else {
-        int64_t off[PML_HIP_MAX_EPI_OPERANDS];
-        for (int k = 0; k < PML_HIP_MAX_EPI_OPERANDS; ++k)
-          off[k] = k < p.tail.n_operands ? m * p.tail.operand_row_stride[k] + nn * p.tail.operand_col_stride[k] : 0;
-        v = run_tail<float, int>(p.tail, v, &cur, p.operands, off, p.outs, o);
-      }
-      store_scalar<float, int>(p.C, o, cur, v);
-    }
-  }
-}
-
-template <int KIND, int BM, int BN, bool CONV>
+// BM x BN output tile, WAVES_M x WAVES_N wavefront grid (WAVES_M * WAVES_N == 4).
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV>
 __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
-  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int WAVES_N = 4 / WAVES_M;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int MI = WM / 32, NI = WN / 32;
   constexpr int A_VECS = BM * 8 / kThreads;  // 16-byte vectors per thread per slab
   constexpr int B_VECS = BN * 8 / kThreads;
+  constexpr int kStage = (BM + BN) * kRowStride;  // one buffer: A rows then Bt rows
   typedef typename Acc<KIND>::type acc_t;
   typedef typename Acc<KIND>::scalar accs_t;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  constexpr int kStage = (BM + BN) * kRowStride;  // one buffer: A rows then Bt rows
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   const int tiles_n = (int)((p.N + BN - 1) / BN);
   const int tiles_m = (int)((p.M + BM - 1) / BM);
@@ -190,32 +108,30 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   const int64_t m0 = (int64_t)(tile / tiles_n) * BM;
   const int64_t n0 = (int64_t)(tile % tiles_n) * BN;
 
-  // ---- per-thread load assignments (fixed across slabs) ----
-  // vector v of row r:  r = tid/8 + 32*i,  v = tid%8
+  // ---- per-thread load assignments (fixed across slabs): vector lv of rows lr + 32*i ----
   const int lv = tid & 7;
   const int lr = tid >> 3;
-  const int64_t kbytes_total = p.K * ES;  // GEMM: bytes per A row;  CONV: CI*ES bytes per tap
+  const int kbytes_row = (int)(CONV ? p.CI * ES : p.K * ES);  // valid bytes per (tap) row
 
-  // A rows
-  const unsigned char* a_row[A_VECS];
+  const unsigned char* a_row[A_VECS];  // GEMM: row start; CONV: image start
   bool a_ok[A_VECS];
   int a_ih0[A_VECS], a_iw0[A_VECS];
 #pragma unroll
   for (int i = 0; i < A_VECS; ++i) {
     const int64_t m = m0 + lr + 32 * i;
     a_ok[i] = m < p.M;
+    const int64_t mm = a_ok[i] ? m : 0;
     if (CONV) {
-      const int64_t mm = a_ok[i] ? m : 0;
       const int ow = (int)(mm % p.OW);
       const int64_t t = mm / p.OW;
       const int oh = (int)(t % p.OH);
       const int64_t nb = t / p.OH;
       a_ih0[i] = oh * p.SH - p.PH;
       a_iw0[i] = ow * p.SW - p.PW;
-      a_row[i] = (const unsigned char*)p.A + nb * p.H * p.W * p.CI * ES;
+      a_row[i] = (const unsigned char*)p.A + nb * ((int64_t)p.H * p.W * p.CI * ES);
     } else {
       a_ih0[i] = a_iw0[i] = 0;
-      a_row[i] = (const unsigned char*)p.A + (a_ok[i] ? m : 0) * p.lda * ES;
+      a_row[i] = (const unsigned char*)p.A + mm * p.lda * ES;
     }
   }
   const unsigned char* b_row[B_VECS];
@@ -227,58 +143,60 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
     b_row[i] = (const unsigned char*)p.Bt + (b_ok[i] ? n : 0) * p.ldbt * ES;
   }
 
-  // number of slabs: GEMM ceil(K*ES/128); CONV taps * ceil(CI*ES/128)
-  const int slabs_per_tap = CONV ? (int)((p.CI * ES + kSlabBytes - 1) / kSlabBytes) : 0;
-  const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : (int)((kbytes_total + kSlabBytes - 1) / kSlabBytes);
+  const int slabs_per_tap = (kbytes_row + kSlabBytes - 1) / kSlabBytes;
+  const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : slabs_per_tap;
+  const int pix_bytes = p.CI * ES;
 
   i32x4_t ra[A_VECS], rb[B_VECS];
+  const i32x4_t zero4 = {0, 0, 0, 0};
 
+  // Loads are unconditional from a clamped (always valid) address; the value is
+  // replaced by zero afterwards when the element is outside the problem.
   auto load_slab = [&](int s) {
     if (CONV) {
       const int tap = s / slabs_per_tap;
       const int cs = s - tap * slabs_per_tap;
       const int kh = tap / p.KW, kw = tap - kh * p.KW;
-      const int64_t cb = (int64_t)cs * kSlabBytes + lv * 16;  // byte offset inside the channel vector
-      const bool c_ok = cb < p.CI * ES;
+      const int cb = cs * kSlabBytes + lv * 16;  // byte offset inside the channel vector
+      const bool c_ok = cb < kbytes_row;
+      const int cbs = c_ok ? cb : 0;
+      const int dh = kh * p.DH, dw = kw * p.DW;
 #pragma unroll
       for (int i = 0; i < A_VECS; ++i) {
-        const int ih = a_ih0[i] + kh * p.DH, iw = a_iw0[i] + kw * p.DW;
-        const bool ok = a_ok[i] && c_ok && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-        i32x4_t v = {0, 0, 0, 0};
-        if (ok) v = *(const i32x4_t*)(a_row[i] + ((int64_t)ih * p.W + iw) * p.CI * ES + cb);
-        ra[i] = v;
+        const int ih = a_ih0[i] + dh, iw = a_iw0[i] + dw;
+        const bool ok = a_ok[i] && c_ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+        const int off = ok ? (ih * p.W + iw) * pix_bytes + cbs : 0;
+        const i32x4_t v = *(const i32x4_t*)(a_row[i] + off);
+        ra[i] = ok ? v : zero4;
       }
-      // Bt row n holds K = taps*CI elements: tap-major, channel-minor
-      const int64_t kb = ((int64_t)tap * p.CI) * ES + cb;
+      const int kb = tap * pix_bytes + cbs;  // Bt row: tap-major, channel-minor
 #pragma unroll
       for (int i = 0; i < B_VECS; ++i) {
-        i32x4_t v = {0, 0, 0, 0};
-        if (b_ok[i] && c_ok) v = *(const i32x4_t*)(b_row[i] + kb);
-        rb[i] = v;
+        const i32x4_t v = *(const i32x4_t*)(b_row[i] + kb);
+        rb[i] = (b_ok[i] && c_ok) ? v : zero4;
       }
     } else {
-      const int64_t kb = (int64_t)s * kSlabBytes + lv * 16;
-      const bool k_ok = kb < kbytes_total;
+      const int kb = s * kSlabBytes + lv * 16;
+      const bool k_ok = kb < kbytes_row;
+      const int kbs = k_ok ? kb : 0;
 #pragma unroll
       for (int i = 0; i < A_VECS; ++i) {
-        i32x4_t v = {0, 0, 0, 0};
-        if (a_ok[i] && k_ok) v = *(const i32x4_t*)(a_row[i] + kb);
-        ra[i] = v;
+        const i32x4_t v = *(const i32x4_t*)(a_row[i] + kbs);
+        ra[i] = (a_ok[i] && k_ok) ? v : zero4;
       }
 #pragma unroll
       for (int i = 0; i < B_VECS; ++i) {
-        i32x4_t v = {0, 0, 0, 0};
-        if (b_ok[i] && k_ok) v = *(const i32x4_t*)(b_row[i] + kb);
-        rb[i] = v;
+        const i32x4_t v = *(const i32x4_t*)(b_row[i] + kbs);
+        rb[i] = (b_ok[i] && k_ok) ? v : zero4;
       }
     }
   };
   auto store_slab = [&](int buf) {
+    unsigned char* base = smem + buf * kStage + lr * kRowStride + lv * 16;
 #pragma unroll
-    for (int i = 0; i < A_VECS; ++i) *(i32x4_t*)(smem + buf * kStage + (lr + 32 * i) * kRowStride + lv * 16) = ra[i];
+    for (int i = 0; i < A_VECS; ++i) *(i32x4_t*)(base + (32 * i) * kRowStride) = ra[i];
 #pragma unroll
-    for (int i = 0; i < B_VECS; ++i)
-      *(i32x4_t*)(smem + buf * kStage + (BM + lr + 32 * i) * kRowStride + lv * 16) = rb[i];
+    for (int i = 0; i < B_VECS; ++i) *(i32x4_t*)(base + (BM + 32 * i) * kRowStride) = rb[i];
   };
 
   acc_t acc[MI][NI];
@@ -293,7 +211,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   store_slab(0);
   __syncthreads();
 
-  const int frow = lane & 31;   // row of the 32x32 block this lane feeds
+  const int frow = lane & 31;       // row of the 32x32 block this lane feeds
   const int fk = (lane >> 5) * 16;  // its 16-byte half of a 32-byte K-block
 
   for (int s = 0; s < n_slabs; ++s) {
@@ -317,23 +235,112 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
     __syncthreads();
   }
 
-  // ---- tail and store.  In a 32x32 block a lane owns column lane%32 and rows
-  // 8*(r/4) + 4*(lane/32) + r%4 for r in [0,16).  Each block is staged through
-  // this wavefront's private LDS patch so that a lane then owns four consecutive
-  // columns of one row: stores are 8/16-byte pieces of contiguous row segments,
-  // and the tail code exists once instead of once per accumulator register.
-  accs_t* patch = (accs_t*)(smem + wave * (32 * 33 * 4));
-  const int ccol = lane & 31;
-  const int crow = (lane >> 5) * 4;
+  // ---- stage the accumulator tile in LDS as ctile[BM][BN + 4] ----
+  // In a 32x32 block a lane owns column lane%32 and rows 8*(r/4) + 4*(lane/32) + r%4.
+  constexpr int CS = BN + 4;
+  static_assert((size_t)BM * CS * 4 <= 2 * (size_t)kStage, "accumulator tile must fit in the pipeline buffers");
+  accs_t* ctile = (accs_t*)smem;
+  {
+    const int ccol = lane & 31;
+    const int crow = (lane >> 5) * 4;
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      __syncthreads();
+      for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) patch[(8 * (r >> 2) + crow + (r & 3)) * 33 + ccol] = acc[i][j][r];
-      __syncthreads();
-      tail_block<KIND>(p, patch, m0 + wm * WM + i * 32, n0 + wn * WN + j * 32, lane);
+        for (int r = 0; r < 16; ++r)
+          ctile[(wm * WM + i * 32 + 8 * (r >> 2) + crow + (r & 3)) * CS + wn * WN + j * 32 + ccol] = acc[i][j][r];
+  }
+  __syncthreads();
+
+  // ---- tail and store: a thread owns 4 consecutive columns, rows advance by RPP per pass ----
+  constexpr int TPR = BN / 4;
+  constexpr int RPP = kThreads / TPR;
+  const int c4 = (tid % TPR) * 4;
+  const int64_t n = n0 + c4;
+  if (n >= p.N) return;
+  const bool full4 = n + 3 < p.N;
+  const bool fast = p.tail_mode == 1 && full4 && (p.ldc & 3) == 0;
+  // a per-column start value (bias) is the same for every row of this thread
+  const bool col_init = p.init != nullptr && p.init_rs == 0;
+  accs_t cinit[4] = {0, 0, 0, 0};
+  if (col_init) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (n + q < p.N) {
+        Scalar<float, int> b = load_scalar<float, int>(p.init, (n + q) * p.init_cs, p.init_dtype);
+        cinit[q] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+      }
+    }
+  }
+  for (int row = tid / TPR; row < BM; row += RPP) {
+    const int64_t m = m0 + row;
+    if (m >= p.M) break;
+    accs_t v4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v4[q] = ctile[row * CS + c4 + q];
+    if (col_init) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v4[q] += cinit[q];
+    } else if (p.init) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (n + q < p.N) {
+          Scalar<float, int> b = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
+          v4[q] += KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+        }
+      }
+    }
+    if (fast) {
+      if (KIND == KIND_I8) {
+        i32x4_t w;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) w[q] = (p.tail_relu && (int)v4[q] < 0) ? 0 : (int)v4[q];
+        *(i32x4_t*)((int*)p.C + m * p.ldc + n) = w;
+      } else if (p.out_dtype == PML_HIP_BF16) {
+        uint32_t h[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          h[q] = f32_to_bf16_bits((float)v4[q]);
+          // relu on the rounded value: negative, non-NaN, non-zero -> 0  (x < 0 ? 0 : x)
+          if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
+        }
+        *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+      } else {
+        f32x4_t w;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) w[q] = (p.tail_relu && (float)v4[q] < 0.f) ? 0.f : (float)v4[q];
+        *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
+      }
+      continue;
+    }
+    for (int q = 0; q < 4; ++q) {
+      if (n + q >= p.N) break;
+      const int64_t nn = n + q;
+      Scalar<float, int> v;
+      v.f = 0;
+      v.i = 0;
+      int cur = p.out_dtype;
+      if (KIND == KIND_I8)
+        v.i = (int)v4[q];
+      else
+        v.f = round_float_to<float>(cur, (float)v4[q]);
+      const int64_t o = m * p.ldc + nn;
+      if (p.tail_mode == 1) {
+        if (p.tail_relu) {
+          if (KIND == KIND_I8)
+            v.i = v.i < 0 ? 0 : v.i;
+          else
+            v.f = v.f < 0.f ? 0.f : v.f;
+        }
+      } else {
+        int64_t off[PML_HIP_MAX_EPI_OPERANDS];
+#pragma unroll
+        for (int k = 0; k < PML_HIP_MAX_EPI_OPERANDS; ++k)
+          off[k] = k < p.tail.n_operands ? m * p.tail.operand_row_stride[k] + nn * p.tail.operand_col_stride[k] : 0;
+        v = run_tail<float, int>(p.tail, v, &cur, p.operands, off, p.outs, o);
+      }
+      store_scalar<float, int>(p.C, o, cur, v);
     }
   }
 }
@@ -356,11 +363,11 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ B,
   }
 }
 
-template <int KIND, int BM, int BN, bool CONV>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
-  auto kern = igemm_kernel<KIND, BM, BN, CONV>;
+  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -374,10 +381,10 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
 template <int KIND, bool CONV>
 hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
   switch (cfg) {
-    case TILE_128x128: return launch_cfg<KIND, 128, 128, CONV>(a, s);
-    case TILE_128x64: return launch_cfg<KIND, 128, 64, CONV>(a, s);
-    case TILE_256x64: return launch_cfg<KIND, 256, 64, CONV>(a, s);
-    case TILE_64x64: return launch_cfg<KIND, 64, 64, CONV>(a, s);
+    case TILE_128x128: return launch_cfg<KIND, 128, 128, 2, CONV>(a, s);
+    case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
+    case TILE_256x64: return launch_cfg<KIND, 256, 64, 4, CONV>(a, s);
+    case TILE_64x64: return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);
   }
   return hipErrorInvalidValue;
 }
@@ -421,7 +428,6 @@ hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int
   }
   return hipGetLastError();
 }
-
 #endif  // PML_KIND == 0
 
 }  // namespace pml

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -72,13 +73,18 @@ const char* tile_name(int t) {
 // flight (one wave of the grid); prefer the largest tile that still yields
 // about two workgroups per CU, and never a tile wider than N.
 int choose_tile(int64_t m, int64_t n) {
+  // PML_HIP_TILE=128x128|128x64|256x64|64x64 overrides the table (for tuning runs)
+  if (const char* e = std::getenv("PML_HIP_TILE")) {
+    const std::string v(e);
+    if (v == "128x128") return TILE_128x128;
+    if (v == "128x64") return TILE_128x64;
+    if (v == "256x64" && n <= 64) return TILE_256x64;
+    if (v == "64x64") return TILE_64x64;
+  }
   auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   const int64_t want = 2 * 256;
-  if (n <= 64) {
-    if (tiles(256, 64) >= want) return TILE_256x64;
-    if (tiles(128, 64) >= 256) return TILE_128x64;
-    return TILE_64x64;
-  }
+  if (n <= 64) return TILE_64x64;  // measured on N128 56x56x64 (*) 3x3x64x64: 64x64 93 us, 128x64 111 us, 256x64 161 us
+  (void)want;
   if (tiles(128, 128) >= want) return TILE_128x128;
   if (tiles(128, 64) >= 256) return TILE_128x64;
   return TILE_64x64;
@@ -322,7 +328,8 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     fail("conv2d: input channels must cover whole 16-byte vectors");
     return 0;
   }
-  if (d->n * d->h * d->w * d->ci >= ((int64_t)1 << 40) || d->h * d->w > (1 << 30)) {
+  if (d->n * d->h * d->w * d->ci >= ((int64_t)1 << 40) || d->h * d->w * d->ci * es >= ((int64_t)1 << 31) ||
+      d->kh * d->kw * d->ci * es >= ((int64_t)1 << 31)) {
     fail("conv2d: tensor too large");
     return 0;
   }
