@@ -1,0 +1,159 @@
+// The operation library for C++: the subset of the reference's builders
+// (plaidml/op/op.h:28-1003) that the contraction hot path uses -- convolution,
+// pool, dot, relu, mean / sum / max / min reductions, softmax, argmax, clip,
+// maximum, minimum -- with the same names, argument order and defaults.  Each
+// call goes through plaidml_op_make and emits EDSL contractions / elementwise
+// operations.
+#pragma once
+
+#include <string>
+#include <vector>
+
+#include "plaidml/edsl/edsl.h"
+#include "plaidml/op/ffi.h"
+
+namespace plaidml {
+namespace op {
+
+inline void init() {
+  plaidml::init();
+  plaidml::edsl::init();
+}
+
+namespace details {
+inline edsl::Value op(const std::string& name, const edsl::Value& args) {
+  return edsl::Value(ffi::call<plaidml_value*>(plaidml_op_make, name.c_str(), args.as_ptr()));
+}
+}  // namespace details
+
+enum class AutoGroupMode { UNGROUPED, EXPLICIT, AUTO, DEPTHWISE, _LAST };
+enum class AutoPadMode { EXPLICIT, SAME_LOWER, SAME_UPPER, VALID, _LAST };
+enum class ConvDerivMode { NONE, DATA, FILTER, _LAST };
+enum class GroupLayout { NONE, SEPARATE, IN_C, IN_K, _LAST };
+enum class PoolMode { AVG, MAX, MIN, SUM, _LAST };
+enum class TensorLayout { NXC, NCX, KCX, XCK, GKCX, XGCK, _LAST };
+
+// a list of integers accepted from vectors and brace lists of the usual integer types
+struct Integers {
+  Integers(const std::vector<int>& elts) : value(edsl::make_tuple(elts)) {}                       // NOLINT
+  Integers(const std::vector<int64_t>& elts) : value(edsl::make_tuple(elts)) {}                   // NOLINT
+  Integers(const std::vector<size_t>& elts)                                                        // NOLINT
+      : value(edsl::make_tuple(std::vector<int64_t>(elts.begin(), elts.end()))) {}
+  Integers(const std::initializer_list<int>& elts) : Integers(std::vector<int>(elts)) {}           // NOLINT
+  Integers(const std::initializer_list<int64_t>& elts) : Integers(std::vector<int64_t>(elts)) {}   // NOLINT
+  Integers(const std::initializer_list<size_t>& elts) : Integers(std::vector<size_t>(elts)) {}     // NOLINT
+  edsl::Value value;
+};
+
+inline edsl::Tensor argmax(const edsl::Tensor& I, const edsl::Value& axes = edsl::None()) {
+  return details::op("argmax", edsl::make_tuple(I, axes)).as_tensor();
+}
+
+inline edsl::Tensor clip(const edsl::Tensor& I, const edsl::Tensor& min, const edsl::Tensor& max) {
+  return details::op("clip", edsl::make_tuple(I, min, max)).as_tensor();
+}
+
+// NXC (x) XCK forward convolution; defaults: stride 1, no dilation, SAME_UPPER padding, ungrouped
+class convolution {
+ public:
+  explicit convolution(edsl::Tensor I, edsl::Tensor F) : I_(I), F_(F) {}
+  convolution& strides(Integers elts) { strides_ = elts.value; return *this; }
+  convolution& dilations(Integers elts) { dilations_ = elts.value; return *this; }
+  convolution& data_dilations(Integers elts) { data_dilations_ = elts.value; return *this; }
+  convolution& filter_shape(Integers elts) { filter_shape_ = elts.value; return *this; }
+  convolution& groups(int groups) { groups_ = groups; return *this; }
+  convolution& manual_padding(Integers elts) { manual_padding_ = elts.value; return *this; }
+  convolution& autopad_mode(AutoPadMode mode) { autopad_mode_ = mode; return *this; }
+  convolution& input_layout(TensorLayout layout) { input_layout_ = layout; return *this; }
+  convolution& filter_layout(TensorLayout layout) { filter_layout_ = layout; return *this; }
+  convolution& group_layout(GroupLayout layout) { group_layout_ = layout; return *this; }
+  convolution& winograd_allowed(bool allowed) { winograd_allowed_ = allowed; return *this; }
+  convolution& name(const std::string& name) { name_ = name; return *this; }
+  convolution& autogroup_mode(AutoGroupMode mode) { autogroup_mode_ = mode; return *this; }
+  convolution& deriv_mode(ConvDerivMode mode) { deriv_mode_ = mode; return *this; }
+  convolution& result_shape(Integers elts) { result_shape_ = elts.value; return *this; }
+  convolution& infer_result_shape(bool infer) { infer_result_shape_ = infer; return *this; }
+
+  operator edsl::Tensor() const {  // NOLINT
+    auto args = edsl::make_tuple(I_, F_, strides_, dilations_, data_dilations_, filter_shape_, groups_,
+                                 static_cast<int>(autopad_mode_), manual_padding_, static_cast<int>(input_layout_),
+                                 static_cast<int>(filter_layout_), static_cast<int>(group_layout_), winograd_allowed_, name_,
+                                 static_cast<int>(autogroup_mode_), static_cast<int>(deriv_mode_), result_shape_,
+                                 infer_result_shape_);
+    return details::op("convolution", args).as_tensor();
+  }
+
+ private:
+  edsl::Tensor I_, F_;
+  edsl::Value strides_, dilations_, data_dilations_, filter_shape_;
+  int groups_ = 1;
+  edsl::Value manual_padding_;
+  AutoPadMode autopad_mode_ = AutoPadMode::SAME_UPPER;
+  TensorLayout input_layout_ = TensorLayout::NXC;
+  TensorLayout filter_layout_ = TensorLayout::XCK;
+  GroupLayout group_layout_ = GroupLayout::NONE;
+  bool winograd_allowed_ = false;
+  std::string name_;
+  AutoGroupMode autogroup_mode_ = AutoGroupMode::UNGROUPED;
+  ConvDerivMode deriv_mode_ = ConvDerivMode::NONE;
+  edsl::Value result_shape_;
+  bool infer_result_shape_ = false;
+};
+
+inline edsl::Tensor dot(const edsl::Tensor& I, const edsl::Tensor& K, const std::string& name = "") {
+  return details::op("dot", edsl::make_tuple(I, K, name)).as_tensor();
+}
+
+inline edsl::Tensor max(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {  // NOLINT
+  return details::op("max", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+inline edsl::Tensor maximum(const edsl::Tensor& X, const edsl::Tensor& Y) {
+  return details::op("maximum", edsl::make_tuple(X, Y)).as_tensor();
+}
+inline edsl::Tensor mean(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
+  return details::op("mean", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+inline edsl::Tensor min(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {  // NOLINT
+  return details::op("min", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+inline edsl::Tensor minimum(const edsl::Tensor& X, const edsl::Tensor& Y) {
+  return details::op("minimum", edsl::make_tuple(X, Y)).as_tensor();
+}
+
+inline edsl::Tensor pool(const edsl::Tensor I, PoolMode pool_mode, const std::vector<int>& pool_size,
+                         const std::vector<int>& strides, AutoPadMode autopad_mode, const std::vector<int>& manual_padding,
+                         TensorLayout input_layout, bool include_padding_in_avg = false,
+                         bool use_ceil_for_output_shape = false, const std::string& name = "") {
+  auto args = edsl::make_tuple(I, static_cast<int>(pool_mode), edsl::make_tuple(pool_size), edsl::make_tuple(strides),
+                               static_cast<int>(autopad_mode), edsl::make_tuple(manual_padding),
+                               static_cast<int>(input_layout), include_padding_in_avg, use_ceil_for_output_shape, name);
+  return details::op("pool", args).as_tensor();
+}
+
+class relu {
+ public:
+  explicit relu(const edsl::Tensor& I) : I_(I) {}
+  relu& alpha(const edsl::Tensor& alpha) { alpha_ = alpha; return *this; }
+  relu& max_value(const edsl::Tensor& max_value) { max_value_ = max_value; return *this; }
+  relu& threshold(double threshold) { threshold_ = edsl::Value(threshold); return *this; }
+  relu& name(const std::string& name) { name_ = name; return *this; }
+  operator edsl::Tensor() const {  // NOLINT
+    return details::op("relu", edsl::make_tuple(I_, alpha_, max_value_, threshold_, name_)).as_tensor();
+  }
+
+ private:
+  edsl::Tensor I_, alpha_, max_value_;
+  edsl::Value threshold_;
+  std::string name_;
+};
+
+inline edsl::Tensor softmax(const edsl::Tensor& I, int axis, const std::string& name = "") {
+  return details::op("softmax", edsl::make_tuple(I, axis, name)).as_tensor();
+}
+
+inline edsl::Tensor sum(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
+  return details::op("sum", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+
+}  // namespace op
+}  // namespace plaidml

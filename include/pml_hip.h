@@ -110,7 +110,7 @@ enum {
   PML_HIP_EPI_CMP_GE,
   PML_HIP_EPI_CMP_EQ,
   PML_HIP_EPI_CMP_NE,
-  PML_HIP_EPI_SIGMOID_UNUSED_
+  PML_HIP_EPI_MAX_GT    /* v = (v > x) ? v : x  (the lower bound of a clip) */
 };
 
 /* where the second operand x of a step comes from */
@@ -168,8 +168,8 @@ typedef struct {
   int32_t init_kind;
   int32_t init_dtype;
   int64_t init_row_stride, init_col_stride;
-  int32_t c_dtype; /* element type stored to C (type after the tail) */
-  int32_t reserved;
+  int32_t c_dtype;  /* element type stored to C (type after the tail) */
+  int32_t b_layout; /* 0: B is [K][N] with leading dimension ldb; 1: B is [N][K] (K contiguous, ldb >= k) */
   pml_hip_epilogue tail;
 } pml_hip_gemm_desc;
 

@@ -186,6 +186,28 @@ def max(I, axes=None, keepdims=False):  # noqa: A001
     return _reduce(I, axes, keepdims, 'max', 'max')[0]
 
 
+def min(I, axes=None, keepdims=False):  # noqa: A001
+    return _reduce(I, axes, keepdims, 'min', 'min')[0]
+
+
+def clip(I, lo, hi):
+    """plaidml/op/lib/ops.cc:584-606: select(O > lo, O, cast(lo)) then select(O < hi, O, cast(hi))."""
+    O = I
+    if lo is not None:
+        O = E.select(O > lo, O, E.cast(lo, O.dt))
+    if hi is not None:
+        O = E.select(O < hi, O, E.cast(hi, O.dt))
+    return O
+
+
+def maximum(X, Y):
+    return E.select(X < Y, Y, X)  # plaidml/op/lib/ops.cc:1958-1968
+
+
+def minimum(X, Y):
+    return E.select(X < Y, X, Y)
+
+
 def mean(I, axes=None, keepdims=False):
     if len(I.shape) == 0 or (isinstance(axes, (list, tuple)) and len(axes) == 0):
         return I

@@ -293,6 +293,7 @@ __device__ inline Scalar<FT, IT> run_tail(const pml_hip_epilogue& t, Scalar<FT, 
         case PML_HIP_EPI_CMP_GE: is_cmp = true; cmp = a >= b; break;
         case PML_HIP_EPI_CMP_EQ: is_cmp = true; cmp = a == b; break;
         case PML_HIP_EPI_CMP_NE: is_cmp = true; cmp = (a < b) || (a > b); break;  // ordered not-equal
+        case PML_HIP_EPI_MAX_GT: r = (a > b) ? a : b; break;
         default: break;
       }
       v.f = round_float_to<FT>(dt, r);
@@ -316,6 +317,7 @@ __device__ inline Scalar<FT, IT> run_tail(const pml_hip_epilogue& t, Scalar<FT, 
         case PML_HIP_EPI_CMP_GE: is_cmp = true; cmp = uns ? (ua >= ub) : (a >= b); break;
         case PML_HIP_EPI_CMP_EQ: is_cmp = true; cmp = a == b; break;
         case PML_HIP_EPI_CMP_NE: is_cmp = true; cmp = a != b; break;
+        case PML_HIP_EPI_MAX_GT: r = (uns ? (ua > ub) : (a > b)) ? a : b; break;
         default: break;
       }
       v.i = wrap_int_to<IT>(dt, r);

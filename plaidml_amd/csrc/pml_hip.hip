@@ -110,7 +110,7 @@ bool valid_tail(const pml_hip_epilogue& t) {
   if (t.n_operands < 0 || t.n_operands > PML_HIP_MAX_EPI_OPERANDS) return false;
   for (int i = 0; i < t.n_ops; ++i) {
     const pml_hip_epi_op& op = t.ops[i];
-    if (op.opcode < PML_HIP_EPI_ADD || op.opcode > PML_HIP_EPI_CMP_NE) return false;
+    if (op.opcode < PML_HIP_EPI_ADD || op.opcode > PML_HIP_EPI_MAX_GT) return false;
     if (op.operand_kind == PML_HIP_OPND_TENSOR && (op.operand < 0 || op.operand >= t.n_operands)) return false;
     if (op.opcode == PML_HIP_EPI_STORE && (op.operand < 0 || op.operand >= PML_HIP_MAX_EPI_OPERANDS)) return false;
     if (dt_size(op.dtype) == 8 && op.opcode != PML_HIP_EPI_STORE) return false;  // 64-bit steps: general path only
@@ -224,13 +224,14 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
     fail("gemm: out_dtype does not fit in_dtype");
     return 0;
   }
-  if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->lda < d->k || d->ldb < d->n || d->ldc < d->n) {
+  if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->lda < d->k || d->ldb < (d->b_layout ? d->k : d->n) || d->ldc < d->n ||
+      (d->b_layout != 0 && d->b_layout != 1)) {
     fail("gemm: bad sizes or leading dimensions");
     return 0;
   }
   const int es = dt_size(d->in_dtype);
-  if ((d->k * es) % 16 != 0 || (d->lda * es) % 16 != 0) {
-    fail("gemm: K and lda must cover whole 16-byte vectors");
+  if ((d->k * es) % 16 != 0 || (d->lda * es) % 16 != 0 || (d->b_layout && (d->ldb * es) % 16 != 0)) {
+    fail("gemm: K and the K-contiguous leading dimensions must cover whole 16-byte vectors");
     return 0;
   }
   if (!valid_tail(d->tail)) {
@@ -244,7 +245,7 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   p->tile = choose_tile(d->m, d->n);
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
-  if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
+  if (!d->b_layout && hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
     delete p;
     fail("gemm: cannot allocate the packed right-hand side");
     return 0;
@@ -263,11 +264,13 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
   const pml_hip_gemm_desc& d = p->gemm;
   if (!a || !c) return fail("gemm_invoke: null operand");
-  if (!b && !p->packed) return fail("gemm_invoke: b is null and no packed right-hand side exists");
+  if (!b && (!p->packed || d.b_layout)) return fail("gemm_invoke: b is null and no packed right-hand side exists");
+  if (d.b_layout && ((uintptr_t)b & 15) != 0) return fail("gemm_invoke: an [N][K] right-hand side must be 16-byte aligned");
   if (((uintptr_t)a & 15) != 0) return fail("gemm_invoke: A must be 16-byte aligned");
   if (d.init_kind && !init) return fail("gemm_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
-  if (b && check(transpose_pack(es, b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack")) return 1;
+  if (b && !d.b_layout && check(transpose_pack(es, b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack"))
+    return 1;
   IgemmArgs g;
   std::memset(&g, 0, sizeof g);
   g.M = d.m;
@@ -275,8 +278,8 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   g.K = d.k;
   g.A = a;
   g.lda = d.lda;
-  g.Bt = p->bt;
-  g.ldbt = p->bt_ld;
+  g.Bt = d.b_layout ? b : p->bt;
+  g.ldbt = d.b_layout ? d.ldb : p->bt_ld;
   g.C = c;
   g.ldc = d.ldc;
   g.out_dtype = d.out_dtype;
@@ -420,6 +423,7 @@ int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s) {
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_GEMM || !b) return fail("gemm_pack_b: bad argument");
   const pml_hip_gemm_desc& d = p->gemm;
+  if (d.b_layout) return fail("gemm_pack_b: an [N][K] right-hand side needs no packing");
   if (check(transpose_pack(dt_size(d.in_dtype), b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   p->packed = true;

@@ -18,7 +18,7 @@ AGG_ASSIGN, AGG_ADD, AGG_MAX, AGG_MIN, AGG_MUL = 0, 1, 2, 3, 4
 COMBO_NONE, COMBO_ADD, COMBO_COND, COMBO_EQ, COMBO_MUL = 0, 1, 2, 3, 4
 (EPI_ADD, EPI_SUB, EPI_RSUB, EPI_MUL, EPI_DIV, EPI_RDIV, EPI_MAX, EPI_MIN, EPI_RELU, EPI_NEG, EPI_EXP, EPI_LOG,
  EPI_SQRT, EPI_TANH, EPI_FLOOR, EPI_CEIL, EPI_ROUND, EPI_CAST, EPI_STORE, EPI_CMP_LT, EPI_CMP_GT, EPI_CMP_LE,
- EPI_CMP_GE, EPI_CMP_EQ, EPI_CMP_NE) = range(1, 26)
+ EPI_CMP_GE, EPI_CMP_EQ, EPI_CMP_NE, EPI_MAX_GT) = range(1, 27)
 OPND_NONE, OPND_IMM, OPND_TENSOR = 0, 1, 2
 MAX_EPI_OPS, MAX_EPI_OPERANDS, MAX_RANK, MAX_IDX, MAX_FORMS = 12, 6, 6, 12, 32
 
@@ -50,7 +50,7 @@ class Epilogue(ctypes.Structure):
 class GemmDesc(ctypes.Structure):
     _fields_ = [('in_dtype', i32), ('out_dtype', i32), ('m', i64), ('n', i64), ('k', i64), ('lda', i64), ('ldb', i64),
                 ('ldc', i64), ('init_kind', i32), ('init_dtype', i32), ('init_row_stride', i64),
-                ('init_col_stride', i64), ('c_dtype', i32), ('reserved', i32), ('tail', Epilogue)]
+                ('init_col_stride', i64), ('c_dtype', i32), ('b_layout', i32), ('tail', Epilogue)]
 
 
 class Conv2dDesc(ctypes.Structure):

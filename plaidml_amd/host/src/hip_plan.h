@@ -1,0 +1,71 @@
+// The `hip` target: turns a Tile program into a kernel plan for the gfx950 kernel
+// library.  It stands where the reference's `llvm_cpu` target pipeline stands
+// (pmlc/target/x86/pipeline.cc:259-402) but does not lower through loops: each
+// contraction is classified by the strides of its accesses (the idea of the
+// reference GEMM stencil, pmlc/dialect/pxa/transforms/stencil_gemm.cc:297-321),
+// its single-use elementwise consumers are folded into the kernel's tail (the
+// role of pxa-fusion and x86-tpp-combine, pmlc/target/x86/tpp_combine.cc:30-140),
+// and the result is a list of launches.  Building a plan needs no device.
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "pml_hip.h"
+#include "tile.h"
+
+namespace pmlc::target::hip {
+
+struct BufferInfo {
+  enum Kind { Input, Output, Constant, Temp } kind = Temp;
+  int index = 0;                 // Input / Output: position in the program signature
+  size_t bytes = 0;
+  util::BufferPtr constant;      // Constant: host bytes uploaded once when the executable is built
+  std::string name;
+};
+
+struct Step {
+  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy } kind = Copy;
+  std::string text;  // one line for the plan dump
+  // descriptors (only the one matching `kind` is meaningful)
+  pml_hip_gemm_desc gemm{};
+  pml_hip_conv2d_desc conv{};
+  pml_hip_dwconv2d_desc dw{};
+  pml_hip_pool2d_desc pool{};
+  pml_hip_eltwise_desc elt{};
+  pml_hip_select_desc sel{};
+  pml_hip_contract_desc con{};
+  int index_axis = 0;
+  std::vector<int64_t> index_sizes;
+  // buffer ids (-1 = none) and element offsets applied to the base pointers
+  int a = -1, b = -1, c = -1, init = -1, out2 = -1;
+  int64_t a_off = 0, b_off = 0, c_off = 0, init_off = 0;
+  std::vector<int> operands;       // tail operands / contraction sources / select inputs
+  std::vector<int64_t> operand_off;
+  std::vector<int> outs;           // extra outputs of STORE steps (index = STORE's operand field)
+  bool b_is_nk = false;            // Gemm: right-hand side is already [N][K]
+  bool b_constant = false;         // Gemm / Conv2d: right-hand side is a program constant (pack once)
+  size_t copy_bytes = 0;           // Copy
+  // roofline bookkeeping for reports
+  double flops = 0;
+  double bytes = 0;
+};
+
+struct Plan {
+  std::vector<BufferInfo> buffers;
+  std::vector<Step> steps;
+  std::vector<int> input_buffers;   // buffer id per program input
+  std::vector<int> output_buffers;  // buffer id per program output
+  std::string dump() const;
+};
+
+struct Options {
+  bool fuse = true;        // fold elementwise consumers into kernel tails
+  bool specialise = true;  // use the MFMA / window kernels; false = every contraction through the general kernel
+};
+
+// Runs the pipeline on a copy of the program's op list and returns the plan.
+std::shared_ptr<Plan> buildPlan(tile::Program* program, const Options& options);
+
+}  // namespace pmlc::target::hip

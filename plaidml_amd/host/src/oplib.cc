@@ -1,0 +1,509 @@
+// The operation library behind plaidml_op_make: the subset of the reference's
+// plaidml/op/lib/ops.cc that the contraction hot path uses, written (as there) on top
+// of the EDSL itself, so that every operation becomes Tile contractions and
+// elementwise operations.
+//
+//   convolution  ops.cc:879-1467 (forward mode; NXC / NCX inputs, XCK / KCX filters;
+//                group layouts NONE and IN_C; autogroup UNGROUPED / EXPLICIT / DEPTHWISE)
+//   padding rule ops.cc:347-382
+//   pool         ops.cc:2562-2703        dot      ops.cc:1512-1561
+//   argmax       ops.cc:505-521          clip     ops.cc:584-606
+//   max / min / sum / mean via AggregationAxes ops.cc:71-127,1970-2003,3424-
+//   maximum / minimum ops.cc:1958-1968   relu     ops.cc:2705-2728
+//   softmax      ops.cc:3049-3098 (softmax over the last axis)
+#include <functional>
+#include <map>
+#include <set>
+
+#include "ffi_internal.h"
+#include "plaidml/op/op.h"
+
+using namespace plaidml;        // NOLINT
+using namespace plaidml::edsl;  // NOLINT
+using plaidml::op::AutoGroupMode;
+using plaidml::op::AutoPadMode;
+using plaidml::op::ConvDerivMode;
+using plaidml::op::GroupLayout;
+using plaidml::op::PoolMode;
+using plaidml::op::TensorLayout;
+
+namespace {
+
+template <typename E>
+E validate(int64_t raw) {
+  if (raw < 0 || raw >= static_cast<int64_t>(E::_LAST)) throw std::runtime_error("Invalid enumeration value in operation arguments");
+  return static_cast<E>(raw);
+}
+
+std::pair<TensorDim, TensorDim> compute_padding_and_output_size(const TensorDim& input_size, const TensorDim& filter_size,
+                                                                int64_t stride, AutoPadMode mode, int64_t pad_lo,
+                                                                int64_t pad_hi, int64_t dilation, int64_t data_dilation,
+                                                                bool use_ceil) {
+  TensorDim i_eff = (data_dilation * (input_size - 1)) + 1;
+  TensorDim f_eff = (dilation * (filter_size - 1)) + 1;
+  const int64_t ceil_term = use_ceil ? stride - 1 : 0;
+  switch (mode) {
+    case AutoPadMode::EXPLICIT:
+      return {TensorDim(pad_lo), (i_eff + pad_lo + pad_hi - f_eff + stride + ceil_term) / stride};
+    case AutoPadMode::VALID:
+      return {TensorDim(0), (i_eff - f_eff + stride + ceil_term) / stride};
+    case AutoPadMode::SAME_LOWER:
+    case AutoPadMode::SAME_UPPER: {
+      TensorDim out = (i_eff + stride - 1) / stride;
+      const int64_t lower = mode == AutoPadMode::SAME_LOWER ? 1 : 0;
+      TensorDim pad = (edsl::max(0, (out - 1) * stride + f_eff - i_eff) + lower) / 2;
+      return {pad, out};
+    }
+    default:
+      throw std::runtime_error("Unexpected autopadding mode");
+  }
+}
+
+struct AggregationAxes {
+  std::vector<TensorIndex> src_idxs, dst_idxs, reduce_idxs;
+  std::vector<TensorDim> src_dims, dst_dims, reduce_dims;
+  std::set<size_t> axes;
+
+  AggregationAxes(size_t ndims, const Value& in_axes, bool keepdims) : src_idxs(ndims), src_dims(ndims) {
+    auto norm = [&](int64_t a) {
+      if (a < 0) a += static_cast<int64_t>(ndims);
+      if (a < 0 || a >= static_cast<int64_t>(ndims)) throw std::out_of_range("axis out of range: " + std::to_string(a));
+      return static_cast<size_t>(a);
+    };
+    if (in_axes.is_none()) {
+      for (size_t i = 0; i < ndims; ++i) axes.insert(i);
+    } else if (in_axes.is_tuple()) {
+      for (const auto& a : in_axes.as_tuple()) axes.insert(norm(a.as_int()));
+    } else if (in_axes.is_int()) {
+      axes.insert(norm(in_axes.as_int()));
+    } else {
+      throw std::runtime_error("Invalid Value type for AggregationAxes: in_axes");
+    }
+    for (size_t a : axes) {
+      reduce_idxs.push_back(src_idxs[a]);
+      reduce_dims.push_back(src_dims[a]);
+    }
+    if (keepdims) {
+      dst_idxs = src_idxs;
+      dst_dims = src_dims;
+      for (size_t a : axes) {
+        dst_idxs[a] = TensorIndex();
+        dst_dims[a] = TensorDim(1);
+      }
+    } else {
+      for (size_t i = 0; i < ndims; ++i) {
+        if (!axes.count(i)) {
+          dst_idxs.push_back(src_idxs[i]);
+          dst_dims.push_back(src_dims[i]);
+        }
+      }
+    }
+  }
+};
+
+Value reduce(const Value& value, const char* what, plaidml_agg_op agg) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error(std::string(what) + " expects 3 arguments");
+  auto I = args[0].as_tensor();
+  if (I.rank() == 0) return Value{I};
+  auto axes = args[1];
+  if (axes.is_tuple() && axes.as_tuple().empty()) return Value{I};
+  AggregationAxes ag(I.rank(), axes, args[2].as_bool());
+  I.bind_dims(ag.src_dims);
+  Contraction c(ag.dst_dims, ag.dst_idxs, what);
+  switch (agg) {
+    case PLAIDML_AGG_OP_MAX: c.max(I(ag.src_idxs)); break;
+    case PLAIDML_AGG_OP_MIN: c.min(I(ag.src_idxs)); break;
+    default: c.sum(I(ag.src_idxs)); break;
+  }
+  Tensor O = c;
+  if (std::string(what) == "mean") {
+    Tensor denom(1);
+    for (size_t a : ag.axes) denom = denom * ag.src_dims.at(a);
+    return Value{O / denom};
+  }
+  return Value{O};
+}
+
+Value op_argmax(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("argmax expects 2 arguments");
+  auto I = args[0].as_tensor();
+  AggregationAxes ag(I.rank(), args[1], false);
+  I.bind_dims(ag.src_dims);
+  Tensor M = Contraction(ag.dst_dims, ag.dst_idxs, "argmax").max(I(ag.src_idxs));
+  Tensor IX = index(ag.reduce_dims, 0);
+  Tensor AM = Contraction(ag.dst_dims, ag.dst_idxs, "argmax").max(cond(I(ag.src_idxs), M(ag.dst_idxs), IX(ag.reduce_idxs)));
+  return Value{cast(AM, DType::UINT32)};
+}
+
+Value op_clip(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("clip expects 3 arguments");
+  auto O = args[0].as_tensor();
+  if (!args[1].is_none()) {
+    auto lo = args[1].as_tensor();
+    O = select(O > lo, O, cast(lo, O.dtype()));
+  }
+  if (!args[2].is_none()) {
+    auto hi = args[2].as_tensor();
+    O = select(O < hi, O, cast(hi, O.dtype()));
+  }
+  return Value{O};
+}
+
+Value op_convolution(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 18) throw std::runtime_error("Convolution op expects 18 arguments");
+  auto I = args[0].as_tensor();
+  auto F = args[1].as_tensor();
+  auto strides = args[2].as_int_tuple_or_empty();
+  auto dilations = args[3].as_int_tuple_or_empty();
+  auto data_dilations = args[4].as_int_tuple_or_empty();
+  auto filter_shape = args[5].as_int_tuple_or_empty();
+  auto groups = args[6].as_int();
+  auto autopad_mode = validate<AutoPadMode>(args[7].as_int());
+  auto manual_padding = args[8].as_int_tuple_or_empty();
+  auto input_layout = validate<TensorLayout>(args[9].as_int());
+  auto filter_layout = validate<TensorLayout>(args[10].as_int());
+  auto group_layout = validate<GroupLayout>(args[11].as_int());
+  auto name = args[13].as_str();
+  auto autogroup_mode = validate<AutoGroupMode>(args[14].as_int());
+  auto deriv_mode = validate<ConvDerivMode>(args[15].as_int());
+  if (name.empty()) name = "conv";
+  if (deriv_mode != ConvDerivMode::NONE) throw std::runtime_error("Only forward convolutions are supported by this backend");
+  if (input_layout != TensorLayout::NXC && input_layout != TensorLayout::NCX) throw std::runtime_error("Invalid input_layout");
+  if (filter_layout != TensorLayout::XCK && filter_layout != TensorLayout::KCX)
+    throw std::runtime_error("Only XCK and KCX filter layouts are supported by this backend");
+  if (group_layout != GroupLayout::NONE && group_layout != GroupLayout::IN_C)
+    throw std::runtime_error("Only the NONE and IN_C group layouts are supported by this backend");
+  if (I.rank() < 3 || F.rank() != I.rank()) throw std::runtime_error("Convolution input and filter rank mismatch");
+  const size_t spatial_rank = I.rank() - 2;
+  if (strides.empty()) strides.assign(spatial_rank, 1);
+  if (dilations.empty()) dilations.assign(spatial_rank, 1);
+  if (data_dilations.empty()) data_dilations.assign(spatial_rank, 1);
+  if (strides.size() != spatial_rank || dilations.size() != spatial_rank || data_dilations.size() != spatial_rank)
+    throw std::runtime_error("Convolution strides / dilations rank mismatch");
+  if (!manual_padding.empty() && autopad_mode != AutoPadMode::EXPLICIT)
+    throw std::runtime_error("Autopadding and manual padding both requested for single conv operation");
+  if (manual_padding.size() == spatial_rank) {
+    // one value per dimension pads both sides
+    auto lo = manual_padding;
+    manual_padding.insert(manual_padding.end(), lo.begin(), lo.end());
+  }
+  manual_padding.resize(2 * spatial_rank, 0);
+  if ((group_layout == GroupLayout::NONE) != (autogroup_mode == AutoGroupMode::UNGROUPED))
+    throw std::runtime_error("Convolution group layout and autogroup mode are inconsistent");
+
+  TensorDim N, CI, CO, G, F_CI, F_CO;
+  TensorIndex n("n"), ci("ci"), co("co"), g("g");
+  std::vector<TensorDim> I_spatial(spatial_rank), F_spatial(spatial_rank);
+  std::vector<TensorIndex> x, k;
+  for (size_t i = 0; i < spatial_rank; ++i) {
+    x.emplace_back("x" + std::to_string(i));
+    k.emplace_back("k" + std::to_string(i));
+  }
+  // bind the input and filter dims
+  std::vector<TensorDim> I_dims = {N};
+  if (input_layout == TensorLayout::NCX) I_dims.push_back(CI);
+  for (auto& d : I_spatial) I_dims.push_back(d);
+  if (input_layout == TensorLayout::NXC) I_dims.push_back(CI);
+  I.bind_dims(I_dims);
+  if (group_layout == GroupLayout::NONE) {
+    F_CI = CI;
+  } else {
+    F_CI = CI;  // IN_C: the filter's input-channel dimension carries the group
+  }
+  std::vector<TensorDim> F_dims;
+  if (filter_layout == TensorLayout::KCX) {
+    F_dims = {F_CO, F_CI};
+    for (auto& d : F_spatial) F_dims.push_back(d);
+  } else {
+    for (auto& d : F_spatial) F_dims.push_back(d);
+    F_dims.push_back(F_CI);
+    F_dims.push_back(F_CO);
+  }
+  F.bind_dims(F_dims);
+  if (!filter_shape.empty()) {
+    if (filter_shape.size() != spatial_rank) throw std::runtime_error("Filter shape rank mismatch");
+    std::vector<TensorDim> explicit_dims = F_dims;
+    const size_t off = filter_layout == TensorLayout::KCX ? 2 : 0;
+    for (size_t i = 0; i < spatial_rank; ++i) explicit_dims[off + i] = TensorDim(filter_shape[i]);
+    F.bind_dims(explicit_dims);
+  }
+  switch (autogroup_mode) {
+    case AutoGroupMode::UNGROUPED: G = TensorDim(1); break;
+    case AutoGroupMode::EXPLICIT: G = TensorDim(groups); break;
+    case AutoGroupMode::DEPTHWISE: G = CI; break;
+    default: throw std::runtime_error("Unsupported autogroup mode");
+  }
+  CO = group_layout == GroupLayout::IN_C ? F_CO * G : F_CO;
+
+  std::vector<TensorDim> O_spatial, pad_before;
+  for (size_t i = 0; i < spatial_rank; ++i) {
+    auto pr = compute_padding_and_output_size(I_spatial[i], F_spatial[i], strides[i], autopad_mode, manual_padding[i],
+                                              manual_padding[i + spatial_rank], dilations[i], data_dilations[i], false);
+    pad_before.push_back(pr.first);
+    O_spatial.push_back(pr.second);
+  }
+  std::vector<TensorDim> O_dims = {N};
+  if (input_layout == TensorLayout::NCX) O_dims.push_back(CO);
+  for (auto& d : O_spatial) O_dims.push_back(d);
+  if (input_layout == TensorLayout::NXC) O_dims.push_back(CO);
+
+  // index formulas (ops.cc:1342-1450)
+  std::vector<Constraint> constraints;
+  TensorIndex i_c = group_layout == GroupLayout::NONE ? ci : (CI / G) * g + ci;
+  TensorIndex o_c = group_layout == GroupLayout::NONE ? co : (CO / G) * g + co;
+  TensorIndex f_ci = group_layout == GroupLayout::NONE ? ci : (CI / G) * g + ci;
+  TensorIndex f_co = co;
+  if (group_layout == GroupLayout::IN_C) constraints.push_back(ci < CI / G);
+  std::vector<TensorIndex> spatial;
+  for (size_t i = 0; i < spatial_rank; ++i)
+    spatial.push_back((strides[i] * x[i] + dilations[i] * k[i] - pad_before[i]) / data_dilations[i]);
+  std::vector<TensorIndex> I_idxs = {n}, O_idxs = {n}, F_idxs;
+  if (input_layout == TensorLayout::NCX) {
+    I_idxs.push_back(i_c);
+    O_idxs.push_back(o_c);
+  }
+  for (size_t i = 0; i < spatial_rank; ++i) {
+    I_idxs.push_back(spatial[i]);
+    O_idxs.push_back(x[i]);
+  }
+  if (input_layout == TensorLayout::NXC) {
+    I_idxs.push_back(i_c);
+    O_idxs.push_back(o_c);
+  }
+  if (filter_layout == TensorLayout::KCX) {
+    F_idxs = {f_co, f_ci};
+    for (auto& kk : k) F_idxs.push_back(kk);
+  } else {
+    for (auto& kk : k) F_idxs.push_back(kk);
+    F_idxs.push_back(f_ci);
+    F_idxs.push_back(f_co);
+  }
+  Tensor O = Contraction(O_dims, O_idxs, name).sum(I(I_idxs) * F(F_idxs)).add_constraints(constraints);
+  return Value{O};
+}
+
+Value op_dot(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("dot expects 3 arguments");
+  auto X = args[0].as_tensor();
+  auto Y = args[1].as_tensor();
+  auto name = args[2].as_str();
+  if (name.empty()) name = "dot";
+  if (X.dtype() != Y.dtype())
+    throw std::runtime_error(std::string("Invalid dtype in dot: X.dtype = '") + to_string(X.dtype()) + "', Y.dtype = '" +
+                             to_string(Y.dtype()) + "'");
+  if (X.rank() == 1 && Y.rank() == 1) {
+    TensorDim I;
+    TensorIndex i;
+    X.bind_dims(I);
+    Y.bind_dims(I);
+    Tensor O = Contraction({I}, {i}, name).sum(X(i) * Y(i));
+    return Value{O};
+  }
+  if (1 <= X.rank() && 2 <= Y.rank()) {
+    std::vector<TensorDim> X_dims(X.rank()), Y_dims(Y.rank());
+    std::vector<TensorIndex> X_idxs(X.rank()), Y_idxs(Y.rank());
+    TensorIndex z;
+    X_idxs[X.rank() - 1] = z;
+    Y_idxs[Y.rank() - 2] = z;
+    X.bind_dims(X_dims);
+    Y.bind_dims(Y_dims);
+    std::vector<TensorDim> O_dims;
+    std::vector<TensorIndex> O_idxs;
+    for (size_t i = 0; i + 1 < X.rank(); ++i) {
+      O_dims.push_back(X_dims[i]);
+      O_idxs.push_back(X_idxs[i]);
+    }
+    for (size_t i = 0; i + 2 < Y.rank(); ++i) {
+      O_dims.push_back(Y_dims[i]);
+      O_idxs.push_back(Y_idxs[i]);
+    }
+    O_dims.push_back(Y_dims[Y.rank() - 1]);
+    O_idxs.push_back(Y_idxs[Y.rank() - 1]);
+    Tensor O = Contraction(O_dims, O_idxs, name).sum(X(X_idxs) * Y(Y_idxs));
+    return Value{O};
+  }
+  throw std::runtime_error("Unsupported dims for dot operation");
+}
+
+Value op_maximum(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("maximum expects 2 arguments");
+  auto X = args[0].as_tensor(), Y = args[1].as_tensor();
+  return Value{select(X < Y, Y, X)};
+}
+Value op_minimum(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("minimum expects 2 arguments");
+  auto X = args[0].as_tensor(), Y = args[1].as_tensor();
+  return Value{select(X < Y, X, Y)};
+}
+
+Value op_pool(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 10) throw std::runtime_error("PlaidML pool op expects 10 arguments");
+  auto I = args[0].as_tensor();
+  auto pool_mode = validate<PoolMode>(args[1].as_int());
+  auto pool_size = args[2].as_int_tuple();
+  auto strides = args[3].as_int_tuple();
+  auto autopad_mode = validate<AutoPadMode>(args[4].as_int());
+  auto manual_padding = args[5].as_int_tuple();
+  auto input_layout = validate<TensorLayout>(args[6].as_int());
+  auto include_padding_in_avg = args[7].as_bool();
+  auto use_ceil = args[8].as_bool();
+  auto name = args[9].as_str();
+  if (name.empty()) name = "pool";
+  const size_t spatial_rank = pool_size.size();
+  if (!manual_padding.empty() && autopad_mode != AutoPadMode::EXPLICIT)
+    throw std::runtime_error("Autopadding and manual padding both requested for single pool operation");
+  if (strides.size() != spatial_rank) throw std::runtime_error("Inconsistent spatial rank in pool op");
+  if (I.rank() != spatial_rank + 2) throw std::runtime_error("Inconsistent spatial rank in pool op");
+  if (input_layout != TensorLayout::NXC && input_layout != TensorLayout::NCX)
+    throw std::runtime_error("Tensor layout requested in pool op does not apply to pooling");
+  if (manual_padding.size() == spatial_rank) {
+    auto lo = manual_padding;
+    manual_padding.insert(manual_padding.end(), lo.begin(), lo.end());
+  }
+  manual_padding.resize(2 * spatial_rank, 0);
+
+  TensorDim N, C;
+  TensorIndex n("n"), c("c");
+  std::vector<TensorDim> X(spatial_rank);
+  std::vector<TensorIndex> x, k;
+  for (size_t i = 0; i < spatial_rank; ++i) {
+    x.emplace_back("x" + std::to_string(i));
+    k.emplace_back("k" + std::to_string(i));
+  }
+  std::vector<TensorDim> I_dims = {N}, O_dims = {N};
+  std::vector<TensorIndex> I_idxs = {n}, O_idxs = {n};
+  std::vector<Constraint> constraints;
+  if (input_layout == TensorLayout::NCX) I_dims.push_back(C);
+  for (auto& d : X) I_dims.push_back(d);
+  if (input_layout == TensorLayout::NXC) I_dims.push_back(C);
+  I.bind_dims(I_dims);
+  if (input_layout == TensorLayout::NCX) {
+    I_idxs.push_back(c);
+    O_dims.push_back(C);
+    O_idxs.push_back(c);
+  }
+  for (size_t i = 0; i < spatial_rank; ++i) {
+    O_idxs.push_back(x[i]);
+    auto pr = compute_padding_and_output_size(X[i], TensorDim(pool_size[i]), strides[i], autopad_mode, manual_padding[i],
+                                              manual_padding[spatial_rank + i], 1, 1, use_ceil);
+    O_dims.push_back(pr.second);
+    I_idxs.push_back(strides[i] * x[i] + k[i] - pr.first);
+    constraints.push_back(k[i] < pool_size[i]);
+  }
+  if (input_layout == TensorLayout::NXC) {
+    I_idxs.push_back(c);
+    O_dims.push_back(C);
+    O_idxs.push_back(c);
+  }
+  Contraction O = Contraction(O_dims, O_idxs, name).add_constraints(constraints);
+  switch (pool_mode) {
+    case PoolMode::MAX: O.max(I(I_idxs)); return Value{Tensor(O)};
+    case PoolMode::MIN: O.min(I(I_idxs)); return Value{Tensor(O)};
+    case PoolMode::SUM: O.sum(I(I_idxs)); return Value{Tensor(O)};
+    case PoolMode::AVG: {
+      O.sum(I(I_idxs));
+      Tensor S = O;
+      if (include_padding_in_avg) {
+        int64_t total = 1;
+        for (auto s : pool_size) total *= s;
+        return Value{S / total};
+      }
+      auto One = cast(Tensor{1}, I.dtype());
+      Tensor Ones = Contraction(I_dims, O_idxs, name).assign(One());
+      Tensor Count = Contraction(O_dims, O_idxs, name).sum(Ones(I_idxs)).add_constraints(constraints);
+      return Value{S / Count};
+    }
+    default: throw std::runtime_error("Unrecognized pool_mode in pool op");
+  }
+}
+
+Value op_relu(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 5) throw std::runtime_error("relu expects 5 arguments");
+  Tensor I = args[0].as_tensor();
+  Value alpha = args[1], max_value = args[2], threshold = args[3];
+  auto name = args[4].as_str();
+  if (name.empty()) name = "relu";
+  const double T = threshold.is_none() ? 0.0 : threshold.as_float();
+  if ((alpha.is_none() || (alpha.is_float() && alpha.as_float() == 0.0)) && max_value.is_none() && T == 0.0)
+    return Value{edsl::relu(I, name)};
+  Tensor A = alpha.is_none() ? Tensor(0.0) : alpha.as_tensor();
+  Tensor O = select(I < T, cast(A * (I - T), I.dtype()), I);
+  if (!max_value.is_none()) {
+    Tensor M = cast(max_value.as_tensor(), I.dtype());
+    O = select(O < M, O, M);
+  }
+  return Value{O};
+}
+
+Value op_softmax(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("softmax expects 3 arguments");
+  auto I = args[0].as_tensor();
+  int64_t axis = args[1].as_int();
+  auto name = args[2].as_str();
+  if (name.empty()) name = "softmax";
+  const int64_t ndims = static_cast<int64_t>(I.rank());
+  if (axis < 0) axis += ndims;
+  if (axis < 0 || axis >= ndims) throw std::runtime_error("Axis out of range for softmax op");
+  if (axis != ndims - 1) throw std::runtime_error("softmax over a non-trailing axis is not supported by this backend");
+  std::vector<TensorDim> I_dims(ndims);
+  std::vector<TensorIndex> I_idxs(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> R_dims = I_dims;
+  std::vector<TensorIndex> R_idxs = I_idxs;
+  R_dims[axis] = TensorDim(1);
+  R_idxs[axis] = TensorIndex(static_cast<int64_t>(0));
+  Tensor M = Contraction(R_dims, R_idxs, name).max(I(I_idxs));
+  auto E = exp(I - M);
+  Tensor Nn = Contraction(R_dims, R_idxs, name).sum(E(I_idxs));
+  return Value{E / Nn};
+}
+
+using OpFn = std::function<Value(const Value&)>;
+const std::map<std::string, OpFn>& registry() {
+  static const std::map<std::string, OpFn> r = {
+      {"argmax", op_argmax},
+      {"clip", op_clip},
+      {"convolution", op_convolution},
+      {"dot", op_dot},
+      {"max", [](const Value& v) { return reduce(v, "max", PLAIDML_AGG_OP_MAX); }},
+      {"maximum", op_maximum},
+      {"mean", [](const Value& v) { return reduce(v, "mean", PLAIDML_AGG_OP_SUM); }},
+      {"min", [](const Value& v) { return reduce(v, "min", PLAIDML_AGG_OP_MIN); }},
+      {"minimum", op_minimum},
+      {"pool", op_pool},
+      {"relu", op_relu},
+      {"softmax", op_softmax},
+      {"sum", [](const Value& v) { return reduce(v, "sum", PLAIDML_AGG_OP_SUM); }},
+  };
+  return r;
+}
+
+}  // namespace
+
+extern "C" plaidml_value* plaidml_op_make(plaidml_error* err, const char* op_name, plaidml_value* value) {
+  err->code = 0;
+  err->msg = nullptr;
+  try {
+    auto it = registry().find(op_name ? op_name : "");
+    if (it == registry().end()) throw std::runtime_error(std::string("Invalid op_name: ") + (op_name ? op_name : "(null)"));
+    // the library functions work on the C++ wrappers; hand them an aliasing copy of the argument
+    plaidml_error e2{0, nullptr};
+    Value arg(plaidml_value_clone(&e2, value));
+    Value ret = it->second(arg);
+    return plaidml_value_clone(&e2, ret.as_ptr());
+  } catch (const std::exception& ex) {
+    err->code = 1;
+    err->msg = new plaidml_string{ex.what()};
+    return nullptr;
+  }
+}

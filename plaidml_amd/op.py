@@ -1,0 +1,84 @@
+"""Python view of the operation library (plaidml_op_make), after plaidml/op/__init__.py of the
+reference.  Keyword defaults follow the C++ builders of plaidml/op/op.h."""
+from . import edsl as E
+
+# enumerations of plaidml/op/op.h:28-130
+AUTOGROUP_UNGROUPED, AUTOGROUP_EXPLICIT, AUTOGROUP_AUTO, AUTOGROUP_DEPTHWISE = range(4)
+AUTOPAD_EXPLICIT, AUTOPAD_SAME_LOWER, AUTOPAD_SAME_UPPER, AUTOPAD_VALID = range(4)
+GROUP_NONE, GROUP_SEPARATE, GROUP_IN_C, GROUP_IN_K = range(4)
+POOL_AVG, POOL_MAX, POOL_MIN, POOL_SUM = range(4)
+LAYOUT_NXC, LAYOUT_NCX, LAYOUT_KCX, LAYOUT_XCK, LAYOUT_GKCX, LAYOUT_XGCK = range(6)
+
+SAME_UPPER, SAME_LOWER, VALID, EXPLICIT = 'same_upper', 'same_lower', 'valid', 'explicit'
+_AUTOPAD = {SAME_UPPER: AUTOPAD_SAME_UPPER, SAME_LOWER: AUTOPAD_SAME_LOWER, VALID: AUTOPAD_VALID, EXPLICIT: AUTOPAD_EXPLICIT}
+_POOL = {'avg': POOL_AVG, 'max': POOL_MAX, 'min': POOL_MIN, 'sum': POOL_SUM}
+
+
+def _ints(x):
+    return None if x is None else [int(v) for v in x]
+
+
+def convolution(I, F, strides=None, dilations=None, data_dilations=None, autopad=SAME_UPPER, manual_padding=None,
+                depthwise=False, name=''):
+    """NXC input, XCK filter.  depthwise=True is GroupLayout IN_C with AutoGroupMode DEPTHWISE."""
+    args = [I, F, _ints(strides), _ints(dilations), _ints(data_dilations), None, 1, _AUTOPAD[autopad],
+            _ints(manual_padding), LAYOUT_NXC, LAYOUT_XCK, GROUP_IN_C if depthwise else GROUP_NONE, False, name,
+            AUTOGROUP_DEPTHWISE if depthwise else AUTOGROUP_UNGROUPED, 0, None, False]
+    return E.op_make('convolution', args).as_tensor()
+
+
+def pool(I, mode, pool_size, strides, autopad=VALID, manual_padding=None, include_padding_in_avg=False, use_ceil=False,
+         name=''):
+    args = [I, _POOL[mode], _ints(pool_size), _ints(strides), _AUTOPAD[autopad], _ints(manual_padding or []), LAYOUT_NXC,
+            bool(include_padding_in_avg), bool(use_ceil), name]
+    return E.op_make('pool', args).as_tensor()
+
+
+def dot(X, Y, name=''):
+    return E.op_make('dot', [X, Y, name]).as_tensor()
+
+
+def _axes(axes):
+    if axes is None or isinstance(axes, int):
+        return axes
+    return [int(a) for a in axes]
+
+
+def sum(I, axes=None, keepdims=False):  # noqa: A001
+    return E.op_make('sum', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def max(I, axes=None, keepdims=False):  # noqa: A001
+    return E.op_make('max', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def min(I, axes=None, keepdims=False):  # noqa: A001
+    return E.op_make('min', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def mean(I, axes=None, keepdims=False):
+    return E.op_make('mean', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def relu(I):
+    return E.op_make('relu', [I, None, None, None, '']).as_tensor()
+
+
+def softmax(I, axis=-1, name=''):
+    return E.op_make('softmax', [I, int(axis), name]).as_tensor()
+
+
+def argmax(I, axis=-1):
+    return E.op_make('argmax', [I, _axes(axis)]).as_tensor()
+
+
+def clip(I, lo, hi):
+    return E.op_make('clip', [I, lo, hi]).as_tensor()
+
+
+def maximum(X, Y):
+    return E.op_make('maximum', [X, Y]).as_tensor()
+
+
+def minimum(X, Y):
+    return E.op_make('minimum', [X, Y]).as_tensor()

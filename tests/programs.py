@@ -1,0 +1,245 @@
+"""Tile programs written once and built twice: with the CPU oracle's EDSL (oracle.tile_oracle /
+oracle.tile_oplib) and with the product's EDSL (plaidml_amd.edsl / plaidml_amd.op, i.e. the plaidml_*
+C ABI).  Each builder takes the two modules and returns (program, input arrays, tolerance class).
+
+Programs restate the reference's own tests where one exists (file:line in each docstring) and the
+five workload configurations of this build at reduced sizes.
+"""
+import numpy as np
+
+EXACT, FP32, BF16 = 'exact', 'fp32', 'bf16'
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+def _bf16(a):
+    from oracle.tile_oracle import round_bf16
+    return round_bf16(np.asarray(a, np.float32))
+
+
+def dot_f32(E, op, M=8, N=32, K=16, seed=2):
+    """CppEdsl.Dot, plaidml/edsl/tests/edsl_test.cc:448-486 (8x16 . 16x32, normal(0,1) inputs)."""
+    A = E.Placeholder(E.DType.FLOAT32, [M, K])
+    B = E.Placeholder(E.DType.FLOAT32, [K, N])
+    I, J, Kd = E.TensorDims(3)
+    i, j, k = E.TensorIndexes(3)
+    A.bind_dims(I, Kd)
+    B.bind_dims(Kd, J)
+    C = E.Contraction().outShape(I, J).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    r = _rng(seed)
+    return E.Program('dot', [A, B], [C]), [r.standard_normal((M, K)).astype(np.float32),
+                                           r.standard_normal((K, N)).astype(np.float32)], FP32
+
+
+def gemm_int(E, op, dtype_name='INT32'):
+    """ExampleCppEdsl.GEMM_*, plaidml/edsl/examples/gemm.cc:16-77: contraction + C, integer types."""
+    dt = getattr(E.DType, dtype_name)
+    npdt = {'INT64': np.int64, 'UINT64': np.uint64, 'INT32': np.int32, 'INT8': np.int8}[dtype_name]
+    A, B, C = (E.Placeholder(dt, [3, 3]) for _ in range(3))
+    i, j, k = E.TensorIndexes(3)
+    O = E.Contraction().outShape(3, 3).outAccess(i, j).sum(A[i, k] * B[k, j]).build() + C
+    a = np.array([1, 1, 1, 1, 1, 2, 3, 3, 3], npdt).reshape(3, 3)
+    b = (np.array([1, 2, 3, 3, 4, 5, 3, 3, 3], npdt) if dtype_name == 'INT8'
+         else np.array([10, 11, 12, 13, 14, 15, 16, 17, 18], npdt)).reshape(3, 3)
+    return E.Program('gemm', [A, B, C], [O]), [a, b, np.ones((3, 3), npdt)], EXACT
+
+
+def funky_sum(E, op):
+    """CppEdsl.FunkySum, plaidml/edsl/tests/edsl_test.cc:2709-2719: fractional index polynomial."""
+    I = E.Placeholder(E.DType.FLOAT32, [3])
+    K = E.Placeholder(E.DType.FLOAT32, [3])
+    i, j = E.TensorIndexes(2)
+    O = E.Contraction().outShape(5).outAccess(i).sum(I[(i - j + 1) // 2] * K[j]).build()
+    return E.Program('funky_sum', [I, K], [O]), [np.array([1, 2, 3], np.float32)] * 2, EXACT
+
+
+def defract_long(E, op):
+    """test_defract_long, plaidml/edsl/tests/edsl_test.py:433-460: transposed-conv style access."""
+    shape = [1, 3, 3, 1]
+    I = E.Placeholder(E.DType.FLOAT32, shape)
+    K = E.Placeholder(E.DType.FLOAT32, shape)
+    n, x0, x1, co, ci, k0, k1 = E.TensorIndexes(7)
+    O = E.Contraction().outShape(1, 5, 5, 1).outAccess(n, x0, x1, co).sum(
+        I[n, (x0 + k0 - 1) // 2, (x1 + k1 - 1) // 2, ci] * K[2 - k0, 2 - k1, co, ci]).build()
+    return E.Program('defract_long', [I, K], [O]), [
+        np.array([[[[1], [3], [-1]], [[0], [2], [4]], [[1], [-1], [-2]]]], np.float32),
+        np.array([[[[2], [3], [4]], [[6], [-3], [-1]], [[-1], [-2], [1]]]], np.float32)], EXACT
+
+
+def max_rows(E, op):
+    """CppEdsl.Max, plaidml/edsl/tests/edsl_test.cc:576-590."""
+    A = E.Placeholder(E.DType.FLOAT32, [3, 3])
+    i, j = E.TensorIndexes(2)
+    R = E.Contraction().outShape(3).outAccess(i).max(A[i, j]).build()
+    return E.Program('max', [A], [R]), [np.array([-5, -6, -7, 4, 5, 6, 7, 8, 9], np.float32).reshape(3, 3)], EXACT
+
+
+def use_default(E, op):
+    """test_use_default, plaidml/edsl/tests/edsl_test.py:390-406: assign into one slice of an initialised output."""
+    P = E.Placeholder(E.DType.FLOAT32, [2, 7, 3, 4])
+    I = E.Placeholder(E.DType.FLOAT32, [2, 3, 4])
+    b, i1, i2 = E.TensorIndexes(3)
+    O = E.Contraction().outShape(2, 7, 3, 4).outAccess(b, 3, i1, i2).init(P).assign(I[b, i1, i2]).build()
+    r = _rng(5)
+    return E.Program('use_default', [I, P], [O]), [r.standard_normal((2, 3, 4)).astype(np.float32),
+                                                   r.standard_normal((2, 7, 3, 4)).astype(np.float32)], EXACT
+
+
+def eltwise_mix(E, op):
+    """Broadcast compare, casts, round and relu in one program (known answers of the single ops:
+    plaidml/edsl/tests/edsl_test.cc:158-182, 319-333, 631-643, 1820-1835; quantize.cc:16-32)."""
+    A = E.Placeholder(E.DType.FLOAT32, [3, 4])
+    B = E.Placeholder(E.DType.FLOAT32, [3, 1])
+    C = E.cast(A >= B, E.DType.INT32)
+    R = E.round(A * 2.5) + E.cast(C, E.DType.FLOAT32)
+    Q = E.cast(E.relu(A - B) * 256.0, E.DType.INT8)
+    r = _rng(6)
+    return E.Program('eltwise', [A, B], [C, R, Q]), [r.uniform(-0.45, 0.45, (3, 4)).astype(np.float32),
+                                                     r.uniform(-0.2, 0.2, (3, 1)).astype(np.float32)], EXACT
+
+
+def u64_add(E, op):
+    """CppEdsl.Add, plaidml/edsl/tests/edsl_test.cc:335-374 (64-bit integer elementwise)."""
+    A = E.Placeholder(E.DType.UINT64, [3, 3])
+    B = E.Placeholder(E.DType.UINT64, [3, 3])
+    a = [1, 2, 3, 4, 5, 6 + (1 << 12), 7 + (1 << 24), 8 + (1 << 32), 9 + (1 << 40)]
+    b = [1, 2 + (1 << 12), 3, 4 + (1 << 24), 5, 6 + (1 << 32), 7, 8 + (1 << 40), 9]
+    return E.Program('add', [A, B], [A + B]), [np.array(a, np.uint64).reshape(3, 3), np.array(b, np.uint64).reshape(3, 3)], EXACT
+
+
+def higher_precision_constants(E, op):
+    """CppEdsl.HigherPrecisionConstants, plaidml/edsl/tests/edsl_test.cc:140-156."""
+    A = E.Placeholder(E.DType.FLOAT32, [3, 3])
+    C = A + E.cast(E.Constant(1), E.DType.UINT64) + E.cast(E.Constant(2.0), E.DType.FLOAT64)
+    return E.Program('hpc', [A], [C]), [np.arange(1, 10, dtype=np.float32).reshape(3, 3)], EXACT
+
+
+# ---- the five workload configurations, reduced ---------------------------------------------------------
+
+def config0_gemm_f32(E, op, n=128, seed=1):
+    """configs[0]: C[M,N] += A[M,K] * B[K,N], fp32, U(-1,1)."""
+    A = E.Placeholder(E.DType.FLOAT32, [n, n])
+    B = E.Placeholder(E.DType.FLOAT32, [n, n])
+    i, j, k = E.TensorIndexes(3)
+    C = E.Contraction().outShape(n, n).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    r = _rng(seed)
+    return E.Program('gemm_f32', [A, B], [C]), [r.uniform(-1, 1, (n, n)).astype(np.float32),
+                                                r.uniform(-1, 1, (n, n)).astype(np.float32)], FP32
+
+
+def config1_conv(E, op, dtype_name='BFLOAT16', N=2, H=14, W=14, CI=64, CO=64):
+    """configs[1]: relu(conv2d(I, F) + B), NHWC, 3x3, stride 1, SAME."""
+    dt = getattr(E.DType, dtype_name)
+    I = E.Placeholder(dt, [N, H, W, CI])
+    F = E.Placeholder(dt, [3, 3, CI, CO])
+    B = E.Placeholder(dt, [CO])
+    O = op.relu(op.convolution(I, F) + B)
+    r = _rng(2)
+    Iv = r.standard_normal((N, H, W, CI)).astype(np.float32)
+    Fv = (_rng(3).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32)
+    Bv = (_rng(4).standard_normal(CO) * 0.1).astype(np.float32)
+    if dtype_name == 'BFLOAT16':
+        Iv, Fv, Bv = _bf16(Iv), _bf16(Fv), _bf16(Bv)
+    return E.Program('conv', [I, F, B], [O]), [Iv, Fv, Bv], BF16 if dtype_name == 'BFLOAT16' else FP32
+
+
+def config2_int8_gemm(E, op, M=64, N=48, K=32):
+    """configs[2]: int8 x int8 -> int32 (cast before the contraction, plaidml/edsl/tests/edsl_test.cc:509-545
+    pattern), then Q = cast(round(clip(cast(C, f32) * S, -127, 127)), int8) with S per output column."""
+    A = E.Placeholder(E.DType.INT8, [M, K])
+    B = E.Placeholder(E.DType.INT8, [K, N])
+    S = E.Placeholder(E.DType.FLOAT32, [N])
+    Ai, Bi = E.cast(A, E.DType.INT32), E.cast(B, E.DType.INT32)
+    i, j, k = E.TensorIndexes(3)
+    C = E.Contraction().outShape(M, N).outAccess(i, j).sum(Ai[i, k] * Bi[k, j]).build()
+    Q = E.cast(E.round(op.clip(E.cast(C, E.DType.FLOAT32) * S, -127.0, 127.0)), E.DType.INT8)
+    r4, r5, r6 = _rng(4), _rng(5), _rng(6)
+    return E.Program('int8_gemm', [A, B, S], [C, Q]), [r4.integers(-127, 128, (M, K), dtype=np.int8),
+                                                       r5.integers(-127, 128, (K, N), dtype=np.int8),
+                                                       r6.uniform(0.001, 0.01, N).astype(np.float32)], EXACT
+
+
+def config3_xception_block(E, op, N=2, H=19, W=19, C=32, dtype_name='BFLOAT16'):
+    """configs[3]: depthwise 3x3 -> pointwise 1x1 -> scale/shift + ReLU -> maxpool 3x3/2 with window argmax."""
+    dt = getattr(E.DType, dtype_name)
+    I = E.Placeholder(dt, [N, H, W, C])
+    Fdw = E.Placeholder(dt, [3, 3, C, 1])
+    Fpw = E.Placeholder(dt, [1, 1, C, C])
+    scale = E.Placeholder(dt, [C])
+    shift = E.Placeholder(dt, [C])
+    D = op.convolution(I, Fdw, depthwise=True)
+    P = op.convolution(D, Fpw)
+    R = op.relu(P * scale + shift)
+    M = op.pool(R, 'max', [3, 3], [2, 2], autopad=op.SAME_UPPER)
+    n, x0, x1, c, k0, k1 = E.TensorIndexes(6)
+    IX = E.index([3, 3], 0) * 3 + E.index([3, 3], 1)
+    AM = E.Contraction().outShape(M.shape).outAccess(n, x0, x1, c).max(
+        E.cond(R[n, 2 * x0 + k0 - 1, 2 * x1 + k1 - 1, c], M[n, x0, x1, c], IX[k0, k1])).build()
+    Iv = _rng(7).standard_normal((N, H, W, C)).astype(np.float32)
+    Fd = (_rng(8).standard_normal((3, 3, C, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    Fp = (_rng(9).standard_normal((1, 1, C, C)) * np.sqrt(2.0 / C)).astype(np.float32)
+    sc = _rng(10).uniform(0.5, 1.5, C).astype(np.float32)
+    sh = _rng(11).uniform(-0.5, 0.5, C).astype(np.float32)
+    vals = [Iv, Fd, Fp, sc, sh]
+    if dtype_name == 'BFLOAT16':
+        vals = [_bf16(v) for v in vals]
+    return E.Program('xception_block', [I, Fdw, Fpw, scale, shift], [M, AM]), vals, BF16 if dtype_name == 'BFLOAT16' else FP32
+
+
+def classifier_tail(E, op, N=4, C=64, K=10, dtype_name='FLOAT32'):
+    """The tail of configs[4]: global average pool -> dense + bias -> softmax."""
+    dt = getattr(E.DType, dtype_name)
+    X = E.Placeholder(dt, [N, 7, 7, C])
+    Wt = E.Placeholder(dt, [C, K])
+    b = E.Placeholder(dt, [K])
+    G = op.mean(X, [1, 2])
+    L = op.dot(G, Wt) + b
+    Y = op.softmax(L, 1)
+    vals = [_rng(20).standard_normal((N, 7, 7, C)).astype(np.float32),
+            (_rng(21).standard_normal((C, K)) * 0.2).astype(np.float32), np.zeros(K, np.float32)]
+    if dtype_name == 'BFLOAT16':
+        vals = [_bf16(v) for v in vals]
+    return E.Program('tail', [X, Wt, b], [Y, op.argmax(L, 1)]), vals, BF16 if dtype_name == 'BFLOAT16' else FP32
+
+
+def residual_block(E, op, N=2, H=8, C=64, dtype_name='BFLOAT16'):
+    """One ResNet bottleneck-style residual: relu(conv1x1(relu(conv3x3(x) + b1)) + b2 + x), weights as constants."""
+    dt = getattr(E.DType, dtype_name)
+    f1 = (_rng(30).standard_normal((3, 3, C, C)) * np.sqrt(2.0 / (9 * C))).astype(np.float32)
+    f2 = (_rng(31).standard_normal((1, 1, C, C)) * np.sqrt(2.0 / C)).astype(np.float32)
+    b1 = (_rng(32).standard_normal(C) * 0.1).astype(np.float32)
+    b2 = (_rng(33).standard_normal(C) * 0.1).astype(np.float32)
+    xv = _rng(34).standard_normal((N, H, H, C)).astype(np.float32)
+    if dtype_name == 'BFLOAT16':
+        f1, f2, b1, b2, xv = (_bf16(v) for v in (f1, f2, b1, b2, xv))
+    X = E.Placeholder(dt, [N, H, H, C])
+    F1, F2, B1, B2 = (E.Constant(v, dt) for v in (f1, f2, b1, b2))
+    Y = op.relu(op.convolution(X, F1) + B1)
+    Z = op.relu(op.convolution(Y, F2) + B2 + X)
+    return E.Program('residual', [X], [Z]), [xv], BF16 if dtype_name == 'BFLOAT16' else FP32
+
+
+ALL = {
+    'dot_f32': dot_f32,
+    'gemm_int32': lambda E, op: gemm_int(E, op, 'INT32'),
+    'gemm_int64': lambda E, op: gemm_int(E, op, 'INT64'),
+    'gemm_uint64': lambda E, op: gemm_int(E, op, 'UINT64'),
+    'gemm_int8': lambda E, op: gemm_int(E, op, 'INT8'),
+    'funky_sum': funky_sum,
+    'defract_long': defract_long,
+    'max_rows': max_rows,
+    'use_default': use_default,
+    'eltwise_mix': eltwise_mix,
+    'u64_add': u64_add,
+    'higher_precision_constants': higher_precision_constants,
+    'config0_gemm_f32': config0_gemm_f32,
+    'config1_conv_bf16': lambda E, op: config1_conv(E, op, 'BFLOAT16'),
+    'config1_conv_f32': lambda E, op: config1_conv(E, op, 'FLOAT32', CI=32, CO=48),
+    'config2_int8_gemm': config2_int8_gemm,
+    'config3_xception_block_bf16': config3_xception_block,
+    'config3_xception_block_f32': lambda E, op: config3_xception_block(E, op, C=16, dtype_name='FLOAT32'),
+    'classifier_tail_f32': classifier_tail,
+    'residual_block_bf16': residual_block,
+}

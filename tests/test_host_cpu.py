@@ -1,0 +1,112 @@
+"""Host-side logic that needs no GPU: building programs through the plaidml_* C ABI, shape / dtype
+inference, error texts, bounds, and the kernel plan the `hip` target chooses."""
+import numpy as np
+import pytest
+
+import programs
+from oracle import tile_oracle as OE
+from oracle import tile_oplib as Oop
+from plaidml_amd import edsl as E
+from plaidml_amd import op
+
+D = E.DType
+
+
+def plan_of(program, target=''):
+    program.compile(target)
+    return dict(program.passes)['hip-plan']
+
+
+@pytest.mark.parametrize('name', sorted(programs.ALL))
+def test_shapes_and_dtypes_match_the_oracle(name):
+    prog, vals, _ = programs.ALL[name](E, op)
+    oprog, ovals, _ = programs.ALL[name](OE, Oop)
+    outs = OE.run(oprog, ovals)
+    shapes = prog.outputs
+    assert len(shapes) == len(outs)
+    for s, o, ot in zip(shapes, outs, oprog.outputs):
+        assert tuple(s.sizes) == tuple(o.shape), name
+        assert int(s.dtype) == int(ot.dt), name
+    text = plan_of(prog)
+    assert text.startswith('hip plan:')
+
+
+def test_plan_choices_for_the_workload_configs():
+    t = plan_of(programs.config0_gemm_f32(E, op)[0])
+    assert 'gemm f32 m=128 n=128 k=128' in t and t.count('\n') == 2
+    t = plan_of(programs.config1_conv(E, op, 'BFLOAT16')[0])
+    assert 'conv2d bf16' in t and '+init' in t and 'tail=[relu]' in t and t.count('\n') == 2
+    t = plan_of(programs.config2_int8_gemm(E, op)[0])
+    # int8 MFMA on the un-cast operands, si32 result stored mid-tail, requantisation fused
+    assert 'gemm si8' in t and 'store' in t and 'cast:si8' in t and t.count('\n') == 2, t
+    t = plan_of(programs.config3_xception_block(E, op)[0])
+    assert 'dwconv2d bf16' in t and 'gemm bf16' in t and 'pool2d max' in t and '+window argmax' in t, t
+    assert 'contract (general)' not in t
+    t = plan_of(programs.residual_block(E, op)[0])
+    assert t.count('conv2d bf16') + t.count('gemm bf16') == 2 and 'constant' in t and 'add(t' in t, t
+
+
+def test_target_options_switch_specialisation_off():
+    prog = programs.config1_conv(E, op, 'BFLOAT16')[0]
+    t = plan_of(prog, 'hip{specialise=0,fuse=0}')
+    assert 'contract (general)' in t and 'conv2d' not in t
+    with pytest.raises(E.PlaidMLError, match='Could not find compiler target'):
+        prog.compile('llvm_cpu')
+
+
+def test_tensor_shape_strings_and_dtype_inference():
+    # plaidml/core/core_test.py / pmlc/util/shape.cc:69-91
+    assert str(E.TensorShape(D.FLOAT32, [8, 32])) == '8x32xf32'
+    assert str(E.TensorShape(D.INT8, [])) == 'si8'
+    assert str(E.TensorShape(D.BFLOAT16, [4])) == '4xbf16'
+    A = E.Placeholder(D.INT8, [3, 3])
+    B = E.Placeholder(D.INT8, [3, 3])
+    i, j, k = E.TensorIndexes(3)
+    C = E.Contraction().outShape(3, 3).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    assert C.dtype == D.INT8  # no widening: plaidml/edsl/tests/edsl_test.cc:1195-1208
+    F = E.Placeholder(D.FLOAT32, [3, 3])
+    assert (F + E.cast(E.Constant(1), D.UINT64)).dtype == D.FLOAT32
+    assert (F + E.cast(E.Constant(2.0), D.FLOAT64)).dtype == D.FLOAT64
+    assert (F < 1.0).dtype == D.BOOLEAN
+    assert E.index([3, 4], 1).dtype == D.INT32 and E.index([3, 4], 1).shape == (3, 4)
+
+
+def test_error_texts():
+    A = E.Placeholder(D.FLOAT32, [3, 4])
+    with pytest.raises(E.PlaidMLError, match='Rank mismatch in bind_dims'):
+        A.bind_dims(*E.TensorDims(3))
+    X, Y = E.TensorDim(5), E.TensorDim()
+    with pytest.raises(E.PlaidMLError, match=r'bind dims mismatch: shape=\[3, 4\] != dims=\[5, 4\]'):
+        A.bind_dims(X, Y)
+    with pytest.raises(E.PlaidMLError, match='Incompatible types'):
+        A + E.Placeholder(D.FLOAT32, [5])
+    i, = E.TensorIndexes(1)
+    with pytest.raises(E.PlaidMLError, match='ambiguous'):
+        E.Contraction().outShape(3).outAccess(i).sum(E.Constant(1)[()] * E.Constant(2)[()]).build()
+    with pytest.raises(E.PlaidMLError, match='unmatched operand types'):
+        E.select(A < 0.0, A, E.cast(A, D.FLOAT64))
+    k, = E.TensorIndexes(1)
+    P = E.Program('unbounded', [A], [E.Contraction().outShape(3).outAccess(i - k).sum(A[i - k, 0]).build()])
+    with pytest.raises(E.PlaidMLError, match="Unbounded index"):
+        P.compile()
+
+
+def test_bounds_of_same_conv_and_pool():
+    prog = programs.config1_conv(E, op, 'FLOAT32', N=1, H=5, W=5, CI=32, CO=48)[0]
+    prog.compile()
+    text = dict(prog.passes)['tile-compute-bounds']
+    # n, x0, x1, co, k0, k1, ci (first-seen order over sink, sources): pmlc/ast/builder.cc:311-323
+    assert 'idxs = [n, x0, x1, co, k0, k1, ci]' in text
+    assert 'lowerBounds = (0, 0, 0, 0, 0, 0, 0), upperBounds = (0, 4, 4, 47, 2, 2, 31)' in text
+    assert 'x0 + k0 - 1' in text
+
+
+def test_run_without_a_device_fails_loudly():
+    if E.list_devices():
+        pytest.skip('a GPU is present')
+    prog = programs.dot_f32(E, op)[0]
+    prog.compile()
+    with pytest.raises(E.PlaidMLError, match='Unable to find hip runtime'):
+        E.Executable(prog)
+    with pytest.raises(E.PlaidMLError, match='Invalid device name'):
+        E.Executable(prog, 'not a device')
