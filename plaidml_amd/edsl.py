@@ -622,10 +622,10 @@ def Constant(value, dtype=None, name=''):
         if dt == DType.BFLOAT16 and value.dtype != np.uint16:
             value = to_bf16_bits(value)
         value = np.ascontiguousarray(value, dtype=dt.into_numpy())
-        buf = Buffer(TensorShape(dt, value.shape), data=value)
-        t = Tensor(ptr=call('plaidml_expr_constant', buf.as_ptr(), name.encode()))
-        t._buffer = buf  # the adopted numpy memory must outlive the expression
-        return t
+        # copied into library-owned memory: the expression graph outlives the numpy array
+        buf = Buffer(TensorShape(dt, value.shape))
+        buf.copy_from_ndarray(value)
+        return Tensor(ptr=call('plaidml_expr_constant', buf.as_ptr(), name.encode()))
     return _wrap_tensor(value)
 
 
