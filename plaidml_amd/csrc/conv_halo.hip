@@ -1,0 +1,656 @@
+// 2-D convolution with the whole filter resident in LDS (unit stride, unit dilation).
+//
+// A persistent workgroup (one per CU, 256 threads = 4 wavefronts) keeps the packed
+// filter Bt[CO][KH*KW*CI] in LDS for its whole life and walks over tiles of 256
+// consecutive output pixels.  For each tile the input window that the tile's
+// pixels touch is brought into LDS once, zero padding included, so that every one
+// of the KH*KW taps reads its operand from LDS at a fixed offset from the pixel's
+// own position: no per-tap address checks, and each input byte crosses the
+// vector L1 once per tile instead of once per tap.  The window of the next tile
+// travels global -> registers while the MFMAs of the current one run.
+//
+// LDS window addressing.  Images are stacked with their padding rows materialised:
+// virtual row v = image * (H + pad_top + pad_bottom) + (ih + pad_top), virtual
+// column = iw + pad_left, so output pixel (image, oh, ow) and tap (kh, kw) read
+// virtual pixel (image * Hv + oh + kh, ow + kw).  A tile that runs across the end
+// of an image simply holds the padding rows between the two.
+//
+// Every pixel is 128 bytes of channels (CI * element size), stored with a 144-byte
+// stride; filter rows use an odd number of 16-byte slots too.  Both strides make
+// the 16-byte-per-lane operand reads free of bank conflicts.
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "device_common.h"
+#include "igemm_tail.h"
+#include "plans.h"
+
+namespace pml {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kBM = 256;          // output pixels per tile (64 per wavefront)
+constexpr int kBN = 64;           // output channels covered (CO <= 64)
+constexpr int kPixBytes = 128;    // channel bytes per pixel
+constexpr int kPixStride = 144;   // LDS stride of a pixel
+constexpr int kMaxLoads = 24;     // 16-byte window vectors a thread may carry for the next tile
+
+struct TileGeom {
+  int64_t m0;   // first output pixel
+  int v0;       // virtual row of that pixel
+  int nb0;      // its image
+  int ihv0;     // its row inside the padded image (= oh)
+  int nrows;    // window rows of the tile
+};
+
+__device__ inline TileGeom tile_geom(const IgemmArgs& p, int t, int Hv) {
+  TileGeom g;
+  // M < 2^31 (checked on the host): 32-bit divisions
+  const unsigned m0 = (unsigned)t * kBM;
+  const unsigned per = (unsigned)(p.OH * p.OW);
+  const unsigned nb = m0 / per;
+  const unsigned oh = (m0 - nb * per) / (unsigned)p.OW;
+  g.m0 = m0;
+  g.nb0 = (int)nb;
+  g.ihv0 = (int)oh;
+  g.v0 = (int)(nb * Hv + oh);
+  unsigned ml = m0 + kBM - 1;
+  if (ml > (unsigned)p.M - 1) ml = (unsigned)p.M - 1;
+  const unsigned nbl = ml / per;
+  const unsigned ohl = (ml - nbl * per) / (unsigned)p.OW;
+  g.nrows = (int)(nbl * Hv + ohl) - g.v0 + p.KH;
+  return g;
+}
+
+template <int KIND>
+__global__ __launch_bounds__(kThreads) void conv_halo_kernel(IgemmArgs p) {
+  constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
+  constexpr int MI = 2, NI = 2;  // 64 pixels x 64 channels per wavefront
+  typedef typename Acc<KIND>::type acc_t;
+  typedef typename Acc<KIND>::scalar accs_t;
+  typedef accs_t acc4_t __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int Hv = p.OH + p.KH - 1, Wv = p.OW + p.KW - 1;
+  const int krow = p.KH * p.KW * kPixBytes;  // filter bytes per output channel
+  const int brow = krow + 16;                // its LDS stride
+  unsigned char* const sB = smem;
+  unsigned char* const sH = smem + kBN * brow;
+
+  // ---- filter -> LDS, once ----
+  {
+    const int vecs_per_row = krow / 16;
+    const int total = kBN * vecs_per_row;
+    const i32x4_t zero4 = {0, 0, 0, 0};
+    for (int q = tid; q < total; q += kThreads) {
+      const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+      i32x4_t v = zero4;
+      if (row < p.N) v = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)row * p.ldbt * ES + vec * 16);
+      *(i32x4_t*)(sB + row * brow + vec * 16) = v;
+    }
+  }
+
+  // ---- a thread's share of a window: vector lv of pixels lp, lp + 32, ... of every row ----
+  const int lv = tid & 7, lp = tid >> 3;
+  const int nchunks = (Wv + 31) >> 5;
+  i32x4_t pf[kMaxLoads];
+  unsigned pf_ok = 0;  // bit j: pf[j] is real data (otherwise the window gets zeros: padding)
+  const i32x4_t zero4 = {0, 0, 0, 0};
+
+  auto load_window = [&](const TileGeom& g) {
+    int r = 0, c = 0, nb = g.nb0, ihv = g.ihv0;
+    pf_ok = 0;
+#pragma unroll
+    for (int j = 0; j < kMaxLoads; ++j) {
+      const int ih = ihv - p.PH;
+      const int px = c * 32 + lp;
+      const int iw = px - p.PW;
+      const bool ok = r < g.nrows && nb < p.NB && (unsigned)ih < (unsigned)p.H && px < Wv && (unsigned)iw < (unsigned)p.W;
+      const int64_t off = ok ? ((int64_t)(nb * p.H + ih) * p.W + iw) * kPixBytes + lv * 16 : 0;
+      pf[j] = *(const i32x4_t*)((const unsigned char*)p.A + off);
+      pf_ok |= (ok ? 1u : 0u) << j;
+      if (++c == nchunks) {
+        c = 0;
+        ++r;
+        if (++ihv == Hv) {
+          ihv = 0;
+          ++nb;
+        }
+      }
+    }
+  };
+  auto store_window = [&](const TileGeom& g) {
+    int r = 0, c = 0;
+#pragma unroll
+    for (int j = 0; j < kMaxLoads; ++j) {
+      const int px = c * 32 + lp;
+      if (r < g.nrows && px < Wv)
+        *(i32x4_t*)(sH + (r * Wv + px) * kPixStride + lv * 16) = ((pf_ok >> j) & 1u) ? pf[j] : zero4;
+      if (++c == nchunks) {
+        c = 0;
+        ++r;
+      }
+    }
+  };
+
+  // bias: the values of the output channels this lane owns (direct store path)
+  const bool direct = p.tail_mode == 1 && (p.init == nullptr || p.init_rs == 0);
+  accs_t cinit[NI][4][4];
+#pragma unroll
+  for (int j = 0; j < NI; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        cinit[j][g][e] = 0;
+        const int co = j * 32 + 8 * g + 4 * (lane >> 5) + e;
+        if (direct && p.init != nullptr && co < p.N) {
+          Scalar<float, int> b = load_scalar<float, int>(p.init, (int64_t)co * p.init_cs, p.init_dtype);
+          cinit[j][g][e] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+        }
+      }
+
+  int t = blockIdx.x;
+  TileGeom g = tile_geom(p, t, Hv);
+  load_window(g);
+  store_window(g);
+  __syncthreads();
+
+  const unsigned per = (unsigned)(p.OH * p.OW);
+  const int n_taps = p.KH * p.KW;
+
+  for (; t < p.n_tiles; t += gridDim.x) {
+    // ---- where this lane's pixels sit in the window ----
+    int a_base[MI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      unsigned m = (unsigned)g.m0 + wave * 64 + i * 32 + (lane & 31);
+      if (m > (unsigned)p.M - 1) m = (unsigned)p.M - 1;
+      const unsigned nb = m / per;
+      const unsigned rem = m - nb * per;
+      const unsigned oh = rem / (unsigned)p.OW, ow = rem - oh * (unsigned)p.OW;
+      a_base[i] = (((int)(nb * Hv + oh) - g.v0) * Wv + (int)ow) * kPixStride + (lane >> 5) * 16;
+    }
+    const int b_base = (lane & 31) * brow + (lane >> 5) * 16;
+
+    // ---- next tile's window: global -> registers ----
+    const int t2 = t + gridDim.x;
+    TileGeom g2 = g;
+    if (t2 < p.n_tiles) {
+      g2 = tile_geom(p, t2, Hv);
+      load_window(g2);
+    }
+
+    acc_t acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    // ---- taps x four 32-byte K-blocks; fragments are fetched one K-block ahead ----
+    i32x4_t fa[2][MI], fb[2][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(sH + a_base[i]);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow);
+    int kh = 0, kw = 0;
+    for (int tap = 0; tap < n_taps; ++tap) {
+      const int a_tap = (kh * Wv + kw) * kPixStride;
+      if (++kw == p.KW) {
+        kw = 0;
+        ++kh;
+      }
+      const bool last = tap + 1 == n_taps;
+      const int a_next = last ? a_tap : (kh * Wv + kw) * kPixStride;
+      const int b_tap = tap * kPixBytes;
+      const int b_next = last ? b_tap : b_tap + kPixBytes;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        const int ao = ks < 3 ? a_tap + (ks + 1) * 32 : a_next;
+        const int bo = ks < 3 ? b_tap + (ks + 1) * 32 : b_next;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[nxt][i] = *(const i32x4_t*)(sH + a_base[i] + ao);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) fb[nxt][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow + bo);
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j) mma_block<KIND>(acc[i][j], fb[cur][j], fa[cur][i]);
+      }
+    }
+
+    // In a 32x32 block a lane owns pixel lane%32 and the output channels
+    // 8*(r/4) + 4*(lane/32) + r%4: four consecutive channels per register quad.
+    if (direct) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int64_t m = g.m0 + wave * 64 + i * 32 + (lane & 31);
+        if (m < p.M) {
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int co = j * 32 + 8 * q + 4 * (lane >> 5);
+              if (co < p.N) {
+                accs_t v4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][4 * q + e] + cinit[j][q][e];
+                if (KIND == KIND_I8) {
+                  i32x4_t w;
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) w[e] = (p.tail_relu && (int)v4[e] < 0) ? 0 : (int)v4[e];
+                  *(i32x4_t*)((int*)p.C + m * p.ldc + co) = w;
+                } else if (p.out_dtype == PML_HIP_BF16) {
+                  uint32_t h[4];
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) {
+                    h[e] = f32_to_bf16_bits((float)v4[e]);
+                    if (p.tail_relu && (h[e] & 0x8000u) && (h[e] & 0x7fffu) <= 0x7f80u && (h[e] & 0x7fffu) != 0) h[e] = 0;
+                  }
+                  *(uint2*)((uint16_t*)p.C + m * p.ldc + co) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                } else {
+                  f32x4_t w;
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) w[e] = (p.tail_relu && (float)v4[e] < 0.f) ? 0.f : (float)v4[e];
+                  *(f32x4_t*)((float*)p.C + m * p.ldc + co) = w;
+                }
+              }
+            }
+        }
+      }
+      __syncthreads();  // every wavefront is done reading the window
+    } else {
+      __syncthreads();
+      constexpr int CS = kBN + 4;
+      accs_t* ctile = (accs_t*)sH;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            acc4_t w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = acc[i][j][4 * q + e];
+            *(acc4_t*)&ctile[(wave * 64 + i * 32 + (lane & 31)) * CS + j * 32 + 8 * q + 4 * (lane >> 5)] = w;
+          }
+      __syncthreads();
+      tile_tail<KIND, kBM, kBN, kThreads>(p, ctile, g.m0, 0, tid);
+      __syncthreads();
+    }
+    if (t2 < p.n_tiles) store_window(g2);
+    g = g2;
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 3x3 filters, exactly 64 output channels, tail = bias? relu? store: the hot case.
+//
+// Same data movement as above, with the instruction streams arranged so that a
+// wavefront's matrix pipe stays fed while it does everything else:
+//  * the nine taps are unrolled, so the whole K loop of a tile is one basic block;
+//  * the result of tile t stays in registers and its bias / relu / convert / store
+//    work is cut into 16 pieces that sit between the MFMAs of tile t+1
+//    (two accumulator sets alternate roles);
+//  * window loads and output stores are buffer instructions: an offset beyond the
+//    buffer reads zeros / drops the store, which is how padding, image ends and the
+//    ragged last tile are handled without any branch in the stream.
+// NCH = 32-pixel chunks per window row (1 or 2).
+// ---------------------------------------------------------------------------
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
+constexpr int kFar = 0x40000000;              // beyond any input this kernel accepts (<= 2^30 bytes); two of them still are
+
+template <int KIND, int NCH>
+__global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
+  constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
+  constexpr int MI = 2, NI = 2;
+  constexpr int OES = KIND == KIND_BF16 ? 2 : 4;  // bytes per output element (bf16 -> bf16, fp32 -> fp32, int8 -> int32)
+  constexpr int kTaps = 9;
+  constexpr int krow = kTaps * kPixBytes, brow = krow + 16;
+  constexpr int kRows = kMaxLoads / NCH;
+  typedef typename Acc<KIND>::type acc_t;
+  typedef typename Acc<KIND>::scalar accs_t;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* const sB = smem;
+  unsigned char* const sH = smem + kBN * brow;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int Hv = p.OH + 2, Wv = p.OW + 2;
+
+  {
+    constexpr int vecs_per_row = krow / 16;
+    for (int q = tid; q < kBN * vecs_per_row; q += kThreads) {
+      const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+      *(i32x4_t*)(sB + row * brow + vec * 16) =
+          *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)row * p.ldbt * ES + vec * 16);
+    }
+  }
+
+  const __amdgpu_buffer_rsrc_t rin =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)((int64_t)p.NB * p.H * p.W * kPixBytes), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t rout =
+      __builtin_amdgcn_make_buffer_rsrc(p.C, 0, (int)(p.M * p.ldc * OES), kRsrcFlags);
+
+  // ---- a thread's share of a window: vector lv of pixels lp (+32) of every row ----
+  const int lv = tid & 7, lp = tid >> 3;
+  int g_off[NCH], l_off[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int px = c * 32 + lp, iw = px - p.PW;
+    g_off[c] = (px < Wv && (unsigned)iw < (unsigned)p.W) ? iw * kPixBytes + lv * 16 : kFar;
+    l_off[c] = px * kPixStride + lv * 16;
+  }
+  const bool chunk0 = lp < Wv, chunk1 = lp + 32 < Wv;  // does this thread's pixel of the chunk exist?
+
+  u32x4_t pf[kMaxLoads];
+  auto load_window = [&](const TileGeom& g) {
+    int nb = g.nb0, ihv = g.ihv0;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int ih = ihv - p.PH;
+      const bool row_ok = r < g.nrows && nb < p.NB && (unsigned)ih < (unsigned)p.H;
+      const int row_base = row_ok ? (nb * p.H + ih) * p.W * kPixBytes : kFar;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) pf[r * NCH + c] = __builtin_amdgcn_raw_buffer_load_b128(rin, row_base + g_off[c], 0, 0);
+      if (++ihv == Hv) {
+        ihv = 0;
+        ++nb;
+      }
+    }
+  };
+  auto store_window = [&]() {
+    const int row_pitch = Wv * kPixStride;
+    if (chunk0) {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r)
+        if (r < p.halo_rows) *(u32x4_t*)(sH + r * row_pitch + l_off[0]) = pf[r * NCH];
+    }
+    if (NCH == 2 && chunk1) {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r)
+        if (r < p.halo_rows) *(u32x4_t*)(sH + r * row_pitch + l_off[NCH - 1]) = pf[r * NCH + NCH - 1];
+    }
+  };
+
+  // bias of the output channels this lane owns; relu as a lower clamp (x < lo ? lo : x keeps NaN)
+  accs_t cinit[NI][4][4];
+#pragma unroll
+  for (int j = 0; j < NI; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        cinit[j][q][e] = 0;
+        if (p.init != nullptr) {
+          Scalar<float, int> b = load_scalar<float, int>(p.init, (int64_t)(j * 32 + 8 * q + 4 * (lane >> 5) + e) * p.init_cs, p.init_dtype);
+          cinit[j][q][e] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+        }
+      }
+  const float lo_f = p.tail_relu ? 0.f : -__builtin_inff();
+  const int lo_i = p.tail_relu ? 0 : (int)0x80000000;
+
+  const unsigned per = (unsigned)(p.OH * p.OW);
+  const int b_base = (lane & 31) * brow + (lane >> 5) * 16;
+
+  // where a tile's pixels of this lane sit: in the window (LDS) and in the output (bytes)
+  auto place = [&](const TileGeom& g, int (&a_base)[MI], int (&m_off)[MI]) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const unsigned m = (unsigned)g.m0 + wave * 64 + i * 32 + (lane & 31);
+      const bool ok = m < (unsigned)p.M;
+      const unsigned mc = ok ? m : (unsigned)p.M - 1;
+      const unsigned nb = mc / per;
+      const unsigned rem = mc - nb * per;
+      const unsigned oh = rem / (unsigned)p.OW, ow = rem - oh * (unsigned)p.OW;
+      a_base[i] = (((int)(nb * Hv + oh) - g.v0) * Wv + (int)ow) * kPixStride + (lane >> 5) * 16;
+      m_off[i] = ok ? (int)((m * (unsigned)p.ldc + 4 * (lane >> 5)) * OES) : (int)0x80000000;
+    }
+  };
+
+  // one of the 16 pieces of a finished tile: 4 consecutive channels of one pixel
+  auto finish_piece = [&](const acc_t (&acc)[MI][NI], const int (&m_off)[MI], int pc) {
+    const int i = pc >> 3, j = (pc >> 2) & 1, q = pc & 3;
+    const int off = m_off[i] + (j * 32 + 8 * q) * OES;
+    if (KIND == KIND_I8) {
+      u32x4_t w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int v = (int)acc[i][j][4 * q + e] + (int)cinit[j][q][e];
+        w[e] = (unsigned)(v < lo_i ? lo_i : v);
+      }
+      __builtin_amdgcn_raw_buffer_store_b128(w, rout, off, 0, 0);
+    } else {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = (float)acc[i][j][4 * q + e] + (float)cinit[j][q][e];
+        v[e] = v[e] < lo_f ? lo_f : v[e];
+      }
+      if (KIND == KIND_BF16) {
+        const f32x2_t a01 = {v[0], v[1]}, a23 = {v[2], v[3]};
+        const bf16x2_t h01 = __builtin_convertvector(a01, bf16x2_t), h23 = __builtin_convertvector(a23, bf16x2_t);
+        unsigned w0, w1;
+        __builtin_memcpy(&w0, &h01, 4);
+        __builtin_memcpy(&w1, &h23, 4);
+        const u32x2_t w = {w0, w1};
+        __builtin_amdgcn_raw_buffer_store_b64(w, rout, off, 0, 0);
+      } else {
+        u32x4_t w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = __float_as_uint(v[e]);
+        __builtin_amdgcn_raw_buffer_store_b128(w, rout, off, 0, 0);
+      }
+    }
+  };
+
+  // K loop of one tile (36 K-blocks of 32 bytes); with EPI the 16 pieces of the previous tile ride along
+  auto k_loop = [&](acc_t (&acc)[MI][NI], const int (&a_base)[MI], auto epi, const acc_t (&pacc)[MI][NI],
+                    const int (&pm_off)[MI]) {
+    constexpr bool EPI = decltype(epi)::value;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    i32x4_t fa[2][MI], fb[2][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(sH + a_base[i]);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow);
+#pragma unroll
+    for (int s = 0; s < kTaps * 4; ++s) {
+      const int cur = s & 1, nxt = cur ^ 1;
+      if (s + 1 < kTaps * 4) {
+        const int tap = (s + 1) >> 2, ks = (s + 1) & 3;
+        const int ao = ((tap / 3) * Wv + tap % 3) * kPixStride + ks * 32;
+        const int bo = tap * kPixBytes + ks * 32;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[nxt][i] = *(const i32x4_t*)(sH + a_base[i] + ao);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) fb[nxt][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow + bo);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) mma_block<KIND>(acc[i][j], fb[cur][j], fa[cur][i]);
+      if (EPI && (s & 1) == 0 && (s >> 1) < 16) finish_piece(pacc, pm_off, s >> 1);
+    }
+  };
+
+  acc_t accA[MI][NI], accB[MI][NI];
+  int a_base[MI], m_offA[MI], m_offB[MI];
+
+  int t = blockIdx.x;
+  TileGeom g = tile_geom(p, t, Hv);
+  load_window(g);
+  store_window();
+  __syncthreads();
+
+  // advance: the window of tile t2 (already in flight) replaces the current one
+  auto next_tile = [&](int t2, const TileGeom& g2) {
+    __syncthreads();  // every wavefront is done reading the window
+    if (t2 < p.n_tiles) store_window();
+    __syncthreads();
+    t = t2;
+    g = g2;
+  };
+
+  {
+    place(g, a_base, m_offA);
+    const int t2 = t + gridDim.x;
+    TileGeom g2 = g;
+    if (t2 < p.n_tiles) {
+      g2 = tile_geom(p, t2, Hv);
+      load_window(g2);
+    }
+    k_loop(accA, a_base, std::false_type(), accA, m_offA);
+    next_tile(t2, g2);
+  }
+  for (;;) {
+    if (t >= p.n_tiles) {
+#pragma unroll
+      for (int pc = 0; pc < 16; ++pc) finish_piece(accA, m_offA, pc);
+      break;
+    }
+    {
+      place(g, a_base, m_offB);
+      const int t2 = t + gridDim.x;
+      TileGeom g2 = g;
+      if (t2 < p.n_tiles) {
+        g2 = tile_geom(p, t2, Hv);
+        load_window(g2);
+      }
+      k_loop(accB, a_base, std::true_type(), accA, m_offA);
+      next_tile(t2, g2);
+    }
+    if (t >= p.n_tiles) {
+#pragma unroll
+      for (int pc = 0; pc < 16; ++pc) finish_piece(accB, m_offB, pc);
+      break;
+    }
+    {
+      place(g, a_base, m_offA);
+      const int t2 = t + gridDim.x;
+      TileGeom g2 = g;
+      if (t2 < p.n_tiles) {
+        g2 = tile_geom(p, t2, Hv);
+        load_window(g2);
+      }
+      k_loop(accA, a_base, std::true_type(), accB, m_offB);
+      next_tile(t2, g2);
+    }
+  }
+}
+
+template <int KIND, int NCH>
+hipError_t launch3x3(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
+  auto kern = conv_halo3x3_kernel<KIND, NCH>;
+  static size_t attr_lds = 0;
+  if (lds > attr_lds) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    attr_lds = lds;
+  }
+  const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), lds, s, a);
+  return hipGetLastError();
+}
+
+template <int KIND>
+hipError_t launch(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
+  auto kern = conv_halo_kernel<KIND>;
+  static size_t attr_lds = 0;
+  if (lds > attr_lds) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    attr_lds = lds;
+  }
+  const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), lds, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+size_t conv_halo_prepare(int kind, IgemmArgs* a) {
+  const int es = kind == KIND_BF16 ? 2 : (kind == KIND_I8 ? 1 : 4);
+  if (a->SH != 1 || a->SW != 1 || a->DH != 1 || a->DW != 1) return 0;
+  if ((int64_t)a->CI * es != kPixBytes) return 0;
+  if (a->N > kBN || (a->N & 7) != 0 || (a->ldc & 3) != 0) return 0;
+  if (a->PH >= a->KH || a->PW >= a->KW) return 0;
+  // the padded image must be exactly what the output geometry implies
+  const int Hv = a->OH + a->KH - 1, Wv = a->OW + a->KW - 1;
+  if (Hv < a->H + a->PH || Wv < a->W + a->PW) return 0;
+  if (a->M >= ((int64_t)1 << 31) - kBM) return 0;
+  const int64_t per = (int64_t)a->OH * a->OW;
+  const int64_t n_tiles = (a->M + kBM - 1) / kBM;
+  int max_rows = 0;
+  for (int64_t t = 0; t < n_tiles; ++t) {
+    const int64_t m0 = t * kBM;
+    int64_t ml = m0 + kBM - 1;
+    if (ml > a->M - 1) ml = a->M - 1;
+    const int64_t v0 = (m0 / per) * Hv + (m0 % per) / a->OW;
+    const int64_t vl = (ml / per) * Hv + (ml % per) / a->OW;
+    const int rows = (int)(vl - v0) + a->KH;
+    if (rows > max_rows) max_rows = rows;
+  }
+  const int nchunks = (Wv + 31) / 32;
+  if ((int64_t)max_rows * nchunks > kMaxLoads) return 0;
+  const size_t filter = (size_t)kBN * ((size_t)a->KH * a->KW * kPixBytes + 16);
+  size_t window = (size_t)max_rows * Wv * kPixStride;
+  const size_t ctile = (size_t)kBM * (kBN + 4) * 4;
+  if (window < ctile) window = ctile;
+  const size_t total = filter + window;
+  if (total > 160 * 1024) return 0;
+  a->halo_rows = max_rows;
+  a->n_tiles = (int)n_tiles;
+  // the pipelined 3x3 kernel: fast tail only, 64 channels out, buffer-addressable operands
+  const int out_es = kind == KIND_BF16 ? 2 : 4;
+  const bool out_fits = kind == KIND_BF16 ? a->out_dtype == PML_HIP_BF16 : true;
+  a->halo_variant = (a->KH == 3 && a->KW == 3 && a->N == kBN && a->tail_mode == 1 && a->init_rs == 0 && out_fits &&
+                     (int64_t)a->NB * a->H * a->W * kPixBytes <= ((int64_t)1 << 30) &&
+                     a->M * a->ldc * out_es < ((int64_t)1 << 31) && nchunks <= 2)
+                        ? nchunks
+                        : 0;
+  return total;
+}
+
+hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s) {
+  if (a.halo_variant == 1) {
+    switch (kind) {
+      case KIND_F32: return launch3x3<KIND_F32, 1>(a, lds_bytes, n_cus, s);
+      case KIND_BF16: return launch3x3<KIND_BF16, 1>(a, lds_bytes, n_cus, s);
+      case KIND_I8: return launch3x3<KIND_I8, 1>(a, lds_bytes, n_cus, s);
+    }
+  } else if (a.halo_variant == 2) {
+    switch (kind) {
+      case KIND_F32: return launch3x3<KIND_F32, 2>(a, lds_bytes, n_cus, s);
+      case KIND_BF16: return launch3x3<KIND_BF16, 2>(a, lds_bytes, n_cus, s);
+      case KIND_I8: return launch3x3<KIND_I8, 2>(a, lds_bytes, n_cus, s);
+    }
+  }
+  switch (kind) {
+    case KIND_F32: return launch<KIND_F32>(a, lds_bytes, n_cus, s);
+    case KIND_BF16: return launch<KIND_BF16>(a, lds_bytes, n_cus, s);
+    case KIND_I8: return launch<KIND_I8>(a, lds_bytes, n_cus, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace pml

@@ -1,0 +1,154 @@
+// Internal: pieces shared by the MFMA kernels (igemm.hip, conv_halo.hip): the
+// accumulator types, one 32-byte K-block of MFMA work per element kind, and the
+// tail that walks an accumulator tile staged in LDS.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "device_common.h"
+#include "plans.h"
+
+namespace pml {
+
+template <int KIND>
+struct Acc;
+template <>
+struct Acc<KIND_BF16> {
+  typedef f32x16_t type;
+  typedef float scalar;
+};
+template <>
+struct Acc<KIND_F32> {
+  typedef f32x16_t type;
+  typedef float scalar;
+};
+template <>
+struct Acc<KIND_I8> {
+  typedef i32x16_t type;
+  typedef int scalar;
+};
+
+template <int KIND>
+__device__ inline void mma_block(typename Acc<KIND>::type& acc, const i32x4_t& a, const i32x4_t& b);
+
+template <>
+__device__ inline void mma_block<KIND_BF16>(f32x16_t& acc, const i32x4_t& a, const i32x4_t& b) {
+  bf16x8_t av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+}
+template <>
+__device__ inline void mma_block<KIND_I8>(i32x16_t& acc, const i32x4_t& a, const i32x4_t& b) {
+  acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+}
+template <>
+__device__ inline void mma_block<KIND_F32>(f32x16_t& acc, const i32x4_t& a, const i32x4_t& b) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[j]), __int_as_float(b[j]), acc, 0, 0, 0);
+  }
+}
+
+// Tail over an accumulator tile held in LDS as ctile[BM][BN + 4] (row-major):
+// adds the initial value, runs the fused elementwise chain once per element and
+// stores contiguous 8/16-byte pieces.  A thread owns 4 consecutive columns; rows
+// advance by NTHREADS / (BN / 4) per pass.
+template <int KIND, int BM, int BN, int NTHREADS>
+__device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc<KIND>::scalar* ctile, int64_t m0,
+                                          int64_t n0, int tid) {
+  typedef typename Acc<KIND>::scalar accs_t;
+  constexpr int CS = BN + 4;
+  constexpr int kThreads = NTHREADS;
+  constexpr int TPR = BN / 4;
+  constexpr int RPP = kThreads / TPR;
+  const int c4 = (tid % TPR) * 4;
+  const int64_t n = n0 + c4;
+  if (n >= p.N) return;
+  const bool full4 = n + 3 < p.N;
+  const bool fast = p.tail_mode == 1 && full4 && (p.ldc & 3) == 0;
+  // a per-column start value (bias) is the same for every row of this thread
+  const bool col_init = p.init != nullptr && p.init_rs == 0;
+  accs_t cinit[4] = {0, 0, 0, 0};
+  if (col_init) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (n + q < p.N) {
+        Scalar<float, int> b = load_scalar<float, int>(p.init, (n + q) * p.init_cs, p.init_dtype);
+        cinit[q] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+      }
+    }
+  }
+  for (int row = tid / TPR; row < BM; row += RPP) {
+    const int64_t m = m0 + row;
+    if (m >= p.M) break;
+    accs_t v4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v4[q] = ctile[row * CS + c4 + q];
+    if (col_init) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v4[q] += cinit[q];
+    } else if (p.init) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (n + q < p.N) {
+          Scalar<float, int> b = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
+          v4[q] += KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+        }
+      }
+    }
+    if (fast) {
+      if (KIND == KIND_I8) {
+        i32x4_t w;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) w[q] = (p.tail_relu && (int)v4[q] < 0) ? 0 : (int)v4[q];
+        *(i32x4_t*)((int*)p.C + m * p.ldc + n) = w;
+      } else if (p.out_dtype == PML_HIP_BF16) {
+        uint32_t h[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          h[q] = f32_to_bf16_bits((float)v4[q]);
+          // relu on the rounded value: negative, non-NaN, non-zero -> 0  (x < 0 ? 0 : x)
+          if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
+        }
+        *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+      } else {
+        f32x4_t w;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) w[q] = (p.tail_relu && (float)v4[q] < 0.f) ? 0.f : (float)v4[q];
+        *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
+      }
+      continue;
+    }
+    for (int q = 0; q < 4; ++q) {
+      if (n + q >= p.N) break;
+      const int64_t nn = n + q;
+      Scalar<float, int> v;
+      v.f = 0;
+      v.i = 0;
+      int cur = p.out_dtype;
+      if (KIND == KIND_I8)
+        v.i = (int)v4[q];
+      else
+        v.f = round_float_to<float>(cur, (float)v4[q]);
+      const int64_t o = m * p.ldc + nn;
+      if (p.tail_mode == 1) {
+        if (p.tail_relu) {
+          if (KIND == KIND_I8)
+            v.i = v.i < 0 ? 0 : v.i;
+          else
+            v.f = v.f < 0.f ? 0.f : v.f;
+        }
+      } else {
+        int64_t off[PML_HIP_MAX_EPI_OPERANDS];
+#pragma unroll
+        for (int k = 0; k < PML_HIP_MAX_EPI_OPERANDS; ++k)
+          off[k] = k < p.tail.n_operands ? m * p.tail.operand_row_stride[k] + nn * p.tail.operand_col_stride[k] : 0;
+        v = run_tail<float, int>(p.tail, v, &cur, p.operands, off, p.outs, o);
+      }
+      store_scalar<float, int>(p.C, o, cur, v);
+    }
+  }
+}
+
+}  // namespace pml

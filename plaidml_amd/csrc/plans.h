@@ -30,6 +30,9 @@ struct IgemmArgs {
   int64_t ldc;
   // convolution geometry (CONV instantiations only)
   int H, W, CI, OH, OW, KH, KW, SH, SW, PH, PW, DH, DW;
+  // resident-filter convolution only: image count, LDS rows of the input window, number of 256-pixel tiles
+  // halo_variant: 0 = general resident kernel, 1 / 2 = pipelined 3x3 kernel with that many 32-pixel chunks per row
+  int NB, halo_rows, n_tiles, halo_variant;
   // result type of the contraction, optional initial value
   int out_dtype;
   const void* init;
@@ -45,6 +48,10 @@ struct IgemmArgs {
 };
 
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
+// Resident-filter convolution (conv_halo.hip): LDS bytes a shape needs, or 0 when the
+// shape does not qualify; `a.halo_rows` and `a.n_tiles` are filled in by conv_halo_prepare.
+size_t conv_halo_prepare(int kind, IgemmArgs* a);
+hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s);
 hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int64_t N, int64_t ldb, int64_t ldbt,
                           hipStream_t s);
 

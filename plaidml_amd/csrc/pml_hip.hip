@@ -44,6 +44,9 @@ struct Plan {
   int64_t bt_ld = 0;
   size_t bt_bytes = 0;
   bool packed = false;
+  // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
+  size_t halo_lds = 0;
+  int halo_rows = 0, halo_tiles = 0, halo_variant = 0, n_cus = 0;
   std::string text;
   ~Plan() {
     if (bt) (void)hipFree(bt);
@@ -116,6 +119,46 @@ bool valid_tail(const pml_hip_epilogue& t) {
     if (dt_size(op.dtype) == 8 && op.opcode != PML_HIP_EPI_STORE) return false;  // 64-bit steps: general path only
   }
   return true;
+}
+
+// Everything of the kernel arguments that the descriptor fixes (no operand pointers).
+void conv_args(const Plan* p, IgemmArgs& g) {
+  const pml_hip_conv2d_desc& d = p->conv;
+  const int64_t K = d.kh * d.kw * d.ci;
+  std::memset(&g, 0, sizeof g);
+  g.M = d.n * d.oh * d.ow;
+  g.N = d.co;
+  g.K = K;
+  g.A = nullptr;
+  g.Bt = p->bt;
+  g.ldbt = p->bt_ld;
+  g.C = nullptr;
+  g.ldc = d.co;
+  g.H = (int)d.h;
+  g.W = (int)d.w;
+  g.CI = (int)d.ci;
+  g.OH = (int)d.oh;
+  g.OW = (int)d.ow;
+  g.KH = (int)d.kh;
+  g.KW = (int)d.kw;
+  g.SH = (int)d.stride_h;
+  g.SW = (int)d.stride_w;
+  g.PH = (int)d.pad_h;
+  g.PW = (int)d.pad_w;
+  g.DH = (int)d.dil_h;
+  g.DW = (int)d.dil_w;
+  g.out_dtype = d.out_dtype;
+  g.init = nullptr;
+  g.init_dtype = d.init_dtype;
+  g.init_rs = d.init_row_stride;
+  g.init_cs = d.init_col_stride;
+  g.c_dtype = d.c_dtype;
+  classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
+  g.tail = d.tail;
+  g.NB = (int)d.n;
+  g.halo_rows = p->halo_rows;
+  g.n_tiles = p->halo_tiles;
+  g.halo_variant = p->halo_variant;
 }
 
 }  // namespace
@@ -354,11 +397,30 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     fail("conv2d: cannot allocate the packed filter");
     return 0;
   }
+  {
+    // Filter small enough to stay in LDS: persistent resident-filter kernel (PML_HIP_CONV=igemm keeps the generic one).
+    const char* e = std::getenv("PML_HIP_CONV");
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (!(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
+        hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+      IgemmArgs g;
+      conv_args(p, g);
+      const size_t lds = conv_halo_prepare(kind, &g);
+      if (lds && lds <= prop.sharedMemPerBlock) {
+        p->halo_lds = lds;
+        p->halo_rows = g.halo_rows;
+        p->halo_tiles = g.n_tiles;
+        p->halo_variant = g.halo_variant;
+        p->n_cus = prop.multiProcessorCount;
+      }
+    }
+  }
   char buf[256];
   std::snprintf(buf, sizeof buf, "conv2d %s n=%lld %lldx%lldx%lld k=%lldx%lld co=%lld -> %lldx%lld (implicit gemm m=%lld n=%lld k=%lld) tile=%s",
                 d->in_dtype == PML_HIP_F32 ? "f32" : d->in_dtype == PML_HIP_BF16 ? "bf16" : "i8", (long long)d->n,
                 (long long)d->h, (long long)d->w, (long long)d->ci, (long long)d->kh, (long long)d->kw, (long long)d->co,
-                (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, tile_name(p->tile));
+                (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, p->halo_lds ? (p->halo_variant ? "256x64 resident filter, pipelined 3x3" : "256x64 resident filter") : tile_name(p->tile));
   p->text = buf;
   return (int64_t)(intptr_t)p;
 }
@@ -378,36 +440,10 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   if (filter && check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   IgemmArgs g;
-  std::memset(&g, 0, sizeof g);
-  g.M = d.n * d.oh * d.ow;
-  g.N = d.co;
-  g.K = K;
+  conv_args(p, g);
   g.A = input;
-  g.Bt = p->bt;
-  g.ldbt = p->bt_ld;
   g.C = output;
-  g.ldc = d.co;
-  g.H = (int)d.h;
-  g.W = (int)d.w;
-  g.CI = (int)d.ci;
-  g.OH = (int)d.oh;
-  g.OW = (int)d.ow;
-  g.KH = (int)d.kh;
-  g.KW = (int)d.kw;
-  g.SH = (int)d.stride_h;
-  g.SW = (int)d.stride_w;
-  g.PH = (int)d.pad_h;
-  g.PW = (int)d.pad_w;
-  g.DH = (int)d.dil_h;
-  g.DW = (int)d.dil_w;
-  g.out_dtype = d.out_dtype;
   g.init = d.init_kind ? init : nullptr;
-  g.init_dtype = d.init_dtype;
-  g.init_rs = d.init_row_stride;
-  g.init_cs = d.init_col_stride;
-  g.c_dtype = d.c_dtype;
-  classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
-  g.tail = d.tail;
   for (int i = 0; i < d.tail.n_operands; ++i) {
     if (!operands || !operands[i]) return fail("conv2d_invoke: missing tail operand");
     g.operands[i] = operands[i];
@@ -416,6 +452,8 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("conv2d_invoke: missing extra output");
+  if (p->halo_lds)
+    return check(conv_halo_launch(p->mfma_kind, g, p->halo_lds, p->n_cus, (hipStream_t)s), "conv_halo_launch");
   return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
 }
 

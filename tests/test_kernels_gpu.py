@@ -236,6 +236,76 @@ def test_conv_bf16_full_size_properties():
         np.testing.assert_allclose(out[n, y, x], ref, rtol=BF16_RTOL, atol=2e-2)
 
 
+def _conv_case(kind, shape, kh, kw, co, autopad, seed):
+    rng = np.random.default_rng(seed)
+    if kind == 'i8':
+        Iv = rng.integers(-127, 128, shape, dtype=np.int8)
+        Fv = rng.integers(-127, 128, (kh, kw, shape[3], co), dtype=np.int8)
+        return Iv, Fv
+    Iv = rng.standard_normal(shape).astype(np.float32)
+    Fv = (rng.standard_normal((kh, kw, shape[3], co)) * np.sqrt(2.0 / (kh * kw * shape[3]))).astype(np.float32)
+    if kind == 'bf16':
+        Iv, Fv = E.round_bf16(Iv), E.round_bf16(Fv)
+    return Iv, Fv
+
+
+# Shapes the resident-filter convolution takes (unit stride, 128 bytes of channels per pixel, CO <= 64):
+# tiles of 256 pixels that run across image ends, odd widths, VALID and SAME windows, non-square filters.
+RESIDENT_CASES = [('bf16', (3, 9, 30, 64), 3, 3, 64, op.SAME_UPPER), ('bf16', (2, 20, 40, 64), 3, 3, 40, op.VALID),
+                  ('bf16', (2, 12, 33, 64), 2, 3, 48, op.VALID), ('bf16', (5, 17, 19, 64), 3, 3, 64, op.SAME_UPPER),
+                  ('f32', (2, 12, 36, 32), 3, 3, 64, op.SAME_UPPER), ('i8', (2, 10, 30, 128), 3, 3, 64, op.SAME_UPPER)]
+
+
+@pytest.mark.parametrize('kind,shape,kh,kw,co,autopad', RESIDENT_CASES)
+def test_conv_resident_filter(kind, shape, kh, kw, co, autopad, capsys):
+    Iv, Fv = _conv_case(kind, shape, kh, kw, co, autopad, 21)
+    rng = np.random.default_rng(22)
+    if kind == 'i8':
+        out = run_conv(Iv, Fv, hk.I8, hk.I32, autopad=autopad)
+        assert 'resident filter' in capsys.readouterr().out
+        I, F = E.Placeholder(D.INT8, Iv.shape), E.Placeholder(D.INT8, Fv.shape)
+        O = op.convolution(E.cast(I, D.INT32), E.cast(F, D.INT32), strides=[1, 1], autopad=autopad)
+        ref, = E.run(E.Program('c', [I, F], [O]), [Iv, Fv])
+        np.testing.assert_array_equal(out, ref)
+        return
+    bias = rng.standard_normal(co).astype(np.float32)
+    if kind == 'bf16':
+        bias = E.round_bf16(bias)
+        out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, autopad=autopad, bias=bf16(bias), relu=True))
+        ref = oracle_conv(Iv, Fv, D.BFLOAT16, 1, autopad, bias, True)
+        np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
+    else:
+        out = run_conv(Iv, Fv, hk.F32, hk.F32, autopad=autopad, bias=bias, relu=True)
+        ref = oracle_conv(Iv, Fv, D.FLOAT32, 1, autopad, bias, True)
+        np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4)
+    assert 'resident filter' in capsys.readouterr().out
+
+
+def test_conv_resident_filter_general_tail(capsys):
+    # relu(conv(I, F) + R) with a full-size residual R: the tail is interpreted, not the fast store path
+    shape, co = (3, 9, 30, 64), 64
+    Iv, Fv = _conv_case('bf16', shape, 3, 3, co, op.SAME_UPPER, 23)
+    Rv = E.round_bf16(np.random.default_rng(24).standard_normal((3, 9, 30, co)).astype(np.float32))
+    tail = hk.make_tail(ops=[(hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_RELU, hk.BF16, 0, 0, 0.0)],
+                        operands=[(hk.BF16, co, 1)])
+    out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, tail=tail, operands=[bf16(Rv)]))
+    assert 'resident filter' in capsys.readouterr().out
+    I, F, R = E.Placeholder(D.BFLOAT16, Iv.shape), E.Placeholder(D.BFLOAT16, Fv.shape), E.Placeholder(D.BFLOAT16, Rv.shape)
+    O = op.relu(op.convolution(I, F, strides=[1, 1], autopad=op.SAME_UPPER) + R)
+    ref, = E.run(E.Program('c', [I, F, R], [O]), [Iv, Fv, Rv])
+    np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
+
+
+def test_conv_resident_filter_matches_generic_kernel(monkeypatch):
+    # same inputs through the generic implicit-GEMM kernel: both accumulate in fp32 and round once
+    Iv, Fv = _conv_case('bf16', (4, 28, 28, 64), 3, 3, 64, op.SAME_UPPER, 25)
+    bias = bf16(E.round_bf16(np.random.default_rng(26).standard_normal(64).astype(np.float32)))
+    a = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
+    monkeypatch.setenv('PML_HIP_CONV', 'igemm')
+    b = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
+    np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
+
+
 def test_dwconv_pool_bf16():
     rng = np.random.default_rng(9)
     N, H, W, C = 2, 19, 19, 32
