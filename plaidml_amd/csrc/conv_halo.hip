@@ -44,21 +44,26 @@ struct TileGeom {
   int nrows;    // window rows of the tile
 };
 
+// n / d for n < 2^31 with the host-made pair (magic, shift) of d: one 32x32 -> 64 multiply and a shift
+__device__ inline unsigned fast_div(unsigned n, unsigned magic, int shift) {
+  return (unsigned)(((unsigned long long)n * magic) >> shift);
+}
+
 __device__ inline TileGeom tile_geom(const IgemmArgs& p, int t, int Hv) {
   TileGeom g;
-  // M < 2^31 (checked on the host): 32-bit divisions
+  // pixel numbers stay below 2^31 (checked on the host)
   const unsigned m0 = (unsigned)t * kBM;
   const unsigned per = (unsigned)(p.OH * p.OW);
-  const unsigned nb = m0 / per;
-  const unsigned oh = (m0 - nb * per) / (unsigned)p.OW;
+  const unsigned nb = fast_div(m0, p.div_per_magic, p.div_per_shift);
+  const unsigned oh = fast_div(m0 - nb * per, p.div_ow_magic, p.div_ow_shift);
   g.m0 = m0;
   g.nb0 = (int)nb;
   g.ihv0 = (int)oh;
   g.v0 = (int)(nb * Hv + oh);
   unsigned ml = m0 + kBM - 1;
   if (ml > (unsigned)p.M - 1) ml = (unsigned)p.M - 1;
-  const unsigned nbl = ml / per;
-  const unsigned ohl = (ml - nbl * per) / (unsigned)p.OW;
+  const unsigned nbl = fast_div(ml, p.div_per_magic, p.div_per_shift);
+  const unsigned ohl = fast_div(ml - nbl * per, p.div_ow_magic, p.div_ow_shift);
   g.nrows = (int)(nbl * Hv + ohl) - g.v0 + p.KH;
   return g;
 }
@@ -170,9 +175,9 @@ __global__ __launch_bounds__(kThreads) void conv_halo_kernel(IgemmArgs p) {
     for (int i = 0; i < MI; ++i) {
       unsigned m = (unsigned)g.m0 + wave * 64 + i * 32 + (lane & 31);
       if (m > (unsigned)p.M - 1) m = (unsigned)p.M - 1;
-      const unsigned nb = m / per;
+      const unsigned nb = fast_div(m, p.div_per_magic, p.div_per_shift);
       const unsigned rem = m - nb * per;
-      const unsigned oh = rem / (unsigned)p.OW, ow = rem - oh * (unsigned)p.OW;
+      const unsigned oh = fast_div(rem, p.div_ow_magic, p.div_ow_shift), ow = rem - oh * (unsigned)p.OW;
       a_base[i] = (((int)(nb * Hv + oh) - g.v0) * Wv + (int)ow) * kPixStride + (lane >> 5) * 16;
     }
     const int b_base = (lane & 31) * brow + (lane >> 5) * 16;
@@ -334,10 +339,13 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
 
   {
     constexpr int vecs_per_row = krow / 16;
+    // LDS row j*32 + 8q + 4h + e holds output channel 32h + 16j + 4q + e: after the MFMAs a lane
+    // (pixel, h) then owns the 16 consecutive channels 32h + 16j .. + 15 of block j in register order.
     for (int q = tid; q < kBN * vecs_per_row; q += kThreads) {
       const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+      const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
       *(i32x4_t*)(sB + row * brow + vec * 16) =
-          *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)row * p.ldbt * ES + vec * 16);
+          *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
     }
   }
 
@@ -347,7 +355,11 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       __builtin_amdgcn_make_buffer_rsrc(p.C, 0, (int)(p.M * p.ldc * OES), kRsrcFlags);
 
   // ---- a thread's share of a window: vector lv of pixels lp (+32) of every row ----
-  const int lv = tid & 7, lp = tid >> 3;
+  // Eight lanes carry one pixel (128 contiguous bytes).  Neighbouring lane groups take pixels 8 apart:
+  // with the 144-byte pixel stride their 16-byte LDS slots then differ by 8 (mod 16) and a 16-lane
+  // write touches every bank once.
+  const int lv = tid & 7, lg = tid >> 3;
+  const int lp = ((lg >> 1) & 7) + 8 * (lg & 1) + 16 * (lg >> 4);
   int g_off[NCH], l_off[NCH];
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
@@ -358,32 +370,38 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   const bool chunk0 = lp < Wv, chunk1 = lp + 32 < Wv;  // does this thread's pixel of the chunk exist?
 
   u32x4_t pf[kMaxLoads];
-  auto load_window = [&](const TileGeom& g) {
+  // byte offset of every window row in the input (uniform), or kFar for padding rows and rows past the tile
+  int row_base[kRows];
+  auto window_rows = [&](const TileGeom& g) {
     int nb = g.nb0, ihv = g.ihv0;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
       const int ih = ihv - p.PH;
       const bool row_ok = r < g.nrows && nb < p.NB && (unsigned)ih < (unsigned)p.H;
-      const int row_base = row_ok ? (nb * p.H + ih) * p.W * kPixBytes : kFar;
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) pf[r * NCH + c] = __builtin_amdgcn_raw_buffer_load_b128(rin, row_base + g_off[c], 0, 0);
+      row_base[r] = row_ok ? (nb * p.H + ih) * p.W * kPixBytes : kFar;
       if (++ihv == Hv) {
         ihv = 0;
         ++nb;
       }
     }
   };
-  auto store_window = [&]() {
+  auto load_vec = [&](int j) { pf[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, row_base[j / NCH] + g_off[j % NCH], 0, 0); };
+  auto load_window = [&](const TileGeom& g) {
+    window_rows(g);
+#pragma unroll
+    for (int j = 0; j < kMaxLoads; ++j) load_vec(j);
+  };
+  auto store_window = [&](int nrows) {
     const int row_pitch = Wv * kPixStride;
     if (chunk0) {
 #pragma unroll
       for (int r = 0; r < kRows; ++r)
-        if (r < p.halo_rows) *(u32x4_t*)(sH + r * row_pitch + l_off[0]) = pf[r * NCH];
+        if (r < nrows) *(u32x4_t*)(sH + r * row_pitch + l_off[0]) = pf[r * NCH];
     }
     if (NCH == 2 && chunk1) {
 #pragma unroll
       for (int r = 0; r < kRows; ++r)
-        if (r < p.halo_rows) *(u32x4_t*)(sH + r * row_pitch + l_off[NCH - 1]) = pf[r * NCH + NCH - 1];
+        if (r < nrows) *(u32x4_t*)(sH + r * row_pitch + l_off[NCH - 1]) = pf[r * NCH + NCH - 1];
     }
   };
 
@@ -397,7 +415,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       for (int e = 0; e < 4; ++e) {
         cinit[j][q][e] = 0;
         if (p.init != nullptr) {
-          Scalar<float, int> b = load_scalar<float, int>(p.init, (int64_t)(j * 32 + 8 * q + 4 * (lane >> 5) + e) * p.init_cs, p.init_dtype);
+          Scalar<float, int> b = load_scalar<float, int>(p.init, (int64_t)(32 * (lane >> 5) + 16 * j + 4 * q + e) * p.init_cs, p.init_dtype);
           cinit[j][q][e] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
         }
       }
@@ -414,18 +432,20 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       const unsigned m = (unsigned)g.m0 + wave * 64 + i * 32 + (lane & 31);
       const bool ok = m < (unsigned)p.M;
       const unsigned mc = ok ? m : (unsigned)p.M - 1;
-      const unsigned nb = mc / per;
+      const unsigned nb = fast_div(mc, p.div_per_magic, p.div_per_shift);
       const unsigned rem = mc - nb * per;
-      const unsigned oh = rem / (unsigned)p.OW, ow = rem - oh * (unsigned)p.OW;
+      const unsigned oh = fast_div(rem, p.div_ow_magic, p.div_ow_shift), ow = rem - oh * (unsigned)p.OW;
       a_base[i] = (((int)(nb * Hv + oh) - g.v0) * Wv + (int)ow) * kPixStride + (lane >> 5) * 16;
-      m_off[i] = ok ? (int)((m * (unsigned)p.ldc + 4 * (lane >> 5)) * OES) : (int)0x80000000;
+      m_off[i] = ok ? (int)((m * (unsigned)p.ldc + 32 * (lane >> 5)) * OES) : (int)0x80000000;
     }
   };
 
   // one of the 16 pieces of a finished tile: 4 consecutive channels of one pixel
+  // (bf16 output: two pieces share one 16-byte store)
+  unsigned held[2] = {0, 0};
   auto finish_piece = [&](const acc_t (&acc)[MI][NI], const int (&m_off)[MI], int pc) {
     const int i = pc >> 3, j = (pc >> 2) & 1, q = pc & 3;
-    const int off = m_off[i] + (j * 32 + 8 * q) * OES;
+    const int off = m_off[i] + (j * 16 + 4 * q) * OES;
     if (KIND == KIND_I8) {
       u32x4_t w;
 #pragma unroll
@@ -447,8 +467,13 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
         unsigned w0, w1;
         __builtin_memcpy(&w0, &h01, 4);
         __builtin_memcpy(&w1, &h23, 4);
-        const u32x2_t w = {w0, w1};
-        __builtin_amdgcn_raw_buffer_store_b64(w, rout, off, 0, 0);
+        if ((q & 1) == 0) {
+          held[0] = w0;
+          held[1] = w1;
+        } else {
+          const u32x4_t w = {held[0], held[1], w0, w1};
+          __builtin_amdgcn_raw_buffer_store_b128(w, rout, off - 4 * OES, 0, 0);
+        }
       } else {
         u32x4_t w;
 #pragma unroll
@@ -459,25 +484,34 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   };
 
   // K loop of one tile (36 K-blocks of 32 bytes); with EPI the 16 pieces of the previous tile ride along
+  int a_next[MI], m_next[MI];  // placement of the tile after the current one
+  // The next tile (geometry g2) is prepared on the way: the offset of window row r is worked out right
+  // before that row's loads are issued, one 16-byte vector per K-block, and its placement near the end.
   auto k_loop = [&](acc_t (&acc)[MI][NI], const int (&a_base)[MI], auto epi, const acc_t (&pacc)[MI][NI],
-                    const int (&pm_off)[MI]) {
+                    const int (&pm_off)[MI], const TileGeom& g2) {
     constexpr bool EPI = decltype(epi)::value;
+    constexpr int kMfmaPerBlock = KIND == KIND_F32 ? 4 : 1;
+    int w_nb = g2.nb0, w_ihv = g2.ihv0;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < NI; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-    i32x4_t fa[2][MI], fb[2][NI];
+    // operand fragments are fetched two K-blocks ahead (three register sets)
+    i32x4_t fa[3][MI], fb[3][NI];
 #pragma unroll
-    for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(sH + a_base[i]);
+    for (int s0 = 0; s0 < 2; ++s0) {
 #pragma unroll
-    for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow);
+      for (int i = 0; i < MI; ++i) fa[s0][i] = *(const i32x4_t*)(sH + a_base[i] + s0 * 32);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) fb[s0][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow + s0 * 32);
+    }
 #pragma unroll
     for (int s = 0; s < kTaps * 4; ++s) {
-      const int cur = s & 1, nxt = cur ^ 1;
-      if (s + 1 < kTaps * 4) {
-        const int tap = (s + 1) >> 2, ks = (s + 1) & 3;
+      const int cur = s % 3, nxt = (s + 2) % 3;
+      if (s + 2 < kTaps * 4) {
+        const int tap = (s + 2) >> 2, ks = (s + 2) & 3;
         const int ao = ((tap / 3) * Wv + tap % 3) * kPixStride + ks * 32;
         const int bo = tap * kPixBytes + ks * 32;
 #pragma unroll
@@ -489,7 +523,29 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j) mma_block<KIND>(acc[i][j], fb[cur][j], fa[cur][i]);
+      if (s < kMaxLoads) {  // the next tile's window, one vector per K-block
+        if (s % NCH == 0) {
+          const int r = s / NCH, ih = w_ihv - p.PH;
+          const bool row_ok = r < g2.nrows && w_nb < p.NB && (unsigned)ih < (unsigned)p.H;
+          row_base[r] = row_ok ? (w_nb * p.H + ih) * p.W * kPixBytes : kFar;
+          if (++w_ihv == Hv) {
+            w_ihv = 0;
+            ++w_nb;
+          }
+        }
+        load_vec(s);
+      }
       if (EPI && (s & 1) == 0 && (s >> 1) < 16) finish_piece(pacc, pm_off, s >> 1);
+      if (s == 33) place(g2, a_next, m_next);
+      // order inside the K-block: LDS reads and the window load first, then VALU work between the MFMAs
+      __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+#pragma unroll
+      for (int q = 0; q < MI * NI; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerBlock, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep loads and pieces in the K-block they were put in
     }
   };
 
@@ -499,28 +555,28 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   int t = blockIdx.x;
   TileGeom g = tile_geom(p, t, Hv);
   load_window(g);
-  store_window();
+  store_window(g.nrows);
+  place(g, a_base, m_offA);
   __syncthreads();
 
-  // advance: the window of tile t2 (already in flight) replaces the current one
-  auto next_tile = [&](int t2, const TileGeom& g2) {
+  // Preparing tile t2 = t + gridDim.x (geometry, window loads, placement) is branch-free -- past the
+  // last tile every row is out of range and every load returns zeros -- so it shares one basic block
+  // with the K loop and is scheduled among the MFMAs.
+  auto advance = [&](int t2, const TileGeom& g2) {
     __syncthreads();  // every wavefront is done reading the window
-    if (t2 < p.n_tiles) store_window();
+    if (t2 < p.n_tiles) store_window(g2.nrows);
     __syncthreads();
     t = t2;
     g = g2;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a_base[i] = a_next[i];
   };
 
   {
-    place(g, a_base, m_offA);
     const int t2 = t + gridDim.x;
-    TileGeom g2 = g;
-    if (t2 < p.n_tiles) {
-      g2 = tile_geom(p, t2, Hv);
-      load_window(g2);
-    }
-    k_loop(accA, a_base, std::false_type(), accA, m_offA);
-    next_tile(t2, g2);
+    const TileGeom g2 = tile_geom(p, t2, Hv);
+    k_loop(accA, a_base, std::false_type(), accA, m_offA, g2);
+    advance(t2, g2);
   }
   for (;;) {
     if (t >= p.n_tiles) {
@@ -529,15 +585,12 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       break;
     }
     {
-      place(g, a_base, m_offB);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) m_offB[i] = m_next[i];
       const int t2 = t + gridDim.x;
-      TileGeom g2 = g;
-      if (t2 < p.n_tiles) {
-        g2 = tile_geom(p, t2, Hv);
-        load_window(g2);
-      }
-      k_loop(accB, a_base, std::true_type(), accA, m_offA);
-      next_tile(t2, g2);
+      const TileGeom g2 = tile_geom(p, t2, Hv);
+      k_loop(accB, a_base, std::true_type(), accA, m_offA, g2);
+      advance(t2, g2);
     }
     if (t >= p.n_tiles) {
 #pragma unroll
@@ -545,15 +598,12 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       break;
     }
     {
-      place(g, a_base, m_offA);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) m_offA[i] = m_next[i];
       const int t2 = t + gridDim.x;
-      TileGeom g2 = g;
-      if (t2 < p.n_tiles) {
-        g2 = tile_geom(p, t2, Hv);
-        load_window(g2);
-      }
-      k_loop(accA, a_base, std::true_type(), accB, m_offB);
-      next_tile(t2, g2);
+      const TileGeom g2 = tile_geom(p, t2, Hv);
+      k_loop(accA, a_base, std::true_type(), accB, m_offB, g2);
+      advance(t2, g2);
     }
   }
 }
@@ -597,7 +647,7 @@ size_t conv_halo_prepare(int kind, IgemmArgs* a) {
   // the padded image must be exactly what the output geometry implies
   const int Hv = a->OH + a->KH - 1, Wv = a->OW + a->KW - 1;
   if (Hv < a->H + a->PH || Wv < a->W + a->PW) return 0;
-  if (a->M >= ((int64_t)1 << 31) - kBM) return 0;
+  if (a->M >= ((int64_t)1 << 31) - ((int64_t)1 << 20)) return 0;  // tile numbers past the end must not wrap
   const int64_t per = (int64_t)a->OH * a->OW;
   const int64_t n_tiles = (a->M + kBM - 1) / kBM;
   int max_rows = 0;
@@ -620,6 +670,14 @@ size_t conv_halo_prepare(int kind, IgemmArgs* a) {
   if (total > 160 * 1024) return 0;
   a->halo_rows = max_rows;
   a->n_tiles = (int)n_tiles;
+  auto magic = [](unsigned d, unsigned* m, int* sh) {
+    int l = 0;
+    while ((1ull << l) < d) ++l;
+    *sh = 31 + l;
+    *m = (unsigned)(((1ull << (31 + l)) + d - 1) / d);
+  };
+  magic((unsigned)per, &a->div_per_magic, &a->div_per_shift);
+  magic((unsigned)a->OW, &a->div_ow_magic, &a->div_ow_shift);
   // the pipelined 3x3 kernel: fast tail only, 64 channels out, buffer-addressable operands
   const int out_es = kind == KIND_BF16 ? 2 : 4;
   const bool out_fits = kind == KIND_BF16 ? a->out_dtype == PML_HIP_BF16 : true;

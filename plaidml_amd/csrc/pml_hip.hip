@@ -47,6 +47,8 @@ struct Plan {
   // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
   size_t halo_lds = 0;
   int halo_rows = 0, halo_tiles = 0, halo_variant = 0, n_cus = 0;
+  unsigned div_magic[2] = {0, 0};
+  int div_shift[2] = {0, 0};
   std::string text;
   ~Plan() {
     if (bt) (void)hipFree(bt);
@@ -159,6 +161,10 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.halo_rows = p->halo_rows;
   g.n_tiles = p->halo_tiles;
   g.halo_variant = p->halo_variant;
+  g.div_per_magic = p->div_magic[0];
+  g.div_ow_magic = p->div_magic[1];
+  g.div_per_shift = p->div_shift[0];
+  g.div_ow_shift = p->div_shift[1];
 }
 
 }  // namespace
@@ -412,6 +418,10 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
         p->halo_rows = g.halo_rows;
         p->halo_tiles = g.n_tiles;
         p->halo_variant = g.halo_variant;
+        p->div_magic[0] = g.div_per_magic;
+        p->div_magic[1] = g.div_ow_magic;
+        p->div_shift[0] = g.div_per_shift;
+        p->div_shift[1] = g.div_ow_shift;
         p->n_cus = prop.multiProcessorCount;
       }
     }
