@@ -316,6 +316,9 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
+#ifndef PML_CONV_AHEAD
+#define PML_CONV_AHEAD 2
+#endif
 constexpr int kFar = 0x40000000;              // beyond any input this kernel accepts (<= 2^30 bytes); two of them still are
 
 template <int KIND, int NCH>
@@ -337,17 +340,28 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   const int lane = tid & 63, wave = tid >> 6;
   const int Hv = p.OH + 2, Wv = p.OW + 2;
 
-  {
-    constexpr int vecs_per_row = krow / 16;
-    // LDS row j*32 + 8q + 4h + e holds output channel 32h + 16j + 4q + e: after the MFMAs a lane
-    // (pixel, h) then owns the 16 consecutive channels 32h + 16j .. + 15 of block j in register order.
-    for (int q = tid; q < kBN * vecs_per_row; q += kThreads) {
-      const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
-      const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
-      *(i32x4_t*)(sB + row * brow + vec * 16) =
-          *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
-    }
+  // ---- filter -> LDS, once: all of a thread's 18 vectors are requested before the first is stored ----
+  // LDS row j*32 + 8q + 4h + e holds output channel 32h + 16j + 4q + e: after the MFMAs a lane
+  // (pixel, h) then owns the 16 consecutive channels 32h + 16j .. + 15 of block j in register order.
+  constexpr int vecs_per_row = krow / 16;
+  constexpr int kFilterVecs = kBN * vecs_per_row / kThreads;
+  static_assert(kBN * vecs_per_row % kThreads == 0, "filter vectors divide evenly over the threads");
+  i32x4_t fl[kFilterVecs];
+#pragma unroll
+  for (int k = 0; k < kFilterVecs; ++k) {
+    const int q = tid + k * kThreads;
+    const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+    const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
+    fl[k] = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
   }
+  auto store_filter = [&]() {
+#pragma unroll
+    for (int k = 0; k < kFilterVecs; ++k) {
+      const int q = tid + k * kThreads;
+      const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+      *(i32x4_t*)(sB + row * brow + vec * 16) = fl[k];
+    }
+  };
 
   const __amdgpu_buffer_rsrc_t rin =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)((int64_t)p.NB * p.H * p.W * kPixBytes), kRsrcFlags);
@@ -498,22 +512,29 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       for (int j = 0; j < NI; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-    // operand fragments are fetched two K-blocks ahead (three register sets)
-    i32x4_t fa[3][MI], fb[3][NI];
+    // operand fragments are fetched kAhead K-blocks ahead (kAhead + 1 register sets)
+    constexpr int kAhead = PML_CONV_AHEAD;
+    i32x4_t fa[kAhead + 1][MI], fb[kAhead + 1][NI];
+    auto frag_offsets = [&](int s1, int& ao, int& bo) {
+      const int tap = s1 >> 2, ks = s1 & 3;
+      ao = ((tap / 3) * Wv + tap % 3) * kPixStride + ks * 32;
+      bo = tap * kPixBytes + ks * 32;
+    };
 #pragma unroll
-    for (int s0 = 0; s0 < 2; ++s0) {
+    for (int s0 = 0; s0 < kAhead; ++s0) {
+      int ao, bo;
+      frag_offsets(s0, ao, bo);
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[s0][i] = *(const i32x4_t*)(sH + a_base[i] + s0 * 32);
+      for (int i = 0; i < MI; ++i) fa[s0][i] = *(const i32x4_t*)(sH + a_base[i] + ao);
 #pragma unroll
-      for (int j = 0; j < NI; ++j) fb[s0][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow + s0 * 32);
+      for (int j = 0; j < NI; ++j) fb[s0][j] = *(const i32x4_t*)(sB + b_base + j * 32 * brow + bo);
     }
 #pragma unroll
     for (int s = 0; s < kTaps * 4; ++s) {
-      const int cur = s % 3, nxt = (s + 2) % 3;
-      if (s + 2 < kTaps * 4) {
-        const int tap = (s + 2) >> 2, ks = (s + 2) & 3;
-        const int ao = ((tap / 3) * Wv + tap % 3) * kPixStride + ks * 32;
-        const int bo = tap * kPixBytes + ks * 32;
+      const int cur = s % (kAhead + 1), nxt = (s + kAhead) % (kAhead + 1);
+      if (s + kAhead < kTaps * 4) {
+        int ao, bo;
+        frag_offsets(s + kAhead, ao, bo);
 #pragma unroll
         for (int i = 0; i < MI; ++i) fa[nxt][i] = *(const i32x4_t*)(sH + a_base[i] + ao);
 #pragma unroll
@@ -526,12 +547,13 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       if (s < kMaxLoads) {  // the next tile's window, one vector per K-block
         if (s % NCH == 0) {
           const int r = s / NCH, ih = w_ihv - p.PH;
-          const bool row_ok = r < g2.nrows && w_nb < p.NB && (unsigned)ih < (unsigned)p.H;
-          row_base[r] = row_ok ? (w_nb * p.H + ih) * p.W * kPixBytes : kFar;
-          if (++w_ihv == Hv) {
-            w_ihv = 0;
-            ++w_nb;
-          }
+          // (mask arithmetic instead of a conditional: a branch here would split the K-block)
+          const int row_ok = (int)(r < g2.nrows) & (int)(w_nb < p.NB) & (int)((unsigned)ih < (unsigned)p.H);
+          const int real = (w_nb * p.H + ih) * p.W * kPixBytes;
+          row_base[r] = kFar ^ ((kFar ^ real) & -row_ok);
+          const int wrap = (int)(w_ihv + 1 == Hv);
+          w_ihv = (w_ihv + 1) & (wrap - 1);
+          w_nb += wrap;
         }
         load_vec(s);
       }
@@ -555,6 +577,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   int t = blockIdx.x;
   TileGeom g = tile_geom(p, t, Hv);
   load_window(g);
+  store_filter();
   store_window(g.nrows);
   place(g, a_base, m_offA);
   __syncthreads();
