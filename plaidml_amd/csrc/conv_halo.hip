@@ -346,20 +346,77 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   constexpr int vecs_per_row = krow / 16;
   constexpr int kFilterVecs = kBN * vecs_per_row / kThreads;
   static_assert(kBN * vecs_per_row % kThreads == 0, "filter vectors divide evenly over the threads");
-  i32x4_t fl[kFilterVecs];
+  // The filter comes either packed as Bt[CO][K] or, with b_raw, as the caller's [K][CO] matrix
+  // (HWCK, 2- or 4-byte elements).  The raw form is transposed on the way in: a task is a square of
+  // kEpv K-indices x kEpv channels, read as kEpv 16-byte vectors along CO, turned in registers and
+  // written as kEpv 16-byte vectors along K.
+  constexpr int kEpv = 16 / ES;             // elements per 16-byte vector
+  constexpr int kCoGroups = kBN / kEpv;
+  constexpr int kTasks = (krow / 16) * kCoGroups;
+  constexpr int kTaskIters = (kTasks + kThreads - 1) / kThreads;
+  constexpr int kRawRegs = ES == 1 ? 1 : kTaskIters * kEpv;
+  constexpr int kFlRegs = kRawRegs > kFilterVecs ? kRawRegs : kFilterVecs;
+  i32x4_t fl[kFlRegs];
+  if (ES != 1 && p.b_raw) {
 #pragma unroll
-  for (int k = 0; k < kFilterVecs; ++k) {
-    const int q = tid + k * kThreads;
-    const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
-    const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
-    fl[k] = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
-  }
-  auto store_filter = [&]() {
+    for (int it = 0; it < kTaskIters; ++it) {
+      int task = tid + it * kThreads;
+      if (task >= kTasks) task = kTasks - 1;
+      const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
+#pragma unroll
+      for (int kk = 0; kk < kEpv; ++kk)
+        fl[(it * kEpv + kk) % kFlRegs] =
+            *(const i32x4_t*)((const unsigned char*)p.Bt + ((int64_t)(kg * kEpv + kk) * kBN + cg * kEpv) * ES);
+    }
+  } else {
 #pragma unroll
     for (int k = 0; k < kFilterVecs; ++k) {
       const int q = tid + k * kThreads;
       const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
-      *(i32x4_t*)(sB + row * brow + vec * 16) = fl[k];
+      const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
+      fl[k] = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
+    }
+  }
+  auto store_filter = [&]() {
+    if (ES != 1 && p.b_raw) {
+#pragma unroll
+      for (int it = 0; it < kTaskIters; ++it) {
+        const int task = tid + it * kThreads;
+        const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
+        i32x4_t out[kEpv];
+        if (ES == 4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) out[e % kEpv][kk] = fl[(it * kEpv + kk) % kFlRegs][e];
+        } else {
+          // 16-bit elements: word w of vector kk holds channels 2w, 2w+1 at K index kk
+#pragma unroll
+          for (int w = 0; w < 4; ++w)
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {
+              const unsigned a = (unsigned)fl[(it * kEpv + 2 * pr) % kFlRegs][w];
+              const unsigned b2 = (unsigned)fl[(it * kEpv + 2 * pr + 1) % kFlRegs][w];
+              out[(2 * w) % kEpv][pr] = (int)((a & 0xffffu) | (b2 << 16));
+              out[(2 * w + 1) % kEpv][pr] = (int)((a >> 16) | (b2 & 0xffff0000u));
+            }
+        }
+        if (task < kTasks) {
+#pragma unroll
+          for (int e = 0; e < kEpv; ++e) {
+            const int co = cg * kEpv + e;
+            const int row = ((co >> 4) & 1) * 32 + ((co >> 2) & 3) * 8 + (co >> 5) * 4 + (co & 3);
+            *(i32x4_t*)(sB + row * brow + kg * 16) = out[e];
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kFilterVecs; ++k) {
+        const int q = tid + k * kThreads;
+        const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+        *(i32x4_t*)(sB + row * brow + vec * 16) = fl[k];
+      }
     }
   };
 
@@ -428,11 +485,41 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         cinit[j][q][e] = 0;
-        if (p.init != nullptr) {
-          Scalar<float, int> b = load_scalar<float, int>(p.init, (int64_t)(32 * (lane >> 5) + 16 * j + 4 * q + e) * p.init_cs, p.init_dtype);
-          cinit[j][q][e] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+      }
+  if (p.init != nullptr) {
+    const int natural = KIND == KIND_BF16 ? PML_HIP_BF16 : (KIND == KIND_I8 ? PML_HIP_I32 : PML_HIP_F32);
+    if (p.init_cs == 1 && p.init_dtype == natural && ((uintptr_t)p.init & 15) == 0) {
+      // a contiguous bias of the result type: a lane's 16 channels of block j are 32 (bf16) or 64 bytes
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const unsigned char* src = (const unsigned char*)p.init + (32 * (lane >> 5) + 16 * j) * OES;
+        u32x4_t raw[OES];
+#pragma unroll
+        for (int v = 0; v < OES; ++v) raw[v] = *(const u32x4_t*)(src + v * 16);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (KIND == KIND_BF16) {
+            const unsigned w = raw[r >> 3][(r >> 1) & 3];
+            cinit[j][r >> 2][r & 3] = (accs_t)__uint_as_float((r & 1) ? (w & 0xffff0000u) : (w << 16));
+          } else if (KIND == KIND_I8) {
+            cinit[j][r >> 2][r & 3] = (accs_t)(int)raw[r >> 2][r & 3];
+          } else {
+            cinit[j][r >> 2][r & 3] = (accs_t)__uint_as_float(raw[r >> 2][r & 3]);
+          }
         }
       }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            Scalar<float, int> b = load_scalar<float, int>(p.init, (int64_t)(32 * (lane >> 5) + 16 * j + 4 * q + e) * p.init_cs, p.init_dtype);
+            cinit[j][q][e] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+          }
+    }
+  }
   const float lo_f = p.tail_relu ? 0.f : -__builtin_inff();
   const int lo_i = p.tail_relu ? 0 : (int)0x80000000;
 

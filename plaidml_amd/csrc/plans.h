@@ -32,7 +32,8 @@ struct IgemmArgs {
   int H, W, CI, OH, OW, KH, KW, SH, SW, PH, PW, DH, DW;
   // resident-filter convolution only: image count, LDS rows of the input window, number of 256-pixel tiles
   // halo_variant: 0 = general resident kernel, 1 / 2 = pipelined 3x3 kernel with that many 32-pixel chunks per row
-  int NB, halo_rows, n_tiles, halo_variant;
+  // b_raw: Bt points at the caller's [K][N] matrix instead of the packed [N][K] one (pipelined kernel only)
+  int NB, halo_rows, n_tiles, halo_variant, b_raw;
   // n / (OH*OW) and n / OW as multiply-and-shift (see fast_div)
   unsigned div_per_magic, div_ow_magic;
   int div_per_shift, div_ow_shift;

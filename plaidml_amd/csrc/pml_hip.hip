@@ -446,11 +446,19 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   if (d.init_kind && !init) return fail("conv2d_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
   const int64_t K = d.kh * d.kw * d.ci;
-  // the HWCK filter is a row-major [K][CO] matrix
-  if (filter && check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
+  // the HWCK filter is a row-major [K][CO] matrix; the pipelined resident-filter kernel transposes it itself
+  const bool raw_filter = filter && p->halo_lds && p->halo_variant && p->mfma_kind != KIND_I8;
+  if (filter && !raw_filter &&
+      check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   IgemmArgs g;
   conv_args(p, g);
+  if (raw_filter) {
+    if (((uintptr_t)filter & 15) != 0) return fail("conv2d_invoke: filter must be 16-byte aligned");
+    g.Bt = filter;
+    g.ldbt = d.co;
+    g.b_raw = 1;
+  }
   g.A = input;
   g.C = output;
   g.init = d.init_kind ? init : nullptr;
