@@ -4,13 +4,19 @@
 Workload (BASELINE.json configs[1]): conv2d NHWC via the contraction
   O[n,y,x,co] += I[n,y+ky-1,x+kx-1,ci] * F[ky,kx,ci,co]   (N128, 56x56x64, 3x3x64x64, stride 1, SAME)
 followed by the fused bias + ReLU tail, bf16 (fp32 accumulate).  One step = one pass over the
-batch: the filter re-layout kernel plus the implicit-GEMM kernel, inputs resident in HBM.
+batch, inputs (image, HWCK filter, bias) resident in HBM: a single launch of the resident-filter
+convolution kernel, which re-lays the filter out on its way into LDS.
 
 Prints ONE JSON line.  `value` is TFLOP/s over the algorithmic FLOPs (2 x valid index tuples:
 SAME-padding taps that fall outside the image are not counted).  `roofline` describes the
-dominant kernel (the implicit-GEMM conv) timed alone with HIP events; `cpu_baseline` is the
+dominant kernel (the convolution kernel with a pre-packed filter) timed with HIP events on the
+launch stream; `roofline.traffic` is the HBM bytes per launch taken from the committed rocprofv3
+counter summary (profiles/), null when that file is absent; `cpu_baseline` is the
 OpenMP restatement (oracle/cpu_baseline.c) on a bounded sample of the same workload.
 `extra` carries the other single-kernel configs for information only.
+
+`--copy-calibration` runs only a plain device copy of a known size (the factor that scales the
+FETCH_SIZE / WRITE_SIZE counters) and prints its byte count.
 """
 import argparse
 import ctypes
@@ -93,6 +99,36 @@ def cpu_baseline_conv(E, N_sample, H, W, CI, CO, seed_i, seed_f, flops_per_image
     }, E.round_bf16(out), Iv, Fv
 
 
+def copy_calibration(hk, steps):
+    """A plain copy kernel of known size: out[i] = in[i] over 256 MiB of fp32."""
+    n = 64 << 20
+    d = hk.EltwiseDesc()
+    d.rank, d.in_dtype, d.out_dtype = 1, hk.F32, hk.F32
+    d.sizes[0] = n
+    d.in_strides[0] = 1
+    plan = hk.lib().pml_hip_eltwise_dispatch(ctypes.byref(d))
+    if not plan:
+        raise RuntimeError(hk.lib().pml_hip_last_error().decode())
+    src, dst = hk.DeviceBuffer(n * 4), hk.DeviceBuffer(n * 4)
+    hk.check(hk.lib().pml_hip_fill_u32(src.ptr, 0x3f800000, n, None))
+    none = hk.ptr_array([])
+    ms, _ = time_loop(hk, lambda: hk.check(hk.lib().pml_hip_eltwise_invoke(plan, src.ptr, dst.ptr, none, none, None)), steps, 2)
+    return {'copy_kernel': hk.describe(plan), 'bytes_read_per_launch': n * 4, 'bytes_written_per_launch': n * 4,
+            'ms': round(ms, 4), 'GBps': round(2 * n * 4 / ms / 1e6, 1)}
+
+
+def committed_traffic():
+    """HBM bytes per launch of the bench kernel from the committed counter summary, or None."""
+    path = os.path.join(ROOT, 'profiles', 'conv_halo3x3_bf16_configs1_hbm_traffic.md')
+    try:
+        for line in open(path):
+            if line.startswith('traffic_bytes_per_launch'):
+                return float(line.split('=')[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -100,6 +136,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-extra', action='store_true')
     ap.add_argument('--no-cpu', action='store_true')
+    ap.add_argument('--copy-calibration', action='store_true')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus, file=sys.stderr)
@@ -110,6 +147,9 @@ def main():
 
     hk.init(0)
     L = hk.lib()
+    if args.copy_calibration:
+        print(json.dumps(copy_calibration(hk, args.steps)))
+        return
     N, H, W, CI, CO = 128, 56, 56, 64, 64
     taps = valid_taps(H, 3, 1) * valid_taps(W, 3, 1)          # valid (y,ky) x (x,kx) pairs
     flops = 2.0 * N * taps * CI * CO
@@ -150,7 +190,7 @@ def main():
                    'host_wall_ms_per_step': round(wall_step, 5)},
         'roofline': {'bound': 'mfma', 'achieved': round(flops / (ms_kernel * 1e-3) / 1e12, 3), 'peak': PEAK['bf16'],
                      'unit': 'TFLOP/s', 'frac': round(flops / (ms_kernel * 1e-3) / 1e12 / PEAK['bf16'], 4),
-                     'traffic': None, 'kernel': 'igemm_kernel<bf16, conv>', 'kernel_ms': round(ms_kernel, 5),
+                     'traffic': committed_traffic(), 'kernel': hk.describe(plan).split('tile=')[-1], 'kernel_ms': round(ms_kernel, 5),
                      'hbm_GBps_at_algorithmic_bytes': round(bytes_alg / (ms_kernel * 1e-3) / 1e9, 1),
                      'hbm_frac': round(bytes_alg / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }

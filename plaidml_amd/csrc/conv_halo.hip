@@ -36,6 +36,15 @@ constexpr int kPixBytes = 128;    // channel bytes per pixel
 constexpr int kPixStride = 144;   // LDS stride of a pixel
 constexpr int kMaxLoads = 24;     // 16-byte window vectors a thread may carry for the next tile
 
+// Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each).  Give every XCD a contiguous run
+// of the tiles worked on at the same time, so the window rows two neighbouring tiles share are
+// fetched from HBM once and found in that L2 by the other.
+__device__ inline int first_tile(int bid, int nblocks) {
+  constexpr int kXcds = 8;
+  if (nblocks % kXcds != 0) return bid;
+  return (bid % kXcds) * (nblocks / kXcds) + bid / kXcds;
+}
+
 struct TileGeom {
   int64_t m0;   // first output pixel
   int v0;       // virtual row of that pixel
@@ -159,7 +168,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo_kernel(IgemmArgs p) {
         }
       }
 
-  int t = blockIdx.x;
+  int t = first_tile(blockIdx.x, gridDim.x);
   TileGeom g = tile_geom(p, t, Hv);
   load_window(g);
   store_window(g);
@@ -661,7 +670,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   acc_t accA[MI][NI], accB[MI][NI];
   int a_base[MI], m_offA[MI], m_offB[MI];
 
-  int t = blockIdx.x;
+  int t = first_tile(blockIdx.x, gridDim.x);
   TileGeom g = tile_geom(p, t, Hv);
   load_window(g);
   store_filter();
