@@ -84,6 +84,53 @@ __device__ inline void aggregate(int agg, int dt, Scalar<FT, IT>& acc, const Sca
   }
 }
 
+// One point of the reduction box: checks every input access, loads, combines and aggregates into acc.
+template <typename FT, typename IT>
+__device__ inline void accumulate_point(const pml_hip_contract_desc& d, const ContractArgs& a, const int64_t* base,
+                                        const int64_t* idx, int acc_dt, Scalar<FT, IT>& acc) {
+  bool ok = true;
+  int64_t off[4] = {0, 0, 0, 0};
+  for (int f = 0; f < d.n_forms && ok; ++f) {
+    const pml_hip_form& fm = d.forms[f];
+    if (fm.operand == 0) continue;
+    int64_t s = base[f];
+    for (int v = d.n_out_idx; v < d.n_idx; ++v) s += (int64_t)fm.coef[v] * idx[v];
+    if (fm.den != 1) {
+      if (s % fm.den != 0) {
+        ok = false;
+        break;
+      }
+      s /= fm.den;
+    }
+    if (s < 0 || s >= fm.size) {
+      ok = false;
+      break;
+    }
+    if (fm.operand > 0) off[fm.operand] += s * fm.stride;
+  }
+  if (ok) {
+    Scalar<FT, IT> x[3];
+    for (int q = 0; q < d.n_src; ++q) {
+      const int sd = d.src_dtype[q];
+      Scalar<FT, IT> raw = load_scalar<FT, IT>(a.srcs[q], off[q + 1], sd);
+      if (d.combo == PML_HIP_COMBO_COND && q < 2) {
+        x[q] = convert_scalar<FT, IT>(raw, sd, d.cmp_dtype);
+      } else if (!dt_is_float(sd) && !dt_is_float(acc_dt) && sd != PML_HIP_BOOL && dt_size(sd) < dt_size(acc_dt) &&
+                 d.combo != PML_HIP_COMBO_COND) {
+        // operands of a contraction body are signless: widening is zero-extension
+        Scalar<FT, IT> z = raw;
+        const int bits = dt_size(sd) * 8;
+        z.i = raw.i & (IT)((((uint64_t)1) << bits) - 1);
+        x[q] = z;
+      } else {
+        x[q] = convert_scalar<FT, IT>(raw, sd, acc_dt);
+      }
+    }
+    Scalar<FT, IT> v = combine<FT, IT>(d.combo, acc_dt, d.cmp_dtype, x);
+    aggregate<FT, IT>(d.agg, acc_dt, acc, v);
+  }
+}
+
 template <typename FT, typename IT>
 __global__ __launch_bounds__(256) void contract_kernel(ContractArgs a) {
   const pml_hip_contract_desc& d = a.d;
@@ -137,47 +184,7 @@ __global__ __launch_bounds__(256) void contract_kernel(ContractArgs a) {
     if (d.lo[v] > d.hi[v]) empty = true;
   }
   while (!empty) {
-    bool ok = true;
-    int64_t off[4] = {0, 0, 0, 0};
-    for (int f = 0; f < d.n_forms && ok; ++f) {
-      const pml_hip_form& fm = d.forms[f];
-      if (fm.operand == 0) continue;
-      int64_t s = base[f];
-      for (int v = d.n_out_idx; v < d.n_idx; ++v) s += (int64_t)fm.coef[v] * idx[v];
-      if (fm.den != 1) {
-        if (s % fm.den != 0) {
-          ok = false;
-          break;
-        }
-        s /= fm.den;
-      }
-      if (s < 0 || s >= fm.size) {
-        ok = false;
-        break;
-      }
-      if (fm.operand > 0) off[fm.operand] += s * fm.stride;
-    }
-    if (ok) {
-      Scalar<FT, IT> x[3];
-      for (int q = 0; q < d.n_src; ++q) {
-        const int sd = d.src_dtype[q];
-        Scalar<FT, IT> raw = load_scalar<FT, IT>(a.srcs[q], off[q + 1], sd);
-        if (d.combo == PML_HIP_COMBO_COND && q < 2) {
-          x[q] = convert_scalar<FT, IT>(raw, sd, d.cmp_dtype);
-        } else if (!dt_is_float(sd) && !dt_is_float(acc_dt) && sd != PML_HIP_BOOL && dt_size(sd) < dt_size(acc_dt) &&
-                   d.combo != PML_HIP_COMBO_COND) {
-          // operands of a contraction body are signless: widening is zero-extension
-          Scalar<FT, IT> z = raw;
-          const int bits = dt_size(sd) * 8;
-          z.i = raw.i & (IT)((((uint64_t)1) << bits) - 1);
-          x[q] = z;
-        } else {
-          x[q] = convert_scalar<FT, IT>(raw, sd, acc_dt);
-        }
-      }
-      Scalar<FT, IT> v = combine<FT, IT>(d.combo, acc_dt, d.cmp_dtype, x);
-      aggregate<FT, IT>(d.agg, acc_dt, acc, v);
-    }
+    accumulate_point<FT, IT>(d, a, base, idx, acc_dt, acc);
     int v = d.n_idx - 1;
     for (; v >= d.n_out_idx; --v) {
       if (++idx[v] <= d.hi[v]) break;
@@ -186,6 +193,86 @@ __global__ __launch_bounds__(256) void contract_kernel(ContractArgs a) {
     if (v < d.n_out_idx) break;
   }
   store_scalar<FT, IT>(a.out, out_off, dt, convert_scalar<FT, IT>(acc, acc_dt, dt));
+}
+
+// Few outputs, long reductions (row max / row sum of a softmax, global pooling): one workgroup per
+// output point.  Thread t takes the points t, t + 256, ... of the linearised reduction box, starting
+// from the aggregation's identity; the 256 partial results and the initial value (if any) are then
+// aggregated once.  Only for add / mul / max / min, whose result does not depend on grouping (up to
+// floating-point rounding).
+template <typename FT, typename IT>
+__global__ __launch_bounds__(256) void contract_coop_kernel(ContractArgs a, int64_t red_count) {
+  const pml_hip_contract_desc& d = a.d;
+  const int64_t gid = blockIdx.x;
+  __shared__ FT part_f[256];
+  __shared__ IT part_i[256];
+
+  int64_t idx[PML_HIP_MAX_IDX];
+  {
+    int64_t t = gid;
+    for (int v = d.n_out_idx - 1; v >= 0; --v) {
+      const int64_t range = d.hi[v] - d.lo[v] + 1;
+      idx[v] = d.lo[v] + t % range;
+      t /= range;
+    }
+  }
+  int64_t base[PML_HIP_MAX_FORMS];
+  for (int f = 0; f < d.n_forms; ++f) {
+    int64_t s = d.forms[f].c0;
+    for (int v = 0; v < d.n_out_idx; ++v) s += (int64_t)d.forms[f].coef[v] * idx[v];
+    base[f] = s;
+  }
+  int64_t out_off = 0;
+  for (int f = 0; f < d.n_forms; ++f) {
+    if (d.forms[f].operand != 0) continue;
+    int64_t q = base[f];
+    const int den = d.forms[f].den;
+    if (den != 1) {
+      if (q % den != 0) return;  // uniform over the workgroup
+      q /= den;
+    }
+    if (q < 0 || q >= d.forms[f].size) return;
+    out_off += q * d.forms[f].stride;
+  }
+  const int dt = d.dtype;
+  const int acc_dt = (dt == PML_HIP_BF16 || dt == PML_HIP_F16) ? PML_HIP_F32 : dt;
+  Scalar<FT, IT> ident;
+  ident.f = dt_is_float(dt) ? (FT)d.identity_f : (FT)0;
+  ident.i = dt_is_float(dt) ? (IT)0 : wrap_int_to<IT>(dt, (IT)d.identity_i);
+  Scalar<FT, IT> acc = ident;
+  for (int64_t r = threadIdx.x; r < red_count; r += 256) {
+    int64_t t = r;
+    for (int v = d.n_idx - 1; v >= d.n_out_idx; --v) {
+      const int64_t range = d.hi[v] - d.lo[v] + 1;
+      idx[v] = d.lo[v] + t % range;
+      t /= range;
+    }
+    accumulate_point<FT, IT>(d, a, base, idx, acc_dt, acc);
+  }
+  part_f[threadIdx.x] = acc.f;
+  part_i[threadIdx.x] = acc.i;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) {
+      Scalar<FT, IT> x, y;
+      x.f = part_f[threadIdx.x], x.i = part_i[threadIdx.x];
+      y.f = part_f[threadIdx.x + w], y.i = part_i[threadIdx.x + w];
+      aggregate<FT, IT>(d.agg, acc_dt, x, y);
+      part_f[threadIdx.x] = x.f;
+      part_i[threadIdx.x] = x.i;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    Scalar<FT, IT> total;
+    total.f = part_f[0], total.i = part_i[0];
+    if (d.has_init) {
+      Scalar<FT, IT> start = convert_scalar<FT, IT>(load_scalar<FT, IT>(a.out, out_off, dt), dt, acc_dt);
+      aggregate<FT, IT>(d.agg, acc_dt, start, total);
+      total = start;
+    }
+    store_scalar<FT, IT>(a.out, out_off, dt, convert_scalar<FT, IT>(total, acc_dt, dt));
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -293,6 +380,16 @@ hipError_t contract_launch(const ContractArgs& a, hipStream_t s) {
   for (int q = 0; q < d.n_src; ++q) wide = wide || is_wide(d.src_dtype[q]);
   const unsigned blocks = (unsigned)((d.out_elems + 255) / 256);
   if (blocks == 0) return hipSuccess;
+  // too few outputs to fill the chip and a long reduction: one workgroup per output
+  int64_t red_count = 1;
+  for (int v = d.n_out_idx; v < d.n_idx; ++v) red_count *= d.hi[v] >= d.lo[v] ? d.hi[v] - d.lo[v] + 1 : 0;
+  if (d.agg != PML_HIP_AGG_ASSIGN && d.out_elems <= 4096 && red_count >= 512) {
+    if (wide)
+      hipLaunchKernelGGL((contract_coop_kernel<double, int64_t>), dim3((unsigned)d.out_elems), dim3(256), 0, s, a, red_count);
+    else
+      hipLaunchKernelGGL((contract_coop_kernel<float, int>), dim3((unsigned)d.out_elems), dim3(256), 0, s, a, red_count);
+    return hipGetLastError();
+  }
   if (wide)
     hipLaunchKernelGGL((contract_kernel<double, int64_t>), dim3(blocks), dim3(256), 0, s, a);
   else

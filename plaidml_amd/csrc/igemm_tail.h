@@ -66,7 +66,10 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
   const int64_t n = n0 + c4;
   if (n >= p.N) return;
   const bool full4 = n + 3 < p.N;
-  const bool fast = p.tail_mode == 1 && full4 && (p.ldc & 3) == 0;
+  // tail_mode 1: relu? ; 2: + residual tensor of the result type (unit column stride), then relu?
+  const bool fast = (p.tail_mode == 1 || p.tail_mode == 2) && full4 && (p.ldc & 3) == 0;
+  const bool residual = p.tail_mode == 2;
+  const int64_t res_rs = p.tail.operand_row_stride[0];
   // a per-column start value (bias) is the same for every row of this thread
   const bool col_init = p.init != nullptr && p.init_rs == 0;
   accs_t cinit[4] = {0, 0, 0, 0};
@@ -100,22 +103,40 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
     if (fast) {
       if (KIND == KIND_I8) {
         i32x4_t w;
+        i32x4_t x = {0, 0, 0, 0};
+        if (residual) x = *(const i32x4_t*)((const int*)p.operands[0] + m * res_rs + n);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) w[q] = (p.tail_relu && (int)v4[q] < 0) ? 0 : (int)v4[q];
+        for (int q = 0; q < 4; ++q) {
+          const int v = (int)((unsigned)(int)v4[q] + (unsigned)x[q]);
+          w[q] = (p.tail_relu && v < 0) ? 0 : v;
+        }
         *(i32x4_t*)((int*)p.C + m * p.ldc + n) = w;
       } else if (p.out_dtype == PML_HIP_BF16) {
         uint32_t h[4];
+        uint2 x = make_uint2(0, 0);
+        if (residual) x = *(const uint2*)((const uint16_t*)p.operands[0] + m * res_rs + n);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           h[q] = f32_to_bf16_bits((float)v4[q]);
+          if (residual) {
+            // the contraction result is rounded first, then the bf16 addition rounds again
+            const uint32_t xw = (q < 2) ? x.x : x.y;
+            const float xf = __uint_as_float((q & 1) ? (xw & 0xffff0000u) : (xw << 16));
+            h[q] = f32_to_bf16_bits(__uint_as_float(h[q] << 16) + xf);
+          }
           // relu on the rounded value: negative, non-NaN, non-zero -> 0  (x < 0 ? 0 : x)
           if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
         }
         *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
       } else {
         f32x4_t w;
+        f32x4_t x = {0.f, 0.f, 0.f, 0.f};
+        if (residual) x = *(const f32x4_t*)((const float*)p.operands[0] + m * res_rs + n);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) w[q] = (p.tail_relu && (float)v4[q] < 0.f) ? 0.f : (float)v4[q];
+        for (int q = 0; q < 4; ++q) {
+          const float v = residual ? (float)v4[q] + x[q] : (float)v4[q];
+          w[q] = (p.tail_relu && v < 0.f) ? 0.f : v;
+        }
         *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
       }
       continue;

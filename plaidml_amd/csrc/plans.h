@@ -92,6 +92,14 @@ struct DwconvArgs {
   void* outs[PML_HIP_MAX_EPI_OPERANDS];
 };
 hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s);
+struct Im2colArgs {
+  const void* in;
+  void* out;
+  int64_t M;  // N * OH * OW rows
+  int K, kpad;  // KH*KW*CI real columns, row length (a multiple of the 16-byte vector)
+  int H, W, CI, OH, OW, KH, KW, SH, SW, PH, PW, DH, DW;
+};
+hipError_t im2col_launch(int elem_size, const Im2colArgs& a, hipStream_t s);
 struct PoolArgs {
   pml_hip_pool2d_desc d;
   const void* in;

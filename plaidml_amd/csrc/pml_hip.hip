@@ -44,6 +44,9 @@ struct Plan {
   int64_t bt_ld = 0;
   size_t bt_bytes = 0;
   bool packed = false;
+  // convolution whose channels do not fill 16-byte vectors: patch matrix [M][kpad] + GEMM
+  void* patches = nullptr;
+  int64_t kpad = 0;
   // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
   size_t halo_lds = 0;
   int halo_rows = 0, halo_tiles = 0, halo_variant = 0, n_cus = 0;
@@ -52,6 +55,7 @@ struct Plan {
   std::string text;
   ~Plan() {
     if (bt) (void)hipFree(bt);
+    if (patches) (void)hipFree(patches);
   }
 };
 
@@ -107,6 +111,15 @@ void classify_tail(const pml_hip_epilogue& t, int out_dtype, int c_dtype, int* m
   if (t.n_ops == 1 && t.ops[0].opcode == PML_HIP_EPI_RELU && t.ops[0].dtype == out_dtype) {
     *mode = 1;
     *relu = 1;
+    return;
+  }
+  // + residual (a full tensor of the result type, unit column stride, rows on 4-element boundaries), relu?
+  if ((t.n_ops == 1 || t.n_ops == 2) && t.ops[0].opcode == PML_HIP_EPI_ADD && t.ops[0].operand_kind == PML_HIP_OPND_TENSOR &&
+      t.ops[0].operand == 0 && t.ops[0].dtype == out_dtype && t.operand_dtype[0] == out_dtype &&
+      t.operand_col_stride[0] == 1 && (t.operand_row_stride[0] & 3) == 0 &&
+      (t.n_ops == 1 || (t.ops[1].opcode == PML_HIP_EPI_RELU && t.ops[1].dtype == out_dtype))) {
+    *mode = 2;
+    *relu = t.n_ops == 2;
   }
 }
 
@@ -343,6 +356,7 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
     if (!operands || !operands[i]) return fail("gemm_invoke: missing tail operand");
     g.operands[i] = operands[i];
   }
+  if (g.tail_mode == 2 && ((uintptr_t)g.operands[0] & 15) != 0) g.tail_mode = 0;
   for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
@@ -376,10 +390,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     return 0;
   }
   const int es = dt_size(d->in_dtype);
-  if ((d->ci * es) % 16 != 0) {
-    fail("conv2d: input channels must cover whole 16-byte vectors");
-    return 0;
-  }
+  const bool via_patches = (d->ci * es) % 16 != 0;
   if (d->n * d->h * d->w * d->ci >= ((int64_t)1 << 40) || d->h * d->w * d->ci * es >= ((int64_t)1 << 31) ||
       d->kh * d->kw * d->ci * es >= ((int64_t)1 << 31)) {
     fail("conv2d: tensor too large");
@@ -397,8 +408,19 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   const int64_t K = d->kh * d->kw * d->ci;
   p->tile = choose_tile(M, d->co);
   p->bt_ld = K;
-  p->bt_bytes = (size_t)d->co * K * es;
-  if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
+  if (via_patches) {
+    // rows padded with zeros to whole 16-byte vectors on both GEMM operands
+    const int64_t v = 16 / es;
+    p->kpad = (K + v - 1) / v * v;
+    p->bt_ld = p->kpad;
+    if (hipMalloc(&p->patches, (size_t)M * p->kpad * es) != hipSuccess) {
+      delete p;
+      fail("conv2d: cannot allocate the patch matrix");
+      return 0;
+    }
+  }
+  p->bt_bytes = (size_t)d->co * p->bt_ld * es;
+  if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess || hipMemset(p->bt, 0, p->bt_bytes) != hipSuccess) {
     delete p;
     fail("conv2d: cannot allocate the packed filter");
     return 0;
@@ -408,7 +430,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     const char* e = std::getenv("PML_HIP_CONV");
     int dev = 0;
     hipDeviceProp_t prop;
-    if (!(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
+    if (!via_patches && !(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
         hipGetDeviceProperties(&prop, dev) == hipSuccess) {
       IgemmArgs g;
       conv_args(p, g);
@@ -432,6 +454,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
                 (long long)d->h, (long long)d->w, (long long)d->ci, (long long)d->kh, (long long)d->kw, (long long)d->co,
                 (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, p->halo_lds ? (p->halo_variant ? "256x64 resident filter, pipelined 3x3" : "256x64 resident filter") : tile_name(p->tile));
   p->text = buf;
+  if (via_patches) p->text += " via patch matrix (k padded to " + std::to_string(p->kpad) + ")";
   return (int64_t)(intptr_t)p;
 }
 
@@ -442,7 +465,7 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   const pml_hip_conv2d_desc& d = p->conv;
   if (!input || !output) return fail("conv2d_invoke: null operand");
   if (!filter && !p->packed) return fail("conv2d_invoke: filter is null and no packed filter exists");
-  if (((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
+  if (!p->patches && ((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
   if (d.init_kind && !init) return fail("conv2d_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
   const int64_t K = d.kh * d.kw * d.ci;
@@ -466,10 +489,26 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     if (!operands || !operands[i]) return fail("conv2d_invoke: missing tail operand");
     g.operands[i] = operands[i];
   }
+  if (g.tail_mode == 2 && ((uintptr_t)g.operands[0] & 15) != 0) g.tail_mode = 0;
   for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("conv2d_invoke: missing extra output");
+  if (p->patches) {
+    Im2colArgs ic;
+    ic.in = input;
+    ic.out = p->patches;
+    ic.M = g.M;
+    ic.K = (int)K;
+    ic.kpad = (int)p->kpad;
+    ic.H = g.H, ic.W = g.W, ic.CI = g.CI, ic.OH = g.OH, ic.OW = g.OW, ic.KH = g.KH, ic.KW = g.KW;
+    ic.SH = g.SH, ic.SW = g.SW, ic.PH = g.PH, ic.PW = g.PW, ic.DH = g.DH, ic.DW = g.DW;
+    if (check(im2col_launch(es, ic, (hipStream_t)s), "im2col_launch")) return 1;
+    g.A = p->patches;
+    g.lda = p->kpad;
+    g.K = p->kpad;
+    return check(igemm_launch(p->mfma_kind, p->tile, false, g, (hipStream_t)s), "igemm_launch");
+  }
   if (p->halo_lds)
     return check(conv_halo_launch(p->mfma_kind, g, p->halo_lds, p->n_cus, (hipStream_t)s), "conv_halo_launch");
   return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");

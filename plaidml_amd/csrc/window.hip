@@ -171,6 +171,38 @@ inline unsigned grid_for(int64_t items) {
   return (unsigned)(blocks < cap ? blocks : cap);
 }
 
+
+// Patch matrix of a convolution whose channel count does not fill 16-byte vectors (a 3-channel
+// image stem): P[m][k] = I[n, oh*sh + kh*dh - ph, ow*sw + kw*dw - pw, ci] with k = (kh*KW + kw)*CI + ci,
+// zero outside the image and for k >= KH*KW*CI.  One thread writes one 16-byte vector of a row.
+template <typename T>
+__global__ __launch_bounds__(256) void im2col_kernel(Im2colArgs a) {
+  constexpr int V = 16 / (int)sizeof(T);
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int vecs = a.kpad / V;
+  if (idx >= a.M * vecs) return;
+  const int64_t m = idx / vecs;
+  const int k0 = (int)(idx - m * vecs) * V;
+  const int ow = (int)(m % a.OW);
+  const int64_t t = m / a.OW;
+  const int oh = (int)(t % a.OH);
+  const int64_t nb = t / a.OH;
+  const T* img = (const T*)a.in + nb * ((int64_t)a.H * a.W * a.CI);
+  T vals[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int k = k0 + e;
+    const int tap = k / a.CI, ci = k - tap * a.CI;
+    const int kh = tap / a.KW, kw = tap - kh * a.KW;
+    const int ih = oh * a.SH + kh * a.DH - a.PH, iw = ow * a.SW + kw * a.DW - a.PW;
+    const bool ok = k < a.K && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+    vals[e] = ok ? img[((int64_t)ih * a.W + iw) * a.CI + ci] : (T)0;
+  }
+  i32x4_t packed;
+  __builtin_memcpy(&packed, vals, 16);
+  *(i32x4_t*)((T*)a.out + m * a.kpad + k0) = packed;
+}
+
 }  // namespace
 
 hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
@@ -196,6 +228,19 @@ hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s) {
     hipLaunchKernelGGL((pool2d_kernel<2>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
   else
     hipLaunchKernelGGL((pool2d_kernel<4>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  return hipGetLastError();
+}
+
+hipError_t im2col_launch(int elem_size, const Im2colArgs& a, hipStream_t s) {
+  const int v = 16 / elem_size;
+  const int64_t total = a.M * (a.kpad / v);
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  switch (elem_size) {
+    case 1: hipLaunchKernelGGL(im2col_kernel<uint8_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    case 2: hipLaunchKernelGGL(im2col_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    case 4: hipLaunchKernelGGL(im2col_kernel<uint32_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    default: return hipErrorInvalidValue;
+  }
   return hipGetLastError();
 }
 

@@ -993,7 +993,7 @@ class Planner {
     for (size_t v = 0; v < n.nIdx; ++v)
       if (n.active[v] && !roles.count(static_cast<int>(v))) return false;
     const int es = in_dt == PML_HIP_F32 ? 4 : (in_dt == PML_HIP_BF16 ? 2 : 1);
-    if ((is.sizes[3] * es) % 16 != 0) return false;
+    // (channel counts that do not fill 16-byte vectors are handled inside the kernel library: patch matrix + GEMM)
 
     Step s;
     s.kind = Step::Conv2d;

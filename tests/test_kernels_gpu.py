@@ -306,6 +306,23 @@ def test_conv_resident_filter_matches_generic_kernel(monkeypatch):
     np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
 
 
+@pytest.mark.parametrize('kind', ['f32', 'bf16'])
+def test_conv_three_channel_stem(kind, capsys):
+    # 7x7 stride 2 over a 3-channel image: channels do not fill 16-byte vectors -> patch matrix + GEMM
+    Iv, Fv = _conv_case(kind, (2, 30, 34, 3), 7, 7, 64, op.SAME_UPPER, 41)
+    bias = np.random.default_rng(42).standard_normal(64).astype(np.float32)
+    if kind == 'bf16':
+        bias = E.round_bf16(bias)
+        out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=2, bias=bf16(bias), relu=True))
+        ref = oracle_conv(Iv, Fv, D.BFLOAT16, 2, op.SAME_UPPER, bias, True)
+        np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
+    else:
+        out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=2, bias=bias, relu=True)
+        ref = oracle_conv(Iv, Fv, D.FLOAT32, 2, op.SAME_UPPER, bias, True)
+        np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4)
+    assert 'patch matrix' in capsys.readouterr().out
+
+
 def test_dwconv_pool_bf16():
     rng = np.random.default_rng(9)
     N, H, W, C = 2, 19, 19, 32
