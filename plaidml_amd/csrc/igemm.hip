@@ -10,10 +10,18 @@
 //   int8: one  v_mfma_i32_32x32x32_i8
 //   fp32: four v_mfma_f32_32x32x2_f32   (the k order inside a block is permuted
 //         identically for A and Bt, which leaves the sum unchanged)
-// 256 threads = 4 wavefronts; LDS is double-buffered and the next slab travels
-// global -> registers while the current one feeds the MFMAs.  After the K loop
-// the accumulator tile is staged through LDS so that the tail runs once per
-// element in row-major order and stores are contiguous 8/16-byte pieces.
+//
+// Data movement.  256 threads = 4 wavefronts.  Slabs travel global -> LDS directly
+// (buffer_load ... lds, 16 bytes per lane, no register staging) into a ring of
+// three stages, two slabs ahead of the MFMAs, with one s_barrier per slab.  A
+// load whose element lies outside the problem (M / N / K tails, convolution
+// padding) carries an offset beyond the buffer and delivers zeros.  One such
+// instruction of a wavefront fills 8 rows x 128 bytes contiguously, so LDS rows
+// are not padded; instead the lane that fills 16-byte slot u of row r fetches
+// chunk u ^ ((r >> 1) & 7) of that row, and readers apply the same XOR: 16
+// consecutive rows then read 16 different slots (no bank conflicts).
+// After the K loop the accumulators are staged through LDS so that the tail runs
+// once per element in row-major order and stores are contiguous 8/16-byte pieces.
 #include <hip/hip_runtime.h>
 
 #include "device_common.h"
@@ -30,9 +38,17 @@ hipError_t igemm_launch_kind_2(int cfg, bool conv, const IgemmArgs& a, hipStream
 
 namespace {
 
-constexpr int kSlabBytes = 128;              // bytes of K per LDS row
-constexpr int kRowStride = kSlabBytes + 16;  // padded LDS row (16B-slot skew: conflict-free b128 reads)
+constexpr int kSlabBytes = 128;  // bytes of K per LDS row
 constexpr int kThreads = 256;
+constexpr int kLdsBytes = 160 * 1024;
+constexpr unsigned kRsrcFlags = 0x00020000u;   // raw buffer, 32-bit data format
+constexpr unsigned kBufRange = 0x80000000u;    // every real offset is below 2 GiB (checked at launch) ...
+constexpr unsigned kOutside = 0x80000000u;     // ... and this one reads as zeros, with any slab offset added
+
+#define PML_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+
+// Sum of two byte offsets, each of which may be the "outside" mark.
+__device__ inline unsigned join_offsets(unsigned x, unsigned y) { return ((x | y) & kOutside) ? kOutside : x + y; }
 
 // XCD-aware tile order: hardware deals consecutive workgroup ids round-robin to
 // the 8 XCDs, each with its own L2.  Re-number so that one XCD works on a
@@ -44,6 +60,13 @@ __device__ inline int xcd_remap(int bid, int nblocks) {
   return (bid % kXcds) * per + (bid / kXcds);
 }
 
+template <int BM, int BN>
+struct Ring {
+  static constexpr int kStage = (BM + BN) * kSlabBytes;                 // A rows then Bt rows
+  static constexpr int kStages = 3 * kStage <= kLdsBytes ? 3 : 2;
+  static constexpr int kBytes = kStages * kStage;
+};
+
 // BM x BN output tile, WAVES_M x WAVES_N wavefront grid (WAVES_M * WAVES_N == 4).
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV>
 __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
@@ -53,7 +76,11 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   constexpr int MI = WM / 32, NI = WN / 32;
   constexpr int A_VECS = BM * 8 / kThreads;  // 16-byte vectors per thread per slab
   constexpr int B_VECS = BN * 8 / kThreads;
-  constexpr int kStage = (BM + BN) * kRowStride;  // one buffer: A rows then Bt rows
+  constexpr int kStage = Ring<BM, BN>::kStage;
+  constexpr int kStages = Ring<BM, BN>::kStages;
+  constexpr int kAhead = kStages - 1;              // slabs in flight ahead of the one being multiplied
+  constexpr int kLoads = A_VECS + B_VECS;          // loads a thread issues per slab
+  static_assert(kAhead * kLoads <= 63, "the vmcnt field counts at most 63 loads");
   typedef typename Acc<KIND>::type acc_t;
   typedef typename Acc<KIND>::scalar accs_t;
   typedef accs_t acc4_t __attribute__((ext_vector_type(4)));
@@ -61,7 +88,8 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   const int tiles_n = (int)((p.N + BN - 1) / BN);
@@ -70,19 +98,22 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   const int64_t m0 = (int64_t)(tile / tiles_n) * BM;
   const int64_t n0 = (int64_t)(tile % tiles_n) * BN;
 
-  // ---- per-thread load assignments (fixed across slabs): vector lv of rows lr + 32*i ----
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)kBufRange, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.Bt, 0, (int)kBufRange, kRsrcFlags);
+
+  // ---- per-thread load assignments (fixed across slabs): slot lv of rows lr + 32*i ----
   const int lv = tid & 7;
   const int lr = tid >> 3;
+  const int lc = lv ^ ((lr >> 1) & 7);                        // the chunk of its row this thread fetches
   const int kbytes_row = (int)(CONV ? p.CI * ES : p.K * ES);  // valid bytes per (tap) row
 
-  const unsigned char* a_row[A_VECS];  // GEMM: row start; CONV: image start
-  bool a_ok[A_VECS];
+  unsigned a_off[A_VECS];  // GEMM: byte offset of the row; CONV: of the image; kOutside for rows past M
   int a_ih0[A_VECS], a_iw0[A_VECS];
 #pragma unroll
   for (int i = 0; i < A_VECS; ++i) {
     const int64_t m = m0 + lr + 32 * i;
-    a_ok[i] = m < p.M;
-    const int64_t mm = a_ok[i] ? m : 0;
+    const bool ok = m < p.M;
+    const int64_t mm = ok ? m : 0;
     if (CONV) {
       const int ow = (int)(mm % p.OW);
       const int64_t t = mm / p.OW;
@@ -90,75 +121,65 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
       const int64_t nb = t / p.OH;
       a_ih0[i] = oh * p.SH - p.PH;
       a_iw0[i] = ow * p.SW - p.PW;
-      a_row[i] = (const unsigned char*)p.A + nb * ((int64_t)p.H * p.W * p.CI * ES);
+      a_off[i] = ok ? (unsigned)(nb * ((int64_t)p.H * p.W * p.CI * ES)) : kOutside;
     } else {
       a_ih0[i] = a_iw0[i] = 0;
-      a_row[i] = (const unsigned char*)p.A + mm * p.lda * ES;
+      a_off[i] = ok ? (unsigned)(mm * p.lda * ES) : kOutside;
     }
   }
-  const unsigned char* b_row[B_VECS];
-  bool b_ok[B_VECS];
+  unsigned b_off[B_VECS];
 #pragma unroll
   for (int i = 0; i < B_VECS; ++i) {
     const int64_t n = n0 + lr + 32 * i;
-    b_ok[i] = n < p.N;
-    b_row[i] = (const unsigned char*)p.Bt + (b_ok[i] ? n : 0) * p.ldbt * ES;
+    b_off[i] = n < p.N ? (unsigned)(n * p.ldbt * ES) : kOutside;
   }
 
   const int slabs_per_tap = (kbytes_row + kSlabBytes - 1) / kSlabBytes;
   const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : slabs_per_tap;
   const int pix_bytes = p.CI * ES;
 
-  i32x4_t ra[A_VECS], rb[B_VECS];
-  const i32x4_t zero4 = {0, 0, 0, 0};
-
-  // Loads are unconditional from a clamped (always valid) address; the value is
-  // replaced by zero afterwards when the element is outside the problem.
-  auto load_slab = [&](int s) {
+  // Requests of slab s into ring stage `stage`, one 16-byte-per-lane load at a time (index l: the A
+  // rows first, then the Bt rows) so that they can be spread between the MFMAs.  Past the last slab
+  // every offset is outside: the request count per slab stays constant, which is what the vmcnt
+  // arithmetic below relies on.
+  unsigned char* req_base = smem;
+  unsigned req_a = 0, req_b = 0;  // slab-dependent part of the A / Bt offsets (CONV: A adds the tap per row)
+  int req_dh = 0, req_dw = 0;
+  bool req_ok = false;
+  auto prepare_slab = [&](int s, int stage) {
+    req_base = smem + stage * kStage + wave * (8 * kSlabBytes);
+    const bool live = s < n_slabs;
     if (CONV) {
       const int tap = s / slabs_per_tap;
       const int cs = s - tap * slabs_per_tap;
       const int kh = tap / p.KW, kw = tap - kh * p.KW;
-      const int cb = cs * kSlabBytes + lv * 16;  // byte offset inside the channel vector
-      const bool c_ok = cb < kbytes_row;
-      const int cbs = c_ok ? cb : 0;
-      const int dh = kh * p.DH, dw = kw * p.DW;
-#pragma unroll
-      for (int i = 0; i < A_VECS; ++i) {
-        const int ih = a_ih0[i] + dh, iw = a_iw0[i] + dw;
-        const bool ok = a_ok[i] && c_ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-        const int off = ok ? (ih * p.W + iw) * pix_bytes + cbs : 0;
-        const i32x4_t v = *(const i32x4_t*)(a_row[i] + off);
-        ra[i] = ok ? v : zero4;
-      }
-      const int kb = tap * pix_bytes + cbs;  // Bt row: tap-major, channel-minor
-#pragma unroll
-      for (int i = 0; i < B_VECS; ++i) {
-        const i32x4_t v = *(const i32x4_t*)(b_row[i] + kb);
-        rb[i] = (b_ok[i] && c_ok) ? v : zero4;
-      }
+      const int cb = cs * kSlabBytes + lc * 16;  // byte offset inside the channel vector
+      req_ok = live && cb < kbytes_row;
+      req_dh = kh * p.DH;
+      req_dw = kw * p.DW;
+      req_a = (unsigned)cb;
+      req_b = req_ok ? (unsigned)(tap * pix_bytes + cb) : kOutside;  // Bt row: tap-major, channel-minor
     } else {
-      const int kb = s * kSlabBytes + lv * 16;
-      const bool k_ok = kb < kbytes_row;
-      const int kbs = k_ok ? kb : 0;
-#pragma unroll
-      for (int i = 0; i < A_VECS; ++i) {
-        const i32x4_t v = *(const i32x4_t*)(a_row[i] + kbs);
-        ra[i] = (a_ok[i] && k_ok) ? v : zero4;
-      }
-#pragma unroll
-      for (int i = 0; i < B_VECS; ++i) {
-        const i32x4_t v = *(const i32x4_t*)(b_row[i] + kbs);
-        rb[i] = (b_ok[i] && k_ok) ? v : zero4;
-      }
+      const int kbo = s * kSlabBytes + lc * 16;
+      req_a = req_b = (live && kbo < kbytes_row) ? (unsigned)kbo : kOutside;
     }
   };
-  auto store_slab = [&](int buf) {
-    unsigned char* base = smem + buf * kStage + lr * kRowStride + lv * 16;
-#pragma unroll
-    for (int i = 0; i < A_VECS; ++i) *(i32x4_t*)(base + (32 * i) * kRowStride) = ra[i];
-#pragma unroll
-    for (int i = 0; i < B_VECS; ++i) *(i32x4_t*)(base + (BM + 32 * i) * kRowStride) = rb[i];
+  auto issue_load = [&](int l) {
+    if (l < A_VECS) {
+      unsigned off;
+      if (CONV) {
+        const int ih = a_ih0[l] + req_dh, iw = a_iw0[l] + req_dw;
+        const bool ok = req_ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+        off = ok ? join_offsets(a_off[l], (unsigned)((ih * p.W + iw) * pix_bytes) + req_a) : kOutside;
+      } else {
+        off = join_offsets(a_off[l], req_a);
+      }
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, PML_LDS(req_base + l * 32 * kSlabBytes), 16, (int)off, 0, 0, 0);
+    } else {
+      const int i = l - A_VECS;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * 32) * kSlabBytes), 16,
+                                               (int)join_offsets(b_off[i], req_b), 0, 0, 0);
+    }
   };
 
   acc_t acc[MI][NI];
@@ -169,44 +190,77 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  load_slab(0);
-  store_slab(0);
-  __syncthreads();
-
-  const int frow = lane & 31;       // row of the 32x32 block this lane feeds
-  const int fk = (lane >> 5) * 16;  // its 16-byte half of a 32-byte K-block
-
-  for (int s = 0; s < n_slabs; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < n_slabs) load_slab(s + 1);
-    const unsigned char* a_base = smem + buf * kStage + (wm * WM + frow) * kRowStride + fk;
-    const unsigned char* b_base = smem + buf * kStage + (BM + wn * WN + frow) * kRowStride + fk;
 #pragma unroll
-    for (int kb = 0; kb < kSlabBytes / 32; ++kb) {
-      i32x4_t fa[MI], fb[NI];
+  for (int s = 0; s < kAhead; ++s) {
+    prepare_slab(s, s);
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[i] = *(const i32x4_t*)(a_base + i * 32 * kRowStride + kb * 32);
-#pragma unroll
-      for (int j = 0; j < NI; ++j) fb[j] = *(const i32x4_t*)(b_base + j * 32 * kRowStride + kb * 32);
-#pragma unroll
-      for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j) mma_block<KIND>(acc[i][j], fb[j], fa[i]);
-    }
-    if (s + 1 < n_slabs) store_slab(buf ^ 1);
-    __syncthreads();
+    for (int l = 0; l < kLoads; ++l) issue_load(l);
   }
 
-  // ---- stage the accumulator tile in LDS as ctile[BM][BN + 4] ----
+  const int frow = lane & 31;  // row of the 32x32 block this lane feeds
+  int fslot[kSlabBytes / 32];  // byte offset of its 16-byte half of each 32-byte K-block, swizzled
+#pragma unroll
+  for (int kb = 0; kb < kSlabBytes / 32; ++kb) fslot[kb] = ((kb * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
+
+  int stage = 0;  // ring stage of slab s
+  for (int s = 0; s < n_slabs; ++s) {
+    // slab s has landed once at most (kAhead - 1) later slabs of this thread are outstanding;
+    // the barrier extends that to every thread and also says: everyone is done with slab s - 1
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (((kAhead - 1) * kLoads) & 15) | ((((kAhead - 1) * kLoads) >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    int free_stage = stage - 1;
+    if (free_stage < 0) free_stage = kStages - 1;
+    prepare_slab(s + kAhead, free_stage);
+    const unsigned char* a_base = smem + stage * kStage + (wm * WM + frow) * kSlabBytes;
+    const unsigned char* b_base = smem + stage * kStage + (BM + wn * WN + frow) * kSlabBytes;
+    // Per K-block: MI*NI MFMA groups in program order; behind the m-th one sit one request of the
+    // slab two ahead and one fragment read of K-block kb + 1, so that neither the texture path nor
+    // LDS latency ever holds up the matrix pipe.  sched_barrier pins that order.
+    constexpr int kBlocks = kSlabBytes / 32;
+    i32x4_t fa[2][MI], fb[2][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(a_base + i * 32 * kSlabBytes + fslot[0]);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(b_base + j * 32 * kSlabBytes + fslot[0]);
+#pragma unroll
+    for (int kb = 0; kb < kBlocks; ++kb) {
+      const int cur = kb & 1, nxt = cur ^ 1;
+      const int l0 = kb * kLoads / kBlocks, l1 = (kb + 1) * kLoads / kBlocks;
+      constexpr int kSlots = MI * NI;
+#pragma unroll
+      for (int m = 0; m < kSlots; ++m) {
+        mma_block<KIND>(acc[m / NI][m % NI], fb[cur][m % NI], fa[cur][m / NI]);
+        // requests and fragment reads of this K-block, dealt over its MFMA slots
+#pragma unroll
+        for (int l = l0 + m; l < l1; l += kSlots) issue_load(l);
+        if (kb + 1 < kBlocks) {
+#pragma unroll
+          for (int d = m; d < MI + NI; d += kSlots) {
+            if (d < MI)
+              fa[nxt][d] = *(const i32x4_t*)(a_base + d * 32 * kSlabBytes + fslot[kb + 1]);
+            else
+              fb[nxt][d - MI] = *(const i32x4_t*)(b_base + (d - MI) * 32 * kSlabBytes + fslot[kb + 1]);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if (++stage == kStages) stage = 0;
+  }
+  // drain the (all-outside) requests still in flight before LDS is reused
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+
+  // ---- stage accumulators in LDS and run the tail ----
   // The MFMAs ran with the Bt fragment as the row operand, so in a 32x32 block a
   // lane owns tile row (m) lane%32 and the columns (n) 8*(r/4) + 4*(lane/32) + r%4:
   // four consecutive columns per register quad, one 16-byte LDS store each.
-  constexpr int CS = BN + 4;
-  static_assert((size_t)BM * CS * 4 <= 2 * (size_t)kStage, "accumulator tile must fit in the pipeline buffers");
-  accs_t* ctile = (accs_t*)smem;
-  {
-    const int crow = lane & 31;
-    const int ccol = (lane >> 5) * 4;
+  const int crow = lane & 31;
+  const int ccol = (lane >> 5) * 4;
+  if constexpr ((size_t)BM * (BN + 4) * 4 <= (size_t)Ring<BM, BN>::kBytes) {
+    // the whole tile fits in the pipeline buffers: ctile[BM][BN + 4], tail by all 256 threads
+    constexpr int CS = BN + 4;
+    accs_t* ctile = (accs_t*)smem;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -218,10 +272,35 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
           for (int e = 0; e < 4; ++e) q[e] = acc[i][j][4 * g + e];
           *(acc4_t*)&ctile[(wm * WM + i * 32 + crow) * CS + wn * WN + j * 32 + 8 * g + ccol] = q;
         }
+    __syncthreads();
+    tile_tail<KIND, BM, BN, kThreads>(p, ctile, m0, n0, tid);
+  } else {
+    // large tiles: every wavefront stages RB of its 32-row blocks at a time in a private
+    // region, wtile[RB * 32][WN + 4], and runs the tail over them with its 64 lanes
+    constexpr int CS = WN + 4;
+    constexpr int kBudget = Ring<BM, BN>::kBytes / 4 / 16 * 16;  // bytes per wavefront
+    constexpr int kFit = kBudget / (32 * CS * 4);
+    constexpr int RB = kFit >= MI ? MI : (kFit >= 4 ? 4 : (kFit >= 2 ? 2 : 1));  // MI is a power of two
+    static_assert(RB >= 1 && MI % RB == 0, "row blocks must stage evenly");
+    accs_t* wtile = (accs_t*)(smem + wave * kBudget);
+#pragma unroll
+    for (int i0 = 0; i0 < MI; i0 += RB) {
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            acc4_t q;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) q[e] = acc[i0 + i][j][4 * g + e];
+            *(acc4_t*)&wtile[(i * 32 + crow) * CS + j * 32 + 8 * g + ccol] = q;
+          }
+      __syncthreads();
+      tile_tail<KIND, RB * 32, WN, 64>(p, wtile, m0 + wm * WM + i0 * 32, n0 + wn * WN, lane);
+      __syncthreads();
+    }
   }
-  __syncthreads();
-
-  tile_tail<KIND, BM, BN, kThreads>(p, ctile, m0, n0, tid);
 }
 
 // Bt[n][k] = B[k][n]: LDS-tiled transpose, 64x64 elements per workgroup.
@@ -245,7 +324,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ B,
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
+  const size_t lds = Ring<BM, BN>::kBytes;
   auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -264,6 +343,8 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
     case TILE_256x64: return launch_cfg<KIND, 256, 64, 4, CONV>(a, s);
     case TILE_64x64: return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);
+    case TILE_256x128: return launch_cfg<KIND, 256, 128, 2, CONV>(a, s);
+    case TILE_256x256: return launch_cfg<KIND, 256, 256, 2, CONV>(a, s);
   }
   return hipErrorInvalidValue;
 }
@@ -281,6 +362,11 @@ hipError_t PML_CAT(igemm_launch_kind_, PML_KIND)(int cfg, bool conv, const Igemm
 
 #if PML_KIND == 0
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s) {
+  // the kernel addresses both operands with 32-bit byte offsets below 2 GiB
+  const int64_t es = kind == KIND_BF16 ? 2 : (kind == KIND_I8 ? 1 : 4);
+  const int64_t a_bytes = conv ? (int64_t)a.NB * a.H * a.W * a.CI * es : a.M * a.lda * es;
+  const int64_t b_bytes = a.N * a.ldbt * es;
+  if (a_bytes >= ((int64_t)1 << 31) || b_bytes >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
   switch (kind) {
     case KIND_F32: return igemm_launch_kind_0(cfg, conv, a, s);
     case KIND_BF16: return igemm_launch_kind_1(cfg, conv, a, s);

@@ -12,7 +12,7 @@
 namespace pml {
 
 enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2 };
-enum { TILE_128x128 = 0, TILE_128x64, TILE_256x64, TILE_64x64 };
+enum { TILE_128x128 = 0, TILE_128x64, TILE_256x64, TILE_64x64, TILE_256x128, TILE_256x256 };
 
 struct TailPtrs {
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];

@@ -74,29 +74,34 @@ const char* tile_name(int t) {
     case TILE_128x64: return "128x64";
     case TILE_256x64: return "256x64";
     case TILE_64x64: return "64x64";
+    case TILE_256x128: return "256x128";
+    case TILE_256x256: return "256x256";
   }
   return "?";
 }
 
-// Stated tiling choice per shape class.  256 CUs want >= 256 workgroups in
-// flight (one wave of the grid); prefer the largest tile that still yields
-// about two workgroups per CU, and never a tile wider than N.
-int choose_tile(int64_t m, int64_t n) {
-  // PML_HIP_TILE=128x128|128x64|256x64|64x64 overrides the table (for tuning runs)
+// Stated tiling choice per shape class (k_bytes = bytes of K per row).  Measured on MI355X:
+//   4096^3 bf16 / int8:            256x256 131 / 80 us, 256x128 147 / 92, 128x64 173 / 107, 128x128 189 / 115
+//   conv 128x28x28x128 (*) 3x3x128: 128x64 79 us, 256x128 93, 128x128 104, 256x256 152
+//   conv 128x14x14x256 (*) 3x3x256: 256x128 68 us, 128x64 71, 128x128 78, 256x256 107
+//   gemm 100352x512x128 bf16:       128x64 96 us, 128x128 151, 256x128 156
+// Long K with enough 256x256 tiles to fill the chip: the big tile (least operand traffic per MFMA);
+// otherwise 128x64, which leaves room for two workgroups per CU; N <= 64: 64x64.
+int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
+  // PML_HIP_TILE=128x128|128x64|256x64|64x64|256x128|256x256 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
     const std::string v(e);
     if (v == "128x128") return TILE_128x128;
     if (v == "128x64") return TILE_128x64;
     if (v == "256x64" && n <= 64) return TILE_256x64;
     if (v == "64x64") return TILE_64x64;
+    if (v == "256x128") return TILE_256x128;
+    if (v == "256x256") return TILE_256x256;
   }
   auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-  const int64_t want = 2 * 256;
-  if (n <= 64) return TILE_64x64;  // measured on N128 56x56x64 (*) 3x3x64x64: 64x64 93 us, 128x64 111 us, 256x64 161 us
-  (void)want;
-  if (tiles(128, 128) >= want) return TILE_128x128;
-  if (tiles(128, 64) >= 256) return TILE_128x64;
-  return TILE_64x64;
+  if (n <= 64) return TILE_64x64;
+  if (k_bytes >= 4096 && tiles(256, 256) >= 128) return TILE_256x256;
+  return TILE_128x64;
 }
 
 // A tail that is only "relu?" can use the fast store path.
@@ -304,7 +309,7 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   p->kind = PLAN_GEMM;
   p->mfma_kind = kind;
   p->gemm = *d;
-  p->tile = choose_tile(d->m, d->n);
+  p->tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype));
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
   if (!d->b_layout && hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
@@ -406,7 +411,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   p->conv = *d;
   const int64_t M = d->n * d->oh * d->ow;
   const int64_t K = d->kh * d->kw * d->ci;
-  p->tile = choose_tile(M, d->co);
+  p->tile = choose_tile(M, d->co, K * es);
   p->bt_ld = K;
   if (via_patches) {
     // rows padded with zeros to whole 16-byte vectors on both GEMM operands
