@@ -74,15 +74,112 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
   const bool col_init = p.init != nullptr && p.init_rs == 0;
   accs_t cinit[4] = {0, 0, 0, 0};
   if (col_init) {
+    const int natural = KIND == KIND_I8 ? PML_HIP_I32 : p.out_dtype;
+    const int ies = natural == PML_HIP_BF16 ? 2 : 4;
+    if (full4 && p.init_cs == 1 && p.init_dtype == natural && (((uintptr_t)p.init + n * ies) & (4 * ies - 1)) == 0) {
+      // contiguous bias of the result type: one 8- or 16-byte load
+      if (natural == PML_HIP_BF16) {
+        const uint2 w = *(const uint2*)((const uint16_t*)p.init + n);
+        cinit[0] = (accs_t)__uint_as_float(w.x << 16);
+        cinit[1] = (accs_t)__uint_as_float(w.x & 0xffff0000u);
+        cinit[2] = (accs_t)__uint_as_float(w.y << 16);
+        cinit[3] = (accs_t)__uint_as_float(w.y & 0xffff0000u);
+      } else if (natural == PML_HIP_I32) {
+        const i32x4_t w = *(const i32x4_t*)((const int*)p.init + n);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (n + q < p.N) {
-        Scalar<float, int> b = load_scalar<float, int>(p.init, (n + q) * p.init_cs, p.init_dtype);
-        cinit[q] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+        for (int q = 0; q < 4; ++q) cinit[q] = (accs_t)w[q];
+      } else {
+        const f32x4_t w = *(const f32x4_t*)((const float*)p.init + n);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) cinit[q] = (accs_t)w[q];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (n + q < p.N) {
+          Scalar<float, int> b = load_scalar<float, int>(p.init, (n + q) * p.init_cs, p.init_dtype);
+          cinit[q] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+        }
       }
     }
   }
-  for (int row = tid / TPR; row < BM; row += RPP) {
+  const int row0 = tid / TPR;
+
+  if (fast) {
+    // Rows in batches of up to 8: all residual loads of a batch are issued before the first is used.
+    constexpr int kIters = (BM + RPP - 1) / RPP;
+    constexpr int kBatch = kIters < 8 ? kIters : 8;
+#pragma unroll
+    for (int it0 = 0; it0 < kIters; it0 += kBatch) {
+      i32x4_t res[kBatch];
+#pragma unroll
+      for (int c = 0; c < kBatch; ++c) {
+        const int row = row0 + (it0 + c) * RPP;
+        const int64_t m = m0 + row;
+        res[c] = i32x4_t{0, 0, 0, 0};
+        if (residual && row < BM && m < p.M) {
+          if (KIND != KIND_I8 && p.out_dtype == PML_HIP_BF16) {
+            const uint2 x = *(const uint2*)((const uint16_t*)p.operands[0] + m * res_rs + n);
+            res[c][0] = (int)x.x;
+            res[c][1] = (int)x.y;
+          } else {
+            res[c] = *(const i32x4_t*)((const int*)p.operands[0] + m * res_rs + n);
+          }
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < kBatch; ++c) {
+        const int row = row0 + (it0 + c) * RPP;
+        const int64_t m = m0 + row;
+        if (row >= BM || m >= p.M) continue;
+        accs_t v4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v4[q] = ctile[row * CS + c4 + q] + cinit[q];
+        if (p.init && !col_init) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            Scalar<float, int> b = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
+            v4[q] += KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
+          }
+        }
+        if (KIND == KIND_I8) {
+          i32x4_t w;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int v = (int)((unsigned)(int)v4[q] + (unsigned)res[c][q]);
+            w[q] = (p.tail_relu && v < 0) ? 0 : v;
+          }
+          *(i32x4_t*)((int*)p.C + m * p.ldc + n) = w;
+        } else if (p.out_dtype == PML_HIP_BF16) {
+          uint32_t h[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            h[q] = f32_to_bf16_bits((float)v4[q]);
+            if (residual) {
+              // the contraction result is rounded first, then the bf16 addition rounds again
+              const uint32_t xw = (uint32_t)res[c][q >> 1];
+              const float xf = __uint_as_float((q & 1) ? (xw & 0xffff0000u) : (xw << 16));
+              h[q] = f32_to_bf16_bits(__uint_as_float(h[q] << 16) + xf);
+            }
+            // relu on the rounded value: negative, non-NaN, non-zero -> 0  (x < 0 ? 0 : x)
+            if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
+          }
+          *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        } else {
+          f32x4_t w;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float v = residual ? (float)v4[q] + __int_as_float(res[c][q]) : (float)v4[q];
+            w[q] = (p.tail_relu && v < 0.f) ? 0.f : v;
+          }
+          *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
+        }
+      }
+    }
+    return;
+  }
+
+  for (int row = row0; row < BM; row += RPP) {
     const int64_t m = m0 + row;
     if (m >= p.M) break;
     accs_t v4[4];
@@ -99,47 +196,6 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
           v4[q] += KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
         }
       }
-    }
-    if (fast) {
-      if (KIND == KIND_I8) {
-        i32x4_t w;
-        i32x4_t x = {0, 0, 0, 0};
-        if (residual) x = *(const i32x4_t*)((const int*)p.operands[0] + m * res_rs + n);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int v = (int)((unsigned)(int)v4[q] + (unsigned)x[q]);
-          w[q] = (p.tail_relu && v < 0) ? 0 : v;
-        }
-        *(i32x4_t*)((int*)p.C + m * p.ldc + n) = w;
-      } else if (p.out_dtype == PML_HIP_BF16) {
-        uint32_t h[4];
-        uint2 x = make_uint2(0, 0);
-        if (residual) x = *(const uint2*)((const uint16_t*)p.operands[0] + m * res_rs + n);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          h[q] = f32_to_bf16_bits((float)v4[q]);
-          if (residual) {
-            // the contraction result is rounded first, then the bf16 addition rounds again
-            const uint32_t xw = (q < 2) ? x.x : x.y;
-            const float xf = __uint_as_float((q & 1) ? (xw & 0xffff0000u) : (xw << 16));
-            h[q] = f32_to_bf16_bits(__uint_as_float(h[q] << 16) + xf);
-          }
-          // relu on the rounded value: negative, non-NaN, non-zero -> 0  (x < 0 ? 0 : x)
-          if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
-        }
-        *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-      } else {
-        f32x4_t w;
-        f32x4_t x = {0.f, 0.f, 0.f, 0.f};
-        if (residual) x = *(const f32x4_t*)((const float*)p.operands[0] + m * res_rs + n);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float v = residual ? (float)v4[q] + x[q] : (float)v4[q];
-          w[q] = (p.tail_relu && v < 0.f) ? 0.f : v;
-        }
-        *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
-      }
-      continue;
     }
     for (int q = 0; q < 4; ++q) {
       if (n + q >= p.N) break;
