@@ -80,13 +80,17 @@ const char* tile_name(int t) {
   return "?";
 }
 
-// Stated tiling choice per shape class (k_bytes = bytes of K per row).  Measured on MI355X:
-//   4096^3 bf16 / int8:            256x256 131 / 80 us, 256x128 147 / 92, 128x64 173 / 107, 128x128 189 / 115
-//   conv 128x28x28x128 (*) 3x3x128: 128x64 79 us, 256x128 93, 128x128 104, 256x256 152
-//   conv 128x14x14x256 (*) 3x3x256: 256x128 68 us, 128x64 71, 128x128 78, 256x256 107
-//   gemm 100352x512x128 bf16:       128x64 96 us, 128x128 151, 256x128 156
-// Long K with enough 256x256 tiles to fill the chip: the big tile (least operand traffic per MFMA);
-// otherwise 128x64, which leaves room for two workgroups per CU; N <= 64: 64x64.
+// Stated tiling choice per shape class (k_bytes = bytes of K per row).  Measured on MI355X (us):
+//   4096^3 bf16 / int8:             256x256 131 / 80, 256x128 147 / 92, 128x64 173 / 107, 128x128 189 / 115
+//   conv 128x28x28x128 (*) 3x3x128: 64x64 73, 128x64 79, 256x128 100, 128x128 104
+//   conv 128x14x14x256 (*) 3x3x256: 64x64 70, 128x64 71, 256x128 75, 128x128 78
+//   conv 128x7x7x512   (*) 3x3x512: 128x64 64, 128x128 65, 64x64 78, 256x128 113
+//   gemm 401408x256x64 bf16:        64x64 142, 128x64 166, 128x128 278
+//   gemm 25088x1024x256 bf16:       64x64 51, 128x64 57, 128x128 90
+// One tile per workgroup and a serial load / multiply / store life per tile: what hides latency is
+// how many workgroups fit a CU (64x64: 3, 128x64: 2, larger: 1).  So: long K with enough 256x256
+// tiles to fill the chip takes the big tile (least operand traffic per MFMA); otherwise the smaller
+// of 64x64 and 128x64 by (rounds of resident workgroups) x (tile area), the larger tile on a tie.
 int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
   // PML_HIP_TILE=128x128|128x64|256x64|64x64|256x128|256x256 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
@@ -101,7 +105,9 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
   auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (n <= 64) return TILE_64x64;
   if (k_bytes >= 4096 && tiles(256, 256) >= 128) return TILE_256x256;
-  return TILE_128x64;
+  const int64_t rounds_small = (tiles(64, 64) + 3 * 256 - 1) / (3 * 256);
+  const int64_t rounds_wide = (tiles(128, 64) + 2 * 256 - 1) / (2 * 256);
+  return rounds_small < 2 * rounds_wide ? TILE_64x64 : TILE_128x64;
 }
 
 // A tail that is only "relu?" can use the fast store path.
