@@ -117,6 +117,76 @@ def copy_calibration(hk, steps):
             'ms': round(ms, 4), 'GBps': round(2 * n * 4 / ms / 1e6, 1)}
 
 
+def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):
+    """Depthwise 3x3, pointwise 728->728 with the fused scale/shift + ReLU tail, max-pool 3x3/2 with window argmax."""
+    out = {}
+    px = N * H * W
+    dI, dD, dP = hk.DeviceBuffer(px * C * 2), hk.DeviceBuffer(px * C * 2), hk.DeviceBuffer(px * C * 2)
+    dI.fill_u32(0x3f803f80)
+    # depthwise
+    d = hk.Dwconv2dDesc()
+    d.dtype = hk.BF16
+    d.n, d.h, d.w, d.c, d.kh, d.kw, d.oh, d.ow = N, H, W, C, 3, 3, H, W
+    d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
+    d.pad_h = d.pad_w = 1
+    plan = L.pml_hip_dwconv2d_dispatch(ctypes.byref(d))
+    dF = hk.DeviceBuffer(9 * C * 2)
+    dF.fill_u32(0x3c003c00)
+    ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_dwconv2d_invoke(plan, dI.ptr, dF.ptr, dD.ptr, none, none, None)), 20, 3)
+    nbytes = 2 * px * C * 2
+    out['depthwise3x3'] = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms / 1e6, 1), 'frac_hbm': round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    # pointwise + scale/shift + relu
+    g = hk.GemmDesc()
+    g.in_dtype = g.out_dtype = g.c_dtype = hk.BF16
+    g.m, g.n, g.k, g.lda, g.ldb, g.ldc = px, C, C, C, C, C
+    g.tail = hk.make_tail(ops=[(hk.EPI_MUL, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 1, 0.0),
+                               (hk.EPI_RELU, hk.BF16, 0, 0, 0.0)], operands=[(hk.BF16, 0, 1), (hk.BF16, 0, 1)])
+    pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+    dW, dS, dT = hk.DeviceBuffer(C * C * 2), hk.DeviceBuffer(C * 2), hk.DeviceBuffer(C * 2)
+    for b in (dW, dS, dT):
+        b.fill_u32(0x3c003c00)
+    hk.check(L.pml_hip_gemm_pack_b(pg, dW.ptr, None))
+    ops = hk.ptr_array([dS.ptr, dT.ptr])
+    ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dD.ptr, None, dP.ptr, None, ops, none, None)), 20, 3)
+    fl = 2.0 * px * C * C
+    out['pointwise_scale_shift_relu'] = {'ms': round(ms, 4), 'TFLOP/s': round(fl / ms / 1e9, 1),
+                                         'frac_mfma_bf16': round(fl / ms / 1e9 / PEAK['bf16'], 4), 'plan': hk.describe(pg)}
+    # max-pool 3x3/2 SAME + window argmax
+    p = hk.Pool2dDesc()
+    p.dtype, p.agg = hk.BF16, hk.AGG_MAX
+    p.n, p.h, p.w, p.c, p.kh, p.kw, p.oh, p.ow = N, H, W, C, 3, 3, 10, 10
+    p.stride_h = p.stride_w = 2
+    p.pad_h = p.pad_w = 1
+    p.with_index = 1
+    pp = L.pml_hip_pool2d_dispatch(ctypes.byref(p))
+    dM, dX = hk.DeviceBuffer(N * 100 * C * 2), hk.DeviceBuffer(N * 100 * C * 4)
+    ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_pool2d_invoke(pp, dP.ptr, dM.ptr, dX.ptr, None)), 20, 3)
+    nbytes = px * C * 2 + N * 100 * C * 6
+    out['maxpool3x3s2_argmax'] = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms / 1e6, 1), 'frac_hbm': round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    for b in (dI, dD, dP, dF, dW, dS, dT, dM, dX):
+        b.free()
+    return out
+
+
+def resnet50_leg(E, batch=128, runs=5):
+    """Whole-network forward through libplaidml.so: device time between the first and the last kernel of a run."""
+    from plaidml_amd import edsl as P, op as Pop, resnet50
+    prog, _, flops_full_box = resnet50.build(P, Pop, batch=batch, round_fn=E.round_bf16)
+    runner = P.Runner(prog, target='hip')
+    x = np.random.default_rng(11).uniform(0, 1, (batch, 224, 224, 3)).astype(np.float32)
+    times = []
+    for _ in range(runs):
+        out, = runner.run([x])
+        times.append(P.last_run_stats())
+    if not (np.isfinite(out).all() and np.allclose(out.sum(axis=1), 1.0, atol=2e-2)):
+        raise SystemExit('bench: ResNet-50 output is not a probability distribution')
+    best = min(times[1:], key=lambda t: t['kernel_ms'])
+    return {'img_per_s': round(batch / (best['kernel_ms'] * 1e-3), 1), 'kernel_ms': round(best['kernel_ms'], 3),
+            'h2d_ms': round(best['h2d_ms'], 3), 'd2h_ms': round(best['d2h_ms'], 3), 'launches': int(best['launches']),
+            'TFLOP/s_full_box': round(flops_full_box / (best['kernel_ms'] * 1e-3) / 1e12, 1),
+            'frac_mfma_bf16': round(flops_full_box / (best['kernel_ms'] * 1e-3) / 1e12 / PEAK['bf16'], 4)}
+
+
 def committed_traffic():
     """HBM bytes per launch of the bench kernel from the committed counter summary, or None."""
     path = os.path.join(ROOT, 'profiles', 'conv_halo3x3_bf16_configs1_hbm_traffic.md')
@@ -240,6 +310,10 @@ def main():
         ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pi, dAi.ptr, dBi.ptr, dCi.ptr, None, none, none, None)), 20, 5)
         extra['gemm_i8_4096_configs2'] = {'ms': round(ms, 4), 'TOP/s': round(2 * 4096 ** 3 / ms / 1e9, 2),
                                           'frac_mfma_i8': round(2 * 4096 ** 3 / ms / 1e9 / PEAK['i8'], 4), 'plan': hk.describe(pi)}
+        # configs[3]: Xception block pieces at full size (N64 19x19x728 bf16), each kernel alone
+        extra['xception_block_configs3'] = xception_leg(hk, L, none)
+        # configs[4]: ResNet-50 v1.5, batch 128, bf16, through the plaidml API (weights are program constants)
+        extra['resnet50_v1_5_b128_bf16'] = resnet50_leg(E)
         result['extra'] = extra
 
     print(json.dumps(result))

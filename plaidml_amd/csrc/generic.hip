@@ -311,23 +311,34 @@ __global__ __launch_bounds__(256) void eltwise_vec_kernel(EltwiseArgs a, int64_t
   const pml_hip_eltwise_desc& d = a.d;
   const int64_t n_vec = a.total / V;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_vec; g += stride) {
-    const int64_t e0 = g * V;
-    i32x4_t raw = *(const i32x4_t*)((const unsigned char*)a.in + e0 * ES);
-    i32x4_t res;
-    const int64_t c0 = e0 % inner;
+  constexpr int U = 4;  // independent 16-byte loads in flight per thread
+  for (int64_t g0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g0 < n_vec; g0 += U * stride) {
+    i32x4_t raw[U];
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      int cur = d.in_dtype;
-      Scalar<float, int> v = load_scalar<float, int>(&raw, e, cur);
-      int64_t off[PML_HIP_MAX_EPI_OPERANDS];
-#pragma unroll
-      for (int q = 0; q < PML_HIP_MAX_EPI_OPERANDS; ++q)
-        off[q] = ((opnd_full_mask >> q) & 1) ? e0 + e : (((opnd_vec_mask >> q) & 1) ? c0 + e : 0);
-      v = run_tail<float, int>(d.tail, v, &cur, a.operands, off, a.outs, e0 + e);
-      store_scalar<float, int>(&res, e, cur, v);
+    for (int u = 0; u < U; ++u) {
+      const int64_t g = g0 + u * stride;
+      if (g < n_vec) raw[u] = *(const i32x4_t*)((const unsigned char*)a.in + g * V * ES);
     }
-    *(i32x4_t*)((unsigned char*)a.out + e0 * ES) = res;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t g = g0 + u * stride;
+      if (g >= n_vec) break;
+      const int64_t e0 = g * V;
+      i32x4_t res;
+      const int64_t c0 = e0 % inner;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        int cur = d.in_dtype;
+        Scalar<float, int> v = load_scalar<float, int>(&raw[u], e, cur);
+        int64_t off[PML_HIP_MAX_EPI_OPERANDS];
+#pragma unroll
+        for (int q = 0; q < PML_HIP_MAX_EPI_OPERANDS; ++q)
+          off[q] = ((opnd_full_mask >> q) & 1) ? e0 + e : (((opnd_vec_mask >> q) & 1) ? c0 + e : 0);
+        v = run_tail<float, int>(d.tail, v, &cur, a.operands, off, a.outs, e0 + e);
+        store_scalar<float, int>(&res, e, cur, v);
+      }
+      *(i32x4_t*)((unsigned char*)a.out + e0 * ES) = res;
+    }
   }
 }
 

@@ -179,6 +179,95 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
     return;
   }
 
+  // tail_mode 3: up to four float steps in the result type whose operands are immediates, scalars
+  // or per-column vectors (scale / shift / clamp chains).  The operand values of this thread's four
+  // columns are fetched once; every step rounds to the result type like the interpreter does.
+  if (KIND != KIND_I8 && p.tail_mode == 3 && full4 && (p.ldc & 3) == 0) {
+    const bool bf = p.out_dtype == PML_HIP_BF16;
+    auto rnd = [&](float x) { return bf ? __uint_as_float(f32_to_bf16_bits(x) << 16) : x; };
+    float xs[4][4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xs[st][q] = 0.f;
+      if (st < p.tail.n_ops) {
+        const pml_hip_epi_op& op = p.tail.ops[st];
+        if (op.operand_kind == PML_HIP_OPND_TENSOR) {
+          const void* base = p.operands[op.operand];
+          if (p.tail.operand_col_stride[op.operand] == 0) {
+            const float x = bf ? __uint_as_float((uint32_t)((const uint16_t*)base)[0] << 16) : ((const float*)base)[0];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xs[st][q] = x;
+          } else if (bf) {
+            const uint2 w = *(const uint2*)((const uint16_t*)base + n);
+            xs[st][0] = __uint_as_float(w.x << 16);
+            xs[st][1] = __uint_as_float(w.x & 0xffff0000u);
+            xs[st][2] = __uint_as_float(w.y << 16);
+            xs[st][3] = __uint_as_float(w.y & 0xffff0000u);
+          } else {
+            const f32x4_t w = *(const f32x4_t*)((const float*)base + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xs[st][q] = w[q];
+          }
+        } else if (op.operand_kind == PML_HIP_OPND_IMM) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) xs[st][q] = rnd((float)op.imm);
+        }
+      }
+    }
+    for (int row = row0; row < BM; row += RPP) {
+      const int64_t m = m0 + row;
+      if (m >= p.M) break;
+      float v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = (float)ctile[row * CS + c4 + q] + (float)cinit[q];
+      if (p.init && !col_init) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          Scalar<float, int> b = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
+          v[q] += b.f;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = rnd(v[q]);
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        if (st < p.tail.n_ops) {
+          const int opc = p.tail.ops[st].opcode;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float a = v[q], b = xs[st][q];
+            float r = a;
+            switch (opc) {
+              case PML_HIP_EPI_ADD: r = a + b; break;
+              case PML_HIP_EPI_SUB: r = a - b; break;
+              case PML_HIP_EPI_RSUB: r = b - a; break;
+              case PML_HIP_EPI_MUL: r = a * b; break;
+              case PML_HIP_EPI_DIV: r = a / b; break;
+              case PML_HIP_EPI_RDIV: r = b / a; break;
+              case PML_HIP_EPI_MAX: r = (a < b) ? b : a; break;
+              case PML_HIP_EPI_MIN: r = (a < b) ? a : b; break;
+              case PML_HIP_EPI_RELU: r = (a < 0.f) ? 0.f : a; break;
+              case PML_HIP_EPI_NEG: r = -a; break;
+              case PML_HIP_EPI_MAX_GT: r = (a > b) ? a : b; break;
+              default: break;
+            }
+            v[q] = rnd(r);
+          }
+        }
+      }
+      if (bf) {
+        const uint32_t h0 = __float_as_uint(v[0]) >> 16, h1 = __float_as_uint(v[1]) >> 16;
+        const uint32_t h2 = __float_as_uint(v[2]) >> 16, h3 = __float_as_uint(v[3]) >> 16;
+        *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h0 | (h1 << 16), h2 | (h3 << 16));
+      } else {
+        const f32x4_t w = {v[0], v[1], v[2], v[3]};
+        *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
+      }
+    }
+    return;
+  }
+
   for (int row = row0; row < BM; row += RPP) {
     const int64_t m = m0 + row;
     if (m >= p.M) break;

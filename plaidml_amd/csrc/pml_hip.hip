@@ -131,6 +131,30 @@ void classify_tail(const pml_hip_epilogue& t, int out_dtype, int c_dtype, int* m
       (t.n_ops == 1 || (t.ops[1].opcode == PML_HIP_EPI_RELU && t.ops[1].dtype == out_dtype))) {
     *mode = 2;
     *relu = t.n_ops == 2;
+    return;
+  }
+  // up to four float steps in the result type on immediates, scalars and per-column vectors
+  if ((out_dtype == PML_HIP_F32 || out_dtype == PML_HIP_BF16) && t.n_ops >= 1 && t.n_ops <= 4) {
+    bool ok = true;
+    for (int i = 0; i < t.n_ops && ok; ++i) {
+      const pml_hip_epi_op& op = t.ops[i];
+      switch (op.opcode) {
+        case PML_HIP_EPI_ADD: case PML_HIP_EPI_SUB: case PML_HIP_EPI_RSUB: case PML_HIP_EPI_MUL: case PML_HIP_EPI_DIV:
+        case PML_HIP_EPI_RDIV: case PML_HIP_EPI_MAX: case PML_HIP_EPI_MIN: case PML_HIP_EPI_RELU: case PML_HIP_EPI_NEG:
+        case PML_HIP_EPI_MAX_GT:
+          break;
+        default:
+          ok = false;
+      }
+      if (op.dtype != out_dtype) ok = false;
+      if (op.operand_kind == PML_HIP_OPND_TENSOR) {
+        const int q = op.operand;
+        if (t.operand_dtype[q] != out_dtype || t.operand_row_stride[q] != 0 ||
+            (t.operand_col_stride[q] != 0 && t.operand_col_stride[q] != 1))
+          ok = false;
+      }
+    }
+    if (ok) *mode = 3;
   }
 }
 
@@ -368,6 +392,9 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
     g.operands[i] = operands[i];
   }
   if (g.tail_mode == 2 && ((uintptr_t)g.operands[0] & 15) != 0) g.tail_mode = 0;
+  if (g.tail_mode == 3)
+    for (int i = 0; i < d.tail.n_operands; ++i)
+      if (((uintptr_t)g.operands[i] & 15) != 0) g.tail_mode = 0;
   for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
@@ -501,6 +528,9 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     g.operands[i] = operands[i];
   }
   if (g.tail_mode == 2 && ((uintptr_t)g.operands[0] & 15) != 0) g.tail_mode = 0;
+  if (g.tail_mode == 3)
+    for (int i = 0; i < d.tail.n_operands; ++i)
+      if (((uintptr_t)g.operands[i] & 15) != 0) g.tail_mode = 0;
   for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])

@@ -221,6 +221,15 @@ def residual_block(E, op, N=2, H=8, C=64, dtype_name='BFLOAT16'):
     return E.Program('residual', [X], [Z]), [xv], BF16 if dtype_name == 'BFLOAT16' else FP32
 
 
+def resnet50_tiny(E, op):
+    """The full ResNet-50 v1.5 topology (plaidml_amd/resnet50.py) at 1/4 width on 2 x 32x32 images."""
+    from plaidml_amd import resnet50
+    from oracle.tile_oracle import round_bf16
+    prog, _, _ = resnet50.build(E, op, batch=2, image=32, classes=10, dtype_name='BFLOAT16', base=16, round_fn=round_bf16)
+    x = _bf16(_rng(11).uniform(0, 1, (2, 32, 32, 3)).astype(np.float32))
+    return prog, [x], BF16
+
+
 ALL = {
     'dot_f32': dot_f32,
     'gemm_int32': lambda E, op: gemm_int(E, op, 'INT32'),
@@ -242,4 +251,5 @@ ALL = {
     'config3_xception_block_f32': lambda E, op: config3_xception_block(E, op, C=16, dtype_name='FLOAT32'),
     'classifier_tail_f32': classifier_tail,
     'residual_block_bf16': residual_block,
+    'resnet50_tiny_bf16': resnet50_tiny,
 }
