@@ -63,7 +63,9 @@ __device__ inline int xcd_remap(int bid, int nblocks) {
 template <int BM, int BN>
 struct Ring {
   static constexpr int kStage = (BM + BN) * kSlabBytes;                 // A rows then Bt rows
-  static constexpr int kStages = 3 * kStage <= kLdsBytes ? 3 : 2;
+  // 64x64 tiles run two stages: 32 KB of LDS lets five workgroups share a CU, and for this tile
+  // residency hides more latency than a third slab in flight does
+  static constexpr int kStages = (BM * BN <= 64 * 64) ? 2 : (3 * kStage <= kLdsBytes ? 3 : 2);
   static constexpr int kBytes = kStages * kStage;
 };
 

@@ -88,7 +88,7 @@ const char* tile_name(int t) {
 //   gemm 401408x256x64 bf16:        64x64 142, 128x64 166, 128x128 278
 //   gemm 25088x1024x256 bf16:       64x64 51, 128x64 57, 128x128 90
 // One tile per workgroup and a serial load / multiply / store life per tile: what hides latency is
-// how many workgroups fit a CU (64x64: 3, 128x64: 2, larger: 1).  So: long K with enough 256x256
+// how many workgroups fit a CU (64x64: 5, 128x64: 2, larger: 1).  So: long K with enough 256x256
 // tiles to fill the chip takes the big tile (least operand traffic per MFMA); otherwise the smaller
 // of 64x64 and 128x64 by (rounds of resident workgroups) x (tile area), the larger tile on a tie.
 int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
@@ -105,7 +105,7 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
   auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (n <= 64) return TILE_64x64;
   if (k_bytes >= 4096 && tiles(256, 256) >= 128) return TILE_256x256;
-  const int64_t rounds_small = (tiles(64, 64) + 3 * 256 - 1) / (3 * 256);
+  const int64_t rounds_small = (tiles(64, 64) + 5 * 256 - 1) / (5 * 256);
   const int64_t rounds_wide = (tiles(128, 64) + 2 * 256 - 1) / (2 * 256);
   return rounds_small < 2 * rounds_wide ? TILE_64x64 : TILE_128x64;
 }
