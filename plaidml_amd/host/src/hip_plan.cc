@@ -735,6 +735,7 @@ class Planner {
       if (tryConv(i)) return;
       if (tryDepthwise(i)) return;
       if (tryPool(i)) return;
+      if (tryGlobalPool(i)) return;
     }
     emitGeneral(i);
   }
@@ -1162,6 +1163,61 @@ class Planner {
     d->stride_w = sx->stride;
     d->pad_h = sy->pad;
     d->pad_w = sx->pad;
+    return true;
+  }
+
+  // out[n,c] (or out[n,0,0,c]) = agg over all (y,x) of I[n,y,x,c]: a pooling window that is the whole image
+  bool tryGlobalPool(size_t i) {
+    const Op& op = prog_->ops[i];
+    if (op.combo != ComboKind::none || op.operands.size() != 1 || op.init) return false;
+    if (op.agg != AggKind::max && op.agg != AggKind::min && op.agg != AggKind::add) return false;
+    const DataType dt = op.result->shape.elementType;
+    if ((dt != DataType::f32 && dt != DataType::bf16) || op.operands[0]->shape.elementType != dt) return false;
+    const TensorShape &os = op.result->shape, &is = op.operands[0]->shape;
+    if (is.getRank() != 4) return false;
+    const bool keep = os.getRank() == 4;
+    if (!keep && os.getRank() != 2) return false;
+    if (keep && (os.sizes[1] != 1 || os.sizes[2] != 1)) return false;
+    if (os.sizes.front() != is.sizes[0] || os.sizes.back() != is.sizes[3]) return false;
+    Normalised n = normalise(op);
+    for (const auto& c : n.cons)
+      if (!impliedByBox(op, c.lhs, c.rhs)) return false;
+    const int on = n.acc[0].front().plainIndex(), oc = n.acc[0].back().plainIndex();
+    if (on < 0 || oc < 0 || on == oc) return false;
+    if (keep && !(n.acc[0][1].isConstant() && n.acc[0][1].c0 == 0 && n.acc[0][2].isConstant() && n.acc[0][2].c0 == 0)) return false;
+    const int iy = n.acc[1][1].plainIndex(), ix = n.acc[1][2].plainIndex();
+    if (n.acc[1][0].plainIndex() != on || n.acc[1][3].plainIndex() != oc || iy < 0 || ix < 0 || iy == ix || iy == on ||
+        iy == oc || ix == on || ix == oc)
+      return false;
+    const int idx[4] = {on, iy, ix, oc};
+    for (int k = 0; k < 4; ++k)
+      if (op.lower[idx[k]] != 0 || op.upper[idx[k]] != is.sizes[k] - 1) return false;
+    for (size_t v = 0; v < n.nIdx; ++v)
+      if (n.active[v] && static_cast<int>(v) != on && static_cast<int>(v) != oc && static_cast<int>(v) != iy &&
+          static_cast<int>(v) != ix)
+        return false;
+    const int V = 16 / static_cast<int>(util::byteSize(dt));
+    if (is.sizes[3] % V != 0) return false;
+    Step s;
+    s.kind = Step::Pool2d;
+    pml_hip_pool2d_desc& d = s.pool;
+    d.dtype = hipType(dt);
+    d.agg = hipAgg(op.agg);
+    d.n = is.sizes[0];
+    d.h = is.sizes[1];
+    d.w = is.sizes[2];
+    d.c = is.sizes[3];
+    d.kh = d.h;
+    d.kw = d.w;
+    d.oh = d.ow = 1;
+    d.stride_h = d.stride_w = 1;
+    d.pad_h = d.pad_w = 0;
+    s.a = bufferFor(op.operands[0]);
+    s.c = bufferFor(op.result);
+    s.bytes = static_cast<double>(is.elements() + os.elements()) * util::byteSize(dt);
+    s.text = "pool2d " + tile::toString(op.agg) + " " + std::string(util::mnemonic(dt)) + " " + is.str() +
+             " over the whole image -> " + os.str();
+    plan_->steps.push_back(s);
     return true;
   }
 
