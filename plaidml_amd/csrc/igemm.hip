@@ -184,6 +184,10 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
     }
   };
 
+  // a residual tensor of the tail is requested now, so that it arrives under the K loop
+  TailPrefetch<KIND, BM, BN, kThreads> pre;
+  tail_prefetch<KIND, BM, BN, kThreads>(p, m0, n0, tid, pre);
+
   acc_t acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -275,7 +279,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
           *(acc4_t*)&ctile[(wm * WM + i * 32 + crow) * CS + wn * WN + j * 32 + 8 * g + ccol] = q;
         }
     __syncthreads();
-    tile_tail<KIND, BM, BN, kThreads>(p, ctile, m0, n0, tid);
+    tile_tail<KIND, BM, BN, kThreads>(p, ctile, m0, n0, tid, &pre);
   } else {
     // large tiles: every wavefront stages RB of its 32-row blocks at a time in a private
     // region, wtile[RB * 32][WN + 4], and runs the tail over them with its 64 lanes

@@ -50,13 +50,54 @@ __device__ inline void mma_block<KIND_F32>(f32x16_t& acc, const i32x4_t& a, cons
   }
 }
 
+// Residual rows of a tile requested ahead of its K loop (tail_mode 2, at most 8 rows per thread):
+// their latency then overlaps the operand loads and the MFMAs instead of following them.
+template <int KIND, int BM, int BN, int NTHREADS>
+struct TailPrefetch {
+  static constexpr int TPR = BN / 4;
+  static constexpr int RPP = NTHREADS / TPR;
+  static constexpr int kIters = (BM + RPP - 1) / RPP;
+  static constexpr bool kFits = kIters <= 8;
+  i32x4_t res[kFits ? kIters : 1];
+  bool valid;
+};
+
+template <int KIND, int BM, int BN, int NTHREADS>
+__device__ __forceinline__ void tail_prefetch(const IgemmArgs& p, int64_t m0, int64_t n0, int tid,
+                                              TailPrefetch<KIND, BM, BN, NTHREADS>& pre) {
+  typedef TailPrefetch<KIND, BM, BN, NTHREADS> P;
+  pre.valid = false;
+  if constexpr (P::kFits) {
+    const int64_t n = n0 + (tid % P::TPR) * 4;
+    if (p.tail_mode != 2 || n + 3 >= p.N || (p.ldc & 3) != 0) return;
+    pre.valid = true;
+    const int64_t res_rs = p.tail.operand_row_stride[0];
+#pragma unroll
+    for (int c = 0; c < P::kIters; ++c) {
+      const int row = tid / P::TPR + c * P::RPP;
+      const int64_t m = m0 + row;
+      pre.res[c] = i32x4_t{0, 0, 0, 0};
+      if (row < BM && m < p.M) {
+        if (KIND != KIND_I8 && p.out_dtype == PML_HIP_BF16) {
+          const uint2 x = *(const uint2*)((const uint16_t*)p.operands[0] + m * res_rs + n);
+          pre.res[c][0] = (int)x.x;
+          pre.res[c][1] = (int)x.y;
+        } else {
+          pre.res[c] = *(const i32x4_t*)((const int*)p.operands[0] + m * res_rs + n);
+        }
+      }
+    }
+  }
+}
+
 // Tail over an accumulator tile held in LDS as ctile[BM][BN + 4] (row-major):
 // adds the initial value, runs the fused elementwise chain once per element and
 // stores contiguous 8/16-byte pieces.  A thread owns 4 consecutive columns; rows
 // advance by NTHREADS / (BN / 4) per pass.
 template <int KIND, int BM, int BN, int NTHREADS>
 __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc<KIND>::scalar* ctile, int64_t m0,
-                                          int64_t n0, int tid) {
+                                          int64_t n0, int tid,
+                                          const TailPrefetch<KIND, BM, BN, NTHREADS>* pre = nullptr) {
   typedef typename Acc<KIND>::scalar accs_t;
   constexpr int CS = BN + 4;
   constexpr int kThreads = NTHREADS;
@@ -117,7 +158,9 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
         const int row = row0 + (it0 + c) * RPP;
         const int64_t m = m0 + row;
         res[c] = i32x4_t{0, 0, 0, 0};
-        if (residual && row < BM && m < p.M) {
+        if (TailPrefetch<KIND, BM, BN, NTHREADS>::kFits && pre != nullptr && pre->valid) {
+          res[c] = pre->res[(it0 + c) % (TailPrefetch<KIND, BM, BN, NTHREADS>::kFits ? kIters : 1)];
+        } else if (residual && row < BM && m < p.M) {
           if (KIND != KIND_I8 && p.out_dtype == PML_HIP_BF16) {
             const uint2 x = *(const uint2*)((const uint16_t*)p.operands[0] + m * res_rs + n);
             res[c][0] = (int)x.x;
