@@ -34,6 +34,7 @@ struct IgemmArgs {
   // halo_variant: 0 = general resident kernel, 1 / 2 = pipelined 3x3 kernel with that many 32-pixel chunks per row
   // b_raw: Bt points at the caller's [K][N] matrix instead of the packed [N][K] one (pipelined kernel only)
   int NB, halo_rows, n_tiles, halo_variant, b_raw;
+  int n_cus;  // compute units of the device (persistent grids)
   // n / (OH*OW) and n / OW as multiply-and-shift (see fast_div)
   unsigned div_per_magic, div_ow_magic;
   int div_per_shift, div_ow_shift;

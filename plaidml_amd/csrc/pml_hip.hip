@@ -171,6 +171,18 @@ bool valid_tail(const pml_hip_epilogue& t) {
   return true;
 }
 
+// Compute units of the current device (persistent kernels size their grids by it).
+int device_cus() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    hipDeviceProp_t prop;
+    cached[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess ? prop.multiProcessorCount : 256;
+  }
+  return cached[dev];
+}
+
 // Everything of the kernel arguments that the descriptor fixes (no operand pointers).
 void conv_args(const Plan* p, IgemmArgs& g) {
   const pml_hip_conv2d_desc& d = p->conv;
@@ -206,6 +218,7 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
   g.tail = d.tail;
   g.NB = (int)d.n;
+  g.n_cus = device_cus();
   g.halo_rows = p->halo_rows;
   g.n_tiles = p->halo_tiles;
   g.halo_variant = p->halo_variant;
@@ -385,6 +398,7 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   g.init_rs = d.init_row_stride;
   g.init_cs = d.init_col_stride;
   g.c_dtype = d.c_dtype;
+  g.n_cus = device_cus();
   classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
   g.tail = d.tail;
   for (int i = 0; i < d.tail.n_operands; ++i) {
