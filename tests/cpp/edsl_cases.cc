@@ -1,0 +1,240 @@
+// C++ programs written against include/plaidml/* exactly as a user of the reference would write them,
+// linked to libplaidml.so and run on the hip device.  Cases and expected values follow the
+// reference's own tests (plaidml/edsl/tests/edsl_test.cc: Dot :48-54 / :1203-1252, Max :576-590,
+// EltwiseAdd :1181-1201, FunkySum :2709-2719, UseDefault :1148-1164, ArgMax :2126-2137 pattern,
+// DotF16_AccF32 pattern :509-545 with int8 -> int32; plaidml/edsl/examples/gemm.cc:66-77).
+// Prints "ok <case>" per passing case; exits 1 on the first failure.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "plaidml/edsl/edsl.h"
+#include "plaidml/exec/exec.h"
+#include "plaidml/op/op.h"
+
+using namespace plaidml;        // NOLINT
+using namespace plaidml::edsl;  // NOLINT
+
+namespace {
+
+template <typename T>
+Buffer makeBuffer(DType dt, const std::vector<int64_t>& dims, const std::vector<T>& data) {
+  Buffer b(TensorShape(dt, dims));
+  b.copy_from(data.data());
+  return b;
+}
+
+template <typename T>
+std::vector<T> readBuffer(Buffer& b) {
+  std::vector<T> out(b.size() / sizeof(T));
+  b.copy_into(out.data());
+  return out;
+}
+
+[[noreturn]] void fail(const std::string& name, const std::string& what) {
+  std::fprintf(stderr, "FAILED %s: %s\n", name.c_str(), what.c_str());
+  std::exit(1);
+}
+
+template <typename T>
+void expectEq(const std::string& name, const std::vector<T>& got, const std::vector<T>& want) {
+  if (got.size() != want.size()) fail(name, "size mismatch");
+  for (size_t i = 0; i < got.size(); ++i)
+    if (got[i] != want[i]) fail(name, "element " + std::to_string(i) + ": got " + std::to_string(got[i]) + " want " + std::to_string(want[i]));
+  std::printf("ok %s\n", name.c_str());
+}
+
+void expectClose(const std::string& name, const std::vector<float>& got, const std::vector<float>& want, float rtol, float atol) {
+  if (got.size() != want.size()) fail(name, "size mismatch");
+  for (size_t i = 0; i < got.size(); ++i)
+    if (std::fabs(got[i] - want[i]) > atol + rtol * std::fabs(want[i]))
+      fail(name, "element " + std::to_string(i) + ": got " + std::to_string(got[i]) + " want " + std::to_string(want[i]));
+  std::printf("ok %s\n", name.c_str());
+}
+
+std::vector<Buffer> run(const Program& program_in, std::vector<Buffer> inputs) {
+  Program program = program_in;
+  program.compile();
+  exec::Executable exe(program);
+  std::vector<Buffer> outputs;
+  for (const TensorShape& shape : program.outputs()) outputs.emplace_back(shape);
+  exe.run(inputs, outputs);
+  return outputs;
+}
+
+Tensor Dot(const Tensor& A, const Tensor& B) {
+  TensorDim I, J, K;
+  TensorIndex i, j, k;
+  A.bind_dims(I, K);
+  B.bind_dims(K, J);
+  return Contraction().outShape(I, J).outAccess(i, j).sum(A(i, k) * B(k, j));
+}
+
+void caseDot() {
+  const int64_t M = 8, N = 32, K = 16;
+  auto A = Placeholder(DType::FLOAT32, {M, K});
+  auto B = Placeholder(DType::FLOAT32, {K, N});
+  auto program = buildProgram("dot", {A, B}, {Dot(A, B)});
+  std::default_random_engine rng(2);
+  std::normal_distribution<float> dist(0.0, 1.0);
+  std::vector<float> a(M * K), b(K * N), want(M * N, 0.f);
+  for (auto& x : a) x = dist(rng);
+  for (auto& x : b) x = dist(rng);
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t j = 0; j < N; ++j)
+      for (int64_t k = 0; k < K; ++k) want[i * N + j] += a[i * K + k] * b[k * N + j];
+  auto out = run(program, {makeBuffer(DType::FLOAT32, {M, K}, a), makeBuffer(DType::FLOAT32, {K, N}, b)});
+  expectClose("dot_f32", readBuffer<float>(out[0]), want, 1e-3f, 1e-4f);
+}
+
+void caseMax() {
+  auto I = Placeholder(DType::FLOAT32, {3, 3});
+  TensorDim M, N;
+  TensorIndex m, n;
+  I.bind_dims(M, N);
+  Tensor O = Contraction().outShape(M).outAccess(m).max(I(m, n));
+  auto program = buildProgram("max", {I}, {O});
+  std::vector<float> in = {-5.0f, -6.0f, -7.0f, 4.0f, 5.0f, 6.0f, 7.0f, 8.0f, 9.0f};
+  auto out = run(program, {makeBuffer(DType::FLOAT32, {3, 3}, in)});
+  expectEq<float>("max_rows", readBuffer<float>(out[0]), {-5.0f, 6.0f, 9.0f});
+}
+
+void caseEltwiseAdd() {
+  auto A = Placeholder(DType::FLOAT32, {10, 20});
+  auto B = Placeholder(DType::FLOAT32, {10, 20});
+  auto program = buildProgram("eltwise_add", {A, B}, {A + B});
+  std::vector<float> a(200), b(200), want(200);
+  for (int i = 0; i < 200; ++i) {
+    a[i] = 0.25f * i;
+    b[i] = 100.f - i;
+    want[i] = a[i] + b[i];
+  }
+  auto out = run(program, {makeBuffer(DType::FLOAT32, {10, 20}, a), makeBuffer(DType::FLOAT32, {10, 20}, b)});
+  expectEq<float>("eltwise_add", readBuffer<float>(out[0]), want);
+}
+
+void caseFunkySum() {
+  // O[i] += I[(i - j + 1) / 2] * K[j] on I = K = [1, 2, 3], five outputs  ->  [2, 5, 4, 9, 6]
+  auto I = Placeholder(DType::FLOAT32, {3});
+  auto Kt = Placeholder(DType::FLOAT32, {3});
+  TensorIndex i, j;
+  Tensor O = Contraction().outShape(5).outAccess(i).sum(I((i - j + 1) / 2) * Kt(j));
+  auto program = buildProgram("funky_sum", {I, Kt}, {O});
+  auto out = run(program, {makeBuffer<float>(DType::FLOAT32, {3}, {1, 2, 3}), makeBuffer<float>(DType::FLOAT32, {3}, {1, 2, 3})});
+  expectEq<float>("funky_sum", readBuffer<float>(out[0]), {2, 5, 4, 9, 6});
+}
+
+void caseUseDefault() {
+  // O[b, 3, i1, i2] = I[b, i1, i2] over a default tensor P
+  auto P = Placeholder(DType::FLOAT32, {1, 7, 10, 10});
+  auto I = Placeholder(DType::FLOAT32, {1, 10, 10});
+  TensorDim B, N1, N2;
+  TensorIndex b, i1, i2;
+  I.bind_dims(B, N1, N2);
+  Tensor O = Contraction().outShape(B, 7, N1, N2).outAccess(b, 3, i1, i2).assign(I(b, i1, i2)).init(P);
+  auto program = buildProgram("use_default", {I, P}, {O});
+  std::vector<float> p(700), in(100), want(700);
+  for (int k = 0; k < 700; ++k) want[k] = p[k] = 0.5f * k;
+  for (int k = 0; k < 100; ++k) want[300 + k] = in[k] = -1.f - k;
+  auto out = run(program, {makeBuffer(DType::FLOAT32, {1, 10, 10}, in), makeBuffer(DType::FLOAT32, {1, 7, 10, 10}, p)});
+  expectEq<float>("use_default", readBuffer<float>(out[0]), want);
+}
+
+void caseInt8Gemm() {
+  // int8 x int8 accumulated in int32: the cast comes before the contraction
+  const int64_t M = 64, N = 48, K = 32;
+  auto A = Placeholder(DType::INT8, {M, K});
+  auto B = Placeholder(DType::INT8, {K, N});
+  auto program = buildProgram("gemm_i8", {A, B}, {Dot(cast(A, DType::INT32), cast(B, DType::INT32))});
+  std::default_random_engine rng(4);
+  std::uniform_int_distribution<int> dist(-127, 127);
+  std::vector<int8_t> a(M * K), b(K * N);
+  std::vector<int32_t> want(M * N, 0);
+  for (auto& x : a) x = static_cast<int8_t>(dist(rng));
+  for (auto& x : b) x = static_cast<int8_t>(dist(rng));
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t j = 0; j < N; ++j)
+      for (int64_t k = 0; k < K; ++k) want[i * N + j] += static_cast<int32_t>(a[i * K + k]) * b[k * N + j];
+  auto out = run(program, {makeBuffer(DType::INT8, {M, K}, a), makeBuffer(DType::INT8, {K, N}, b)});
+  expectEq<int32_t>("gemm_i8_i32", readBuffer<int32_t>(out[0]), want);
+}
+
+void caseConvRelu() {
+  // op::relu(op::convolution(I, F) + B): NXC / XCK / SAME_UPPER / stride 1 defaults
+  const int64_t N = 2, H = 9, W = 11, CI = 32, CO = 48;
+  auto I = Placeholder(DType::FLOAT32, {N, H, W, CI});
+  auto F = Placeholder(DType::FLOAT32, {3, 3, CI, CO});
+  auto Bv = Placeholder(DType::FLOAT32, {CO});
+  Tensor O = op::relu(op::convolution(I, F) + Bv);
+  auto program = buildProgram("conv_relu", {I, F, Bv}, {O});
+  std::default_random_engine rng(7);
+  std::normal_distribution<float> dist(0.0, 1.0);
+  std::vector<float> in(N * H * W * CI), f(9 * CI * CO), bias(CO), want(N * H * W * CO);
+  for (auto& x : in) x = dist(rng);
+  for (auto& x : f) x = 0.1f * dist(rng);
+  for (auto& x : bias) x = dist(rng);
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t y = 0; y < H; ++y)
+      for (int64_t x = 0; x < W; ++x)
+        for (int64_t co = 0; co < CO; ++co) {
+          double acc = bias[co];
+          for (int64_t ky = 0; ky < 3; ++ky)
+            for (int64_t kx = 0; kx < 3; ++kx) {
+              const int64_t iy = y + ky - 1, ix = x + kx - 1;
+              if (iy < 0 || iy >= H || ix < 0 || ix >= W) continue;
+              for (int64_t ci = 0; ci < CI; ++ci)
+                acc += static_cast<double>(in[((n * H + iy) * W + ix) * CI + ci]) * f[((ky * 3 + kx) * CI + ci) * CO + co];
+            }
+          want[((n * H + y) * W + x) * CO + co] = acc < 0 ? 0.f : static_cast<float>(acc);
+        }
+  auto out = run(program, {makeBuffer(DType::FLOAT32, {N, H, W, CI}, in), makeBuffer(DType::FLOAT32, {3, 3, CI, CO}, f),
+                           makeBuffer(DType::FLOAT32, {CO}, bias)});
+  expectClose("conv_bias_relu", readBuffer<float>(out[0]), want, 1e-3f, 1e-4f);
+}
+
+void caseErrors() {
+  auto A = Placeholder(DType::FLOAT32, {4, 4});
+  auto program = buildProgram("ident", {A}, {A + 1.0});
+  program.compile();
+  exec::Executable exe(program);
+  Buffer out(TensorShape(DType::FLOAT32, {4, 4}));
+  try {
+    exe.run({}, {out});
+  } catch (const std::exception& e) {
+    if (std::string(e.what()).find("Program expects 1 inputs, but 0 were specified") == std::string::npos)
+      fail("arity_error", std::string("unexpected text: ") + e.what());
+    std::printf("ok arity_error\n");
+    return;
+  }
+  fail("arity_error", "no exception");
+}
+
+}  // namespace
+
+int main() {
+  plaidml::init();
+  plaidml::edsl::init();
+  plaidml::op::init();
+  plaidml::exec::init();
+  Settings::set("PLAIDML_DEVICE", "hip.0");
+  Settings::set("PLAIDML_TARGET", "hip");
+  try {
+    caseDot();
+    caseMax();
+    caseEltwiseAdd();
+    caseFunkySum();
+    caseUseDefault();
+    caseInt8Gemm();
+    caseConvRelu();
+    caseErrors();
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "FAILED with exception: %s\n", e.what());
+    return 1;
+  }
+  std::printf("all cases passed\n");
+  return 0;
+}

@@ -110,3 +110,17 @@ def test_run_without_a_device_fails_loudly():
         E.Executable(prog)
     with pytest.raises(E.PlaidMLError, match='Invalid device name'):
         E.Executable(prog, 'not a device')
+
+
+def test_cpp_cases_fail_loudly_without_a_device():
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'cpp', 'edsl_cases')
+    if not os.path.exists(exe):
+        pytest.skip('tests/cpp/edsl_cases is built by __graft_entry__.build()')
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip('a GPU is present')
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0
+    assert 'hip' in res.stderr.lower()

@@ -60,3 +60,15 @@ def test_run_checks_arity_and_shapes():
         exe.run([bad, b], [o])
     assert exe.run([a, b], [o]) >= 0.0
     assert 'hip.0' in E.list_devices()
+
+
+def test_cpp_header_api_cases():
+    """User C++ against include/plaidml/* (tests/cpp/edsl_cases.cc, built by __graft_entry__.build) on the hip device."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'cpp', 'edsl_cases')
+    assert os.path.exists(exe), 'run __graft_entry__.build() first'
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(res.stdout, res.stderr, flush=True)
+    assert res.returncode == 0, res.stderr
+    assert 'all cases passed' in res.stdout
