@@ -311,6 +311,130 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
     return;
   }
 
+  // tail_mode 4 (int32 accumulators): up to eight steps that store the running value to an extra
+  // output, cast between si32 / f32 / si8, or are f32 arithmetic on immediates, scalars and per-column
+  // vectors -- the requantisation chain  store, cast f32, * scale[col], clamp, round, cast si8.
+  // Four columns at a time, 4 / 16-byte stores; the step semantics are the interpreter's.
+  if (KIND == KIND_I8 && p.tail_mode == 4 && full4 && (p.ldc & 3) == 0) {
+    float xs[8][4];
+#pragma unroll
+    for (int st = 0; st < 8; ++st) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xs[st][q] = 0.f;
+      if (st < p.tail.n_ops) {
+        const pml_hip_epi_op& op = p.tail.ops[st];
+        if (op.opcode != PML_HIP_EPI_STORE && op.opcode != PML_HIP_EPI_CAST) {
+          if (op.operand_kind == PML_HIP_OPND_TENSOR) {
+            const float* base = (const float*)p.operands[op.operand];
+            if (p.tail.operand_col_stride[op.operand] == 0) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) xs[st][q] = base[0];
+            } else {
+              const f32x4_t w = *(const f32x4_t*)(base + n);
+#pragma unroll
+              for (int q = 0; q < 4; ++q) xs[st][q] = w[q];
+            }
+          } else if (op.operand_kind == PML_HIP_OPND_IMM) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xs[st][q] = (float)op.imm;
+          }
+        }
+      }
+    }
+    // rows in batches of kRows, so that decoding a step is paid once per batch
+    constexpr int kIters = (BM + RPP - 1) / RPP;
+    constexpr int kRows = kIters < 4 ? kIters : 4;
+    for (int it0 = 0; it0 < kIters; it0 += kRows) {
+      int vi[kRows][4];
+      float vf[kRows][4];
+      bool live[kRows];
+#pragma unroll
+      for (int c = 0; c < kRows; ++c) {
+        const int row = row0 + (it0 + c) * RPP;
+        const int64_t m = m0 + row;
+        live[c] = row < BM && m < p.M;
+        const int rr = live[c] ? row : row0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          vi[c][q] = (int)ctile[rr * CS + c4 + q] + (int)cinit[q];
+          vf[c][q] = 0.f;
+        }
+        if (live[c] && p.init && !col_init) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            Scalar<float, int> bb = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
+            vi[c][q] = (int)((unsigned)vi[c][q] + (unsigned)bb.i);
+          }
+        }
+      }
+      int cur = PML_HIP_I32;
+      auto store4 = [&](void* dst, int c) {
+        const int64_t o = (m0 + row0 + (it0 + c) * RPP) * p.ldc + n;
+        if (cur == PML_HIP_F32) {
+          *(f32x4_t*)((float*)dst + o) = f32x4_t{vf[c][0], vf[c][1], vf[c][2], vf[c][3]};
+        } else if (cur == PML_HIP_I32) {
+          *(i32x4_t*)((int*)dst + o) = i32x4_t{vi[c][0], vi[c][1], vi[c][2], vi[c][3]};
+        } else {
+          *(uint32_t*)((uint8_t*)dst + o) = (uint32_t)(vi[c][0] & 255) | ((uint32_t)(vi[c][1] & 255) << 8) |
+                                            ((uint32_t)(vi[c][2] & 255) << 16) | ((uint32_t)(vi[c][3] & 255) << 24);
+        }
+      };
+#pragma unroll
+      for (int st = 0; st < 8; ++st) {
+        if (st < p.tail.n_ops) {
+          const pml_hip_epi_op& op = p.tail.ops[st];
+          if (op.opcode == PML_HIP_EPI_STORE) {
+#pragma unroll
+            for (int c = 0; c < kRows; ++c)
+              if (live[c]) store4(p.outs[op.operand], c);
+          } else if (op.opcode == PML_HIP_EPI_CAST) {
+#pragma unroll
+            for (int c = 0; c < kRows; ++c)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                if (op.dtype == PML_HIP_F32) {
+                  if (cur != PML_HIP_F32) vf[c][q] = (float)vi[c][q];
+                } else {
+                  int t = cur == PML_HIP_F32 ? (int)vf[c][q] : vi[c][q];
+                  if (op.dtype == PML_HIP_I8) t = (int)(signed char)t;
+                  vi[c][q] = t;
+                }
+              }
+            cur = op.dtype;
+          } else {
+            auto each = [&](auto fn) {
+#pragma unroll
+              for (int c = 0; c < kRows; ++c)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) vf[c][q] = fn(vf[c][q], xs[st][q]);
+            };
+            switch (op.opcode) {
+              case PML_HIP_EPI_ADD: each([](float a, float b) { return a + b; }); break;
+              case PML_HIP_EPI_SUB: each([](float a, float b) { return a - b; }); break;
+              case PML_HIP_EPI_RSUB: each([](float a, float b) { return b - a; }); break;
+              case PML_HIP_EPI_MUL: each([](float a, float b) { return a * b; }); break;
+              case PML_HIP_EPI_DIV: each([](float a, float b) { return a / b; }); break;
+              case PML_HIP_EPI_RDIV: each([](float a, float b) { return b / a; }); break;
+              case PML_HIP_EPI_MAX: each([](float a, float b) { return (a < b) ? b : a; }); break;
+              case PML_HIP_EPI_MIN: each([](float a, float b) { return (a < b) ? a : b; }); break;
+              case PML_HIP_EPI_RELU: each([](float a, float) { return (a < 0.f) ? 0.f : a; }); break;
+              case PML_HIP_EPI_NEG: each([](float a, float) { return -a; }); break;
+              case PML_HIP_EPI_MAX_GT: each([](float a, float b) { return (a > b) ? a : b; }); break;
+              case PML_HIP_EPI_ROUND: each([](float a, float) { return c_round<float>(a); }); break;
+              case PML_HIP_EPI_FLOOR: each([](float a, float) { return floorf(a); }); break;
+              case PML_HIP_EPI_CEIL: each([](float a, float) { return ceilf(a); }); break;
+              default: break;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < kRows; ++c)
+        if (live[c]) store4(p.C, c);
+    }
+    return;
+  }
+
   for (int row = row0; row < BM; row += RPP) {
     const int64_t m = m0 + row;
     if (m >= p.M) break;

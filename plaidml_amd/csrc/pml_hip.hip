@@ -114,6 +114,44 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
 void classify_tail(const pml_hip_epilogue& t, int out_dtype, int c_dtype, int* mode, int* relu) {
   *mode = 0;
   *relu = 0;
+  // int32 accumulators followed by stores / casts between si32, f32, si8 / f32 arithmetic on immediates,
+  // scalars and per-column vectors (requantisation): checked by walking the element type through the chain
+  if (out_dtype == PML_HIP_I32 && t.n_ops >= 1 && t.n_ops <= 8) {
+    int cur = PML_HIP_I32;
+    bool ok = true;
+    for (int i = 0; i < t.n_ops && ok; ++i) {
+      const pml_hip_epi_op& op = t.ops[i];
+      if (op.opcode == PML_HIP_EPI_STORE) continue;
+      if (op.opcode == PML_HIP_EPI_CAST) {
+        if (op.dtype != PML_HIP_F32 && op.dtype != PML_HIP_I32 && op.dtype != PML_HIP_I8) ok = false;
+        if (cur == PML_HIP_I8 && op.dtype != PML_HIP_I8) ok = false;  // si8 is only ever the last type
+        cur = op.dtype;
+        continue;
+      }
+      switch (op.opcode) {
+        case PML_HIP_EPI_ADD: case PML_HIP_EPI_SUB: case PML_HIP_EPI_RSUB: case PML_HIP_EPI_MUL: case PML_HIP_EPI_DIV:
+        case PML_HIP_EPI_RDIV: case PML_HIP_EPI_MAX: case PML_HIP_EPI_MIN: case PML_HIP_EPI_RELU: case PML_HIP_EPI_NEG:
+        case PML_HIP_EPI_MAX_GT: case PML_HIP_EPI_ROUND: case PML_HIP_EPI_FLOOR: case PML_HIP_EPI_CEIL:
+          break;
+        default:
+          ok = false;
+      }
+      if (cur != PML_HIP_F32 || op.dtype != PML_HIP_F32) ok = false;
+      if (op.operand_kind == PML_HIP_OPND_TENSOR) {
+        const int q = op.operand;
+        if (t.operand_dtype[q] != PML_HIP_F32 || t.operand_row_stride[q] != 0 ||
+            (t.operand_col_stride[q] != 0 && t.operand_col_stride[q] != 1))
+          ok = false;
+      }
+    }
+    bool plain = true;  // a chain of nothing but "relu" on si32 stays with mode 1 below
+    for (int i = 0; i < t.n_ops; ++i)
+      if (t.ops[i].opcode != PML_HIP_EPI_RELU) plain = false;
+    if (ok && !plain && cur == c_dtype) {
+      *mode = 4;
+      return;
+    }
+  }
   if (c_dtype != out_dtype) return;
   if (t.n_ops == 0) {
     *mode = 1;
@@ -405,11 +443,15 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
     if (!operands || !operands[i]) return fail("gemm_invoke: missing tail operand");
     g.operands[i] = operands[i];
   }
+  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
+  // the vector tails need 16-byte aligned operands and extra outputs; otherwise the interpreter runs
   if (g.tail_mode == 2 && ((uintptr_t)g.operands[0] & 15) != 0) g.tail_mode = 0;
-  if (g.tail_mode == 3)
+  if (g.tail_mode == 3 || g.tail_mode == 4) {
     for (int i = 0; i < d.tail.n_operands; ++i)
       if (((uintptr_t)g.operands[i] & 15) != 0) g.tail_mode = 0;
-  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
+    for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i)
+      if (((uintptr_t)g.outs[i] & 15) != 0) g.tail_mode = 0;
+  }
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("gemm_invoke: missing extra output");
@@ -541,11 +583,15 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     if (!operands || !operands[i]) return fail("conv2d_invoke: missing tail operand");
     g.operands[i] = operands[i];
   }
+  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
+  // the vector tails need 16-byte aligned operands and extra outputs; otherwise the interpreter runs
   if (g.tail_mode == 2 && ((uintptr_t)g.operands[0] & 15) != 0) g.tail_mode = 0;
-  if (g.tail_mode == 3)
+  if (g.tail_mode == 3 || g.tail_mode == 4) {
     for (int i = 0; i < d.tail.n_operands; ++i)
       if (((uintptr_t)g.operands[i] & 15) != 0) g.tail_mode = 0;
-  for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) g.outs[i] = outs ? outs[i] : nullptr;
+    for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i)
+      if (((uintptr_t)g.outs[i] & 15) != 0) g.tail_mode = 0;
+  }
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("conv2d_invoke: missing extra output");

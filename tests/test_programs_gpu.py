@@ -46,6 +46,28 @@ def test_program_matches_oracle(name, target):
     check(name, got, ref, tol)
 
 
+def test_config2_full_size_properties():
+    """BASELINE configs[2] at full size through the plaidml API: int8 4096^3 -> int32 (bit-exact by a checksum of
+    checksums: row sums of C against A . rowsum(B) in int64) and the per-column requantised int8 output (exact
+    elementwise restatement of the Tile program on the GPU's own C)."""
+    prog, vals, _ = programs.config2_int8_gemm(E, op, 4096, 4096, 4096)
+    runner = E.Runner(prog, target='hip')
+    C, Q = runner.run(vals)
+    A, B, S = vals
+    assert C.dtype == np.int32 and Q.dtype == np.int8
+    np.testing.assert_array_equal(C.astype(np.int64).sum(axis=1), A.astype(np.int64) @ B.astype(np.int64).sum(axis=1))
+    np.testing.assert_array_equal(C.astype(np.int64).sum(axis=0), A.astype(np.int64).sum(axis=0) @ B.astype(np.int64))
+    cols = [0, 1, 777, 4095]
+    np.testing.assert_array_equal(C[:, cols], (A.astype(np.int32) @ B[:, cols].astype(np.int32)))
+    x = C.astype(np.float32) * S[None, :]
+    x = np.where(x > np.float32(-127.0), x, np.float32(-127.0))   # op::clip: select(O > min, O, min), then select(O < max, O, max)
+    x = np.where(x < np.float32(127.0), x, np.float32(127.0))
+    q = (np.sign(x) * np.floor(np.abs(x) + np.float32(0.5))).astype(np.int8)   # C roundf: half away from zero
+    np.testing.assert_array_equal(Q, q)
+    runner.run(vals)
+    print('configs[2] run stats (second run)', E.last_run_stats(), flush=True)
+
+
 def test_run_checks_arity_and_shapes():
     prog, vals, _ = programs.dot_f32(E, op)
     prog.compile()
