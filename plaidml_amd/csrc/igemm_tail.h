@@ -194,20 +194,36 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
           }
           *(i32x4_t*)((int*)p.C + m * p.ldc + n) = w;
         } else if (p.out_dtype == PML_HIP_BF16) {
-          uint32_t h[4];
+          // v_cvt_pk_bf16_f32 rounds to nearest even.  relu is applied to the fp32 value just before
+          // the last rounding (a result in (-2^-134, 0) stores +0 where the definition gives -0).
+          typedef float f32x2 __attribute__((ext_vector_type(2)));
+          typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+          float v[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            h[q] = f32_to_bf16_bits((float)v4[q]);
-            if (residual) {
-              // the contraction result is rounded first, then the bf16 addition rounds again
-              const uint32_t xw = (uint32_t)res[c][q >> 1];
-              const float xf = __uint_as_float((q & 1) ? (xw & 0xffff0000u) : (xw << 16));
-              h[q] = f32_to_bf16_bits(__uint_as_float(h[q] << 16) + xf);
-            }
-            // relu on the rounded value: negative, non-NaN, non-zero -> 0  (x < 0 ? 0 : x)
-            if (p.tail_relu && (h[q] & 0x8000u) && (h[q] & 0x7fffu) <= 0x7f80u && (h[q] & 0x7fffu) != 0) h[q] = 0;
+          for (int q = 0; q < 4; ++q) v[q] = (float)v4[q];
+          if (residual) {
+            // the contraction result is rounded first, then the bf16 addition rounds again
+            const bf16x2 r01 = __builtin_convertvector(f32x2{v[0], v[1]}, bf16x2);
+            const bf16x2 r23 = __builtin_convertvector(f32x2{v[2], v[3]}, bf16x2);
+            uint32_t w01, w23;
+            __builtin_memcpy(&w01, &r01, 4);
+            __builtin_memcpy(&w23, &r23, 4);
+            const uint32_t x01 = (uint32_t)res[c][0], x23 = (uint32_t)res[c][1];
+            v[0] = __uint_as_float(w01 << 16) + __uint_as_float(x01 << 16);
+            v[1] = __uint_as_float(w01 & 0xffff0000u) + __uint_as_float(x01 & 0xffff0000u);
+            v[2] = __uint_as_float(w23 << 16) + __uint_as_float(x23 << 16);
+            v[3] = __uint_as_float(w23 & 0xffff0000u) + __uint_as_float(x23 & 0xffff0000u);
           }
-          *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+          if (p.tail_relu) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = v[q] < 0.f ? 0.f : v[q];
+          }
+          const bf16x2 h01 = __builtin_convertvector(f32x2{v[0], v[1]}, bf16x2);
+          const bf16x2 h23 = __builtin_convertvector(f32x2{v[2], v[3]}, bf16x2);
+          uint32_t o01, o23;
+          __builtin_memcpy(&o01, &h01, 4);
+          __builtin_memcpy(&o23, &h23, 4);
+          *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(o01, o23);
         } else {
           f32x4_t w;
 #pragma unroll
