@@ -123,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
       const int64_t nb = t / p.OH;
       a_ih0[i] = oh * p.SH - p.PH;
       a_iw0[i] = ow * p.SW - p.PW;
-      a_off[i] = ok ? (unsigned)(nb * ((int64_t)p.H * p.W * p.CI * ES)) : kOutside;
+      a_off[i] = ok ? (unsigned)(nb * ((int64_t)p.H * p.W * (p.pix_pitch ? p.pix_pitch : p.CI * ES))) : kOutside;
     } else {
       a_ih0[i] = a_iw0[i] = 0;
       a_off[i] = ok ? (unsigned)(mm * p.lda * ES) : kOutside;
@@ -138,7 +138,8 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
 
   const int slabs_per_tap = (kbytes_row + kSlabBytes - 1) / kSlabBytes;
   const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : slabs_per_tap;
-  const int pix_bytes = p.CI * ES;
+  const int pix_bytes = p.CI * ES;                              // bytes of one tap's K-run
+  const int pix_pitch = p.pix_pitch ? p.pix_pitch : pix_bytes;  // bytes between neighbouring input pixels
 
   // Requests of slab s into ring stage `stage`, one 16-byte-per-lane load at a time (index l: the A
   // rows first, then the Bt rows) so that they can be spread between the MFMAs.  Past the last slab
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   // arithmetic below relies on.
   unsigned char* req_base = smem;
   unsigned req_a = 0, req_b = 0;  // slab-dependent part of the A / Bt offsets (CONV: A adds the tap per row)
-  int req_dh = 0, req_dw = 0;
+  int req_dh = 0, req_dw = 0, req_px = 0;  // req_px: pixels the chunk lies beyond the tap's first one (pitch < run)
   bool req_ok = false;
   auto prepare_slab = [&](int s, int stage) {
     req_base = smem + stage * kStage + wave * (8 * kSlabBytes);
@@ -159,6 +160,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
       req_ok = live && cb < kbytes_row;
       req_dh = kh * p.DH;
       req_dw = kw * p.DW;
+      req_px = cb / pix_pitch;
       req_a = (unsigned)cb;
       req_b = req_ok ? (unsigned)(tap * pix_bytes + cb) : kOutside;  // Bt row: tap-major, channel-minor
     } else {
@@ -171,8 +173,8 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
       unsigned off;
       if (CONV) {
         const int ih = a_ih0[l] + req_dh, iw = a_iw0[l] + req_dw;
-        const bool ok = req_ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-        off = ok ? join_offsets(a_off[l], (unsigned)((ih * p.W + iw) * pix_bytes) + req_a) : kOutside;
+        const bool ok = req_ok && (unsigned)ih < (unsigned)p.H && (unsigned)(iw + req_px) < (unsigned)p.W;
+        off = ok ? join_offsets(a_off[l], (unsigned)((ih * p.W + iw) * pix_pitch + (int)req_a)) : kOutside;
       } else {
         off = join_offsets(a_off[l], req_a);
       }
@@ -370,7 +372,7 @@ hipError_t PML_CAT(igemm_launch_kind_, PML_KIND)(int cfg, bool conv, const Igemm
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s) {
   // the kernel addresses both operands with 32-bit byte offsets below 2 GiB
   const int64_t es = kind == KIND_BF16 ? 2 : (kind == KIND_I8 ? 1 : 4);
-  const int64_t a_bytes = conv ? (int64_t)a.NB * a.H * a.W * a.CI * es : a.M * a.lda * es;
+  const int64_t a_bytes = conv ? (int64_t)a.NB * a.H * a.W * (a.pix_pitch ? a.pix_pitch : a.CI * es) + 256 : a.M * a.lda * es;
   const int64_t b_bytes = a.N * a.ldbt * es;
   if (a_bytes >= ((int64_t)1 << 31) || b_bytes >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
   switch (kind) {

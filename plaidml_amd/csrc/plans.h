@@ -30,6 +30,9 @@ struct IgemmArgs {
   int64_t ldc;
   // convolution geometry (CONV instantiations only)
   int H, W, CI, OH, OW, KH, KW, SH, SW, PH, PW, DH, DW;
+  // bytes between consecutive input pixels; 0 = CI * element size.  Smaller than that when the "channel
+  // vector" of a tap spans several pixels (igemm_kernel only)
+  int pix_pitch;
   // resident-filter convolution only: image count, LDS rows of the input window, number of 256-pixel tiles
   // halo_variant: 0 = general resident kernel, 1 / 2 = pipelined 3x3 kernel with that many 32-pixel chunks per row
   // b_raw: Bt points at the caller's [K][N] matrix instead of the packed [N][K] one (pipelined kernel only)
@@ -101,6 +104,19 @@ struct Im2colArgs {
   int H, W, CI, OH, OW, KH, KW, SH, SW, PH, PW, DH, DW;
 };
 hipError_t im2col_launch(int elem_size, const Im2colArgs& a, hipStream_t s);
+// Stride-2 convolution over few channels as a unit-stride one over 2x2 pixel blocks ("space to depth").
+//   ih = 2*oh + kh - PH  with  kh + eh = 2*a + b  (eh = PH & 1)   ->   ih = 2*(oh + a - (PH + eh)/2) + b
+// and likewise in w.  S[n][r][c][(b*2 + bw)*CI + ci] = I[n][2r + b][2c + bw][ci] (zero past the image,
+// channels padded to CH); the filter becomes G[co][a][aw][(b*2 + bw)*CI + ci] = F[2a + b - eh][2aw + bw - ew][ci][co].
+struct S2dArgs {
+  const void* in;      // [N][H][W][CI]
+  void* out;           // [N][HS][WS][CH]
+  const void* filter;  // [KH][KW][CI][CO]  (filter kernel only)
+  void* gt;            // [CO][KA][KAW][CH] (filter kernel only)
+  int N, H, W, CI, HS, WS, CH, KH, KW, CO, KA, KAW, EH, EW;
+};
+hipError_t s2d_input_launch(int elem_size, const S2dArgs& a, hipStream_t s);
+hipError_t s2d_filter_launch(int elem_size, const S2dArgs& a, hipStream_t s);
 struct PoolArgs {
   pml_hip_pool2d_desc d;
   const void* in;

@@ -47,6 +47,10 @@ struct Plan {
   // convolution whose channels do not fill 16-byte vectors: patch matrix [M][kpad] + GEMM
   void* patches = nullptr;
   int64_t kpad = 0;
+  // stride-2 convolution over few channels, run as a unit-stride one over 2x2 pixel blocks: the
+  // re-blocked input [N][s2d_h][s2d_w][s2d_ch]; filter taps s2d_ka x s2d_kaw blocks
+  void* s2d = nullptr;
+  int s2d_h = 0, s2d_w = 0, s2d_ch = 0, s2d_ka = 0, s2d_kaw = 0;
   // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
   size_t halo_lds = 0;
   int halo_rows = 0, halo_tiles = 0, halo_variant = 0, n_cus = 0;
@@ -56,6 +60,7 @@ struct Plan {
   ~Plan() {
     if (bt) (void)hipFree(bt);
     if (patches) (void)hipFree(patches);
+    if (s2d) (void)hipFree(s2d);
   }
 };
 
@@ -264,6 +269,45 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.div_ow_magic = p->div_magic[1];
   g.div_per_shift = p->div_shift[0];
   g.div_ow_shift = p->div_shift[1];
+  if (p->s2d) {
+    // unit-stride convolution over the re-blocked input: one "tap" per block row, whose K-run covers
+    // s2d_kaw neighbouring blocks of s2d_ch channels
+    const int es = dt_size(d.in_dtype);
+    g.K = (int64_t)p->s2d_ka * p->s2d_kaw * p->s2d_ch;
+    g.H = p->s2d_h;
+    g.W = p->s2d_w;
+    g.CI = p->s2d_kaw * p->s2d_ch;
+    g.pix_pitch = p->s2d_ch * es;
+    g.KH = p->s2d_ka;
+    g.KW = 1;
+    g.SH = g.SW = 1;
+    g.PH = ((int)d.pad_h + ((int)d.pad_h & 1)) / 2;
+    g.PW = ((int)d.pad_w + ((int)d.pad_w & 1)) / 2;
+  }
+}
+
+void s2d_args(const Plan* p, S2dArgs& a) {
+  const pml_hip_conv2d_desc& d = p->conv;
+  std::memset(&a, 0, sizeof a);
+  a.N = (int)d.n, a.H = (int)d.h, a.W = (int)d.w, a.CI = (int)d.ci;
+  a.HS = p->s2d_h, a.WS = p->s2d_w, a.CH = p->s2d_ch;
+  a.KH = (int)d.kh, a.KW = (int)d.kw, a.CO = (int)d.co;
+  a.KA = p->s2d_ka, a.KAW = p->s2d_kaw;
+  a.EH = (int)d.pad_h & 1, a.EW = (int)d.pad_w & 1;
+}
+
+// Packs the caller's HWCK filter into the plan's Bt.
+hipError_t pack_conv_filter(Plan* p, const void* filter, hipStream_t s) {
+  const pml_hip_conv2d_desc& d = p->conv;
+  const int es = dt_size(d.in_dtype);
+  if (p->s2d) {
+    S2dArgs a;
+    s2d_args(p, a);
+    a.filter = filter;
+    a.gt = p->bt;
+    return s2d_filter_launch(es, a, s);
+  }
+  return transpose_pack(es, filter, p->bt, d.kh * d.kw * d.ci, d.co, d.co, p->bt_ld, s);
 }
 
 }  // namespace
@@ -484,7 +528,12 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     return 0;
   }
   const int es = dt_size(d->in_dtype);
-  const bool via_patches = (d->ci * es) % 16 != 0;
+  // channels that do not fill 16-byte vectors: stride 2 runs over 2x2 pixel blocks, anything else over a patch matrix
+  const bool odd_channels = (d->ci * es) % 16 != 0;
+  const char* conv_env = std::getenv("PML_HIP_CONV");
+  const bool via_s2d = odd_channels && d->stride_h == 2 && d->stride_w == 2 && d->dil_h == 1 && d->dil_w == 1 &&
+                       es >= 2 && d->ci <= 16 && !(conv_env && std::string(conv_env) == "patches");
+  const bool via_patches = odd_channels && !via_s2d;
   if (d->n * d->h * d->w * d->ci >= ((int64_t)1 << 40) || d->h * d->w * d->ci * es >= ((int64_t)1 << 31) ||
       d->kh * d->kw * d->ci * es >= ((int64_t)1 << 31)) {
     fail("conv2d: tensor too large");
@@ -502,6 +551,23 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   const int64_t K = d->kh * d->kw * d->ci;
   p->tile = choose_tile(M, d->co, K * es);
   p->bt_ld = K;
+  if (via_s2d) {
+    const int v = 16 / es;
+    p->s2d_h = (int)(d->h + 1) / 2;
+    p->s2d_w = (int)(d->w + 1) / 2;
+    p->s2d_ch = (int)(4 * d->ci + v - 1) / v * v;
+    p->s2d_ka = (int)(d->kh + (d->pad_h & 1) + 1) / 2;
+    p->s2d_kaw = (int)(d->kw + (d->pad_w & 1) + 1) / 2;
+    const int64_t k2 = (int64_t)p->s2d_ka * p->s2d_kaw * p->s2d_ch;
+    p->tile = choose_tile(M, d->co, k2 * es);
+    p->bt_ld = k2;
+    // 256 spare bytes: a K-run that starts left of the image is addressed (never read) below the buffer's end only
+    if (hipMalloc(&p->s2d, (size_t)d->n * p->s2d_h * p->s2d_w * p->s2d_ch * es + 256) != hipSuccess) {
+      delete p;
+      fail("conv2d: cannot allocate the re-blocked input");
+      return 0;
+    }
+  }
   if (via_patches) {
     // rows padded with zeros to whole 16-byte vectors on both GEMM operands
     const int64_t v = 16 / es;
@@ -524,7 +590,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     const char* e = std::getenv("PML_HIP_CONV");
     int dev = 0;
     hipDeviceProp_t prop;
-    if (!via_patches && !(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
+    if (!odd_channels && !(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
         hipGetDeviceProperties(&prop, dev) == hipSuccess) {
       IgemmArgs g;
       conv_args(p, g);
@@ -549,6 +615,9 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
                 (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, p->halo_lds ? (p->halo_variant ? "256x64 resident filter, pipelined 3x3" : "256x64 resident filter") : tile_name(p->tile));
   p->text = buf;
   if (via_patches) p->text += " via patch matrix (k padded to " + std::to_string(p->kpad) + ")";
+  if (via_s2d)
+    p->text += " over 2x2 pixel blocks (" + std::to_string(p->s2d_ka) + "x" + std::to_string(p->s2d_kaw) + " block taps of " +
+               std::to_string(p->s2d_ch) + " channels, k=" + std::to_string(p->bt_ld) + ")";
   return (int64_t)(intptr_t)p;
 }
 
@@ -559,15 +628,13 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   const pml_hip_conv2d_desc& d = p->conv;
   if (!input || !output) return fail("conv2d_invoke: null operand");
   if (!filter && !p->packed) return fail("conv2d_invoke: filter is null and no packed filter exists");
-  if (!p->patches && ((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
+  if (!p->patches && !p->s2d && ((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
   if (d.init_kind && !init) return fail("conv2d_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
   const int64_t K = d.kh * d.kw * d.ci;
   // the HWCK filter is a row-major [K][CO] matrix; the pipelined resident-filter kernel transposes it itself
   const bool raw_filter = filter && p->halo_lds && p->halo_variant && p->mfma_kind != KIND_I8;
-  if (filter && !raw_filter &&
-      check(transpose_pack(es, filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
-    return 1;
+  if (filter && !raw_filter && check(pack_conv_filter(p, filter, (hipStream_t)s), "pack_conv_filter")) return 1;
   IgemmArgs g;
   conv_args(p, g);
   if (raw_filter) {
@@ -610,6 +677,15 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     g.K = p->kpad;
     return check(igemm_launch(p->mfma_kind, p->tile, false, g, (hipStream_t)s), "igemm_launch");
   }
+  if (p->s2d) {
+    S2dArgs sa;
+    s2d_args(p, sa);
+    sa.in = input;
+    sa.out = p->s2d;
+    if (check(s2d_input_launch(es, sa, (hipStream_t)s), "s2d_input_launch")) return 1;
+    g.A = p->s2d;
+    return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
+  }
   if (p->halo_lds)
     return check(conv_halo_launch(p->mfma_kind, g, p->halo_lds, p->n_cus, (hipStream_t)s), "conv_halo_launch");
   return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
@@ -630,9 +706,8 @@ int pml_hip_conv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream 
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_CONV || !filter) return fail("conv2d_pack_filter: bad argument");
   const pml_hip_conv2d_desc& d = p->conv;
-  const int64_t K = d.kh * d.kw * d.ci;
-  if (check(transpose_pack(dt_size(d.in_dtype), filter, p->bt, K, d.co, d.co, p->bt_ld, (hipStream_t)s), "transpose_pack"))
-    return 1;
+  (void)d;
+  if (check(pack_conv_filter(p, filter, (hipStream_t)s), "pack_conv_filter")) return 1;
   p->packed = true;
   return 0;
 }

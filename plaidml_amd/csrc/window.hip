@@ -203,6 +203,52 @@ __global__ __launch_bounds__(256) void im2col_kernel(Im2colArgs a) {
   *(i32x4_t*)((T*)a.out + m * a.kpad + k0) = packed;
 }
 
+// One thread writes one 16-byte vector of S (see S2dArgs).
+template <typename T>
+__global__ __launch_bounds__(256) void s2d_input_kernel(S2dArgs a) {
+  constexpr int V = 16 / (int)sizeof(T);
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int vecs = a.CH / V;
+  const int64_t total = (int64_t)a.N * a.HS * a.WS * vecs;
+  if (idx >= total) return;
+  const int v = (int)(idx % vecs);
+  int64_t t = idx / vecs;
+  const int c = (int)(t % a.WS);
+  t /= a.WS;
+  const int r = (int)(t % a.HS);
+  const int64_t n = t / a.HS;
+  const T* img = (const T*)a.in + n * ((int64_t)a.H * a.W * a.CI);
+  T vals[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int ch = v * V + e;
+    const int blk = ch / a.CI, ci = ch - blk * a.CI;  // blk = b*2 + bw
+    const int ih = 2 * r + (blk >> 1), iw = 2 * c + (blk & 1);
+    const bool ok = blk < 4 && ih < a.H && iw < a.W;
+    vals[e] = ok ? img[((int64_t)ih * a.W + iw) * a.CI + ci] : (T)0;
+  }
+  i32x4_t packed;
+  __builtin_memcpy(&packed, vals, 16);
+  *(i32x4_t*)((T*)a.out + idx * V) = packed;
+}
+
+// One thread writes one element of G (see S2dArgs).
+template <typename T>
+__global__ __launch_bounds__(256) void s2d_filter_kernel(S2dArgs a) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t per_co = (int64_t)a.KA * a.KAW * a.CH;
+  if (idx >= per_co * a.CO) return;
+  const int co = (int)(idx / per_co);
+  int rem = (int)(idx - co * per_co);
+  const int ch = rem % a.CH;
+  rem /= a.CH;
+  const int aw = rem % a.KAW, ah = rem / a.KAW;
+  const int blk = ch / a.CI, ci = ch - blk * a.CI;
+  const int kh = 2 * ah + (blk >> 1) - a.EH, kw = 2 * aw + (blk & 1) - a.EW;
+  const bool ok = blk < 4 && kh >= 0 && kh < a.KH && kw >= 0 && kw < a.KW;
+  ((T*)a.gt)[idx] = ok ? ((const T*)a.filter)[(((int64_t)kh * a.KW + kw) * a.CI + ci) * a.CO + co] : (T)0;
+}
+
 }  // namespace
 
 hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
@@ -239,6 +285,28 @@ hipError_t im2col_launch(int elem_size, const Im2colArgs& a, hipStream_t s) {
     case 1: hipLaunchKernelGGL(im2col_kernel<uint8_t>, dim3(blocks), dim3(256), 0, s, a); break;
     case 2: hipLaunchKernelGGL(im2col_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, a); break;
     case 4: hipLaunchKernelGGL(im2col_kernel<uint32_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t s2d_input_launch(int elem_size, const S2dArgs& a, hipStream_t s) {
+  const int64_t total = (int64_t)a.N * a.HS * a.WS * (a.CH * elem_size / 16);
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  switch (elem_size) {
+    case 2: hipLaunchKernelGGL(s2d_input_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    case 4: hipLaunchKernelGGL(s2d_input_kernel<uint32_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t s2d_filter_launch(int elem_size, const S2dArgs& a, hipStream_t s) {
+  const int64_t total = (int64_t)a.CO * a.KA * a.KAW * a.CH;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  switch (elem_size) {
+    case 2: hipLaunchKernelGGL(s2d_filter_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, a); break;
+    case 4: hipLaunchKernelGGL(s2d_filter_kernel<uint32_t>, dim3(blocks), dim3(256), 0, s, a); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

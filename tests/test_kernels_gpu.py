@@ -150,6 +150,9 @@ def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bia
     KH, KW, _, CO = F.shape
     ph, OH = op.compute_padding_and_output_size(H, KH, stride, autopad)
     pw, OW = op.compute_padding_and_output_size(W, KW, stride, autopad)
+    if pad is not None:  # explicit symmetric padding
+        ph = pw = pad
+        OH, OW = (H + 2 * pad - KH) // stride + 1, (W + 2 * pad - KW) // stride + 1
     d = hk.Conv2dDesc()
     d.in_dtype, d.out_dtype, d.c_dtype = in_dt, out_dt, out_dt
     d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, KH, KW, CO, OH, OW
@@ -179,10 +182,13 @@ def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bia
     return out
 
 
-def oracle_conv(Iv, Fv, dt, stride, autopad, bias=None, relu=False):
+def oracle_conv(Iv, Fv, dt, stride, autopad, bias=None, relu=False, pad=None):
     I, F = E.Placeholder(dt, Iv.shape), E.Placeholder(dt, Fv.shape)
     ins, vals = [I, F], [Iv, Fv]
-    O = op.convolution(I, F, strides=[stride, stride], autopad=autopad)
+    if pad is not None:
+        O = op.convolution(I, F, strides=[stride, stride], autopad=op.EXPLICIT, manual_padding=[pad, pad])
+    else:
+        O = op.convolution(I, F, strides=[stride, stride], autopad=autopad)
     if bias is not None:
         B = E.Placeholder(dt, bias.shape)
         ins.append(B)
@@ -306,20 +312,40 @@ def test_conv_resident_filter_matches_generic_kernel(monkeypatch):
     np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
 
 
-@pytest.mark.parametrize('kind', ['f32', 'bf16'])
-def test_conv_three_channel_stem(kind, capsys):
-    # 7x7 stride 2 over a 3-channel image: channels do not fill 16-byte vectors -> patch matrix + GEMM
-    Iv, Fv = _conv_case(kind, (2, 30, 34, 3), 7, 7, 64, op.SAME_UPPER, 41)
-    bias = np.random.default_rng(42).standard_normal(64).astype(np.float32)
+def _stem_case(kind, shape, k, co, stride, pad, seed):
+    Iv, Fv = _conv_case(kind, shape, k, k, co, op.SAME_UPPER, seed)
+    bias = np.random.default_rng(seed + 1).standard_normal(co).astype(np.float32)
     if kind == 'bf16':
         bias = E.round_bf16(bias)
-        out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=2, bias=bf16(bias), relu=True))
-        ref = oracle_conv(Iv, Fv, D.BFLOAT16, 2, op.SAME_UPPER, bias, True)
+        out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=stride, pad=pad, bias=bf16(bias),
+                                        relu=True))
+        ref = oracle_conv(Iv, Fv, D.BFLOAT16, stride, op.SAME_UPPER, bias, True, pad=pad)
         np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
     else:
-        out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=2, bias=bias, relu=True)
-        ref = oracle_conv(Iv, Fv, D.FLOAT32, 2, op.SAME_UPPER, bias, True)
+        out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, pad=pad, bias=bias, relu=True)
+        ref = oracle_conv(Iv, Fv, D.FLOAT32, stride, op.SAME_UPPER, bias, True, pad=pad)
         np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4)
+
+
+# stride 2 over channels that do not fill 16-byte vectors: unit-stride convolution over 2x2 pixel blocks.
+# (shape, k, co, pad): even and odd padding, odd image sides, 1- and 5-channel images, a 3x3 and a 2x2 filter
+STEM_CASES = [((2, 30, 34, 3), 7, 64, None), ((2, 32, 32, 3), 7, 64, 3), ((2, 31, 29, 3), 7, 64, 3),
+              ((3, 17, 23, 1), 3, 32, 1), ((1, 20, 18, 5), 5, 48, 0), ((2, 16, 16, 3), 2, 64, 0)]
+
+
+@pytest.mark.parametrize('kind', ['f32', 'bf16'])
+@pytest.mark.parametrize('shape,k,co,pad', STEM_CASES)
+def test_conv_few_channel_stride2(kind, shape, k, co, pad, capsys):
+    _stem_case(kind, shape, k, co, 2, pad, 41)
+    assert '2x2 pixel blocks' in capsys.readouterr().out
+
+
+@pytest.mark.parametrize('kind', ['f32', 'bf16'])
+@pytest.mark.parametrize('stride', [1, 2])
+def test_conv_few_channel_patch_matrix(kind, stride, capsys, monkeypatch):
+    # other strides (and stride 2 on request) gather a patch matrix [M][K padded] and run a plain GEMM
+    monkeypatch.setenv('PML_HIP_CONV', 'patches')
+    _stem_case(kind, (2, 30, 34, 3), 7, 64, stride, None, 43)
     assert 'patch matrix' in capsys.readouterr().out
 
 
