@@ -20,6 +20,8 @@
 // the 16-byte-per-lane operand reads free of bank conflicts.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+#include <string>
 #include <type_traits>
 
 #include "device_common.h"
@@ -305,88 +307,55 @@ __global__ __launch_bounds__(kThreads) void conv_halo_kernel(IgemmArgs p) {
   }
 }
 
-// ---------------------------------------------------------------------------
-// 3x3 filters, exactly 64 output channels, tail = bias? relu? store: the hot case.
-//
-// Same data movement as above, with the instruction streams arranged so that a
-// wavefront's matrix pipe stays fed while it does everything else:
-//  * the nine taps are unrolled, so the whole K loop of a tile is one basic block;
-//  * the result of tile t stays in registers and its bias / relu / convert / store
-//    work is cut into 16 pieces that sit between the MFMAs of tile t+1
-//    (two accumulator sets alternate roles);
-//  * window loads and output stores are buffer instructions: an offset beyond the
-//    buffer reads zeros / drops the store, which is how padding, image ends and the
-//    ragged last tile are handled without any branch in the stream.
-// NCH = 32-pixel chunks per window row (1 or 2).
-// ---------------------------------------------------------------------------
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
-constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
-#ifndef PML_CONV_AHEAD
-#define PML_CONV_AHEAD 2
-#endif
-constexpr int kFar = 0x40000000;              // beyond any input this kernel accepts (<= 2^30 bytes); two of them still are
-
-template <int KIND, int NCH>
-__global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
-  constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
-  constexpr int MI = 2, NI = 2;
-  constexpr int OES = KIND == KIND_BF16 ? 2 : 4;  // bytes per output element (bf16 -> bf16, fp32 -> fp32, int8 -> int32)
-  constexpr int kTaps = 9;
-  constexpr int krow = kTaps * kPixBytes, brow = krow + 16;
-  constexpr int kRows = kMaxLoads / NCH;
-  typedef typename Acc<KIND>::type acc_t;
-  typedef typename Acc<KIND>::scalar accs_t;
-
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* const sB = smem;
-  unsigned char* const sH = smem + kBN * brow;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int Hv = p.OH + 2, Wv = p.OW + 2;
-
-  // ---- filter -> LDS, once: all of a thread's 18 vectors are requested before the first is stored ----
-  // LDS row j*32 + 8q + 4h + e holds output channel 32h + 16j + 4q + e: after the MFMAs a lane
-  // (pixel, h) then owns the 16 consecutive channels 32h + 16j .. + 15 of block j in register order.
-  constexpr int vecs_per_row = krow / 16;
-  constexpr int kFilterVecs = kBN * vecs_per_row / kThreads;
+// The 3x3 filter of 64 output channels on its way into LDS, held in registers between the two
+// steps so that a kernel can put other work between requesting it and storing it.
+// LDS row j*32 + 8q + 4h + e holds output channel 32h + 16j + 4q + e: after the MFMAs a lane
+// (pixel, h) then owns the 16 consecutive channels 32h + 16j .. + 15 of block j in register order.
+// The filter comes either packed as Bt[CO][K] or, with b_raw, as the caller's [K][CO] matrix
+// (HWCK, 2- or 4-byte elements).  The raw form is transposed on the way in: a task is a square of
+// kEpv K-indices x kEpv channels, read as kEpv 16-byte vectors along CO, turned in registers and
+// written as kEpv 16-byte vectors along K.
+template <int KIND>
+struct FilterStager {
+  static constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
+  static constexpr int krow = 9 * kPixBytes;
+  static constexpr int vecs_per_row = krow / 16;
+  static constexpr int kFilterVecs = kBN * vecs_per_row / kThreads;
   static_assert(kBN * vecs_per_row % kThreads == 0, "filter vectors divide evenly over the threads");
-  // The filter comes either packed as Bt[CO][K] or, with b_raw, as the caller's [K][CO] matrix
-  // (HWCK, 2- or 4-byte elements).  The raw form is transposed on the way in: a task is a square of
-  // kEpv K-indices x kEpv channels, read as kEpv 16-byte vectors along CO, turned in registers and
-  // written as kEpv 16-byte vectors along K.
-  constexpr int kEpv = 16 / ES;             // elements per 16-byte vector
-  constexpr int kCoGroups = kBN / kEpv;
-  constexpr int kTasks = (krow / 16) * kCoGroups;
-  constexpr int kTaskIters = (kTasks + kThreads - 1) / kThreads;
-  constexpr int kRawRegs = ES == 1 ? 1 : kTaskIters * kEpv;
-  constexpr int kFlRegs = kRawRegs > kFilterVecs ? kRawRegs : kFilterVecs;
+  static constexpr int kEpv = 16 / ES;  // elements per 16-byte vector
+  static constexpr int kCoGroups = kBN / kEpv;
+  static constexpr int kTasks = (krow / 16) * kCoGroups;
+  static constexpr int kTaskIters = (kTasks + kThreads - 1) / kThreads;
+  static constexpr int kRawRegs = ES == 1 ? 1 : kTaskIters * kEpv;
+  static constexpr int kFlRegs = kRawRegs > kFilterVecs ? kRawRegs : kFilterVecs;
   i32x4_t fl[kFlRegs];
-  if (ES != 1 && p.b_raw) {
+
+  __device__ __forceinline__ void load(const IgemmArgs& p, int tid) {
+    if (ES != 1 && p.b_raw) {
 #pragma unroll
-    for (int it = 0; it < kTaskIters; ++it) {
-      int task = tid + it * kThreads;
-      if (task >= kTasks) task = kTasks - 1;
-      const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
+      for (int it = 0; it < kTaskIters; ++it) {
+        int task = tid + it * kThreads;
+        if (task >= kTasks) task = kTasks - 1;
+        const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
 #pragma unroll
-      for (int kk = 0; kk < kEpv; ++kk)
-        fl[(it * kEpv + kk) % kFlRegs] =
-            *(const i32x4_t*)((const unsigned char*)p.Bt + ((int64_t)(kg * kEpv + kk) * kBN + cg * kEpv) * ES);
-    }
-  } else {
+        for (int kk = 0; kk < kEpv; ++kk)
+          fl[(it * kEpv + kk) % kFlRegs] =
+              *(const i32x4_t*)((const unsigned char*)p.Bt + ((int64_t)(kg * kEpv + kk) * kBN + cg * kEpv) * ES);
+      }
+    } else {
 #pragma unroll
-    for (int k = 0; k < kFilterVecs; ++k) {
-      const int q = tid + k * kThreads;
-      const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
-      const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
-      fl[k] = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
+      for (int k = 0; k < kFilterVecs; ++k) {
+        const int q = tid + k * kThreads;
+        const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
+        const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
+        fl[k] = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
+      }
     }
   }
-  auto store_filter = [&]() {
+
+  // row_ptr(row): LDS address of filter row `row`
+  template <typename F>
+  __device__ __forceinline__ void store(const IgemmArgs& p, int tid, F row_ptr) {
     if (ES != 1 && p.b_raw) {
 #pragma unroll
       for (int it = 0; it < kTaskIters; ++it) {
@@ -415,7 +384,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
           for (int e = 0; e < kEpv; ++e) {
             const int co = cg * kEpv + e;
             const int row = ((co >> 4) & 1) * 32 + ((co >> 2) & 3) * 8 + (co >> 5) * 4 + (co & 3);
-            *(i32x4_t*)(sB + row * brow + kg * 16) = out[e];
+            *(i32x4_t*)(row_ptr(row) + kg * 16) = out[e];
           }
         }
       }
@@ -424,10 +393,61 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
       for (int k = 0; k < kFilterVecs; ++k) {
         const int q = tid + k * kThreads;
         const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
-        *(i32x4_t*)(sB + row * brow + vec * 16) = fl[k];
+        *(i32x4_t*)(row_ptr(row) + vec * 16) = fl[k];
       }
     }
-  };
+  }
+};
+
+// ---------------------------------------------------------------------------
+// 3x3 filters, exactly 64 output channels, tail = bias? relu? store: the hot case.
+//
+// Same data movement as above, with the instruction streams arranged so that a
+// wavefront's matrix pipe stays fed while it does everything else:
+//  * the nine taps are unrolled, so the whole K loop of a tile is one basic block;
+//  * the result of tile t stays in registers and its bias / relu / convert / store
+//    work is cut into 16 pieces that sit between the MFMAs of tile t+1
+//    (two accumulator sets alternate roles);
+//  * window loads and output stores are buffer instructions: an offset beyond the
+//    buffer reads zeros / drops the store, which is how padding, image ends and the
+//    ragged last tile are handled without any branch in the stream.
+// NCH = 32-pixel chunks per window row (1 or 2).
+// ---------------------------------------------------------------------------
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
+#define PML_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#ifndef PML_CONV_AHEAD
+#define PML_CONV_AHEAD 2
+#endif
+constexpr int kFar = 0x40000000;              // beyond any input this kernel accepts (<= 2^30 bytes); two of them still are
+
+template <int KIND, int NCH>
+__global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
+  constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
+  constexpr int MI = 2, NI = 2;
+  constexpr int OES = KIND == KIND_BF16 ? 2 : 4;  // bytes per output element (bf16 -> bf16, fp32 -> fp32, int8 -> int32)
+  constexpr int kTaps = 9;
+  constexpr int krow = kTaps * kPixBytes, brow = krow + 16;
+  constexpr int kRows = kMaxLoads / NCH;
+  typedef typename Acc<KIND>::type acc_t;
+  typedef typename Acc<KIND>::scalar accs_t;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* const sB = smem;
+  unsigned char* const sH = smem + kBN * brow;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int Hv = p.OH + 2, Wv = p.OW + 2;
+
+  // ---- filter -> LDS, once: all of a thread's 18 vectors are requested before the first is stored ----
+  FilterStager<KIND> filter;
+  filter.load(p, tid);
+  auto store_filter = [&]() { filter.store(p, tid, [&](int row) { return sB + row * brow; }); };
 
   const __amdgpu_buffer_rsrc_t rin =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)((int64_t)p.NB * p.H * p.W * kPixBytes), kRsrcFlags);
@@ -727,6 +747,318 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same hot case with the filter in registers (16-bit and 8-bit elements).
+//
+// With the filter in LDS every MFMA needs one 16-byte LDS read per lane, and four wavefronts
+// cannot pull that much out of LDS: the matrix pipe waits.  A wavefront owns 64 pixels x 64 channels,
+// so it needs the whole 3x3x(128 bytes)x64 filter: 72 16-byte fragments per lane, 288 of the 512
+// registers a lane has at one wavefront per SIMD.  They are loaded once; LDS traffic halves and LDS
+// itself is free for two window buffers, filled by loads that write LDS directly (no register
+// staging, no store phase): the window of tile t+1 arrives while tile t is computed.
+//
+// Window layout: pixel slot q = row * Wv + column (Wv = padded image width), 128 bytes each, rows
+// packed without gaps.  Slot q keeps its eight 16-byte channel vectors permuted: vector u sits at
+// position u ^ ((q >> 1) & 7), which spreads the 32 pixels of an operand read over all banks.
+// A wavefront-wide request (64 lanes x 16 bytes) fills 8 consecutive slots; requests are issued per
+// row in 8 groups of 8 columns, and a lane whose column is past the row's end fetches what belongs
+// into the slot it really writes, a pixel of the next row (written twice then, with the same bytes).
+// ---------------------------------------------------------------------------
+constexpr int kRegRows = 10;                   // window rows per buffer
+constexpr int kRegBrow = 9 * kPixBytes + 16;   // stride of a staged filter row
+// one window buffer: the last row's requests reach 64 columns
+__host__ __device__ constexpr int reg_win_bytes(int Wv) { return ((kRegRows - 1) * Wv + 64) * kPixBytes; }
+// staged filter rows that fit below the second window buffer (the first window is loaded into that one)
+__host__ __device__ constexpr int reg_rows_low(int Wv) {
+  return reg_win_bytes(Wv) / kRegBrow < kBN ? reg_win_bytes(Wv) / kRegBrow : kBN;
+}
+// 64 accumulator-typed initial values sit behind the window buffers and the staged filter rows beyond them
+__host__ __device__ constexpr int reg_bias_off(int Wv) { return 2 * reg_win_bytes(Wv) + (kBN - reg_rows_low(Wv)) * kRegBrow; }
+__host__ __device__ constexpr int reg_lds_bytes(int Wv) { return reg_bias_off(Wv) + kBN * 4; }
+
+template <int KIND>
+__global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p) {
+  static_assert(KIND != KIND_F32, "16-bit and 8-bit elements only");
+  constexpr int MI = 2, NI = 2;
+  constexpr int OES = KIND == KIND_BF16 ? 2 : 4;
+  constexpr int kTaps = 9, kBlocks = kTaps * 4;  // K-blocks of 32 bytes
+  typedef typename Acc<KIND>::type acc_t;
+  typedef typename Acc<KIND>::scalar accs_t;
+  typedef accs_t acc4_t __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5;
+  const int Hv = p.OH + 2, Wv = p.OW + 2;
+  const int win_bytes = reg_win_bytes(Wv);
+#ifdef PML_CONV_TRACE
+  const long long t_entry = clock64();
+#endif
+
+  const __amdgpu_buffer_rsrc_t rin =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)((int64_t)p.NB * p.H * p.W * kPixBytes), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t rout =
+      __builtin_amdgcn_make_buffer_rsrc(p.C, 0, (int)(p.M * p.ldc * OES), kRsrcFlags);
+
+  // ---- window requests: wavefront w fills columns 8w .. 8w+7 and 8(w+4) .. 8(w+4)+7 of every row ----
+  // Fixed for the kernel's life: a lane's column, whether that column is really one of the next row,
+  // and its byte offset inside the input row (kFar where the slot is padding).
+  int req_px[2], req_col[2];
+  bool req_next[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    req_px[c] = (wave + 4 * c) * 8 + (lane >> 3);
+    req_next[c] = req_px[c] >= Wv;
+    const int iw = req_px[c] - (req_next[c] ? Wv : 0) - p.PW;
+    req_col[c] = (unsigned)iw < (unsigned)p.W ? iw * kPixBytes : kFar;
+  }
+  // rb_cur / rb_next: byte offset of input row r / r + 1 of the window, kFar for a row of padding
+  auto request = [&](unsigned char* win, int r, int c, int rb_cur, int rb_next) {
+    const int q = r * Wv + req_px[c];
+    const int vec = (lane & 7) ^ ((q >> 1) & 7);
+    const int voff = (req_next[c] ? rb_next : rb_cur) + req_col[c] + vec * 16;  // two kFar still are outside
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rin, PML_LDS(win + (r * Wv + (wave + 4 * c) * 8) * kPixBytes), 16, voff, 0, 0,
+                                             0);
+  };
+  // offset of window row r of a tile (row `ihv` of padded image `nb`), and the step to the row after it
+  auto row_offset = [&](int r, int nrows, int nb, int ihv) {
+    const int ih = ihv - p.PH;
+    const int ok = (int)(r < nrows) & (int)(nb < p.NB) & (int)((unsigned)ih < (unsigned)p.H);
+    const int real = (nb * p.H + ih) * p.W * kPixBytes;
+    return kFar ^ ((kFar ^ real) & -ok);
+  };
+  auto next_row = [&](int& nb, int& ihv) {
+    const int wrap = (int)(ihv + 1 == Hv);
+    ihv = (ihv + 1) & (wrap - 1);
+    nb += wrap;
+  };
+
+  int t = first_tile(blockIdx.x, gridDim.x);
+  TileGeom g = tile_geom(p, t, Hv);
+  unsigned char* const win0 = smem;
+  unsigned char* const win1 = smem + win_bytes;
+  {
+    // the first window goes into the second buffer: the filter is staged around it
+    int nb = g.nb0, ihv = g.ihv0;
+    int rb_next = row_offset(0, g.nrows, nb, ihv);
+#pragma unroll
+    for (int r = 0; r < kRegRows; ++r) {
+      const int rb_cur = rb_next;
+      next_row(nb, ihv);
+      rb_next = row_offset(r + 1, g.nrows, nb, ihv);
+      request(win1, r, 0, rb_cur, rb_next);
+      request(win1, r, 1, rb_cur, rb_next);
+    }
+  }
+
+  // ---- filter -> LDS (transposed if raw) -> registers; initial values -> LDS ----
+  const int rows_low = reg_rows_low(Wv), bias_off = reg_bias_off(Wv);
+  auto filter_row = [&](int row) {
+    return smem + (row < rows_low ? row * kRegBrow : 2 * win_bytes + (row - rows_low) * kRegBrow);
+  };
+  {
+    FilterStager<KIND> filter;
+    filter.load(p, tid);
+    filter.store(p, tid, filter_row);
+  }
+  if (tid < kBN) {
+    accs_t b = 0;
+    if (p.init != nullptr) {
+      Scalar<float, int> v = load_scalar<float, int>(p.init, (int64_t)tid * p.init_cs, p.init_dtype);
+      b = KIND == KIND_I8 ? (accs_t)v.i : (accs_t)v.f;
+    }
+    *(accs_t*)(smem + bias_off + tid * 4) = b;
+  }
+  __syncthreads();
+  i32x4_t breg[kBlocks][NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const unsigned char* src = filter_row(j * 32 + (lane & 31)) + half * 16;
+#pragma unroll
+    for (int s = 0; s < kBlocks; ++s) breg[s][j] = *(const i32x4_t*)(src + s * 32);
+  }
+  const unsigned char* const bias_src = smem + bias_off + 32 * half * 4;
+
+  const float lo_f = p.tail_relu ? 0.f : -__builtin_inff();
+  const int lo_i = p.tail_relu ? 0 : (int)0x80000000;
+  const unsigned per = (unsigned)(p.OH * p.OW);
+
+  // where the pixel of this lane in half `i` of a tile sits: its window slot and its output byte offset
+  auto place = [&](const TileGeom& tg, int i, int& a_q, int& m_off) {
+    const unsigned m = (unsigned)tg.m0 + wave * 64 + i * 32 + (lane & 31);
+    const bool ok = m < (unsigned)p.M;
+    const unsigned mc = ok ? m : (unsigned)p.M - 1;
+    const unsigned nb = fast_div(mc, p.div_per_magic, p.div_per_shift);
+    const unsigned rem = mc - nb * per;
+    const unsigned oh = fast_div(rem, p.div_ow_magic, p.div_ow_shift), ow = rem - oh * (unsigned)p.OW;
+    a_q = ((int)(nb * Hv + oh) - tg.v0) * Wv + (int)ow;
+    m_off = ok ? (int)((m * (unsigned)p.ldc + 32 * half) * OES) : (int)0x80000000;
+  };
+
+  // one of the 8 pieces of a finished half tile: 4 consecutive channels of the lane's pixel
+  // (bf16 output: two pieces share one 16-byte store)
+  unsigned held[2] = {0, 0};
+  auto finish_piece = [&](const acc_t (&acc)[NI], int m_off, int pc) {
+    const int j = pc >> 2, q = pc & 3;
+    const int off = m_off + (j * 16 + 4 * q) * OES;
+    if (KIND == KIND_I8) {
+      u32x4_t w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int v = (int)acc[j][4 * q + e];
+        w[e] = (unsigned)(v < lo_i ? lo_i : v);
+      }
+      __builtin_amdgcn_raw_buffer_store_b128(w, rout, off, 0, 0);
+    } else {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = (float)acc[j][4 * q + e];
+        v[e] = v[e] < lo_f ? lo_f : v[e];
+      }
+      const f32x2_t a01 = {v[0], v[1]}, a23 = {v[2], v[3]};
+      const bf16x2_t h01 = __builtin_convertvector(a01, bf16x2_t), h23 = __builtin_convertvector(a23, bf16x2_t);
+      unsigned w0, w1;
+      __builtin_memcpy(&w0, &h01, 4);
+      __builtin_memcpy(&w1, &h23, 4);
+      if ((q & 1) == 0) {
+        held[0] = w0;
+        held[1] = w1;
+      } else {
+        const u32x4_t w = {held[0], held[1], w0, w1};
+        __builtin_amdgcn_raw_buffer_store_b128(w, rout, off - 4 * OES, 0, 0);
+      }
+    }
+  };
+
+  // placement of the two halves of the current tile and of the tile after it
+  int a_q[MI], m_off[MI];
+  int a_next[MI], m_next[MI];
+
+  // K loop of half I of a tile (32 pixels x 64 channels per wavefront) out of window `cur`.  Two
+  // accumulator sets alternate between the halves, so the finished half rides along: its 8 pieces
+  // (pacc, pm_off) sit between the MFMAs of this one.  Half 0 also carries the requests for the next
+  // tile's window (geometry g2, into `nxt`), half 1 the placement of the next tile.  Past the last
+  // tile every row is out of range and every request reads zeros, so none of this needs a branch.
+  auto k_loop = [&](auto half_tag, acc_t (&acc)[NI], const unsigned char* cur, unsigned char* nxt,
+                    const acc_t (&pacc)[NI], int pm_off, const TileGeom& g2) {
+    constexpr int I = decltype(half_tag)::value;
+    int w_nb = g2.nb0, w_ihv = g2.ihv0;
+    int rb_cur = kFar, rb_next = I == 0 ? row_offset(0, g2.nrows, w_nb, w_ihv) : kFar;
+    // accumulators start from the initial values of the lane's channels
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const acc4_t v = *(const acc4_t*)(bias_src + (16 * j + 4 * q) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[j][4 * q + e] = v[e];
+      }
+    // Operand fragments are fetched kAhead K-blocks ahead.
+    constexpr int kAhead = 2 * PML_CONV_AHEAD;
+    i32x4_t fa[kAhead + 1];
+    auto fetch = [&](int s1) {
+      const int tap = s1 >> 2, ks = s1 & 3;
+      const int qt = a_q[I] + (tap / 3) * Wv + tap % 3;
+      const int vec16 = ((((qt >> 1) & 7) ^ half) << 4) ^ (ks << 5);  // vector 2*ks + half of the slot, permuted
+      fa[s1 % (kAhead + 1)] = *(const i32x4_t*)(cur + qt * kPixBytes + vec16);
+    };
+#pragma unroll
+    for (int s0 = 0; s0 < kAhead; ++s0) fetch(s0);
+#pragma unroll
+    for (int s = 0; s < kBlocks; ++s) {
+      if (s + kAhead < kBlocks) fetch(s + kAhead);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) mma_block<KIND>(acc[j], breg[s][j], fa[s % (kAhead + 1)]);
+      if (I == 0 && s < 2 * kRegRows) {  // the next tile's window, one request per K-block
+        if ((s & 1) == 0) {
+          rb_cur = rb_next;
+          next_row(w_nb, w_ihv);
+          rb_next = row_offset((s >> 1) + 1, g2.nrows, w_nb, w_ihv);
+        }
+        request(nxt, s >> 1, s & 1, rb_cur, rb_next);
+      }
+      if ((s & 3) == 1 && (s >> 2) < 8) finish_piece(pacc, pm_off, s >> 2);
+      if (I == 1 && s == 32) place(g2, 0, a_next[0], m_next[0]);
+      if (I == 1 && s == 34) place(g2, 1, a_next[1], m_next[1]);
+      // order inside the K-block: the LDS read and the window request first, then VALU work between the MFMAs
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+#pragma unroll
+      for (int q = 0; q < NI; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep requests and pieces in the K-block they were put in
+    }
+  };
+
+  acc_t accX[NI], accY[NI];
+  place(g, 0, a_q[0], m_off[0]);
+  place(g, 1, a_q[1], m_off[1]);
+  int m_last = (int)0x80000000;  // second half of the tile before: none precedes the first, its pieces are dropped
+#pragma unroll
+  for (int j = 0; j < NI; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accY[j][r] = 0;
+  __syncthreads();  // the filter is out of LDS, the first window is in
+
+  unsigned char* cur = win1;
+  unsigned char* nxt = win0;
+#ifdef PML_CONV_TRACE
+  long long* trace = (long long*)p.outs[5];
+  int tn = 0;
+  const bool tracing = trace && blockIdx.x == 0 && lane == 0;
+#define PML_STAMP() do { if (tracing && tn < 60) trace[wave * 64 + tn++] = clock64(); } while (0)
+  if (tracing) { trace[wave * 64 + 59] = t_entry; trace[wave * 64 + 60] = clock64(); trace[wave * 64 + 62] = wall_clock64(); }
+#else
+#define PML_STAMP()
+#endif
+  for (;;) {
+    const int t2 = t + gridDim.x;
+    const TileGeom g2 = tile_geom(p, t2, Hv);
+    PML_STAMP();
+    k_loop(std::integral_constant<int, 0>(), accX, cur, nxt, accY, m_last, g2);
+    PML_STAMP();
+    k_loop(std::integral_constant<int, 1>(), accY, cur, nxt, accX, m_off[0], g2);
+    PML_STAMP();
+    __syncthreads();  // every wavefront is done with the current window; the next one has arrived
+    PML_STAMP();
+    m_last = m_off[1];
+    t = t2;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      a_q[i] = a_next[i];
+      m_off[i] = m_next[i];
+    }
+    unsigned char* const w = cur;
+    cur = nxt;
+    nxt = w;
+    if (t >= p.n_tiles) break;
+  }
+#pragma unroll
+  for (int pc = 0; pc < 8; ++pc) finish_piece(accY, m_last, pc);
+#ifdef PML_CONV_TRACE
+  if (tracing) { trace[wave * 64 + 61] = clock64(); trace[wave * 64 + 63] = wall_clock64(); }
+#endif
+}
+
+template <int KIND>
+hipError_t launch_regfilter(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
+  auto kern = conv_regfilter3x3_kernel<KIND>;
+  static size_t attr_lds = 0;
+  if (lds > attr_lds) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    attr_lds = lds;
+  }
+  const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), lds, s, a);
+  return hipGetLastError();
+}
+
 template <int KIND, int NCH>
 hipError_t launch3x3(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
   auto kern = conv_halo3x3_kernel<KIND, NCH>;
@@ -805,6 +1137,14 @@ size_t conv_halo_prepare(int kind, IgemmArgs* a) {
                      a->M * a->ldc * out_es < ((int64_t)1 << 31) && nchunks <= 2)
                         ? nchunks
                         : 0;
+  // filter in registers: 16- and 8-bit elements, two windows of at most kRegRows rows of 32 .. 64 pixels in LDS
+  // (PML_HIP_CONV=ldsfilter keeps the filter in LDS)
+  const char* e = std::getenv("PML_HIP_CONV");
+  if (a->halo_variant && kind != KIND_F32 && max_rows <= kRegRows && Wv >= 32 && Wv <= 64 &&
+      reg_lds_bytes(Wv) <= 160 * 1024 && !(e && std::string(e) == "ldsfilter")) {
+    a->halo_variant = 3;
+    return (size_t)reg_lds_bytes(Wv);
+  }
   return total;
 }
 
@@ -815,6 +1155,12 @@ hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int 
       case KIND_BF16: return launch3x3<KIND_BF16, 1>(a, lds_bytes, n_cus, s);
       case KIND_I8: return launch3x3<KIND_I8, 1>(a, lds_bytes, n_cus, s);
     }
+  } else if (a.halo_variant == 3) {
+    switch (kind) {
+      case KIND_BF16: return launch_regfilter<KIND_BF16>(a, lds_bytes, n_cus, s);
+      case KIND_I8: return launch_regfilter<KIND_I8>(a, lds_bytes, n_cus, s);
+    }
+    return hipErrorInvalidValue;
   } else if (a.halo_variant == 2) {
     switch (kind) {
       case KIND_F32: return launch3x3<KIND_F32, 2>(a, lds_bytes, n_cus, s);

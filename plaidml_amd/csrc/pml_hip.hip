@@ -612,7 +612,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   std::snprintf(buf, sizeof buf, "conv2d %s n=%lld %lldx%lldx%lld k=%lldx%lld co=%lld -> %lldx%lld (implicit gemm m=%lld n=%lld k=%lld) tile=%s",
                 d->in_dtype == PML_HIP_F32 ? "f32" : d->in_dtype == PML_HIP_BF16 ? "bf16" : "i8", (long long)d->n,
                 (long long)d->h, (long long)d->w, (long long)d->ci, (long long)d->kh, (long long)d->kw, (long long)d->co,
-                (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, p->halo_lds ? (p->halo_variant ? "256x64 resident filter, pipelined 3x3" : "256x64 resident filter") : tile_name(p->tile));
+                (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, p->halo_lds ? (p->halo_variant == 3 ? "256x64 resident filter, in registers" : p->halo_variant ? "256x64 resident filter, pipelined 3x3" : "256x64 resident filter") : tile_name(p->tile));
   p->text = buf;
   if (via_patches) p->text += " via patch matrix (k padded to " + std::to_string(p->kpad) + ")";
   if (via_s2d)

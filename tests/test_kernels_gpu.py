@@ -287,6 +287,42 @@ def test_conv_resident_filter(kind, shape, kh, kw, co, autopad, capsys):
     assert 'resident filter' in capsys.readouterr().out
 
 
+# Windows of at most 10 rows of 32 to 64 pixels with 16- or 8-bit elements: the filter lives in registers.
+# Ragged last tile, images that end inside a tile, the widest and the tallest window, VALID and SAME.
+REGISTER_CASES = [('bf16', (2, 56, 56, 64), op.SAME_UPPER, True), ('bf16', (3, 11, 60, 64), op.SAME_UPPER, True),
+                  ('bf16', (2, 9, 62, 64), op.VALID, False), ('bf16', (9, 9, 62, 64), op.SAME_UPPER, True),
+                  ('i8', (2, 20, 50, 128), op.SAME_UPPER, False), ('i8', (1, 7, 47, 128), op.VALID, False)]
+
+
+@pytest.mark.parametrize('kind,shape,autopad,with_bias', REGISTER_CASES)
+def test_conv_register_filter(kind, shape, autopad, with_bias, capsys):
+    Iv, Fv = _conv_case(kind, shape, 3, 3, 64, autopad, 27)
+    if kind == 'i8':
+        out = run_conv(Iv, Fv, hk.I8, hk.I32, autopad=autopad)
+        assert 'in registers' in capsys.readouterr().out
+        I, F = E.Placeholder(D.INT8, Iv.shape), E.Placeholder(D.INT8, Fv.shape)
+        O = op.convolution(E.cast(I, D.INT32), E.cast(F, D.INT32), strides=[1, 1], autopad=autopad)
+        ref, = E.run(E.Program('c', [I, F], [O]), [Iv, Fv])
+        np.testing.assert_array_equal(out, ref)
+        return
+    bias = E.round_bf16(np.random.default_rng(28).standard_normal(64).astype(np.float32)) if with_bias else None
+    out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, autopad=autopad,
+                                    bias=bf16(bias) if with_bias else None, relu=with_bias))
+    assert 'in registers' in capsys.readouterr().out
+    ref = oracle_conv(Iv, Fv, D.BFLOAT16, 1, autopad, bias, with_bias)
+    np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
+
+
+def test_conv_register_filter_matches_lds_filter(monkeypatch):
+    # same inputs with the filter kept in LDS: both accumulate in fp32 and round once
+    Iv, Fv = _conv_case('bf16', (3, 56, 56, 64), 3, 3, 64, op.SAME_UPPER, 29)
+    bias = bf16(E.round_bf16(np.random.default_rng(30).standard_normal(64).astype(np.float32)))
+    a = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
+    monkeypatch.setenv('PML_HIP_CONV', 'ldsfilter')
+    b = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
+    np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
+
+
 def test_conv_resident_filter_general_tail(capsys):
     # relu(conv(I, F) + R) with a full-size residual R: the tail is interpreted, not the fast store path
     shape, co = (3, 9, 30, 64), 64
