@@ -315,17 +315,17 @@ __global__ __launch_bounds__(kThreads) void conv_halo_kernel(IgemmArgs p) {
 // (HWCK, 2- or 4-byte elements).  The raw form is transposed on the way in: a task is a square of
 // kEpv K-indices x kEpv channels, read as kEpv 16-byte vectors along CO, turned in registers and
 // written as kEpv 16-byte vectors along K.
-template <int KIND>
+template <int KIND, int NT = kThreads>
 struct FilterStager {
   static constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
   static constexpr int krow = 9 * kPixBytes;
   static constexpr int vecs_per_row = krow / 16;
-  static constexpr int kFilterVecs = kBN * vecs_per_row / kThreads;
-  static_assert(kBN * vecs_per_row % kThreads == 0, "filter vectors divide evenly over the threads");
+  static constexpr int kFilterVecs = kBN * vecs_per_row / NT;
+  static_assert(kBN * vecs_per_row % NT == 0, "filter vectors divide evenly over the threads");
   static constexpr int kEpv = 16 / ES;  // elements per 16-byte vector
   static constexpr int kCoGroups = kBN / kEpv;
   static constexpr int kTasks = (krow / 16) * kCoGroups;
-  static constexpr int kTaskIters = (kTasks + kThreads - 1) / kThreads;
+  static constexpr int kTaskIters = (kTasks + NT - 1) / NT;
   static constexpr int kRawRegs = ES == 1 ? 1 : kTaskIters * kEpv;
   static constexpr int kFlRegs = kRawRegs > kFilterVecs ? kRawRegs : kFilterVecs;
   i32x4_t fl[kFlRegs];
@@ -334,18 +334,19 @@ struct FilterStager {
     if (ES != 1 && p.b_raw) {
 #pragma unroll
       for (int it = 0; it < kTaskIters; ++it) {
-        int task = tid + it * kThreads;
-        if (task >= kTasks) task = kTasks - 1;
-        const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
+        const int task = tid + it * NT;
+        if (task < kTasks) {
+          const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
 #pragma unroll
-        for (int kk = 0; kk < kEpv; ++kk)
-          fl[(it * kEpv + kk) % kFlRegs] =
-              *(const i32x4_t*)((const unsigned char*)p.Bt + ((int64_t)(kg * kEpv + kk) * kBN + cg * kEpv) * ES);
+          for (int kk = 0; kk < kEpv; ++kk)
+            fl[(it * kEpv + kk) % kFlRegs] =
+                *(const i32x4_t*)((const unsigned char*)p.Bt + ((int64_t)(kg * kEpv + kk) * kBN + cg * kEpv) * ES);
+        }
       }
     } else {
 #pragma unroll
       for (int k = 0; k < kFilterVecs; ++k) {
-        const int q = tid + k * kThreads;
+        const int q = tid + k * NT;
         const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
         const int co = 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3);
         fl[k] = *(const i32x4_t*)((const unsigned char*)p.Bt + (int64_t)co * p.ldbt * ES + vec * 16);
@@ -359,7 +360,8 @@ struct FilterStager {
     if (ES != 1 && p.b_raw) {
 #pragma unroll
       for (int it = 0; it < kTaskIters; ++it) {
-        const int task = tid + it * kThreads;
+        const int task = tid + it * NT;
+        if (task >= kTasks) break;
         const int kg = task / kCoGroups, cg = task - kg * kCoGroups;
         i32x4_t out[kEpv];
         if (ES == 4) {
@@ -379,19 +381,17 @@ struct FilterStager {
               out[(2 * w + 1) % kEpv][pr] = (int)((a >> 16) | (b2 & 0xffff0000u));
             }
         }
-        if (task < kTasks) {
 #pragma unroll
-          for (int e = 0; e < kEpv; ++e) {
-            const int co = cg * kEpv + e;
-            const int row = ((co >> 4) & 1) * 32 + ((co >> 2) & 3) * 8 + (co >> 5) * 4 + (co & 3);
-            *(i32x4_t*)(row_ptr(row) + kg * 16) = out[e];
-          }
+        for (int e = 0; e < kEpv; ++e) {
+          const int co = cg * kEpv + e;
+          const int row = ((co >> 4) & 1) * 32 + ((co >> 2) & 3) * 8 + (co >> 5) * 4 + (co & 3);
+          *(i32x4_t*)(row_ptr(row) + kg * 16) = out[e];
         }
       }
     } else {
 #pragma unroll
       for (int k = 0; k < kFilterVecs; ++k) {
-        const int q = tid + k * kThreads;
+        const int q = tid + k * NT;
         const int row = q / vecs_per_row, vec = q - row * vecs_per_row;
         *(i32x4_t*)(row_ptr(row) + vec * 16) = fl[k];
       }
@@ -758,8 +758,9 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
 // staging, no store phase): the window of tile t+1 arrives while tile t is computed.
 //
 // Window layout: pixel slot q = row * Wv + column (Wv = padded image width), 128 bytes each, rows
-// packed without gaps.  Slot q keeps its eight 16-byte channel vectors permuted: vector u sits at
-// position u ^ ((q >> 1) & 7), which spreads the 32 pixels of an operand read over all banks.
+// packed without gaps.  A slot keeps its eight 16-byte channel vectors permuted: vector u sits at
+// position u ^ ((column >> 1) & 7), which spreads the 32 pixels of an operand read over all banks
+// and, depending on the column only, is the same for the three taps of a filter column.
 // A wavefront-wide request (64 lanes x 16 bytes) fills 8 consecutive slots; requests are issued per
 // row in 8 groups of 8 columns, and a lane whose column is past the row's end fetches what belongs
 // into the slot it really writes, a pixel of the next row (written twice then, with the same bytes).
@@ -776,10 +777,17 @@ __host__ __device__ constexpr int reg_rows_low(int Wv) {
 __host__ __device__ constexpr int reg_bias_off(int Wv) { return 2 * reg_win_bytes(Wv) + (kBN - reg_rows_low(Wv)) * kRegBrow; }
 __host__ __device__ constexpr int reg_lds_bytes(int Wv) { return reg_bias_off(Wv) + kBN * 4; }
 
-template <int KIND>
-__global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p) {
+// WV: the padded image width if known at compile time (the row offsets of the taps then are
+// immediates of the LDS reads), 0 = taken from the arguments.
+// NI: 32-channel blocks per wavefront.  1: eight wavefronts (two per SIMD, 256 registers each), a
+// wavefront holds the filter of its 32 channels.  2: four wavefronts with 512 registers, each
+// holding the whole filter; one LDS read then feeds two MFMAs, but half of the filter sits in
+// accumulation registers and is copied out before use, which costs more than the reads saved.
+template <int KIND, int WV, int NI>
+__global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p) {
   static_assert(KIND != KIND_F32, "16-bit and 8-bit elements only");
-  constexpr int MI = 2, NI = 2;
+  constexpr int kNT = 512 / NI;
+  constexpr int MI = 2;
   constexpr int OES = KIND == KIND_BF16 ? 2 : 4;
   constexpr int kTaps = 9, kBlocks = kTaps * 4;  // K-blocks of 32 bytes
   typedef typename Acc<KIND>::type acc_t;
@@ -790,67 +798,64 @@ __global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pg = wave & 3;                   // the wavefront's 64 pixels of a tile
+  const int cb0 = NI == 1 ? wave >> 2 : 0;   // its first 32-channel block
   const int half = lane >> 5;
-  const int Hv = p.OH + 2, Wv = p.OW + 2;
+  const int Hv = p.OH + 2, Wv = WV ? WV : p.OW + 2;
   const int win_bytes = reg_win_bytes(Wv);
-#ifdef PML_CONV_TRACE
-  const long long t_entry = clock64();
-#endif
 
   const __amdgpu_buffer_rsrc_t rin =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)((int64_t)p.NB * p.H * p.W * kPixBytes), kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rout =
       __builtin_amdgcn_make_buffer_rsrc(p.C, 0, (int)(p.M * p.ldc * OES), kRsrcFlags);
 
-  // ---- window requests: wavefront w fills columns 8w .. 8w+7 and 8(w+4) .. 8(w+4)+7 of every row ----
+  // ---- window requests: a row is covered by 8 requests of 8 columns; wavefront w issues number w (+ 4) ----
   // Fixed for the kernel's life: a lane's column, whether that column is really one of the next row,
   // and its byte offset inside the input row (kFar where the slot is padding).
-  int req_px[2], req_col[2];
-  bool req_next[2];
+  int req_next[NI], req_col[NI];
 #pragma unroll
-  for (int c = 0; c < 2; ++c) {
-    req_px[c] = (wave + 4 * c) * 8 + (lane >> 3);
-    req_next[c] = req_px[c] >= Wv;
-    const int iw = req_px[c] - (req_next[c] ? Wv : 0) - p.PW;
-    req_col[c] = (unsigned)iw < (unsigned)p.W ? iw * kPixBytes : kFar;
+  for (int c = 0; c < NI; ++c) {
+    const int px = (wave + 4 * c) * 8 + (lane >> 3);
+    req_next[c] = px >= Wv ? -1 : 0;  // all ones: the lane's slot belongs to the next row
+    const int col = px - (Wv & req_next[c]), iw = col - p.PW;
+    const int vec = (lane & 7) ^ ((col >> 1) & 7);  // the input vector that belongs into this lane's 16 bytes of the slot
+    req_col[c] = (unsigned)iw < (unsigned)p.W ? iw * kPixBytes + vec * 16 : kFar;
   }
-  // rb_cur / rb_next: byte offset of input row r / r + 1 of the window, kFar for a row of padding
-  auto request = [&](unsigned char* win, int r, int c, int rb_cur, int rb_next) {
-    const int q = r * Wv + req_px[c];
-    const int vec = (lane & 7) ^ ((q >> 1) & 7);
-    const int voff = (req_next[c] ? rb_next : rb_cur) + req_col[c] + vec * 16;  // two kFar still are outside
+  // Lane r works out the input byte offset of window row r of a tile (kFar for rows of padding, rows
+  // past the tile's window and rows past the last image); the requests pick the rows up from there.
+  auto row_offsets = [&](const TileGeom& tg) {
+    int nb = tg.nb0, ihv = tg.ihv0 + lane;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {  // a window of kRegRows rows ends at most 3 images further on
+      const bool wrap = ihv >= Hv;
+      ihv -= wrap ? Hv : 0;
+      nb += wrap ? 1 : 0;
+    }
+    const int ih = ihv - p.PH;
+    const bool ok = lane < tg.nrows && nb < p.NB && (unsigned)ih < (unsigned)p.H;
+    return ok ? (nb * p.H + ih) * p.W * kPixBytes : kFar;
+  };
+  // rows: what row_offsets returned for the window's tile
+  auto request = [&](unsigned char* win, int r, int c, int rows) {
+    const int rb_cur = __builtin_amdgcn_readlane(rows, r), rb_next = __builtin_amdgcn_readlane(rows, r + 1);
+    const int voff = rb_cur + ((rb_next - rb_cur) & req_next[c]) + req_col[c];  // two kFar still are outside
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rin, PML_LDS(win + (r * Wv + (wave + 4 * c) * 8) * kPixBytes), 16, voff, 0, 0,
                                              0);
   };
-  // offset of window row r of a tile (row `ihv` of padded image `nb`), and the step to the row after it
-  auto row_offset = [&](int r, int nrows, int nb, int ihv) {
-    const int ih = ihv - p.PH;
-    const int ok = (int)(r < nrows) & (int)(nb < p.NB) & (int)((unsigned)ih < (unsigned)p.H);
-    const int real = (nb * p.H + ih) * p.W * kPixBytes;
-    return kFar ^ ((kFar ^ real) & -ok);
-  };
-  auto next_row = [&](int& nb, int& ihv) {
-    const int wrap = (int)(ihv + 1 == Hv);
-    ihv = (ihv + 1) & (wrap - 1);
-    nb += wrap;
-  };
 
+  FilterStager<KIND, kNT> filter;
+  filter.load(p, tid);
   int t = first_tile(blockIdx.x, gridDim.x);
   TileGeom g = tile_geom(p, t, Hv);
   unsigned char* const win0 = smem;
   unsigned char* const win1 = smem + win_bytes;
   {
     // the first window goes into the second buffer: the filter is staged around it
-    int nb = g.nb0, ihv = g.ihv0;
-    int rb_next = row_offset(0, g.nrows, nb, ihv);
+    const int rows = row_offsets(g);
 #pragma unroll
-    for (int r = 0; r < kRegRows; ++r) {
-      const int rb_cur = rb_next;
-      next_row(nb, ihv);
-      rb_next = row_offset(r + 1, g.nrows, nb, ihv);
-      request(win1, r, 0, rb_cur, rb_next);
-      request(win1, r, 1, rb_cur, rb_next);
-    }
+    for (int r = 0; r < kRegRows; ++r)
+#pragma unroll
+      for (int c = 0; c < NI; ++c) request(win1, r, c, rows);
   }
 
   // ---- filter -> LDS (transposed if raw) -> registers; initial values -> LDS ----
@@ -858,11 +863,7 @@ __global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p
   auto filter_row = [&](int row) {
     return smem + (row < rows_low ? row * kRegBrow : 2 * win_bytes + (row - rows_low) * kRegBrow);
   };
-  {
-    FilterStager<KIND> filter;
-    filter.load(p, tid);
-    filter.store(p, tid, filter_row);
-  }
+  filter.store(p, tid, filter_row);
   if (tid < kBN) {
     accs_t b = 0;
     if (p.init != nullptr) {
@@ -872,37 +873,44 @@ __global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p
     *(accs_t*)(smem + bias_off + tid * 4) = b;
   }
   __syncthreads();
+  // MFMA row 8q + 4h + e of channel block cb is given output channel 32cb + 16h + 4q + e, so that
+  // a lane (pixel, h) ends up owning the 16 consecutive channels 32cb + 16h .. + 15 in register order;
+  // the staged filter keeps that channel in row 32h + 8q + 4cb + e
   i32x4_t breg[kBlocks][NI];
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
-    const unsigned char* src = filter_row(j * 32 + (lane & 31)) + half * 16;
+    const int row = lane & 31;
+    const unsigned char* src = filter_row(((row >> 2) & 1) * 32 + (row >> 3) * 8 + 4 * (cb0 + j) + (row & 3)) + half * 16;
 #pragma unroll
     for (int s = 0; s < kBlocks; ++s) breg[s][j] = *(const i32x4_t*)(src + s * 32);
   }
-  const unsigned char* const bias_src = smem + bias_off + 32 * half * 4;
+  const int co0 = 32 * cb0 + 16 * half;  // first of the lane's 16 output channels in its first block
+  const unsigned char* const bias_src = smem + bias_off + co0 * 4;
 
   const float lo_f = p.tail_relu ? 0.f : -__builtin_inff();
   const int lo_i = p.tail_relu ? 0 : (int)0x80000000;
   const unsigned per = (unsigned)(p.OH * p.OW);
 
-  // where the pixel of this lane in half `i` of a tile sits: its window slot and its output byte offset
-  auto place = [&](const TileGeom& tg, int i, int& a_q, int& m_off) {
-    const unsigned m = (unsigned)tg.m0 + wave * 64 + i * 32 + (lane & 31);
+  // where the pixel of this lane in half `i` of a tile sits: byte offset of its window slot, its column
+  // and its output byte offset
+  auto place = [&](const TileGeom& tg, int i, int& a_q, int& a_ow, int& m_off) {
+    const unsigned m = (unsigned)tg.m0 + pg * 64 + i * 32 + (lane & 31);
     const bool ok = m < (unsigned)p.M;
     const unsigned mc = ok ? m : (unsigned)p.M - 1;
     const unsigned nb = fast_div(mc, p.div_per_magic, p.div_per_shift);
     const unsigned rem = mc - nb * per;
     const unsigned oh = fast_div(rem, p.div_ow_magic, p.div_ow_shift), ow = rem - oh * (unsigned)p.OW;
-    a_q = ((int)(nb * Hv + oh) - tg.v0) * Wv + (int)ow;
-    m_off = ok ? (int)((m * (unsigned)p.ldc + 32 * half) * OES) : (int)0x80000000;
+    a_q = (((int)(nb * Hv + oh) - tg.v0) * Wv + (int)ow) * kPixBytes;
+    a_ow = (int)ow;
+    m_off = ok ? (int)((m * (unsigned)p.ldc + co0) * OES) : (int)0x80000000;
   };
 
-  // one of the 8 pieces of a finished half tile: 4 consecutive channels of the lane's pixel
+  // one of the 4 NI pieces of a finished half tile: 4 consecutive channels of the lane's pixel
   // (bf16 output: two pieces share one 16-byte store)
   unsigned held[2] = {0, 0};
   auto finish_piece = [&](const acc_t (&acc)[NI], int m_off, int pc) {
     const int j = pc >> 2, q = pc & 3;
-    const int off = m_off + (j * 16 + 4 * q) * OES;
+    const int off = m_off + (32 * j + 4 * q) * OES;
     if (KIND == KIND_I8) {
       u32x4_t w;
 #pragma unroll
@@ -934,70 +942,76 @@ __global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p
   };
 
   // placement of the two halves of the current tile and of the tile after it
-  int a_q[MI], m_off[MI];
-  int a_next[MI], m_next[MI];
+  int a_q[MI], a_ow[MI], m_off[MI];
+  int a_next[MI], ow_next[MI], m_next[MI];
 
-  // K loop of half I of a tile (32 pixels x 64 channels per wavefront) out of window `cur`.  Two
-  // accumulator sets alternate between the halves, so the finished half rides along: its 8 pieces
+  // K loop of half I of a tile (32 pixels x 32 NI channels per wavefront) out of window `cur`.  Two
+  // accumulator sets alternate between the halves, so the finished half rides along: its pieces
   // (pacc, pm_off) sit between the MFMAs of this one.  Half 0 also carries the requests for the next
   // tile's window (geometry g2, into `nxt`), half 1 the placement of the next tile.  Past the last
   // tile every row is out of range and every request reads zeros, so none of this needs a branch.
   auto k_loop = [&](auto half_tag, acc_t (&acc)[NI], const unsigned char* cur, unsigned char* nxt,
                     const acc_t (&pacc)[NI], int pm_off, const TileGeom& g2) {
     constexpr int I = decltype(half_tag)::value;
-    int w_nb = g2.nb0, w_ihv = g2.ihv0;
-    int rb_cur = kFar, rb_next = I == 0 ? row_offset(0, g2.nrows, w_nb, w_ihv) : kFar;
-    // accumulators start from the initial values of the lane's channels
+    const int rows2 = I == 0 ? row_offsets(g2) : 0;
+    // the accumulators start from the initial values of the lane's channels
 #pragma unroll
     for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const acc4_t v = *(const acc4_t*)(bias_src + (16 * j + 4 * q) * 4);
+        const acc4_t v = *(const acc4_t*)(bias_src + (32 * j + 4 * q) * 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[j][4 * q + e] = v[e];
       }
     // Operand fragments are fetched kAhead K-blocks ahead.
     constexpr int kAhead = 2 * PML_CONV_AHEAD;
     i32x4_t fa[kAhead + 1];
+    // K-blocks run filter column by filter column (kw outermost): the four permuted vector offsets of
+    // a column serve its three taps, which differ by a uniform row offset only
+    int col_off[4] = {0, 0, 0, 0};
     auto fetch = [&](int s1) {
-      const int tap = s1 >> 2, ks = s1 & 3;
-      const int qt = a_q[I] + (tap / 3) * Wv + tap % 3;
-      const int vec16 = ((((qt >> 1) & 7) ^ half) << 4) ^ (ks << 5);  // vector 2*ks + half of the slot, permuted
-      fa[s1 % (kAhead + 1)] = *(const i32x4_t*)(cur + qt * kPixBytes + vec16);
+      const int ks = s1 & 3, kh = (s1 >> 2) % 3, kw = s1 / 12;
+      if (ks == 0 && kh == 0) {
+        const int key = ((((a_ow[I] + kw) >> 1) & 7) ^ half) << 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) col_off[k] = a_q[I] + kw * kPixBytes + (key ^ (k << 5));  // vector 2k + half
+      }
+      fa[s1 % (kAhead + 1)] = *(const i32x4_t*)(cur + col_off[ks] + kh * Wv * kPixBytes);
     };
 #pragma unroll
     for (int s0 = 0; s0 < kAhead; ++s0) fetch(s0);
 #pragma unroll
     for (int s = 0; s < kBlocks; ++s) {
+      asm volatile("" ::: "memory");  // LDS reads stay in the K-block they were put in
       if (s + kAhead < kBlocks) fetch(s + kAhead);
+      const int sb = (((s >> 2) % 3) * 3 + s / 12) * 4 + (s & 3);  // the K-block in the filter's own tap order
+      // the MFMAs are kept from sinking past the end of their K-block (the compiler's first instruction
+      // order otherwise gathers the pure MFMAs of a half behind all of its LDS reads)
 #pragma unroll
-      for (int j = 0; j < NI; ++j) mma_block<KIND>(acc[j], breg[s][j], fa[s % (kAhead + 1)]);
-      if (I == 0 && s < 2 * kRegRows) {  // the next tile's window, one request per K-block
-        if ((s & 1) == 0) {
-          rb_cur = rb_next;
-          next_row(w_nb, w_ihv);
-          rb_next = row_offset((s >> 1) + 1, g2.nrows, w_nb, w_ihv);
-        }
-        request(nxt, s >> 1, s & 1, rb_cur, rb_next);
+      for (int j = 0; j < NI; ++j) {
+        mma_block<KIND>(acc[j], breg[sb][j], fa[s % (kAhead + 1)]);
+        asm volatile("" ::"v"(acc[j][0]));
       }
-      if ((s & 3) == 1 && (s >> 2) < 8) finish_piece(pacc, pm_off, s >> 2);
-      if (I == 1 && s == 32) place(g2, 0, a_next[0], m_next[0]);
-      if (I == 1 && s == 34) place(g2, 1, a_next[1], m_next[1]);
-      // order inside the K-block: the LDS read and the window request first, then VALU work between the MFMAs
+      // the next tile's window, one request per K-block
+      if (I == 0 && s < NI * kRegRows) request(nxt, s / NI, s % NI, rows2);
+      if ((s % (8 / NI)) == 4 / NI && s / (8 / NI) < 4 * NI) finish_piece(pacc, pm_off, s / (8 / NI));
+      if (I == 1 && s == 32) place(g2, 0, a_next[0], ow_next[0], m_next[0]);
+      if (I == 1 && s == 34) place(g2, 1, a_next[1], ow_next[1], m_next[1]);
+      // order inside the K-block: the LDS read and the window request first, then the MFMAs with VALU work behind them
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
 #pragma unroll
-      for (int q = 0; q < NI; ++q) {
+      for (int j = 0; j < NI; ++j) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 12 / NI, 0);
       }
       __builtin_amdgcn_sched_barrier(0);  // keep requests and pieces in the K-block they were put in
     }
   };
 
   acc_t accX[NI], accY[NI];
-  place(g, 0, a_q[0], m_off[0]);
-  place(g, 1, a_q[1], m_off[1]);
+  place(g, 0, a_q[0], a_ow[0], m_off[0]);
+  place(g, 1, a_q[1], a_ow[1], m_off[1]);
   int m_last = (int)0x80000000;  // second half of the tile before: none precedes the first, its pieces are dropped
 #pragma unroll
   for (int j = 0; j < NI; ++j)
@@ -1007,30 +1021,18 @@ __global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p
 
   unsigned char* cur = win1;
   unsigned char* nxt = win0;
-#ifdef PML_CONV_TRACE
-  long long* trace = (long long*)p.outs[5];
-  int tn = 0;
-  const bool tracing = trace && blockIdx.x == 0 && lane == 0;
-#define PML_STAMP() do { if (tracing && tn < 60) trace[wave * 64 + tn++] = clock64(); } while (0)
-  if (tracing) { trace[wave * 64 + 59] = t_entry; trace[wave * 64 + 60] = clock64(); trace[wave * 64 + 62] = wall_clock64(); }
-#else
-#define PML_STAMP()
-#endif
   for (;;) {
     const int t2 = t + gridDim.x;
     const TileGeom g2 = tile_geom(p, t2, Hv);
-    PML_STAMP();
-    k_loop(std::integral_constant<int, 0>(), accX, cur, nxt, accY, m_last, g2);
-    PML_STAMP();
-    k_loop(std::integral_constant<int, 1>(), accY, cur, nxt, accX, m_off[0], g2);
-    PML_STAMP();
-    __syncthreads();  // every wavefront is done with the current window; the next one has arrived
-    PML_STAMP();
-    m_last = m_off[1];
+      k_loop(std::integral_constant<int, 0>(), accX, cur, nxt, accY, m_last, g2);
+      k_loop(std::integral_constant<int, 1>(), accY, cur, nxt, accX, m_off[0], g2);
+      __syncthreads();  // every wavefront is done with the current window; the next one has arrived
+      m_last = m_off[1];
     t = t2;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       a_q[i] = a_next[i];
+      a_ow[i] = ow_next[i];
       m_off[i] = m_next[i];
     }
     unsigned char* const w = cur;
@@ -1039,15 +1041,13 @@ __global__ __launch_bounds__(kThreads) void conv_regfilter3x3_kernel(IgemmArgs p
     if (t >= p.n_tiles) break;
   }
 #pragma unroll
-  for (int pc = 0; pc < 8; ++pc) finish_piece(accY, m_last, pc);
-#ifdef PML_CONV_TRACE
-  if (tracing) { trace[wave * 64 + 61] = clock64(); trace[wave * 64 + 63] = wall_clock64(); }
-#endif
+  for (int pc = 0; pc < 4 * NI; ++pc) finish_piece(accY, m_last, pc);
 }
 
-template <int KIND>
+template <int KIND, int WV>
 hipError_t launch_regfilter(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
-  auto kern = conv_regfilter3x3_kernel<KIND>;
+  constexpr int NI = 1;  // measured on the 128 x 56 x 56 x 64 case: 33.7 us against 42.7 us with NI = 2
+  auto kern = conv_regfilter3x3_kernel<KIND, WV, NI>;
   static size_t attr_lds = 0;
   if (lds > attr_lds) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1055,7 +1055,7 @@ hipError_t launch_regfilter(const IgemmArgs& a, size_t lds, int n_cus, hipStream
     attr_lds = lds;
   }
   const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512 / NI), lds, s, a);
   return hipGetLastError();
 }
 
@@ -1157,8 +1157,13 @@ hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int 
     }
   } else if (a.halo_variant == 3) {
     switch (kind) {
-      case KIND_BF16: return launch_regfilter<KIND_BF16>(a, lds_bytes, n_cus, s);
-      case KIND_I8: return launch_regfilter<KIND_I8>(a, lds_bytes, n_cus, s);
+      // 56-pixel rows (58 with padding) are compiled in
+      case KIND_BF16:
+        return a.OW + 2 == 58 ? launch_regfilter<KIND_BF16, 58>(a, lds_bytes, n_cus, s)
+                              : launch_regfilter<KIND_BF16, 0>(a, lds_bytes, n_cus, s);
+      case KIND_I8:
+        return a.OW + 2 == 58 ? launch_regfilter<KIND_I8, 58>(a, lds_bytes, n_cus, s)
+                              : launch_regfilter<KIND_I8, 0>(a, lds_bytes, n_cus, s);
     }
     return hipErrorInvalidValue;
   } else if (a.halo_variant == 2) {
