@@ -212,7 +212,7 @@ def resnet50_leg(E, batch=128, runs=5):
 
 def committed_traffic():
     """HBM bytes per launch of the bench kernel from the committed counter summary, or None."""
-    path = os.path.join(ROOT, 'profiles', 'conv_halo3x3_bf16_configs1_hbm_traffic.md')
+    path = os.path.join(ROOT, 'profiles', 'conv_regfilter3x3_bf16_configs1_hbm_traffic.md')
     try:
         for line in open(path):
             if line.startswith('traffic_bytes_per_launch'):
