@@ -69,15 +69,18 @@ struct Ring {
   static constexpr int kBytes = kStages * kStage;
 };
 
-// BM x BN output tile, WAVES_M x WAVES_N wavefront grid (WAVES_M * WAVES_N == 4).
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV>
-__global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
+// BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4 or 8 wavefronts (one or two per SIMD).
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads>
+__global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
-  constexpr int WAVES_N = 4 / WAVES_M;
+  constexpr int kWaves = NT / 64;
+  constexpr int kRowsPerPass = NT / 8;  // operand rows one load of all threads covers (8 lanes per 128-byte row)
+  constexpr int WAVES_N = kWaves / WAVES_M;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int MI = WM / 32, NI = WN / 32;
-  constexpr int A_VECS = BM * 8 / kThreads;  // 16-byte vectors per thread per slab
-  constexpr int B_VECS = BN * 8 / kThreads;
+  constexpr int A_VECS = BM * 8 / NT;  // 16-byte vectors per thread per slab
+  constexpr int B_VECS = BN * 8 / NT;
+  static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0, "tile sides are whole load passes");
   constexpr int kStage = Ring<BM, BN>::kStage;
   constexpr int kStages = Ring<BM, BN>::kStages;
   constexpr int kAhead = kStages - 1;              // slabs in flight ahead of the one being multiplied
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)kBufRange, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.Bt, 0, (int)kBufRange, kRsrcFlags);
 
-  // ---- per-thread load assignments (fixed across slabs): slot lv of rows lr + 32*i ----
+  // ---- per-thread load assignments (fixed across slabs): slot lv of rows lr + kRowsPerPass*i ----
   const int lv = tid & 7;
   const int lr = tid >> 3;
   const int lc = lv ^ ((lr >> 1) & 7);                        // the chunk of its row this thread fetches
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   int a_ih0[A_VECS], a_iw0[A_VECS];
 #pragma unroll
   for (int i = 0; i < A_VECS; ++i) {
-    const int64_t m = m0 + lr + 32 * i;
+    const int64_t m = m0 + lr + kRowsPerPass * i;
     const bool ok = m < p.M;
     const int64_t mm = ok ? m : 0;
     if (CONV) {
@@ -132,7 +135,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   unsigned b_off[B_VECS];
 #pragma unroll
   for (int i = 0; i < B_VECS; ++i) {
-    const int64_t n = n0 + lr + 32 * i;
+    const int64_t n = n0 + lr + kRowsPerPass * i;
     b_off[i] = n < p.N ? (unsigned)(n * p.ldbt * ES) : kOutside;
   }
 
@@ -178,17 +181,17 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
       } else {
         off = join_offsets(a_off[l], req_a);
       }
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, PML_LDS(req_base + l * 32 * kSlabBytes), 16, (int)off, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, PML_LDS(req_base + l * kRowsPerPass * kSlabBytes), 16, (int)off, 0, 0, 0);
     } else {
       const int i = l - A_VECS;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * 32) * kSlabBytes), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16,
                                                (int)join_offsets(b_off[i], req_b), 0, 0, 0);
     }
   };
 
   // a residual tensor of the tail is requested now, so that it arrives under the K loop
-  TailPrefetch<KIND, BM, BN, kThreads> pre;
-  tail_prefetch<KIND, BM, BN, kThreads>(p, m0, n0, tid, pre);
+  TailPrefetch<KIND, BM, BN, NT> pre;
+  tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
 
   acc_t acc[MI][NI];
 #pragma unroll
@@ -266,7 +269,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
   const int crow = lane & 31;
   const int ccol = (lane >> 5) * 4;
   if constexpr ((size_t)BM * (BN + 4) * 4 <= (size_t)Ring<BM, BN>::kBytes) {
-    // the whole tile fits in the pipeline buffers: ctile[BM][BN + 4], tail by all 256 threads
+    // the whole tile fits in the pipeline buffers: ctile[BM][BN + 4], tail by all threads
     constexpr int CS = BN + 4;
     accs_t* ctile = (accs_t*)smem;
 #pragma unroll
@@ -281,12 +284,12 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(IgemmArgs p) {
           *(acc4_t*)&ctile[(wm * WM + i * 32 + crow) * CS + wn * WN + j * 32 + 8 * g + ccol] = q;
         }
     __syncthreads();
-    tile_tail<KIND, BM, BN, kThreads>(p, ctile, m0, n0, tid, &pre);
+    tile_tail<KIND, BM, BN, NT>(p, ctile, m0, n0, tid, &pre);
   } else {
     // large tiles: every wavefront stages RB of its 32-row blocks at a time in a private
     // region, wtile[RB * 32][WN + 4], and runs the tail over them with its 64 lanes
     constexpr int CS = WN + 4;
-    constexpr int kBudget = Ring<BM, BN>::kBytes / 4 / 16 * 16;  // bytes per wavefront
+    constexpr int kBudget = Ring<BM, BN>::kBytes / kWaves / 16 * 16;  // bytes per wavefront
     constexpr int kFit = kBudget / (32 * CS * 4);
     constexpr int RB = kFit >= MI ? MI : (kFit >= 4 ? 4 : (kFit >= 2 ? 2 : 1));  // MI is a power of two
     static_assert(RB >= 1 && MI % RB == 0, "row blocks must stage evenly");
@@ -329,30 +332,30 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ B,
   }
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const size_t lds = Ring<BM, BN>::kBytes;
-  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV>;
+  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kThreads), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), lds, s, a);
   return hipGetLastError();
 }
 
 template <int KIND, bool CONV>
 hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
   switch (cfg) {
-    case TILE_128x128: return launch_cfg<KIND, 128, 128, 2, CONV>(a, s);
-    case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
-    case TILE_256x64: return launch_cfg<KIND, 256, 64, 4, CONV>(a, s);
     case TILE_64x64: return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);
-    case TILE_256x128: return launch_cfg<KIND, 256, 128, 2, CONV>(a, s);
-    case TILE_256x256: return launch_cfg<KIND, 256, 256, 2, CONV>(a, s);
+    case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
+    case TILE_128x128: return launch_cfg<KIND, 128, 128, 2, CONV>(a, s);
+    case TILE_128x64_W8: return launch_cfg<KIND, 128, 64, 4, CONV, 512>(a, s);
+    case TILE_128x128_W8: return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
+    case TILE_256x128_W16: return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
   }
   return hipErrorInvalidValue;
 }

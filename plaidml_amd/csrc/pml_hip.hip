@@ -75,41 +75,53 @@ int mfma_kind_of(int in_dtype) {
 
 const char* tile_name(int t) {
   switch (t) {
-    case TILE_128x128: return "128x128";
-    case TILE_128x64: return "128x64";
-    case TILE_256x64: return "256x64";
     case TILE_64x64: return "64x64";
-    case TILE_256x128: return "256x128";
-    case TILE_256x256: return "256x256";
+    case TILE_128x64: return "128x64";
+    case TILE_128x128: return "128x128";
+    case TILE_128x64_W8: return "128x64 (8 wavefronts)";
+    case TILE_128x128_W8: return "128x128 (8 wavefronts)";
+    case TILE_256x128_W16: return "256x128 (16 wavefronts)";
   }
   return "?";
 }
 
-// Stated tiling choice per shape class (k_bytes = bytes of K per row).  Measured on MI355X (us):
-//   4096^3 bf16 / int8:             256x256 131 / 80, 256x128 147 / 92, 128x64 173 / 107, 128x128 189 / 115
-//   conv 128x28x28x128 (*) 3x3x128: 64x64 73, 128x64 79, 256x128 100, 128x128 104
-//   conv 128x14x14x256 (*) 3x3x256: 64x64 70, 128x64 71, 256x128 75, 128x128 78
-//   conv 128x7x7x512   (*) 3x3x512: 128x64 64, 128x128 65, 64x64 78, 256x128 113
-//   gemm 401408x256x64 bf16:        64x64 142, 128x64 166, 128x128 278
-//   gemm 25088x1024x256 bf16:       64x64 51, 128x64 57, 128x128 90
-// One tile per workgroup and a serial load / multiply / store life per tile: what hides latency is
-// how many workgroups fit a CU (64x64: 5, 128x64: 2, larger: 1).  So: long K with enough 256x256
-// tiles to fill the chip takes the big tile (least operand traffic per MFMA); otherwise the smaller
-// of 64x64 and 128x64 by (rounds of resident workgroups) x (tile area), the larger tile on a tie.
+// Stated tiling choice per shape class.  Measured on MI355X, bf16 unless said otherwise (us; w8 / w16 =
+// 8 / 16 wavefronts per workgroup, i.e. 2 / 4 per SIMD; the 4-wavefront 256x128 and 256x256 tiles that
+// were tried as well are slower than 256x128w16 everywhere and are no longer built):
+//                                    64x64  128x64  128x64w8  128x128  128x128w8  256x128w16
+//   4096^3 (int8)                        -       -       117      119       110          83
+//   4096^3                               -       -       169      173       161         107
+//   conv 128x28x28x128 (*) 3x3x128      66      76        75       89        72          53
+//   conv 128x14x14x256 (*) 3x3x256      66      72        75       73        62          46
+//   conv 128x7x7x512   (*) 3x3x512      72      67        73       64        57          78
+//   gemm 401408x256x64                  82     127        93      177       113          78
+//   gemm 401408x64x256                  47      55        45        -         -           -
+//   gemm 100352x512x128                 52      71        54      100        66          49
+//   gemm 25088x256x1024                 27      27        25       30        24          22
+//   gemm 6272x512x2048                  25      23        22       25        21          28
+//   gemm 23104x728x728                  72      67        61       78        63          57
+//   gemm 1024^3 (fp32)                  33      45        41       77        71         127
+// One tile per workgroup and a serial load / multiply / store life per tile: latency is hidden by the
+// other wavefronts of a SIMD, and more of them per workgroup do that better than more workgroups of four.
+// So: the 256x128 tile with 16 wavefronts whenever it yields enough workgroups to occupy most CUs, the
+// 128x128 one with 8 below that, and for small problems the smaller of 64x64 and 128x64 by (rounds of
+// resident workgroups) x (tile area), the larger tile on a tie.
 int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
-  // PML_HIP_TILE=128x128|128x64|256x64|64x64|256x128|256x256 overrides the table (for tuning runs)
+  (void)k_bytes;
+  // PML_HIP_TILE=64x64|128x64|128x128|128x64w8|128x128w8|256x128w16 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
     const std::string v(e);
-    if (v == "128x128") return TILE_128x128;
-    if (v == "128x64") return TILE_128x64;
-    if (v == "256x64" && n <= 64) return TILE_256x64;
     if (v == "64x64") return TILE_64x64;
-    if (v == "256x128") return TILE_256x128;
-    if (v == "256x256") return TILE_256x256;
+    if (v == "128x64") return TILE_128x64;
+    if (v == "128x128") return TILE_128x128;
+    if (v == "128x64w8") return TILE_128x64_W8;
+    if (v == "128x128w8") return TILE_128x128_W8;
+    if (v == "256x128w16") return TILE_256x128_W16;
   }
-  auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-  if (n <= 64) return TILE_64x64;
-  if (k_bytes >= 4096 && tiles(256, 256) >= 128) return TILE_256x256;
+  auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+  if (n <= 64) return tiles(128, 64) >= 1024 ? TILE_128x64_W8 : TILE_64x64;
+  if (tiles(256, 128) >= 160) return TILE_256x128_W16;
+  if (tiles(128, 128) >= 128) return TILE_128x128_W8;
   const int64_t rounds_small = (tiles(64, 64) + 5 * 256 - 1) / (5 * 256);
   const int64_t rounds_wide = (tiles(128, 64) + 2 * 256 - 1) / (2 * 256);
   return rounds_small < 2 * rounds_wide ? TILE_64x64 : TILE_128x64;
