@@ -243,7 +243,16 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
   // columns are fetched once; every step rounds to the result type like the interpreter does.
   if (KIND != KIND_I8 && p.tail_mode == 3 && full4 && (p.ldc & 3) == 0) {
     const bool bf = p.out_dtype == PML_HIP_BF16;
-    auto rnd = [&](float x) { return bf ? __uint_as_float(f32_to_bf16_bits(x) << 16) : x; };
+    // rounding to the result type: the hardware conversion (round to nearest even, NaN quieted)
+    auto rnd = [&](float x) {
+      if (!bf) return x;
+      typedef float f32x2 __attribute__((ext_vector_type(2)));
+      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+      const bf16x2 h = __builtin_convertvector(f32x2{x, 0.f}, bf16x2);
+      uint32_t w;
+      __builtin_memcpy(&w, &h, 4);
+      return __uint_as_float(w << 16);
+    };
     float xs[4][4];
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
@@ -274,54 +283,75 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
         }
       }
     }
-    for (int row = row0; row < BM; row += RPP) {
-      const int64_t m = m0 + row;
-      if (m >= p.M) break;
-      float v[4];
+    // rows in batches of up to 8: all LDS reads of a batch are issued before the first value is used,
+    // and a step's opcode is decoded once per batch instead of once per element
+    constexpr int kRowsPerThread = (BM + RPP - 1) / RPP;
+    constexpr int RB = kRowsPerThread < 8 ? kRowsPerThread : 8;
+    for (int rowb = row0; rowb < BM; rowb += RB * RPP) {
+      float v[RB][4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = (float)ctile[row * CS + c4 + q] + (float)cinit[q];
-      if (p.init && !col_init) {
+      for (int r = 0; r < RB; ++r) {
+        const int row = rowb + r * RPP;
+        const int rr = row < BM ? row : BM - 1;
+        if constexpr (sizeof(accs_t) == 4) {
+          typedef accs_t acc4_t __attribute__((ext_vector_type(4)));
+          const acc4_t c = *(const acc4_t*)&ctile[rr * CS + c4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          Scalar<float, int> b = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
-          v[q] += b.f;
+          for (int q = 0; q < 4; ++q) v[r][q] = (float)c[q] + (float)cinit[q];
         }
       }
+      if (p.init && !col_init) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = rnd(v[q]);
+        for (int r = 0; r < RB; ++r) {
+          const int64_t m = m0 + rowb + r * RPP;
+          if (rowb + r * RPP < BM && m < p.M) {
 #pragma unroll
-      for (int st = 0; st < 4; ++st) {
-        if (st < p.tail.n_ops) {
-          const int opc = p.tail.ops[st].opcode;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float a = v[q], b = xs[st][q];
-            float r = a;
-            switch (opc) {
-              case PML_HIP_EPI_ADD: r = a + b; break;
-              case PML_HIP_EPI_SUB: r = a - b; break;
-              case PML_HIP_EPI_RSUB: r = b - a; break;
-              case PML_HIP_EPI_MUL: r = a * b; break;
-              case PML_HIP_EPI_DIV: r = a / b; break;
-              case PML_HIP_EPI_RDIV: r = b / a; break;
-              case PML_HIP_EPI_MAX: r = (a < b) ? b : a; break;
-              case PML_HIP_EPI_MIN: r = (a < b) ? a : b; break;
-              case PML_HIP_EPI_RELU: r = (a < 0.f) ? 0.f : a; break;
-              case PML_HIP_EPI_NEG: r = -a; break;
-              case PML_HIP_EPI_MAX_GT: r = (a > b) ? a : b; break;
-              default: break;
+            for (int q = 0; q < 4; ++q) {
+              Scalar<float, int> b = load_scalar<float, int>(p.init, m * p.init_rs + (n + q) * p.init_cs, p.init_dtype);
+              v[r][q] += b.f;
             }
-            v[q] = rnd(r);
           }
         }
       }
-      if (bf) {
-        const uint32_t h0 = __float_as_uint(v[0]) >> 16, h1 = __float_as_uint(v[1]) >> 16;
-        const uint32_t h2 = __float_as_uint(v[2]) >> 16, h3 = __float_as_uint(v[3]) >> 16;
-        *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h0 | (h1 << 16), h2 | (h3 << 16));
-      } else {
-        const f32x4_t w = {v[0], v[1], v[2], v[3]};
-        *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
+      auto each = [&](int st, auto fn) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[r][q] = rnd(fn(v[r][q], xs[st][q]));
+      };
+      each(0, [](float a, float) { return a; });  // the contraction's own result, rounded to the result type
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        if (st < p.tail.n_ops) {
+          switch (p.tail.ops[st].opcode) {
+            case PML_HIP_EPI_ADD: each(st, [](float a, float b) { return a + b; }); break;
+            case PML_HIP_EPI_SUB: each(st, [](float a, float b) { return a - b; }); break;
+            case PML_HIP_EPI_RSUB: each(st, [](float a, float b) { return b - a; }); break;
+            case PML_HIP_EPI_MUL: each(st, [](float a, float b) { return a * b; }); break;
+            case PML_HIP_EPI_DIV: each(st, [](float a, float b) { return a / b; }); break;
+            case PML_HIP_EPI_RDIV: each(st, [](float a, float b) { return b / a; }); break;
+            case PML_HIP_EPI_MAX: each(st, [](float a, float b) { return (a < b) ? b : a; }); break;
+            case PML_HIP_EPI_MIN: each(st, [](float a, float b) { return (a < b) ? a : b; }); break;
+            case PML_HIP_EPI_RELU: each(st, [](float a, float) { return (a < 0.f) ? 0.f : a; }); break;
+            case PML_HIP_EPI_NEG: each(st, [](float a, float) { return -a; }); break;
+            case PML_HIP_EPI_MAX_GT: each(st, [](float a, float b) { return (a > b) ? a : b; }); break;
+            default: break;
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const int row = rowb + r * RPP;
+        const int64_t m = m0 + row;
+        if (row >= BM || m >= p.M) continue;
+        if (bf) {
+          const uint32_t h0 = __float_as_uint(v[r][0]) >> 16, h1 = __float_as_uint(v[r][1]) >> 16;
+          const uint32_t h2 = __float_as_uint(v[r][2]) >> 16, h3 = __float_as_uint(v[r][3]) >> 16;
+          *(uint2*)((uint16_t*)p.C + m * p.ldc + n) = make_uint2(h0 | (h1 << 16), h2 | (h3 << 16));
+        } else {
+          const f32x4_t w = {v[r][0], v[r][1], v[r][2], v[r][3]};
+          *(f32x4_t*)((float*)p.C + m * p.ldc + n) = w;
+        }
       }
     }
     return;

@@ -102,25 +102,48 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
     const int64_t n = t / d.oh;
     const int64_t c0 = cv * V;
     float acc[V];
+    int best[V];  // with_index: largest window index whose (in-range) tap equals the pooled value; 0 if none
     const float ident = d.agg == PML_HIP_AGG_MAX ? -INFINITY : (d.agg == PML_HIP_AGG_MIN ? INFINITY : 0.f);
 #pragma unroll
-    for (int i = 0; i < V; ++i) acc[i] = ident;
-    for (int ky = 0; ky < d.kh; ++ky) {
-      const int64_t iy = (int64_t)oy * d.stride_h + ky - d.pad_h;
-      if (iy < 0 || iy >= d.h) continue;
-      for (int kx = 0; kx < d.kw; ++kx) {
-        const int64_t ix = (int64_t)ox * d.stride_w + kx - d.pad_w;
-        if (ix < 0 || ix >= d.w) continue;
-        float x[V];
-        VecIO<ES>::load(a.in, ((n * d.h + iy) * d.w + ix) * d.c + c0, x);
+    for (int i = 0; i < V; ++i) {
+      acc[i] = ident;
+      best[i] = 0;
+    }
+    // The window is walked in groups of kGroup taps: all loads of a group are issued (taps outside the
+    // image read the tensor's first vector and are ignored) before the first value is used, so a
+    // thread has kGroup loads in flight instead of one.
+    constexpr int kGroup = 9;
+    const int taps = (int)(d.kh * d.kw);
+    const int64_t iy0 = (int64_t)oy * d.stride_h - d.pad_h, ix0 = (int64_t)ox * d.stride_w - d.pad_w;
+    int ky = 0, kx = 0;
+    for (int k0 = 0; k0 < taps; k0 += kGroup) {
+      float x[kGroup][V];
+      bool ok[kGroup];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const int64_t iy = iy0 + ky, ix = ix0 + kx;
+        ok[u] = k0 + u < taps && iy >= 0 && iy < d.h && ix >= 0 && ix < d.w;
+        VecIO<ES>::load(a.in, ok[u] ? ((n * d.h + iy) * d.w + ix) * d.c + c0 : 0, x[u]);
+        if (++kx == d.kw) {
+          kx = 0;
+          ++ky;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        if (!ok[u]) continue;
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          if (d.agg == PML_HIP_AGG_MAX)
-            acc[i] = (x[i] > acc[i]) ? x[i] : acc[i];
-          else if (d.agg == PML_HIP_AGG_MIN)
-            acc[i] = (x[i] < acc[i]) ? x[i] : acc[i];
-          else
-            acc[i] += x[i];
+          if (d.agg == PML_HIP_AGG_MAX) {
+            // taps come in rising window index, so ">=" leaves the largest index among equal values
+            best[i] = (x[u][i] >= acc[i]) ? k0 + u : best[i];
+            acc[i] = (x[u][i] > acc[i]) ? x[u][i] : acc[i];
+          } else if (d.agg == PML_HIP_AGG_MIN) {
+            best[i] = (x[u][i] <= acc[i]) ? k0 + u : best[i];
+            acc[i] = (x[u][i] < acc[i]) ? x[u][i] : acc[i];
+          } else {
+            acc[i] += x[u][i];
+          }
         }
       }
     }
@@ -134,26 +157,6 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
       store_scalar<float, int>(a.out, o0 + i, dt, v);
     }
     if (d.with_index) {
-      // largest window index whose (in-range) tap equals the pooled value; 0 if none
-      int best[V];
-#pragma unroll
-      for (int i = 0; i < V; ++i) best[i] = 0;
-      for (int ky = 0; ky < d.kh; ++ky) {
-        const int64_t iy = (int64_t)oy * d.stride_h + ky - d.pad_h;
-        if (iy < 0 || iy >= d.h) continue;
-        for (int kx = 0; kx < d.kw; ++kx) {
-          const int64_t ix = (int64_t)ox * d.stride_w + kx - d.pad_w;
-          if (ix < 0 || ix >= d.w) continue;
-          float x[V];
-          VecIO<ES>::load(a.in, ((n * d.h + iy) * d.w + ix) * d.c + c0, x);
-          const int k = ky * (int)d.kw + kx;
-#pragma unroll
-          for (int i = 0; i < V; ++i) {
-            const int cand = (x[i] == acc[i]) ? k : 0;
-            best[i] = cand > best[i] ? cand : best[i];
-          }
-        }
-      }
       int32_t* ip = (int32_t*)a.idx + o0;
 #pragma unroll
       for (int i = 0; i < V; i += 4) {
