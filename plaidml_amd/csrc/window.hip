@@ -7,6 +7,8 @@
 // byte about once.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "device_common.h"
 #include "plans.h"
 
@@ -56,20 +58,48 @@ __global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t tot
     float acc[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) acc[i] = 0.f;
-    for (int ky = 0; ky < d.kh; ++ky) {
-      const int64_t iy = (int64_t)oy * d.stride_h + (int64_t)ky * d.dil_h - d.pad_h;
-      if (iy < 0 || iy >= d.h) continue;
-      for (int kx = 0; kx < d.kw; ++kx) {
-        const int64_t ix = (int64_t)ox * d.stride_w + (int64_t)kx * d.dil_w - d.pad_w;
-        if (ix < 0 || ix >= d.w) continue;
-        float x[V], w[V];
-        VecIO<ES>::load(a.in, ((n * d.h + iy) * d.w + ix) * d.c + c0, x);
-        VecIO<ES>::load(a.filter, ((int64_t)ky * d.kw + kx) * d.c + c0, w);
+    // The taps are walked in groups of kGroup: all loads of a group (input and filter; taps outside
+    // the image read the tensor's first vector and are ignored) are issued before the first product.
+    constexpr int kGroup = 9;
+    const int taps = (int)(d.kh * d.kw);
+    const int64_t iy0 = (int64_t)oy * d.stride_h - d.pad_h, ix0 = (int64_t)ox * d.stride_w - d.pad_w;
+    int ky = 0, kx = 0;
+    for (int k0 = 0; k0 < taps; k0 += kGroup) {
+      float x[kGroup][V], w[kGroup][V];
+      bool ok[kGroup];
 #pragma unroll
-        for (int i = 0; i < V; ++i) acc[i] += x[i] * w[i];
+      for (int u = 0; u < kGroup; ++u) {
+        const int64_t iy = iy0 + (int64_t)ky * d.dil_h, ix = ix0 + (int64_t)kx * d.dil_w;
+        ok[u] = k0 + u < taps && iy >= 0 && iy < d.h && ix >= 0 && ix < d.w;
+        VecIO<ES>::load(a.in, ok[u] ? ((n * d.h + iy) * d.w + ix) * d.c + c0 : 0, x[u]);
+        VecIO<ES>::load(a.filter, ok[u] ? (int64_t)(k0 + u) * d.c + c0 : 0, w[u]);
+        if (++kx == d.kw) {
+          kx = 0;
+          ++ky;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        if (!ok[u]) continue;
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] += x[u][i] * w[u][i];
       }
     }
     const int64_t o0 = pix * d.c + c0;
+    if (d.tail.n_ops == 0 && (dt == PML_HIP_BF16 || dt == PML_HIP_F32)) {
+      // no tail: one 16-byte store of the rounded values
+      if constexpr (ES == 2) {
+        i32x4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[2 * i + 1]) << 16));
+        *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+      } else {
+        const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
+        *(f32x4_t*)((float*)a.out + o0) = o;
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       Scalar<float, int> v;
@@ -82,6 +112,104 @@ __global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t tot
         off[q] = q < d.tail.n_operands ? pix * d.tail.operand_row_stride[q] + (c0 + i) * d.tail.operand_col_stride[q] : 0;
       v = run_tail<float, int>(d.tail, v, &cur, a.operands, off, a.outs, o0 + i);
       store_scalar<float, int>(a.out, o0 + i, cur, v);
+    }
+  }
+}
+
+// 3x3 depthwise convolution, unit stride and dilation, no tail: a thread computes kDwPx neighbouring
+// output pixels of a row for one 16-byte channel vector, so the three rows of kDwPx + 2 input vectors
+// it loads serve all of them and the nine filter vectors are loaded once (27 loads for 4 outputs
+// instead of 72).  A tap outside the image takes no part in the sum (it is not multiplied by zero).
+constexpr int kDwPx = 4;
+template <int ES>
+__global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t total) {
+  constexpr int V = VecIO<ES>::V;
+  const pml_hip_dwconv2d_desc& d = a.d;
+  const int64_t cvecs = d.c / V;
+  const int64_t xblocks = (d.ow + kDwPx - 1) / kDwPx;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
+    const int64_t cv = g % cvecs;
+    int64_t t = g / cvecs;
+    const int ox0 = (int)(t % xblocks) * kDwPx;
+    t /= xblocks;
+    const int oy = (int)(t % d.oh);
+    const int64_t n = t / d.oh;
+    const int64_t c0 = cv * V;
+    i32x4_t xr[3][kDwPx + 2], wr[9];
+    bool ok[3][kDwPx + 2];
+    bool all_ok = true;
+#pragma unroll
+    for (int k = 0; k < 9; ++k) wr[k] = *(const i32x4_t*)((const unsigned char*)a.filter + ((int64_t)k * d.c + c0) * ES);
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+      const int64_t iy = (int64_t)oy + ky - d.pad_h;
+#pragma unroll
+      for (int c = 0; c < kDwPx + 2; ++c) {
+        const int64_t ix = (int64_t)ox0 + c - d.pad_w;
+        ok[ky][c] = iy >= 0 && iy < d.h && ix >= 0 && ix < d.w;
+        all_ok = all_ok && ok[ky][c];
+        const int64_t off = ok[ky][c] ? ((n * d.h + iy) * d.w + ix) * d.c + c0 : 0;
+        xr[ky][c] = *(const i32x4_t*)((const unsigned char*)a.in + off * ES);
+      }
+    }
+    auto unpack = [](const i32x4_t& raw, float* f) {
+      if constexpr (ES == 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          f[2 * i] = __uint_as_float(((uint32_t)raw[i]) << 16);
+          f[2 * i + 1] = __uint_as_float(((uint32_t)raw[i]) & 0xffff0000u);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __int_as_float(raw[i]);
+      }
+    };
+    float acc[kDwPx][V];
+#pragma unroll
+    for (int px = 0; px < kDwPx; ++px)
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[px][i] = 0.f;
+    // taps in the reference's order (ky outer, kx inner) for every pixel
+    auto accumulate = [&](auto checked) {
+#pragma unroll
+      for (int ky = 0; ky < 3; ++ky) {
+        float w[3][V];
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) unpack(wr[ky * 3 + kx], w[kx]);
+#pragma unroll
+        for (int c = 0; c < kDwPx + 2; ++c) {
+          if (decltype(checked)::value && !ok[ky][c]) continue;
+          float x[V];
+          unpack(xr[ky][c], x);
+#pragma unroll
+          for (int kx = 0; kx < 3; ++kx) {
+            const int px = c - kx;
+            if (px < 0 || px >= kDwPx) continue;
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[px][i] += x[i] * w[kx][i];
+          }
+        }
+      }
+    };
+    if (all_ok)
+      accumulate(std::false_type());
+    else
+      accumulate(std::true_type());
+#pragma unroll
+    for (int px = 0; px < kDwPx; ++px) {
+      if (ox0 + px >= d.ow) break;
+      const int64_t o0 = ((n * d.oh + oy) * d.ow + ox0 + px) * d.c + c0;
+      if constexpr (ES == 2) {
+        i32x4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[px][2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[px][2 * i + 1]) << 16));
+        *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+      } else {
+        const f32x4_t o = {acc[px][0], acc[px][1], acc[px][2], acc[px][3]};
+        *(f32x4_t*)((float*)a.out + o0) = o;
+      }
     }
   }
 }
@@ -260,6 +388,15 @@ hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
   const int V = 16 / es;
   const int64_t total = d.n * d.oh * d.ow * (d.c / V);
   if (total == 0) return hipSuccess;
+  if (d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.dil_h == 1 && d.dil_w == 1 && d.tail.n_ops == 0 &&
+      (d.dtype == PML_HIP_BF16 || d.dtype == PML_HIP_F32)) {
+    const int64_t total4 = d.n * d.oh * ((d.ow + kDwPx - 1) / kDwPx) * (d.c / V);
+    if (es == 2)
+      hipLaunchKernelGGL((dwconv3x3_kernel<2>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
+    else
+      hipLaunchKernelGGL((dwconv3x3_kernel<4>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
+    return hipGetLastError();
+  }
   if (es == 2)
     hipLaunchKernelGGL((dwconv2d_kernel<2>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
   else

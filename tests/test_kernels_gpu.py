@@ -385,6 +385,49 @@ def test_conv_few_channel_patch_matrix(kind, stride, capsys, monkeypatch):
     assert 'patch matrix' in capsys.readouterr().out
 
 
+# (dtype, N, H, W, C, k, stride, pad): the 3x3 unit-stride kernel that computes four pixels per thread (widths
+# that are and are not multiples of four, SAME and VALID windows, an infinity in the filter that a padded tap
+# must not turn into NaN) and the general one (5x5, stride 2)
+DW_CASES = [('bf16', 2, 19, 19, 32, 3, 1, 1), ('bf16', 1, 9, 24, 16, 3, 1, 0), ('f32', 2, 11, 13, 8, 3, 1, 1),
+            ('bf16', 1, 12, 15, 16, 5, 1, 2), ('f32', 1, 14, 14, 8, 3, 2, 1)]
+
+
+@pytest.mark.parametrize('kind,N,H,W,C,k,stride,pad', DW_CASES)
+def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad):
+    rng = np.random.default_rng(90)
+    Iv = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    Fv = (rng.standard_normal((k, k, C, 1)) * 0.3).astype(np.float32)
+    if k == 3 and stride == 1 and pad == 1:
+        Fv[0, 0, 0, 0] = np.inf  # only pixels whose top-left tap lies inside the image see it
+    if kind == 'bf16':
+        Iv, Fv = E.round_bf16(Iv), E.round_bf16(Fv)
+    OH, OW = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    d = hk.Dwconv2dDesc()
+    d.dtype = hk.BF16 if kind == 'bf16' else hk.F32
+    d.n, d.h, d.w, d.c, d.kh, d.kw, d.oh, d.ow = N, H, W, C, k, k, OH, OW
+    d.stride_h = d.stride_w = stride
+    d.dil_h = d.dil_w = 1
+    d.pad_h = d.pad_w = pad
+    plan = hk.lib().pml_hip_dwconv2d_dispatch(ctypes.byref(d))
+    assert plan, hk.lib().pml_hip_last_error()
+    es = 2 if kind == 'bf16' else 4
+    dI = hk.DeviceBuffer.from_numpy(bf16(Iv) if kind == 'bf16' else Iv)
+    dF = hk.DeviceBuffer.from_numpy(bf16(Fv) if kind == 'bf16' else Fv)
+    dO = hk.DeviceBuffer(N * OH * OW * C * es)
+    hk.check(hk.lib().pml_hip_dwconv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, hk.ptr_array([]), hk.ptr_array([]), None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    out = dO.to_numpy(np.uint16 if kind == 'bf16' else np.float32, (N, OH, OW, C))
+    if kind == 'bf16':
+        out = E.bf16_from_bits(out)
+    dt = D.BFLOAT16 if kind == 'bf16' else D.FLOAT32
+    I, F = E.Placeholder(dt, Iv.shape), E.Placeholder(dt, Fv.shape)
+    O = op.convolution(I, F, strides=[stride, stride], autopad=op.EXPLICIT, manual_padding=[pad, pad], depthwise=True)
+    ref, = E.run(E.Program('dw', [I, F], [O]), [Iv, Fv])
+    assert np.isinf(ref).any() == (k == 3 and stride == 1 and pad == 1) and not np.isnan(ref).any()
+    np.testing.assert_allclose(out, ref, rtol=BF16_RTOL if kind == 'bf16' else FP32_RTOL, atol=1e-2 if kind == 'bf16' else 1e-4)
+    hk.lib().pml_hip_plan_free(plan)
+
+
 def test_dwconv_pool_bf16():
     rng = np.random.default_rng(9)
     N, H, W, C = 2, 19, 19, 32
