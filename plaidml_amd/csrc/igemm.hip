@@ -332,6 +332,36 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ B,
   }
 }
 
+// The same for one-byte elements without LDS: a thread takes 16 K-rows x 4 N-columns as 16 dwords,
+// turns the four 4x4 byte blocks in registers (v_perm_b32) and writes 16 bytes of K to each of its four
+// Bt rows.  A wavefront covers 64 x 64 elements: 64-byte runs on both sides.
+// K % 16 == 0, N % 4 == 0, ldb % 4 == 0, ldbt % 16 == 0, B 4-byte and Bt 16-byte aligned.
+__global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __restrict__ B, uint8_t* __restrict__ Bt,
+                                                              int64_t K, int64_t N, int64_t ldb, int64_t ldbt) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t n = ((int64_t)blockIdx.x * 4 + wave) * 64 + 4 * (lane & 15);
+  const int64_t k = (int64_t)blockIdx.y * 64 + 16 * (lane >> 4);
+  if (n >= N || k >= K) return;
+  unsigned r[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r[i] = *(const unsigned*)(B + (k + i) * ldb + n);
+  i32x4_t out[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    // rows 4b .. 4b+3: t0 = {r0.0 r1.0 r0.1 r1.1}, t1 = {r0.2 r1.2 r0.3 r1.3}, t2 / t3 the same of rows 2, 3
+    const unsigned t0 = __builtin_amdgcn_perm(r[4 * b + 1], r[4 * b], 0x05010400u);
+    const unsigned t1 = __builtin_amdgcn_perm(r[4 * b + 1], r[4 * b], 0x07030602u);
+    const unsigned t2 = __builtin_amdgcn_perm(r[4 * b + 3], r[4 * b + 2], 0x05010400u);
+    const unsigned t3 = __builtin_amdgcn_perm(r[4 * b + 3], r[4 * b + 2], 0x07030602u);
+    out[0][b] = (int)__builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    out[1][b] = (int)__builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    out[2][b] = (int)__builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    out[3][b] = (int)__builtin_amdgcn_perm(t3, t1, 0x07060302u);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) *(i32x4_t*)(Bt + (n + j) * ldbt + k) = out[j];
+}
+
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
@@ -391,6 +421,11 @@ hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int
   dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
   switch (elem_size) {
     case 1:
+      if (K % 16 == 0 && N % 4 == 0 && ldb % 4 == 0 && ldbt % 16 == 0 && ((uintptr_t)B & 3) == 0 && ((uintptr_t)Bt & 15) == 0) {
+        dim3 grid_b((unsigned)((N + 255) / 256), (unsigned)((K + 63) / 64));
+        hipLaunchKernelGGL(transpose_bytes_kernel, grid_b, dim3(256), 0, s, (const uint8_t*)B, (uint8_t*)Bt, K, N, ldb, ldbt);
+        break;
+      }
       hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, s, (const uint8_t*)B, (uint8_t*)Bt, K, N, ldb, ldbt);
       break;
     case 2:
