@@ -1019,15 +1019,25 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
     for (int r = 0; r < 16; ++r) accY[j][r] = 0;
   __syncthreads();  // the filter is out of LDS, the first window is in
 
+  // Tiles that do not fill a last round of all workgroups are dealt out in halves: with 1568 tiles on
+  // 256 workgroups the 32 left after six rounds keep 64 workgroups busy for half a tile instead of 32
+  // for a whole one.  t_half: the tile this workgroup takes one half of at the end (n_tiles: none).
+  const int grid = (int)gridDim.x, pos = t;
+  const int rem = p.n_tiles % grid, n_full = p.n_tiles - rem;
+  const bool split = rem != 0 && 2 * rem <= grid;
+  const int t_half = split && pos < 2 * rem ? n_full + (pos >> 1) : p.n_tiles;
+  const int t_end = split ? n_full : p.n_tiles;
+
   unsigned char* cur = win1;
   unsigned char* nxt = win0;
   for (;;) {
-    const int t2 = t + gridDim.x;
+    int t2 = t + grid;
+    if (split && t2 >= n_full) t2 = t_half;
     const TileGeom g2 = tile_geom(p, t2, Hv);
-      k_loop(std::integral_constant<int, 0>(), accX, cur, nxt, accY, m_last, g2);
-      k_loop(std::integral_constant<int, 1>(), accY, cur, nxt, accX, m_off[0], g2);
-      __syncthreads();  // every wavefront is done with the current window; the next one has arrived
-      m_last = m_off[1];
+    k_loop(std::integral_constant<int, 0>(), accX, cur, nxt, accY, m_last, g2);
+    k_loop(std::integral_constant<int, 1>(), accY, cur, nxt, accX, m_off[0], g2);
+    __syncthreads();  // every wavefront is done with the current window; the next one has arrived
+    m_last = m_off[1];
     t = t2;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
@@ -1038,10 +1048,26 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
     unsigned char* const w = cur;
     cur = nxt;
     nxt = w;
-    if (t >= p.n_tiles) break;
+    if (t >= t_end) break;
   }
+  auto flush = [&](const acc_t (&acc)[NI], int off) {
 #pragma unroll
-  for (int pc = 0; pc < 4 * NI; ++pc) finish_piece(accY, m_last, pc);
+    for (int pc = 0; pc < 4 * NI; ++pc) finish_piece(acc, off, pc);
+  };
+  if (t < p.n_tiles) {
+    // one half of tile t_half: its window is in `cur`, its placement is made; nothing comes after it
+    const TileGeom none = tile_geom(p, p.n_tiles, Hv);
+    if ((pos & 1) == 0) {
+      k_loop(std::integral_constant<int, 0>(), accX, cur, nxt, accY, m_last, none);
+      flush(accX, m_off[0]);
+    } else {
+      flush(accY, m_last);
+      k_loop(std::integral_constant<int, 1>(), accY, cur, nxt, accX, (int)0x80000000, none);
+      flush(accY, m_off[1]);
+    }
+  } else {
+    flush(accY, m_last);
+  }
 }
 
 template <int KIND, int WV>

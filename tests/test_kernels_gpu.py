@@ -313,14 +313,22 @@ def test_conv_register_filter(kind, shape, autopad, with_bias, capsys):
     np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
 
 
-def test_conv_register_filter_matches_lds_filter(monkeypatch):
-    # same inputs with the filter kept in LDS: both accumulate in fp32 and round once
-    Iv, Fv = _conv_case('bf16', (3, 56, 56, 64), 3, 3, 64, op.SAME_UPPER, 29)
+@pytest.mark.parametrize('batch', [3, 24])
+def test_conv_register_filter_matches_lds_filter(batch, monkeypatch):
+    # same inputs with the filter kept in LDS: both accumulate in fp32 and round once.
+    # batch 24 = 294 tiles on 256 workgroups: the 38 tiles of the last round are dealt out in halves
+    Iv, Fv = _conv_case('bf16', (batch, 56, 56, 64), 3, 3, 64, op.SAME_UPPER, 29)
     bias = bf16(E.round_bf16(np.random.default_rng(30).standard_normal(64).astype(np.float32)))
     a = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
     monkeypatch.setenv('PML_HIP_CONV', 'ldsfilter')
     b = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
     np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
+    # the last image (part of the halved tiles when batch = 24) against a float64 evaluation of the definition
+    Ip = np.pad(Iv[-1].astype(np.float64), ((1, 1), (1, 1), (0, 0)))
+    ref = sum(np.einsum('yxc,cd->yxd', Ip[ky:ky + 56, kx:kx + 56], Fv[ky, kx].astype(np.float64))
+              for ky in range(3) for kx in range(3))
+    ref = np.maximum(ref + E.bf16_from_bits(bias).astype(np.float64), 0)
+    np.testing.assert_allclose(a[-1], ref, rtol=BF16_RTOL, atol=2e-2)
 
 
 def test_conv_resident_filter_general_tail(capsys):
