@@ -55,10 +55,6 @@ struct TileGeom {
   int nrows;    // window rows of the tile
 };
 
-// n / d for n < 2^31 with the host-made pair (magic, shift) of d: one 32x32 -> 64 multiply and a shift
-__device__ inline unsigned fast_div(unsigned n, unsigned magic, int shift) {
-  return (unsigned)(((unsigned long long)n * magic) >> shift);
-}
 
 __device__ inline TileGeom tile_geom(const IgemmArgs& p, int t, int Hv) {
   TileGeom g;
@@ -1147,14 +1143,8 @@ size_t conv_halo_prepare(int kind, IgemmArgs* a) {
   if (total > 160 * 1024) return 0;
   a->halo_rows = max_rows;
   a->n_tiles = (int)n_tiles;
-  auto magic = [](unsigned d, unsigned* m, int* sh) {
-    int l = 0;
-    while ((1ull << l) < d) ++l;
-    *sh = 31 + l;
-    *m = (unsigned)(((1ull << (31 + l)) + d - 1) / d);
-  };
-  magic((unsigned)per, &a->div_per_magic, &a->div_per_shift);
-  magic((unsigned)a->OW, &a->div_ow_magic, &a->div_ow_shift);
+  fast_div_magic((unsigned)per, &a->div_per_magic, &a->div_per_shift);
+  fast_div_magic((unsigned)a->OW, &a->div_ow_magic, &a->div_ow_shift);
   // the pipelined 3x3 kernel: fast tail only, 64 channels out, buffer-addressable operands
   const int out_es = kind == KIND_BF16 ? 2 : 4;
   const bool out_fits = kind == KIND_BF16 ? a->out_dtype == PML_HIP_BF16 : true;

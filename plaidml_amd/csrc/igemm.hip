@@ -60,18 +60,23 @@ __device__ inline int xcd_remap(int bid, int nblocks) {
   return (bid % kXcds) * per + (bid / kXcds);
 }
 
-template <int BM, int BN>
+// STAGES = 0: as many as pay for the tile; 2: two, and LDS rounded up to what staging the whole result
+// tile needs (a short-K, bandwidth-bound GEMM gains more from a second workgroup on the CU than from a
+// third slab in flight)
+template <int BM, int BN, int STAGES = 0>
 struct Ring {
   static constexpr int kStage = (BM + BN) * kSlabBytes;                 // A rows then Bt rows
   // 64x64 tiles run two stages: 32 KB of LDS lets five workgroups share a CU, and for this tile
   // residency hides more latency than a third slab in flight does
-  static constexpr int kStages = (BM * BN <= 64 * 64) ? 2 : (3 * kStage <= kLdsBytes ? 3 : 2);
-  static constexpr int kBytes = kStages * kStage;
+  static constexpr int kStages = STAGES ? STAGES : ((BM * BN <= 64 * 64) ? 2 : (3 * kStage <= kLdsBytes ? 3 : 2));
+  static constexpr int kTileBytes = BM * (BN + 4) * 4;
+  static constexpr int kBytes = (STAGES && kTileBytes > kStages * kStage) ? kTileBytes : kStages * kStage;
 };
 
 // BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4 or 8 wavefronts (one or two per SIMD).
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0>
 __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
+  typedef Ring<BM, BN, STAGES> ring_t;
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
   constexpr int kWaves = NT / 64;
   constexpr int kRowsPerPass = NT / 8;  // operand rows one load of all threads covers (8 lanes per 128-byte row)
@@ -81,8 +86,8 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   constexpr int A_VECS = BM * 8 / NT;  // 16-byte vectors per thread per slab
   constexpr int B_VECS = BN * 8 / NT;
   static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0, "tile sides are whole load passes");
-  constexpr int kStage = Ring<BM, BN>::kStage;
-  constexpr int kStages = Ring<BM, BN>::kStages;
+  constexpr int kStage = ring_t::kStage;
+  constexpr int kStages = ring_t::kStages;
   constexpr int kAhead = kStages - 1;              // slabs in flight ahead of the one being multiplied
   constexpr int kLoads = A_VECS + B_VECS;          // loads a thread issues per slab
   static_assert(kAhead * kLoads <= 63, "the vmcnt field counts at most 63 loads");
@@ -120,13 +125,15 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
     const bool ok = m < p.M;
     const int64_t mm = ok ? m : 0;
     if (CONV) {
-      const int ow = (int)(mm % p.OW);
-      const int64_t t = mm / p.OW;
-      const int oh = (int)(t % p.OH);
-      const int64_t nb = t / p.OH;
+      // pixel numbers stay below 2^31 (the launcher checks the operand sizes)
+      const unsigned mu = (unsigned)mm;
+      const unsigned nb = fast_div(mu, p.div_per_magic, p.div_per_shift);
+      const unsigned rem = mu - nb * (unsigned)(p.OH * p.OW);
+      const unsigned ohu = fast_div(rem, p.div_ow_magic, p.div_ow_shift);
+      const int oh = (int)ohu, ow = (int)(rem - ohu * (unsigned)p.OW);
       a_ih0[i] = oh * p.SH - p.PH;
       a_iw0[i] = ow * p.SW - p.PW;
-      a_off[i] = ok ? (unsigned)(nb * ((int64_t)p.H * p.W * (p.pix_pitch ? p.pix_pitch : p.CI * ES))) : kOutside;
+      a_off[i] = ok ? (unsigned)((int64_t)nb * ((int64_t)p.H * p.W * (p.pix_pitch ? p.pix_pitch : p.CI * ES))) : kOutside;
     } else {
       a_ih0[i] = a_iw0[i] = 0;
       a_off[i] = ok ? (unsigned)(mm * p.lda * ES) : kOutside;
@@ -268,7 +275,7 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   // four consecutive columns per register quad, one 16-byte LDS store each.
   const int crow = lane & 31;
   const int ccol = (lane >> 5) * 4;
-  if constexpr ((size_t)BM * (BN + 4) * 4 <= (size_t)Ring<BM, BN>::kBytes) {
+  if constexpr ((size_t)BM * (BN + 4) * 4 <= (size_t)ring_t::kBytes) {
     // the whole tile fits in the pipeline buffers: ctile[BM][BN + 4], tail by all threads
     constexpr int CS = BN + 4;
     accs_t* ctile = (accs_t*)smem;
@@ -289,7 +296,7 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
     // large tiles: every wavefront stages RB of its 32-row blocks at a time in a private
     // region, wtile[RB * 32][WN + 4], and runs the tail over them with its 64 lanes
     constexpr int CS = WN + 4;
-    constexpr int kBudget = Ring<BM, BN>::kBytes / kWaves / 16 * 16;  // bytes per wavefront
+    constexpr int kBudget = ring_t::kBytes / kWaves / 16 * 16;  // bytes per wavefront
     constexpr int kFit = kBudget / (32 * CS * 4);
     constexpr int RB = kFit >= MI ? MI : (kFit >= 4 ? 4 : (kFit >= 2 ? 2 : 1));  // MI is a power of two
     static_assert(RB >= 1 && MI % RB == 0, "row blocks must stage evenly");
@@ -362,11 +369,11 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
   for (int j = 0; j < 4; ++j) *(i32x4_t*)(Bt + (n + j) * ldbt + k) = out[j];
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  const size_t lds = Ring<BM, BN>::kBytes;
-  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT>;
+  const size_t lds = Ring<BM, BN, STAGES>::kBytes;
+  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -386,6 +393,7 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_128x64_W8: return launch_cfg<KIND, 128, 64, 4, CONV, 512>(a, s);
     case TILE_128x128_W8: return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
     case TILE_256x128_W16: return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
+    case TILE_128x128_W8_S2: return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
   }
   return hipErrorInvalidValue;
 }
@@ -407,7 +415,7 @@ hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStr
   const int64_t es = kind == KIND_BF16 ? 2 : (kind == KIND_I8 ? 1 : 4);
   const int64_t a_bytes = conv ? (int64_t)a.NB * a.H * a.W * (a.pix_pitch ? a.pix_pitch : a.CI * es) + 256 : a.M * a.lda * es;
   const int64_t b_bytes = a.N * a.ldbt * es;
-  if (a_bytes >= ((int64_t)1 << 31) || b_bytes >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
+  if (a_bytes >= ((int64_t)1 << 31) || b_bytes >= ((int64_t)1 << 31) || (conv && a.M >= ((int64_t)1 << 31))) return hipErrorInvalidValue;
   switch (kind) {
     case KIND_F32: return igemm_launch_kind_0(cfg, conv, a, s);
     case KIND_BF16: return igemm_launch_kind_1(cfg, conv, a, s);

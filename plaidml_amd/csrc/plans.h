@@ -12,8 +12,8 @@
 namespace pml {
 
 enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2 };
-// _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four
-enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16 };
+// _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages
+enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2 };
 
 struct TailPtrs {
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
@@ -21,6 +21,19 @@ struct TailPtrs {
 };
 
 // Arguments of the MFMA GEMM / implicit-GEMM kernel (passed by value).
+// n / d for n < 2^31 as one 32x32 -> 64 multiply and a shift, with a pair (magic, shift) made on the host
+inline void fast_div_magic(unsigned d, unsigned* magic, int* shift) {
+  int l = 0;
+  while ((1ull << l) < d) ++l;
+  *shift = 31 + l;
+  *magic = (unsigned)(((1ull << (31 + l)) + d - 1) / d);
+}
+#if defined(__HIPCC__)
+__device__ inline unsigned fast_div(unsigned n, unsigned magic, int shift) {
+  return (unsigned)(((unsigned long long)n * magic) >> shift);
+}
+#endif
+
 struct IgemmArgs {
   int64_t M, N, K;
   const void* A;
@@ -39,7 +52,7 @@ struct IgemmArgs {
   // b_raw: Bt points at the caller's [K][N] matrix instead of the packed [N][K] one (pipelined kernel only)
   int NB, halo_rows, n_tiles, halo_variant, b_raw;
   int n_cus;  // compute units of the device (persistent grids)
-  // n / (OH*OW) and n / OW as multiply-and-shift (see fast_div)
+  // n / (OH*OW) and n / OW as multiply-and-shift (see fast_div); set for every convolution
   unsigned div_per_magic, div_ow_magic;
   int div_per_shift, div_ow_shift;
   // result type of the contraction, optional initial value

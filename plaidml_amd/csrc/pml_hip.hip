@@ -54,8 +54,6 @@ struct Plan {
   // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
   size_t halo_lds = 0;
   int halo_rows = 0, halo_tiles = 0, halo_variant = 0, n_cus = 0;
-  unsigned div_magic[2] = {0, 0};
-  int div_shift[2] = {0, 0};
   std::string text;
   ~Plan() {
     if (bt) (void)hipFree(bt);
@@ -81,34 +79,38 @@ const char* tile_name(int t) {
     case TILE_128x64_W8: return "128x64 (8 wavefronts)";
     case TILE_128x128_W8: return "128x128 (8 wavefronts)";
     case TILE_256x128_W16: return "256x128 (16 wavefronts)";
+    case TILE_128x128_W8_S2: return "128x128 (8 wavefronts, 2 stages)";
   }
   return "?";
 }
 
 // Stated tiling choice per shape class.  Measured on MI355X, bf16 unless said otherwise (us; w8 / w16 =
-// 8 / 16 wavefronts per workgroup, i.e. 2 / 4 per SIMD; the 4-wavefront 256x128 and 256x256 tiles that
-// were tried as well are slower than 256x128w16 everywhere and are no longer built):
-//                                    64x64  128x64  128x64w8  128x128  128x128w8  256x128w16
-//   4096^3 (int8)                        -       -       117      119       110          83
-//   4096^3                               -       -       169      173       161         107
-//   conv 128x28x28x128 (*) 3x3x128      66      76        75       89        72          53
-//   conv 128x14x14x256 (*) 3x3x256      66      72        75       73        62          46
-//   conv 128x7x7x512   (*) 3x3x512      72      67        73       64        57          78
-//   gemm 401408x256x64                  82     127        93      177       113          78
-//   gemm 401408x64x256                  47      55        45        -         -           -
-//   gemm 100352x512x128                 52      71        54      100        66          49
-//   gemm 25088x256x1024                 27      27        25       30        24          22
-//   gemm 6272x512x2048                  25      23        22       25        21          28
-//   gemm 23104x728x728                  72      67        61       78        63          57
-//   gemm 1024^3 (fp32)                  33      45        41       77        71         127
+// 8 / 16 wavefronts per workgroup; s2 = two ring stages and LDS cut to what the result tile needs, so that two
+// workgroups share a CU; the 4-wavefront 256x128 and 256x256 tiles that were tried as well are slower than
+// 256x128w16 everywhere and are no longer built):
+//                                    64x64  128x64  128x128  128x128w8  128x128w8s2  256x128w16
+//   4096^3 (int8)                      137       -      119        112          121          83
+//   4096^3                             198       -      173        163          115         108
+//   conv 128x28x28x128 (*) 3x3x128      66      76       89         71           49          52
+//   conv 128x14x14x256 (*) 3x3x256      64      72       73         61           45          45
+//   conv 128x7x7x512   (*) 3x3x512      72      67       64         57           65          77
+//   conv 128x56x56x256 (*) 1x1x512 /2   83     101        -         99           62          74
+//   gemm 401408x256x64                  82     127      177        123           76          84
+//   gemm 100352x512x128                 52      71      100         70           44          51
+//   gemm 25088x256x1024                 27      27       30         24           20          22
+//   gemm 6272x512x2048                  25      23       25         21           30          28
+//   gemm 23104x728x728                  72      67       78         65           57          58
+//   gemm 128x1000x2048                  14       -        -         19           19          25
+//   gemm 1024^3 (fp32)                  33      45       77         71            -         127
 // One tile per workgroup and a serial load / multiply / store life per tile: latency is hidden by the
-// other wavefronts of a SIMD, and more of them per workgroup do that better than more workgroups of four.
-// So: the 256x128 tile with 16 wavefronts whenever it yields enough workgroups to occupy most CUs, the
-// 128x128 one with 8 below that, and for small problems the smaller of 64x64 and 128x64 by (rounds of
-// resident workgroups) x (tile area), the larger tile on a tie.
+// other wavefronts of a SIMD -- 8 or 16 per workgroup instead of 4 -- and, for the bandwidth-bound shapes
+// with a short K, by a second workgroup on the CU whose loads run under the first one's tail.  So: long K
+// and at least two rounds of 256x128 tiles take that tile with 16 wavefronts; otherwise 128x128 with 8
+// wavefronts, two to a CU if that still gives every CU a workgroup, one to a CU (three stages) below
+// that; and for small problems the smaller of 64x64 and 128x64 by (rounds of resident workgroups) x
+// (tile area), the larger tile on a tie.
 int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
-  (void)k_bytes;
-  // PML_HIP_TILE=64x64|128x64|128x128|128x64w8|128x128w8|256x128w16 overrides the table (for tuning runs)
+  // PML_HIP_TILE=64x64|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
     const std::string v(e);
     if (v == "64x64") return TILE_64x64;
@@ -116,11 +118,13 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
     if (v == "128x128") return TILE_128x128;
     if (v == "128x64w8") return TILE_128x64_W8;
     if (v == "128x128w8") return TILE_128x128_W8;
+    if (v == "128x128w8s2") return TILE_128x128_W8_S2;
     if (v == "256x128w16") return TILE_256x128_W16;
   }
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (n <= 64) return TILE_64x64;  // (the 7x7 stem of ResNet-50 over 2x2 pixel blocks: 191 us against 207 us with 128x64w8)
-  if (tiles(256, 128) >= 160) return TILE_256x128_W16;
+  if (k_bytes >= 4096 && tiles(256, 128) >= 512) return TILE_256x128_W16;
+  if (tiles(128, 128) >= 256) return TILE_128x128_W8_S2;
   if (tiles(128, 128) >= 128) return TILE_128x128_W8;
   const int64_t rounds_small = (tiles(64, 64) + 5 * 256 - 1) / (5 * 256);
   const int64_t rounds_wide = (tiles(128, 64) + 2 * 256 - 1) / (2 * 256);
@@ -277,10 +281,8 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.halo_rows = p->halo_rows;
   g.n_tiles = p->halo_tiles;
   g.halo_variant = p->halo_variant;
-  g.div_per_magic = p->div_magic[0];
-  g.div_ow_magic = p->div_magic[1];
-  g.div_per_shift = p->div_shift[0];
-  g.div_ow_shift = p->div_shift[1];
+  fast_div_magic((unsigned)(d.oh * d.ow), &g.div_per_magic, &g.div_per_shift);
+  fast_div_magic((unsigned)d.ow, &g.div_ow_magic, &g.div_ow_shift);
   if (p->s2d) {
     // unit-stride convolution over the re-blocked input: one "tap" per block row, whose K-run covers
     // s2d_kaw neighbouring blocks of s2d_ch channels
@@ -612,10 +614,6 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
         p->halo_rows = g.halo_rows;
         p->halo_tiles = g.n_tiles;
         p->halo_variant = g.halo_variant;
-        p->div_magic[0] = g.div_per_magic;
-        p->div_magic[1] = g.div_ow_magic;
-        p->div_shift[0] = g.div_per_shift;
-        p->div_shift[1] = g.div_ow_shift;
         p->n_cus = prop.multiProcessorCount;
       }
     }
