@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t to
   }
 }
 
-template <int ES>
+template <int ES, bool WITH_INDEX>
 __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_vecs) {
   constexpr int V = VecIO<ES>::V;
   const pml_hip_pool2d_desc& d = a.d;
@@ -264,10 +264,10 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
         for (int i = 0; i < V; ++i) {
           if (d.agg == PML_HIP_AGG_MAX) {
             // taps come in rising window index, so ">=" leaves the largest index among equal values
-            best[i] = (x[u][i] >= acc[i]) ? k0 + u : best[i];
+            if (WITH_INDEX) best[i] = (x[u][i] >= acc[i]) ? k0 + u : best[i];
             acc[i] = (x[u][i] > acc[i]) ? x[u][i] : acc[i];
           } else if (d.agg == PML_HIP_AGG_MIN) {
-            best[i] = (x[u][i] <= acc[i]) ? k0 + u : best[i];
+            if (WITH_INDEX) best[i] = (x[u][i] <= acc[i]) ? k0 + u : best[i];
             acc[i] = (x[u][i] < acc[i]) ? x[u][i] : acc[i];
           } else {
             acc[i] += x[u][i];
@@ -276,15 +276,28 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
       }
     }
     const int64_t o0 = pix * d.c + c0;
+    if (dt == PML_HIP_BF16 || dt == PML_HIP_F32) {
+      // one 16-byte store of the rounded values
+      if constexpr (ES == 2) {
+        i32x4_t o;
 #pragma unroll
-    for (int i = 0; i < V; ++i) {
-      Scalar<float, int> v;
-      v.i = 0;
-      v.f = round_float_to<float>(dt, acc[i]);
-      acc[i] = v.f;
-      store_scalar<float, int>(a.out, o0 + i, dt, v);
+        for (int i = 0; i < 4; ++i)
+          o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[2 * i + 1]) << 16));
+        *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+      } else {
+        const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
+        *(f32x4_t*)((float*)a.out + o0) = o;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        Scalar<float, int> v;
+        v.i = 0;
+        v.f = round_float_to<float>(dt, acc[i]);
+        store_scalar<float, int>(a.out, o0 + i, dt, v);
+      }
     }
-    if (d.with_index) {
+    if (WITH_INDEX) {
       int32_t* ip = (int32_t*)a.idx + o0;
 #pragma unroll
       for (int i = 0; i < V; i += 4) {
@@ -410,10 +423,14 @@ hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s) {
   const int V = 16 / es;
   const int64_t total = d.n * d.oh * d.ow * (d.c / V);
   if (total == 0) return hipSuccess;
-  if (es == 2)
-    hipLaunchKernelGGL((pool2d_kernel<2>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  if (es == 2 && d.with_index)
+    hipLaunchKernelGGL((pool2d_kernel<2, true>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  else if (es == 2)
+    hipLaunchKernelGGL((pool2d_kernel<2, false>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  else if (d.with_index)
+    hipLaunchKernelGGL((pool2d_kernel<4, true>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
   else
-    hipLaunchKernelGGL((pool2d_kernel<4>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+    hipLaunchKernelGGL((pool2d_kernel<4, false>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
   return hipGetLastError();
 }
 
