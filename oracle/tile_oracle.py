@@ -45,6 +45,10 @@ Pinned by tests/test_oracle_golden.py against these reference-held vectors:
   BroadcastCmp / Add known answers of edsl_test.cc; convolution and pooling are
   additionally checked against torch.nn.functional on the CPU (a library routine,
   not the reference) and brute-force enumeration.
+And by tests/test_golden_network.py against the stored fp32 output of the reference
+benchmark tool's toy_parallel_conv network (its own weights and input image; strided
+SAME convolutions 7x7 / 1x1 / 3x3, bias, ReLU, add: plaidbench/plaidbench/golden/
+toy_parallel_conv/infer,bs-1.npy, tolerance of plaidbench/core.py:395-399).
 """
 import builtins
 import ctypes

@@ -91,6 +91,9 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   constexpr int kAhead = kStages - 1;              // slabs in flight ahead of the one being multiplied
   constexpr int kLoads = A_VECS + B_VECS;          // loads a thread issues per slab
   static_assert(kAhead * kLoads <= 63, "the vmcnt field counts at most 63 loads");
+  // (The vmcnt arithmetic below counts this kernel's own requests: a configuration whose registers spill
+  // puts scratch loads and stores into the same counter and is wrong, not just slow -- 256x256 with 16
+  // wavefronts needs 198 registers of the 128 it may have and failed its tests for that reason.)
   typedef typename Acc<KIND>::type acc_t;
   typedef typename Acc<KIND>::scalar accs_t;
   typedef accs_t acc4_t __attribute__((ext_vector_type(4)));

@@ -221,6 +221,30 @@ def residual_block(E, op, N=2, H=8, C=64, dtype_name='BFLOAT16'):
     return E.Program('residual', [X], [Z]), [xv], BF16 if dtype_name == 'BFLOAT16' else FP32
 
 
+def toy_parallel_conv(E, op):
+    """The reference benchmark tool's `toy_parallel_conv` network with its own weights and input
+    (plaidbench/plaidbench/networks/keras/toy_parallel_conv.py:18-41), fp32: conv 7x7/2 SAME 3->64 + ReLU, then
+    relu(relu(conv 1x1/2 64->256) + relu(conv 3x3/2 SAME 64->256)).  Returns the program, its inputs (the 224x224x3
+    image first, then weights and biases) and the golden fixture (tests/golden/toy_parallel_conv.npz)."""
+    import os
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'toy_parallel_conv.npz'))
+    f32 = E.DType.FLOAT32
+    image = np.repeat(np.repeat(fx['image'][None].astype(np.float32), 7, axis=1), 7, axis=2)  # values 0..255, unscaled
+    X = E.Placeholder(f32, list(image.shape))
+    ins, vals = [X], [image]
+
+    def conv(x, i, stride):
+        W = E.Placeholder(f32, list(fx['kernel%d' % i].shape))
+        B = E.Placeholder(f32, list(fx['bias%d' % i].shape))
+        ins.extend([W, B])
+        vals.extend([fx['kernel%d' % i], fx['bias%d' % i]])
+        return op.relu(op.convolution(x, W, strides=[stride, stride], autopad=op.SAME_UPPER) + B)
+
+    l1 = conv(X, 1, 2)
+    out = op.relu(conv(l1, 2, 2) + conv(l1, 3, 2))
+    return E.Program('toy_parallel_conv', ins, [out]), vals, fx
+
+
 def resnet50_tiny(E, op):
     """The full ResNet-50 v1.5 topology (plaidml_amd/resnet50.py) at 1/4 width on 2 x 32x32 images."""
     from plaidml_amd import resnet50
