@@ -32,6 +32,10 @@ enum class ConvDerivMode { NONE, DATA, FILTER, _LAST };
 enum class GroupLayout { NONE, SEPARATE, IN_C, IN_K, _LAST };
 enum class PoolMode { AVG, MAX, MIN, SUM, _LAST };
 enum class TensorLayout { NXC, NCX, KCX, XCK, GKCX, XGCK, _LAST };
+enum class PadMode { CONSTANT, EDGE, REFLECT, SYMMETRIC, _LAST };
+// reshape: take the dimension from the input / infer it from the element count
+static const int AUTO_DIM_MATCH = 0;
+static const int AUTO_DIM_FILL = -1;
 
 // a list of integers accepted from vectors and brace lists of the usual integer types
 struct Integers {
@@ -100,6 +104,44 @@ class convolution {
   bool infer_result_shape_ = false;
 };
 
+inline edsl::Tensor abs(const edsl::Tensor& I) { return details::op("abs", edsl::make_tuple(I)).as_tensor(); }
+
+inline edsl::Tensor concatenate(const std::vector<edsl::Tensor>& tensors, int axis) {
+  return details::op("concatenate", edsl::make_tuple(edsl::make_tuple(tensors), axis)).as_tensor();
+}
+
+inline edsl::Tensor cumsum(const edsl::Tensor& I, int axis, bool exclusive = false) {
+  return details::op("cumsum", edsl::make_tuple(I, axis, exclusive)).as_tensor();
+}
+
+inline edsl::Tensor elu(const edsl::Tensor& I, double alpha) { return details::op("elu", edsl::make_tuple(I, alpha)).as_tensor(); }
+
+class explicit_padding {
+ public:
+  explicit explicit_padding(const edsl::Tensor& I, const std::vector<int>& lo_pads, const std::vector<int>& hi_pads)
+      : I_(I), lo_pads_(lo_pads), hi_pads_(hi_pads), mode_(PadMode::CONSTANT), padval_(edsl::Constant(0)) {}
+  explicit_padding& lo_pads(const std::vector<int>& lo_pads) { lo_pads_ = lo_pads; return *this; }
+  explicit_padding& hi_pads(const std::vector<int>& hi_pads) { hi_pads_ = hi_pads; return *this; }
+  explicit_padding& mode(PadMode mode) { mode_ = mode; return *this; }
+  explicit_padding& padval(const edsl::Tensor& padval) { padval_ = padval; return *this; }
+  operator edsl::Tensor() const {  // NOLINT
+    auto args = edsl::make_tuple(I_, edsl::make_tuple(lo_pads_), edsl::make_tuple(hi_pads_), static_cast<int>(mode_), padval_);
+    return details::op("explicit_padding", args).as_tensor();
+  }
+
+ private:
+  edsl::Tensor I_;
+  std::vector<int> lo_pads_, hi_pads_;
+  PadMode mode_;
+  edsl::Tensor padval_;
+};
+
+inline edsl::Tensor flip(const edsl::Tensor& I, int axis) { return details::op("flip", edsl::make_tuple(I, axis)).as_tensor(); }
+
+inline edsl::Tensor hard_sigmoid(const edsl::Tensor& I, double slope) {
+  return details::op("hard_sigmoid", edsl::make_tuple(I, slope)).as_tensor();
+}
+
 inline edsl::Tensor dot(const edsl::Tensor& I, const edsl::Tensor& K, const std::string& name = "") {
   return details::op("dot", edsl::make_tuple(I, K, name)).as_tensor();
 }
@@ -130,6 +172,10 @@ inline edsl::Tensor pool(const edsl::Tensor I, PoolMode pool_mode, const std::ve
   return details::op("pool", args).as_tensor();
 }
 
+inline edsl::Tensor prod(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
+  return details::op("prod", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+
 class relu {
  public:
   explicit relu(const edsl::Tensor& I) : I_(I) {}
@@ -147,12 +193,50 @@ class relu {
   std::string name_;
 };
 
+inline edsl::Tensor repeat(const edsl::Tensor& I, int repeats, int axis) {
+  return details::op("repeat", edsl::make_tuple(I, repeats, axis)).as_tensor();
+}
+
+inline edsl::Tensor reshape(const edsl::Tensor& I, const edsl::Value& dims) {
+  return details::op("reshape", edsl::make_tuple(I, dims)).as_tensor();
+}
+
+inline edsl::Tensor sigmoid(const edsl::Tensor& I) { return details::op("sigmoid", edsl::make_tuple(I)).as_tensor(); }
+
+inline edsl::Tensor spatial_padding(const edsl::Tensor& x, const std::vector<int>& lo_pads, const std::vector<int>& hi_pads,
+                                    TensorLayout data_layout) {
+  auto args = edsl::make_tuple(x, edsl::make_tuple(lo_pads), edsl::make_tuple(hi_pads), static_cast<int>(data_layout));
+  return details::op("spatial_padding", args).as_tensor();
+}
+
+inline edsl::Tensor square(const edsl::Tensor& x) { return details::op("square", edsl::Value(x)).as_tensor(); }
+
+inline edsl::Tensor squeeze(const edsl::Tensor& I, const std::vector<int>& axes) {
+  return details::op("squeeze", edsl::make_tuple(I, edsl::make_tuple(axes))).as_tensor();
+}
+
 inline edsl::Tensor softmax(const edsl::Tensor& I, int axis, const std::string& name = "") {
   return details::op("softmax", edsl::make_tuple(I, axis, name)).as_tensor();
 }
 
 inline edsl::Tensor sum(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
   return details::op("sum", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+
+inline edsl::Tensor tile(const edsl::Tensor& I, const std::vector<int>& tiling_factors) {
+  return details::op("tile", edsl::make_tuple(I, edsl::make_tuple(tiling_factors))).as_tensor();
+}
+
+inline edsl::Tensor transpose(const edsl::Tensor& I, const edsl::Value& axes = edsl::None()) {
+  return details::op("transpose", edsl::make_tuple(I, axes)).as_tensor();
+}
+
+inline edsl::Tensor unsqueeze(const edsl::Tensor& I, const std::vector<int64_t>& axes) {
+  return details::op("unsqueeze", edsl::make_tuple(I, edsl::make_tuple(axes))).as_tensor();
+}
+
+inline edsl::Tensor variance(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
+  return details::op("variance", edsl::make_tuple(I, axes, keepdims)).as_tensor();
 }
 
 }  // namespace op

@@ -246,3 +246,218 @@ def argmax(I, axis=-1):
     AM = E.Contraction('argmax').outShape(a.dst_dims).outAccess(a.dst_idxs).max(
         E.cond(I[a.src_idxs], M[a.dst_idxs], IX[a.reduce_idxs])).build()
     return E.cast(AM, E.DType.UINT32)
+
+
+# ---------------------------------------------------------------------------
+# Data movement and simple arithmetic of the operation library, each restated as the single
+# contraction / elementwise chain the reference builds (plaidml/op/lib/ops.cc, lines per function).
+# ---------------------------------------------------------------------------
+PAD_CONSTANT, PAD_EDGE, PAD_REFLECT, PAD_SYMMETRIC = range(4)
+LAYOUT_NXC, LAYOUT_NCX = 0, 1
+AUTO_DIM_MATCH, AUTO_DIM_FILL = 0, -1
+
+
+def _axis(axis, nd, what):
+    if axis < -nd or axis >= nd:
+        raise ValueError('axis out of range in %s: %d for a tensor of rank %d' % (what, axis, nd))
+    return axis + nd if axis < 0 else axis
+
+
+def _axis_list(axes):
+    return [axes] if isinstance(axes, int) else list(axes)
+
+
+def abs(I):  # noqa: A001
+    return E.select(I < 0.0, -I, I)  # ops.cc:439-447
+
+
+def concatenate(tensors, axis):
+    """ops.cc:608-668: every input assigned at its offset into an otherwise zero result; the results added."""
+    tensors = list(tensors)
+    nd = len(tensors[0].shape)
+    axis = _axis(axis, nd, 'concatenate')
+    dims = list(tensors[0].shape)
+    dims[axis] = builtins.sum(t.shape[axis] for t in tensors)
+    idxs = E.TensorIndexes(nd)
+    out, off = None, 0
+    for t in tensors:
+        o_idxs = list(idxs)
+        o_idxs[axis] = idxs[axis] + off
+        r = E.Contraction('concatenate').outShape(dims).outAccess(o_idxs).assign(t[idxs]).build()
+        out = r if out is None else out + r
+        off += t.shape[axis]
+    return out
+
+
+def cumsum(I, axis, exclusive=False):
+    """ops.cc:1490-1510: O[.., i, ..] += I[.., i - k (- 1), ..] for 0 <= k < dim."""
+    nd = len(I.shape)
+    axis = _axis(axis, nd, 'cumsum')
+    o_idxs = E.TensorIndexes(nd)
+    i_idxs = list(o_idxs)
+    k = E.TensorIndex()
+    i_idxs[axis] = o_idxs[axis] - k - 1 if exclusive else o_idxs[axis] - k
+    return E.Contraction('cumsum').outShape(I.shape).outAccess(o_idxs).sum(I[i_idxs]).add_constraint(k < I.shape[axis]).build()
+
+
+def elu(I, alpha):
+    return E.select(I < 0.0, alpha * E.exp(I) - alpha, I)  # ops.cc:1563-1584
+
+
+def explicit_padding(I, lo_pads, hi_pads, mode=PAD_CONSTANT, padval=0):
+    """ops.cc:1586-1685: CONSTANT = assign at the offset into a result initialised with padval; EDGE = per
+    dimension, the first / last slice repeated and joined around the tensor."""
+    nd = len(I.shape)
+    if len(lo_pads) != nd or len(hi_pads) != nd:
+        raise ValueError('Inconsistent shapes in explicit_padding op')
+    idxs = E.TensorIndexes(nd)
+    if mode == PAD_CONSTANT:
+        o_dims = [I.shape[i] + lo_pads[i] + hi_pads[i] for i in range(nd)]
+        o_idxs = [idxs[i] + lo_pads[i] for i in range(nd)]
+        pv = padval if isinstance(padval, E.Tensor) else E.Constant(padval)
+        return E.Contraction('explicit_padding').outShape(o_dims).outAccess(o_idxs).assign(I[idxs]).init(pv).build()
+    if mode == PAD_EDGE:
+        O = I
+        for i in range(nd):
+            dst = E.TensorIndexes(nd)
+            src_lo, src_hi = list(dst), list(dst)
+            src_lo[i] = 0
+            src_hi[i] = O.shape[i] - 1
+            lo_dims, hi_dims = list(O.shape), list(O.shape)
+            lo_dims[i], hi_dims[i] = lo_pads[i], hi_pads[i]
+            Lo = E.Contraction('explicit_padding').outShape(lo_dims).outAccess(dst).assign(O[src_lo]).build()
+            Hi = E.Contraction('explicit_padding').outShape(hi_dims).outAccess(dst).assign(O[src_hi]).build()
+            O = concatenate([Lo, O, Hi], i)
+        return O
+    raise NotImplementedError('padding mode %d' % mode)
+
+
+def flip(I, axis=None):
+    """ops.cc:1687-1725: O[.., dim - 1 - i, ..] = I[.., i, ..]."""
+    nd = len(I.shape)
+    axes = range(nd) if axis is None else [_axis(a, nd, 'flip') for a in _axis_list(axis)]
+    i_idxs = E.TensorIndexes(nd)
+    o_idxs = list(i_idxs)
+    for a in axes:
+        o_idxs[a] = I.shape[a] - 1 - i_idxs[a]
+    return E.Contraction('flip').outShape(I.shape).outAccess(o_idxs).assign(I[i_idxs]).build()
+
+
+def hard_sigmoid(I, slope):
+    """ops.cc:1803-1820."""
+    if slope <= 0:
+        raise ValueError('hard_sigmoid expects positive slope')
+    hi_cusp = 1.0 / (2.0 * slope)
+    lo = E.cast(E.Constant(0.0), I.dt)
+    hi = E.cast(E.Constant(1.0), I.dt)
+    return E.select(I < -hi_cusp, lo, E.select(I > hi_cusp, hi, slope * I + 0.5))
+
+
+def prod(I, axes=None, keepdims=False):
+    return _reduce(I, axes, keepdims, 'product', 'prod')[0]  # ops.cc:2532-
+
+
+def repeat(I, repeats, axis):
+    """ops.cc:2782-2819: O[.., r * i + k, ..] = I[.., i, ..] for 0 <= k < r."""
+    nd = len(I.shape)
+    axis = _axis(axis, nd, 'repeat')
+    o_dims = list(I.shape)
+    o_dims[axis] = repeats * I.shape[axis]
+    i_idxs = E.TensorIndexes(nd)
+    o_idxs = list(i_idxs)
+    k = E.TensorIndex()
+    o_idxs[axis] = repeats * i_idxs[axis] + k
+    return E.Contraction('repeat').outShape(o_dims).outAccess(o_idxs).assign(I[i_idxs]).add_constraint(k < repeats).build()
+
+
+def reshape(I, dims):
+    """ops.cc:2821-2885: 0 / None take the input's dimension, -1 is inferred from the element count."""
+    out, fill = [], None
+    for i, d in enumerate(dims):
+        if d is None or d == AUTO_DIM_MATCH:
+            if i >= len(I.shape):
+                raise ValueError('matching dimension requested at %d from %d-dimensional tensor' % (i + 1, len(I.shape)))
+            out.append(I.shape[i])
+        elif d == AUTO_DIM_FILL:
+            if fill is not None:
+                raise ValueError("at most one dimension's size may be inferred")
+            fill = i
+            out.append(1)
+        else:
+            out.append(int(d))
+    if fill is not None:
+        num = den = 1
+        for d in I.shape:
+            num *= d
+        for d in out:
+            den *= d
+        out[fill] = num // den
+    return E.reshape(I, out)
+
+
+def sigmoid(I):
+    return 1.0 / (1.0 + E.exp(-I))  # ops.cc:2906-2915
+
+
+def spatial_padding(I, lo_pads, hi_pads, layout=LAYOUT_NXC):
+    """ops.cc:3129-: zero padding of the spatial dimensions (NXC / NCX)."""
+    nd = len(I.shape)
+    first = 1 if layout == LAYOUT_NXC else 2
+    if len(lo_pads) != nd - 2 or len(hi_pads) != nd - 2:
+        raise ValueError('Inconsistent spatial rank in spatial_padding op')
+    i_idxs = E.TensorIndexes(nd)
+    o_dims, o_idxs = list(I.shape), list(i_idxs)
+    for i in range(nd - 2):
+        o_dims[first + i] = I.shape[first + i] + lo_pads[i] + hi_pads[i]
+        o_idxs[first + i] = i_idxs[first + i] + lo_pads[i]
+    return E.Contraction('spatial_padding').outShape(o_dims).outAccess(o_idxs).assign(I[i_idxs]).build()
+
+
+def square(I):
+    return I * I  # ops.cc:3380-3384
+
+
+def squeeze(I, axes):
+    nd = len(I.shape)
+    drop = {_axis(a, nd, 'squeeze') for a in _axis_list(axes)}
+    return E.reshape(I, [I.shape[i] for i in range(nd) if i not in drop])  # ops.cc:3386-3422
+
+
+def tile(I, tiling_factors):
+    """ops.cc:3454-3489: O[.., t * dim + i, ..] = I[.., i, ..] for every repetition t."""
+    nd = len(I.shape)
+    reps = list(tiling_factors) + [1] * (nd - len(tiling_factors))
+    if not tiling_factors or len(reps) > nd:
+        raise ValueError('bad tiling factors')
+    i_idxs = E.TensorIndexes(nd)
+    o_dims = [I.shape[i] * reps[i] for i in range(nd)]
+    o_idxs = [E.TensorIndex() * I.shape[i] + i_idxs[i] for i in range(nd)]
+    return E.Contraction('tile').outShape(o_dims).outAccess(o_idxs).assign(I[i_idxs]).build()
+
+
+def transpose(I, axes=None):
+    """ops.cc:3491-3537: dimension i of the output is dimension axes[i] of the input (default: reversed)."""
+    nd = len(I.shape)
+    pattern = list(range(nd - 1, -1, -1)) if axes is None else list(axes)
+    i_idxs = E.TensorIndexes(nd)
+    return E.Contraction('transpose').outShape([I.shape[p] for p in pattern]).outAccess([i_idxs[p] for p in pattern]) \
+        .assign(I[i_idxs]).build()
+
+
+def unsqueeze(I, axes):
+    axes = _axis_list(axes)
+    nd = len(I.shape) + len(axes)
+    new = {_axis(a, nd, 'unsqueeze') for a in axes}
+    src = iter(I.shape)
+    return E.reshape(I, [1 if i in new else next(src) for i in range(nd)])  # ops.cc:3539-3584 (same element order)
+
+
+def variance(I, axes=None, keepdims=False):
+    """ops.cc:3586-3632: mean of squared differences from the mean (denominator n)."""
+    M = mean(I, axes, True)
+    d2 = (I - M) * (I - M)
+    so, a = _reduce(d2, axes, keepdims, 'sum', 'variance')
+    denom = 1
+    for ax in a.axes:
+        denom *= I.shape[ax]
+    return so / denom

@@ -11,6 +11,11 @@
 //   max / min / sum / mean via AggregationAxes ops.cc:71-127,1970-2003,3424-
 //   maximum / minimum ops.cc:1958-1968   relu     ops.cc:2705-2728
 //   softmax      ops.cc:3049-3098 (softmax over the last axis)
+//   data movement and simple arithmetic (every one a single contraction or elementwise chain):
+//   abs 439-447, concatenate 608-668, cumsum 1490-1510, elu 1563-1584, explicit_padding 1586-1685
+//   (CONSTANT and EDGE), flip 1687-1725, hard_sigmoid 1803-1820, prod 2532-, repeat 2782-2819,
+//   reshape 2821-2885, sigmoid 2906-2915, spatial_padding 3129- (NXC and NCX), square 3380-3384,
+//   squeeze 3386-3422, tile 3454-3489, transpose 3491-3537, unsqueeze 3539-3584, variance 3586-3632
 #include <functional>
 #include <map>
 #include <set>
@@ -468,22 +473,438 @@ Value op_softmax(const Value& value) {
   return Value{E / Nn};
 }
 
+size_t normalize_axis(int64_t axis, size_t ndims, const char* what) {
+  const int64_t n = static_cast<int64_t>(ndims);
+  if (axis < -n || axis >= n)
+    throw std::runtime_error(std::string("axis out of range in ") + what + ": " + std::to_string(axis) + " for a tensor of rank " +
+                             std::to_string(ndims));
+  return static_cast<size_t>(axis < 0 ? axis + n : axis);
+}
+
+std::vector<int64_t> int_or_ints(const Value& v) {
+  if (v.is_int()) return {v.as_int()};
+  return v.as_int_tuple();
+}
+
+Value op_abs(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 1) throw std::runtime_error("abs expects 1 argument");
+  auto I = args[0].as_tensor();
+  return Value{select(I < 0., -I, I)};
+}
+
+Tensor concatenate(std::vector<Tensor> tensors, int64_t raw_axis) {
+  if (tensors.empty()) throw std::runtime_error("The concatenate op requires at least one input tensor");
+  const size_t ndims = tensors[0].rank();
+  const size_t axis = normalize_axis(raw_axis, ndims, "concatenate");
+  // every input is placed at its offset along the axis of an otherwise empty result; the results are added
+  std::vector<TensorDim> dims(ndims);
+  std::vector<TensorIndex> I_idxs(ndims);
+  std::vector<TensorDim> axis_dims(tensors.size());
+  std::vector<TensorDim> offsets{TensorDim(0)};
+  for (size_t i = 0; i < tensors.size(); ++i) {
+    if (tensors[i].rank() != ndims) throw std::runtime_error("concatenate: inputs differ in rank");
+    dims[axis] = axis_dims[i];
+    tensors[i].bind_dims(dims);
+    offsets.push_back(axis_dims[i] + offsets.back());
+  }
+  dims[axis] = offsets.back();
+  Tensor result;
+  for (size_t i = 0; i < tensors.size(); ++i) {
+    std::vector<TensorIndex> O_idxs = I_idxs;
+    O_idxs[axis] = I_idxs[axis] + offsets[i];
+    Tensor R = Contraction(dims, O_idxs, "concatenate").assign(tensors[i](I_idxs));
+    result = i == 0 ? R : result + R;
+  }
+  return result;
+}
+
+Value op_concatenate(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("concatenate expects 2 arguments");
+  std::vector<Tensor> tensors;
+  for (const auto& t : args[0].as_tuple()) tensors.push_back(t.as_tensor());
+  return Value{concatenate(tensors, args[1].as_int())};
+}
+
+Value op_cumsum(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("cumsum expects 3 arguments");
+  auto I = args[0].as_tensor();
+  const size_t ndims = I.rank();
+  const size_t axis = normalize_axis(args[1].as_int(), ndims, "cumsum");
+  const bool exclusive = args[2].as_bool();
+  std::vector<TensorDim> dims(ndims);
+  I.bind_dims(dims);
+  std::vector<TensorIndex> O_idxs(ndims);
+  std::vector<TensorIndex> I_idxs = O_idxs;
+  TensorIndex back;
+  I_idxs[axis] = exclusive ? O_idxs[axis] - back - 1 : O_idxs[axis] - back;
+  Tensor O = Contraction(dims, O_idxs, "cumsum").sum(I(I_idxs)).add_constraint(back < dims[axis]);
+  return Value{O};
+}
+
+Value op_elu(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("elu expects 2 arguments");
+  auto I = args[0].as_tensor();
+  if (args[1].is_float()) {
+    const double alpha = args[1].as_float();
+    return Value{select(I < 0., alpha * exp(I) - alpha, I)};
+  }
+  if (args[1].is_int()) {
+    const int64_t alpha = args[1].as_int();
+    return Value{select(I < 0., alpha * exp(I) - alpha, I)};
+  }
+  throw std::runtime_error("Unexpected type for alpha in elu");
+}
+
+Value op_explicit_padding(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() < 5) throw std::runtime_error("explicit_padding expects 5 arguments");
+  auto I = args[0].as_tensor();
+  auto lo = args[1].as_int_tuple();
+  auto hi = args[2].as_int_tuple();
+  const auto mode = validate<plaidml::op::PadMode>(args[3].as_int());
+  const size_t ndims = I.rank();
+  if (lo.size() != ndims || hi.size() != ndims)
+    throw std::runtime_error("Inconsistent shapes in explicit_padding op (one lower and one upper padding per dimension expected)");
+  std::vector<TensorDim> X(ndims);
+  std::vector<TensorIndex> x(ndims);
+  I.bind_dims(X);
+  if (mode == plaidml::op::PadMode::CONSTANT) {
+    std::vector<TensorDim> O_dims;
+    std::vector<TensorIndex> O_idxs;
+    for (size_t i = 0; i < ndims; ++i) {
+      O_dims.push_back(X[i] + lo[i] + hi[i]);
+      O_idxs.push_back(x[i] + lo[i]);
+    }
+    Tensor O = Contraction(O_dims, O_idxs, "explicit_padding").assign(I(x)).init(args[4].as_tensor());
+    return Value{O};
+  }
+  if (mode == plaidml::op::PadMode::EDGE) {
+    // dimension by dimension: the first / last slice repeated lo / hi times, joined around the tensor so far
+    Tensor O = I;
+    for (size_t i = 0; i < ndims; ++i) {
+      std::vector<TensorDim> D(ndims);
+      O.bind_dims(D);
+      std::vector<TensorIndex> dst(ndims);
+      std::vector<TensorIndex> src_lo = dst, src_hi = dst;
+      src_lo[i] = TensorIndex(static_cast<int64_t>(0));
+      src_hi[i] = D[i] - TensorIndex(static_cast<int64_t>(1));
+      std::vector<TensorDim> lo_dims = D, hi_dims = D;
+      lo_dims[i] = TensorDim(lo[i]);
+      hi_dims[i] = TensorDim(hi[i]);
+      Tensor Lo = Contraction(lo_dims, dst, "explicit_padding").assign(O(src_lo));
+      Tensor Hi = Contraction(hi_dims, dst, "explicit_padding").assign(O(src_hi));
+      O = concatenate({Lo, O, Hi}, static_cast<int64_t>(i));
+    }
+    return Value{O};
+  }
+  throw std::runtime_error("Unimplemented padding mode (only CONSTANT and EDGE exist, as in the reference)");
+}
+
+Value op_flip(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("flip expects 2 arguments");
+  auto I = args[0].as_tensor();
+  const size_t ndims = I.rank();
+  std::vector<int64_t> raw;
+  if (args[1].is_none()) {
+    for (size_t i = 0; i < ndims; ++i) raw.push_back(static_cast<int64_t>(i));
+  } else {
+    raw = int_or_ints(args[1]);
+  }
+  std::vector<TensorDim> dims(ndims);
+  std::vector<TensorIndex> I_idxs(ndims);
+  std::vector<TensorIndex> O_idxs = I_idxs;
+  I.bind_dims(dims);
+  for (int64_t a : raw) {
+    const size_t axis = normalize_axis(a, ndims, "flip");
+    O_idxs[axis] = dims[axis] - 1 - I_idxs[axis];
+  }
+  Tensor O = Contraction(dims, O_idxs, "flip").assign(I(I_idxs));
+  return Value{O};
+}
+
+Value op_hard_sigmoid(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("hard_sigmoid expects 2 arguments");
+  auto I = args[0].as_tensor();
+  const double slope = args[1].as_float();
+  if (slope <= 0) throw std::runtime_error("hard_sigmoid expects positive slope, received " + std::to_string(slope));
+  const double hi_cusp = 1. / (2. * slope), lo_cusp = -hi_cusp;
+  auto lo = cast(Tensor(0.), I.dtype());
+  auto hi = cast(Tensor(1.), I.dtype());
+  return Value{select(I < lo_cusp, lo, select(I > hi_cusp, hi, slope * I + 0.5))};
+}
+
+Value op_prod(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("prod expects 3 arguments");
+  auto I = args[0].as_tensor();
+  if (I.rank() == 0) return Value{I};
+  auto axes = args[1];
+  if (axes.is_tuple() && axes.as_tuple().empty()) return Value{I};
+  AggregationAxes ag(I.rank(), axes, args[2].as_bool());
+  I.bind_dims(ag.src_dims);
+  Tensor O = Contraction(ag.dst_dims, ag.dst_idxs, "prod").product(I(ag.src_idxs));
+  return Value{O};
+}
+
+Value op_repeat(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("repeat expects 3 arguments");
+  auto I = args[0].as_tensor();
+  TensorDim repeats;
+  if (args[1].is_int())
+    repeats = TensorDim(args[1].as_int());
+  else if (args[1].is_dim())
+    repeats = args[1].as_dim();
+  else
+    throw std::runtime_error("Repeat only accepts int or TensorDim for repeats parameter");
+  const size_t ndims = I.rank();
+  const size_t axis = normalize_axis(args[2].as_int(), ndims, "repeat");
+  std::vector<TensorDim> I_dims(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> O_dims = I_dims;
+  O_dims[axis] = repeats * I_dims[axis];
+  std::vector<TensorIndex> I_idxs(ndims);
+  std::vector<TensorIndex> O_idxs = I_idxs;
+  TensorIndex inner;
+  O_idxs[axis] = repeats * I_idxs[axis] + inner;
+  Tensor O = Contraction(O_dims, O_idxs, "repeat").assign(I(I_idxs)).add_constraint(inner < repeats);
+  return Value{O};
+}
+
+Value op_reshape(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("reshape expects 2 arguments");
+  auto I = args[0].as_tensor();
+  std::vector<TensorDim> I_dims(I.rank());
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> O_dims;
+  size_t fill_dim = 0;
+  bool fill = false;
+  auto target = args[1].as_tuple();
+  auto match = [&](size_t i) {
+    if (i >= I_dims.size())
+      throw std::runtime_error("matching dimension requested at " + std::to_string(i + 1) + " from " + std::to_string(I_dims.size()) +
+                               "-dimensional tensor");
+    O_dims.push_back(I_dims[i]);
+  };
+  for (size_t i = 0; i < target.size(); ++i) {
+    if (target[i].is_int()) {
+      const int64_t d = target[i].as_int();
+      if (d == plaidml::op::AUTO_DIM_MATCH) {
+        match(i);
+      } else if (d == plaidml::op::AUTO_DIM_FILL) {
+        if (fill) throw std::runtime_error("at most one dimension's size may be inferred");
+        fill = true;
+        fill_dim = i;
+        O_dims.emplace_back(1);
+      } else {
+        O_dims.emplace_back(d);
+      }
+    } else if (target[i].is_dim()) {
+      O_dims.push_back(target[i].as_dim());
+    } else if (target[i].is_none()) {
+      match(i);
+    } else {
+      throw std::runtime_error("reshape: a dimension must be an integer, a TensorDim or None");
+    }
+  }
+  if (fill) {
+    TensorDim num(1), den(1);
+    for (const auto& d : I_dims) num = d * num;
+    for (const auto& d : O_dims) den = d * den;
+    O_dims[fill_dim] = TensorDim(num / den);
+  }
+  return Value{edsl::reshape(I, O_dims)};
+}
+
+Value op_sigmoid(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 1) throw std::runtime_error("sigmoid expects 1 argument");
+  auto I = args[0].as_tensor();
+  return Value{1.0 / (1.0 + exp(-I))};
+}
+
+Value op_spatial_padding(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 4) throw std::runtime_error("spatial_padding expects 4 arguments");
+  auto I = args[0].as_tensor();
+  auto lo = args[1].as_int_tuple();
+  auto hi = args[2].as_int_tuple();
+  const auto layout = validate<TensorLayout>(args[3].as_int());
+  if (layout != TensorLayout::NXC && layout != TensorLayout::NCX)
+    throw std::runtime_error("spatial_padding: only the NXC and NCX layouts are supported by this backend");
+  const size_t ndims = I.rank();
+  if (ndims < 3) throw std::runtime_error("Insufficient spatial rank in spatial_padding op (at least 1 spatial dim required)");
+  const size_t spatial = ndims - 2;
+  if (lo.size() != spatial || hi.size() != spatial)
+    throw std::runtime_error("Inconsistent spatial rank in spatial_padding op (one lower and one upper padding per spatial dim expected)");
+  const size_t first = layout == TensorLayout::NXC ? 1 : 2;  // position of the first spatial dimension
+  std::vector<TensorDim> I_dims(ndims);
+  std::vector<TensorIndex> I_idxs(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> O_dims = I_dims;
+  std::vector<TensorIndex> O_idxs = I_idxs;
+  for (size_t i = 0; i < spatial; ++i) {
+    O_dims[first + i] = I_dims[first + i] + lo[i] + hi[i];
+    O_idxs[first + i] = I_idxs[first + i] + lo[i];
+  }
+  Tensor O = Contraction(O_dims, O_idxs, "spatial_padding").assign(I(I_idxs));
+  return Value{O};
+}
+
+Value op_square(const Value& value) {
+  auto x = value.is_tuple() ? value.as_tuple().at(0).as_tensor() : value.as_tensor();
+  return Value{x * x};
+}
+
+Value op_squeeze(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("Squeeze expects 2 arguments");
+  auto I = args[0].as_tensor();
+  const size_t ndims = I.rank();
+  std::vector<TensorDim> I_dims(ndims);
+  I.bind_dims(I_dims);
+  std::set<size_t> axes;
+  for (int64_t a : int_or_ints(args[1])) axes.insert(normalize_axis(a, ndims, "squeeze"));
+  std::vector<TensorDim> O_dims;
+  for (size_t i = 0; i < ndims; ++i)
+    if (!axes.count(i)) O_dims.push_back(I_dims[i]);
+  return Value{edsl::reshape(I, O_dims)};
+}
+
+Value op_tile(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("Tile expects 2 arguments");
+  auto I = args[0].as_tensor();
+  auto reps = args[1].as_int_tuple();
+  const size_t ndims = I.rank();
+  if (reps.empty()) throw std::runtime_error("No tiling factors provided to tile operation");
+  while (reps.size() < ndims) reps.push_back(1);
+  if (reps.size() > ndims) throw std::runtime_error("More tiling factors provided to tile operation than tensor dimensions");
+  std::vector<TensorDim> I_dims(ndims);
+  std::vector<TensorIndex> I_idxs(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> O_dims;
+  std::vector<TensorIndex> O_idxs;
+  for (size_t i = 0; i < ndims; ++i) {
+    O_dims.push_back(I_dims[i] * reps[i]);
+    O_idxs.push_back(TensorIndex() * I_dims[i] + I_idxs[i]);
+  }
+  Tensor O = Contraction(O_dims, O_idxs, "tile").assign(I(I_idxs));
+  return Value{O};
+}
+
+Value op_transpose(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("Transpose expects 2 arguments");
+  auto I = args[0].as_tensor();
+  const size_t ndims = I.rank();
+  std::vector<int64_t> pattern;
+  if (args[1].is_none()) {
+    for (size_t i = 0; i < ndims; ++i) pattern.push_back(static_cast<int64_t>(ndims - 1 - i));
+  } else if (args[1].is_tuple()) {
+    pattern = args[1].as_int_tuple();
+  } else {
+    throw std::runtime_error("Transpose 2nd argument must be none or integer tuple");
+  }
+  if (pattern.size() != ndims) throw std::runtime_error("Transpose pattern must name every dimension once");
+  for (int64_t i : pattern)
+    if (i < 0 || static_cast<size_t>(i) >= ndims)
+      throw std::runtime_error("Transpose of nonexistent axis " + std::to_string(i) + " requested (input has " + std::to_string(ndims) +
+                               " dimensions)");
+  std::vector<TensorDim> I_dims(ndims);
+  std::vector<TensorIndex> I_idxs(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> O_dims;
+  std::vector<TensorIndex> O_idxs;
+  for (size_t i = 0; i < ndims; ++i) {
+    O_dims.push_back(I_dims[pattern[i]]);
+    O_idxs.push_back(I_idxs[pattern[i]]);
+  }
+  Tensor O = Contraction(O_dims, O_idxs, "transpose").assign(I(I_idxs));
+  return Value{O};
+}
+
+Value op_unsqueeze(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("unsqueeze expects 2 arguments");
+  auto I = args[0].as_tensor();
+  const size_t ndims = I.rank();
+  auto raw = int_or_ints(args[1]);
+  std::set<size_t> axes;
+  for (int64_t a : raw) axes.insert(normalize_axis(a, ndims + raw.size(), "unsqueeze"));
+  std::vector<TensorDim> I_dims(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorDim> O_dims;
+  size_t src = 0;
+  for (size_t i = 0; i < ndims + axes.size(); ++i) {
+    if (axes.count(i))
+      O_dims.emplace_back(1);
+    else if (src < ndims)
+      O_dims.push_back(I_dims[src++]);
+  }
+  if (src != ndims) throw std::runtime_error("Unsqueeze did not replicate entirety of input into output");
+  return Value{edsl::reshape(I, O_dims)};
+}
+
+Value op_variance(const Value& value) {
+  // the uncorrected sample variance (denominator n)
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("Variance expects 3 arguments");
+  auto I = args[0].as_tensor();
+  auto axes = args[1];
+  if (I.rank() == 0) return Value{Tensor(static_cast<int64_t>(0))};
+  if (axes.is_tuple() && axes.as_tuple().empty()) throw std::runtime_error("Variance expects nonempty axis list");
+  Tensor Mean = reduce(make_tuple(I, axes, true), "mean", PLAIDML_AGG_OP_SUM).as_tensor();
+  AggregationAxes ag(I.rank(), axes, args[2].as_bool());
+  I.bind_dims(ag.src_dims);
+  Tensor D2 = (I - Mean) * (I - Mean);
+  Tensor S = Contraction(ag.dst_dims, ag.dst_idxs, "variance").sum(D2(ag.src_idxs));
+  Tensor denom(1);
+  for (size_t a : ag.axes) denom = denom * ag.src_dims.at(a);
+  return Value{S / denom};
+}
+
 using OpFn = std::function<Value(const Value&)>;
 const std::map<std::string, OpFn>& registry() {
   static const std::map<std::string, OpFn> r = {
+      {"abs", op_abs},
       {"argmax", op_argmax},
       {"clip", op_clip},
+      {"concatenate", op_concatenate},
       {"convolution", op_convolution},
+      {"cumsum", op_cumsum},
       {"dot", op_dot},
+      {"elu", op_elu},
+      {"explicit_padding", op_explicit_padding},
+      {"flip", op_flip},
+      {"hard_sigmoid", op_hard_sigmoid},
       {"max", [](const Value& v) { return reduce(v, "max", PLAIDML_AGG_OP_MAX); }},
       {"maximum", op_maximum},
       {"mean", [](const Value& v) { return reduce(v, "mean", PLAIDML_AGG_OP_SUM); }},
       {"min", [](const Value& v) { return reduce(v, "min", PLAIDML_AGG_OP_MIN); }},
       {"minimum", op_minimum},
       {"pool", op_pool},
+      {"prod", op_prod},
       {"relu", op_relu},
+      {"repeat", op_repeat},
+      {"reshape", op_reshape},
+      {"sigmoid", op_sigmoid},
       {"softmax", op_softmax},
+      {"spatial_padding", op_spatial_padding},
+      {"square", op_square},
+      {"squeeze", op_squeeze},
       {"sum", [](const Value& v) { return reduce(v, "sum", PLAIDML_AGG_OP_SUM); }},
+      {"tile", op_tile},
+      {"transpose", op_transpose},
+      {"unsqueeze", op_unsqueeze},
+      {"variance", op_variance},
   };
   return r;
 }

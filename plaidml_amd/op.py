@@ -82,3 +82,80 @@ def maximum(X, Y):
 
 def minimum(X, Y):
     return E.op_make('minimum', [X, Y]).as_tensor()
+
+
+PAD_CONSTANT, PAD_EDGE, PAD_REFLECT, PAD_SYMMETRIC = range(4)
+AUTO_DIM_MATCH, AUTO_DIM_FILL = 0, -1
+
+
+def abs(I):  # noqa: A001
+    return E.op_make('abs', [I]).as_tensor()
+
+
+def concatenate(tensors, axis):
+    return E.op_make('concatenate', [list(tensors), int(axis)]).as_tensor()
+
+
+def cumsum(I, axis, exclusive=False):
+    return E.op_make('cumsum', [I, int(axis), bool(exclusive)]).as_tensor()
+
+
+def elu(I, alpha):
+    return E.op_make('elu', [I, alpha]).as_tensor()
+
+
+def explicit_padding(I, lo_pads, hi_pads, mode=PAD_CONSTANT, padval=0):
+    pv = padval if isinstance(padval, E.Tensor) else E.Constant(padval)
+    return E.op_make('explicit_padding', [I, _ints(lo_pads), _ints(hi_pads), int(mode), pv]).as_tensor()
+
+
+def flip(I, axis=None):
+    return E.op_make('flip', [I, _axes(axis)]).as_tensor()
+
+
+def hard_sigmoid(I, slope):
+    return E.op_make('hard_sigmoid', [I, float(slope)]).as_tensor()
+
+
+def prod(I, axes=None, keepdims=False):
+    return E.op_make('prod', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def repeat(I, repeats, axis):
+    return E.op_make('repeat', [I, int(repeats), int(axis)]).as_tensor()
+
+
+def reshape(I, dims):
+    return E.op_make('reshape', [I, [None if d is None else int(d) for d in dims]]).as_tensor()
+
+
+def sigmoid(I):
+    return E.op_make('sigmoid', [I]).as_tensor()
+
+
+def spatial_padding(I, lo_pads, hi_pads, layout=LAYOUT_NXC):
+    return E.op_make('spatial_padding', [I, _ints(lo_pads), _ints(hi_pads), int(layout)]).as_tensor()
+
+
+def square(I):
+    return E.op_make('square', [I]).as_tensor()
+
+
+def squeeze(I, axes):
+    return E.op_make('squeeze', [I, _axes(axes)]).as_tensor()
+
+
+def tile(I, tiling_factors):
+    return E.op_make('tile', [I, _ints(tiling_factors)]).as_tensor()
+
+
+def transpose(I, axes=None):
+    return E.op_make('transpose', [I, _axes(axes)]).as_tensor()
+
+
+def unsqueeze(I, axes):
+    return E.op_make('unsqueeze', [I, _axes(axes)]).as_tensor()
+
+
+def variance(I, axes=None, keepdims=False):
+    return E.op_make('variance', [I, _axes(axes), bool(keepdims)]).as_tensor()

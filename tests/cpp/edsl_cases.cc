@@ -196,6 +196,47 @@ void caseConvRelu() {
   expectClose("conv_bias_relu", readBuffer<float>(out[0]), want, 1e-3f, 1e-4f);
 }
 
+// op library data movement, written as plaidml/op/op_test.cc writes it (ExplicitPadding :318-333,
+// ExplicitPaddingEdge :385-418, CumSumExclusive :297-304, Transpose / Concatenate patterns :174-180,698-702)
+void caseOpLibrary() {
+  {
+    auto I = Placeholder(DType::FLOAT32, {2, 3});
+    Tensor O = op::explicit_padding(I, {2, 1}, {2, 1}).mode(op::PadMode::CONSTANT).padval(Constant(-1.0));
+    auto program = buildProgram("explicit_padding", {I}, {O});
+    auto out = run(program, {makeBuffer<float>(DType::FLOAT32, {2, 3}, {1, 2, 3, 4, 5, 6})});
+    expectEq<float>("explicit_padding", readBuffer<float>(out[0]),
+                    {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, 1, 2, 3, -1, -1, 4, 5, 6, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1});
+  }
+  {
+    auto I = Placeholder(DType::FLOAT32, {1, 2, 3});
+    Tensor O = op::explicit_padding(I, {1, 2, 1}, {2, 1, 3}).mode(op::PadMode::EDGE);
+    auto program = buildProgram("explicit_padding_edge", {I}, {O});
+    auto out = run(program, {makeBuffer<float>(DType::FLOAT32, {1, 2, 3}, {1, 2, 3, 4, 5, 6})});
+    std::vector<float> want;
+    for (int n = 0; n < 4; ++n)
+      for (int r = 0; r < 5; ++r) {
+        const std::vector<float> row = r < 3 ? std::vector<float>{1, 1, 2, 3, 3, 3, 3} : std::vector<float>{4, 4, 5, 6, 6, 6, 6};
+        want.insert(want.end(), row.begin(), row.end());
+      }
+    expectEq<float>("explicit_padding_edge", readBuffer<float>(out[0]), want);
+  }
+  {
+    auto I = Placeholder(DType::FLOAT32, {4});
+    auto program = buildProgram("cumsum", {I}, {op::cumsum(I, 0, true)});
+    auto out = run(program, {makeBuffer<float>(DType::FLOAT32, {4}, {2, 4, 6, 8})});
+    expectEq<float>("cumsum_exclusive", readBuffer<float>(out[0]), {0, 2, 6, 12});
+  }
+  {
+    auto A = Placeholder(DType::FLOAT32, {2, 3});
+    auto B = Placeholder(DType::FLOAT32, {2, 2});
+    Tensor O = op::transpose(op::concatenate({A, B}, 1), edsl::make_tuple(std::vector<int64_t>{1, 0}));
+    auto program = buildProgram("concat_transpose", {A, B}, {O});
+    auto out = run(program, {makeBuffer<float>(DType::FLOAT32, {2, 3}, {1, 2, 3, 4, 5, 6}),
+                             makeBuffer<float>(DType::FLOAT32, {2, 2}, {7, 8, 9, 10})});
+    expectEq<float>("concat_transpose", readBuffer<float>(out[0]), {1, 4, 2, 5, 3, 6, 7, 9, 8, 10});
+  }
+}
+
 void caseErrors() {
   auto A = Placeholder(DType::FLOAT32, {4, 4});
   auto program = buildProgram("ident", {A}, {A + 1.0});
@@ -230,6 +271,7 @@ int main() {
     caseUseDefault();
     caseInt8Gemm();
     caseConvRelu();
+    caseOpLibrary();
     caseErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAILED with exception: %s\n", e.what());
