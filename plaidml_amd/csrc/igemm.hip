@@ -73,14 +73,16 @@ struct Ring {
   static constexpr int kBytes = (STAGES && kTileBytes > kStages * kStage) ? kTileBytes : kStages * kStage;
 };
 
-// BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4 or 8 wavefronts (one or two per SIMD).
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0>
+// BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4, 8 or 16 wavefronts (one, two or four
+// per SIMD).  WAVES_K = 2: two such grids, each multiplying one half of the K-blocks of every slab; their
+// partial results meet in LDS before the tail (more wavefronts for problems with few tiles and a long K).
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1>
 __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   typedef Ring<BM, BN, STAGES> ring_t;
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
   constexpr int kWaves = NT / 64;
   constexpr int kRowsPerPass = NT / 8;  // operand rows one load of all threads covers (8 lanes per 128-byte row)
-  constexpr int WAVES_N = kWaves / WAVES_M;
+  constexpr int WAVES_N = kWaves / WAVES_M / WAVES_K;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int MI = WM / 32, NI = WN / 32;
   constexpr int A_VECS = BM * 8 / NT;  // 16-byte vectors per thread per slab
@@ -103,7 +105,8 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int wk = wave / (WAVES_M * WAVES_N);  // which part of every slab's K-blocks
+  const int wm = (wave % (WAVES_M * WAVES_N)) / WAVES_N, wn = wave % WAVES_N;
 
   const int tiles_n = (int)((p.N + BN - 1) / BN);
   const int tiles_m = (int)((p.M + BM - 1) / BM);
@@ -219,9 +222,11 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   }
 
   const int frow = lane & 31;  // row of the 32x32 block this lane feeds
-  int fslot[kSlabBytes / 32];  // byte offset of its 16-byte half of each 32-byte K-block, swizzled
+  // byte offset of its 16-byte half of each of the wavefront's 32-byte K-blocks, swizzled
+  constexpr int kBlocks = kSlabBytes / 32 / WAVES_K;
+  int fslot[kBlocks];
 #pragma unroll
-  for (int kb = 0; kb < kSlabBytes / 32; ++kb) fslot[kb] = ((kb * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
+  for (int kb = 0; kb < kBlocks; ++kb) fslot[kb] = (((wk * kBlocks + kb) * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
 
   int stage = 0;  // ring stage of slab s
   for (int s = 0; s < n_slabs; ++s) {
@@ -237,7 +242,6 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
     // Per K-block: MI*NI MFMA groups in program order; behind the m-th one sit one request of the
     // slab two ahead and one fragment read of K-block kb + 1, so that neither the texture path nor
     // LDS latency ever holds up the matrix pipe.  sched_barrier pins that order.
-    constexpr int kBlocks = kSlabBytes / 32;
     i32x4_t fa[2][MI], fb[2][NI];
 #pragma unroll
     for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(a_base + i * 32 * kSlabBytes + fslot[0]);
@@ -278,22 +282,30 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   // four consecutive columns per register quad, one 16-byte LDS store each.
   const int crow = lane & 31;
   const int ccol = (lane >> 5) * 4;
+  static_assert(WAVES_K == 1 || (size_t)BM * (BN + 4) * 4 <= (size_t)ring_t::kBytes, "partial results meet in the whole-tile buffer");
   if constexpr ((size_t)BM * (BN + 4) * 4 <= (size_t)ring_t::kBytes) {
     // the whole tile fits in the pipeline buffers: ctile[BM][BN + 4], tail by all threads
     constexpr int CS = BN + 4;
     accs_t* ctile = (accs_t*)smem;
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int part = 0; part < WAVES_K; ++part) {
+      if (part == wk) {
 #pragma unroll
-      for (int j = 0; j < NI; ++j)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          acc4_t q;
+          for (int j = 0; j < NI; ++j)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) q[e] = acc[i][j][4 * g + e];
-          *(acc4_t*)&ctile[(wm * WM + i * 32 + crow) * CS + wn * WN + j * 32 + 8 * g + ccol] = q;
-        }
-    __syncthreads();
+            for (int g = 0; g < 4; ++g) {
+              acc4_t* dst = (acc4_t*)&ctile[(wm * WM + i * 32 + crow) * CS + wn * WN + j * 32 + 8 * g + ccol];
+              acc4_t q;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) q[e] = acc[i][j][4 * g + e];
+              if (part > 0) q += *dst;  // the parts before this one are already there
+              *dst = q;
+            }
+      }
+      __syncthreads();
+    }
     tile_tail<KIND, BM, BN, NT>(p, ctile, m0, n0, tid, &pre);
   } else {
     // large tiles: every wavefront stages RB of its 32-row blocks at a time in a private
@@ -372,11 +384,11 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
   for (int j = 0; j < 4; ++j) *(i32x4_t*)(Bt + (n + j) * ldbt + k) = out[j];
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const size_t lds = Ring<BM, BN, STAGES>::kBytes;
-  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES>;
+  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -397,6 +409,7 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_128x128_W8: return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
     case TILE_256x128_W16: return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
     case TILE_128x128_W8_S2: return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
+    case TILE_64x64_W8_K2: return launch_cfg<KIND, 64, 64, 2, CONV, 512, 0, 2>(a, s);
   }
   return hipErrorInvalidValue;
 }

@@ -79,6 +79,7 @@ const char* tile_name(int t) {
     case TILE_128x64_W8: return "128x64 (8 wavefronts)";
     case TILE_128x128_W8: return "128x128 (8 wavefronts)";
     case TILE_256x128_W16: return "256x128 (16 wavefronts)";
+    case TILE_64x64_W8_K2: return "64x64 (8 wavefronts, K split in two)";
     case TILE_128x128_W8_S2: return "128x128 (8 wavefronts, 2 stages)";
   }
   return "?";
@@ -110,7 +111,7 @@ const char* tile_name(int t) {
 // that; and for small problems the smaller of 64x64 and 128x64 by (rounds of resident workgroups) x
 // (tile area), the larger tile on a tie.
 int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
-  // PML_HIP_TILE=64x64|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16 overrides the table (for tuning runs)
+  // PML_HIP_TILE=64x64|64x64w8k2|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
     const std::string v(e);
     if (v == "64x64") return TILE_64x64;
@@ -120,12 +121,16 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
     if (v == "128x128w8") return TILE_128x128_W8;
     if (v == "128x128w8s2") return TILE_128x128_W8_S2;
     if (v == "256x128w16") return TILE_256x128_W16;
+    if (v == "64x64w8k2") return TILE_64x64_W8_K2;
   }
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (n <= 64) return TILE_64x64;  // (the 7x7 stem of ResNet-50 over 2x2 pixel blocks: 191 us against 207 us with 128x64w8)
   if (k_bytes >= 4096 && tiles(256, 128) >= 512) return TILE_256x128_W16;
   if (tiles(128, 128) >= 256) return TILE_128x128_W8_S2;
   if (tiles(128, 128) >= 128) return TILE_128x128_W8;
+  // at most two 64x64 tiles per CU and a long K: a second wavefront grid takes half of every slab
+  // (fp32 1024^3: 32.5 -> 28.8 us; bf16 128x1000x2048: 13.4 -> 11.6 us; bf16 2048^3, 1024 tiles: 26.7 -> 40.5 us)
+  if (tiles(64, 64) <= 512 && k_bytes >= 2048) return TILE_64x64_W8_K2;
   const int64_t rounds_small = (tiles(64, 64) + 5 * 256 - 1) / (5 * 256);
   const int64_t rounds_wide = (tiles(128, 64) + 2 * 256 - 1) / (2 * 256);
   return rounds_small < 2 * rounds_wide ? TILE_64x64 : TILE_128x64;
