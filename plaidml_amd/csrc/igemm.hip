@@ -384,6 +384,35 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
   for (int j = 0; j < 4; ++j) *(i32x4_t*)(Bt + (n + j) * ldbt + k) = out[j];
 }
 
+// The same for 4-byte elements with 16-byte global accesses on both sides: a workgroup turns a 64 x 64
+// tile through LDS (row stride 65 words: the transposed reads touch every bank once).
+// K % 4 == 0, N % 4 == 0, ldb % 4 == 0, ldbt % 4 == 0, both pointers 16-byte aligned.
+__global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __restrict__ B, uint32_t* __restrict__ Bt,
+                                                              int64_t K, int64_t N, int64_t ldb, int64_t ldbt) {
+  __shared__ uint32_t tile[64][65];
+  const int c4 = (threadIdx.x & 15) * 4, r0 = threadIdx.x >> 4;
+  const int64_t k0 = (int64_t)blockIdx.y * 64, n0 = (int64_t)blockIdx.x * 64;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + 16 * i;
+    i32x4_t v = {0, 0, 0, 0};
+    if (k0 + r < K && n0 + c4 < N) v = *(const i32x4_t*)(B + (k0 + r) * ldb + n0 + c4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile[r][c4 + j] = (uint32_t)v[j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = r0 + 16 * i;
+    if (n0 + n < N && k0 + c4 < K) {
+      i32x4_t v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (int)tile[c4 + j][n];
+      *(i32x4_t*)(Bt + (n0 + n) * ldbt + k0 + c4) = v;
+    }
+  }
+}
+
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
@@ -456,6 +485,10 @@ hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int
       hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, s, (const uint16_t*)B, (uint16_t*)Bt, K, N, ldb, ldbt);
       break;
     case 4:
+      if (K % 4 == 0 && N % 4 == 0 && ldb % 4 == 0 && ldbt % 4 == 0 && (((uintptr_t)B | (uintptr_t)Bt) & 15) == 0) {
+        hipLaunchKernelGGL(transpose_words_kernel, grid, dim3(256), 0, s, (const uint32_t*)B, (uint32_t*)Bt, K, N, ldb, ldbt);
+        break;
+      }
       hipLaunchKernelGGL(transpose_kernel<uint32_t>, grid, dim3(256), 0, s, (const uint32_t*)B, (uint32_t*)Bt, K, N, ldb, ldbt);
       break;
     default:
