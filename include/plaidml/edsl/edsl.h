@@ -346,6 +346,19 @@ inline Tensor relu(const Tensor& x, const std::string& name = "") { return intri
 inline Tensor round(const Tensor& x) { return intrinsicCall("round", {x}); }
 inline Tensor sqrt(const Tensor& x) { return intrinsicCall("sqrt", {x}); }
 inline Tensor tanh(const Tensor& x) { return intrinsicCall("tanh", {x}); }
+inline Tensor sin(const Tensor& x) { return intrinsicCall("sin", {x}); }
+inline Tensor cos(const Tensor& x) { return intrinsicCall("cos", {x}); }
+inline Tensor tan(const Tensor& x) { return intrinsicCall("tan", {x}); }
+inline Tensor sinh(const Tensor& x) { return intrinsicCall("sinh", {x}); }
+inline Tensor cosh(const Tensor& x) { return intrinsicCall("cosh", {x}); }
+inline Tensor asin(const Tensor& x) { return intrinsicCall("asin", {x}); }
+inline Tensor acos(const Tensor& x) { return intrinsicCall("acos", {x}); }
+inline Tensor atan(const Tensor& x) { return intrinsicCall("atan", {x}); }
+inline Tensor asinh(const Tensor& x) { return intrinsicCall("asinh", {x}); }
+inline Tensor acosh(const Tensor& x) { return intrinsicCall("acosh", {x}); }
+inline Tensor atanh(const Tensor& x) { return intrinsicCall("atanh", {x}); }
+inline Tensor erf(const Tensor& x) { return intrinsicCall("erf", {x}); }
+inline Tensor pow(const Tensor& x, const Tensor& y) { return intrinsicCall("pow", {x, y}); }
 // a tensor of shape `dims` whose elements are their own coordinate along `axis`
 inline Tensor index(const std::vector<TensorDim>& dims, size_t axis) {
   TensorVec args = {Tensor(static_cast<int64_t>(axis))};
@@ -414,6 +427,12 @@ PLAIDML_EDSL_TENSOR_OPS(<, "cmp_lt")
 PLAIDML_EDSL_TENSOR_OPS(>, "cmp_gt")
 PLAIDML_EDSL_TENSOR_OPS(<=, "cmp_le")
 PLAIDML_EDSL_TENSOR_OPS(>=, "cmp_ge")
+PLAIDML_EDSL_TENSOR_OPS(%, "mod")
+PLAIDML_EDSL_TENSOR_OPS(<<, "bit_shl")
+PLAIDML_EDSL_TENSOR_OPS(>>, "bit_shr")
+PLAIDML_EDSL_TENSOR_OPS(&, "bit_and")
+PLAIDML_EDSL_TENSOR_OPS(|, "bit_or")
+PLAIDML_EDSL_TENSOR_OPS(^, "bit_xor")
 PLAIDML_EDSL_TENSOR_OPS(&&, "logical_and")
 PLAIDML_EDSL_TENSOR_OPS(||, "logical_or")
 #undef PLAIDML_EDSL_TENSOR_OPS

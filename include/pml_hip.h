@@ -110,7 +110,40 @@ enum {
   PML_HIP_EPI_CMP_GE,
   PML_HIP_EPI_CMP_EQ,
   PML_HIP_EPI_CMP_NE,
-  PML_HIP_EPI_MAX_GT    /* v = (v > x) ? v : x  (the lower bound of a clip) */
+  PML_HIP_EPI_MAX_GT,   /* v = (v > x) ? v : x  (the lower bound of a clip) */
+  /* float-only functions (tile.sin ... tile.erf lower to libm calls, pmlc/rt/llvm/builtin.cc:13-26) */
+  PML_HIP_EPI_SIN,
+  PML_HIP_EPI_COS,
+  PML_HIP_EPI_TAN,
+  PML_HIP_EPI_SINH,
+  PML_HIP_EPI_COSH,
+  PML_HIP_EPI_ASIN,
+  PML_HIP_EPI_ACOS,
+  PML_HIP_EPI_ATAN,
+  PML_HIP_EPI_ASINH,
+  PML_HIP_EPI_ACOSH,
+  PML_HIP_EPI_ATANH,
+  PML_HIP_EPI_ERF,
+  PML_HIP_EPI_POW,      /* v = pow(v, x), float result types only */
+  PML_HIP_EPI_RPOW,     /* v = pow(x, v) */
+  PML_HIP_EPI_MOD,      /* v = v % x: fmod for floats, C remainder for integers (0 when x == 0) */
+  PML_HIP_EPI_RMOD,     /* v = x % v */
+  /* integer-only bit operations on the promoted type */
+  PML_HIP_EPI_BIT_AND,
+  PML_HIP_EPI_BIT_OR,
+  PML_HIP_EPI_BIT_XOR,
+  PML_HIP_EPI_BIT_NOT,  /* v = -1 - v */
+  PML_HIP_EPI_SHL,      /* v = v << x */
+  PML_HIP_EPI_RSHL,     /* v = x << v */
+  PML_HIP_EPI_SHR,      /* v = v >> x: arithmetic when the step type is signed, logical when unsigned */
+  PML_HIP_EPI_RSHR,     /* v = x >> v */
+  /* truth-value operations: each side is first tested against zero (ordered for floats, so NaN counts
+   * as false), result BOOL (LogicalOp / LogicalNotOp, pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:311-370) */
+  PML_HIP_EPI_LOGICAL_AND,
+  PML_HIP_EPI_LOGICAL_OR,
+  PML_HIP_EPI_LOGICAL_XOR,
+  PML_HIP_EPI_LOGICAL_NOT, /* v = (v == 0) */
+  PML_HIP_EPI_LAST_ = PML_HIP_EPI_LOGICAL_NOT
 };
 
 /* where the second operand x of a step comes from */

@@ -418,6 +418,46 @@ class Tensor:
     def __ne__(self, r):
         return intrinsic('cmp_ne', self, r)
 
+    # plaidml/edsl/edsl.h:1255,1262-1266 and the unary ~ (edsl.h:1131)
+    def __mod__(self, r):
+        return intrinsic('mod', self, r)
+
+    def __rmod__(self, l):
+        return intrinsic('mod', l, self)
+
+    def __and__(self, r):
+        return intrinsic('bit_and', self, r)
+
+    def __rand__(self, l):
+        return intrinsic('bit_and', l, self)
+
+    def __or__(self, r):
+        return intrinsic('bit_or', self, r)
+
+    def __ror__(self, l):
+        return intrinsic('bit_or', l, self)
+
+    def __xor__(self, r):
+        return intrinsic('bit_xor', self, r)
+
+    def __rxor__(self, l):
+        return intrinsic('bit_xor', l, self)
+
+    def __lshift__(self, r):
+        return intrinsic('bit_shl', self, r)
+
+    def __rlshift__(self, l):
+        return intrinsic('bit_shl', l, self)
+
+    def __rshift__(self, r):
+        return intrinsic('bit_shr', self, r)
+
+    def __rrshift__(self, l):
+        return intrinsic('bit_shr', l, self)
+
+    def __invert__(self):
+        return intrinsic('bit_not', self)
+
     __hash__ = object.__hash__
 
 
@@ -544,6 +584,35 @@ def sqrt(x):
 
 def tanh(x):
     return intrinsic('tanh', x)
+
+
+def _unary(fn):
+    def f(x):
+        return intrinsic(fn, x)
+    f.__name__ = fn
+    return f
+
+
+# plaidml/edsl/edsl.h:1011-1126: one intrinsic per libm function
+sin, cos, tan, sinh, cosh, asin, acos, atan, asinh, acosh, atanh, erf = (
+    _unary(n) for n in ('sin', 'cos', 'tan', 'sinh', 'cosh', 'asin', 'acos', 'atan', 'asinh', 'acosh', 'atanh', 'erf'))
+logical_not = _unary('logical_not')
+
+
+def pow(x, y):  # noqa: A001 - mirrors the EDSL name
+    return intrinsic('pow', x, y)
+
+
+def logical_and(x, y):
+    return intrinsic('logical_and', x, y)
+
+
+def logical_or(x, y):
+    return intrinsic('logical_or', x, y)
+
+
+def logical_xor(x, y):
+    return intrinsic('logical_xor', x, y)
 
 
 def floor(x):
@@ -780,6 +849,11 @@ def contract(agg, combo, out_dt, out_shape, sink, srcs, accs, cons=(), init=None
     return out
 
 
+_LIBM = {'sin': np.sin, 'cos': np.cos, 'tan': np.tan, 'sinh': np.sinh, 'cosh': np.cosh, 'asin': np.arcsin,
+         'acos': np.arccos, 'atan': np.arctan, 'asinh': np.arcsinh, 'acosh': np.arccosh, 'atanh': np.arctanh,
+         'erf': lambda a: np.vectorize(math.erf, otypes=[np.float64])(a.astype(np.float64)).astype(a.dtype)}
+
+
 def _c_round(a):
     # C roundf: half away from zero
     return np.where(a >= 0, np.floor(a + 0.5), np.ceil(a - 0.5)).astype(a.dtype)
@@ -796,9 +870,14 @@ def _eltwise(fn, vals, dts, out_dt):
                     'cmp_ne': lambda x, y: np.logical_and(np.not_equal(x, y), ~(np.isnan(x) | np.isnan(y)))
                     if is_float(ct) else np.not_equal(x, y)}[fn](a, b)
     if fn in _LOGICAL:
-        b = [np.asarray(v) != 0 for v in vals]
+        # LogicalOp / LogicalNotOp (pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:311-370): every operand is
+        # tested against zero in its own type, ordered for floats (ONE / OEQ), so a NaN is neither true nor zero
+        with np.errstate(invalid='ignore'):
+            if fn == 'logical_not':
+                return np.asarray(vals[0]) == 0
+            b = [(np.asarray(v) < 0) | (np.asarray(v) > 0) for v in vals]
         return {'logical_and': lambda: b[0] & b[1], 'logical_or': lambda: b[0] | b[1],
-                'logical_xor': lambda: b[0] ^ b[1], 'logical_not': lambda: ~b[0]}[fn]()
+                'logical_xor': lambda: b[0] ^ b[1]}[fn]()
     if fn == 'select':
         t = convert(vals[1], dts[1], out_dt)
         f = convert(vals[2], dts[2], out_dt)
@@ -839,6 +918,41 @@ def _eltwise(fn, vals, dts, out_dt):
             r = np.ceil(p[0])
         elif fn == 'round':
             r = _c_round(p[0])
+        elif fn in _LIBM:
+            # float operands only (OperandsAre / ResultIs<EltwiseFloat>, tile_to_linalg.cc:1271-1311); the
+            # reference calls libm (pmlc/rt/llvm/builtin.cc:13-26)
+            if not is_float(out_dt):
+                raise TypeError("'%s' needs floating-point operands" % fn)
+            r = _LIBM[fn](p[0])
+        elif fn == 'pow':
+            if not is_float(out_dt):
+                raise TypeError("'pow' needs floating-point operands")
+            r = np.power(p[0], p[1])
+        elif fn == 'mod':
+            # RemFOp / RemSIOp / RemUIOp (tile_to_linalg.cc:1326-1331): the sign follows the dividend.  An
+            # integer remainder by zero is undefined in the reference; 0 here, as on the device.
+            if is_float(out_dt):
+                r = np.fmod(p[0], p[1])
+            else:
+                safe = np.where(p[1] == 0, np.ones_like(p[1]), p[1])
+                r = np.where(p[1] == 0, np.zeros_like(p[0]), np.fmod(p[0], safe))
+        elif fn in ('bit_and', 'bit_or', 'bit_xor', 'bit_not', 'bit_shl', 'bit_shr'):
+            # integer operands only (tile_to_linalg.cc:1356-1369)
+            if is_float(out_dt):
+                raise TypeError("'%s' needs integer operands" % fn)
+            if fn == 'bit_and':
+                r = p[0] & p[1]
+            elif fn == 'bit_or':
+                r = p[0] | p[1]
+            elif fn == 'bit_xor':
+                r = p[0] ^ p[1]
+            elif fn == 'bit_not':
+                r = ~p[0]  # -1 - x (NotOp, tile_to_linalg.cc:238-247)
+            elif fn == 'bit_shl':
+                r = np.left_shift(p[0], p[1])
+            else:
+                # ShRSIOp for signed, ShRUIOp for unsigned: numpy's >> follows the operand's signedness too
+                r = np.right_shift(p[0], p[1])
         else:
             raise NotImplementedError(fn)
     return _store(r, out_dt)

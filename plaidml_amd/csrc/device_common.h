@@ -294,6 +294,38 @@ __device__ inline Scalar<FT, IT> run_tail(const pml_hip_epilogue& t, Scalar<FT, 
         case PML_HIP_EPI_CMP_EQ: is_cmp = true; cmp = a == b; break;
         case PML_HIP_EPI_CMP_NE: is_cmp = true; cmp = (a < b) || (a > b); break;  // ordered not-equal
         case PML_HIP_EPI_MAX_GT: r = (a > b) ? a : b; break;
+#define PML_MATH1(OP, FN) \
+  case OP: r = sizeof(FT) == 4 || dt != PML_HIP_F64 ? (FT)FN##f((float)a) : (FT)FN((double)a); break;
+        PML_MATH1(PML_HIP_EPI_SIN, sin)
+        PML_MATH1(PML_HIP_EPI_COS, cos)
+        PML_MATH1(PML_HIP_EPI_TAN, tan)
+        PML_MATH1(PML_HIP_EPI_SINH, sinh)
+        PML_MATH1(PML_HIP_EPI_COSH, cosh)
+        PML_MATH1(PML_HIP_EPI_ASIN, asin)
+        PML_MATH1(PML_HIP_EPI_ACOS, acos)
+        PML_MATH1(PML_HIP_EPI_ATAN, atan)
+        PML_MATH1(PML_HIP_EPI_ASINH, asinh)
+        PML_MATH1(PML_HIP_EPI_ACOSH, acosh)
+        PML_MATH1(PML_HIP_EPI_ATANH, atanh)
+        PML_MATH1(PML_HIP_EPI_ERF, erf)
+#undef PML_MATH1
+        case PML_HIP_EPI_POW:
+          r = sizeof(FT) == 4 || dt != PML_HIP_F64 ? (FT)powf((float)a, (float)b) : (FT)pow((double)a, (double)b);
+          break;
+        case PML_HIP_EPI_RPOW:
+          r = sizeof(FT) == 4 || dt != PML_HIP_F64 ? (FT)powf((float)b, (float)a) : (FT)pow((double)b, (double)a);
+          break;
+        case PML_HIP_EPI_MOD:
+          r = sizeof(FT) == 4 || dt != PML_HIP_F64 ? (FT)fmodf((float)a, (float)b) : (FT)fmod((double)a, (double)b);
+          break;
+        case PML_HIP_EPI_RMOD:
+          r = sizeof(FT) == 4 || dt != PML_HIP_F64 ? (FT)fmodf((float)b, (float)a) : (FT)fmod((double)b, (double)a);
+          break;
+        // truth values: ordered "not equal to zero", so a NaN is false
+        case PML_HIP_EPI_LOGICAL_AND: is_cmp = true; cmp = (a < 0 || a > 0) && (b < 0 || b > 0); break;
+        case PML_HIP_EPI_LOGICAL_OR: is_cmp = true; cmp = (a < 0 || a > 0) || (b < 0 || b > 0); break;
+        case PML_HIP_EPI_LOGICAL_XOR: is_cmp = true; cmp = (a < 0 || a > 0) != (b < 0 || b > 0); break;
+        case PML_HIP_EPI_LOGICAL_NOT: is_cmp = true; cmp = a == (FT)0; break;
         default: break;
       }
       v.f = round_float_to<FT>(dt, r);
@@ -318,6 +350,30 @@ __device__ inline Scalar<FT, IT> run_tail(const pml_hip_epilogue& t, Scalar<FT, 
         case PML_HIP_EPI_CMP_EQ: is_cmp = true; cmp = a == b; break;
         case PML_HIP_EPI_CMP_NE: is_cmp = true; cmp = a != b; break;
         case PML_HIP_EPI_MAX_GT: r = (uns ? (ua > ub) : (a > b)) ? a : b; break;
+        case PML_HIP_EPI_MOD: r = b == 0 ? 0 : (uns ? (IT)(ua % ub) : a % b); break;
+        case PML_HIP_EPI_RMOD: r = a == 0 ? 0 : (uns ? (IT)(ub % ua) : b % a); break;
+        case PML_HIP_EPI_BIT_AND: r = a & b; break;
+        case PML_HIP_EPI_BIT_OR: r = a | b; break;
+        case PML_HIP_EPI_BIT_XOR: r = a ^ b; break;
+        case PML_HIP_EPI_BIT_NOT: r = (IT)((UT)-1 - ua); break;
+        // shift counts at or beyond the type's width are undefined in the reference: 0 here (sign fill for
+        // an arithmetic right shift)
+        case PML_HIP_EPI_SHL: r = ub >= sizeof(IT) * 8 ? 0 : (IT)(ua << ub); break;
+        case PML_HIP_EPI_RSHL: r = ua >= sizeof(IT) * 8 ? 0 : (IT)(ub << ua); break;
+        case PML_HIP_EPI_SHR: {
+          const UT n = ub >= sizeof(IT) * 8 ? (UT)(sizeof(IT) * 8 - 1) : ub;
+          r = uns ? (ub >= sizeof(IT) * 8 ? 0 : (IT)(ua >> n)) : (a >> n);
+          break;
+        }
+        case PML_HIP_EPI_RSHR: {
+          const UT n = ua >= sizeof(IT) * 8 ? (UT)(sizeof(IT) * 8 - 1) : ua;
+          r = uns ? (ua >= sizeof(IT) * 8 ? 0 : (IT)(ub >> n)) : (b >> n);
+          break;
+        }
+        case PML_HIP_EPI_LOGICAL_AND: is_cmp = true; cmp = a != 0 && b != 0; break;
+        case PML_HIP_EPI_LOGICAL_OR: is_cmp = true; cmp = a != 0 || b != 0; break;
+        case PML_HIP_EPI_LOGICAL_XOR: is_cmp = true; cmp = (a != 0) != (b != 0); break;
+        case PML_HIP_EPI_LOGICAL_NOT: is_cmp = true; cmp = a == 0; break;
         default: break;
       }
       v.i = wrap_int_to<IT>(dt, r);

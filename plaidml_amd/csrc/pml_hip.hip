@@ -227,7 +227,7 @@ bool valid_tail(const pml_hip_epilogue& t) {
   if (t.n_operands < 0 || t.n_operands > PML_HIP_MAX_EPI_OPERANDS) return false;
   for (int i = 0; i < t.n_ops; ++i) {
     const pml_hip_epi_op& op = t.ops[i];
-    if (op.opcode < PML_HIP_EPI_ADD || op.opcode > PML_HIP_EPI_MAX_GT) return false;
+    if (op.opcode < PML_HIP_EPI_ADD || op.opcode > PML_HIP_EPI_LAST_) return false;
     if (op.operand_kind == PML_HIP_OPND_TENSOR && (op.operand < 0 || op.operand >= t.n_operands)) return false;
     if (op.opcode == PML_HIP_EPI_STORE && (op.operand < 0 || op.operand >= PML_HIP_MAX_EPI_OPERANDS)) return false;
     if (dt_size(op.dtype) == 8 && op.opcode != PML_HIP_EPI_STORE) return false;  // 64-bit steps: general path only

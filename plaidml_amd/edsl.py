@@ -516,6 +516,45 @@ class Tensor(_Handle):
     def __ge__(self, r):
         return intrinsic('cmp_ge', self, r)
 
+    def __mod__(self, r):
+        return intrinsic('mod', self, r)
+
+    def __rmod__(self, l):
+        return intrinsic('mod', l, self)
+
+    def __and__(self, r):
+        return intrinsic('bit_and', self, r)
+
+    def __rand__(self, l):
+        return intrinsic('bit_and', l, self)
+
+    def __or__(self, r):
+        return intrinsic('bit_or', self, r)
+
+    def __ror__(self, l):
+        return intrinsic('bit_or', l, self)
+
+    def __xor__(self, r):
+        return intrinsic('bit_xor', self, r)
+
+    def __rxor__(self, l):
+        return intrinsic('bit_xor', l, self)
+
+    def __lshift__(self, r):
+        return intrinsic('bit_shl', self, r)
+
+    def __rlshift__(self, l):
+        return intrinsic('bit_shl', l, self)
+
+    def __rshift__(self, r):
+        return intrinsic('bit_shr', self, r)
+
+    def __rrshift__(self, l):
+        return intrinsic('bit_shr', l, self)
+
+    def __invert__(self):
+        return intrinsic('bit_not', self)
+
     __hash__ = object.__hash__
 
     def compute_shape(self):
@@ -655,6 +694,25 @@ def _unary(fn):
 
 ceil, exp, floor, ident, log, relu, sqrt, tanh = (_unary(n) for n in ('ceil', 'exp', 'floor', 'ident', 'log', 'relu', 'sqrt', 'tanh'))
 round = _unary('round')  # noqa: A001
+sin, cos, tan, sinh, cosh, asin, acos, atan, asinh, acosh, atanh, erf = (
+    _unary(n) for n in ('sin', 'cos', 'tan', 'sinh', 'cosh', 'asin', 'acos', 'atan', 'asinh', 'acosh', 'atanh', 'erf'))
+logical_not = _unary('logical_not')
+
+
+def pow(x, y):  # noqa: A001
+    return intrinsic('pow', x, y)
+
+
+def logical_and(x, y):
+    return intrinsic('logical_and', x, y)
+
+
+def logical_or(x, y):
+    return intrinsic('logical_or', x, y)
+
+
+def logical_xor(x, y):
+    return intrinsic('logical_xor', x, y)
 
 
 def max(x, y):  # noqa: A001

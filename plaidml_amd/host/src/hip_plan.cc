@@ -351,10 +351,26 @@ class Planner {
     static const std::map<std::string, int> m = {
         {"relu", PML_HIP_EPI_RELU}, {"neg", PML_HIP_EPI_NEG},     {"exp", PML_HIP_EPI_EXP},   {"log", PML_HIP_EPI_LOG},
         {"sqrt", PML_HIP_EPI_SQRT}, {"tanh", PML_HIP_EPI_TANH},   {"floor", PML_HIP_EPI_FLOOR}, {"ceil", PML_HIP_EPI_CEIL},
-        {"round", PML_HIP_EPI_ROUND}};
+        {"round", PML_HIP_EPI_ROUND}, {"sin", PML_HIP_EPI_SIN},     {"cos", PML_HIP_EPI_COS},   {"tan", PML_HIP_EPI_TAN},
+        {"sinh", PML_HIP_EPI_SINH}, {"cosh", PML_HIP_EPI_COSH},   {"asin", PML_HIP_EPI_ASIN}, {"acos", PML_HIP_EPI_ACOS},
+        {"atan", PML_HIP_EPI_ATAN}, {"asinh", PML_HIP_EPI_ASINH}, {"acosh", PML_HIP_EPI_ACOSH}, {"atanh", PML_HIP_EPI_ATANH},
+        {"erf", PML_HIP_EPI_ERF},   {"bit_not", PML_HIP_EPI_BIT_NOT}, {"logical_not", PML_HIP_EPI_LOGICAL_NOT}};
     auto it = m.find(fn);
     return it == m.end() ? 0 : it->second;
   }
+  // The operand types an operation accepts (the OperandsAre / ResultIs predicates of the eltwise pattern
+  // table, pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:1271-1385): `dt` is the type the step computes in.
+  static void checkStepType(const std::string& fn, DataType dt) {
+    static const std::set<std::string> float_only = {"sin",  "cos",   "tan",   "sinh",  "cosh", "asin", "acos",
+                                                     "atan", "asinh", "acosh", "atanh", "erf",  "pow"};
+    static const std::set<std::string> int_only = {"bit_and", "bit_or", "bit_xor", "bit_not", "bit_shl", "bit_shr"};
+    if (float_only.count(fn) && !util::isFloat(dt))
+      throw std::runtime_error("'" + fn + "' needs floating-point operands, got " + util::mnemonic(dt));
+    if (int_only.count(fn) && !util::isInteger(dt))
+      throw std::runtime_error("'" + fn + "' needs integer operands, got " + util::mnemonic(dt));
+  }
+  // comparisons and truth-value operations compute in their operands' promoted type and yield i1
+  static bool computesInOperandType(const std::string& fn) { return ast::isCompareOp(fn) || ast::isLogicalOp(fn); }
   // opcode when the running value is the first / second operand (0 = not expressible)
   static int binaryOpcode(const std::string& fn, bool running_first) {
     struct E { int first, second; };
@@ -363,6 +379,13 @@ class Planner {
         {"mul", {PML_HIP_EPI_MUL, PML_HIP_EPI_MUL}},       {"div", {PML_HIP_EPI_DIV, PML_HIP_EPI_RDIV}},
         {"max", {PML_HIP_EPI_MAX, 0}},                     {"min", {PML_HIP_EPI_MIN, 0}},
         {"maxgt", {PML_HIP_EPI_MAX_GT, 0}},
+        {"pow", {PML_HIP_EPI_POW, PML_HIP_EPI_RPOW}},      {"mod", {PML_HIP_EPI_MOD, PML_HIP_EPI_RMOD}},
+        {"bit_and", {PML_HIP_EPI_BIT_AND, PML_HIP_EPI_BIT_AND}}, {"bit_or", {PML_HIP_EPI_BIT_OR, PML_HIP_EPI_BIT_OR}},
+        {"bit_xor", {PML_HIP_EPI_BIT_XOR, PML_HIP_EPI_BIT_XOR}}, {"bit_shl", {PML_HIP_EPI_SHL, PML_HIP_EPI_RSHL}},
+        {"bit_shr", {PML_HIP_EPI_SHR, PML_HIP_EPI_RSHR}},
+        {"logical_and", {PML_HIP_EPI_LOGICAL_AND, PML_HIP_EPI_LOGICAL_AND}},
+        {"logical_or", {PML_HIP_EPI_LOGICAL_OR, PML_HIP_EPI_LOGICAL_OR}},
+        {"logical_xor", {PML_HIP_EPI_LOGICAL_XOR, PML_HIP_EPI_LOGICAL_XOR}},
         {"cmp_lt", {PML_HIP_EPI_CMP_LT, PML_HIP_EPI_CMP_GT}}, {"cmp_gt", {PML_HIP_EPI_CMP_GT, PML_HIP_EPI_CMP_LT}},
         {"cmp_le", {PML_HIP_EPI_CMP_LE, PML_HIP_EPI_CMP_GE}}, {"cmp_ge", {PML_HIP_EPI_CMP_GE, PML_HIP_EPI_CMP_LE}},
         {"cmp_eq", {PML_HIP_EPI_CMP_EQ, PML_HIP_EPI_CMP_EQ}}, {"cmp_ne", {PML_HIP_EPI_CMP_NE, PML_HIP_EPI_CMP_NE}}};
@@ -465,7 +488,10 @@ class Planner {
         } else {
           step.opcode = unaryOpcode(u.fn);
           if (!step.opcode) return;
-          step.dtype = hipType(rdt);
+          const DataType sdt = computesInOperandType(u.fn) ? cur->shape.elementType : rdt;
+          checkStepType(u.fn, sdt);
+          step.dtype = hipType(sdt);
+          if (!allow64 && is64(sdt)) return;
         }
         if (!allow64 && is64(rdt)) return;
       } else if (u.operands.size() == 2) {
@@ -476,10 +502,11 @@ class Planner {
         if (!step.opcode) return;
         // arithmetic happens in the promoted operand type; comparisons too, their result is i1
         DataType cdt = rdt;
-        if (ast::isCompareOp(u.fn)) {
+        if (computesInOperandType(u.fn)) {
           cdt = other->kind == Value::Literal ? cur->shape.elementType
                                               : util::promoteTypes(cur->shape.elementType, other->shape.elementType);
         }
+        checkStepType(u.fn, cdt);
         if (!allow64 && (is64(cdt) || is64(other->shape.elementType))) return;
         step.dtype = hipType(cdt);
         if (other->kind == Value::Literal) {
@@ -537,7 +564,11 @@ class Planner {
     if (tb.tail.n_ops == 0) return "";
     static const char* names[] = {"?",    "add",  "sub",   "rsub", "mul",   "div",  "rdiv",  "max",  "min",
                                   "relu", "neg",  "exp",   "log",  "sqrt",  "tanh", "floor", "ceil", "round",
-                                  "cast", "store", "lt",   "gt",   "le",    "ge",   "eq",    "ne",   "maxgt"};
+                                  "cast", "store", "lt",   "gt",   "le",    "ge",   "eq",    "ne",   "maxgt",
+                                  "sin",  "cos",  "tan",   "sinh", "cosh",  "asin", "acos",  "atan", "asinh",
+                                  "acosh", "atanh", "erf", "pow",  "rpow",  "mod",  "rmod",  "and",  "or",
+                                  "xor",  "not",  "shl",   "rshl", "shr",   "rshr", "land",  "lor",  "lxor", "lnot"};
+    static_assert(sizeof(names) / sizeof(names[0]) == PML_HIP_EPI_LAST_ + 1, "one name per opcode");
     std::stringstream ss;
     ss << " tail=[";
     for (int i = 0; i < tb.tail.n_ops; ++i) {
@@ -668,7 +699,9 @@ class Planner {
         if (op.fn != "ident") {
           step.opcode = unaryOpcode(op.fn);
           if (!step.opcode) throw std::runtime_error("elementwise operation '" + op.fn + "' is not supported by the hip target");
-          step.dtype = hipType(rdt);
+          const DataType sdt = computesInOperandType(op.fn) ? main->shape.elementType : rdt;
+          checkStepType(op.fn, sdt);
+          step.dtype = hipType(sdt);
         }
       } else if (op.operands.size() == 2) {
         const bool first = main_pos == 0;
@@ -681,9 +714,10 @@ class Planner {
         }
         if (!step.opcode) throw std::runtime_error("elementwise operation '" + op.fn + "' is not supported by the hip target");
         DataType cdt = rdt;
-        if (ast::isCompareOp(op.fn))
+        if (computesInOperandType(op.fn))
           cdt = other->kind == Value::Literal ? main->shape.elementType
                                               : util::promoteTypes(main->shape.elementType, other->shape.elementType);
+        checkStepType(op.fn, cdt);
         step.dtype = hipType(cdt);
         if (other->kind == Value::Literal) {
           step.operand_kind = PML_HIP_OPND_IMM;

@@ -237,6 +237,55 @@ void caseOpLibrary() {
   }
 }
 
+// Operators and libm intrinsics of the header, with the reference's own answers
+// (plaidml/edsl/tests/edsl_test.cc: BitRightScalar :273-287, BitNot :289-302, EltwiseMod :606-629,
+// LogicalAnd_mixed :1223-1241, LogicalNot_float :1315-1328, Pow :1796-1817, Tan :1857-1873).
+void caseIntrinsics() {
+  {
+    auto A = Placeholder(DType::UINT64, {3, 3});
+    std::vector<uint64_t> a, want;
+    for (uint64_t k = 1; k <= 9; ++k) {
+      a.push_back(k << (9 + k));
+      want.push_back(k << k);
+    }
+    auto out = run(buildProgram("bit_right_scalar", {A}, {A >> 9}), {makeBuffer<uint64_t>(DType::UINT64, {3, 3}, a)});
+    expectEq<uint64_t>("bit_right_scalar", readBuffer<uint64_t>(out[0]), want);
+  }
+  {
+    auto A = Placeholder(DType::UINT8, {3, 3});
+    auto out = run(buildProgram("bit_not", {A}, {~A}),
+                   {makeBuffer<uint8_t>(DType::UINT8, {3, 3}, {0x00, 0x01, 0x02, 0x10, 0x11, 0x22, 0xF0, 0x0F, 0xFF})});
+    expectEq<uint8_t>("bit_not", readBuffer<uint8_t>(out[0]), {0xFF, 0xFE, 0xFD, 0xEF, 0xEE, 0xDD, 0x0F, 0xF0, 0x00});
+  }
+  {
+    auto A = Placeholder(DType::INT32, {3, 3});
+    auto B = Placeholder(DType::INT32, {3, 3});
+    auto out = run(buildProgram("mod", {A, B}, {A % B}), {makeBuffer<int32_t>(DType::INT32, {3, 3}, {2, 4, 8, 16, 32, 64, 128, 256, 512}),
+                                                          makeBuffer<int32_t>(DType::INT32, {3, 3}, {1, 2, 3, 4, 5, 6, 7, 8, 9})});
+    expectEq<int32_t>("mod", readBuffer<int32_t>(out[0]), {2 % 1, 4 % 2, 8 % 3, 16 % 4, 32 % 5, 64 % 6, 128 % 7, 256 % 8, 512 % 9});
+  }
+  {
+    auto A = Placeholder(DType::UINT64, {3, 3});
+    auto B = Placeholder(DType::FLOAT32, {3, 3});
+    auto out = run(buildProgram("logical_and", {A, B}, {A && B, !B}),
+                   {makeBuffer<uint64_t>(DType::UINT64, {3, 3}, {1, 2, 3, 4, 0, 6, 7, 0, 9}),
+                    makeBuffer<float>(DType::FLOAT32, {3, 3}, {10, 11, 12, 13, 0, 15, 16, 17, 18})});
+    expectEq<int8_t>("logical_and_mixed", readBuffer<int8_t>(out[0]), {1, 1, 1, 1, 0, 1, 1, 0, 1});
+    expectEq<int8_t>("logical_not_float", readBuffer<int8_t>(out[1]), {0, 0, 0, 0, 1, 0, 0, 0, 0});
+  }
+  {
+    auto A = Placeholder(DType::FLOAT32, {3, 3});
+    auto B = Placeholder(DType::FLOAT32, {3, 3});
+    auto out = run(buildProgram("pow_tan", {A, B}, {pow(A, B), tan(B * 0.4)}),
+                   {makeBuffer<float>(DType::FLOAT32, {3, 3}, {0.5, 1.5, 2.5, 0.5, 1.5, 2.5, 0.5, 1.5, 2.5}),
+                    makeBuffer<float>(DType::FLOAT32, {3, 3}, {0.5, 0.5, 0.5, 1.5, 1.5, 1.5, 2.5, 2.5, 2.5})});
+    expectClose("pow", readBuffer<float>(out[0]), {0.707107, 1.22474, 1.58114, 0.353553, 1.83712, 3.95285, 0.176777, 2.75568, 9.88212},
+                2e-5f, 0.f);
+    expectClose("tan", readBuffer<float>(out[1]), {0.20271, 0.20271, 0.20271, 0.684137, 0.684137, 0.684137, 1.55741, 1.55741, 1.55741},
+                2e-4f, 0.f);
+  }
+}
+
 void caseErrors() {
   auto A = Placeholder(DType::FLOAT32, {4, 4});
   auto program = buildProgram("ident", {A}, {A + 1.0});
@@ -272,6 +321,7 @@ int main() {
     caseInt8Gemm();
     caseConvRelu();
     caseOpLibrary();
+    caseIntrinsics();
     caseErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAILED with exception: %s\n", e.what());

@@ -100,6 +100,47 @@ def eltwise_mix(E, op):
                                                      r.uniform(-0.2, 0.2, (3, 1)).astype(np.float32)], EXACT
 
 
+def libm_tail_f32(E, op, M=24, N=40, K=16):
+    """Float intrinsics as the fused tail of a contraction and with broadcast operands: dot -> sin -> erf,
+    pow with a per-column exponent, fmod, tan/atan/sinh chains (single ops pinned by tests/intrinsic_cases.py)."""
+    A = E.Placeholder(E.DType.FLOAT32, [M, K])
+    B = E.Placeholder(E.DType.FLOAT32, [K, N])
+    P = E.Placeholder(E.DType.FLOAT32, [N])
+    i, j, k = E.TensorIndexes(3)
+    C = E.Contraction().outShape(M, N).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    S = E.erf(E.sin(C)) + E.cos(C)
+    W = E.pow(E.abs(C) + 0.5, P) % 1.5
+    T = E.atan(E.sinh(E.tanh(C))) - E.asinh(C) + E.cosh(E.tan(C * 0.1))
+    U = E.asin(E.tanh(C)) + E.acos(E.tanh(C)) + E.atanh(E.tanh(C) * 0.5) + E.acosh(E.abs(C) + 1.0)
+    r = _rng(21)
+    return E.Program('libm_tail', [A, B, P], [S, W, T, U]), [r.uniform(-1, 1, (M, K)).astype(np.float32),
+                                                            r.uniform(-1, 1, (K, N)).astype(np.float32),
+                                                            r.uniform(0.5, 2.5, (N,)).astype(np.float32)], FP32
+
+
+def bits_and_truth(E, op):
+    """Integer bit operations with mixed widths, broadcasting and immediates, and truth-value operations on
+    floats with NaNs (ordered compares: pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:311-370)."""
+    A = E.Placeholder(E.DType.INT32, [6, 8])
+    B = E.Placeholder(E.DType.INT32, [8])
+    Cc = E.Placeholder(E.DType.UINT8, [6, 1])
+    F = E.Placeholder(E.DType.FLOAT32, [6, 8])
+    X = ((A & B) | (A << 3)) ^ (~B)
+    Y = (A >> 2) % 7 + (1 << Cc)
+    Z = (Cc >> 1) | 0x80
+    L = E.logical_xor(E.logical_and(F, A), E.logical_or(E.logical_not(F), B))
+    r = _rng(22)
+    f = r.uniform(-1, 1, (6, 8)).astype(np.float32)
+    f[r.uniform(size=f.shape) < 0.3] = 0.0
+    f[0, 0] = np.nan
+    f[1, 3] = -0.0
+    a = r.integers(-1000, 1000, (6, 8)).astype(np.int32)
+    a[2, 2] = 0
+    b = r.integers(-50, 50, (8,)).astype(np.int32)
+    b[1] = 0
+    return E.Program('bits', [A, B, Cc, F], [X, Y, Z, L]), [a, b, r.integers(0, 8, (6, 1)).astype(np.uint8), f], EXACT
+
+
 def u64_add(E, op):
     """CppEdsl.Add, plaidml/edsl/tests/edsl_test.cc:335-374 (64-bit integer elementwise)."""
     A = E.Placeholder(E.DType.UINT64, [3, 3])
@@ -265,6 +306,8 @@ ALL = {
     'max_rows': max_rows,
     'use_default': use_default,
     'eltwise_mix': eltwise_mix,
+    'libm_tail_f32': libm_tail_f32,
+    'bits_and_truth': bits_and_truth,
     'u64_add': u64_add,
     'higher_precision_constants': higher_precision_constants,
     'config0_gemm_f32': config0_gemm_f32,

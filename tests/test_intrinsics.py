@@ -1,0 +1,76 @@
+"""Elementwise intrinsics beyond the arithmetic set (libm functions, pow, mod, bit and truth-value operations):
+the oracle and the hip device against the answers held by the reference's tests (tests/intrinsic_cases.py)."""
+import numpy as np
+import pytest
+
+import intrinsic_cases as IC
+from oracle import tile_oracle as OE
+
+NAMES = sorted(IC.CASES)
+
+
+@pytest.mark.parametrize('name', NAMES)
+def test_oracle_reproduces_reference_answers(name):
+    IC.check_case(name, IC.run_case(name, OE))
+
+
+def test_oracle_truth_values_are_ordered_compares():
+    """A NaN is neither non-zero (ONE) nor zero (OEQ): LogicalOp / LogicalNotOp,
+    pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:311-370."""
+    a = OE.Placeholder(OE.DType.FLOAT32, [4])
+    b = OE.Placeholder(OE.DType.FLOAT32, [4])
+    outs = [OE.logical_and(a, b), OE.logical_or(a, b), OE.logical_xor(a, b), OE.logical_not(a)]
+    x = np.array([np.nan, np.nan, 0.0, 2.0], np.float32)
+    y = np.array([1.0, 0.0, np.nan, -0.0], np.float32)
+    land, lor, lxor, lnot = OE.run(OE.Program('truth', [a, b], outs), [x, y])
+    np.testing.assert_array_equal(land, [False, False, False, False])
+    np.testing.assert_array_equal(lor, [True, False, False, True])
+    np.testing.assert_array_equal(lxor, [True, False, False, True])
+    np.testing.assert_array_equal(lnot, [False, False, True, False])
+
+
+def test_oracle_rejects_wrong_operand_kinds():
+    f = OE.Placeholder(OE.DType.FLOAT32, [3])
+    i = OE.Placeholder(OE.DType.INT32, [3])
+    with pytest.raises(TypeError):
+        OE.run(OE.Program('p', [f], [f & f]), [np.zeros(3, np.float32)])
+    with pytest.raises(TypeError):
+        OE.run(OE.Program('p', [i], [OE.sin(i)]), [np.zeros(3, np.int32)])
+
+
+def test_oracle_signed_shift_and_remainder_follow_c():
+    a = OE.Placeholder(OE.DType.INT32, [4])
+    b = OE.Placeholder(OE.DType.INT32, [4])
+    x = np.array([-17, 17, -16, 5], np.int32)
+    y = np.array([5, -5, 2, 0], np.int32)
+    rem, shr = OE.run(OE.Program('p', [a, b], [a % b, a >> 2]), [x, y])
+    np.testing.assert_array_equal(rem, [-2, 2, 0, 0])      # truncated division; x % 0 is pinned to 0
+    np.testing.assert_array_equal(shr, [-5, 4, -4, 1])     # arithmetic shift for a signed operand
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('target', ['hip', 'hip{specialise=0,fuse=0}'])
+@pytest.mark.parametrize('name', NAMES)
+def test_hip_reproduces_reference_answers(name, target):
+    from plaidml_amd import edsl as E
+    print('intrinsic', name, 'target', target, flush=True)
+    c = IC.CASES[name]
+    ins, out = c['build'](E)
+    got = E.run(E.Program(name, ins, [out]), c['inputs'], target=target)[0]
+    IC.check_case(name, got)
+    ref = IC.run_case(name, OE)
+    if c['tol'] is None:
+        np.testing.assert_array_equal(got, ref)
+    else:
+        np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_hip_rejects_wrong_operand_kinds():
+    from plaidml_amd import edsl as E
+    f = E.Placeholder(E.DType.FLOAT32, [3])
+    with pytest.raises(E.PlaidMLError, match='needs integer operands'):
+        E.run(E.Program('p', [f], [f & f]), [np.zeros(3, np.float32)])
+    i = E.Placeholder(E.DType.INT32, [3])
+    with pytest.raises(E.PlaidMLError, match='needs floating-point operands'):
+        E.run(E.Program('p', [i], [E.sin(i)]), [np.zeros(3, np.int32)])
