@@ -104,8 +104,10 @@ class TensorLens {
   TensorLens() = default;
   TensorLens(const std::string& source, const std::string& target) {
     if (source.size() != target.size()) throw ffi_exception("source and target rank mismatch in TensorLens");
-    for (char c : target) {
-      auto pos = source.find(c);
+    // entry i of the tensor's own order (source) is taken from where its letter sits in the order the
+    // caller writes dims and indices in (target)
+    for (char c : source) {
+      auto pos = target.find(c);
       if (pos == std::string::npos) throw ffi_exception("source and target dims mismatch in TensorLens");
       map_.push_back(pos);
     }
@@ -524,6 +526,13 @@ inline Value as_value(int v) { return Value(static_cast<int64_t>(v)); }
 inline Value as_value(int64_t v) { return Value(v); }
 inline Value as_value(uint64_t v) { return Value(v); }
 inline Value as_value(double v) { return Value(v); }
+// a vector among the elements becomes a nested tuple
+template <typename T>
+Value as_value(const std::vector<T>& v) {
+  std::vector<Value> vec;
+  for (const auto& e : v) vec.push_back(as_value(e));
+  return Value(vec);
+}
 }  // namespace details
 
 template <typename... Ts>

@@ -33,6 +33,7 @@ enum class GroupLayout { NONE, SEPARATE, IN_C, IN_K, _LAST };
 enum class PoolMode { AVG, MAX, MIN, SUM, _LAST };
 enum class TensorLayout { NXC, NCX, KCX, XCK, GKCX, XGCK, _LAST };
 enum class PadMode { CONSTANT, EDGE, REFLECT, SYMMETRIC, _LAST };
+enum class EpsMode { ADD, MAX, _LAST };
 // reshape: take the dimension from the input / infer it from the element count
 static const int AUTO_DIM_MATCH = 0;
 static const int AUTO_DIM_FILL = -1;
@@ -47,6 +48,122 @@ struct Integers {
   Integers(const std::initializer_list<int64_t>& elts) : Integers(std::vector<int64_t>(elts)) {}   // NOLINT
   Integers(const std::initializer_list<size_t>& elts) : Integers(std::vector<size_t>(elts)) {}     // NOLINT
   edsl::Value value;
+};
+
+inline edsl::Tensor all(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
+  return details::op("all", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+
+inline edsl::Tensor any(const edsl::Tensor& I, const edsl::Value& axes = edsl::None(), bool keepdims = false) {
+  return details::op("any", edsl::make_tuple(I, axes, keepdims)).as_tensor();
+}
+
+inline edsl::Tensor binary_crossentropy(const edsl::Tensor& I, const edsl::Tensor& O, double epsilon) {
+  return details::op("binary_crossentropy", edsl::make_tuple(I, O, epsilon)).as_tensor();
+}
+
+inline edsl::Tensor broadcast(const edsl::Tensor& I, const std::vector<int64_t>& result_shape,
+                              const std::vector<int64_t>& bcast_axes) {
+  return details::op("broadcast", edsl::make_tuple(I, edsl::make_tuple(result_shape), edsl::make_tuple(bcast_axes))).as_tensor();
+}
+
+inline edsl::Tensor cumprod(const edsl::Tensor& I, int axis) { return details::op("cumprod", edsl::make_tuple(I, axis)).as_tensor(); }
+
+class l2norm {
+ public:
+  explicit l2norm(const edsl::Tensor& I, const std::vector<int64_t> axes) : I_(I), axes_(axes) {}
+  l2norm& epsilon(float epsilon) { epsilon_ = epsilon; return *this; }
+  l2norm& eps_mode(EpsMode eps_mode) { eps_mode_ = eps_mode; return *this; }
+  operator edsl::Tensor() const {
+    return details::op("l2norm", edsl::make_tuple(I_, edsl::make_tuple(axes_), epsilon_, static_cast<int>(eps_mode_))).as_tensor();
+  }
+
+ private:
+  edsl::Tensor I_;
+  std::vector<int64_t> axes_;
+  double epsilon_ = 0;
+  EpsMode eps_mode_ = EpsMode::ADD;
+};
+
+class lrn {
+ public:
+  explicit lrn(const edsl::Tensor& I, const std::vector<int64_t>& window_size) : I_(I), window_size_(window_size) {}
+  lrn& alpha(double alpha) { alpha_ = alpha; return *this; }
+  lrn& beta(double beta) { beta_ = beta; return *this; }
+  lrn& epsilon(double epsilon) { epsilon_ = epsilon; return *this; }
+  lrn& window_size(const std::vector<int64_t>& window_size) { window_size_ = window_size; return *this; }
+  lrn& axes(const std::vector<int64_t>& axes) { axes_ = axes; return *this; }
+  operator edsl::Tensor() const {
+    auto args = edsl::make_tuple(I_, edsl::make_tuple(window_size_), edsl::make_tuple(axes_), alpha_, beta_, epsilon_);
+    return details::op("lrn", args).as_tensor();
+  }
+
+ private:
+  edsl::Tensor I_;
+  std::vector<int64_t> window_size_;
+  std::vector<int64_t> axes_ = {-1};
+  double alpha_ = 1., beta_ = 1., epsilon_ = 1.e-5;
+};
+
+class mvn {
+ public:
+  explicit mvn(const edsl::Tensor& I) : I_(I), axes_(edsl::None()) {}
+  mvn& axes(const std::vector<int64_t>& axes) {
+    if (!across_channels_ || !layout_.empty()) throw std::runtime_error("When using layout and across_channels, axes may not be specified");
+    axes_ = edsl::make_tuple(axes);
+    return *this;
+  }
+  mvn& across_channels(bool flag) {
+    if (!axes_.is_none()) throw std::runtime_error("May not specify both axes and across_channels for MVN");
+    across_channels_ = flag;
+    return *this;
+  }
+  mvn& normalize_variance(bool flag) { normalize_variance_ = flag; return *this; }
+  mvn& epsilon(double value) { epsilon_ = value; return *this; }
+  mvn& layout(const std::string& value) {
+    if (!axes_.is_none()) throw std::runtime_error("May not specify both axes and layout for MVN");
+    layout_ = value;
+    return *this;
+  }
+  operator edsl::Tensor() const {
+    return details::op("mvn", edsl::make_tuple(I_, axes_, normalize_variance_, epsilon_, across_channels_, layout_)).as_tensor();
+  }
+
+ private:
+  edsl::Tensor I_;
+  edsl::Value axes_;
+  bool normalize_variance_ = true;
+  double epsilon_ = 1e-9;
+  bool across_channels_ = true;
+  std::string layout_;
+};
+
+inline edsl::Tensor reorg_yolo(const edsl::Tensor& I, int stride, bool decrease, const std::string& layout = "NCHW") {
+  return details::op("reorg_yolo", edsl::make_tuple(I, stride, decrease, layout)).as_tensor();
+}
+
+inline edsl::Tensor scale_gradient(const edsl::Tensor& I, double scale = -1.0) {
+  return details::op("scale_gradient", edsl::make_tuple(I, scale)).as_tensor();
+}
+
+class slice {
+ public:
+  explicit slice(const edsl::Tensor& I) : I_(I) {}
+  slice& add_dims(const std::vector<int>& dims) {
+    for (auto dim : dims) dims_.emplace_back(dim);
+    return *this;
+  }
+  slice& add_dim(int dim) { dims_.emplace_back(dim); return *this; }
+  slice& add_dim(int start, int stop, int step = 1) { dims_.emplace_back(edsl::make_tuple(start, stop, step)); return *this; }
+  slice& add_dim(edsl::Value start, edsl::Value stop, edsl::Value step = edsl::Value(1)) {
+    dims_.emplace_back(edsl::make_tuple(start, stop, step));
+    return *this;
+  }
+  operator edsl::Tensor() const { return details::op("slice", edsl::make_tuple(I_, dims_)).as_tensor(); }
+
+ private:
+  edsl::Tensor I_;
+  std::vector<edsl::Value> dims_;
 };
 
 inline edsl::Tensor argmax(const edsl::Tensor& I, const edsl::Value& axes = edsl::None()) {

@@ -52,7 +52,7 @@ def convolution(I, F, strides=None, dilations=None, data_dilations=None, autopad
         manual_padding = manual_padding + manual_padding  # symmetric shorthand
     while len(manual_padding) < 2 * rank:
         manual_padding.append(0)
-    if manual_padding and any(manual_padding) and autopad != EXPLICIT:
+    if manual_padding and builtins.any(manual_padding) and autopad != EXPLICIT:
         raise ValueError('Autopadding and manual padding both requested for single conv operation')
     N, CI = I.shape[0], I.shape[-1]
     xs = I.shape[1:-1]
@@ -461,3 +461,168 @@ def variance(I, axes=None, keepdims=False):
     for ax in a.axes:
         denom *= I.shape[ax]
     return so / denom
+
+
+EPS_ADD, EPS_MAX = range(2)
+
+
+def _truth(I):
+    one = E.cast(1, I.dt)
+    zero = E.cast(0, I.dt)
+    return E.select(I == 0, zero, one), zero, one
+
+
+def all(I, axes=None, keepdims=False):  # noqa: A001
+    """ops.cc:450-475: product of the 0 / 1 image of the input, as UINT8."""
+    T, zero, one = _truth(I)
+    if len(I.shape) == 0 or (isinstance(axes, (list, tuple)) and len(axes) == 0):
+        return E.cast(T, E.DType.UINT8)
+    return E.cast(_reduce(T, axes, keepdims, 'product', 'all')[0], E.DType.UINT8)
+
+
+def any(I, axes=None, keepdims=False):  # noqa: A001
+    """ops.cc:477-503: sum of the 0 / 1 image, compared with 0, as UINT8."""
+    T, zero, one = _truth(I)
+    if len(I.shape) == 0 or (isinstance(axes, (list, tuple)) and len(axes) == 0):
+        return E.cast(T, E.DType.UINT8)
+    S = _reduce(T, axes, keepdims, 'sum', 'any')[0]
+    return E.cast(E.select(S == 0, zero, one), E.DType.UINT8)
+
+
+def binary_crossentropy(targets, preds, epsilon):
+    """ops.cc:523-544."""
+    if epsilon < 0. or epsilon >= 0.5:
+        raise ValueError('The epsilon used in binary_crossentropy must be between 0 and 0.5, received %s' % epsilon)
+    P = clip(preds, float(epsilon), 1. - float(epsilon))
+    return -targets * E.log(P) - (1 - targets) * E.log(1 - P)
+
+
+def broadcast(I, result_shape, bcast_axes):
+    """ops.cc:546-582."""
+    if len(I.shape) != len(bcast_axes):
+        raise ValueError('Mismatched broadcast axes')
+    o_idxs = E.TensorIndexes(len(result_shape))
+    i_idxs = [0 if I.shape[i] == 1 else o_idxs[a] for i, a in enumerate(bcast_axes)]
+    return E.Contraction('broadcast').outShape(list(result_shape)).outAccess(o_idxs).assign(I[i_idxs]).build()
+
+
+def cumprod(I, axis):
+    """ops.cc:1469-1488."""
+    nd = len(I.shape)
+    axis = _axis(axis, nd, 'cumprod')
+    o_idxs = E.TensorIndexes(nd)
+    i_idxs = list(o_idxs)
+    k = E.TensorIndex()
+    i_idxs[axis] = o_idxs[axis] - k
+    return E.Contraction('cumprod').outShape(I.shape).outAccess(o_idxs).product(I[i_idxs]).add_constraint(k < I.shape[axis]).build()
+
+
+def l2norm(I, axes, epsilon=0.0, eps_mode=EPS_ADD):
+    """ops.cc:2505-2530."""
+    X = sum(I * I, list(axes), True)
+    if eps_mode == EPS_ADD:
+        X = X + float(epsilon)
+    elif eps_mode == EPS_MAX:
+        X = maximum(X, E.cast(float(epsilon), X.dt))
+    else:
+        raise ValueError('Unrecognized eps_mode in l2norm op')
+    return E.sqrt(X)
+
+
+def lrn(I, window_size, axes=(-1,), alpha=1.0, beta=1.0, epsilon=1e-5):
+    """ops.cc:129-160, 1920-1941: the window over axis a covers offsets -w/2 .. w - 1 - w/2 (integer division)."""
+    nd = len(I.shape)
+    ax = sorted(set(a + nd if a < 0 else a for a in axes))
+    if len(ax) != len(window_size):
+        raise ValueError('Inconsistent axis count and window width count in LRN')
+    dst = E.TensorIndexes(nd)
+    src = list(dst)
+    c = E.Contraction('lrn').outShape(I.shape).outAccess(dst)
+    cons = []
+    for a, w in zip(ax, window_size):
+        k = E.TensorIndex()
+        cons.append(k < int(w))
+        src[a] = dst[a] + k - int(w) // 2
+    c.sum((I * I)[src])
+    for k in cons:
+        c.add_constraint(k)
+    return I / E.pow(float(alpha) * c.build() + float(epsilon), float(beta))
+
+
+def mvn(I, axes=None, normalize_variance=True, epsilon=1e-9, across_channels=True, layout=''):
+    """ops.cc:2469-2503."""
+    if axes is None:
+        if not layout:
+            raise ValueError('Either axes or layout must be specified for MVN')
+        axes = [i for i, d in enumerate(layout) if d != 'N' and not (d == 'C' and not across_channels)]
+    R = I - mean(I, axes, True)
+    if normalize_variance:
+        stdev = E.sqrt(variance(I, axes, True))
+        R = R / maximum(stdev, E.cast(float(epsilon), I.dt))
+    return R
+
+
+def reorg_yolo(I, stride, decrease, layout='NCHW'):
+    """ops.cc:2730-2780, written for NCHW and permuted for any other arrangement of those four letters."""
+    if len(I.shape) != 4:
+        raise ValueError('PlaidML reorg_yolo op expects I to have 4 dimensions')
+    perm = [layout.index(ch) for ch in 'NCHW']       # position of N, C, H, W in the tensor's layout
+    N, C, H, W = (I.shape[p] for p in perm)
+    s = int(stride)
+
+    def place(vals):                                    # NCHW-ordered values -> the tensor's own order
+        out = [None] * 4
+        for v, p in zip(vals, perm):
+            out[p] = v
+        return out
+
+    b, i, j, k, x, y = E.TensorIndexes(6)
+    h = j * s + y
+    w = i * s + x
+    if decrease:
+        c_out = C // (s * s)
+        c = k + ((x + y * s) * c_out)
+        con = E.Contraction('reorg_yolo').outShape(place([N, c_out, H * s, W * s])).outAccess(place([b, k, h, w]))
+        con.assign(I[place([b, c, j, i])])
+    else:
+        c = k + ((x + y * s) * C)
+        con = E.Contraction('reorg_yolo').outShape(place([N, C * s * s, H // s, W // s])).outAccess(place([b, c, j, i]))
+        con.assign(I[place([b, k, h, w])])
+    return con.add_constraint(y < s).add_constraint(x < s).build()
+
+
+def scale_gradient(I, scale=-1.0):
+    return I  # ops.cc:2888-2904: identity on the forward pass
+
+
+def slice_of(I, slices):
+    """ops.cc:2917-3047 (entries: int or Python slice, plaidml/op/__init__.py:246-257)."""
+    nd = len(I.shape)
+    if nd == 0:
+        return I
+    if len(slices) != nd:
+        raise ValueError('%d slice axes provided to slice %d-dimensional tensor' % (len(slices), nd))
+    o_idxs, o_dims, i_idxs = [], [], []
+    for d, sl in enumerate(slices):
+        dim = I.shape[d]
+        if isinstance(sl, int):
+            i_idxs.append(sl + dim if sl < 0 else sl)
+            continue
+        step = 1 if sl.step is None else int(sl.step)
+        if step == 0:
+            raise ValueError('Cannot slice with step size 0')
+        if sl.start is None:
+            start = 0 if step > 0 else dim - 1
+        else:
+            start = dim + sl.start if sl.start < 0 else sl.start
+        if sl.stop is None:
+            stop = dim if step > 0 else -1
+        else:
+            stop = dim + sl.stop if sl.stop < 0 else sl.stop
+        to_ceil = step - 1 if step > 0 else step + 1
+        num = stop - start + to_ceil
+        o_dims.append(int(num / step) if num % step else num // step)  # C division: toward zero
+        o = E.TensorIndex()
+        o_idxs.append(o)
+        i_idxs.append(start + step * o)
+    return E.Contraction('slice').outShape(o_dims).outAccess(o_idxs).assign(I[i_idxs]).build()

@@ -809,6 +809,8 @@ def contract(agg, combo, out_dt, out_shape, sink, srcs, accs, cons=(), init=None
                 else:
                     a = convert(a, adt, cdt)
             bufs.append(np.ascontiguousarray(a, dtype=npdt))
+    # ascontiguousarray promotes a 0-d array to 1-d: a scalar operand keeps rank 0, matching its empty access
+    bufs = [b.reshape(np.shape(s[0])) for b, s in zip(bufs, srcs)]
     ranks = [len(out_shape)] + [b.ndim for b in bufs]
     sizes = list(out_shape)
     for b in bufs:

@@ -28,6 +28,7 @@ using namespace plaidml::edsl;  // NOLINT
 using plaidml::op::AutoGroupMode;
 using plaidml::op::AutoPadMode;
 using plaidml::op::ConvDerivMode;
+using plaidml::op::EpsMode;
 using plaidml::op::GroupLayout;
 using plaidml::op::PoolMode;
 using plaidml::op::TensorLayout;
@@ -639,6 +640,270 @@ Value op_hard_sigmoid(const Value& value) {
   return Value{select(I < lo_cusp, lo, select(I > hi_cusp, hi, slope * I + 0.5))};
 }
 
+Value op_variance(const Value& value);
+
+// all / any (plaidml/op/lib/ops.cc:450-503): the input as 0 / 1 in its own type, multiplied (all) or summed and
+// tested (any) over the axes, as UINT8.
+Tensor truth_of(const Tensor& I, Tensor* zero, Tensor* one) {
+  *one = cast(Tensor(int64_t{1}), I.dtype());
+  *zero = cast(Tensor(int64_t{0}), I.dtype());
+  return select(I == 0, *zero, *one);
+}
+
+Value op_all(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("all expects 3 arguments");
+  auto I = args[0].as_tensor();
+  Tensor zero, one;
+  Tensor T = truth_of(I, &zero, &one);
+  if (I.rank() == 0 || (args[1].is_tuple() && args[1].as_tuple().empty())) return Value{cast(T, DType::UINT8)};
+  AggregationAxes ag(I.rank(), args[1], args[2].as_bool());
+  I.bind_dims(ag.src_dims);
+  Tensor O = Contraction(ag.dst_dims, ag.dst_idxs, "all").product(T(ag.src_idxs));
+  return Value{cast(O, DType::UINT8)};
+}
+
+Value op_any(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("any expects 3 arguments");
+  auto I = args[0].as_tensor();
+  Tensor zero, one;
+  Tensor T = truth_of(I, &zero, &one);
+  if (I.rank() == 0 || (args[1].is_tuple() && args[1].as_tuple().empty())) return Value{cast(T, DType::UINT8)};
+  AggregationAxes ag(I.rank(), args[1], args[2].as_bool());
+  I.bind_dims(ag.src_dims);
+  Tensor S = Contraction(ag.dst_dims, ag.dst_idxs, "any").sum(T(ag.src_idxs));
+  return Value{cast(select(S == 0, zero, one), DType::UINT8)};
+}
+
+// plaidml/op/lib/ops.cc:523-544: predictions clipped to [eps, 1 - eps], then -T log P - (1 - T) log(1 - P)
+Value op_binary_crossentropy(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("binary_crossentropy expects 3 arguments");
+  auto T = args[0].as_tensor();
+  const double epsilon = args[2].as_float();
+  if (epsilon < 0. || epsilon >= 0.5)
+    throw std::runtime_error("The epsilon used in binary_crossentropy must be between 0 and 0.5, received " + std::to_string(epsilon));
+  auto P = op_clip(make_tuple(args[1], Value{epsilon}, Value{1. - epsilon})).as_tensor();
+  return Value{-T * log(P) - (1 - T) * log(1 - P)};
+}
+
+// plaidml/op/lib/ops.cc:546-582: input dimension i becomes output dimension axes[i]; an input extent of 1 repeats
+Value op_broadcast(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3)
+    throw std::runtime_error("PlaidML broadcast op expects 3 arguments (received " + std::to_string(args.size()) + ")");
+  auto I = args[0].as_tensor();
+  auto axes = args[2].as_int_tuple_or_empty();
+  if (I.rank() != axes.size())
+    throw std::runtime_error("Mismatched broadcast axes (received " + std::to_string(axes.size()) +
+                             " broadcast axes for input tensor of rank " + std::to_string(I.rank()) + ")");
+  const auto in_sizes = I.compute_shape().sizes();
+  auto target = args[1].as_int_tuple_or_empty();
+  std::vector<TensorDim> O_dims(target.begin(), target.end());
+  std::vector<TensorDim> I_dims(I.rank());
+  I.bind_dims(I_dims);
+  std::vector<TensorIndex> O_idxs(target.size()), I_idxs;
+  for (size_t i = 0; i < axes.size(); ++i) {
+    if (in_sizes[i] == 1) {
+      I_idxs.emplace_back(0);
+    } else {
+      if (axes[i] < 0 || axes[i] >= static_cast<int64_t>(target.size())) throw std::out_of_range("broadcast axis out of range");
+      I_idxs.push_back(O_idxs[axes[i]]);
+    }
+  }
+  Tensor O = Contraction(O_dims, O_idxs, "broadcast").assign(I(I_idxs));
+  return Value{O};
+}
+
+// plaidml/op/lib/ops.cc:1469-1488
+Value op_cumprod(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("cumprod expects 2 arguments");
+  auto I = args[0].as_tensor();
+  const size_t ndims = I.rank();
+  const size_t axis = normalize_axis(args[1].as_int(), ndims, "cumprod");
+  std::vector<TensorDim> dims(ndims);
+  I.bind_dims(dims);
+  std::vector<TensorIndex> O_idxs(ndims);
+  std::vector<TensorIndex> I_idxs = O_idxs;
+  TensorIndex back;
+  I_idxs[axis] = O_idxs[axis] - back;
+  Tensor O = Contraction(dims, O_idxs, "cumprod").product(I(I_idxs)).add_constraint(back < dims[axis]);
+  return Value{O};
+}
+
+// plaidml/op/lib/ops.cc:2505-2530: sqrt(sum of squares over the axes (kept), + eps or max(., eps))
+Value op_l2norm(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 4) throw std::runtime_error("norm expects 4 arguments");
+  auto I = args[0].as_tensor();
+  const double epsilon = args[2].as_float();
+  const auto mode = validate<EpsMode>(args[3].as_int());
+  Tensor X = reduce(make_tuple(Value{I * I}, args[1], Value{true}), "sum", PLAIDML_AGG_OP_SUM).as_tensor();
+  switch (mode) {
+    case EpsMode::ADD: X = X + epsilon; break;
+    case EpsMode::MAX: X = op_maximum(make_tuple(Value{X}, Value{cast(Tensor(epsilon), X.dtype())})).as_tensor(); break;
+    default: throw std::runtime_error("Unrecognized eps_mode in l2norm op");
+  }
+  return Value{sqrt(X)};
+}
+
+// plaidml/op/lib/ops.cc:129-160, 1920-1941: I / (alpha * sum of squares over a centred window + eps) ^ beta
+Value op_lrn(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 6) throw std::runtime_error("lrn expects 6 arguments");
+  auto I = args[0].as_tensor();
+  const auto widths = args[1].as_int_tuple_or_empty();
+  const auto in_axes = args[2].as_int_tuple_or_empty();
+  const double alpha = args[3].as_float(), beta = args[4].as_float(), epsilon = args[5].as_float();
+  const size_t ndims = I.rank();
+  std::set<int64_t> axes;
+  for (int64_t a : in_axes) {
+    if (a < 0) a += ndims;
+    if (a < 0 || a >= static_cast<int64_t>(ndims)) throw std::out_of_range("axis out of range: " + std::to_string(a));
+    axes.insert(a);
+  }
+  if (axes.size() != widths.size())
+    throw std::runtime_error("Inconsistent axis count and window width count in LRN (" + std::to_string(axes.size()) + " vs " +
+                             std::to_string(widths.size()) + ")");
+  std::vector<TensorDim> dims(ndims);
+  I.bind_dims(dims);
+  std::vector<TensorIndex> dst(ndims);
+  std::vector<TensorIndex> src = dst;
+  std::vector<TensorIndex> win(widths.size());
+  std::vector<Constraint> cons;
+  size_t k = 0;
+  for (int64_t a : axes) {
+    cons.push_back(win[k] < widths[k]);
+    src[a] = dst[a] + win[k] - widths[k] / 2;
+    ++k;
+  }
+  Tensor sq = I * I;
+  Tensor local = Contraction(dims, dst, "lrn").sum(sq(src)).add_constraints(cons);
+  return Value{I / pow(alpha * local + epsilon, Tensor(beta))};
+}
+
+// plaidml/op/lib/ops.cc:2469-2503
+Value op_mvn(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 6) throw std::runtime_error("mvn expects 6 arguments");
+  auto I = args[0].as_tensor();
+  Value axes = args[1];
+  const bool normalize_variance = args[2].as_bool();
+  const double epsilon = args[3].as_float();
+  const bool across_channels = args[4].as_bool();
+  const std::string layout = args[5].as_str();
+  if (axes.is_none()) {
+    if (layout.empty()) throw std::runtime_error("Either axes or layout must be specified for MVN");
+    std::vector<Value> raw;
+    for (size_t i = 0; i < layout.size(); ++i) {
+      if (layout[i] == 'N') continue;
+      if (layout[i] == 'C' && !across_channels) continue;
+      raw.emplace_back(static_cast<int64_t>(i));
+    }
+    axes = Value(raw);
+  }
+  Tensor R = I - reduce(make_tuple(args[0], axes, Value{true}), "mean", PLAIDML_AGG_OP_SUM).as_tensor();
+  if (normalize_variance) {
+    Tensor stdev = sqrt(op_variance(make_tuple(args[0], axes, Value{true})).as_tensor());
+    R = R / op_maximum(make_tuple(Value{stdev}, Value{cast(Tensor(epsilon), I.dtype())})).as_tensor();
+  }
+  return Value{R};
+}
+
+// plaidml/op/lib/ops.cc:2730-2780: blocks of stride x stride pixels move between the spatial and the channel
+// dimensions; the contraction is written in NCHW and seen through a lens for other layouts
+Value op_reorg_yolo(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 4)
+    throw std::runtime_error("PlaidML reorg_yolo op expects 4 arguments (received " + std::to_string(args.size()) + ")");
+  auto I = args[0].as_tensor();
+  const int64_t stride = args[1].as_int();
+  const bool decrease = args[2].as_bool();
+  const std::string layout = args[3].as_str();
+  if (I.rank() != 4)
+    throw std::runtime_error("PlaidML reorg_yolo op expects I to have 4 dimensions (received " + std::to_string(I.rank()) + ")");
+  TensorLens lens(layout, "NCHW");
+  I = I.use(lens);
+  TensorDim N, C, H, W;
+  I.bind_dims(N, C, H, W);
+  TensorIndex b, i, j, k, x, y;
+  auto h = j * stride + y;
+  auto w = i * stride + x;
+  Tensor O;
+  if (decrease) {
+    auto C_out = C / (stride * stride);
+    auto c = k + ((x + y * stride) * C_out);
+    O = Contraction(lens, "reorg_yolo").outShape(N, C_out, H * stride, W * stride).outAccess(b, k, h, w).assign(I(b, c, j, i))
+            .add_constraint(y < stride).add_constraint(x < stride);
+  } else {
+    auto C_out = C * (stride * stride);
+    auto c = k + ((x + y * stride) * C);
+    O = Contraction(lens, "reorg_yolo").outShape(N, C_out, H / stride, W / stride).outAccess(b, c, j, i).assign(I(b, k, h, w))
+            .add_constraint(y < stride).add_constraint(x < stride);
+  }
+  return Value{O};
+}
+
+// plaidml/op/lib/ops.cc:2888-2904: the forward pass is the identity
+Value op_scale_gradient(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("scale_gradient expects 2 arguments");
+  return Value{args[0].as_tensor()};
+}
+
+// plaidml/op/lib/ops.cc:2917-3047: per axis an integer (the axis disappears) or (start, stop, step) with None
+// defaults and negative values counted from the end; no clamping, as in the reference
+Value op_slice(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 2) throw std::runtime_error("slice expects 2 arguments");
+  auto I = args[0].as_tensor();
+  auto slices = args[1].as_tuple();
+  const size_t ndims = I.rank();
+  if (ndims == 0) return Value{I};
+  if (slices.size() != ndims)
+    throw std::runtime_error(std::to_string(slices.size()) + " slice axes provided to slice " + std::to_string(ndims) + "-dimensional tensor");
+  std::vector<TensorDim> I_dims(ndims);
+  I.bind_dims(I_dims);
+  std::vector<TensorIndex> O_idxs, I_idxs;
+  std::vector<TensorDim> O_dims;
+  for (size_t i = 0; i < ndims; ++i) {
+    if (slices[i].is_int()) {
+      const int64_t at = slices[i].as_int();
+      TensorIndex idx(at);
+      if (at < 0) idx = idx + I_dims[i];
+      I_idxs.push_back(idx);
+      continue;
+    }
+    if (!slices[i].is_tuple()) throw std::runtime_error("Attempted to define slice with invalid type");
+    auto sl = slices[i].as_tuple();
+    if (sl.size() != 3) throw std::runtime_error("Attempted to slice with " + std::to_string(sl.size()) + " entries, 3 required");
+    const int64_t step = sl[2].is_none() ? 1 : sl[2].as_int();
+    if (step == 0) throw std::runtime_error("Cannot slice with step size 0");
+    TensorDim start, stop;
+    if (sl[0].is_none()) {
+      start = step > 0 ? TensorDim(0) : I_dims[i] - 1;
+    } else {
+      const int64_t v = sl[0].as_int();
+      start = v < 0 ? I_dims[i] + v : TensorDim(v);
+    }
+    if (sl[1].is_none()) {
+      stop = step > 0 ? I_dims[i] : TensorDim(-1);
+    } else {
+      const int64_t v = sl[1].as_int();
+      stop = v < 0 ? I_dims[i] + v : TensorDim(v);
+    }
+    const int64_t to_ceil = step > 0 ? step - 1 : step + 1;
+    O_dims.push_back((stop - start + to_ceil) / step);
+    TensorIndex o;
+    O_idxs.push_back(o);
+    I_idxs.push_back(start + step * o);
+  }
+  Tensor O = Contraction(O_dims, O_idxs, "slice").assign(I(I_idxs));
+  return Value{O};
+}
+
 Value op_prod(const Value& value) {
   auto args = value.as_tuple();
   if (args.size() != 3) throw std::runtime_error("prod expects 3 arguments");
@@ -875,27 +1140,38 @@ using OpFn = std::function<Value(const Value&)>;
 const std::map<std::string, OpFn>& registry() {
   static const std::map<std::string, OpFn> r = {
       {"abs", op_abs},
+      {"all", op_all},
+      {"any", op_any},
       {"argmax", op_argmax},
+      {"binary_crossentropy", op_binary_crossentropy},
+      {"broadcast", op_broadcast},
       {"clip", op_clip},
       {"concatenate", op_concatenate},
       {"convolution", op_convolution},
+      {"cumprod", op_cumprod},
       {"cumsum", op_cumsum},
       {"dot", op_dot},
       {"elu", op_elu},
       {"explicit_padding", op_explicit_padding},
       {"flip", op_flip},
       {"hard_sigmoid", op_hard_sigmoid},
+      {"l2norm", op_l2norm},
+      {"lrn", op_lrn},
       {"max", [](const Value& v) { return reduce(v, "max", PLAIDML_AGG_OP_MAX); }},
       {"maximum", op_maximum},
       {"mean", [](const Value& v) { return reduce(v, "mean", PLAIDML_AGG_OP_SUM); }},
       {"min", [](const Value& v) { return reduce(v, "min", PLAIDML_AGG_OP_MIN); }},
       {"minimum", op_minimum},
+      {"mvn", op_mvn},
       {"pool", op_pool},
       {"prod", op_prod},
       {"relu", op_relu},
+      {"reorg_yolo", op_reorg_yolo},
       {"repeat", op_repeat},
       {"reshape", op_reshape},
+      {"scale_gradient", op_scale_gradient},
       {"sigmoid", op_sigmoid},
+      {"slice", op_slice},
       {"softmax", op_softmax},
       {"spatial_padding", op_spatial_padding},
       {"square", op_square},

@@ -159,3 +159,59 @@ def unsqueeze(I, axes):
 
 def variance(I, axes=None, keepdims=False):
     return E.op_make('variance', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+EPS_ADD, EPS_MAX = range(2)
+
+
+def all(I, axes=None, keepdims=False):  # noqa: A001
+    return E.op_make('all', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def any(I, axes=None, keepdims=False):  # noqa: A001
+    return E.op_make('any', [I, _axes(axes), bool(keepdims)]).as_tensor()
+
+
+def binary_crossentropy(targets, preds, epsilon):
+    return E.op_make('binary_crossentropy', [targets, preds, float(epsilon)]).as_tensor()
+
+
+def broadcast(I, result_shape, bcast_axes):
+    return E.op_make('broadcast', [I, _ints(result_shape), _ints(bcast_axes)]).as_tensor()
+
+
+def cumprod(I, axis):
+    return E.op_make('cumprod', [I, int(axis)]).as_tensor()
+
+
+def l2norm(I, axes, epsilon=0.0, eps_mode=EPS_ADD):
+    return E.op_make('l2norm', [I, _ints(axes), float(epsilon), int(eps_mode)]).as_tensor()
+
+
+def lrn(I, window_size, axes=(-1,), alpha=1.0, beta=1.0, epsilon=1e-5):
+    return E.op_make('lrn', [I, _ints(window_size), _ints(axes), float(alpha), float(beta), float(epsilon)]).as_tensor()
+
+
+def mvn(I, axes=None, normalize_variance=True, epsilon=1e-9, across_channels=True, layout=''):
+    return E.op_make('mvn', [I, _axes(axes), bool(normalize_variance), float(epsilon), bool(across_channels), layout]).as_tensor()
+
+
+def reorg_yolo(I, stride, decrease, layout='NCHW'):
+    return E.op_make('reorg_yolo', [I, int(stride), bool(decrease), layout]).as_tensor()
+
+
+def scale_gradient(I, scale=-1.0):
+    return E.op_make('scale_gradient', [I, float(scale)]).as_tensor()
+
+
+def slice_of(I, slices):
+    """Each entry an int or a Python slice, as plaidml/op/__init__.py:246-257."""
+    out = []
+    for s in slices:
+        if isinstance(s, int):
+            out.append(s)
+        elif isinstance(s, slice):
+            out.append([s.start, s.stop, s.step])
+        else:
+            raise ValueError('Unexpected type {} used to slice tensor'.format(type(s)))
+    return E.op_make('slice', [I, out]).as_tensor()

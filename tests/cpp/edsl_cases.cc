@@ -286,6 +286,43 @@ void caseIntrinsics() {
   }
 }
 
+// Builder classes of the op header: slice (int and (start, stop, step) entries), broadcast with the reference's
+// own case (plaidml/op/op_test.cc:115-127), l2norm, lrn, mvn, reorg_yolo shapes.
+void caseOpBuilders() {
+  auto A = Placeholder(DType::FLOAT32, {3, 4});
+  std::vector<float> a = {0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11};
+  {
+    Tensor S = op::slice(A).add_dim(1, 3).add_dim(edsl::Value(edsl::None()), edsl::Value(edsl::None()), edsl::Value(-2));
+    Tensor R = op::slice(A).add_dim(-1).add_dim(0, 4, 3);
+    auto out = run(buildProgram("slice", {A}, {S, R}), {makeBuffer<float>(DType::FLOAT32, {3, 4}, a)});
+    expectEq<float>("slice_steps", readBuffer<float>(out[0]), {7, 5, 11, 9});
+    expectEq<float>("slice_int", readBuffer<float>(out[1]), {8, 11});
+  }
+  {
+    auto B = Placeholder(DType::FLOAT32, {3, 1});
+    auto out = run(buildProgram("broadcast", {B}, {op::broadcast(B, {3, 4}, {0, 1})}), {makeBuffer<float>(DType::FLOAT32, {3, 1}, {0, 1, 2})});
+    expectEq<float>("broadcast_numpy2", readBuffer<float>(out[0]), {0, 0, 0, 0, 1, 1, 1, 1, 2, 2, 2, 2});
+  }
+  {
+    Tensor N = op::l2norm(A, {1}).epsilon(1.0f).eps_mode(op::EpsMode::MAX);
+    Tensor L = op::lrn(A, {3}).alpha(0.0).beta(2.0).epsilon(2.0);  // x / (0 + 2)^2
+    Tensor M = op::mvn(A).axes({1}).normalize_variance(false);
+    auto out = run(buildProgram("norms", {A}, {N, L, M}), {makeBuffer<float>(DType::FLOAT32, {3, 4}, a)});
+    expectClose("l2norm", readBuffer<float>(out[0]), {std::sqrt(14.f), std::sqrt(126.f), std::sqrt(366.f)}, 1e-5f, 0.f);
+    std::vector<float> quarter;
+    for (float v : a) quarter.push_back(v / 4);
+    expectClose("lrn", readBuffer<float>(out[1]), quarter, 1e-6f, 0.f);
+    expectClose("mvn", readBuffer<float>(out[2]), {-1.5, -.5, .5, 1.5, -1.5, -.5, .5, 1.5, -1.5, -.5, .5, 1.5}, 1e-6f, 1e-6f);
+  }
+  {
+    auto I = Placeholder(DType::INT64, {1, 4, 6, 6});
+    Tensor O = op::reorg_yolo(I, 2, /*decrease=*/false);
+    auto dims = O.compute_shape().sizes();
+    if (dims != std::vector<int64_t>{1, 16, 3, 3}) fail("reorg_yolo_shape", "unexpected result shape");
+    std::printf("ok reorg_yolo_shape\n");
+  }
+}
+
 void caseErrors() {
   auto A = Placeholder(DType::FLOAT32, {4, 4});
   auto program = buildProgram("ident", {A}, {A + 1.0});
@@ -322,6 +359,7 @@ int main() {
     caseConvRelu();
     caseOpLibrary();
     caseIntrinsics();
+    caseOpBuilders();
     caseErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAILED with exception: %s\n", e.what());

@@ -4,7 +4,8 @@ and product EDSL): name -> builder(E, op) returning (program, inputs, expected n
 Expected values are numpy closed forms (np.concatenate, np.pad, np.cumsum, ...) and, where the reference holds
 an exact case, that case (plaidml/op/op_test.cc: CumSumExclusive :297-304, ExplicitPadding :318-333,
 ExplicitPaddingNegInf :335-351, ExplicitPaddingInf :353-370, ExplicitPaddingNoOp :372-383,
-ExplicitPaddingEdge :385-418).
+ExplicitPaddingEdge :385-418, Broadcast* :52-158, ReorgYoloDecrease / ReorgYoloIncrease :552-581 with their loop-nest
+reference :524-550).  A case may return lists of outputs / expected arrays.
 """
 import numpy as np
 
@@ -133,7 +134,160 @@ def arithmetic(E, op):
     return E.Program('arithmetic', [X], [O]), [x], ref, False
 
 
+def _broadcast_ref(E, op, in_shape, data, rshape, axes, expected):
+    X = _f32(E, in_shape)
+    x = np.asarray(data, np.float32).reshape(in_shape)
+    return E.Program('broadcast', [X], [op.broadcast(X, rshape, axes)]), [x], np.asarray(expected, np.float32).reshape(rshape), True
+
+
+def broadcast_noop_reference(E, op):
+    return _broadcast_ref(E, op, (3,), [0, 1, 2], [3], [0], [0, 1, 2])
+
+
+def broadcast_scalar_reference(E, op):
+    return _broadcast_ref(E, op, (), [3], [3, 4], [], [3] * 12)
+
+
+def broadcast_noop_large_reference(E, op):
+    return _broadcast_ref(E, op, (3, 4), [0, 1, 2, 3] * 3, [3, 4], [0, 1], [0, 1, 2, 3] * 3)
+
+
+def broadcast_numpy_reference(E, op):
+    return _broadcast_ref(E, op, (1, 3, 3), [0, 1, 2] * 3, [1, 4, 3, 3], [0, 2, 3], [0, 1, 2] * 12)
+
+
+def broadcast_numpy2_reference(E, op):
+    return _broadcast_ref(E, op, (3, 1), [0, 1, 2], [3, 4], [0, 1], [0] * 4 + [1] * 4 + [2] * 4)
+
+
+def broadcast_numpy3_reference(E, op):
+    return _broadcast_ref(E, op, (3,), [0, 1, 2], [4, 3], [1], [0, 1, 2] * 4)
+
+
+def broadcast_non_numpy_reference(E, op):
+    return _broadcast_ref(E, op, (3,), [0, 1, 2], [3, 4], [0], [0] * 4 + [1] * 4 + [2] * 4)
+
+
+def _reorg_yolo_ref(x, stride, decrease):
+    """What the reference's test expects (its loop nest, plaidml/op/op_test.cc:524-550, in closed form), NCHW:
+    channel k = off * C_small + c of the wide tensor holds pixel (oy, ox) = (off / s, off % s) of every s x s block
+    of channel c of the spatially large tensor.  decrease: wide -> large; otherwise large -> wide."""
+    s_ = stride
+    if decrease:
+        n, c, h, w = x.shape
+        cs = c // (s_ * s_)
+        return x.reshape(n, s_, s_, cs, h, w).transpose(0, 3, 4, 1, 5, 2).reshape(n, cs, h * s_, w * s_)
+    n, c, h, w = x.shape
+    return x.reshape(n, c, h // s_, s_, w // s_, s_).transpose(0, 3, 5, 1, 2, 4).reshape(n, c * s_ * s_, h // s_, w // s_)
+
+
+def _reorg(E, op, decrease):
+    N, C, H, W, S = 1, 4, 6, 6, 2
+    X = E.Placeholder(E.DType.INT64, [N, C, H, W])
+    x = np.arange(N * C * H * W, dtype=np.int64).reshape(N, C, H, W)
+    return E.Program('reorg_yolo', [X], [op.reorg_yolo(X, S, decrease)]), [x], _reorg_yolo_ref(x, S, decrease), True
+
+
+def reorg_yolo_decrease_reference(E, op):
+    return _reorg(E, op, True)
+
+
+def reorg_yolo_increase_reference(E, op):
+    return _reorg(E, op, False)
+
+
+def reorg_yolo_nhwc(E, op):
+    """The NHWC lens: the same rearrangement as NCHW on the transposed tensor."""
+    N, C, H, W, S = 2, 8, 4, 6, 2
+    X = E.Placeholder(E.DType.FLOAT32, [N, H, W, C])
+    x = _rng().standard_normal((N, H, W, C)).astype(np.float32)
+    ref = _reorg_yolo_ref(x.transpose(0, 3, 1, 2), S, False).transpose(0, 2, 3, 1)
+    return E.Program('reorg_yolo', [X], [op.reorg_yolo(X, S, False, 'NHWC')]), [x], ref, True
+
+
+def all_any(E, op):
+    X = E.Placeholder(E.DType.INT32, [3, 4, 5])
+    x = _rng().integers(-1, 2, (3, 4, 5)).astype(np.int32)
+    x[1] = np.abs(x[1]) + 1
+    outs = [op.all(X, [1]), op.any(X, [0, 2], True), op.all(X), op.any(X, [])]
+    ref = [x.all(1).astype(np.uint8), x.any((0, 2), keepdims=True).astype(np.uint8), np.uint8(x.all()), (x != 0).astype(np.uint8)]
+    return E.Program('all_any', [X], outs), [x], ref, True
+
+
+def binary_crossentropy(E, op):
+    T, P = _f32(E, (4, 6)), _f32(E, (4, 6))
+    r = _rng()
+    t = r.integers(0, 2, (4, 6)).astype(np.float32)
+    p = r.uniform(-0.1, 1.1, (4, 6)).astype(np.float32)
+    pc = np.clip(p.astype(np.float64), 0.01, 0.99)
+    ref = -t * np.log(pc) - (1 - t) * np.log(1 - pc)
+    return E.Program('bce', [T, P], [op.binary_crossentropy(T, P, 0.01)]), [t, p], ref, False
+
+
+def cumprod(E, op):
+    p, ins, x = _one(E, 'cumprod', (3, 6, 4), lambda X: op.cumprod(X, 1))
+    return p, ins, np.cumprod(x.astype(np.float64), 1), False
+
+
+def l2norm(E, op):
+    X = _f32(E, (3, 5, 4))
+    x = _rng().standard_normal((3, 5, 4)).astype(np.float32)
+    x[1] = 0
+    x64 = x.astype(np.float64)
+    ss = (x64 * x64).sum((1, 2), keepdims=True)
+    outs = [op.l2norm(X, [1, 2], 0.25, op.EPS_ADD), op.l2norm(X, [1, 2], 0.25, op.EPS_MAX)]
+    return E.Program('l2norm', [X], outs), [x], [np.sqrt(ss + 0.25), np.sqrt(np.maximum(ss, 0.25))], False
+
+
+def lrn(E, op):
+    """Across-channel normalisation, window 5 (AlexNet's), against the explicit window sum; an even window
+    too, which reaches one element further back than forward (offsets -w/2 .. w - 1 - w/2)."""
+    X = _f32(E, (2, 3, 4, 9))
+    x = _rng().standard_normal((2, 3, 4, 9)).astype(np.float32)
+    x64 = x.astype(np.float64)
+
+    def ref(w, alpha, beta, eps):
+        sq = np.zeros_like(x64)
+        for c in range(9):
+            lo, hi = c - w // 2, c + w - 1 - w // 2
+            sq[..., c] = (x64[..., max(lo, 0):min(hi, 8) + 1] ** 2).sum(-1)
+        return x64 / (alpha * sq + eps) ** beta
+
+    outs = [op.lrn(X, [5], (-1,), 1e-2, 0.75, 2.0), op.lrn(X, [4], (3,), 0.5, 0.5, 1.0)]
+    return E.Program('lrn', [X], outs), [x], [ref(5, 1e-2, 0.75, 2.0), ref(4, 0.5, 0.5, 1.0)], False
+
+
+def mvn(E, op):
+    X = _f32(E, (2, 5, 4, 3))
+    x = _rng().standard_normal((2, 5, 4, 3)).astype(np.float32) * 3 + 1
+    x64 = x.astype(np.float64)
+    m = x64.mean((1, 2), keepdims=True)
+    sd = x64.std((1, 2), keepdims=True)
+    m2 = x64.mean((1, 2, 3), keepdims=True)
+    outs = [op.mvn(X, layout='NHWC', across_channels=False), op.mvn(X, axes=[1, 2, 3], normalize_variance=False)]
+    return E.Program('mvn', [X], outs), [x], [(x64 - m) / np.maximum(sd, 1e-9), x64 - m2], False
+
+
+def slice_of(E, op):
+    X = _f32(E, (6, 7, 5))
+    x = _rng().standard_normal((6, 7, 5)).astype(np.float32)
+    outs = [op.slice_of(X, [slice(1, 5, 2), 3, slice(None, None, None)]),
+            op.slice_of(X, [slice(None, None, -1), slice(-3, None, None), -1]),
+            op.slice_of(X, [slice(4, 0, -2), slice(None, -2, 3), slice(1, 2, None)])]
+    ref = [x[1:5:2, 3, :], x[::-1, -3:, -1], x[4:0:-2, :-2:3, 1:2]]
+    return E.Program('slice', [X], outs), [x], ref, True
+
+
+def scale_gradient(E, op):
+    p, ins, x = _one(E, 'scale_gradient', (3, 4), lambda X: op.scale_gradient(X, 0.5) + 0.0)
+    return p, ins, x, True
+
+
 CASES = {f.__name__: f for f in (
+    broadcast_noop_reference, broadcast_scalar_reference, broadcast_noop_large_reference, broadcast_numpy_reference,
+    broadcast_numpy2_reference, broadcast_numpy3_reference, broadcast_non_numpy_reference, reorg_yolo_decrease_reference,
+    reorg_yolo_increase_reference, reorg_yolo_nhwc, all_any, binary_crossentropy, cumprod, l2norm, lrn, mvn, slice_of,
+    scale_gradient,
     concatenate, cumsum, cumsum_exclusive_reference, explicit_padding_reference, explicit_padding_neg_inf_reference,
     explicit_padding_inf_reference, explicit_padding_noop_reference, explicit_padding_edge_reference, spatial_padding, flip,
     repeat, tile, transpose, transpose_default, reshape, squeeze_unsqueeze, prod, variance, arithmetic)}

@@ -8,7 +8,15 @@ from oracle import tile_oracle as E
 from oracle import tile_oplib as op
 
 
-def check(out, ref, exact):
+def check(outs, refs, exact):
+    if not isinstance(refs, list):
+        refs = [refs]
+    assert len(outs) == len(refs)
+    for out, ref in zip(outs, refs):
+        check_one(out, ref, exact)
+
+
+def check_one(out, ref, exact):
     assert np.asarray(out).shape == np.asarray(ref).shape
     if exact:
         np.testing.assert_array_equal(out, ref)
@@ -19,8 +27,7 @@ def check(out, ref, exact):
 @pytest.mark.parametrize('name', sorted(oplib_cases.CASES))
 def test_oracle(name):
     prog, ins, ref, exact = oplib_cases.CASES[name](E, op)
-    out, = E.run(prog, ins)
-    check(out, ref, exact)
+    check(E.run(prog, ins), ref, exact)
 
 
 @pytest.mark.gpu
@@ -30,5 +37,4 @@ def test_hip(name, target):
     from plaidml_amd import edsl as P
     from plaidml_amd import op as Pop
     prog, ins, ref, exact = oplib_cases.CASES[name](P, Pop)
-    out, = P.run(prog, ins, target=target)
-    check(out, ref, exact)
+    check(P.run(prog, ins, target=target), ref, exact)
