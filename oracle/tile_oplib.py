@@ -40,49 +40,231 @@ def compute_padding_and_output_size(input_size, filter_size, stride, autopad, pa
     raise ValueError('Unexpected autopadding mode: %s' % autopad)
 
 
-def convolution(I, F, strides=None, dilations=None, data_dilations=None, autopad=SAME_UPPER,
-                manual_padding=None, depthwise=False, name='conv'):
-    """NXC input, XCK filter.  depthwise=True is GroupLayout IN_C + AutoGroupMode DEPTHWISE."""
-    rank = len(I.shape) - 2
+def compute_padding_and_input_size(output_size, filter_size, stride, autopad, pad_lo=0, pad_hi=0, dilation=1,
+                                   data_dilation=1):
+    """plaidml/op/lib/ops.cc:383-418: the smallest input extent giving `output_size`.  The SAME modes return the
+    output extent itself as the input extent (so written there)."""
+    if data_dilation != 1:
+        raise ValueError('Cannot infer input data size for transposed convolution with data dilation')
+    f_eff = dilation * (filter_size - 1) + 1
+    if autopad == EXPLICIT:
+        return pad_lo, output_size * stride - pad_lo - pad_hi + f_eff - stride
+    if autopad == VALID:
+        return 0, output_size * stride + f_eff - stride
+    if autopad in (SAME_LOWER, SAME_UPPER):
+        input_size = output_size * stride - stride + 1
+        lower = 1 if autopad == SAME_LOWER else 0
+        return (builtins.max(0, (output_size - 1) * stride + f_eff - input_size) + lower) // 2, output_size
+    raise ValueError('Unexpected autopadding mode: %s' % autopad)
+
+
+LAYOUT_NXC, LAYOUT_NCX, LAYOUT_KCX, LAYOUT_XCK, LAYOUT_GKCX, LAYOUT_XGCK = range(6)
+GROUP_NONE, GROUP_SEPARATE, GROUP_IN_C, GROUP_IN_K = range(4)
+AUTOGROUP_UNGROUPED, AUTOGROUP_EXPLICIT, AUTOGROUP_AUTO, AUTOGROUP_DEPTHWISE = range(4)
+DERIV_NONE, DERIV_DATA, DERIV_FILTER = range(3)
+
+
+def _data_order(layout, n, c, spatial):
+    return [n] + ([c] if layout == LAYOUT_NCX else []) + list(spatial) + ([c] if layout == LAYOUT_NXC else [])
+
+
+def _filter_order(layout, g, k, c, spatial):
+    if layout in (LAYOUT_GKCX, LAYOUT_KCX):
+        return ([g] if layout == LAYOUT_GKCX else []) + [k, c] + list(spatial)
+    return list(spatial) + ([g] if layout == LAYOUT_XGCK else []) + [c, k]
+
+
+def convolution(I_or_O, F_or_O, strides=None, dilations=None, data_dilations=None, autopad=SAME_UPPER,
+                manual_padding=None, depthwise=False, name='conv', groups=1, input_layout=LAYOUT_NXC,
+                filter_layout=LAYOUT_XCK, group_layout=GROUP_NONE, autogroup_mode=AUTOGROUP_UNGROUPED,
+                deriv_mode=DERIV_NONE, result_shape=None, infer_result_shape=False, filter_shape=None):
+    """plaidml/op/lib/ops.cc:879-1467 with the validation of :671-877, on concrete shapes.  One contraction over
+    I (data), F (filters), O (forward result); deriv_mode names the one computed: NONE -> O, DATA -> I (first
+    argument is O), FILTER -> F (second argument is O).  depthwise=True is the IN_C layout with DEPTHWISE grouping."""
+    if depthwise:
+        group_layout, autogroup_mode = GROUP_IN_C, AUTOGROUP_DEPTHWISE
+    if input_layout not in (LAYOUT_NXC, LAYOUT_NCX):
+        raise ValueError('Input tensor layout requested in conv op does not apply to convolution input tensors')
+    if filter_layout not in (LAYOUT_KCX, LAYOUT_XCK, LAYOUT_GKCX, LAYOUT_XGCK):
+        raise ValueError('Filter tensor layout requested in conv op does not apply to convolution filter tensors')
+    separate = filter_layout in (LAYOUT_GKCX, LAYOUT_XGCK)
+    rank = len(strides) if strides else len(I_or_O.shape) - 2
     strides = list(strides or [1] * rank)
     dilations = list(dilations or [1] * rank)
     data_dilations = list(data_dilations or [1] * rank)
     manual_padding = list(manual_padding or [])
-    if len(manual_padding) == rank:
-        manual_padding = manual_padding + manual_padding  # symmetric shorthand
-    while len(manual_padding) < 2 * rank:
-        manual_padding.append(0)
-    if manual_padding and builtins.any(manual_padding) and autopad != EXPLICIT:
+    result_shape = list(result_shape or [])
+    if manual_padding and autopad != EXPLICIT:
         raise ValueError('Autopadding and manual padding both requested for single conv operation')
-    N, CI = I.shape[0], I.shape[-1]
-    xs = I.shape[1:-1]
-    ks = F.shape[:rank]
-    F_CI, F_CO = F.shape[rank], F.shape[rank + 1]
-    if F_CI != CI:
-        raise ValueError('bind dims mismatch: filter input channels %d != %d' % (F_CI, CI))
-    G = CI if depthwise else 1
-    CO = F_CO * G if depthwise else F_CO
+    if len(dilations) != rank or len(data_dilations) != rank:
+        raise ValueError('Inconsistent spatial rank in conv op')
+    if separate != (group_layout == GROUP_SEPARATE):
+        raise ValueError('Filter layout and group layout disagree about separate groups')
+    if not result_shape and deriv_mode != DERIV_NONE and not infer_result_shape:
+        raise ValueError('Transposed/gradient convolutions require specifying the result_shape')
+    if result_shape and len(result_shape) != rank:
+        raise ValueError('Inconsistent spatial rank in conv op (result shape)')
+    while len(manual_padding) < rank:
+        manual_padding.append(0)
+    while len(manual_padding) < 2 * rank:
+        manual_padding.append(manual_padding[len(manual_padding) - rank])  # pad_hi defaults to pad_lo
+    # grouping strategy, ops.cc:811-875
+    if autogroup_mode == AUTOGROUP_UNGROUPED:
+        if groups != 1:
+            raise ValueError('Convolution AutoGroupMode::UNGROUPED requires groups == 1')
+    elif autogroup_mode == AUTOGROUP_AUTO:
+        if group_layout == GROUP_NONE:
+            groups, autogroup_mode = 1, AUTOGROUP_UNGROUPED
+        if group_layout == GROUP_IN_C:
+            raise ValueError('Cannot automatically detect group size of convolution with IN_C GroupLayout')
+    elif autogroup_mode == AUTOGROUP_EXPLICIT:
+        if groups < 1:
+            raise ValueError('Requested grouped convolution with fewer than 1 groups')
+        if group_layout == GROUP_NONE and groups != 1:
+            raise ValueError('GroupLayout not specified for grouped convolution')
+        if groups == 1:
+            autogroup_mode = AUTOGROUP_UNGROUPED
+    elif autogroup_mode == AUTOGROUP_DEPTHWISE:
+        if group_layout == GROUP_NONE:
+            raise ValueError('Convolution GroupLayout must be specified to use DEPTHWISE AutoGroupMode')
+    else:
+        raise ValueError('Unrecognized AutoGroupMode')
+
+    I = I_or_O if deriv_mode != DERIV_DATA else None
+    F = F_or_O if deriv_mode != DERIV_FILTER else None
+    O = I_or_O if deriv_mode == DERIV_DATA else (F_or_O if deriv_mode == DERIV_FILTER else None)
+
+    def split_data(t):
+        sh = list(t.shape)
+        if len(sh) != rank + 2:
+            raise ValueError('Inconsistent spatial rank in conv op (data tensor)')
+        return (sh[0], sh[1], sh[2:]) if input_layout == LAYOUT_NCX else (sh[0], sh[-1], sh[1:-1])
+
+    # what binding the tensors' dims yields
+    N = CI = CO = G = F_CI = F_CO = None
+    I_sp = O_sp = F_sp = None
+    if I is not None:
+        N, CI, I_sp = split_data(I)
+    if O is not None:
+        N, CO, O_sp = split_data(O)
+    if F is not None:
+        sh = list(F.shape)
+        if len(sh) != rank + (3 if separate else 2):
+            raise ValueError('Inconsistent spatial rank in conv op (filter tensor)')
+        if filter_layout in (LAYOUT_GKCX, LAYOUT_KCX):
+            if separate:
+                G, sh = sh[0], sh[1:]
+            F_CO, F_CI, F_sp = sh[0], sh[1], sh[2:]
+        else:
+            F_sp = sh[:rank]
+            if separate:
+                G = sh[rank]
+            F_CI, F_CO = sh[-2], sh[-1]
+        if filter_shape and list(filter_shape) != list(F_sp):
+            raise ValueError('bind dims mismatch: filter_shape %s != %s' % (list(filter_shape), F_sp))
+    if autogroup_mode in (AUTOGROUP_UNGROUPED, AUTOGROUP_EXPLICIT):
+        if G is not None and G != groups:
+            raise ValueError('bind dims mismatch: groups')
+        G = groups
+    elif autogroup_mode == AUTOGROUP_DEPTHWISE:
+        # G is the dim CI itself; IN_K and SEPARATE also pin the filter's input channels to 1
+        if group_layout in (GROUP_IN_K, GROUP_SEPARATE) and F_CI is not None and F_CI != 1:
+            raise ValueError('bind dims mismatch: depthwise filter input channels')
+        if group_layout == GROUP_IN_C and CI is None:
+            CI = F_CI
+        if CI is None:
+            raise ValueError('unbound dimension CI')
+        if G is not None and G != CI:
+            raise ValueError('bind dims mismatch: groups')
+        G = CI
+    if G is None:
+        raise ValueError('unbound dimension G')
+    # channel dims shared with, or derived from, the filter's (ops.cc:1063-1083, 1184-1199)
+    def same(a, b, what):
+        if a is not None and b is not None and a != b:
+            raise ValueError('bind dims mismatch: %s %d != %d' % (what, a, b))
+        return a if a is not None else b
+    if group_layout == GROUP_NONE:
+        CO, CI = same(CO, F_CO, 'CO'), same(CI, F_CI, 'CI')
+        F_CO, F_CI = CO, CI
+    elif group_layout == GROUP_IN_C:
+        CI = same(CI, F_CI, 'CI')
+        F_CI = CI
+        if F_CO is not None:
+            CO = F_CO * G
+    elif group_layout == GROUP_IN_K:
+        CO = same(CO, F_CO, 'CO')
+        F_CO = CO
+        if F_CI is not None:
+            CI = F_CI * G
+    else:
+        if F_CO is not None:
+            CO = F_CO * G
+        if F_CI is not None:
+            CI = F_CI * G
+    if deriv_mode == DERIV_FILTER:
+        # the filter's channel extents are whatever stayed unbound-but-derivable in the reference: only the
+        # layouts whose filter dims alias the data dims can be computed
+        if group_layout == GROUP_NONE:
+            F_CO, F_CI = CO, CI
+        elif group_layout == GROUP_IN_C:
+            F_CI = CI
+        elif group_layout == GROUP_IN_K:
+            F_CO = CO
+        if F_CO is None or F_CI is None:
+            raise ValueError('unbound filter channel dimension')
+    if CI is None or CO is None:
+        raise ValueError('unbound channel dimension')
+
+    pads = []
+    if deriv_mode == DERIV_NONE:
+        O_sp = []
+    if deriv_mode == DERIV_DATA:
+        I_sp = []
+    for i in range(rank):
+        if deriv_mode == DERIV_DATA and not result_shape:
+            p, size = compute_padding_and_input_size(O_sp[i], F_sp[i], strides[i], autopad, manual_padding[i],
+                                                     manual_padding[i + rank], dilations[i], data_dilations[i])
+            pads.append(p)
+            I_sp.append(size)
+            continue
+        if deriv_mode == DERIV_FILTER and not result_shape:
+            raise ValueError('Result shape inference not yet supported for filter transposed/derivative convolutions')
+        in_size = result_shape[i] if deriv_mode == DERIV_DATA else I_sp[i]
+        f_size = result_shape[i] if deriv_mode == DERIV_FILTER else F_sp[i]
+        p, o = compute_padding_and_output_size(in_size, f_size, strides[i], autopad, manual_padding[i],
+                                               manual_padding[i + rank], dilations[i], data_dilations[i])
+        pads.append(p)
+        if deriv_mode == DERIV_NONE:
+            O_sp.append(o)
+        if deriv_mode == DERIV_DATA:
+            I_sp.append(result_shape[i])
+
     n, co, ci, g = E.TensorIndexes(4)
     x = E.TensorIndexes(rank)
     k = E.TensorIndexes(rank)
-    pads, outs = [], []
-    for i in range(rank):
-        p, o = compute_padding_and_output_size(xs[i], ks[i], strides[i], autopad, manual_padding[i],
-                                               manual_padding[i + rank], dilations[i], data_dilations[i])
-        pads.append(p)
-        outs.append(o)
+    grouped = group_layout != GROUP_NONE
     sp = [(strides[i] * x[i] + dilations[i] * k[i] - pads[i]) // data_dilations[i] for i in range(rank)]
-    cons = []
-    if depthwise:
-        i_c = (CI // G) * g + ci
-        f_ci, f_co = (CI // G) * g + ci, co
-        o_c = (CO // G) * g + co
+    i_idxs = _data_order(input_layout, n, (CI // G) * g + ci if grouped else ci, sp)
+    o_idxs = _data_order(input_layout, n, (CO // G) * g + co if grouped else co, x)
+    f_co, f_ci, cons = co, ci, []
+    if group_layout == GROUP_IN_C:
+        f_ci = (CI // G) * g + ci
         cons.append(ci < CI // G)
+    elif group_layout == GROUP_IN_K:
+        f_co = (CO // G) * g + co
+        cons.append(co < CO // G)
+    f_idxs = _filter_order(filter_layout, g, f_co, f_ci, k)
+    if deriv_mode == DERIV_NONE:
+        c = E.Contraction(name).outShape(_data_order(input_layout, N, CO, O_sp)).outAccess(o_idxs)
+        c.sum(I[i_idxs] * F[f_idxs])
+    elif deriv_mode == DERIV_DATA:
+        c = E.Contraction(name).outShape(_data_order(input_layout, N, CI, I_sp)).outAccess(i_idxs)
+        c.sum(O[o_idxs] * F[f_idxs])
     else:
-        i_c, f_ci, f_co, o_c = ci, ci, co, co
-    c = E.Contraction(name).outShape([N] + outs + [CO]).outAccess([n] + x + [o_c])
-    c.sum(I[[n] + sp + [i_c]] * F[k + [f_ci, f_co]]).add_constraints(cons)
-    return c.build()
+        c = E.Contraction(name).outShape(_filter_order(filter_layout, G, F_CO, F_CI, result_shape)).outAccess(f_idxs)
+        c.sum(I[i_idxs] * O[o_idxs])
+    return c.add_constraints(cons).build()
 
 
 def pool(I, mode, pool_size, strides, autopad=VALID, manual_padding=None, include_padding_in_avg=False,

@@ -158,15 +158,76 @@ Value op_clip(const Value& value) {
   return Value{O};
 }
 
+// ---- convolution (plaidml/op/lib/ops.cc:671-877 validation, :879-1467 construction) ------------------------
+// One contraction relates I (data), F (filters) and O (result of the forward pass):
+//   O[n, x.., g*(CO/G)+co] += I[n, (s*x + d*k - pad)/dd .., g*(CI/G)+ci] * F[k.., f_ci, f_co]
+// deriv_mode picks which of the three is computed from the other two: NONE -> O, DATA -> I (a transposed
+// convolution), FILTER -> F.  The group layout says which filter channel dimension carries the group.
+
+size_t nonspatial_dims(TensorLayout layout) {
+  switch (layout) {
+    case TensorLayout::GKCX:
+    case TensorLayout::XGCK: return 3;
+    default: return 2;
+  }
+}
+
+// smallest input extent that yields `output_size` (ops.cc:383-418).  For the SAME modes the reference hands
+// back the output extent itself as the input extent; kept, since result shapes must agree with it.
+std::pair<TensorDim, TensorDim> compute_padding_and_input_size(const TensorDim& output_size, const TensorDim& filter_size,
+                                                               int64_t stride, AutoPadMode mode, int64_t pad_lo, int64_t pad_hi,
+                                                               int64_t dilation, int64_t data_dilation) {
+  if (data_dilation != 1) throw std::runtime_error("Cannot infer input data size for transposed convolution with data dilation");
+  TensorDim f_eff = (dilation * (filter_size - 1)) + 1;
+  switch (mode) {
+    case AutoPadMode::EXPLICIT: return {TensorDim(pad_lo), output_size * stride - pad_lo - pad_hi + f_eff - stride};
+    case AutoPadMode::VALID: return {TensorDim(0), output_size * stride + f_eff - stride};
+    case AutoPadMode::SAME_LOWER:
+    case AutoPadMode::SAME_UPPER: {
+      TensorDim input_size = output_size * stride - stride + 1;
+      const int64_t lower = mode == AutoPadMode::SAME_LOWER ? 1 : 0;
+      TensorDim pad_before = (edsl::max(0, (output_size - 1) * stride + f_eff - input_size) + lower) / 2;
+      return {pad_before, output_size};
+    }
+    default: throw std::runtime_error("Unexpected autopadding mode");
+  }
+}
+
+template <typename T>
+std::vector<T> data_order(TensorLayout layout, const T& n, const T& c, const std::vector<T>& spatial) {
+  std::vector<T> r = {n};
+  if (layout == TensorLayout::NCX) r.push_back(c);
+  r.insert(r.end(), spatial.begin(), spatial.end());
+  if (layout == TensorLayout::NXC) r.push_back(c);
+  return r;
+}
+
+template <typename T>
+std::vector<T> filter_order(TensorLayout layout, const T& g, const T& k, const T& c, const std::vector<T>& spatial) {
+  std::vector<T> r;
+  if (layout == TensorLayout::GKCX || layout == TensorLayout::KCX) {
+    if (layout == TensorLayout::GKCX) r.push_back(g);
+    r.push_back(k);
+    r.push_back(c);
+    r.insert(r.end(), spatial.begin(), spatial.end());
+  } else {
+    r.insert(r.end(), spatial.begin(), spatial.end());
+    if (layout == TensorLayout::XGCK) r.push_back(g);
+    r.push_back(c);
+    r.push_back(k);
+  }
+  return r;
+}
+
 Value op_convolution(const Value& value) {
   auto args = value.as_tuple();
   if (args.size() != 18) throw std::runtime_error("Convolution op expects 18 arguments");
-  auto I = args[0].as_tensor();
-  auto F = args[1].as_tensor();
+  auto I_or_O = args[0].as_tensor();  // O when deriv_mode is DATA
+  auto F_or_O = args[1].as_tensor();  // O when deriv_mode is FILTER
   auto strides = args[2].as_int_tuple_or_empty();
   auto dilations = args[3].as_int_tuple_or_empty();
   auto data_dilations = args[4].as_int_tuple_or_empty();
-  auto filter_shape = args[5].as_int_tuple_or_empty();
+  auto filter_shape = args[5].as_int_tuple_or_empty();  // spatial filter dims only
   auto groups = args[6].as_int();
   auto autopad_mode = validate<AutoPadMode>(args[7].as_int());
   auto manual_padding = args[8].as_int_tuple_or_empty();
@@ -176,120 +237,195 @@ Value op_convolution(const Value& value) {
   auto name = args[13].as_str();
   auto autogroup_mode = validate<AutoGroupMode>(args[14].as_int());
   auto deriv_mode = validate<ConvDerivMode>(args[15].as_int());
+  auto result_shape = args[16].as_int_tuple_or_empty();
+  const bool infer_result_shape = args[17].as_bool();
   if (name.empty()) name = "conv";
-  if (deriv_mode != ConvDerivMode::NONE) throw std::runtime_error("Only forward convolutions are supported by this backend");
-  if (input_layout != TensorLayout::NXC && input_layout != TensorLayout::NCX) throw std::runtime_error("Invalid input_layout");
-  if (filter_layout != TensorLayout::XCK && filter_layout != TensorLayout::KCX)
-    throw std::runtime_error("Only XCK and KCX filter layouts are supported by this backend");
-  if (group_layout != GroupLayout::NONE && group_layout != GroupLayout::IN_C)
-    throw std::runtime_error("Only the NONE and IN_C group layouts are supported by this backend");
-  if (I.rank() < 3 || F.rank() != I.rank()) throw std::runtime_error("Convolution input and filter rank mismatch");
-  const size_t spatial_rank = I.rank() - 2;
-  if (strides.empty()) strides.assign(spatial_rank, 1);
-  if (dilations.empty()) dilations.assign(spatial_rank, 1);
-  if (data_dilations.empty()) data_dilations.assign(spatial_rank, 1);
-  if (strides.size() != spatial_rank || dilations.size() != spatial_rank || data_dilations.size() != spatial_rank)
-    throw std::runtime_error("Convolution strides / dilations rank mismatch");
+
+  Tensor I, F, O;
+  switch (deriv_mode) {
+    case ConvDerivMode::NONE: I = I_or_O; F = F_or_O; break;
+    case ConvDerivMode::DATA: O = I_or_O; F = F_or_O; break;
+    case ConvDerivMode::FILTER: I = I_or_O; O = F_or_O; break;
+    default: throw std::runtime_error("Invalid ConvDerivMode");
+  }
+
+  // ---- validation and defaults (ops.cc:671-877)
+  const bool is_data_layout = input_layout == TensorLayout::NXC || input_layout == TensorLayout::NCX;
+  if (!is_data_layout) throw std::runtime_error("Input tensor layout requested in conv op does not apply to convolution input tensors");
+  const bool separate_groups = filter_layout == TensorLayout::GKCX || filter_layout == TensorLayout::XGCK;
+  if (!separate_groups && filter_layout != TensorLayout::KCX && filter_layout != TensorLayout::XCK)
+    throw std::runtime_error("Filter tensor layout requested in conv op does not apply to convolution filter tensors");
+  size_t spatial_rank = strides.size();
+  if (spatial_rank == 0) {
+    if (I_or_O.rank() < nonspatial_dims(input_layout)) throw std::runtime_error("Convolution data tensor has too few dimensions");
+    spatial_rank = I_or_O.rank() - nonspatial_dims(input_layout);
+    strides.assign(spatial_rank, 1);
+  }
   if (!manual_padding.empty() && autopad_mode != AutoPadMode::EXPLICIT)
     throw std::runtime_error("Autopadding and manual padding both requested for single conv operation");
-  if (manual_padding.size() == spatial_rank) {
-    // one value per dimension pads both sides
-    auto lo = manual_padding;
-    manual_padding.insert(manual_padding.end(), lo.begin(), lo.end());
+  auto rank_text = [&](size_t got, const char* what) {
+    return "Inconsistent spatial rank in conv op (expecting rank " + std::to_string(spatial_rank) + ", received " +
+           std::to_string(got) + "D " + what + ")";
+  };
+  if (dilations.empty()) dilations.assign(spatial_rank, 1);
+  if (dilations.size() != spatial_rank) throw std::runtime_error(rank_text(dilations.size(), "dilations"));
+  if (data_dilations.empty()) data_dilations.assign(spatial_rank, 1);
+  if (data_dilations.size() != spatial_rank) throw std::runtime_error(rank_text(data_dilations.size(), "data_dilations"));
+  if (deriv_mode != ConvDerivMode::DATA && I.rank() != spatial_rank + nonspatial_dims(input_layout))
+    throw std::runtime_error("Inconsistent spatial rank in conv op (expected spatial rank " + std::to_string(spatial_rank) +
+                             " but input tensor has " + std::to_string(I.rank()) + " dimensions)");
+  if (deriv_mode != ConvDerivMode::FILTER && F.rank() != spatial_rank + nonspatial_dims(filter_layout))
+    throw std::runtime_error("Inconsistent spatial rank in conv op (expected spatial rank " + std::to_string(spatial_rank) +
+                             " but filter tensor has " + std::to_string(F.rank()) + " dimensions)");
+  if (!filter_shape.empty() && filter_shape.size() != spatial_rank)
+    throw std::runtime_error("Filter shape manually specified with inconsistent rank (expected spatial rank " +
+                             std::to_string(spatial_rank) + " but filter_shape has " + std::to_string(filter_shape.size()) + " dimensions)");
+  if (separate_groups && group_layout != GroupLayout::SEPARATE)
+    throw std::runtime_error("Filter_layout specifies separate groups but group_layout isn't SEPARATE");
+  if (!separate_groups && group_layout == GroupLayout::SEPARATE)
+    throw std::runtime_error("Filter_layout lacks separate groups but group_layout is SEPARATE");
+  if (result_shape.empty()) {
+    if (deriv_mode != ConvDerivMode::NONE && !infer_result_shape)
+      throw std::runtime_error(
+          "Transposed/gradient convolutions require specifying the result_shape. This can be bypassed by setting "
+          "infer_result_shape = true, but be warned that infered result shapes do not necessarily match the input "
+          "shape used in the forward convolution, as multiple input shapes produce the same output shape.");
+  } else if (result_shape.size() != spatial_rank) {
+    throw std::runtime_error("Inconsistent spatial rank in conv op (received " + std::to_string(spatial_rank) +
+                             " spatial dimensions based on strides but result shape has " + std::to_string(result_shape.size()) +
+                             " spatial dims).");
   }
-  manual_padding.resize(2 * spatial_rank, 0);
-  if ((group_layout == GroupLayout::NONE) != (autogroup_mode == AutoGroupMode::UNGROUPED))
-    throw std::runtime_error("Convolution group layout and autogroup mode are inconsistent");
+  if (manual_padding.size() > 2 * spatial_rank)
+    throw std::runtime_error("Inconsistent spatial rank: operation with " + std::to_string(spatial_rank) + " spatial dimensions had " +
+                             std::to_string(manual_padding.size()) + " manual padding values given");
+  while (manual_padding.size() < spatial_rank) manual_padding.push_back(0);
+  while (manual_padding.size() < 2 * spatial_rank) manual_padding.push_back(manual_padding[manual_padding.size() - spatial_rank]);
+  // grouping strategy (ops.cc:811-875)
+  switch (autogroup_mode) {
+    case AutoGroupMode::UNGROUPED:
+      if (groups != 1) throw std::runtime_error("Convolution AutoGroupMode::UNGROUPED requires groups == 1");
+      break;
+    case AutoGroupMode::AUTO:
+      if (group_layout == GroupLayout::NONE) {
+        groups = 1;
+        autogroup_mode = AutoGroupMode::UNGROUPED;
+      }
+      if (group_layout == GroupLayout::IN_C)
+        throw std::runtime_error("Cannot automatically detect group size of convolution with IN_C GroupLayout");
+      break;
+    case AutoGroupMode::EXPLICIT:
+      if (groups < 1) throw std::runtime_error("Requested grouped convolution with fewer than 1 groups");
+      if (groups == 1) autogroup_mode = AutoGroupMode::UNGROUPED;
+      if (group_layout == GroupLayout::NONE && groups != 1) throw std::runtime_error("GroupLayout not specified for grouped convolution");
+      break;
+    case AutoGroupMode::DEPTHWISE:
+      if (group_layout == GroupLayout::NONE)
+        throw std::runtime_error("Convolution GroupLayout must be specified to use DEPTHWISE AutoGroupMode");
+      break;
+    default: throw std::runtime_error("Unrecognized AutoGroupMode");
+  }
 
+  // ---- dimensions.  TensorDims alias on copy, so a dim bound through one name is bound under every name.
   TensorDim N, CI, CO, G, F_CI, F_CO;
   TensorIndex n("n"), ci("ci"), co("co"), g("g");
-  std::vector<TensorDim> I_spatial(spatial_rank), F_spatial(spatial_rank);
+  std::vector<TensorDim> I_spatial(spatial_rank), O_spatial(spatial_rank), F_spatial(spatial_rank);
   std::vector<TensorIndex> x, k;
   for (size_t i = 0; i < spatial_rank; ++i) {
     x.emplace_back("x" + std::to_string(i));
     k.emplace_back("k" + std::to_string(i));
   }
-  // bind the input and filter dims
-  std::vector<TensorDim> I_dims = {N};
-  if (input_layout == TensorLayout::NCX) I_dims.push_back(CI);
-  for (auto& d : I_spatial) I_dims.push_back(d);
-  if (input_layout == TensorLayout::NXC) I_dims.push_back(CI);
-  I.bind_dims(I_dims);
-  if (group_layout == GroupLayout::NONE) {
-    F_CI = CI;
-  } else {
-    F_CI = CI;  // IN_C: the filter's input-channel dimension carries the group
-  }
-  std::vector<TensorDim> F_dims;
-  if (filter_layout == TensorLayout::KCX) {
-    F_dims = {F_CO, F_CI};
-    for (auto& d : F_spatial) F_dims.push_back(d);
-  } else {
-    for (auto& d : F_spatial) F_dims.push_back(d);
-    F_dims.push_back(F_CI);
-    F_dims.push_back(F_CO);
-  }
-  F.bind_dims(F_dims);
-  if (!filter_shape.empty()) {
-    if (filter_shape.size() != spatial_rank) throw std::runtime_error("Filter shape rank mismatch");
-    std::vector<TensorDim> explicit_dims = F_dims;
-    const size_t off = filter_layout == TensorLayout::KCX ? 2 : 0;
-    for (size_t i = 0; i < spatial_rank; ++i) explicit_dims[off + i] = TensorDim(filter_shape[i]);
-    F.bind_dims(explicit_dims);
-  }
   switch (autogroup_mode) {
-    case AutoGroupMode::UNGROUPED: G = TensorDim(1); break;
-    case AutoGroupMode::EXPLICIT: G = TensorDim(groups); break;
-    case AutoGroupMode::DEPTHWISE: G = CI; break;
-    default: throw std::runtime_error("Unsupported autogroup mode");
+    case AutoGroupMode::EXPLICIT:
+    case AutoGroupMode::UNGROUPED: G = TensorDim(groups); break;
+    case AutoGroupMode::DEPTHWISE:
+      G = CI;
+      if (group_layout == GroupLayout::IN_K || group_layout == GroupLayout::SEPARATE) F_CI = TensorDim(1);
+      break;
+    case AutoGroupMode::AUTO:  // SEPARATE / IN_K: G is whatever binding the tensors gives it
+      break;
+    default: break;
   }
-  CO = group_layout == GroupLayout::IN_C ? F_CO * G : F_CO;
+  switch (group_layout) {
+    case GroupLayout::NONE: F_CO = CO; F_CI = CI; break;
+    case GroupLayout::IN_C: F_CI = CI; break;   // CO = F_CO * G below
+    case GroupLayout::IN_K: F_CO = CO; break;   // CI = F_CI * G below
+    case GroupLayout::SEPARATE: break;          // both below
+    default: throw std::runtime_error("Invalid group_layout");
+  }
+  if (deriv_mode != ConvDerivMode::DATA) I.bind_dims(data_order(input_layout, N, CI, I_spatial));
+  if (deriv_mode != ConvDerivMode::FILTER) {
+    F.bind_dims(filter_order(filter_layout, G, F_CO, F_CI, F_spatial));
+    if (!filter_shape.empty()) {
+      std::vector<TensorDim> stated;
+      for (int64_t v : filter_shape) stated.emplace_back(v);
+      F.bind_dims(filter_order(filter_layout, G, F_CO, F_CI, stated));  // must agree with the tensor's own extents
+    }
+  }
+  if (deriv_mode != ConvDerivMode::NONE) O.bind_dims(data_order(input_layout, N, CO, O_spatial));
+  switch (group_layout) {
+    case GroupLayout::IN_C: CO = F_CO * G; break;
+    case GroupLayout::IN_K: CI = F_CI * G; break;
+    case GroupLayout::SEPARATE: CO = F_CO * G; CI = F_CI * G; break;
+    default: break;
+  }
 
-  std::vector<TensorDim> O_spatial, pad_before;
+  // ---- padding and the extents of whichever tensor is being computed (ops.cc:1201-1255)
+  std::vector<TensorDim> pad_before;
+  if (deriv_mode == ConvDerivMode::NONE) O_spatial.clear();
+  if (deriv_mode == ConvDerivMode::DATA) I_spatial.clear();
   for (size_t i = 0; i < spatial_rank; ++i) {
-    auto pr = compute_padding_and_output_size(I_spatial[i], F_spatial[i], strides[i], autopad_mode, manual_padding[i],
+    if (deriv_mode == ConvDerivMode::DATA && result_shape.empty()) {
+      auto pr = compute_padding_and_input_size(O_spatial[i], F_spatial[i], strides[i], autopad_mode, manual_padding[i],
+                                               manual_padding[i + spatial_rank], dilations[i], data_dilations[i]);
+      pad_before.push_back(pr.first);
+      I_spatial.push_back(pr.second);
+      continue;
+    }
+    if (deriv_mode == ConvDerivMode::FILTER && result_shape.empty())
+      throw std::runtime_error("Result shape inference not yet supported for filter transposed/derivative convolutions");
+    TensorDim in_size = deriv_mode == ConvDerivMode::DATA ? TensorDim(result_shape[i]) : I_spatial[i];
+    TensorDim f_size = deriv_mode == ConvDerivMode::FILTER ? TensorDim(result_shape[i]) : F_spatial[i];
+    auto pr = compute_padding_and_output_size(in_size, f_size, strides[i], autopad_mode, manual_padding[i],
                                               manual_padding[i + spatial_rank], dilations[i], data_dilations[i], false);
     pad_before.push_back(pr.first);
-    O_spatial.push_back(pr.second);
+    if (deriv_mode == ConvDerivMode::NONE) O_spatial.push_back(pr.second);
+    if (deriv_mode == ConvDerivMode::DATA) I_spatial.push_back(TensorDim(result_shape[i]));
   }
-  std::vector<TensorDim> O_dims = {N};
-  if (input_layout == TensorLayout::NCX) O_dims.push_back(CO);
-  for (auto& d : O_spatial) O_dims.push_back(d);
-  if (input_layout == TensorLayout::NXC) O_dims.push_back(CO);
 
-  // index formulas (ops.cc:1342-1450)
+  // ---- index formulas (ops.cc:1342-1450)
   std::vector<Constraint> constraints;
-  TensorIndex i_c = group_layout == GroupLayout::NONE ? ci : (CI / G) * g + ci;
-  TensorIndex o_c = group_layout == GroupLayout::NONE ? co : (CO / G) * g + co;
-  TensorIndex f_ci = group_layout == GroupLayout::NONE ? ci : (CI / G) * g + ci;
-  TensorIndex f_co = co;
-  if (group_layout == GroupLayout::IN_C) constraints.push_back(ci < CI / G);
-  std::vector<TensorIndex> spatial;
+  const bool grouped = group_layout != GroupLayout::NONE;
+  std::vector<TensorIndex> I_sp;
   for (size_t i = 0; i < spatial_rank; ++i)
-    spatial.push_back((strides[i] * x[i] + dilations[i] * k[i] - pad_before[i]) / data_dilations[i]);
-  std::vector<TensorIndex> I_idxs = {n}, O_idxs = {n}, F_idxs;
-  if (input_layout == TensorLayout::NCX) {
-    I_idxs.push_back(i_c);
-    O_idxs.push_back(o_c);
+    I_sp.push_back((strides[i] * x[i] + dilations[i] * k[i] - pad_before[i]) / data_dilations[i]);
+  auto I_idxs = data_order<TensorIndex>(input_layout, n, grouped ? (CI / G) * g + ci : ci, I_sp);
+  auto O_idxs = data_order<TensorIndex>(input_layout, n, grouped ? (CO / G) * g + co : co, x);
+  TensorIndex f_co = co, f_ci = ci;
+  if (group_layout == GroupLayout::IN_C) {
+    f_ci = (CI / G) * g + ci;
+    constraints.push_back(ci < CI / G);
+  } else if (group_layout == GroupLayout::IN_K) {
+    f_co = (CO / G) * g + co;
+    constraints.push_back(co < CO / G);
   }
-  for (size_t i = 0; i < spatial_rank; ++i) {
-    I_idxs.push_back(spatial[i]);
-    O_idxs.push_back(x[i]);
+  auto F_idxs = filter_order<TensorIndex>(filter_layout, g, f_co, f_ci, k);
+
+  switch (deriv_mode) {
+    case ConvDerivMode::NONE: {
+      Tensor R = Contraction(data_order(input_layout, N, CO, O_spatial), O_idxs, name).sum(I(I_idxs) * F(F_idxs)).add_constraints(constraints);
+      return Value{R};
+    }
+    case ConvDerivMode::DATA: {
+      Tensor R = Contraction(data_order(input_layout, N, CI, I_spatial), I_idxs, name).sum(O(O_idxs) * F(F_idxs)).add_constraints(constraints);
+      return Value{R};
+    }
+    default: {
+      std::vector<TensorDim> stated;
+      for (int64_t v : result_shape) stated.emplace_back(v);
+      Tensor R = Contraction(filter_order(filter_layout, G, F_CO, F_CI, stated), F_idxs, name).sum(I(I_idxs) * O(O_idxs)).add_constraints(constraints);
+      return Value{R};
+    }
   }
-  if (input_layout == TensorLayout::NXC) {
-    I_idxs.push_back(i_c);
-    O_idxs.push_back(o_c);
-  }
-  if (filter_layout == TensorLayout::KCX) {
-    F_idxs = {f_co, f_ci};
-    for (auto& kk : k) F_idxs.push_back(kk);
-  } else {
-    for (auto& kk : k) F_idxs.push_back(kk);
-    F_idxs.push_back(f_ci);
-    F_idxs.push_back(f_co);
-  }
-  Tensor O = Contraction(O_dims, O_idxs, name).sum(I(I_idxs) * F(F_idxs)).add_constraints(constraints);
-  return Value{O};
 }
 
 Value op_dot(const Value& value) {

@@ -18,12 +18,21 @@ def _ints(x):
     return None if x is None else [int(v) for v in x]
 
 
+DERIV_NONE, DERIV_DATA, DERIV_FILTER = range(3)
+
+
 def convolution(I, F, strides=None, dilations=None, data_dilations=None, autopad=SAME_UPPER, manual_padding=None,
-                depthwise=False, name=''):
-    """NXC input, XCK filter.  depthwise=True is GroupLayout IN_C with AutoGroupMode DEPTHWISE."""
-    args = [I, F, _ints(strides), _ints(dilations), _ints(data_dilations), None, 1, _AUTOPAD[autopad],
-            _ints(manual_padding), LAYOUT_NXC, LAYOUT_XCK, GROUP_IN_C if depthwise else GROUP_NONE, False, name,
-            AUTOGROUP_DEPTHWISE if depthwise else AUTOGROUP_UNGROUPED, 0, None, False]
+                depthwise=False, name='', groups=1, input_layout=LAYOUT_NXC, filter_layout=LAYOUT_XCK,
+                group_layout=GROUP_NONE, autogroup_mode=AUTOGROUP_UNGROUPED, deriv_mode=DERIV_NONE, result_shape=None,
+                infer_result_shape=False, filter_shape=None):
+    """The 18 arguments of the reference's convolution (plaidml/op/op.h:192-335).  With deriv_mode DATA the first
+    tensor is the forward result, with FILTER the second one is.  depthwise=True is GroupLayout IN_C with
+    AutoGroupMode DEPTHWISE."""
+    if depthwise:
+        group_layout, autogroup_mode = GROUP_IN_C, AUTOGROUP_DEPTHWISE
+    args = [I, F, _ints(strides), _ints(dilations), _ints(data_dilations), _ints(filter_shape), int(groups), _AUTOPAD[autopad],
+            _ints(manual_padding), int(input_layout), int(filter_layout), int(group_layout), False, name,
+            int(autogroup_mode), int(deriv_mode), _ints(result_shape), bool(infer_result_shape)]
     return E.op_make('convolution', args).as_tensor()
 
 
