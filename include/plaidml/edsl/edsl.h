@@ -441,6 +441,95 @@ PLAIDML_EDSL_TENSOR_OPS(||, "logical_or")
 
 inline Tensor abs(const Tensor& x) { return select(x < 0.0, -x, x); }
 
+// ---- special operations: argsort, gather, scatter (plaidml/edsl/edsl.h:800-811, 1034-1066, 1625-1765) ----
+enum class SortDirection : uint64_t { ASC, DESC };
+
+inline Tensor argsort(const Tensor& x, int axis = -1, SortDirection direction = SortDirection::ASC) {
+  return intrinsicCall("argsort", {x, Tensor(static_cast<int64_t>(axis)), Tensor(static_cast<int64_t>(direction))});
+}
+
+enum class InterpolationMode : uint64_t { NEAREST, LINEAR, CUBIC, NONE };
+enum class NearestMode : uint64_t { ROUND_PREFER_FLOOR, ROUND_PREFER_CEIL, FLOOR, CEIL, SIMPLE, NONE };
+enum class GatherMode : uint64_t { NORMAL, ND };
+enum class OutOfBoundsMode : uint64_t { GATHER_EDGE_PADDED_INPUT, RETURN_ZERO };
+enum class ScatterMode : uint64_t { NORMAL, UPDATE_SLICE, UPDATE_ELT, UPDATE_ND };
+
+// the nine-argument gather intrinsic; `gather` below and op::gatherND fill it in
+class gatherBuilder {
+ public:
+  gatherBuilder(Tensor x, Tensor y, uint64_t axis, InterpolationMode interpolation_mode, NearestMode nearest_mode,
+                OutOfBoundsMode out_of_bounds_mode, float cube_coeff)
+      : x_(x), y_(y), axis_(axis), cube_coeff_(cube_coeff), mode_(GatherMode::NORMAL), out_of_bounds_mode_(out_of_bounds_mode),
+        nearest_mode_(nearest_mode), interpolation_mode_(interpolation_mode) {}
+  gatherBuilder(Tensor x, Tensor y, uint64_t batch_dims, InterpolationMode interpolation_mode)
+      : x_(x), y_(y), batch_dims_(batch_dims), mode_(GatherMode::ND), interpolation_mode_(interpolation_mode) {}
+  Tensor build() const {
+    return intrinsicCall("gather", {x_, y_, Tensor(axis_), Tensor(static_cast<uint64_t>(interpolation_mode_)),
+                                    Tensor(static_cast<uint64_t>(nearest_mode_)), Tensor(static_cast<double>(cube_coeff_)),
+                                    Tensor(static_cast<uint64_t>(mode_)), Tensor(batch_dims_),
+                                    Tensor(static_cast<uint64_t>(out_of_bounds_mode_))});
+  }
+
+ private:
+  Tensor x_, y_;
+  uint64_t axis_ = 0, batch_dims_ = 0;
+  float cube_coeff_ = -0.75;
+  GatherMode mode_ = GatherMode::NORMAL;
+  OutOfBoundsMode out_of_bounds_mode_ = OutOfBoundsMode::GATHER_EDGE_PADDED_INPUT;
+  NearestMode nearest_mode_ = NearestMode::ROUND_PREFER_FLOOR;
+  InterpolationMode interpolation_mode_ = InterpolationMode::NONE;
+};
+
+// x taken along `axis` at the positions y; a number in place of y reads that one position
+class gather {
+ public:
+  gather(const Tensor& x, const Tensor& y) : x_(x), y_(y) {}
+  gather(const Tensor& x, int i) : x_(x), y_(cast(index({TensorDim(1)}, 0), DType::INT32) + i) {}
+  gather(const Tensor& x, int64_t i) : x_(x), y_(cast(index({TensorDim(1)}, 0), DType::INT64) + i) {}
+  gather(const Tensor& x, uint64_t i) : x_(x), y_(cast(index({TensorDim(1)}, 0), DType::UINT64) + i) {}
+  gather(const Tensor& x, float f) : x_(x), y_(cast(index({TensorDim(1)}, 0), DType::FLOAT32) + static_cast<double>(f)) {}
+  gather(const Tensor& x, double f) : x_(x), y_(cast(index({TensorDim(1)}, 0), DType::FLOAT64) + f) {}
+  gather& axis(int64_t axis) {
+    if (axis < 0) axis += static_cast<int64_t>(x_.rank());
+    axis_ = static_cast<uint64_t>(axis);
+    return *this;
+  }
+  gather& interpolationMode(InterpolationMode mode) { interpolation_mode_ = mode; return *this; }
+  gather& nearestMode(NearestMode mode) { nearest_mode_ = mode; return *this; }
+  gather& cubeCoeff(float cube_coeff) { cube_coeff_ = cube_coeff; return *this; }
+  gather& outOfBoundsMode(OutOfBoundsMode mode) { out_of_bounds_mode_ = mode; return *this; }
+  operator Tensor() const {  // NOLINT: the reference converts implicitly
+    return gatherBuilder(x_, y_, axis_, interpolation_mode_, nearest_mode_, out_of_bounds_mode_, cube_coeff_).build();
+  }
+
+ private:
+  Tensor x_, y_;
+  uint64_t axis_ = 0;
+  InterpolationMode interpolation_mode_ = InterpolationMode::NONE;
+  NearestMode nearest_mode_ = NearestMode::ROUND_PREFER_FLOOR;
+  OutOfBoundsMode out_of_bounds_mode_ = OutOfBoundsMode::GATHER_EDGE_PADDED_INPUT;
+  float cube_coeff_ = -0.75;
+};
+
+// a copy of x with the elements of z written (or, in NORMAL mode, added) at the places y names
+class scatter {
+ public:
+  scatter(const Tensor& x, const Tensor& y, const Tensor& z) : x_(x), y_(y), z_(z) {}
+  scatter& axis(int64_t axis) {
+    if (axis < 0) axis += static_cast<int64_t>(x_.rank());
+    axis_ = axis;
+    return *this;
+  }
+  scatter& mode(ScatterMode mode) { mode_ = mode; return *this; }
+  Tensor build() const { return intrinsicCall("scatter", {x_, y_, z_, Tensor(axis_), Tensor(static_cast<uint64_t>(mode_))}); }
+  operator Tensor() const { return build(); }  // NOLINT
+
+ private:
+  Tensor x_, y_, z_;
+  int64_t axis_ = 0;
+  ScatterMode mode_ = ScatterMode::NORMAL;
+};
+
 // ---- Value: the variant handed to the operation library --------------------------
 class Value {
  public:

@@ -323,6 +323,68 @@ int pml_hip_select(const pml_hip_select_desc* desc, const void* cond, const void
 /* index(dims, axis) (tile.index, IndexOpConversion tile_to_linalg.cc:863-): int32 iota along `axis` */
 int pml_hip_index(void* out, int32_t rank, const int64_t* sizes, int32_t axis, pml_hip_stream s);
 
+/* ---- special operations --------------------------------------------------------
+ * The three Tile operations that are not contractions or elementwise maps
+ * (ArgSortOpConversion / GatherOpConversion / ScatterOpConversion,
+ * pmlc/conversion/linalg_to_pxa/tile_to_pxa_special_patterns.cc:29-896).  Dense
+ * row-major tensors; enum values follow plaidml/edsl/edsl.h:1034,1625-1642. */
+#define PML_HIP_MAX_SPECIAL_RANK 8
+
+enum { PML_HIP_INTERP_NEAREST = 0, PML_HIP_INTERP_LINEAR, PML_HIP_INTERP_CUBIC, PML_HIP_INTERP_NONE };
+enum {
+  PML_HIP_NEAREST_ROUND_PREFER_FLOOR = 0,
+  PML_HIP_NEAREST_ROUND_PREFER_CEIL,
+  PML_HIP_NEAREST_FLOOR,
+  PML_HIP_NEAREST_CEIL,
+  PML_HIP_NEAREST_SIMPLE,
+  PML_HIP_NEAREST_NONE
+};
+enum { PML_HIP_GATHER_NORMAL = 0, PML_HIP_GATHER_ND = 1 };
+enum { PML_HIP_OOB_EDGE_PADDED_INPUT = 0, PML_HIP_OOB_RETURN_ZERO = 1 };
+enum { PML_HIP_SCATTER_NORMAL = 0, PML_HIP_SCATTER_UPDATE_SLICE, PML_HIP_SCATTER_UPDATE_ELT, PML_HIP_SCATTER_UPDATE_ND };
+
+/* gather: NORMAL  out[a.., i.., b..] = tensor[a.., f(indices[i..]), b..] along `axis`; integer indices address
+ * directly (no clamping, as in the reference), floating indices of a floating tensor interpolate (nearest /
+ * linear / cubic, taps clamped to the edge, optionally zero outside), floating indices of an integer tensor
+ * truncate.  ND  out[i.., b..] = tensor[batch.., indices[i.., 0..k-1].., b..] with `batch_dims` leading
+ * dimensions shared by tensor and indices. */
+typedef struct {
+  int32_t dtype;     /* element type of tensor and result */
+  int32_t idx_dtype; /* element type of indices */
+  int32_t mode, interpolation, nearest, oob;
+  int32_t axis, batch_dims;
+  int32_t rank, idx_rank;
+  double cube_coeff;
+  int64_t sizes[PML_HIP_MAX_SPECIAL_RANK];     /* tensor */
+  int64_t idx_sizes[PML_HIP_MAX_SPECIAL_RANK]; /* indices */
+} pml_hip_gather_desc;
+int pml_hip_gather(const pml_hip_gather_desc* desc, const void* tensor, const void* indices, void* out, pml_hip_stream s);
+
+/* scatter: out = data, then every element of `updates` goes to the place its indices name: NORMAL adds
+ * (duplicates accumulate; floating sums in arrival order), the UPDATE modes assign (duplicate targets are a
+ * race there, as in the reference's parallel loop).  Indices are si32 / ui32.  `out` must not alias `data`. */
+typedef struct {
+  int32_t dtype;
+  int32_t idx_dtype;
+  int32_t mode, axis;
+  int32_t rank, idx_rank, upd_rank, reserved;
+  int64_t sizes[PML_HIP_MAX_SPECIAL_RANK];     /* data and result */
+  int64_t idx_sizes[PML_HIP_MAX_SPECIAL_RANK];
+  int64_t upd_sizes[PML_HIP_MAX_SPECIAL_RANK];
+} pml_hip_scatter_desc;
+int pml_hip_scatter(const pml_hip_scatter_desc* desc, const void* data, const void* indices, const void* updates, void* out,
+                    pml_hip_stream s);
+
+/* argsort along `axis`: out (si32, shape of the input) holds the positions of the input's elements in
+ * ascending (direction 0) or descending (1) order; equal elements keep their input order (the reference's
+ * stable selection sort with strict ordered compares). */
+typedef struct {
+  int32_t dtype;
+  int32_t rank, axis, direction;
+  int64_t sizes[PML_HIP_MAX_SPECIAL_RANK];
+} pml_hip_argsort_desc;
+int pml_hip_argsort(const pml_hip_argsort_desc* desc, const void* tensor, void* out, pml_hip_stream s);
+
 /* ---- any contraction ---------------------------------------------------------
  * The loop-nest form a contraction takes after bounds computation: the
  * `affine.parallel` + `pxa.load` + `pxa.reduce` nest of
@@ -372,7 +434,7 @@ int pml_hip_contract_invoke(int64_t plan, const void* const* srcs, void* out, pm
 
 /* sizeof() of a descriptor struct as this library was compiled, so that a foreign-language
  * binding can verify its own layout: 0 epilogue, 1 gemm, 2 conv2d, 3 dwconv2d, 4 pool2d,
- * 5 eltwise, 6 select, 7 contract, 8 form.  Returns 0 for an unknown id. */
+ * 5 eltwise, 6 select, 7 contract, 8 form, 9 gather, 10 scatter, 11 argsort.  Returns 0 for an unknown id. */
 size_t pml_hip_struct_size(int which);
 
 /* Releases a plan returned by any *_dispatch. */

@@ -21,6 +21,8 @@ computes for a Tile program:
   * `C + bias` after a sum contraction starts the accumulator from the bias
     (pmlc/dialect/tile/transforms/algebraic_opt.cc:30-75)
   * contraction scalar semantics: tile_oracle.c
+  * the special operations argsort / gather / scatter:
+    pmlc/conversion/linalg_to_pxa/tile_to_pxa_special_patterns.cc:29-896, shapes pmlc/ast/ast_ops.cc:41-257
   * elementwise scalar semantics and casts:
     pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:1227-1385,
     pmlc/conversion/tile_to_linalg/utils.cc:35-91 (fp->int truncates toward zero,
@@ -627,6 +629,173 @@ def round(x):  # noqa: A001 - mirrors the EDSL name
     return intrinsic('round', x)
 
 
+# ---- special operations ------------------------------------------------------------------------------------
+SORT_ASC, SORT_DESC = range(2)
+INTERP_NEAREST, INTERP_LINEAR, INTERP_CUBIC, INTERP_NONE = range(4)
+NEAREST_ROUND_PREFER_FLOOR, NEAREST_ROUND_PREFER_CEIL, NEAREST_FLOOR, NEAREST_CEIL, NEAREST_SIMPLE, NEAREST_NONE = range(6)
+GATHER_NORMAL, GATHER_ND = range(2)
+OOB_EDGE_PADDED_INPUT, OOB_RETURN_ZERO = range(2)
+SCATTER_NORMAL, SCATTER_UPDATE_SLICE, SCATTER_UPDATE_ELT, SCATTER_UPDATE_ND = range(4)
+
+
+def argsort(x, axis=-1, direction=SORT_ASC):
+    """Shape rule pmlc/ast/ast_ops.cc:41-60: si32 positions, the input's shape."""
+    x = _literal(x)
+    return Tensor('special', DType.INT32, x.shape, (x,), {'fn': 'argsort', 'axis': int(axis), 'direction': int(direction)})
+
+
+def gather(x, y, axis=0, interpolation_mode=INTERP_NONE, nearest_mode=NEAREST_ROUND_PREFER_FLOOR, cube_coeff=-0.75,
+           mode=GATHER_NORMAL, batch_dims=0, out_of_bounds_mode=OOB_EDGE_PADDED_INPUT):
+    """Shape rule pmlc/ast/ast_ops.cc:88-178."""
+    x, y = _literal(x), _literal(y)
+    rank = len(x.shape)
+    if rank == 0:
+        raise ValueError("'gather' requires first operand to have at least one dimension.")
+    if axis < 0:
+        axis += rank
+    if not 0 <= axis < rank:
+        raise ValueError("'gather' primitive expects the 'axis' argument to be a positive integer that is less than the tensor rank.")
+    if mode == GATHER_NORMAL:
+        shape = list(x.shape[:axis]) + list(y.shape) + list(x.shape[axis + 1:])
+    else:
+        if is_float(y.dt):
+            raise ValueError("'gather' ND mode requires indices elements to be integers.")
+        shape = list(y.shape[:-1]) + list(x.shape[y.shape[-1] + batch_dims:])
+    attrs = {'fn': 'gather', 'axis': int(axis), 'interp': int(interpolation_mode), 'nearest': int(nearest_mode),
+             'cube_coeff': float(cube_coeff), 'mode': int(mode), 'batch_dims': int(batch_dims), 'oob': int(out_of_bounds_mode)}
+    return Tensor('special', x.dt, shape, (x, y), attrs)
+
+
+def scatter(x, y, z, axis=0, mode=SCATTER_NORMAL):
+    """Shape rule pmlc/ast/ast_ops.cc:219-257: the data's shape and type; indices si32 / ui32."""
+    x, y, z = _literal(x), _literal(y), _literal(z)
+    if len(x.shape) == 0:
+        raise ValueError("'scatter' requires operand #1 to have at least one dimension.")
+    if y.dt not in (DType.INT32, DType.UINT32):
+        raise ValueError("'scatter' requires operand #2 to be an integer.")
+    if axis < 0:
+        axis += len(x.shape)
+    if axis >= len(x.shape):
+        raise ValueError("'scatter' primitive expects the 'axis' argument to be a positive integer that is less than the "
+                         "updates tensor rank.")
+    return Tensor('special', x.dt, x.shape, (x, y, z), {'fn': 'scatter', 'axis': int(axis), 'mode': int(mode)})
+
+
+def _eval_argsort(x, axis, direction):
+    """ArgSortOpConversion, pmlc/conversion/linalg_to_pxa/tile_to_pxa_special_patterns.cc:29-298: a stable
+    selection sort of the positions with strict ordered compares (`<` ascending, `>` descending), so equal
+    elements keep their input order in both directions."""
+    if axis < 0:
+        axis += x.ndim
+    if direction == SORT_ASC:
+        return np.argsort(x, axis=axis, kind='stable').astype(np.int32)
+    # stable descending: sort the mirrored line ascending-stably from the right
+    n = x.shape[axis]
+    flipped = np.flip(x, axis)
+    order = np.argsort(flipped, axis=axis, kind='stable')       # ascending, ties by larger original position first...
+    order = np.flip(n - 1 - order, axis)                        # ... mirrored back: descending, ties by smaller position
+    return order.astype(np.int32)
+
+
+def _eval_gather(x, y, a, dt, idt):
+    """GatherOpConversion, tile_to_pxa_special_patterns.cc:300-760.  Interpolation arithmetic runs in the tensor's
+    element type, one rounding per operation."""
+    axis, mode = a['axis'], a['mode']
+    if mode == GATHER_ND:
+        bd = a['batch_dims']
+        depth = y.shape[-1]
+        out = np.empty(tuple(y.shape[:-1]) + tuple(x.shape[bd + depth:]), x.dtype)
+        for lead in np.ndindex(*y.shape[:-1]):
+            src = tuple(lead[:bd]) + tuple(int(v) for v in y[lead])
+            out[lead] = x[src]
+        return out
+    out_shape = tuple(x.shape[:axis]) + tuple(y.shape) + tuple(x.shape[axis + 1:])
+    xm = np.moveaxis(x, axis, 0)                                  # [axis, before.., after..]
+    upper = x.shape[axis] - 1
+    if not is_float(idt):
+        res = xm[np.asarray(y, np.int64)]                         # [idx.., before.., after..]
+    elif not is_float(dt):
+        res = xm[np.trunc(y).astype(np.int64)]                    # fptosi, then a plain read
+    else:
+        ft = np.float64 if x.dtype == np.float64 else np.float32
+        rnd = lambda v: _store(np.asarray(v, ft), dt).astype(ft)  # noqa: E731
+        pos = np.asarray(y, ft)
+        fl, ce = np.floor(pos), np.ceil(pos)
+
+        def tap(i):
+            return xm[np.clip(i.astype(np.int64), 0, upper)].astype(ft)
+
+        def bc(v):                                                # weights broadcast over the non-axis dims
+            return v.reshape(v.shape + (1,) * (xm.ndim - 1))
+        interp = a['interp']
+        if interp == INTERP_NEAREST:
+            half = pos == rnd(fl + ft(0.5))
+            rounded = np.floor(rnd(pos + ft(0.5)))
+            nm = a['nearest']
+            if nm == NEAREST_ROUND_PREFER_FLOOR:
+                i = np.where(half, fl, rounded)
+            elif nm == NEAREST_ROUND_PREFER_CEIL:
+                i = np.where(half, ce, rounded)
+            elif nm == NEAREST_FLOOR:
+                i = fl
+            elif nm == NEAREST_CEIL:
+                i = ce
+            elif nm == NEAREST_SIMPLE:
+                i = np.trunc(pos)
+            else:
+                raise ValueError('Unsupported NearestMode')
+            res = tap(i)
+        elif interp == INTERP_LINEAR:
+            g0, g1 = tap(ce), tap(fl)
+            c0 = rnd(pos - fl)
+            c1 = rnd(ft(1) - c0)
+            res = rnd(rnd(bc(c0) * g0) + rnd(bc(c1) * g1))
+        elif interp == INTERP_CUBIC:
+            aa = rnd(ft(a['cube_coeff']))
+            g = [tap(fl - 1), tap(fl), tap(ce), tap(ce + 1)]
+            s1 = rnd(pos - fl)
+            s2 = rnd(s1 * s1)
+            s3 = rnd(s2 * s1)
+            s_a, s2_a, s3_a = rnd(aa * s1), rnd(aa * s2), rnd(aa * s3)
+            s3_a2 = rnd(rnd(aa + ft(2)) * s3)
+            s2_a3 = rnd(rnd(aa + ft(3)) * s2)
+            s2_2a3 = rnd(rnd(rnd(aa + aa) + ft(3)) * s2)
+            p = [rnd(rnd(s3_a - rnd(s2_a * ft(2))) + s_a), rnd(rnd(s3_a2 - s2_a3) + ft(1)), rnd(rnd(s2_2a3 - s3_a2) - s_a),
+                 rnd(s2_a - s3_a)]
+            p = [rnd(bc(pi) * gi) for pi, gi in zip(p, g)]
+            res = rnd(rnd(rnd(p[0] + p[1]) + p[2]) + p[3])
+        else:
+            raise ValueError('floating-point indices need an interpolation mode')
+        if a['oob'] == OOB_RETURN_ZERO:
+            res = np.where(bc((pos > upper) | (pos < 0)), ft(0), res)
+        res = _store(res, dt)
+    # res is [idx dims.., before.., after..] -> [before.., idx dims.., after..]
+    ni, nb = y.ndim, axis
+    perm = list(range(ni, ni + nb)) + list(range(ni)) + list(range(ni + nb, res.ndim))
+    return np.ascontiguousarray(np.transpose(res, perm)).reshape(out_shape)
+
+
+def _eval_scatter(x, y, z, a, dt):
+    """ScatterOpConversion, tile_to_pxa_special_patterns.cc:762-896: copy the data, then visit every update element;
+    NORMAL adds, the UPDATE modes assign."""
+    out = np.array(x, copy=True)
+    axis, mode = a['axis'], a['mode']
+    yi = np.asarray(y, np.int64)
+    for c in np.ndindex(*z.shape):
+        if mode == SCATTER_UPDATE_ND:
+            lead = yi.ndim - 1
+            dst = tuple(int(v) for v in yi[c[:lead]]) + tuple(c[lead:])
+        elif mode == SCATTER_UPDATE_SLICE:
+            dst = tuple(c[:axis]) + (int(yi[c[axis:axis + yi.ndim]]),) + tuple(c[axis + yi.ndim:])
+        else:
+            dst = tuple(c[:axis]) + (int(yi[c[:yi.ndim]]),) + tuple(c[axis + 1:])
+        if mode == SCATTER_NORMAL:
+            out[dst] = _store(np.asarray(out[dst] + z[c]), dt)
+        else:
+            out[dst] = z[c]
+    return out
+
+
 def abs(x):  # noqa: A001
     return select(x < 0., -x, x)
 
@@ -994,6 +1163,16 @@ def evaluate(outputs, feeds):
             v = np.broadcast_to(np.arange(n.shape[ax], dtype=np.int32).reshape(shp), n.shape).copy()
         elif k == 'reshape':
             v = ev(n.args[0]).reshape(n.shape)
+        elif k == 'special':
+            fn = n.attrs['fn']
+            vals = [np.asarray(ev(a)) for a in n.args]
+            if fn == 'argsort':
+                v = _eval_argsort(vals[0], n.attrs['axis'], n.attrs['direction'])
+            elif fn == 'gather':
+                v = _eval_gather(vals[0], vals[1], n.attrs, n.args[0].dt, n.args[1].dt)
+            else:
+                v = _eval_scatter(vals[0], vals[1], vals[2], n.attrs, n.dt)
+            v = np.asarray(v).reshape(n.shape)
         elif k == 'eltwise':
             vals, dts = [], []
             # literal operands adopt the promoted dtype of the tensor operands

@@ -100,6 +100,12 @@ hipError_t select_launch(const pml_hip_select_desc& d, const void* c, const void
 hipError_t index_launch(void* out, int rank, const int64_t* sizes, int axis, hipStream_t s);
 hipError_t fill_u32_launch(void* p, uint32_t pattern, size_t n_words, hipStream_t s);
 
+// special operations (special.hip)
+hipError_t gather_launch(const pml_hip_gather_desc& d, const void* tensor, const void* indices, void* out, hipStream_t s);
+hipError_t scatter_launch(const pml_hip_scatter_desc& d, const void* data, const void* indices, const void* updates, void* out,
+                          hipStream_t s);
+hipError_t argsort_launch(const pml_hip_argsort_desc& d, const void* tensor, void* out, hipStream_t s);
+
 // window kernels (window.hip)
 struct DwconvArgs {
   pml_hip_dwconv2d_desc d;

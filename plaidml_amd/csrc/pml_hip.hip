@@ -890,6 +890,108 @@ int pml_hip_index(void* out, int32_t rank, const int64_t* sizes, int32_t axis, p
 }
 
 // ---------------------------------------------------------------------------
+// special operations
+// ---------------------------------------------------------------------------
+
+namespace {
+bool sizes_ok(const int64_t* sizes, int rank) {
+  for (int i = 0; i < rank; ++i)
+    if (sizes[i] < 0) return false;
+  return true;
+}
+int64_t count_of(const int64_t* sizes, int rank) {
+  int64_t n = 1;
+  for (int i = 0; i < rank; ++i) n *= sizes[i];
+  return n;
+}
+}  // namespace
+
+int pml_hip_gather(const pml_hip_gather_desc* d, const void* tensor, const void* indices, void* out, pml_hip_stream s) {
+  if (!d || !tensor || !indices || !out) return fail("gather: null argument");
+  if (d->rank < 1 || d->rank > PML_HIP_MAX_SPECIAL_RANK || d->idx_rank < 0 || d->idx_rank > PML_HIP_MAX_SPECIAL_RANK)
+    return fail("gather: rank out of range");
+  if (!sizes_ok(d->sizes, d->rank) || !sizes_ok(d->idx_sizes, d->idx_rank)) return fail("gather: negative size");
+  if (dt_size(d->dtype) == 0 || dt_size(d->idx_dtype) == 0) return fail("gather: bad element type");
+  if (d->mode == PML_HIP_GATHER_NORMAL) {
+    if (d->axis < 0 || d->axis >= d->rank) return fail("gather: axis out of range");
+    if (d->rank - 1 + d->idx_rank > PML_HIP_MAX_SPECIAL_RANK) return fail("gather: result rank out of range");
+    if (dt_is_float(d->idx_dtype) && dt_is_float(d->dtype)) {
+      if (d->interpolation < PML_HIP_INTERP_NEAREST || d->interpolation > PML_HIP_INTERP_CUBIC)
+        return fail("gather: floating indices need an interpolation mode");
+      if (d->interpolation == PML_HIP_INTERP_NEAREST && (d->nearest < 0 || d->nearest > PML_HIP_NEAREST_SIMPLE))
+        return fail("gather: bad nearest mode");
+      if (d->oob != PML_HIP_OOB_EDGE_PADDED_INPUT && d->oob != PML_HIP_OOB_RETURN_ZERO) return fail("gather: bad out-of-bounds mode");
+    }
+  } else if (d->mode == PML_HIP_GATHER_ND) {
+    if (dt_is_float(d->idx_dtype)) return fail("gather: ND mode needs integer indices");
+    if (d->idx_rank < 1) return fail("gather: ND mode needs indices of rank >= 1");
+    const int64_t k = d->idx_sizes[d->idx_rank - 1];
+    if (d->batch_dims < 0 || d->batch_dims > d->idx_rank - 1 || d->batch_dims + k > d->rank)
+      return fail("gather: ND index depth out of range");
+    if (d->idx_rank - 1 + d->rank - d->batch_dims - k > PML_HIP_MAX_SPECIAL_RANK) return fail("gather: result rank out of range");
+    for (int i = 0; i < d->batch_dims; ++i)
+      if (d->sizes[i] != d->idx_sizes[i]) return fail("gather: batch dimensions differ");
+  } else {
+    return fail("gather: bad mode");
+  }
+  return check(gather_launch(*d, tensor, indices, out, (hipStream_t)s), "gather_launch");
+}
+
+int pml_hip_scatter(const pml_hip_scatter_desc* d, const void* data, const void* indices, const void* updates, void* out,
+                    pml_hip_stream s) {
+  if (!d || !data || !indices || !updates || !out) return fail("scatter: null argument");
+  if (out == data) return fail("scatter: the result must not alias the data");
+  if (d->rank < 1 || d->rank > PML_HIP_MAX_SPECIAL_RANK || d->idx_rank < 1 || d->idx_rank > PML_HIP_MAX_SPECIAL_RANK ||
+      d->upd_rank < 1 || d->upd_rank > PML_HIP_MAX_SPECIAL_RANK)
+    return fail("scatter: rank out of range");
+  if (!sizes_ok(d->sizes, d->rank) || !sizes_ok(d->idx_sizes, d->idx_rank) || !sizes_ok(d->upd_sizes, d->upd_rank))
+    return fail("scatter: negative size");
+  if (d->idx_dtype != PML_HIP_I32 && d->idx_dtype != PML_HIP_U32) return fail("scatter: indices must be si32 or ui32");
+  if (dt_size(d->dtype) == 0) return fail("scatter: bad element type");
+  if (d->axis < 0 || d->axis >= d->rank) return fail("scatter: axis out of range");
+  // every update element must name a full coordinate of the result
+  int dst_rank = 0;
+  switch (d->mode) {
+    case PML_HIP_SCATTER_UPDATE_ND: {
+      const int64_t k = d->idx_sizes[d->idx_rank - 1];
+      if (d->upd_rank < d->idx_rank - 1) return fail("scatter: updates have too few dimensions");
+      dst_rank = (int)k + d->upd_rank - (d->idx_rank - 1);
+      for (int i = 0; i + 1 < d->idx_rank; ++i)
+        if (d->upd_sizes[i] != d->idx_sizes[i]) return fail("scatter: updates and indices disagree");
+      break;
+    }
+    case PML_HIP_SCATTER_UPDATE_SLICE:
+      if (d->upd_rank < d->axis + d->idx_rank) return fail("scatter: updates have too few dimensions");
+      dst_rank = d->upd_rank - d->idx_rank + 1;
+      for (int i = 0; i < d->idx_rank; ++i)
+        if (d->upd_sizes[d->axis + i] != d->idx_sizes[i]) return fail("scatter: updates and indices disagree");
+      break;
+    case PML_HIP_SCATTER_NORMAL:
+    case PML_HIP_SCATTER_UPDATE_ELT:
+      if (d->upd_rank < d->idx_rank) return fail("scatter: updates have too few dimensions");
+      dst_rank = d->upd_rank;
+      for (int i = 0; i < d->idx_rank; ++i)
+        if (d->upd_sizes[i] != d->idx_sizes[i]) return fail("scatter: updates and indices disagree");
+      break;
+    default: return fail("scatter: bad mode");
+  }
+  if (dst_rank != d->rank) return fail("scatter: updates do not address the result's rank");
+  return check(scatter_launch(*d, data, indices, updates, out, (hipStream_t)s), "scatter_launch");
+}
+
+int pml_hip_argsort(const pml_hip_argsort_desc* d, const void* tensor, void* out, pml_hip_stream s) {
+  if (!d || !tensor || !out) return fail("argsort: null argument");
+  if (d->rank < 1 || d->rank > PML_HIP_MAX_SPECIAL_RANK) return fail("argsort: rank out of range");
+  if (!sizes_ok(d->sizes, d->rank)) return fail("argsort: negative size");
+  if (d->axis < 0 || d->axis >= d->rank) return fail("argsort: axis out of range");
+  if (d->direction != 0 && d->direction != 1) return fail("argsort: bad direction");
+  if (dt_size(d->dtype) == 0 || d->dtype == PML_HIP_BOOL) return fail("argsort: bad element type");
+  if (d->sizes[d->axis] > INT32_MAX) return fail("argsort: axis too long for si32 positions");
+  if (count_of(d->sizes, d->rank) == 0) return 0;
+  return check(argsort_launch(*d, tensor, out, (hipStream_t)s), "argsort_launch");
+}
+
+// ---------------------------------------------------------------------------
 // any contraction
 // ---------------------------------------------------------------------------
 
@@ -959,6 +1061,9 @@ size_t pml_hip_struct_size(int which) {
     case 6: return sizeof(pml_hip_select_desc);
     case 7: return sizeof(pml_hip_contract_desc);
     case 8: return sizeof(pml_hip_form);
+    case 9: return sizeof(pml_hip_gather_desc);
+    case 10: return sizeof(pml_hip_scatter_desc);
+    case 11: return sizeof(pml_hip_argsort_desc);
   }
   return 0;
 }

@@ -727,6 +727,49 @@ def abs(x):  # noqa: A001
     return select(x < 0.0, -x, x)
 
 
+# ---- special operations (plaidml/edsl/edsl.h:800-811, 1034-1066, 1625-1765) ----------------------------------
+SORT_ASC, SORT_DESC = range(2)
+INTERP_NEAREST, INTERP_LINEAR, INTERP_CUBIC, INTERP_NONE = range(4)
+NEAREST_ROUND_PREFER_FLOOR, NEAREST_ROUND_PREFER_CEIL, NEAREST_FLOOR, NEAREST_CEIL, NEAREST_SIMPLE, NEAREST_NONE = range(6)
+GATHER_NORMAL, GATHER_ND = range(2)
+OOB_EDGE_PADDED_INPUT, OOB_RETURN_ZERO = range(2)
+SCATTER_NORMAL, SCATTER_UPDATE_SLICE, SCATTER_UPDATE_ELT, SCATTER_UPDATE_ND = range(4)
+
+
+def _const(ptr):
+    return Tensor(ptr=ptr)
+
+
+def _uint(v):
+    return _const(call('plaidml_expr_uint', int(v)))
+
+
+def _int(v):
+    return _const(call('plaidml_expr_int', int(v)))
+
+
+def _float(v):
+    return _const(call('plaidml_expr_float', float(v)))
+
+
+def argsort(x, axis=-1, direction=SORT_ASC):
+    return intrinsic('argsort', x, _int(axis), _int(direction))
+
+
+def gather(x, y, axis=0, interpolation_mode=INTERP_NONE, nearest_mode=NEAREST_ROUND_PREFER_FLOOR, cube_coeff=-0.75,
+           mode=GATHER_NORMAL, batch_dims=0, out_of_bounds_mode=OOB_EDGE_PADDED_INPUT):
+    if axis < 0:
+        axis += x.rank
+    return intrinsic('gather', x, y, _uint(axis), _uint(interpolation_mode), _uint(nearest_mode), _float(cube_coeff), _uint(mode),
+                     _uint(batch_dims), _uint(out_of_bounds_mode))
+
+
+def scatter(x, y, z, axis=0, mode=SCATTER_NORMAL):
+    if axis < 0:
+        axis += x.rank
+    return intrinsic('scatter', x, y, z, _int(axis), _uint(mode))
+
+
 # ---- values (arguments of the operation library) ------------------------------------------------------
 
 class Value(_Handle):

@@ -32,6 +32,7 @@ EXPORTS = [
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
     'pml_hip_plan_describe', 'pml_hip_struct_size', 'pml_hip_gemm_pack_b', 'pml_hip_conv2d_pack_filter',
+    'pml_hip_gather', 'pml_hip_scatter', 'pml_hip_argsort',
 ]
 
 i32, i64, f64 = ctypes.c_int32, ctypes.c_int64, ctypes.c_double
@@ -96,6 +97,25 @@ class ContractDesc(ctypes.Structure):
                 ('identity_i', i64), ('forms', Form * MAX_FORMS)]
 
 
+MAX_SPECIAL_RANK = 8
+
+
+class GatherDesc(ctypes.Structure):
+    _fields_ = [('dtype', i32), ('idx_dtype', i32), ('mode', i32), ('interpolation', i32), ('nearest', i32), ('oob', i32),
+                ('axis', i32), ('batch_dims', i32), ('rank', i32), ('idx_rank', i32), ('cube_coeff', f64),
+                ('sizes', i64 * MAX_SPECIAL_RANK), ('idx_sizes', i64 * MAX_SPECIAL_RANK)]
+
+
+class ScatterDesc(ctypes.Structure):
+    _fields_ = [('dtype', i32), ('idx_dtype', i32), ('mode', i32), ('axis', i32), ('rank', i32), ('idx_rank', i32),
+                ('upd_rank', i32), ('reserved', i32), ('sizes', i64 * MAX_SPECIAL_RANK), ('idx_sizes', i64 * MAX_SPECIAL_RANK),
+                ('upd_sizes', i64 * MAX_SPECIAL_RANK)]
+
+
+class ArgsortDesc(ctypes.Structure):
+    _fields_ = [('dtype', i32), ('rank', i32), ('axis', i32), ('direction', i32), ('sizes', i64 * MAX_SPECIAL_RANK)]
+
+
 _lib = None
 
 
@@ -136,6 +156,9 @@ def lib():
         L.pml_hip_plan_describe.argtypes = [ctypes.c_int64, ctypes.c_char_p, sz]
         L.pml_hip_struct_size.restype = sz
         L.pml_hip_gemm_pack_b.argtypes = [ctypes.c_int64, vp, vp]
+        L.pml_hip_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp]
+        L.pml_hip_scatter.argtypes = [ctypes.POINTER(ScatterDesc), vp, vp, vp, vp, vp]
+        L.pml_hip_argsort.argtypes = [ctypes.POINTER(ArgsortDesc), vp, vp, vp]
         L.pml_hip_conv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
         _lib = L
     return _lib

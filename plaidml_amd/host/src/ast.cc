@@ -91,7 +91,8 @@ bool isKnownIntrinsic(const std::string& fn) {
       "abs",     "add",     "sub",     "mul",      "div",      "mod",     "neg",     "ident",   "relu",   "exp",
       "log",     "sqrt",    "tanh",    "floor",    "ceil",     "round",   "pow",     "sin",     "cos",    "tan",
       "sinh",    "cosh",    "erf",     "select",   "index",    "reshape", "shape",   "bit_and", "bit_or", "bit_xor",
-      "bit_not", "bit_shl", "bit_shr", "acos",     "asin",     "atan",    "acosh",   "asinh",   "atanh"};
+      "bit_not", "bit_shl", "bit_shr", "acos",     "asin",     "atan",    "acosh",   "asinh",   "atanh",
+      "gather",  "scatter", "argsort"};
   return s.count(fn) != 0 || isCompareOp(fn) || isLogicalOp(fn);
 }
 
@@ -251,6 +252,64 @@ TensorShape Evaluator::computeShape(const ExprNodePtr& node) {
           ret.sizes.push_back(v);
         }
         return ret;
+      }
+      // the special operations: pmlc/ast/ast_ops.cc:41-60 (argsort), :88-178 (gather), :219-257 (scatter)
+      if (fn == "argsort") {
+        if (node->operands.size() != 3) throw std::runtime_error("'argsort' requires 3 arguments.");
+        int64_t v;
+        if (!integerOperand(this, node->operands[1], &v)) throw std::runtime_error("'argsort' requires operand #2 to be an integer.");
+        if (!integerOperand(this, node->operands[2], &v)) throw std::runtime_error("'argsort' requires operand #3 to be an integer.");
+        return TensorShape(DataType::si32, shapes[0].sizes);
+      }
+      if (fn == "gather") {
+        if (node->operands.size() != 9) throw std::runtime_error("'gather' requires nine arguments.");
+        const TensorShape& tensor = shapes[0];
+        const TensorShape& idxs = shapes[1];
+        const int64_t rank = static_cast<int64_t>(tensor.getRank());
+        if (!rank) throw std::runtime_error("'gather' requires first operand to have at least one dimension.");
+        int64_t axis, interp, nearest, mode, batch_dims, oob;
+        if (!integerOperand(this, node->operands[2], &axis) || axis >= rank || axis < 0)
+          throw std::runtime_error(
+              "'gather' primitive expects the 'axis' argument to be a positive integer that is less than the tensor rank.");
+        if (!integerOperand(this, node->operands[3], &interp))
+          throw std::runtime_error("'gather' primitive expects the 'interpolationMode' argument to be a constant integer");
+        if (!integerOperand(this, node->operands[4], &nearest))
+          throw std::runtime_error("'gather' primitive expects the 'nearestMode' argument to be a constant integer");
+        if (node->operands[5]->kind != ExprNode::ConstFloat)
+          throw std::runtime_error("'gather' primitive expects the 'cubeCoeff' argument to be a constant float");
+        if (!integerOperand(this, node->operands[6], &mode))
+          throw std::runtime_error("'gather' primitive expects the 'mode' argument to be a constant integer");
+        if (mode == 1 && !util::isInteger(idxs.elementType))
+          throw std::runtime_error("'gather' ND mode requires indices elements to be integers.");
+        if (!integerOperand(this, node->operands[7], &batch_dims))
+          throw std::runtime_error("'gather' primitive expects the 'batchDims' argument to be a constant integer");
+        if (!integerOperand(this, node->operands[8], &oob))
+          throw std::runtime_error("'gather' primitive expects the 'outOfBoundsMode' argument to be a constant integer");
+        TensorShape shape(tensor.elementType);
+        if (mode == 0) {
+          for (int64_t i = 0; i < axis; ++i) shape.sizes.push_back(tensor.sizes[i]);
+          shape.sizes.insert(shape.sizes.end(), idxs.sizes.begin(), idxs.sizes.end());
+          for (int64_t i = axis + 1; i < rank; ++i) shape.sizes.push_back(tensor.sizes[i]);
+        } else {
+          if (idxs.getRank() == 0) throw std::runtime_error("'gather' ND mode requires indices of at least one dimension.");
+          for (size_t i = 0; i + 1 < idxs.getRank(); ++i) shape.sizes.push_back(idxs.sizes[i]);
+          for (int64_t i = idxs.sizes.back() + batch_dims; i < rank; ++i) shape.sizes.push_back(tensor.sizes[i]);
+        }
+        return shape;
+      }
+      if (fn == "scatter") {
+        if (node->operands.size() != 5) throw std::runtime_error("'scatter' requires 5 operands.");
+        const int64_t rank = static_cast<int64_t>(shapes[0].getRank());
+        if (!rank) throw std::runtime_error("'scatter' requires operand #1 to have at least one dimension.");
+        if (shapes[1].elementType != DataType::si32 && shapes[1].elementType != DataType::ui32)
+          throw std::runtime_error("'scatter' requires operand #2 to be an integer.");
+        int64_t axis, mode;
+        if (!integerOperand(this, node->operands[3], &axis) || axis >= rank)
+          throw std::runtime_error(
+              "'scatter' primitive expects the 'axis' argument to be a positive integer that is less than the updates tensor rank.");
+        if (!integerOperand(this, node->operands[4], &mode))
+          throw std::runtime_error("'scatter' primitive expects the 'mode' argument to be a constant integer.");
+        return TensorShape(shapes[0].elementType, shapes[0].sizes);
       }
       if (fn == "shape") {
         if (node->operands.size() != 1) throw std::runtime_error("'shape' requires exactly one argument.");

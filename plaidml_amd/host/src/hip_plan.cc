@@ -606,6 +606,7 @@ class Planner {
         plan_->steps.push_back(s);
         break;
       }
+      case Op::Special: emitSpecial(i); break;
       case Op::Reshape: {
         Step s;
         s.kind = Step::Copy;
@@ -617,6 +618,74 @@ class Planner {
         break;
       }
     }
+  }
+
+  // gather / scatter / argsort: one launch each, operands and constants passed through
+  void emitSpecial(size_t i) {
+    const Op& op = prog_->ops[i];
+    auto fill = [](const TensorShape& sh, int64_t* sizes, int32_t* rank, const char* what) {
+      if (sh.getRank() > PML_HIP_MAX_SPECIAL_RANK)
+        throw std::runtime_error(std::string("'") + what + "' operands of rank > 8 are not supported by the hip target");
+      *rank = static_cast<int32_t>(sh.getRank());
+      for (size_t d = 0; d < sh.getRank(); ++d) sizes[d] = sh.sizes[d];
+    };
+    auto param = [&](size_t k) { return static_cast<int64_t>(op.params.at(k)); };
+    Step s;
+    s.c = bufferFor(op.result);
+    for (const ValuePtr& v : op.operands) s.operands.push_back(bufferFor(v));
+    if (op.fn == "gather") {
+      s.kind = Step::Gather;
+      auto& d = s.gat;
+      d.dtype = hipType(op.operands[0]->shape.elementType);
+      d.idx_dtype = hipType(op.operands[1]->shape.elementType);
+      fill(op.operands[0]->shape, d.sizes, &d.rank, "gather");
+      fill(op.operands[1]->shape, d.idx_sizes, &d.idx_rank, "gather");
+      d.axis = static_cast<int32_t>(param(0));
+      d.interpolation = static_cast<int32_t>(param(1));
+      d.nearest = static_cast<int32_t>(param(2));
+      d.cube_coeff = op.params.at(3);
+      d.mode = static_cast<int32_t>(param(4));
+      d.batch_dims = static_cast<int32_t>(param(5));
+      d.oob = static_cast<int32_t>(param(6));
+      if (op.result->shape.getRank() > PML_HIP_MAX_SPECIAL_RANK)
+        throw std::runtime_error("'gather' results of rank > 8 are not supported by the hip target");
+      if (d.mode == PML_HIP_GATHER_NORMAL && util::isFloat(op.operands[1]->shape.elementType) &&
+          util::isFloat(op.operands[0]->shape.elementType) && d.interpolation == PML_HIP_INTERP_NONE)
+        throw std::runtime_error("'gather' with floating-point indices needs an interpolation mode");
+      s.text = std::string("gather ") + (d.mode == PML_HIP_GATHER_ND ? "nd batch_dims=" + std::to_string(d.batch_dims)
+                                                                     : "axis=" + std::to_string(d.axis)) +
+               " -> " + op.result->shape.str();
+      s.bytes = static_cast<double>(op.result->shape.getByteSize()) * 2 + static_cast<double>(op.operands[1]->shape.getByteSize());
+    } else if (op.fn == "scatter") {
+      s.kind = Step::Scatter;
+      auto& d = s.sca;
+      d.dtype = hipType(op.operands[0]->shape.elementType);
+      d.idx_dtype = hipType(op.operands[1]->shape.elementType);
+      if (op.operands[2]->shape.elementType != op.operands[0]->shape.elementType)
+        throw std::runtime_error("'scatter' needs updates of the data's element type, use a cast");
+      fill(op.operands[0]->shape, d.sizes, &d.rank, "scatter");
+      fill(op.operands[1]->shape, d.idx_sizes, &d.idx_rank, "scatter");
+      fill(op.operands[2]->shape, d.upd_sizes, &d.upd_rank, "scatter");
+      d.axis = static_cast<int32_t>(param(0));
+      d.mode = static_cast<int32_t>(param(1));
+      static const char* modes[] = {"normal", "update_slice", "update_elt", "update_nd"};
+      s.text = std::string("scatter ") + (d.mode >= 0 && d.mode < 4 ? modes[d.mode] : "?") + " axis=" + std::to_string(d.axis) +
+               " -> " + op.result->shape.str();
+      s.bytes = static_cast<double>(op.result->shape.getByteSize()) * 2 + static_cast<double>(op.operands[2]->shape.getByteSize()) * 2;
+    } else {
+      s.kind = Step::ArgSort;
+      auto& d = s.srt;
+      d.dtype = hipType(op.operands[0]->shape.elementType);
+      fill(op.operands[0]->shape, d.sizes, &d.rank, "argsort");
+      int64_t axis = param(0);
+      if (axis < 0) axis += d.rank;
+      if (axis < 0 || axis >= d.rank) throw std::runtime_error("'argsort' axis out of range");
+      d.axis = static_cast<int32_t>(axis);
+      d.direction = static_cast<int32_t>(param(1));
+      s.text = std::string("argsort axis=") + std::to_string(d.axis) + (d.direction ? " desc" : " asc") + " -> " + op.result->shape.str();
+      s.bytes = static_cast<double>(op.result->shape.getByteSize()) + static_cast<double>(op.operands[0]->shape.getByteSize());
+    }
+    plan_->steps.push_back(s);
   }
 
   void emitEltwise(size_t i) {

@@ -26,7 +26,7 @@ struct BufferInfo {
 };
 
 struct Step {
-  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy } kind = Copy;
+  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy, Gather, Scatter, ArgSort } kind = Copy;
   std::string text;  // one line for the plan dump
   // descriptors (only the one matching `kind` is meaningful)
   pml_hip_gemm_desc gemm{};
@@ -36,6 +36,9 @@ struct Step {
   pml_hip_eltwise_desc elt{};
   pml_hip_select_desc sel{};
   pml_hip_contract_desc con{};
+  pml_hip_gather_desc gat{};
+  pml_hip_scatter_desc sca{};
+  pml_hip_argsort_desc srt{};
   int index_axis = 0;
   std::vector<int64_t> index_sizes;
   // buffer ids (-1 = none) and element offsets applied to the base pointers

@@ -126,6 +126,9 @@ class HipExecutable final : public Executable {
       case Step::Contract: h = pml_hip_contract_dispatch(&s.con); break;
       case Step::Select:
       case Step::Index:
+      case Step::Gather:
+      case Step::Scatter:
+      case Step::ArgSort:
       case Step::Copy: return;
     }
     if (!h) throw std::runtime_error("hip dispatch failed for '" + s.text + "': " + pml_hip_last_error());
@@ -178,6 +181,15 @@ class HipExecutable final : public Executable {
         break;
       case Step::Copy:
         hipCheck(pml_hip_memcpy_d2d(ptr(s.c), ptr(s.a), s.copy_bytes, nullptr), s.text.c_str());
+        break;
+      case Step::Gather:
+        hipCheck(pml_hip_gather(&s.gat, operands[0], operands[1], ptr(s.c), nullptr), s.text.c_str());
+        break;
+      case Step::Scatter:
+        hipCheck(pml_hip_scatter(&s.sca, operands[0], operands[1], operands[2], ptr(s.c), nullptr), s.text.c_str());
+        break;
+      case Step::ArgSort:
+        hipCheck(pml_hip_argsort(&s.srt, operands[0], ptr(s.c), nullptr), s.text.c_str());
         break;
     }
   }

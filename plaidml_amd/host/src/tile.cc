@@ -310,6 +310,27 @@ struct Builder {
           op.operands = {src};
         } else if (node->op == "shape") {
           throw std::runtime_error("'shape' is not supported by this backend");
+        } else if (node->op == "gather" || node->op == "scatter" || node->op == "argsort") {
+          // tensor operands first, then constants (plaidml/edsl/edsl.h:809-811, 1036-1066, 1645-1690)
+          op.kind = Op::Special;
+          op.fn = node->op;
+          const size_t n_tensors = node->op == "gather" ? 2 : (node->op == "scatter" ? 3 : 1);
+          for (size_t k = 0; k < node->operands.size(); ++k) {
+            const ExprNodePtr& o = node->operands[k];
+            if (k < n_tensors) {
+              ValuePtr v = visit(o);
+              if (v->kind == Value::Literal) v = materialiseLiteral(v, materialise(v->shape.elementType));
+              op.operands.push_back(v);
+              continue;
+            }
+            switch (o->kind) {
+              case ExprNode::ConstSigned: op.params.push_back(static_cast<double>(o->ivalue)); break;
+              case ExprNode::ConstUnsigned: op.params.push_back(static_cast<double>(o->uvalue)); break;
+              case ExprNode::ConstFloat: op.params.push_back(o->fvalue); break;
+              case ExprNode::Dim: op.params.push_back(static_cast<double>(ev.evaluate(o->dimNode))); break;
+              default: throw std::runtime_error("'" + node->op + "' expects constant arguments after its tensors");
+            }
+          }
         } else {
           op.kind = Op::Eltwise;
           op.fn = node->op;
@@ -559,6 +580,13 @@ std::string Program::str() const {
         break;
       case Op::Reshape:
         ss << "tile.reshape " << valueRef(op.operands[0]);
+        break;
+      case Op::Special:
+        ss << "tile." << op.fn;
+        for (size_t i = 0; i < op.operands.size(); ++i) ss << (i ? ", " : " ") << valueRef(op.operands[i]);
+        ss << " {";
+        for (size_t i = 0; i < op.params.size(); ++i) ss << (i ? ", " : "") << op.params[i];
+        ss << "}";
         break;
     }
     ss << " : tensor<" << op.result->shape.str() << ">\n";

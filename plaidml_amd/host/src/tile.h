@@ -68,7 +68,7 @@ struct ConstraintForm {
 };
 
 struct Op {
-  enum Kind { Contraction, Eltwise, Cast, Index, Reshape } kind = Eltwise;
+  enum Kind { Contraction, Eltwise, Cast, Index, Reshape, Special } kind = Eltwise;
   ValuePtr result;
   std::vector<ValuePtr> operands;
   std::string name;
@@ -76,6 +76,9 @@ struct Op {
   std::string fn;
   // Index
   int axis = 0;
+  // Special (fn = gather / scatter / argsort): the tensor operands are in `operands`, the constant arguments here
+  // in the order the intrinsic takes them
+  std::vector<double> params;
   // Contraction
   AggKind agg = AggKind::assign;
   ComboKind combo = ComboKind::none;

@@ -26,7 +26,8 @@ def test_kernel_library_exports_every_declared_symbol():
 def test_descriptor_layouts_match():
     L = hk.lib()
     for which, cls in enumerate([hk.Epilogue, hk.GemmDesc, hk.Conv2dDesc, hk.Dwconv2dDesc, hk.Pool2dDesc,
-                                 hk.EltwiseDesc, hk.SelectDesc, hk.ContractDesc, hk.Form]):
+                                 hk.EltwiseDesc, hk.SelectDesc, hk.ContractDesc, hk.Form, hk.GatherDesc, hk.ScatterDesc,
+                                 hk.ArgsortDesc]):
         assert L.pml_hip_struct_size(which) == ctypes.sizeof(cls), cls.__name__
 
 
@@ -40,3 +41,12 @@ def test_dispatch_rejects_bad_descriptors_without_a_gpu():
     c.in_dtype, c.out_dtype = hk.BF16, hk.BF16
     assert L.pml_hip_conv2d_dispatch(ctypes.byref(c)) == 0
     assert b'geometry' in L.pml_hip_last_error()
+    g = hk.GatherDesc()
+    g.rank, g.idx_rank, g.dtype, g.idx_dtype, g.axis = 1, 1, hk.F32, hk.I32, 3
+    one = ctypes.c_void_p(1)   # never dereferenced: the descriptor is rejected first
+    assert L.pml_hip_gather(ctypes.byref(g), one, one, one, None) != 0
+    assert b'axis out of range' in L.pml_hip_last_error()
+    sc = hk.ScatterDesc()
+    sc.rank, sc.idx_rank, sc.upd_rank, sc.dtype, sc.idx_dtype = 1, 1, 1, hk.F32, hk.F32
+    assert L.pml_hip_scatter(ctypes.byref(sc), one, ctypes.c_void_p(2), one, ctypes.c_void_p(3), None) != 0
+    assert b'si32 or ui32' in L.pml_hip_last_error()

@@ -1,0 +1,130 @@
+"""argsort, gather and scatter: the oracle and the hip device against the reference tests' own answers
+(tests/special_cases.py) and, on seeded inputs, against numpy closed forms and each other."""
+import numpy as np
+import pytest
+
+import special_cases as SC
+from oracle import tile_oracle as OE
+
+NAMES = sorted(SC.CASES)
+
+
+@pytest.mark.parametrize('name', NAMES)
+def test_oracle_reproduces_reference_answers(name):
+    prog, ins = SC.build_case(name, OE)
+    SC.check_case(name, OE.run(prog, ins)[0])
+
+
+def random_programs(E):
+    """Larger seeded cases: (name, program, inputs, numpy expectation or None)."""
+    r = np.random.default_rng(31)
+    out = []
+    x = r.integers(-5, 6, (7, 33, 5)).astype(np.float32)          # many ties
+    X = E.Placeholder(E.DType.FLOAT32, [7, 33, 5])
+    asc = np.argsort(x, axis=1, kind='stable').astype(np.int32)
+    desc = np.flip(32 - np.argsort(np.flip(x, 1), axis=1, kind='stable'), 1).astype(np.int32)
+    out.append(('argsort_ties', E.Program('p', [X], [E.argsort(x=X, axis=1), E.argsort(X, -2, E.SORT_DESC)]), [x], [asc, desc]))
+    u = r.integers(0, 2 ** 63, (300,), dtype=np.uint64)
+    u[7] = 2 ** 64 - 1
+    U = E.Placeholder(E.DType.UINT64, [300])
+    out.append(('argsort_u64', E.Program('p', [U], [E.argsort(U, 0, E.SORT_DESC)]), [u],
+                [np.argsort(-u.astype(np.float64), kind='stable').astype(np.int32)]))
+    t = r.standard_normal((4, 9, 6)).astype(np.float32)
+    i = r.integers(0, 9, (5, 3)).astype(np.int32)
+    T, I = E.Placeholder(E.DType.FLOAT32, [4, 9, 6]), E.Placeholder(E.DType.INT32, [5, 3])
+    out.append(('gather_axis1', E.Program('p', [T, I], [E.gather(T, I, axis=1)]), [t, i], [np.take(t, i, axis=1)]))
+    pos = r.uniform(-1.5, 9.5, (11,)).astype(np.float32)
+    P = E.Placeholder(E.DType.FLOAT32, [11])
+    lin = E.gather(T, P, axis=1, interpolation_mode=E.INTERP_LINEAR)
+    cub = E.gather(T, P, axis=1, interpolation_mode=E.INTERP_CUBIC, out_of_bounds_mode=E.OOB_RETURN_ZERO)
+    near = [E.gather(T, P, axis=1, interpolation_mode=E.INTERP_NEAREST, nearest_mode=m) for m in range(5)]
+    out.append(('gather_interpolated', E.Program('p', [T, P], [lin, cub] + near), [t, pos], None))
+    d = r.standard_normal((6, 5, 4)).astype(np.float32)
+    si = r.integers(0, 5, (3, 2)).astype(np.int32)
+    su = r.standard_normal((6, 3, 2, 4)).astype(np.float32)
+    D, SI, SU = E.Placeholder(E.DType.FLOAT32, [6, 5, 4]), E.Placeholder(E.DType.INT32, [3, 2]), E.Placeholder(E.DType.FLOAT32, [6, 3, 2, 4])
+    di = r.integers(-100, 100, (6, 5, 4)).astype(np.int32)
+    ui = r.integers(-100, 100, (3, 2, 4)).astype(np.int32)
+    ii = r.integers(0, 6, (3, 2)).astype(np.int32)
+    DI, II, UI = E.Placeholder(E.DType.INT32, [6, 5, 4]), E.Placeholder(E.DType.INT32, [3, 2]), E.Placeholder(E.DType.INT32, [3, 2, 4])
+    ref = di.copy()
+    np.add.at(ref, (ii[:, :, None], np.arange(2)[None, :, None], np.arange(4)[None, None, :]), ui)
+    out.append(('scatter_add_int_dups', E.Program('p', [DI, II, UI], [E.scatter(DI, II, UI)]), [di, ii, ui], [ref]))
+    return out, (D, SI, SU, d, si, su)
+
+
+def test_oracle_matches_numpy_on_seeded_cases():
+    progs, _ = random_programs(OE)
+    for name, prog, ins, refs in progs:
+        outs = OE.run(prog, ins)
+        if refs is not None:
+            for o, r in zip(outs, refs):
+                np.testing.assert_array_equal(o, r, err_msg=name)
+
+
+def test_oracle_linear_gather_is_piecewise_linear_interpolation():
+    """Inside the range the LINEAR mode equals numpy's interp; outside it holds the edge value (or zero)."""
+    t = np.array([0.5, -2.0, 4.0, 1.0, 3.5], np.float32)
+    pos = np.linspace(-1, 5, 25).astype(np.float32)
+    T, P = OE.Placeholder(OE.DType.FLOAT32, [5]), OE.Placeholder(OE.DType.FLOAT32, [25])
+    edge, zero = OE.run(OE.Program('p', [T, P], [OE.gather(T, P, interpolation_mode=OE.INTERP_LINEAR),
+                                                 OE.gather(T, P, interpolation_mode=OE.INTERP_LINEAR,
+                                                           out_of_bounds_mode=OE.OOB_RETURN_ZERO)]), [t, pos])
+    want = np.interp(pos, np.arange(5), t)
+    np.testing.assert_allclose(edge, want, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(zero, np.where((pos < 0) | (pos > 4), 0, want), rtol=1e-6, atol=1e-6)
+
+
+def test_oracle_cubic_gather_reproduces_cubics_exactly_at_interior_points():
+    """Keys' cubic convolution with a = -0.5 reproduces any quadratic between interior samples."""
+    k = np.arange(8, dtype=np.float64)
+    t = (0.25 * k * k - k + 2).astype(np.float64)
+    pos = np.linspace(1, 6, 21)
+    T, P = OE.Placeholder(OE.DType.FLOAT64, [8]), OE.Placeholder(OE.DType.FLOAT64, [21])
+    got, = OE.run(OE.Program('p', [T, P], [OE.gather(T, P, interpolation_mode=OE.INTERP_CUBIC, cube_coeff=-0.5)]), [t, pos])
+    np.testing.assert_allclose(got, 0.25 * pos * pos - pos + 2, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('name', NAMES)
+def test_hip_reproduces_reference_answers(name):
+    from plaidml_amd import edsl as E
+    print('special case', name, flush=True)
+    prog, ins = SC.build_case(name, E)
+    got = E.run(prog, ins, target='hip')[0]
+    SC.check_case(name, got)
+    oprog, oins = SC.build_case(name, OE)
+    ref = OE.run(oprog, oins)[0]
+    if SC.CASES[name]['tol'] is None:
+        np.testing.assert_array_equal(got, ref)
+    else:
+        np.testing.assert_allclose(got.astype(np.float64), ref.astype(np.float64), rtol=2e-3 if got.dtype == np.float16 else 1e-6,
+                                   atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_hip_matches_oracle_on_seeded_cases():
+    from plaidml_amd import edsl as E
+    progs, _ = random_programs(E)
+    oprogs, _ = random_programs(OE)
+    for (name, prog, ins, refs), (_, oprog, oins, _) in zip(progs, oprogs):
+        print('seeded special case', name, flush=True)
+        outs = E.run(prog, ins, target='hip')
+        want = OE.run(oprog, oins)
+        for k, (o, w) in enumerate(zip(outs, want)):
+            if name == 'gather_interpolated':
+                np.testing.assert_allclose(o, w, rtol=1e-6, atol=1e-6, err_msg='%s output %d' % (name, k))
+            else:
+                np.testing.assert_array_equal(o, w, err_msg='%s output %d' % (name, k))
+
+
+@pytest.mark.gpu
+def test_hip_index_outside_the_tensor_reads_zero_and_drops_updates():
+    """Undefined in the reference; this device never touches memory outside the tensors."""
+    from plaidml_amd import edsl as E
+    T, I = E.Placeholder(E.DType.FLOAT32, [4]), E.Placeholder(E.DType.INT32, [3])
+    U = E.Placeholder(E.DType.FLOAT32, [3])
+    g, s = E.run(E.Program('p', [T, I, U], [E.gather(T, I), E.scatter(T, I, U)]),
+                 [np.arange(1, 5, dtype=np.float32), np.array([2, 9, -1], np.int32), np.array([10, 20, 30], np.float32)], target='hip')
+    np.testing.assert_array_equal(g, [3, 0, 0])
+    np.testing.assert_array_equal(s, [1, 2, 13, 4])
