@@ -34,6 +34,7 @@ enum class PoolMode { AVG, MAX, MIN, SUM, _LAST };
 enum class TensorLayout { NXC, NCX, KCX, XCK, GKCX, XGCK, _LAST };
 enum class PadMode { CONSTANT, EDGE, REFLECT, SYMMETRIC, _LAST };
 enum class EpsMode { ADD, MAX, _LAST };
+enum class TopKSortType { VALUE, INDEX, _LAST };
 // reshape: take the dimension from the input / infer it from the element count
 static const int AUTO_DIM_MATCH = 0;
 static const int AUTO_DIM_FILL = -1;
@@ -164,6 +165,49 @@ class slice {
  private:
   edsl::Tensor I_;
   std::vector<edsl::Value> dims_;
+};
+
+class gatherND {
+ public:
+  explicit gatherND(const edsl::Tensor& x, const edsl::Tensor& y) : x_(x), y_(y) {}
+  gatherND& interpolationMode(edsl::InterpolationMode mode) { interpolation_mode_ = mode; return *this; }
+  gatherND& batchDims(int batch_dims) { batch_dims_ = batch_dims; return *this; }
+  operator edsl::Tensor() const {  // NOLINT
+    return details::op("gatherND", edsl::make_tuple(x_, y_, batch_dims_, static_cast<int>(interpolation_mode_))).as_tensor();
+  }
+
+ private:
+  edsl::Tensor x_, y_;
+  int64_t batch_dims_ = 0;
+  edsl::InterpolationMode interpolation_mode_ = edsl::InterpolationMode::NONE;
+};
+
+inline edsl::Tensor sort(const edsl::Tensor& I, int axis, edsl::SortDirection direction = edsl::SortDirection::ASC) {
+  return details::op("sort", edsl::make_tuple(I, axis, static_cast<int>(direction))).as_tensor();
+}
+
+class topk {
+ public:
+  explicit topk(edsl::Tensor I, int k) : I_(I), k_(k) {}
+  topk& axis(int axis) { axis_ = axis; return *this; }
+  topk& sort_direction(edsl::SortDirection sort_direction) { sort_direction_ = sort_direction; return *this; }
+  topk& sort_type(TopKSortType sort_type) { sort_type_ = sort_type; return *this; }
+  topk& index_element_type(DType index_element_type) { index_element_type_ = index_element_type; return *this; }
+  // {values, positions}
+  std::vector<edsl::Tensor> build() {
+    auto args = edsl::make_tuple(I_, k_, axis_, static_cast<int>(sort_direction_), static_cast<int>(sort_type_),
+                                 static_cast<int>(index_element_type_));
+    auto R = details::op("topk", args).as_tuple();
+    return {R[0].as_tensor(), R[1].as_tensor()};
+  }
+
+ private:
+  edsl::Tensor I_;
+  int k_;
+  int axis_ = -1;
+  edsl::SortDirection sort_direction_ = edsl::SortDirection::DESC;
+  TopKSortType sort_type_ = TopKSortType::VALUE;
+  DType index_element_type_ = DType::INT32;
 };
 
 inline edsl::Tensor argmax(const edsl::Tensor& I, const edsl::Value& axes = edsl::None()) {

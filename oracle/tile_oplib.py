@@ -808,3 +808,65 @@ def slice_of(I, slices):
         o_idxs.append(o)
         i_idxs.append(start + step * o)
     return E.Contraction('slice').outShape(o_dims).outAccess(o_idxs).assign(I[i_idxs]).build()
+
+
+TOPK_VALUE, TOPK_INDEX = range(2)
+
+
+def gatherND(x, y, batch_dims=0, interpolation_mode=E.INTERP_NONE):
+    """ops.cc:1728-1801: the ND mode of gather; LINEAR pads the addressed dimensions with two zeros per side and sums
+    the 2^k corners of the surrounding cell weighted by the opposite distances."""
+    idx_dims = y.shape[-1]
+    if idx_dims + batch_dims > len(x.shape):
+        raise ValueError('Invalid Indices')
+    if interpolation_mode == E.INTERP_NONE:
+        return E.gather(x, y, mode=E.GATHER_ND, batch_dims=batch_dims)
+    if interpolation_mode != E.INTERP_LINEAR:
+        raise ValueError('Unsupported InterpolationMode in gatherND')
+    pads = [0] * len(x.shape)
+    for i in range(idx_dims):
+        pads[i + batch_dims] = 2
+    X = explicit_padding(x, pads, pads, PAD_CONSTANT, 0)
+    Y = y + 2
+    if len(y.shape) - batch_dims != 2:
+        raise ValueError('Indices dimension should be batch_dims plus two in interpolated gatherND')
+    Yf = E.cast(Y, E.DType.FLOAT32)
+    dims = [E.gather(Yf, E.cast(E.index([1], 0), E.DType.INT32) + i, axis=-1) for i in range(idx_dims)]
+    lower = [E.floor(d) for d in dims]
+    upper = [E.floor(d) + 1.0 for d in dims]
+    zero = E.cast(E.index([1], 0), E.DType.FLOAT32)
+    result = zero
+    for corner in range(2 ** idx_dims):
+        at, coeff, j = [], zero + 1, corner
+        for k in range(idx_dims):
+            high = j % 2
+            j //= 2
+            at.append(upper[k] if high else lower[k])
+            coeff = coeff * squeeze(dims[k] - lower[k], [-1]) if high else coeff * squeeze(upper[k] - dims[k], [-1])
+        vertex = E.gather(X, E.cast(concatenate(at, -1), E.DType.INT32), mode=E.GATHER_ND, batch_dims=batch_dims)
+        result = result + vertex * broadcast(coeff, list(vertex.shape), list(range(len(coeff.shape))))
+    return result
+
+
+def _sorted_by(I, order, axis):
+    nd = len(I.shape)
+    coords = [unsqueeze(order if i == axis else E.index(list(order.shape), i), [nd]) for i in range(nd)]
+    return E.gather(I, concatenate(coords, -1), mode=E.GATHER_ND)
+
+
+def sort(I, axis=-1, direction=E.SORT_ASC):
+    """ops.cc:3100-3127."""
+    axis = _axis(axis, len(I.shape), 'sort')
+    return _sorted_by(I, E.argsort(I, axis, direction), axis)
+
+
+def topk(I, k, axis=-1, sort_direction=E.SORT_DESC, sort_type=TOPK_VALUE, index_element_type=None):
+    """ops.cc:2420-2467; returns (values, positions)."""
+    axis = _axis(axis, len(I.shape), 'topk')
+    order = E.argsort(I, axis, sort_direction)
+    first_k = E.index([int(k)], 0)
+    idxs = E.gather(order, first_k, axis=axis)
+    if sort_type == TOPK_VALUE:
+        return E.gather(_sorted_by(I, order, axis), first_k, axis=axis), idxs
+    by_position = _sorted_by(idxs, E.argsort(idxs, axis, E.SORT_ASC), axis)
+    return _sorted_by(I, by_position, axis), by_position

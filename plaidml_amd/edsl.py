@@ -801,6 +801,14 @@ class Value(_Handle):
     def as_tensor(self):
         return Tensor(ptr=call('plaidml_value_expr_get', self._ptr))
 
+    def as_tuple(self):
+        # the elements become this caller's handles; plaidml_tuple_free releases the container only
+        lst = call('plaidml_value_tuple_get', self._ptr)
+        try:
+            return [Value(ptr=lst.contents.elts[i]) for i in range(lst.contents.size)]
+        finally:
+            call('plaidml_tuple_free', lst)
+
     def __str__(self):
         return _take_str(call('plaidml_value_repr', self._ptr))
 

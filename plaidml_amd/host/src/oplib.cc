@@ -1272,6 +1272,123 @@ Value op_variance(const Value& value) {
   return Value{S / denom};
 }
 
+// ---- operations built on the special intrinsics ------------------------------------------------------------
+Value int_tuple(const std::vector<int64_t>& v) {
+  std::vector<Value> vals;
+  for (int64_t x : v) vals.emplace_back(x);
+  return Value(vals);
+}
+Tensor unsqueeze_at(const Tensor& t, int64_t axis) { return op_unsqueeze(make_tuple(Value{t}, int_tuple({axis}))).as_tensor(); }
+Tensor squeeze_last(const Tensor& t) { return op_squeeze(make_tuple(Value{t}, int_tuple({-1}))).as_tensor(); }
+
+// plaidml/op/lib/ops.cc:1728-1801.  Without interpolation this is the ND mode of the gather intrinsic.  LINEAR
+// (floating coordinates) pads the addressed dimensions with two zeros on each side and sums the 2^k corners of
+// the surrounding cell, each gathered with integer coordinates and weighted by the opposite distances.
+Value op_gatherND(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 4) throw std::runtime_error("gatherND expects 4 arguments");
+  auto I = args[0].as_tensor();
+  auto idx = args[1].as_tensor();
+  const int64_t batch_dims = args[2].as_int();
+  const int64_t I_rank = static_cast<int64_t>(I.rank());
+  const auto idx_shape = idx.compute_shape().sizes();
+  if (idx_shape.empty()) throw std::runtime_error("gatherND needs indices of at least one dimension");
+  const int64_t idx_dims = idx_shape.back();
+  if (idx_dims + batch_dims > I_rank)
+    throw std::runtime_error("Invalid Indices: Data(shape: '" + I.compute_shape().str() + "'), Indices(shape: '" +
+                             idx.compute_shape().str() + "'), BatchDims('" + std::to_string(batch_dims) + "')");
+  const auto mode = static_cast<InterpolationMode>(args[3].as_int());
+  if (mode == InterpolationMode::NONE) return Value{gatherBuilder(I, idx, static_cast<uint64_t>(batch_dims), mode).build()};
+  if (mode != InterpolationMode::LINEAR) throw std::runtime_error("Unsupported InterpolationMode in gatherND");
+  const int64_t pad_length = 2;
+  std::vector<int64_t> pads(I_rank, 0);
+  for (int64_t i = 0; i < idx_dims; ++i) pads[i + batch_dims] = pad_length;
+  Tensor X = op_explicit_padding(make_tuple(Value{I}, int_tuple(pads), int_tuple(pads),
+                                            Value{static_cast<int64_t>(plaidml::op::PadMode::CONSTANT)}, Value{Tensor(int64_t{0})}))
+                 .as_tensor();
+  Tensor Y = idx + pad_length;
+  if (static_cast<int64_t>(idx_shape.size()) - batch_dims != 2)
+    throw std::runtime_error(
+        " Indices dimension should be batch_dims plus two in interpolated gatherND, please reshape indices to satisfy this "
+        "requirement.");
+  Tensor Y_float = cast(Y, DType::FLOAT32);
+  std::vector<Tensor> dims, lower, upper;
+  for (int64_t i = 0; i < idx_dims; ++i) {
+    Tensor dim = gather(Y_float, static_cast<int>(i)).axis(-1);
+    dims.push_back(dim);
+    lower.push_back(floor(dim));
+    upper.push_back(floor(dim) + 1.0);
+  }
+  Tensor ZERO = cast(index({TensorDim(1)}, 0), DType::FLOAT32);
+  Tensor result = ZERO;
+  const int64_t corners = int64_t{1} << idx_dims;
+  for (int64_t corner = 0; corner < corners; ++corner) {
+    std::vector<Tensor> at;
+    Tensor coeff = ZERO + 1;
+    for (int64_t k = 0, j = corner; k < idx_dims; ++k, j /= 2) {
+      const bool high = (j % 2) != 0;
+      at.push_back(high ? upper[k] : lower[k]);
+      coeff = high ? coeff * squeeze_last(dims[k] - lower[k]) : coeff * squeeze_last(upper[k] - dims[k]);
+    }
+    Tensor at_int = cast(concatenate(at, -1), DType::INT32);
+    Tensor vertex = gatherBuilder(X, at_int, static_cast<uint64_t>(batch_dims), InterpolationMode::NONE).build();
+    std::vector<int64_t> axes;
+    for (size_t i = 0; i < coeff.rank(); ++i) axes.push_back(static_cast<int64_t>(i));
+    Tensor spread = op_broadcast(make_tuple(Value{coeff}, int_tuple(vertex.compute_shape().sizes()), int_tuple(axes))).as_tensor();
+    result = result + vertex * spread;
+  }
+  return Value{result};
+}
+
+// plaidml/op/lib/ops.cc:3100-3127: the sorted values are gathered with full coordinates whose `axis` entry is the
+// argsort and whose other entries are the element's own position
+Tensor sorted_by(const Tensor& I, const Tensor& order, int64_t axis) {
+  const int64_t ndims = static_cast<int64_t>(I.rank());
+  std::vector<TensorDim> dims(order.rank());
+  order.bind_dims(dims);
+  std::vector<Tensor> coords;
+  for (int64_t i = 0; i < ndims; ++i) coords.push_back(unsqueeze_at(i == axis ? order : index(dims, static_cast<size_t>(i)), ndims));
+  return gatherBuilder(I, concatenate(coords, -1), 0, InterpolationMode::NONE).build();
+}
+
+Value op_sort(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 3) throw std::runtime_error("sort expects 3 arguments");
+  auto I = args[0].as_tensor();
+  const int64_t raw_direction = args[2].as_int();
+  if (raw_direction != 0 && raw_direction != 1) throw std::runtime_error("Invalid enumeration value in operation arguments");
+  const auto direction = static_cast<SortDirection>(raw_direction);
+  const int64_t axis = static_cast<int64_t>(normalize_axis(args[1].as_int(), I.rank(), "sort"));
+  return Value{sorted_by(I, argsort(I, static_cast<int>(axis), direction), axis)};
+}
+
+// plaidml/op/lib/ops.cc:2420-2467: the first k of the sorted values and positions; sort type INDEX re-orders those k
+// by position
+Value op_topk(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 6) throw std::runtime_error("topk expects 6 arguments");
+  auto I = args[0].as_tensor();
+  const int64_t k = args[1].as_int();
+  const int64_t raw_direction = args[3].as_int();
+  if (raw_direction != 0 && raw_direction != 1) throw std::runtime_error("Invalid enumeration value in operation arguments");
+  const auto direction = static_cast<SortDirection>(raw_direction);
+  const auto sort_type = validate<plaidml::op::TopKSortType>(args[4].as_int());
+  const int64_t axis = static_cast<int64_t>(normalize_axis(args[2].as_int(), I.rank(), "topk"));
+  Tensor order = argsort(I, static_cast<int>(axis), direction);
+  Tensor first_k = index({TensorDim(k)}, 0);
+  Tensor idxs_topk = gather(order, first_k).axis(axis);
+  std::vector<Value> out;
+  if (sort_type == plaidml::op::TopKSortType::VALUE) {
+    Tensor values = sorted_by(I, order, axis);
+    Tensor vals_topk = gather(values, first_k).axis(axis);
+    out = {Value{vals_topk}, Value{idxs_topk}};
+  } else {
+    Tensor by_position = sorted_by(idxs_topk, argsort(idxs_topk, static_cast<int>(axis), SortDirection::ASC), axis);
+    out = {Value{sorted_by(I, by_position, axis)}, Value{by_position}};
+  }
+  return Value(out);
+}
+
 using OpFn = std::function<Value(const Value&)>;
 const std::map<std::string, OpFn>& registry() {
   static const std::map<std::string, OpFn> r = {
@@ -1290,6 +1407,7 @@ const std::map<std::string, OpFn>& registry() {
       {"elu", op_elu},
       {"explicit_padding", op_explicit_padding},
       {"flip", op_flip},
+      {"gatherND", op_gatherND},
       {"hard_sigmoid", op_hard_sigmoid},
       {"l2norm", op_l2norm},
       {"lrn", op_lrn},
@@ -1309,11 +1427,13 @@ const std::map<std::string, OpFn>& registry() {
       {"sigmoid", op_sigmoid},
       {"slice", op_slice},
       {"softmax", op_softmax},
+      {"sort", op_sort},
       {"spatial_padding", op_spatial_padding},
       {"square", op_square},
       {"squeeze", op_squeeze},
       {"sum", [](const Value& v) { return reduce(v, "sum", PLAIDML_AGG_OP_SUM); }},
       {"tile", op_tile},
+      {"topk", op_topk},
       {"transpose", op_transpose},
       {"unsqueeze", op_unsqueeze},
       {"variance", op_variance},

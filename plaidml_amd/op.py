@@ -224,3 +224,20 @@ def slice_of(I, slices):
         else:
             raise ValueError('Unexpected type {} used to slice tensor'.format(type(s)))
     return E.op_make('slice', [I, out]).as_tensor()
+
+
+TOPK_VALUE, TOPK_INDEX = range(2)
+
+
+def gatherND(x, y, batch_dims=0, interpolation_mode=E.INTERP_NONE):
+    return E.op_make('gatherND', [x, y, int(batch_dims), int(interpolation_mode)]).as_tensor()
+
+
+def sort(I, axis=-1, direction=E.SORT_ASC):
+    return E.op_make('sort', [I, int(axis), int(direction)]).as_tensor()
+
+
+def topk(I, k, axis=-1, sort_direction=E.SORT_DESC, sort_type=TOPK_VALUE, index_element_type=E.DType.INT32):
+    """Returns (values, positions)."""
+    r = E.op_make('topk', [I, int(k), int(axis), int(sort_direction), int(sort_type), int(index_element_type)]).as_tuple()
+    return r[0].as_tensor(), r[1].as_tensor()

@@ -323,6 +323,65 @@ void caseOpBuilders() {
   }
 }
 
+// argsort / gather / scatter and the operations built on them, with the reference's answers
+// (plaidml/edsl/tests/edsl_test.cc: Gather :1490-1508, InterpolatedGatherLinear :1523-1533, ScatterDup1D :1917-1930,
+// ScatterElt :2080-2107, ArgSort1dDup :2462-2492; plaidml/op/op_test.cc: Sort :638-658).
+void caseSpecialOps() {
+  {
+    auto A = Placeholder(DType::FLOAT32, {3, 2});
+    auto B = Placeholder(DType::INT32, {4});
+    Tensor O = gather(A, B).axis(1);
+    auto out = run(buildProgram("gather", {A, B}, {O}),
+                   {makeBuffer<float>(DType::FLOAT32, {3, 2}, {-5, -6, -7, 4, 5, 6}), makeBuffer<int32_t>(DType::INT32, {4}, {0, 1, 1, 0})});
+    expectEq<float>("gather", readBuffer<float>(out[0]), {-5, -6, -6, -5, -7, 4, 4, -7, 5, 6, 6, 5});
+  }
+  {
+    auto A = Placeholder(DType::FLOAT32, {1, 6});
+    auto B = Placeholder(DType::FLOAT32, {12});
+    Tensor O = gather(A, B).axis(-1).interpolationMode(InterpolationMode::LINEAR).outOfBoundsMode(OutOfBoundsMode::RETURN_ZERO);
+    auto out = run(buildProgram("gather_linear", {A, B}, {O}),
+                   {makeBuffer<float>(DType::FLOAT32, {1, 6}, {0, 1, 8, 5, 5, 2}),
+                    makeBuffer<float>(DType::FLOAT32, {12}, {-0.25, 0.25, 0.75, 1.25, 1.75, 2.25, 2.75, 3.25, 3.75, 4.25, 4.75, 5.25})});
+    expectEq<float>("gather_linear_return_zero", readBuffer<float>(out[0]), {0, 0.25, 0.75, 2.75, 6.25, 7.25, 5.75, 5, 5, 4.25, 2.75, 0});
+  }
+  {
+    auto D = Placeholder(DType::FLOAT32, {8});
+    auto I = Placeholder(DType::INT32, {4});
+    auto U = Placeholder(DType::FLOAT32, {4});
+    Tensor O = scatter(D, I, U);
+    auto out = run(buildProgram("scatter", {D, I, U}, {O}),
+                   {makeBuffer<float>(DType::FLOAT32, {8}, {0, 0, 0, 0, 0, 0, 0, 0}), makeBuffer<int32_t>(DType::INT32, {4}, {4, 3, 3, 7}),
+                    makeBuffer<float>(DType::FLOAT32, {4}, {9, 10, 11, 12})});
+    expectEq<float>("scatter_dup", readBuffer<float>(out[0]), {0, 0, 0, 21, 9, 0, 0, 12});
+  }
+  {
+    auto D = Placeholder(DType::FLOAT32, {4, 4});
+    auto I = Placeholder(DType::INT32, {2, 2});
+    auto U = Placeholder(DType::FLOAT32, {2, 2});
+    Tensor O = scatter(D, I, U).axis(1).mode(ScatterMode::UPDATE_ELT);
+    auto out = run(buildProgram("scatter_elt", {D, I, U}, {O}),
+                   {makeBuffer<float>(DType::FLOAT32, {4, 4}, std::vector<float>(16, 1.f)), makeBuffer<int32_t>(DType::INT32, {2, 2}, {2, 0, 3, 1}),
+                    makeBuffer<float>(DType::FLOAT32, {2, 2}, {9, 9, 9, 9})});
+    expectEq<float>("scatter_elt", readBuffer<float>(out[0]), {9, 1, 9, 1, 1, 9, 1, 9, 1, 1, 1, 1, 1, 1, 1, 1});
+  }
+  {
+    std::vector<float> x = {81.69, 81.69, 27.74, 43.69, 55.79, 56.79, 57.52, 7.11, 39.48, 5.9,
+                            14.81, 66.23, 20.25, 66.05, 64.5,  71.07, 67.6,  54.42, 87.59, 80.02};
+    auto I = Placeholder(DType::FLOAT32, {20});
+    auto out = run(buildProgram("argsort", {I}, {argsort(I, 0)}), {makeBuffer<float>(DType::FLOAT32, {20}, x)});
+    expectEq<int32_t>("argsort_dup", readBuffer<int32_t>(out[0]), {9, 7, 10, 12, 2, 8, 3, 17, 4, 5, 6, 14, 13, 11, 16, 15, 19, 0, 1, 18});
+    auto A = Placeholder(DType::FLOAT32, {5, 4});
+    auto top = op::topk(A, 2).axis(1).build();
+    auto res = run(buildProgram("sort_topk", {A}, {op::sort(A, 1, SortDirection::ASC), top[0], top[1]}),
+                   {makeBuffer<float>(DType::FLOAT32, {5, 4}, {81.69, 95.74, 27.74, 43.69, 55.79, 56.79, 57.52, 5.9, 39.48, 7.11,
+                                                                14.81, 66.23, 20.25, 66.05, 64.5,  71.07, 67.6,  54.42, 87.59, 80.02})});
+    expectEq<float>("sort", readBuffer<float>(res[0]), {27.74, 43.69, 81.69, 95.74, 5.9,   55.79, 56.79, 57.52, 7.11,  14.81,
+                                                        39.48, 66.23, 20.25, 64.5,  66.05, 71.07, 54.42, 67.6,  80.02, 87.59});
+    expectEq<float>("topk_values", readBuffer<float>(res[1]), {95.74, 81.69, 57.52, 56.79, 66.23, 39.48, 71.07, 66.05, 87.59, 80.02});
+    expectEq<int32_t>("topk_positions", readBuffer<int32_t>(res[2]), {1, 0, 2, 1, 3, 0, 3, 1, 2, 3});
+  }
+}
+
 void caseErrors() {
   auto A = Placeholder(DType::FLOAT32, {4, 4});
   auto program = buildProgram("ident", {A}, {A + 1.0});
@@ -360,6 +419,7 @@ int main() {
     caseOpLibrary();
     caseIntrinsics();
     caseOpBuilders();
+    caseSpecialOps();
     caseErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAILED with exception: %s\n", e.what());

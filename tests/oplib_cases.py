@@ -283,7 +283,64 @@ def scale_gradient(E, op):
     return p, ins, x, True
 
 
+def sort_reference(E, op):
+    """OpTest.Sort, plaidml/op/op_test.cc:638-658."""
+    data = [81.69, 95.74, 27.74, 43.69, 55.79, 56.79, 57.52, 5.9, 39.48, 7.11, 14.81, 66.23, 20.25, 66.05, 64.5, 71.07, 67.6,
+            54.42, 87.59, 80.02]
+    want = [27.74, 43.69, 81.69, 95.74, 5.9, 55.79, 56.79, 57.52, 7.11, 14.81, 39.48, 66.23, 20.25, 64.5, 66.05, 71.07, 54.42,
+            67.6, 80.02, 87.59]
+    p, ins, _ = _one(E, 'sort', (5, 4), lambda X: op.sort(X, 1, E.SORT_ASC), data)
+    return p, ins, np.array(want, np.float32).reshape(5, 4), True
+
+
+def sort_descending_axis0(E, op):
+    p, ins, x = _one(E, 'sort', (6, 3, 4), lambda X: op.sort(X, 0, E.SORT_DESC))
+    return p, ins, -np.sort(-x, axis=0), True
+
+
+def gather_nd_reference(E, op):
+    """CppEdsl.GatherND / GatherNDWithBatchDims, plaidml/edsl/tests/edsl_test.cc:1661-1710."""
+    A, B = _f32(E, (2, 2, 2)), E.Placeholder(E.DType.INT32, [2, 2])
+    C, D = _f32(E, (2, 3, 4)), E.Placeholder(E.DType.INT32, [2, 3, 1, 1])
+    prog = E.Program('gatherND', [A, B, C, D], [op.gatherND(A, B), op.gatherND(C, D, batch_dims=2)])
+    ins = [np.array([-5, -6, 1.3, 4.5, -7, 4, 5, 6], np.float32).reshape(2, 2, 2), np.array([0, 1, 1, 0], np.int32).reshape(2, 2),
+           np.arange(1, 25, dtype=np.float32).reshape(2, 3, 4), np.array([1, 0, 2, 0, 2, 2], np.int32).reshape(2, 3, 1, 1)]
+    return prog, ins, [np.array([1.3, 4.5, -7, 4], np.float32).reshape(2, 2),
+                       np.array([2, 5, 11, 13, 19, 23], np.float32).reshape(2, 3, 1)], True
+
+
+def gather_nd_linear_reference(E, op):
+    """CppEdsl.InterpolatedGatherND1 / ND2 / ND3, plaidml/edsl/tests/edsl_test.cc:1712-1794."""
+    A, B1, B3 = _f32(E, (2, 2)), _f32(E, (3, 1)), _f32(E, (3, 2))
+    C, B2 = _f32(E, (4, 3, 2)), _f32(E, (4, 1, 2))
+    lin = E.INTERP_LINEAR
+    prog = E.Program('gatherND', [A, B1, B3, C, B2],
+                     [op.gatherND(A, B1, interpolation_mode=lin), op.gatherND(C, B2, batch_dims=1, interpolation_mode=lin),
+                      op.gatherND(A, B3, interpolation_mode=lin)])
+    a = np.array([-5, -6, 1.3, 4.5], np.float32).reshape(2, 2)
+    c = np.array([-5, -6, 1.3, 4.5, 2, 3.5, 0.3, 4.1, -5, 6, 1.1, 0.5, 1, 2, 3, 4, 5, 6, 0.8, 0.5, 2, -6, 1.9, 9.5],
+                 np.float32).reshape(4, 3, 2)
+    ins = [a, np.array([0.2, 0.5, 0.9], np.float32).reshape(3, 1), np.array([0.2, 0.5, 0.3, 0.9, 0.5, 0.5], np.float32).reshape(3, 2),
+           c, np.array([0.2, 0.5, 0.2, 0.9, 0.2, 0.5, 0.2, 0.9], np.float32).reshape(4, 1, 2)]
+    want = [np.array([-3.74, -3.9, -1.85, -0.75, 0.67, 3.45], np.float32).reshape(3, 2),
+            np.array([-3.82, 3.956, 1.9, -0.616], np.float32).reshape(4, 1),
+            np.array([-3.82, -2.876, -1.3], np.float32)]
+    return prog, ins, want, False
+
+
+def topk(E, op):
+    X = _f32(E, (4, 9))
+    x = _rng().standard_normal((4, 9)).astype(np.float32)
+    v, i = op.topk(X, 3, axis=1)                                              # largest three, by value
+    v2, i2 = op.topk(X, 4, axis=1, sort_direction=E.SORT_ASC, sort_type=op.TOPK_INDEX)   # smallest four, in position order
+    order = np.argsort(-x, axis=1, kind='stable')[:, :3]
+    small = np.sort(np.argsort(x, axis=1, kind='stable')[:, :4], axis=1)
+    want = [np.take_along_axis(x, order, 1), order.astype(np.int32), np.take_along_axis(x, small, 1), small.astype(np.int32)]
+    return E.Program('topk', [X], [v, i, v2, i2]), [x], want, True
+
+
 CASES = {f.__name__: f for f in (
+    sort_reference, sort_descending_axis0, gather_nd_reference, gather_nd_linear_reference, topk,
     broadcast_noop_reference, broadcast_scalar_reference, broadcast_noop_large_reference, broadcast_numpy_reference,
     broadcast_numpy2_reference, broadcast_numpy3_reference, broadcast_non_numpy_reference, reorg_yolo_decrease_reference,
     reorg_yolo_increase_reference, reorg_yolo_nhwc, all_any, binary_crossentropy, cumprod, l2norm, lrn, mvn, slice_of,
