@@ -35,6 +35,7 @@ enum class TensorLayout { NXC, NCX, KCX, XCK, GKCX, XGCK, _LAST };
 enum class PadMode { CONSTANT, EDGE, REFLECT, SYMMETRIC, _LAST };
 enum class EpsMode { ADD, MAX, _LAST };
 enum class TopKSortType { VALUE, INDEX, _LAST };
+enum class InterpolationMode { NEAREST, BILINEAR, _LAST };
 // reshape: take the dimension from the input / infer it from the element count
 static const int AUTO_DIM_MATCH = 0;
 static const int AUTO_DIM_FILL = -1;
@@ -69,6 +70,12 @@ inline edsl::Tensor broadcast(const edsl::Tensor& I, const std::vector<int64_t>&
 }
 
 inline edsl::Tensor cumprod(const edsl::Tensor& I, int axis) { return details::op("cumprod", edsl::make_tuple(I, axis)).as_tensor(); }
+
+inline edsl::Tensor image_resize(const edsl::Tensor& I, const std::vector<int>& factors, InterpolationMode interpolation,
+                                 TensorLayout layout) {
+  return details::op("image_resize", edsl::make_tuple(I, edsl::make_tuple(factors), static_cast<int>(interpolation),
+                                                      static_cast<int>(layout))).as_tensor();
+}
 
 class l2norm {
  public:

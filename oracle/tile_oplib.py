@@ -870,3 +870,37 @@ def topk(I, k, axis=-1, sort_direction=E.SORT_DESC, sort_type=TOPK_VALUE, index_
         return E.gather(_sorted_by(I, order, axis), first_k, axis=axis), idxs
     by_position = _sorted_by(idxs, E.argsort(idxs, axis, E.SORT_ASC), axis)
     return _sorted_by(I, by_position, axis), by_position
+
+
+RESIZE_NEAREST, RESIZE_BILINEAR = range(2)
+
+
+def image_resize(I, factors, interp=RESIZE_NEAREST, layout=LAYOUT_NXC):
+    """ops.cc:1822-1918: NEAREST repeats pixels; BILINEAR spreads every pixel with a (2f-1) x (2f-1) tent kernel
+    (corners aligned to 0 and f * (dim - 1), zero outside)."""
+    if builtins.any(f <= 0 for f in factors):
+        raise ValueError('All scaling factors in image_resize must be positive')
+    if len(I.shape) != 4 or len(factors) != 2:
+        raise ValueError('image_resize expects 2 spatial dims and 2 factors')
+    if layout not in (LAYOUT_NXC, LAYOUT_NCX):
+        raise ValueError('Unable to apply image_resize to a tensor with this layout')
+    pre = 2 if layout == LAYOUT_NCX else 1
+    fh, fw = int(factors[0]), int(factors[1])
+    if interp == RESIZE_NEAREST:
+        return repeat(repeat(I, fh, pre), fw, pre + 1)
+    if interp != RESIZE_BILINEAR:
+        raise ValueError('Unrecognized InterpolationMode in image_resize')
+    j, i, y, x = E.TensorIndexes(4)
+    hcoef = E.cast(1.0 / fh, E.DType.FLOAT32)
+    wcoef = E.cast(1.0 / fw, E.DType.FLOAT32)
+    hvec = E.Contraction('image_resize').outShape([fh]).outAccess([y]).assign(hcoef[[]]).build()
+    wvec = E.Contraction('image_resize').outShape([fw]).outAccess([x]).assign(wcoef[[]]).build()
+    hk = E.Contraction('image_resize').outShape([2 * fh - 1]).outAccess([y]).sum(hvec[j + y - fh + 1]).add_constraint(j < fh).build()
+    wk = E.Contraction('image_resize').outShape([2 * fw - 1]).outAccess([x]).sum(wvec[i + x - fw + 1]).add_constraint(i < fw).build()
+    K = E.Contraction('image_resize').outShape([2 * fh - 1, 2 * fw - 1]).outAccess([y, x]).assign(hk[y] * wk[x]).build()
+    idxs = E.TensorIndexes(4)
+    o_dims, o_idxs = list(I.shape), list(idxs)
+    o_dims[pre], o_dims[pre + 1] = fh * I.shape[pre], fw * I.shape[pre + 1]
+    o_idxs[pre] = fh * idxs[pre] + j - fh + 1
+    o_idxs[pre + 1] = fw * idxs[pre + 1] + i - fw + 1
+    return E.Contraction('image_resize').outShape(o_dims).outAccess(o_idxs).sum(I[idxs] * K[j, i]).build()

@@ -1389,6 +1389,62 @@ Value op_topk(const Value& value) {
   return Value(out);
 }
 
+// plaidml/op/lib/ops.cc:1822-1918: both spatial dimensions of an image grow by integer factors.  NEAREST repeats
+// pixels; BILINEAR spreads every pixel with a (2f-1) x (2f-1) tent kernel, which aligns the corners to 0 and
+// f * (dim - 1) and treats the outside as zero.
+Value op_image_resize(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 4) throw std::runtime_error("image_resize expects 4 arguments");
+  auto I = args[0].as_tensor();
+  const auto factors = args[1].as_int_tuple();
+  const auto interp = validate<plaidml::op::InterpolationMode>(args[2].as_int());
+  const auto layout = validate<TensorLayout>(args[3].as_int());
+  for (int64_t f : factors)
+    if (f <= 0) throw std::runtime_error("All scaling factors in image_resize must be positive (received " + std::to_string(f) + ")");
+  const size_t ndims = I.rank();
+  int64_t pre_axes;
+  switch (layout) {
+    case TensorLayout::NCX: pre_axes = 2; break;
+    case TensorLayout::NXC: pre_axes = 1; break;
+    default: throw std::runtime_error("Unable to apply image_resize to a tensor with this layout");
+  }
+  if (ndims != 4) throw std::runtime_error("Expected 2 spatial dims for resize_images, received " + std::to_string(static_cast<int64_t>(ndims) - 2));
+  if (factors.size() != 2)
+    throw std::runtime_error("Cannot resize a 2D image using " + std::to_string(factors.size()) + " spatial scaling factors");
+  if (interp == plaidml::op::InterpolationMode::NEAREST) {
+    Value R = op_repeat(make_tuple(args[0], Value{factors[0]}, Value{pre_axes}));
+    return op_repeat(make_tuple(R, Value{factors[1]}, Value{pre_axes + 1}));
+  }
+  if (interp != plaidml::op::InterpolationMode::BILINEAR) throw std::runtime_error("Unrecognized InterpolationMode in image_resize");
+  Tensor HCoeff = cast(Tensor(1.0 / factors[0]), DType::FLOAT32);
+  Tensor WCoeff = cast(Tensor(1.0 / factors[1]), DType::FLOAT32);
+  TensorDim HFactor(factors[0]), WFactor(factors[1]);
+  TensorIndex j("j"), i("i"), y("y"), x("x");
+  Tensor HCoeffVec = Contraction({HFactor}, {y}, "image_resize").assign(HCoeff());
+  Tensor WCoeffVec = Contraction({WFactor}, {x}, "image_resize").assign(WCoeff());
+  TensorDim HK_dim = 2 * HFactor - 1, WK_dim = 2 * WFactor - 1;
+  Tensor HK = Contraction({HK_dim}, {y}, "image_resize").sum(HCoeffVec(j + y - HFactor + 1)).add_constraint(j < HFactor);
+  Tensor WK = Contraction({WK_dim}, {x}, "image_resize").sum(WCoeffVec(i + x - WFactor + 1)).add_constraint(i < WFactor);
+  Tensor K = Contraction({HK_dim, WK_dim}, {y, x}, "image_resize").assign(HK(y) * WK(x));
+  std::vector<TensorDim> I_dims(ndims), O_dims;
+  std::vector<TensorIndex> I_idxs(ndims), O_idxs;
+  I.bind_dims(I_dims);
+  for (int64_t ax = 0; ax < pre_axes; ++ax) {
+    O_dims.push_back(I_dims[ax]);
+    O_idxs.push_back(I_idxs[ax]);
+  }
+  O_dims.push_back(HFactor * I_dims[pre_axes]);
+  O_dims.push_back(WFactor * I_dims[pre_axes + 1]);
+  O_idxs.push_back(HFactor * I_idxs[pre_axes] + j - HFactor + 1);
+  O_idxs.push_back(WFactor * I_idxs[pre_axes + 1] + i - WFactor + 1);
+  for (size_t ax = pre_axes + 2; ax < ndims; ++ax) {
+    O_dims.push_back(I_dims[ax]);
+    O_idxs.push_back(I_idxs[ax]);
+  }
+  Tensor O = Contraction(O_dims, O_idxs, "image_resize").sum(I(I_idxs) * K(j, i));
+  return Value{O};
+}
+
 using OpFn = std::function<Value(const Value&)>;
 const std::map<std::string, OpFn>& registry() {
   static const std::map<std::string, OpFn> r = {
@@ -1409,6 +1465,7 @@ const std::map<std::string, OpFn>& registry() {
       {"flip", op_flip},
       {"gatherND", op_gatherND},
       {"hard_sigmoid", op_hard_sigmoid},
+      {"image_resize", op_image_resize},
       {"l2norm", op_l2norm},
       {"lrn", op_lrn},
       {"max", [](const Value& v) { return reduce(v, "max", PLAIDML_AGG_OP_MAX); }},

@@ -241,3 +241,10 @@ def topk(I, k, axis=-1, sort_direction=E.SORT_DESC, sort_type=TOPK_VALUE, index_
     """Returns (values, positions)."""
     r = E.op_make('topk', [I, int(k), int(axis), int(sort_direction), int(sort_type), int(index_element_type)]).as_tuple()
     return r[0].as_tensor(), r[1].as_tensor()
+
+
+RESIZE_NEAREST, RESIZE_BILINEAR = range(2)
+
+
+def image_resize(I, factors, interp=RESIZE_NEAREST, layout=LAYOUT_NXC):
+    return E.op_make('image_resize', [I, _ints(factors), int(interp), int(layout)]).as_tensor()

@@ -339,7 +339,35 @@ def topk(E, op):
     return E.Program('topk', [X], [v, i, v2, i2]), [x], want, True
 
 
+def _tent_resize(x, fh, fw):
+    """Every input pixel spread over the output with the separable tent weights 1 - |d| / f at offsets |d| < f
+    around f * position (direct accumulation; float64)."""
+    n, h, w, c = x.shape
+    out = np.zeros((n, fh * h, fw * w, c))
+    for a in range(h):
+        for b in range(w):
+            for dy in range(-fh + 1, fh):
+                for dx in range(-fw + 1, fw):
+                    oy, ox = fh * a + dy, fw * b + dx
+                    if 0 <= oy < fh * h and 0 <= ox < fw * w:
+                        out[:, oy, ox, :] += x[:, a, b, :] * (1 - abs(dy) / fh) * (1 - abs(dx) / fw)
+    return out
+
+
+def image_resize(E, op):
+    X = _f32(E, (2, 4, 5, 3))
+    x = _rng().standard_normal((2, 4, 5, 3)).astype(np.float32)
+    Xc = _f32(E, (2, 3, 4, 5))
+    outs = [op.image_resize(X, [2, 3], op.RESIZE_NEAREST), op.image_resize(X, [3, 2], op.RESIZE_BILINEAR),
+            op.image_resize(Xc, [2, 2], op.RESIZE_BILINEAR, op.LAYOUT_NCX)]
+    xc = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    want = [np.repeat(np.repeat(x, 2, 1), 3, 2), _tent_resize(x.astype(np.float64), 3, 2),
+            _tent_resize(x.astype(np.float64), 2, 2).transpose(0, 3, 1, 2)]
+    return E.Program('image_resize', [X, Xc], outs), [x, xc], want, False
+
+
 CASES = {f.__name__: f for f in (
+    image_resize,
     sort_reference, sort_descending_axis0, gather_nd_reference, gather_nd_linear_reference, topk,
     broadcast_noop_reference, broadcast_scalar_reference, broadcast_noop_large_reference, broadcast_numpy_reference,
     broadcast_numpy2_reference, broadcast_numpy3_reference, broadcast_non_numpy_reference, reorg_yolo_decrease_reference,
