@@ -348,6 +348,7 @@ inline Tensor relu(const Tensor& x, const std::string& name = "") { return intri
 inline Tensor round(const Tensor& x) { return intrinsicCall("round", {x}); }
 inline Tensor sqrt(const Tensor& x) { return intrinsicCall("sqrt", {x}); }
 inline Tensor tanh(const Tensor& x) { return intrinsicCall("tanh", {x}); }
+inline Tensor shape(const Tensor& x) { return intrinsicCall("shape", {x}); }
 inline Tensor sin(const Tensor& x) { return intrinsicCall("sin", {x}); }
 inline Tensor cos(const Tensor& x) { return intrinsicCall("cos", {x}); }
 inline Tensor tan(const Tensor& x) { return intrinsicCall("tan", {x}); }

@@ -601,6 +601,12 @@ sin, cos, tan, sinh, cosh, asin, acos, atan, asinh, acosh, atanh, erf = (
 logical_not = _unary('logical_not')
 
 
+def shape_of(x):
+    """The extents of a tensor as an si32 vector (edsl `shape`, pmlc/ast/ast_ops.cc:287-296)."""
+    x = _literal(x)
+    return Tensor('const', DType.INT32, [len(x.shape)], attrs={'value': np.array(x.shape, np.int32)})
+
+
 def pow(x, y):  # noqa: A001 - mirrors the EDSL name
     return intrinsic('pow', x, y)
 

@@ -697,6 +697,7 @@ round = _unary('round')  # noqa: A001
 sin, cos, tan, sinh, cosh, asin, acos, atan, asinh, acosh, atanh, erf = (
     _unary(n) for n in ('sin', 'cos', 'tan', 'sinh', 'cosh', 'asin', 'acos', 'atan', 'asinh', 'acosh', 'atanh', 'erf'))
 logical_not = _unary('logical_not')
+shape_of = _unary('shape')   # the extents of a tensor as an si32 vector (edsl `shape`)
 
 
 def pow(x, y):  # noqa: A001

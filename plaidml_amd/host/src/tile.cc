@@ -309,7 +309,17 @@ struct Builder {
             throw std::runtime_error("'reshape' must preserve the number of elements");
           op.operands = {src};
         } else if (node->op == "shape") {
-          throw std::runtime_error("'shape' is not supported by this backend");
+          // shapes are static here: the extents of the operand as a constant si32 vector
+          // (ShapeOpConversion, pmlc/conversion/tile_to_linalg/tile_to_linalg.cc)
+          const TensorShape src = ev.getShape(node->operands.at(0));
+          auto buf = std::make_shared<util::SimpleBuffer>(shape);
+          for (size_t d = 0; d < src.getRank(); ++d) {
+            const int32_t extent = static_cast<int32_t>(src.sizes[d]);
+            std::memcpy(buf->data() + 4 * d, &extent, 4);
+          }
+          ValuePtr v = newValue(Value::Constant, shape, "shape");
+          v->constant = buf;
+          return v;
         } else if (node->op == "gather" || node->op == "scatter" || node->op == "argsort") {
           // tensor operands first, then constants (plaidml/edsl/edsl.h:809-811, 1036-1066, 1645-1690)
           op.kind = Op::Special;

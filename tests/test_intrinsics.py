@@ -74,3 +74,22 @@ def test_hip_rejects_wrong_operand_kinds():
     i = E.Placeholder(E.DType.INT32, [3])
     with pytest.raises(E.PlaidMLError, match='needs floating-point operands'):
         E.run(E.Program('p', [i], [E.sin(i)]), [np.zeros(3, np.int32)])
+
+
+def test_oracle_shape():
+    """CppEdsl.Shape, plaidml/edsl/tests/edsl_test.cc:1120-1136."""
+    I = OE.Placeholder(OE.DType.FLOAT32, [2, 3])
+    out, = OE.run(OE.Program('shape', [I], [OE.shape_of(I)]), [np.array([[1, 2, 3], [1, 2, 3]], np.float32)])
+    assert out.dtype == np.int32
+    np.testing.assert_array_equal(out, [2, 3])
+
+
+@pytest.mark.gpu
+def test_hip_shape():
+    from plaidml_amd import edsl as E
+    I = E.Placeholder(E.DType.FLOAT32, [2, 3])
+    x = np.array([[1, 2, 3], [1, 2, 3]], np.float32)
+    out, scaled = E.run(E.Program('shape', [I], [E.shape_of(I), E.cast(E.shape_of(I), E.DType.FLOAT32) * 0.5]), [x])
+    assert out.dtype == np.int32
+    np.testing.assert_array_equal(out, [2, 3])
+    np.testing.assert_array_equal(scaled, [1.0, 1.5])
