@@ -796,7 +796,7 @@ def _eval_scatter(x, y, z, a, dt):
         else:
             dst = tuple(c[:axis]) + (int(yi[c[:yi.ndim]]),) + tuple(c[axis + 1:])
         if mode == SCATTER_NORMAL:
-            out[dst] = _store(np.asarray(out[dst] + z[c]), dt)
+            out[dst] = _store(np.asarray(out[dst] + z[c]).reshape(1), dt)[0]
         else:
             out[dst] = z[c]
     return out

@@ -50,6 +50,23 @@ def random_programs(E):
     ref = di.copy()
     np.add.at(ref, (ii[:, :, None], np.arange(2)[None, :, None], np.arange(4)[None, None, :]), ui)
     out.append(('scatter_add_int_dups', E.Program('p', [DI, II, UI], [E.scatter(DI, II, UI)]), [di, ii, ui], [ref]))
+    # scatter-add on the narrow and wide element types (compare-and-swap paths on the device); small integers, so
+    # that every partial sum is exact whatever order the duplicates arrive in
+    for dt_name, npdt in (('BFLOAT16', np.float32), ('INT8', np.int8), ('FLOAT64', np.float64), ('INT64', np.int64), ('FLOAT16', np.float16)):
+        base = r.integers(-3, 4, (5, 7)).astype(npdt)
+        upd = r.integers(-2, 3, (9, 7)).astype(npdt)
+        idx = r.integers(0, 5, (9,)).astype(np.int32)
+        Dd, Ii, Uu = (E.Placeholder(getattr(E.DType, dt_name), [5, 7]), E.Placeholder(E.DType.INT32, [9]),
+                      E.Placeholder(getattr(E.DType, dt_name), [9, 7]))
+        want = base.astype(np.float64).copy()
+        np.add.at(want, idx, upd.astype(np.float64))
+        out.append(('scatter_add_' + dt_name.lower(), E.Program('p', [Dd, Ii, Uu], [E.scatter(Dd, Ii, Uu)]), [base, idx, upd],
+                    [want.astype(npdt)]))
+    # a line longer than the device stages in LDS
+    long_line = r.integers(0, 50, (2, 9000)).astype(np.int32)
+    LL = E.Placeholder(E.DType.INT32, [2, 9000])
+    out.append(('argsort_long_line', E.Program('p', [LL], [E.argsort(LL, 1)]), [long_line],
+                [np.argsort(long_line, axis=1, kind='stable').astype(np.int32)]))
     return out, (D, SI, SU, d, si, su)
 
 
