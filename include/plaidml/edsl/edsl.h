@@ -455,6 +455,15 @@ enum class GatherMode : uint64_t { NORMAL, ND };
 enum class OutOfBoundsMode : uint64_t { GATHER_EDGE_PADDED_INPUT, RETURN_ZERO };
 enum class ScatterMode : uint64_t { NORMAL, UPDATE_SLICE, UPDATE_ELT, UPDATE_ND };
 
+// dims values in [0, 1) drawn from the three-word state, and the state advanced past them
+// (plaidml/edsl/edsl.h:971-979, pmlc/rt/prng.cc)
+inline std::pair<Tensor, Tensor> prng(const Tensor& state, const std::vector<int64_t>& dims) {
+  TensorVec args = {state};
+  for (int64_t d : dims) args.emplace_back(TensorDim(d));
+  Tensor R = intrinsicCall("prng", args);
+  return std::make_pair(R.element(0), R.element(1));
+}
+
 // the nine-argument gather intrinsic; `gather` below and op::gatherND fill it in
 class gatherBuilder {
  public:

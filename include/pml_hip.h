@@ -385,6 +385,12 @@ typedef struct {
 } pml_hip_argsort_desc;
 int pml_hip_argsort(const pml_hip_argsort_desc* desc, const void* tensor, void* out, pml_hip_stream s);
 
+/* prng: the three-component Tausworthe generator of the reference runtime (pmlc/rt/prng.cc:8-44).  `state` holds
+ * three uint32 words; value i is (s0 ^ s1 ^ s2) / 2^32 of the state after i steps, `new_state` the state after
+ * `count` steps.  Either output may be null.  The recurrences are linear over GF(2), so a thread reaches the start
+ * of its run of values by applying precomputed powers of the step matrix instead of stepping from the beginning. */
+int pml_hip_prng(const void* state, int64_t count, void* values, void* new_state, pml_hip_stream s);
+
 /* ---- any contraction ---------------------------------------------------------
  * The loop-nest form a contraction takes after bounds computation: the
  * `affine.parallel` + `pxa.load` + `pxa.reduce` nest of

@@ -644,6 +644,30 @@ OOB_EDGE_PADDED_INPUT, OOB_RETURN_ZERO = range(2)
 SCATTER_NORMAL, SCATTER_UPDATE_SLICE, SCATTER_UPDATE_ELT, SCATTER_UPDATE_ND = range(4)
 
 
+def prng(state, dims):
+    """The reference runtime's generator, pmlc/rt/prng.cc:8-44: value i is (s0 ^ s1 ^ s2) / 2^32 (float32) of the
+    three-word state after i steps of three independent Tausworthe recurrences; returns (values, advanced state)."""
+    state = _literal(state)
+    if state.dt != DType.UINT32 or int(np.prod(state.shape)) != 3:
+        raise ValueError("'prng' needs a state of three ui32 words")
+    shape = [int(d) for d in dims]
+    vals = Tensor('special', DType.FLOAT32, shape, (state,), {'fn': 'prng', 'part': 0})
+    new_state = Tensor('special', DType.UINT32, state.shape, (state,), {'fn': 'prng', 'part': 1, 'count': int(np.prod(shape))})
+    return vals, new_state
+
+
+def _eval_prng(state, count):
+    M = 0xFFFFFFFF
+    s0, s1, s2 = (int(v) for v in np.asarray(state).reshape(-1))
+    out = np.empty(count, np.float32)
+    for i in range(count):
+        out[i] = np.float32((s0 ^ s1 ^ s2) / 4294967296.0)
+        s0 = (((s0 & 4294967294) << 12) & M) ^ ((((s0 << 13) & M) ^ s0) >> 19)
+        s1 = (((s1 & 4294967288) << 4) & M) ^ ((((s1 << 2) & M) ^ s1) >> 25)
+        s2 = (((s2 & 4294967280) << 17) & M) ^ ((((s2 << 3) & M) ^ s2) >> 11)
+    return out, np.array([s0, s1, s2], np.uint32)
+
+
 def argsort(x, axis=-1, direction=SORT_ASC):
     """Shape rule pmlc/ast/ast_ops.cc:41-60: si32 positions, the input's shape."""
     x = _literal(x)
@@ -1172,7 +1196,10 @@ def evaluate(outputs, feeds):
         elif k == 'special':
             fn = n.attrs['fn']
             vals = [np.asarray(ev(a)) for a in n.args]
-            if fn == 'argsort':
+            if fn == 'prng':
+                count = int(np.prod(n.shape)) if n.attrs['part'] == 0 else n.attrs['count']
+                v = _eval_prng(vals[0], count)[n.attrs['part']]
+            elif fn == 'argsort':
                 v = _eval_argsort(vals[0], n.attrs['axis'], n.attrs['direction'])
             elif fn == 'gather':
                 v = _eval_gather(vals[0], vals[1], n.attrs, n.args[0].dt, n.args[1].dt)

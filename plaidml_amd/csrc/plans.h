@@ -105,6 +105,7 @@ hipError_t gather_launch(const pml_hip_gather_desc& d, const void* tensor, const
 hipError_t scatter_launch(const pml_hip_scatter_desc& d, const void* data, const void* indices, const void* updates, void* out,
                           hipStream_t s);
 hipError_t argsort_launch(const pml_hip_argsort_desc& d, const void* tensor, void* out, hipStream_t s);
+hipError_t prng_launch(const void* state, int64_t count, void* values, void* new_state, hipStream_t s);
 
 // window kernels (window.hip)
 struct DwconvArgs {

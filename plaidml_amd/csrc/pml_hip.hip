@@ -979,6 +979,13 @@ int pml_hip_scatter(const pml_hip_scatter_desc* d, const void* data, const void*
   return check(scatter_launch(*d, data, indices, updates, out, (hipStream_t)s), "scatter_launch");
 }
 
+int pml_hip_prng(const void* state, int64_t count, void* values, void* new_state, pml_hip_stream s) {
+  if (!state) return fail("prng: null state");
+  if (count < 0) return fail("prng: negative count");
+  if (!values && !new_state) return 0;
+  return check(prng_launch(state, count, values, new_state, (hipStream_t)s), "prng_launch");
+}
+
 int pml_hip_argsort(const pml_hip_argsort_desc* d, const void* tensor, void* out, pml_hip_stream s) {
   if (!d || !tensor || !out) return fail("argsort: null argument");
   if (d->rank < 1 || d->rank > PML_HIP_MAX_SPECIAL_RANK) return fail("argsort: rank out of range");

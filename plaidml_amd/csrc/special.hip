@@ -5,6 +5,7 @@
 // workgroup per sorted line (argsort).
 #include <hip/hip_runtime.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "device_common.h"
@@ -342,7 +343,101 @@ __global__ __launch_bounds__(256) void argsort_kernel(pml_hip_argsort_desc d, co
   }
 }
 
+// ---- prng -----------------------------------------------------------------------------------------------
+// One step of the three recurrences (pmlc/rt/prng.cc:31-37).  Each is linear over GF(2): masks, shifts, XORs.
+__host__ __device__ inline uint32_t taus_step(int c, uint32_t s) {
+  switch (c) {
+    case 0: return ((s & 4294967294u) << 12) ^ (((s << 13) ^ s) >> 19);
+    case 1: return ((s & 4294967288u) << 4) ^ (((s << 2) ^ s) >> 25);
+    default: return ((s & 4294967280u) << 17) ^ (((s << 3) ^ s) >> 11);
+  }
+}
+
+// jump[c][j] is the matrix of 2^j steps of component c, stored by columns: column b = image of bit b
+struct JumpTable {
+  uint32_t col[3][40][32];
+};
+__device__ JumpTable g_jump;
+
+__device__ inline uint32_t apply_jump(const uint32_t* cols, uint32_t x) {
+  uint32_t r = 0;
+  for (int b = 0; b < 32; ++b)
+    if ((x >> b) & 1u) r ^= cols[b];
+  return r;
+}
+
+// the state after `n` steps from `s`
+__device__ inline uint32_t jump_ahead(int c, uint32_t s, uint64_t n) {
+  for (int j = 0; j < 40 && n; ++j, n >>= 1)
+    if (n & 1) s = apply_jump(g_jump.col[c][j], s);
+  return s;
+}
+
+constexpr int kPrngRun = 64;  // consecutive values per thread
+
+__global__ __launch_bounds__(256) void prng_kernel(const uint32_t* state, int64_t count, float* values, uint32_t* new_state) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t first = t * kPrngRun;
+  if (values && first < count) {
+    uint32_t s0 = jump_ahead(0, state[0], (uint64_t)first), s1 = jump_ahead(1, state[1], (uint64_t)first),
+             s2 = jump_ahead(2, state[2], (uint64_t)first);
+    const int64_t last = first + kPrngRun < count ? first + kPrngRun : count;
+    for (int64_t i = first; i < last; ++i) {
+      values[i] = (float)((double)(s0 ^ s1 ^ s2) / 4294967296.0);
+      s0 = taus_step(0, s0);
+      s1 = taus_step(1, s1);
+      s2 = taus_step(2, s2);
+    }
+  }
+  if (new_state && t == 0) {
+    const uint32_t in0 = state[0], in1 = state[1], in2 = state[2];  // read before writing: the two may alias
+    new_state[0] = jump_ahead(0, in0, (uint64_t)count);
+    new_state[1] = jump_ahead(1, in1, (uint64_t)count);
+    new_state[2] = jump_ahead(2, in2, (uint64_t)count);
+  }
+}
+
 }  // namespace
+
+hipError_t prng_launch(const void* state, int64_t count, void* values, void* new_state, hipStream_t s) {
+  if (count >= (int64_t{1} << 40)) return hipErrorInvalidValue;
+  // the table depends on nothing but the recurrences: built on the host once and uploaded to each device on first use
+  static JumpTable table;
+  static bool built = false;
+  static bool uploaded[64] = {false};
+  static std::mutex mu;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!built) {
+      for (int c = 0; c < 3; ++c) {
+        for (int b = 0; b < 32; ++b) table.col[c][0][b] = taus_step(c, 1u << b);
+        for (int j = 1; j < 40; ++j)
+          for (int b = 0; b < 32; ++b) {
+            // (M^2) e_b = M (M e_b)
+            uint32_t x = table.col[c][j - 1][b], r = 0;
+            for (int k = 0; k < 32; ++k)
+              if ((x >> k) & 1u) r ^= table.col[c][j - 1][k];
+            table.col[c][j][b] = r;
+          }
+      }
+      built = true;
+    }
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    if (!uploaded[dev]) {
+      e = hipMemcpyToSymbol(HIP_SYMBOL(g_jump), &table, sizeof(table));
+      if (e != hipSuccess) return e;
+      uploaded[dev] = true;
+    }
+  }
+  const int64_t threads = values ? (count + kPrngRun - 1) / kPrngRun : 1;
+  const int64_t blocks = threads > 0 ? (threads + 255) / 256 : 1;
+  hipLaunchKernelGGL(prng_kernel, dim3((unsigned)(blocks > 0 ? blocks : 1)), dim3(256), 0, s, (const uint32_t*)state, count,
+                     (float*)values, (uint32_t*)new_state);
+  return hipGetLastError();
+}
 
 hipError_t gather_launch(const pml_hip_gather_desc& d, const void* tensor, const void* indices, void* out, hipStream_t s) {
   GatherGeom g{};

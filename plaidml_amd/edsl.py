@@ -753,6 +753,12 @@ def _float(v):
     return _const(call('plaidml_expr_float', float(v)))
 
 
+def prng(state, dims):
+    """(values of shape dims in [0, 1), advanced state): plaidml/edsl/edsl.h:971-979."""
+    r = intrinsic('prng', state, *[TensorDim(int(d)) for d in dims])
+    return (Tensor(ptr=call('plaidml_expr_element', r.as_ptr(), 0)), Tensor(ptr=call('plaidml_expr_element', r.as_ptr(), 1)))
+
+
 def argsort(x, axis=-1, direction=SORT_ASC):
     return intrinsic('argsort', x, _int(axis), _int(direction))
 

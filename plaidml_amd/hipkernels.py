@@ -32,7 +32,7 @@ EXPORTS = [
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
     'pml_hip_plan_describe', 'pml_hip_struct_size', 'pml_hip_gemm_pack_b', 'pml_hip_conv2d_pack_filter',
-    'pml_hip_gather', 'pml_hip_scatter', 'pml_hip_argsort',
+    'pml_hip_gather', 'pml_hip_scatter', 'pml_hip_argsort', 'pml_hip_prng',
 ]
 
 i32, i64, f64 = ctypes.c_int32, ctypes.c_int64, ctypes.c_double
@@ -159,6 +159,7 @@ def lib():
         L.pml_hip_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp]
         L.pml_hip_scatter.argtypes = [ctypes.POINTER(ScatterDesc), vp, vp, vp, vp, vp]
         L.pml_hip_argsort.argtypes = [ctypes.POINTER(ArgsortDesc), vp, vp, vp]
+        L.pml_hip_prng.argtypes = [vp, ctypes.c_int64, vp, vp, vp]
         L.pml_hip_conv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
         _lib = L
     return _lib

@@ -92,7 +92,7 @@ bool isKnownIntrinsic(const std::string& fn) {
       "log",     "sqrt",    "tanh",    "floor",    "ceil",     "round",   "pow",     "sin",     "cos",    "tan",
       "sinh",    "cosh",    "erf",     "select",   "index",    "reshape", "shape",   "bit_and", "bit_or", "bit_xor",
       "bit_not", "bit_shl", "bit_shr", "acos",     "asin",     "atan",    "acosh",   "asinh",   "atanh",
-      "gather",  "scatter", "argsort"};
+      "gather",  "scatter", "argsort", "prng"};
   return s.count(fn) != 0 || isCompareOp(fn) || isLogicalOp(fn);
 }
 
@@ -206,6 +206,12 @@ TensorShape Evaluator::computeShape(const ExprNodePtr& node) {
       return TensorShape(node->dtype, s.sizes);
     }
     case ExprNode::Element:
+      // prng is the one intrinsic with two results: the values and the advanced state (pmlc/ast/ast_ops.cc:180-195)
+      if (node->expr && node->expr->kind == ExprNode::Intrinsic && node->expr->op == "prng") {
+        if (node->ordinal == 0) return getShape(node->expr);
+        if (node->ordinal == 1) return getShape(node->expr->operands.at(0));
+        throw std::runtime_error("'prng' has two results");
+      }
       if (node->ordinal != 0) throw std::runtime_error("only single-result expressions are supported");
       return getShape(node->expr);
     case ExprNode::Pragma:
@@ -249,6 +255,18 @@ TensorShape Evaluator::computeShape(const ExprNodePtr& node) {
           int64_t v;
           if (!integerOperand(this, node->operands[i], &v))
             throw std::runtime_error("Additional parameters to 'reshape' must be integers or TensorDims.");
+          ret.sizes.push_back(v);
+        }
+        return ret;
+      }
+      if (fn == "prng") {
+        // the shape of the first result; operands: the state, then the dims of the values
+        if (node->operands.empty()) throw std::runtime_error("'prng' requires at least one argument.");
+        TensorShape ret(DataType::f32);
+        for (size_t i = 1; i < node->operands.size(); ++i) {
+          int64_t v;
+          if (!integerOperand(this, node->operands[i], &v))
+            throw std::runtime_error("'prng' has invalid operands, dims must be tensor dimensions");
           ret.sizes.push_back(v);
         }
         return ret;

@@ -633,7 +633,14 @@ class Planner {
     Step s;
     s.c = bufferFor(op.result);
     for (const ValuePtr& v : op.operands) s.operands.push_back(bufferFor(v));
-    if (op.fn == "gather") {
+    if (op.fn == "prng_values" || op.fn == "prng_state") {
+      s.kind = Step::Prng;
+      s.prng_count = param(0);
+      s.prng_state = op.fn == "prng_state";
+      s.text = std::string("prng ") + (s.prng_state ? "state after " : "values x ") + std::to_string(s.prng_count) + " -> " +
+               op.result->shape.str();
+      s.bytes = static_cast<double>(op.result->shape.getByteSize());
+    } else if (op.fn == "gather") {
       s.kind = Step::Gather;
       auto& d = s.gat;
       d.dtype = hipType(op.operands[0]->shape.elementType);

@@ -26,7 +26,7 @@ struct BufferInfo {
 };
 
 struct Step {
-  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy, Gather, Scatter, ArgSort } kind = Copy;
+  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy, Gather, Scatter, ArgSort, Prng } kind = Copy;
   std::string text;  // one line for the plan dump
   // descriptors (only the one matching `kind` is meaningful)
   pml_hip_gemm_desc gemm{};
@@ -39,6 +39,8 @@ struct Step {
   pml_hip_gather_desc gat{};
   pml_hip_scatter_desc sca{};
   pml_hip_argsort_desc srt{};
+  int64_t prng_count = 0;   // Prng: values drawn
+  bool prng_state = false;  //       the step yields the advanced state instead of the values
   int index_axis = 0;
   std::vector<int64_t> index_sizes;
   // buffer ids (-1 = none) and element offsets applied to the base pointers

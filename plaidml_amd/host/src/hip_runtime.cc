@@ -129,6 +129,7 @@ class HipExecutable final : public Executable {
       case Step::Gather:
       case Step::Scatter:
       case Step::ArgSort:
+      case Step::Prng:
       case Step::Copy: return;
     }
     if (!h) throw std::runtime_error("hip dispatch failed for '" + s.text + "': " + pml_hip_last_error());
@@ -190,6 +191,10 @@ class HipExecutable final : public Executable {
         break;
       case Step::ArgSort:
         hipCheck(pml_hip_argsort(&s.srt, operands[0], ptr(s.c), nullptr), s.text.c_str());
+        break;
+      case Step::Prng:
+        hipCheck(pml_hip_prng(operands[0], s.prng_count, s.prng_state ? nullptr : ptr(s.c), s.prng_state ? ptr(s.c) : nullptr, nullptr),
+                 s.text.c_str());
         break;
     }
   }

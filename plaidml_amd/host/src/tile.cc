@@ -254,6 +254,24 @@ struct Builder {
         return v;
       }
       case ExprNode::Element:
+        if (node->expr && node->expr->kind == ExprNode::Intrinsic && node->expr->op == "prng") {
+          // the two results of prng are functions of (state, number of values) alone: each becomes an operation
+          // of its own, "prng_values" and "prng_state"
+          const ExprNodePtr& call = node->expr;
+          TensorShape values = ev.getShape(call);
+          ValuePtr state = visit(call->operands.at(0));
+          if (state->shape.elementType != DataType::ui32 || state->shape.elements() != 3)
+            throw std::runtime_error("'prng' needs a state of three ui32 words");
+          Op op;
+          op.kind = Op::Special;
+          op.fn = node->ordinal == 0 ? "prng_values" : "prng_state";
+          op.operands = {state};
+          op.params = {static_cast<double>(values.elements())};
+          op.result = newValue(Value::Temp, ev.getShape(node), call->name);
+          program->ops.push_back(op);
+          return op.result;
+        }
+        return visit(node->expr);
       case ExprNode::Pragma:
         return visit(node->expr);
       case ExprNode::Cast: {
@@ -320,6 +338,8 @@ struct Builder {
           ValuePtr v = newValue(Value::Constant, shape, "shape");
           v->constant = buf;
           return v;
+        } else if (node->op == "prng") {
+          throw std::runtime_error("'prng' yields two results: use element(0) for the values and element(1) for the new state");
         } else if (node->op == "gather" || node->op == "scatter" || node->op == "argsort") {
           // tensor operands first, then constants (plaidml/edsl/edsl.h:809-811, 1036-1066, 1645-1690)
           op.kind = Op::Special;

@@ -145,3 +145,46 @@ def test_hip_index_outside_the_tensor_reads_zero_and_drops_updates():
                  [np.arange(1, 5, dtype=np.float32), np.array([2, 9, -1], np.int32), np.array([10, 20, 30], np.float32)], target='hip')
     np.testing.assert_array_equal(g, [3, 0, 0])
     np.testing.assert_array_equal(s, [1, 2, 13, 4])
+
+
+# CppEdsl.Prng, plaidml/edsl/tests/edsl_test.cc:1138-1160: state {5, 6, 7}, six values, the state after them
+PRNG_VALUES = np.array([9.31323e-10, 3.8147e-06, 0.0156251, 0.000244171, 0.000125885, 0.515625], np.float32).reshape(2, 3)
+PRNG_STATE = np.array([1052804, 0, 0], np.uint32).reshape(1, 3)
+
+
+def _prng_program(E, dims):
+    S = E.Placeholder(E.DType.UINT32, [1, 3])
+    vals, new_state = E.prng(S, dims)
+    return E.Program('prng', [S], [vals, new_state])
+
+
+def test_oracle_prng_reproduces_reference_answers():
+    vals, st = OE.run(_prng_program(OE, [2, 3]), [np.array([[5, 6, 7]], np.uint32)])
+    np.testing.assert_allclose(vals, PRNG_VALUES, rtol=1e-5)
+    np.testing.assert_array_equal(st, PRNG_STATE)
+
+
+def test_oracle_prng_streams_compose():
+    """Drawing n values and then m from the returned state equals drawing n + m at once."""
+    s = np.array([[123456789, 362436069, 521288629]], np.uint32)
+    a, sa = OE.run(_prng_program(OE, [100]), [s])
+    b, sb = OE.run(_prng_program(OE, [57]), [sa])
+    c, sc = OE.run(_prng_program(OE, [157]), [s])
+    np.testing.assert_array_equal(np.concatenate([a, b]), c)
+    np.testing.assert_array_equal(sb, sc)
+    assert 0.0 <= c.min() and c.max() <= 1.0   # a quotient just below 1 rounds to 1.0f, as in the reference
+    assert abs(c.mean() - 0.5) < 0.1
+
+
+@pytest.mark.gpu
+def test_hip_prng_matches_reference_answers_and_oracle():
+    from plaidml_amd import edsl as E
+    vals, st = E.run(_prng_program(E, [2, 3]), [np.array([[5, 6, 7]], np.uint32)], target='hip')
+    np.testing.assert_allclose(vals, PRNG_VALUES, rtol=1e-5)
+    np.testing.assert_array_equal(st, PRNG_STATE)
+    # a count that spans many threads and is not a multiple of a thread's run: bit-exact against the serial oracle
+    s = np.array([[123456789, 362436069, 521288629]], np.uint32)
+    got, gst = E.run(_prng_program(E, [7, 1001]), [s], target='hip')
+    want, wst = OE.run(_prng_program(OE, [7, 1001]), [s])
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(gst, wst)
