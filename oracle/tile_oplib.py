@@ -3,15 +3,25 @@
 Restates, on top of oracle/tile_oracle.py, the contractions that the reference
 op library emits for the operations on the hot path (plaidml/op/lib/ops.cc):
 
-  convolution   :879-1467 (NXC input, XCK filter; strides, dilations, autopad,
-                 explicit padding, group layouts NONE and IN_C with DEPTHWISE
-                 autogrouping), padding rule :347-382
+  convolution   :879-1467 with the validation of :671-877 (NXC / NCX data, XCK / KCX /
+                 XGCK / GKCX filters; strides, dilations, data dilations, autopad,
+                 explicit padding; the four group layouts and autogroup modes; the
+                 DATA and FILTER derivative modes), padding rules :347-418
   pool          :2562-2703 (MAX / MIN / SUM / AVG, NXC)
   dot           :1512-1561
   mean          :1970-2003, sum / max via the same AggregationAxes :71-127
   relu          :2705-2728 (plain form only)
   softmax       :3049-3098 (last-axis form)
   argmax        :505-521
+  and, each cited where it is defined below: abs, all, any, binary_crossentropy,
+  broadcast, clip, concatenate, cumprod, cumsum, elu, explicit_padding, flip,
+  gatherND, hard_sigmoid, image_resize, l2norm, lrn, mvn, prod, reorg_yolo, repeat,
+  reshape, scale_gradient, sigmoid, slice, sort, spatial_padding, square, squeeze,
+  tile, topk, transpose, unsqueeze, variance
+
+Pinned by tests/test_oplib_ops.py, tests/test_conv_general.py and the op-level
+cases of tests/test_oracle_golden.py (numpy closed forms, the exact cases of
+plaidml/op/op_test.cc, direct numpy evaluations of the definitions).
 
 Nothing in the shipped package imports this module.
 """

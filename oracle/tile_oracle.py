@@ -47,6 +47,13 @@ Pinned by tests/test_oracle_golden.py against these reference-held vectors:
   BroadcastCmp / Add known answers of edsl_test.cc; convolution and pooling are
   additionally checked against torch.nn.functional on the CPU (a library routine,
   not the reference) and brute-force enumeration.
+By tests/test_intrinsics.py against the answers the reference's tests hold for every elementwise intrinsic
+(BitAnd ... Tan, 31 cases of plaidml/edsl/tests/edsl_test.cc:180-1873), by tests/test_special_ops.py against
+its Gather* / Scatter* / ArgSort* / Prng answers (26 + 1 cases, edsl_test.cc:1138-2572) plus numpy closed forms
+(np.take, np.interp, stable np.argsort, np.add.at), by tests/test_oplib_ops.py against numpy closed forms and the
+exact cases of plaidml/op/op_test.cc (Broadcast*, CumSumExclusive, ExplicitPadding*, ReorgYolo*, Sort) and the
+InterpolatedGatherND answers, and by tests/test_conv_general.py against a direct numpy evaluation of the general
+convolution and the adjoint identities of its two derivative modes.
 And by tests/test_golden_network.py against the stored fp32 output of the reference
 benchmark tool's toy_parallel_conv network (its own weights and input image; strided
 SAME convolutions 7x7 / 1x1 / 3x3, bias, ReLU, add: plaidbench/plaidbench/golden/
