@@ -382,6 +382,25 @@ void caseSpecialOps() {
   }
 }
 
+// CppEdsl.Lens, plaidml/edsl/tests/edsl_test.cc:2122-2162: a transposition written once for "MN" and read through a
+// lens gives the same answer whichever of the two orders names the tensor's own layout
+Tensor TransposeThroughLens(Tensor I, const std::string& layout) {
+  TensorLens lens(layout, "MN");
+  I = I.use(lens);
+  TensorDim M, N;
+  TensorIndex i, j;
+  I.bind_dims(M, N);
+  return Contraction(lens).outShape(N, M).outAccess(j, i).assign(I(i, j));
+}
+
+void caseLens() {
+  for (const char* layout : {"MN", "NM"}) {
+    auto I = Placeholder(DType::FLOAT32, {2, 3});
+    auto out = run(buildProgram("transpose", {I}, {TransposeThroughLens(I, layout)}), {makeBuffer<float>(DType::FLOAT32, {2, 3}, {1, 2, 3, 4, 5, 6})});
+    expectEq<float>(std::string("lens_transpose_") + layout, readBuffer<float>(out[0]), {1, 4, 2, 5, 3, 6});
+  }
+}
+
 void caseErrors() {
   auto A = Placeholder(DType::FLOAT32, {4, 4});
   auto program = buildProgram("ident", {A}, {A + 1.0});
@@ -420,6 +439,7 @@ int main() {
     caseIntrinsics();
     caseOpBuilders();
     caseSpecialOps();
+    caseLens();
     caseErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAILED with exception: %s\n", e.what());

@@ -93,3 +93,20 @@ def test_hip_shape():
     assert out.dtype == np.int32
     np.testing.assert_array_equal(out, [2, 3])
     np.testing.assert_array_equal(scaled, [1.0, 1.5])
+
+
+import reference_cases as RC
+
+
+@pytest.mark.parametrize('name', sorted(RC.CASES))
+def test_oracle_small_program_answers(name):
+    RC.run_case(name, OE)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('target', ['hip', 'hip{specialise=0,fuse=0}'])
+@pytest.mark.parametrize('name', sorted(RC.CASES))
+def test_hip_small_program_answers(name, target):
+    from plaidml_amd import edsl as E
+    print('small program', name, target, flush=True)
+    RC.run_case(name, E, target=target)
