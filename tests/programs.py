@@ -141,6 +141,18 @@ def bits_and_truth(E, op):
     return E.Program('bits', [A, B, Cc, F], [X, Y, Z, L]), [a, b, r.integers(0, 8, (6, 1)).astype(np.uint8), f], EXACT
 
 
+def dot_f16_acc_f32(E, op, M=8, N=32, K=16):
+    """CppEdsl.DotF16_AccF32, plaidml/edsl/tests/edsl_test.cc:500-545: half inputs widened, summed in fp32, narrowed
+    (the reference compares with tolerance 1e-2 against the same fp32 loop)."""
+    A = E.Placeholder(E.DType.FLOAT16, [M, K])
+    B = E.Placeholder(E.DType.FLOAT16, [K, N])
+    i, j, k = E.TensorIndexes(3)
+    C32 = E.Contraction().outShape(M, N).outAccess(i, j).sum(E.cast(A, E.DType.FLOAT32)[i, k] * E.cast(B, E.DType.FLOAT32)[k, j]).build()
+    r = _rng(2)
+    return E.Program('dot_f16_acc_f32', [A, B], [E.cast(C32, E.DType.FLOAT16)]), [
+        r.standard_normal((M, K)).astype(np.float16), r.standard_normal((K, N)).astype(np.float16)], BF16
+
+
 def u64_add(E, op):
     """CppEdsl.Add, plaidml/edsl/tests/edsl_test.cc:335-374 (64-bit integer elementwise)."""
     A = E.Placeholder(E.DType.UINT64, [3, 3])
@@ -307,6 +319,7 @@ ALL = {
     'use_default': use_default,
     'eltwise_mix': eltwise_mix,
     'libm_tail_f32': libm_tail_f32,
+    'dot_f16_acc_f32': dot_f16_acc_f32,
     'bits_and_truth': bits_and_truth,
     'u64_add': u64_add,
     'higher_precision_constants': higher_precision_constants,
