@@ -19,11 +19,12 @@ def _he(rng, shape, fan_in):
 
 
 def build(E, op, batch=128, image=224, classes=1000, dtype_name='BFLOAT16', seed=12, base=64, stages=None,
-          round_fn=None):
+          round_fn=None, with_logits=False):
     """Returns (program, weights) where weights is the list of host arrays in creation order.
 
     base scales every width (64 = the real network); stages overrides the (blocks, width) list;
-    round_fn maps fp32 arrays to the values representable in dtype_name (identity for FLOAT32).
+    round_fn maps fp32 arrays to the values representable in dtype_name (identity for FLOAT32);
+    with_logits adds the values before the softmax as a second program output.
     """
     dt = getattr(E.DType, dtype_name)
     round_fn = round_fn or (lambda a: a)
@@ -69,5 +70,5 @@ def build(E, op, batch=128, image=224, classes=1000, dtype_name='BFLOAT16', seed
     logits = op.dot(x, Wd) + bd
     flops[0] += 2.0 * batch * ci * classes
     probs = op.softmax(logits, axis=1)
-    program = E.Program('resnet50_v1_5', [X], [probs])
+    program = E.Program('resnet50_v1_5', [X], [probs, logits] if with_logits else [probs])
     return program, weights, flops[0]
