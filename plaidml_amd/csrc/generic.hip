@@ -275,6 +275,138 @@ __global__ __launch_bounds__(256) void contract_coop_kernel(ContractArgs a, int6
   }
 }
 
+// Reductions along memory: one source, no combination, every access always in range, and the reduced
+// indices together walk a contiguous run of the source.  A group of `lanes` threads (one wavefront, or
+// the whole workgroup for long runs) owns one output point, reads its run with consecutive lanes on
+// consecutive elements, and folds the partial results with cross-lane shuffles.  What a softmax's row
+// max / row sum, a mean or a norm over the innermost axes turn into.
+struct RowsArgs {
+  int64_t out_stride[PML_HIP_MAX_IDX];  // of each output index, in elements of the output
+  int64_t src_stride[PML_HIP_MAX_IDX];  // of each output index, in elements of the source
+  int64_t range[PML_HIP_MAX_IDX];
+  int64_t out_base, src_base;           // offsets of the box's lowest corner
+  int64_t cols;                         // length of the contiguous run
+  int32_t lanes;                        // 64 or 256
+};
+
+// DT / AGG fix the element type (source and result alike) and the aggregation at compile time, which
+// folds every type switch away: a reduction launched once per network pass finds its code nowhere in
+// the caches, and what it costs is then the length of the code it has to fetch.  DT = 0: both from the
+// descriptor.
+template <typename FT, typename IT, int DT, int AGG>
+__global__ __launch_bounds__(256) void contract_rows_kernel(ContractArgs a, RowsArgs ra) {
+  const pml_hip_contract_desc& d = a.d;
+  __shared__ FT part_f[4];
+  __shared__ IT part_i[4];
+  const int per_block = 256 / ra.lanes;
+  const int64_t row = (int64_t)blockIdx.x * per_block + (ra.lanes == 64 ? (int)(threadIdx.x >> 6) : 0);
+  const bool live = row < d.out_elems;  // uniform over a wavefront
+  const int lane = ra.lanes == 64 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
+  int64_t out_off = ra.out_base, src_off = ra.src_base;
+  {
+    int64_t t = live ? row : 0;
+    for (int v = d.n_out_idx - 1; v >= 0; --v) {
+      const int64_t c = t % ra.range[v];
+      t /= ra.range[v];
+      out_off += c * ra.out_stride[v];
+      src_off += c * ra.src_stride[v];
+    }
+  }
+  const int dt = DT ? DT : d.dtype, sd = DT ? DT : d.src_dtype[0], agg = DT ? AGG : d.agg;
+  const int acc_dt = (dt == PML_HIP_BF16 || dt == PML_HIP_F16) ? PML_HIP_F32 : dt;
+  const bool widen = !dt_is_float(sd) && !dt_is_float(acc_dt) && sd != PML_HIP_BOOL && dt_size(sd) < dt_size(acc_dt);
+  Scalar<FT, IT> acc;
+  acc.f = dt_is_float(dt) ? (FT)d.identity_f : (FT)0;
+  acc.i = dt_is_float(dt) ? (IT)0 : wrap_int_to<IT>(dt, (IT)d.identity_i);
+  if (live) {
+    constexpr int U = 8;  // loads in flight per lane: a row is short, so its latency is what costs
+    for (int64_t j0 = lane; j0 < ra.cols; j0 += (int64_t)U * ra.lanes) {
+      Scalar<FT, IT> raw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t j = j0 + (int64_t)u * ra.lanes;
+        if (j < ra.cols) raw[u] = load_scalar<FT, IT>(a.srcs[0], src_off + j, sd);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (j0 + (int64_t)u * ra.lanes >= ra.cols) break;
+        Scalar<FT, IT> x = raw[u];
+        if (widen)
+          x.i = raw[u].i & (IT)((((uint64_t)1) << (dt_size(sd) * 8)) - 1);
+        else
+          x = convert_scalar<FT, IT>(raw[u], sd, acc_dt);
+        aggregate<FT, IT>(agg, acc_dt, acc, x);
+      }
+    }
+  }
+  for (int w = 32; w > 0; w >>= 1) {
+    Scalar<FT, IT> y;
+    y.f = __shfl_xor(acc.f, w, 64);
+    y.i = __shfl_xor(acc.i, w, 64);
+    aggregate<FT, IT>(agg, acc_dt, acc, y);
+  }
+  if (ra.lanes == 256) {
+    if ((threadIdx.x & 63) == 0) {
+      part_f[threadIdx.x >> 6] = acc.f;
+      part_i[threadIdx.x >> 6] = acc.i;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < 4; ++w) {
+        Scalar<FT, IT> y;
+        y.f = part_f[w], y.i = part_i[w];
+        aggregate<FT, IT>(agg, acc_dt, acc, y);
+      }
+    }
+  }
+  if (live && lane == 0) {
+    if (d.has_init) {
+      Scalar<FT, IT> start = convert_scalar<FT, IT>(load_scalar<FT, IT>(a.out, out_off, dt), dt, acc_dt);
+      aggregate<FT, IT>(agg, acc_dt, start, acc);
+      acc = start;
+    }
+    store_scalar<FT, IT>(a.out, out_off, dt, convert_scalar<FT, IT>(acc, acc_dt, dt));
+  }
+}
+
+// Fills `ra` if the contraction is a reduction along memory in the sense above.
+bool rows_form(const pml_hip_contract_desc& d, RowsArgs* ra) {
+  if (d.combo != PML_HIP_COMBO_NONE || d.n_src != 1 || d.agg == PML_HIP_AGG_ASSIGN) return false;
+  if (d.n_idx <= d.n_out_idx || d.out_elems <= 0) return false;
+  int64_t os[PML_HIP_MAX_IDX] = {}, ss[PML_HIP_MAX_IDX] = {};
+  ra->out_base = ra->src_base = 0;
+  for (int v = 0; v < d.n_idx; ++v)
+    if (d.hi[v] < d.lo[v]) return false;
+  for (int f = 0; f < d.n_forms; ++f) {
+    const pml_hip_form& fm = d.forms[f];
+    if (fm.den != 1 || (fm.operand != 0 && fm.operand != 1)) return false;
+    int64_t lo = fm.c0, hi = fm.c0;
+    for (int v = 0; v < d.n_idx; ++v) {
+      lo += (int64_t)fm.coef[v] * (fm.coef[v] >= 0 ? d.lo[v] : d.hi[v]);
+      hi += (int64_t)fm.coef[v] * (fm.coef[v] >= 0 ? d.hi[v] : d.lo[v]);
+    }
+    if (lo < 0 || hi >= fm.size) return false;
+    int64_t corner = fm.c0;
+    for (int v = 0; v < d.n_idx; ++v) {
+      corner += (int64_t)fm.coef[v] * d.lo[v];
+      (fm.operand == 0 ? os : ss)[v] += (int64_t)fm.coef[v] * fm.stride;
+    }
+    (fm.operand == 0 ? ra->out_base : ra->src_base) += corner * fm.stride;
+  }
+  int64_t run = 1;
+  for (int v = d.n_idx - 1; v >= d.n_out_idx; --v) {
+    if (os[v] != 0 || ss[v] != run) return false;
+    run *= d.hi[v] - d.lo[v] + 1;
+  }
+  for (int v = 0; v < d.n_out_idx; ++v) {
+    ra->out_stride[v] = os[v];
+    ra->src_stride[v] = ss[v];
+    ra->range[v] = d.hi[v] - d.lo[v] + 1;
+  }
+  ra->cols = run;
+  return true;
+}
+
 // ---------------------------------------------------------------------------
 // elementwise chain with N-d broadcasting
 // ---------------------------------------------------------------------------
@@ -342,6 +474,95 @@ __global__ __launch_bounds__(256) void eltwise_vec_kernel(EltwiseArgs a, int64_t
   }
 }
 
+// The same layout, for the chains most networks are made of: every step a plain arithmetic function
+// in the chain's own floating element type (DT: fp32 or bf16), no extra outputs.  The step's opcode is
+// decoded once per 16-byte vector, not once per element, and the kernel carries none of the rarely used
+// functions, so its code stays small enough to run from the instruction cache.
+__host__ __device__ inline bool short_chain_op(int opcode) {
+  switch (opcode) {
+    case PML_HIP_EPI_ADD: case PML_HIP_EPI_SUB: case PML_HIP_EPI_RSUB: case PML_HIP_EPI_MUL: case PML_HIP_EPI_DIV:
+    case PML_HIP_EPI_RDIV: case PML_HIP_EPI_MAX: case PML_HIP_EPI_MIN: case PML_HIP_EPI_RELU: case PML_HIP_EPI_NEG:
+    case PML_HIP_EPI_EXP: case PML_HIP_EPI_LOG: case PML_HIP_EPI_SQRT: case PML_HIP_EPI_TANH: case PML_HIP_EPI_MAX_GT:
+      return true;
+    default:
+      return false;
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void eltwise_short_kernel(EltwiseArgs a, int64_t inner, unsigned opnd_full_mask,
+                                                            unsigned opnd_vec_mask, unsigned opnd_row_mask) {
+  constexpr int ES = DT == PML_HIP_F32 ? 4 : 2;
+  constexpr int V = 16 / ES;
+  const pml_hip_eltwise_desc& d = a.d;
+  const int64_t n_vec = a.total / V;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_vec; g += stride) {
+    const int64_t e0 = g * V;
+    const int64_t c0 = e0 % inner;
+    i32x4_t raw = *(const i32x4_t*)((const unsigned char*)a.in + e0 * ES);
+    float x[V], y[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[e] = load_scalar<float, int>(&raw, e, DT).f;
+    for (int s = 0; s < d.tail.n_ops; ++s) {
+      const pml_hip_epi_op& op = d.tail.ops[s];
+      if (op.operand_kind == PML_HIP_OPND_TENSOR) {
+        const int q = op.operand;
+        const unsigned char* base = (const unsigned char*)a.operands[q];
+        if (((opnd_full_mask | opnd_vec_mask) >> q) & 1) {
+          const int64_t at = ((opnd_full_mask >> q) & 1) ? e0 : c0;
+          i32x4_t w = *(const i32x4_t*)(base + at * ES);
+#pragma unroll
+          for (int e = 0; e < V; ++e) y[e] = load_scalar<float, int>(&w, e, DT).f;
+        } else {
+          // one value for the whole tensor, or one per innermost line (a vector never crosses a line)
+          const float b = load_scalar<float, int>(base, ((opnd_row_mask >> q) & 1) ? e0 / inner : 0, DT).f;
+#pragma unroll
+          for (int e = 0; e < V; ++e) y[e] = b;
+        }
+      } else {
+        const float b = op.operand_kind == PML_HIP_OPND_IMM ? round_float_to<float>(DT, (float)op.imm) : 0.0f;
+#pragma unroll
+        for (int e = 0; e < V; ++e) y[e] = b;
+      }
+#define PML_EACH(EXPR)                   \
+  _Pragma("unroll") for (int e = 0; e < V; ++e) { \
+    const float p = x[e], q = y[e];      \
+    x[e] = round_float_to<float>(DT, EXPR); \
+  }                                      \
+  break;
+      switch (op.opcode) {
+        case PML_HIP_EPI_ADD: PML_EACH(p + q)
+        case PML_HIP_EPI_SUB: PML_EACH(p - q)
+        case PML_HIP_EPI_RSUB: PML_EACH(q - p)
+        case PML_HIP_EPI_MUL: PML_EACH(p * q)
+        case PML_HIP_EPI_DIV: PML_EACH(p / q)
+        case PML_HIP_EPI_RDIV: PML_EACH(q / p)
+        case PML_HIP_EPI_MAX: PML_EACH((p < q) ? q : p)
+        case PML_HIP_EPI_MIN: PML_EACH((p < q) ? p : q)
+        case PML_HIP_EPI_RELU: PML_EACH((p < 0.0f) ? 0.0f : p)
+        case PML_HIP_EPI_NEG: PML_EACH(-p)
+        case PML_HIP_EPI_EXP: PML_EACH(expf(p))
+        case PML_HIP_EPI_LOG: PML_EACH(logf(p))
+        case PML_HIP_EPI_SQRT: PML_EACH(sqrtf(p))
+        case PML_HIP_EPI_TANH: PML_EACH(tanhf(p))
+        case PML_HIP_EPI_MAX_GT: PML_EACH((p > q) ? p : q)
+        default: break;
+      }
+#undef PML_EACH
+    }
+    i32x4_t res;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      Scalar<float, int> v;
+      v.f = x[e];
+      v.i = 0;
+      store_scalar<float, int>(&res, e, DT, v);
+    }
+    *(i32x4_t*)((unsigned char*)a.out + e0 * ES) = res;
+  }
+}
+
 template <typename FT, typename IT>
 __global__ __launch_bounds__(256) void select_kernel(pml_hip_select_desc d, const void* c, const void* t, const void* f,
                                                      void* out, int64_t total) {
@@ -394,6 +615,31 @@ hipError_t contract_launch(const ContractArgs& a, hipStream_t s) {
   // too few outputs to fill the chip and a long reduction: one workgroup per output
   int64_t red_count = 1;
   for (int v = d.n_out_idx; v < d.n_idx; ++v) red_count *= d.hi[v] >= d.lo[v] ? d.hi[v] - d.lo[v] + 1 : 0;
+  RowsArgs ra;
+  if (!wide && red_count >= 64 && rows_form(d, &ra)) {
+    // a wavefront per output point; the whole workgroup when the points alone would not fill the chip
+    ra.lanes = (ra.cols >= 2048 && d.out_elems * 64 < (int64_t)256 * 1024) ? 256 : 64;
+    const int per_block = 256 / ra.lanes;
+    const int64_t nb = (d.out_elems + per_block - 1) / per_block;
+    if (nb <= 0x7fffffff) {
+      const dim3 grid((unsigned)nb), block(256);
+      const bool same = d.src_dtype[0] == d.dtype;
+#define PML_ROWS(DT, AGG)                                                                                   \
+  if (same && d.dtype == DT && d.agg == AGG) {                                                              \
+    hipLaunchKernelGGL((contract_rows_kernel<float, int, DT, AGG>), grid, block, 0, s, a, ra);              \
+    return hipGetLastError();                                                                               \
+  }
+      PML_ROWS(PML_HIP_BF16, PML_HIP_AGG_ADD)
+      PML_ROWS(PML_HIP_BF16, PML_HIP_AGG_MAX)
+      PML_ROWS(PML_HIP_BF16, PML_HIP_AGG_MIN)
+      PML_ROWS(PML_HIP_F32, PML_HIP_AGG_ADD)
+      PML_ROWS(PML_HIP_F32, PML_HIP_AGG_MAX)
+      PML_ROWS(PML_HIP_F32, PML_HIP_AGG_MIN)
+#undef PML_ROWS
+      hipLaunchKernelGGL((contract_rows_kernel<float, int, 0, 0>), grid, block, 0, s, a, ra);
+      return hipGetLastError();
+    }
+  }
   if (d.agg != PML_HIP_AGG_ASSIGN && d.out_elems <= 4096 && red_count >= 512) {
     if (wide)
       hipLaunchKernelGGL((contract_coop_kernel<double, int64_t>), dim3((unsigned)d.out_elems), dim3(256), 0, s, a, red_count);
@@ -419,7 +665,7 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
   const int es = dt_size(d.in_dtype);
   bool vec_ok = (es == 2 || es == 4) && dt_size(d.out_dtype) == es && d.rank >= 1;
   int64_t inner = d.rank >= 1 ? d.sizes[d.rank - 1] : 1;
-  unsigned full_mask = 0, vec_mask = 0;
+  unsigned full_mask = 0, vec_mask = 0, row_mask = 0;
   if (vec_ok) {
     int64_t st = 1;
     for (int r = d.rank - 1; r >= 0; --r) {
@@ -427,7 +673,7 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
       st *= d.sizes[r];
     }
     for (int q = 0; q < d.tail.n_operands && vec_ok; ++q) {
-      bool full = true, vec = true, scal = true;
+      bool full = true, vec = true, scal = true, row = true;
       int64_t st2 = 1;
       for (int r = d.rank - 1; r >= 0; --r) {
         const int64_t os = d.operand_strides[q][r];
@@ -435,6 +681,7 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
           if (os != st2) full = false;
           if (os != ((r == d.rank - 1) ? 1 : 0)) vec = false;
           if (os != 0) scal = false;
+          if (os != ((r == d.rank - 1) ? 0 : st2 / inner)) row = false;
         }
         st2 *= d.sizes[r];
       }
@@ -442,7 +689,11 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
         full_mask |= 1u << q;
       else if (vec)
         vec_mask |= 1u << q;
-      else if (!scal)
+      else if (scal)
+        ;
+      else if (row)
+        row_mask |= 1u << q;  // one value per innermost line: only the short-chain kernel takes these
+      else
         vec_ok = false;
     }
     for (int k = 0; k < d.tail.n_ops; ++k) {
@@ -457,11 +708,30 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
   if (vec_ok) {
     const int V = 16 / es;
     const unsigned g = grid_for(a.total / V);
-    if (es == 2)
-      hipLaunchKernelGGL((eltwise_vec_kernel<2>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
-    else
-      hipLaunchKernelGGL((eltwise_vec_kernel<4>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
-    return hipGetLastError();
+    bool short_chain = (d.in_dtype == PML_HIP_F32 || d.in_dtype == PML_HIP_BF16) && d.out_dtype == d.in_dtype;
+    for (int k = 0; k < d.tail.n_ops && short_chain; ++k) {
+      const pml_hip_epi_op& op = d.tail.ops[k];
+      short_chain = short_chain_op(op.opcode) && op.dtype == d.in_dtype &&
+                    (op.operand_kind != PML_HIP_OPND_TENSOR || d.tail.operand_dtype[op.operand] == d.in_dtype);
+    }
+    for (int q = 0; q < d.tail.n_operands; ++q)  // it reads whole-tensor and per-column operands 16 bytes at a time
+      if ((((full_mask | vec_mask) >> q) & 1) && ((uintptr_t)a.operands[q] & 15)) short_chain = false;
+    if (short_chain) {
+      if (d.in_dtype == PML_HIP_F32)
+        hipLaunchKernelGGL((eltwise_short_kernel<PML_HIP_F32>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask,
+                           row_mask);
+      else
+        hipLaunchKernelGGL((eltwise_short_kernel<PML_HIP_BF16>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask,
+                           row_mask);
+      return hipGetLastError();
+    }
+    if (row_mask == 0) {
+      if (es == 2)
+        hipLaunchKernelGGL((eltwise_vec_kernel<2>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
+      else
+        hipLaunchKernelGGL((eltwise_vec_kernel<4>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
+      return hipGetLastError();
+    }
   }
   hipLaunchKernelGGL((eltwise_kernel<float, int>), dim3(grid_for(a.total)), dim3(256), 0, s, a);
   return hipGetLastError();

@@ -153,6 +153,68 @@ def dot_f16_acc_f32(E, op, M=8, N=32, K=16):
         r.standard_normal((M, K)).astype(np.float16), r.standard_normal((K, N)).astype(np.float16)], BF16
 
 
+def row_reductions(E, op, dtype_name='FLOAT32'):
+    """Reductions along memory (the shape of a softmax's row max and row sum, a mean, a norm): over the
+    innermost axis, over the two innermost axes, into a strided output, onto an initial value, over a
+    shifted window, and over rows long enough for a whole workgroup.  Integer types wrap."""
+    dt = getattr(E.DType, dtype_name)
+    X = E.Placeholder(dt, [6, 5, 200])
+    Y = E.Placeholder(dt, [2, 5000])
+    P = E.Placeholder(dt, [6, 5])
+    i, j, k = E.TensorIndexes(3)
+    outs = [
+        E.Contraction().outShape(6, 5).outAccess(i, j).sum(X[i, j, k]).build(),
+        E.Contraction().outShape(6).outAccess(i).max(X[i, j, k]).build(),
+        E.Contraction().outShape(6, 1, 5).outAccess(i, 0, j).min(X[i, j, k]).build(),
+        E.Contraction().outShape(6, 5).outAccess(i, j).init(P).sum(X[i, j, k]).build(),
+        E.Contraction().outShape(6, 5).outAccess(i, j).sum(X[i, j, k + 3]).build(),
+        E.Contraction().outShape(2).outAccess(i).sum(Y[i, k]).build(),
+        E.Contraction().outShape(2).outAccess(i).max(Y[i, k]).build(),
+        E.Contraction().outShape(5).outAccess(j).sum(X[i, j, k]).build(),  # not along memory: the general kernel
+    ]
+    r = _rng(31)
+    if dtype_name in ('FLOAT32', 'BFLOAT16', 'FLOAT16'):
+        outs.append(E.Contraction().outShape(6, 5).outAccess(i, j).product(X[i, j, k]).build())
+        vals = [r.uniform(0.97, 1.03, (6, 5, 200)), r.standard_normal((2, 5000)), r.standard_normal((6, 5))]
+        vals = [v.astype(np.float32) for v in vals]
+        if dtype_name == 'BFLOAT16':
+            vals = [_bf16(v) for v in vals]
+        elif dtype_name == 'FLOAT16':
+            vals = [v.astype(np.float16) for v in vals]
+        tol = FP32 if dtype_name == 'FLOAT32' else BF16
+    else:
+        nd = np.dtype(dtype_name.lower())
+        info = np.iinfo(nd)
+        vals = [r.integers(info.min, int(info.max) + 1, shape, dtype=nd) for shape in ((6, 5, 200), (2, 5000), (6, 5))]
+        tol = EXACT
+    return E.Program('row_reductions', [X, Y, P], outs), vals, tol
+
+
+def float_chains(E, op, dtype_name='FLOAT32', inner=40):
+    """Standalone elementwise chains of plain float arithmetic with every kind of second operand: a whole
+    tensor, one value per column, one value per row, a single value and an immediate."""
+    dt = getattr(E.DType, dtype_name)
+    A = E.Placeholder(dt, [6, inner])
+    B = E.Placeholder(dt, [6, inner])
+    col = E.Placeholder(dt, [inner])
+    row = E.Placeholder(dt, [6, 1])
+    one = E.Placeholder(dt, [1])
+    outs = [
+        E.relu(A * B + col) - row,
+        E.exp(A - row) / (B * B + 1.5),
+        E.tanh(E.sqrt(A * A + 0.25)) * one,
+        E.max(A, col) + E.min(B, row) - (-A),
+        E.log(A * A + 1.0) / row,
+        (2.0 - A) * (3.0 / (B * B + 1.0)),
+    ]
+    r = _rng(32)
+    vals = [r.standard_normal(s).astype(np.float32) for s in ((6, inner), (6, inner), (inner,))]
+    vals += [r.uniform(0.5, 2.0, (6, 1)).astype(np.float32), np.array([1.75], np.float32)]
+    if dtype_name == 'BFLOAT16':
+        vals = [_bf16(v) for v in vals]
+    return E.Program('float_chains', [A, B, col, row, one], outs), vals, FP32 if dtype_name == 'FLOAT32' else BF16
+
+
 def u64_add(E, op):
     """CppEdsl.Add, plaidml/edsl/tests/edsl_test.cc:335-374 (64-bit integer elementwise)."""
     A = E.Placeholder(E.DType.UINT64, [3, 3])
@@ -321,6 +383,15 @@ ALL = {
     'libm_tail_f32': libm_tail_f32,
     'dot_f16_acc_f32': dot_f16_acc_f32,
     'bits_and_truth': bits_and_truth,
+    'row_reductions_f32': row_reductions,
+    'row_reductions_bf16': lambda E, op: row_reductions(E, op, 'BFLOAT16'),
+    'row_reductions_f16': lambda E, op: row_reductions(E, op, 'FLOAT16'),
+    'row_reductions_int32': lambda E, op: row_reductions(E, op, 'INT32'),
+    'row_reductions_uint8': lambda E, op: row_reductions(E, op, 'UINT8'),
+    'row_reductions_int16': lambda E, op: row_reductions(E, op, 'INT16'),
+    'float_chains_f32': float_chains,
+    'float_chains_bf16': lambda E, op: float_chains(E, op, 'BFLOAT16'),
+    'float_chains_f32_ragged': lambda E, op: float_chains(E, op, 'FLOAT32', inner=37),
     'u64_add': u64_add,
     'higher_precision_constants': higher_precision_constants,
     'config0_gemm_f32': config0_gemm_f32,
