@@ -35,6 +35,8 @@ enum class TensorLayout { NXC, NCX, KCX, XCK, GKCX, XGCK, _LAST };
 enum class PadMode { CONSTANT, EDGE, REFLECT, SYMMETRIC, _LAST };
 enum class EpsMode { ADD, MAX, _LAST };
 enum class TopKSortType { VALUE, INDEX, _LAST };
+enum class BoxesDecodeMode { NMS, SSD, _LAST };
+enum class NmsStyle { CAFFE, MXNET, OV, _LAST };
 enum class InterpolationMode { NEAREST, BILINEAR, _LAST };
 // reshape: take the dimension from the input / infer it from the element count
 static const int AUTO_DIM_MATCH = 0;
@@ -192,6 +194,60 @@ class gatherND {
 inline edsl::Tensor sort(const edsl::Tensor& I, int axis, edsl::SortDirection direction = edsl::SortDirection::ASC) {
   return details::op("sort", edsl::make_tuple(I, axis, static_cast<int>(direction))).as_tensor();
 }
+
+// Non-maximum suppression over Boxes [batch, box, 4] and Scores [batch, class, box].  Three styles: OV (every
+// score takes part), CAFFE (only each class's top scores) and MXNET (every box in its best class only, top boxes of
+// the batch).  build() returns {selected (batch, class, box) triples, (batch, class, score) triples, the number of
+// valid selections}; rows not used hold -1.
+class nms {
+ public:
+  explicit nms(edsl::Tensor Boxes, edsl::Tensor Scores, edsl::Tensor IOU_threshold, edsl::Tensor Score_threshold,
+               int max_output_boxes_per_class)
+      : Boxes_(Boxes), Scores_(Scores), IOU_threshold_(IOU_threshold), Score_threshold_(Score_threshold),
+        max_output_boxes_per_class_(max_output_boxes_per_class) {}
+  nms& soft_nms_sigma(float v) { soft_nms_sigma_ = v; return *this; }
+  nms& center_point_box(bool v) { center_point_box_ = v; return *this; }
+  nms& sort_result_descending(bool v) { sort_result_descending_ = v; return *this; }
+  nms& box_output_type(DType v) { box_output_type_ = v; return *this; }
+  nms& boxes_decode_mode(BoxesDecodeMode v) { boxes_decode_mode_ = v; return *this; }
+  nms& clip_before_nms(bool v) { clip_before_nms_ = v; return *this; }
+  nms& clip_after_nms(bool v) { clip_after_nms_ = v; return *this; }
+  nms& ssd_input_height(int v) { ssd_input_height_ = v; return *this; }
+  nms& ssd_input_width(int v) { ssd_input_width_ = v; return *this; }
+  nms& ssd_variances(edsl::Tensor v) { ssd_variances_ = v; return *this; }
+  nms& ssd_location(edsl::Tensor v) { ssd_location_ = v; return *this; }
+  nms& ssd_arm_location(edsl::Tensor v) { ssd_arm_location_ = v; return *this; }
+  nms& ssd_with_arm_loc(bool v) { ssd_with_arm_loc_ = v; return *this; }
+  nms& nms_style(NmsStyle v) { nms_style_ = v; return *this; }
+  nms& share_location(bool v) { share_location_ = v; return *this; }
+  nms& hard_suppression(bool v) { hard_suppression_ = v; return *this; }
+  std::vector<edsl::Tensor> build() {
+    auto args = edsl::make_tuple(Boxes_, Scores_, IOU_threshold_, Score_threshold_, max_output_boxes_per_class_,
+                                 static_cast<double>(soft_nms_sigma_), center_point_box_, sort_result_descending_,
+                                 static_cast<int>(box_output_type_), static_cast<int>(boxes_decode_mode_), clip_before_nms_,
+                                 clip_after_nms_, ssd_input_height_, ssd_input_width_, ssd_variances_, ssd_location_,
+                                 ssd_with_arm_loc_, ssd_arm_location_, static_cast<int>(nms_style_), share_location_,
+                                 hard_suppression_);
+    auto R = details::op("nms", args).as_tuple();
+    return {R[0].as_tensor(), R[1].as_tensor(), R[2].as_tensor()};
+  }
+
+ private:
+  edsl::Tensor Boxes_, Scores_, IOU_threshold_, Score_threshold_;
+  edsl::Tensor ssd_variances_, ssd_location_, ssd_arm_location_;  // unset: passed as none
+  int max_output_boxes_per_class_;
+  float soft_nms_sigma_ = 0.0f;
+  bool center_point_box_ = false;
+  bool sort_result_descending_ = false;
+  DType box_output_type_ = DType::INT32;
+  BoxesDecodeMode boxes_decode_mode_ = BoxesDecodeMode::NMS;
+  bool clip_before_nms_ = false, clip_after_nms_ = false;
+  int ssd_input_height_ = 0, ssd_input_width_ = 0;
+  bool ssd_with_arm_loc_ = false;
+  NmsStyle nms_style_ = NmsStyle::OV;
+  bool share_location_ = true;
+  bool hard_suppression_ = true;
+};
 
 class topk {
  public:

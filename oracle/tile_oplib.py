@@ -15,17 +15,22 @@ op library emits for the operations on the hot path (plaidml/op/lib/ops.cc):
   argmax        :505-521
   and, each cited where it is defined below: abs, all, any, binary_crossentropy,
   broadcast, clip, concatenate, cumprod, cumsum, elu, explicit_padding, flip,
-  gatherND, hard_sigmoid, image_resize, l2norm, lrn, mvn, prod, reorg_yolo, repeat,
+  gatherND, hard_sigmoid, image_resize, l2norm, lrn, mvn, nms, prod, reorg_yolo, repeat,
   reshape, scale_gradient, sigmoid, slice, sort, spatial_padding, square, squeeze,
   tile, topk, transpose, unsqueeze, variance
 
 Pinned by tests/test_oplib_ops.py, tests/test_conv_general.py and the op-level
 cases of tests/test_oracle_golden.py (numpy closed forms, the exact cases of
 plaidml/op/op_test.cc, direct numpy evaluations of the definitions).
+nms has no test in the reference: tests/test_nms.py pins it against a loop-written
+greedy suppression for the NMS box formats and the three styles; its SSD box
+decoding (_box_corners, SSD branches) has no independent check: PARITY UNPINNED.
 
 Nothing in the shipped package imports this module.
 """
 import builtins
+
+import numpy as np
 
 from . import tile_oracle as E
 
@@ -914,3 +919,179 @@ def image_resize(I, factors, interp=RESIZE_NEAREST, layout=LAYOUT_NXC):
     o_idxs[pre] = fh * idxs[pre] + j - fh + 1
     o_idxs[pre + 1] = fw * idxs[pre + 1] + i - fw + 1
     return E.Contraction('image_resize').outShape(o_dims).outAccess(o_idxs).sum(I[idxs] * K[j, i]).build()
+
+
+BOXES_NMS, BOXES_SSD = range(2)
+NMS_CAFFE, NMS_MXNET, NMS_OV = range(3)
+
+
+def _box_corners(boxes, variances, location, decode, in_h, in_w, clip_boxes, centered):
+    """decode_boxes, ops.cc:2034-2117: (y1, x1, y2, x2), each the box tensor without its last axis."""
+    col = lambda t, k: E.gather(t, k, axis=3)  # noqa: E731
+    if centered:
+        if decode == BOXES_NMS:  # [x, y, width, height]
+            xc, yc, hw, hh = col(boxes, 0), col(boxes, 1), col(boxes, 2) / 2.0, col(boxes, 3) / 2.0
+        elif decode == BOXES_SSD:
+            px1, py1 = col(boxes, 0) / in_w, col(boxes, 1) / in_h
+            px2, py2 = col(boxes, 2) / in_w, col(boxes, 3) / in_h
+            v = [col(variances, k) for k in range(4)]
+            loc = [col(location, k) for k in range(4)]
+            pw, ph = px2 - px1, py2 - py1
+            xc = v[0] * loc[0] * pw + (px1 + px2) / 2.0
+            yc = v[1] * loc[1] * ph + (py1 + py2) / 2.0
+            hw = E.exp(v[2] * loc[2]) * pw / 2.0
+            hh = E.exp(v[3] * loc[3]) * ph / 2.0
+        else:
+            raise ValueError('Unrecognized boxes decode mode')
+        x1, x2, y1, y2 = xc - hw, xc + hw, yc - hh, yc + hh
+    elif decode == BOXES_NMS:  # [y1, x1, y2, x2] with either corner first
+        ya, xa, yb, xb = (col(boxes, k) for k in range(4))
+        y1, x1, y2, x2 = minimum(ya, yb), minimum(xa, xb), maximum(ya, yb), maximum(xa, xb)
+    elif decode == BOXES_SSD:  # [x1, y1, x2, y2]
+        boxes = boxes / in_w + variances * location
+        x1, y1, x2, y2 = (col(boxes, k) for k in range(4))
+    else:
+        raise ValueError('Unrecognized boxes decode mode')
+    if clip_boxes:
+        lo, hi = E.cast(0.0, E.DType.FLOAT32), E.cast(1.0, E.DType.FLOAT32)
+        y1, x1, y2, x2 = (clip(t, lo, hi) for t in (y1, x1, y2, x2))
+    return [y1, x1, y2, x2]
+
+
+
+def _pairwise_iou(corners, nb, nbox, nloc):
+    """compute_iou, ops.cc:2119-2153: [batch, location class, box, box]."""
+    zero = E.cast(E.index([1], 0), corners[0].dt)
+    y1, x1, y2, x2 = (E.reshape(t, [nb, nloc, nbox]) for t in corners)
+    area = (y2 - y1) * (x2 - x1)
+    as_rows = lambda t: E.reshape(t, [nb, nloc, nbox, 1])  # noqa: E731
+    as_cols = lambda t: E.reshape(t, [nb, nloc, 1, nbox])  # noqa: E731
+    ygap = minimum(as_rows(y2), as_cols(y2)) - maximum(as_rows(y1), as_cols(y1))
+    xgap = minimum(as_rows(x2), as_cols(x2)) - maximum(as_rows(x1), as_cols(x1))
+    inter = E.select(ygap > 0.0, ygap, zero) * E.select(xgap > 0.0, xgap, zero)
+    union = unsqueeze(area, [-1]) + unsqueeze(area, [-2]) - inter
+    return inter * E.select(union <= 0.0, zero, 1.0 / union)
+
+
+def nms(Boxes, Scores, iou_threshold, score_threshold, max_output_boxes_per_class, soft_nms_sigma=0.0,
+        center_point_box=False, sort_result_descending=False, box_output_type=E.DType.INT32,
+        boxes_decode_mode=BOXES_NMS, clip_before_nms=False, clip_after_nms=False, ssd_input_height=0,
+        ssd_input_width=0, ssd_variances=None, ssd_location=None, ssd_with_arm_loc=False, ssd_arm_location=None,
+        nms_style=NMS_OV, share_location=True, hard_suppression=True):
+    """ops.cc:2157-2417.  Greedy non-maximum suppression unrolled max_output_boxes_per_class times over
+    Scores [batch, class, box]: each round takes every (batch, class)'s best remaining box, records it, and zeroes
+    the scores of the boxes that overlap it.  Returns [selected (batch, class, box) triples, (batch, class, score)
+    triples, the number of valid selections]; unused rows are -1."""
+    if boxes_decode_mode not in (BOXES_NMS, BOXES_SSD):
+        raise ValueError('Invalid enumeration value')
+    if nms_style not in (NMS_CAFFE, NMS_MXNET, NMS_OV):
+        raise ValueError('Invalid enumeration value')
+    in_dt, thr_dt, out_dt = Boxes.dt, iou_threshold.dt, E.DType(box_output_type)
+    nb, nc, nbox = Scores.shape
+    nloc = 1 if share_location else nc
+
+    zero = E.cast(E.index([1], 0), in_dt)
+    zero_int = E.cast(zero, E.DType.INT32)
+    one = zero + 1
+    neg1 = -one
+    neg1_o = E.cast(neg1, out_dt)
+    valid_outputs = zero
+
+    Boxes = unsqueeze(Boxes, [1])
+    if ssd_with_arm_loc:
+        ssd_variances = unsqueeze(ssd_variances, [1])
+        p = _box_corners(Boxes, ssd_variances, ssd_arm_location, boxes_decode_mode, ssd_input_height, ssd_input_width,
+                         clip_before_nms, center_point_box)
+        priors = concatenate([p[1], p[0], p[3], p[2]], -1)
+        corners = _box_corners(priors, ssd_variances, ssd_location, boxes_decode_mode, ssd_input_height,
+                               ssd_input_width, clip_before_nms, center_point_box)
+    else:
+        if boxes_decode_mode == BOXES_SSD:
+            ssd_variances = unsqueeze(ssd_variances, [1])
+        corners = _box_corners(Boxes, ssd_variances, ssd_location, boxes_decode_mode, ssd_input_height,
+                               ssd_input_width, clip_before_nms, center_point_box)
+    iou = _pairwise_iou(corners, nb, nbox, nloc)
+    weight = -0.5 / soft_nms_sigma if soft_nms_sigma != 0 else 0.0
+
+    invalid_node = E.cast(E.Constant(np.array([[[-1, -1]]], np.float32), name='invalid_node'), out_dt)
+    per_class = builtins.min(nbox, max_output_boxes_per_class) if max_output_boxes_per_class != 0 else nbox
+    index_bc = E.cast(concatenate([E.index([nb, nc, 1], 0), E.index([nb, nc, 1], 1)], 2), out_dt)
+    score_thr = E.cast(score_threshold, in_dt)
+    iou_thr = E.cast(iou_threshold, in_dt)
+    new_scores = E.select(Scores > score_thr, Scores, zero)
+
+    def zeros(shape):
+        return E.Contraction('nms').outShape(shape).outAccess(E.TensorIndexes(3)).assign(zero[0]).build()
+
+    if nms_style == NMS_CAFFE:  # only the top scores of each class take part
+        vals, idxs = topk(new_scores, per_class, axis=2)
+        new_scores = E.scatter(zeros([nb, nc, nbox]), idxs, vals, axis=2, mode=E.SCATTER_UPDATE_ELT)
+    elif nms_style == NMS_MXNET:  # each box competes in its best class only, and only the top boxes do
+        best_class = squeeze(E.gather(E.argsort(new_scores, 1, E.SORT_DESC), 0, axis=1), [1])
+        best_score = squeeze(E.gather(sort(new_scores, 1, E.SORT_DESC), 0, axis=1), [1])
+        top_scores, top_boxes = topk(best_score, per_class, axis=1, sort_type=TOPK_INDEX)
+        top_classes = gatherND(best_class, unsqueeze(top_boxes, [-1]), batch_dims=1)
+        batch_idx = unsqueeze(E.index(list(top_classes.shape), 0), [-1])
+        where = concatenate([batch_idx, unsqueeze(top_classes, [-1]), unsqueeze(top_boxes, [-1])], -1)
+        new_scores = E.scatter(zeros([nb, nc, nbox]), where, top_scores, mode=E.SCATTER_UPDATE_ND)
+
+    zero_cell = zeros([nb, nc, 1])
+    boxes, scores = [], []
+    for _ in range(per_class):
+        candidate = E.gather(E.argsort(new_scores, 2, E.SORT_DESC), 0, axis=2)
+        score = E.reshape(max(new_scores, 2), [nb, nc, 1])
+        node = E.select(score > 0.0, index_bc, invalid_node)
+        valid_outputs = valid_outputs + sum(E.select(score != 0.0, one, zero))
+        scores.append(E.cast(node, thr_dt))
+        score = E.select(score > 0.0, score, neg1)
+        scores.append(E.cast(score, thr_dt))
+        # the winner itself goes to zero by position (equal scores may exist), its neighbours by overlap
+        new_scores = E.reshape(E.scatter(new_scores, candidate, zero_cell, axis=2, mode=E.SCATTER_UPDATE_ELT),
+                               [nb, nc, nbox])
+        if share_location:
+            class_idx = broadcast(zero_int, list(candidate.shape), [1])
+        else:
+            class_idx = E.index(list(candidate.shape), 1)
+        overlap = gatherND(iou, concatenate([class_idx, candidate], 2), batch_dims=1)
+        suppressed = (overlap >= iou_thr) if hard_suppression else (overlap > iou_thr)
+        new_scores = E.select(suppressed, zero, new_scores)
+        box_index = E.select(score > 0.0, E.cast(candidate, out_dt), neg1_o)
+        boxes.append(node)
+        boxes.append(E.reshape(box_index, [nb, nc, 1]))
+        if soft_nms_sigma != 0:
+            new_scores = new_scores * E.exp(overlap * overlap * weight)
+            new_scores = E.select(new_scores > score_thr, new_scores, zero)
+
+    valid_outputs = E.cast(valid_outputs, out_dt)
+    rows = nb * nc * per_class
+    scores_result = E.reshape(concatenate(scores, 2), [rows, 3])
+    boxes_result = E.reshape(concatenate(boxes, 2), [rows, 3])
+    if sort_result_descending:
+        order = E.argsort(E.reshape(E.gather(scores_result, 2, axis=1), [rows]), 0, E.SORT_DESC)
+        scores_result = E.gather(scores_result, order, axis=0)
+        boxes_result = E.gather(boxes_result, order, axis=0)
+    else:
+        # a stable sort on "position, or past-the-end for a -1" moves the unused entries to the back
+        n = rows * 3
+        flat_scores, flat_boxes = E.reshape(scores_result, [n]), E.reshape(boxes_result, [n])
+        key = E.select(flat_scores != E.cast(-1, thr_dt), E.index([n], 0), E.cast(n, E.DType.INT32))
+        order = E.argsort(E.cast(key, E.DType.FLOAT32), 0)
+        scores_result = E.reshape(E.gather(flat_scores, order, axis=0), [rows, 3])
+        boxes_result = E.reshape(E.gather(flat_boxes, order, axis=0), [rows, 3])
+        if boxes_decode_mode == BOXES_SSD:
+            decoded = concatenate([corners[1], corners[0], corners[3], corners[2]], -1)
+            if clip_after_nms:
+                decoded = clip(decoded, E.cast(0.0, E.DType.FLOAT32), E.cast(1.0, E.DType.FLOAT32))
+            if share_location:
+                pick = E.gather(boxes_result, concatenate([zero_int, zero_int + 2], 0), axis=1)
+                out_boxes = gatherND(squeeze(decoded, [0]), pick)
+            else:
+                out_boxes = gatherND(decoded, boxes_result)
+            if nms_style == NMS_MXNET:
+                classes = E.gather(boxes_result, 1, axis=1) - 1  # drops the background class
+                one_int = zero_int + 1
+                scores_result = E.scatter(scores_result, one_int, E.cast(classes, scores_result.dt), axis=1,
+                                          mode=E.SCATTER_UPDATE_SLICE)
+                boxes_result = E.scatter(boxes_result, one_int, classes, axis=1, mode=E.SCATTER_UPDATE_SLICE)
+            scores_result = concatenate([scores_result, out_boxes], 1)
+    return [boxes_result, scores_result, valid_outputs]

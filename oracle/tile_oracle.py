@@ -683,7 +683,12 @@ def argsort(x, axis=-1, direction=SORT_ASC):
 
 def gather(x, y, axis=0, interpolation_mode=INTERP_NONE, nearest_mode=NEAREST_ROUND_PREFER_FLOOR, cube_coeff=-0.75,
            mode=GATHER_NORMAL, batch_dims=0, out_of_bounds_mode=OOB_EDGE_PADDED_INPUT):
-    """Shape rule pmlc/ast/ast_ops.cc:88-178."""
+    """Shape rule pmlc/ast/ast_ops.cc:88-178.  A plain number is one position and keeps the axis
+    (plaidml/edsl/edsl.h:1699-1717)."""
+    if isinstance(y, (int, np.integer)) and not isinstance(y, bool):
+        y = cast(index([1], 0), DType.INT32) + int(y)
+    elif isinstance(y, (float, np.floating)):
+        y = cast(index([1], 0), DType.FLOAT32) + float(y)
     x, y = _literal(x), _literal(y)
     rank = len(x.shape)
     if rank == 0:
@@ -743,14 +748,18 @@ def _eval_gather(x, y, a, dt, idt):
         depth = y.shape[-1]
         out = np.empty(tuple(y.shape[:-1]) + tuple(x.shape[bd + depth:]), x.dtype)
         for lead in np.ndindex(*y.shape[:-1]):
-            src = tuple(lead[:bd]) + tuple(int(v) for v in y[lead])
-            out[lead] = x[src]
+            at = tuple(int(v) for v in y[lead])
+            # a coordinate outside the tensor is undefined in the reference; declared here (and on the device) to read 0
+            inside = builtins.all(0 <= v < n for v, n in zip(at, x.shape[bd:bd + depth]))
+            out[lead] = x[tuple(lead[:bd]) + at] if inside else 0
         return out
     out_shape = tuple(x.shape[:axis]) + tuple(y.shape) + tuple(x.shape[axis + 1:])
     xm = np.moveaxis(x, axis, 0)                                  # [axis, before.., after..]
     upper = x.shape[axis] - 1
     if not is_float(idt):
-        res = xm[np.asarray(y, np.int64)]                         # [idx.., before.., after..]
+        at = np.asarray(y, np.int64)
+        res = xm[np.clip(at, 0, upper)]                           # [idx.., before.., after..]
+        res = np.where(((at < 0) | (at > upper)).reshape(at.shape + (1,) * (xm.ndim - 1)), res.dtype.type(0), res)  # declared: 0
     elif not is_float(dt):
         res = xm[np.trunc(y).astype(np.int64)]                    # fptosi, then a plain read
     else:

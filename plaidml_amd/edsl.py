@@ -765,6 +765,14 @@ def argsort(x, axis=-1, direction=SORT_ASC):
 
 def gather(x, y, axis=0, interpolation_mode=INTERP_NONE, nearest_mode=NEAREST_ROUND_PREFER_FLOOR, cube_coeff=-0.75,
            mode=GATHER_NORMAL, batch_dims=0, out_of_bounds_mode=OOB_EDGE_PADDED_INPUT):
+    # a plain number addresses one position and keeps the axis, as the C++ builder's scalar overloads do
+    # (plaidml/edsl/edsl.h:1699-1717)
+    if isinstance(y, bool):
+        raise TypeError('gather index must be a tensor or a number')
+    if isinstance(y, int):
+        y = cast(index([1], 0), DType.INT32) + y
+    elif isinstance(y, float):
+        y = cast(index([1], 0), DType.FLOAT32) + y
     if axis < 0:
         axis += x.rank
     return intrinsic('gather', x, y, _uint(axis), _uint(interpolation_mode), _uint(nearest_mode), _float(cube_coeff), _uint(mode),

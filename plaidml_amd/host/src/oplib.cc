@@ -1389,6 +1389,241 @@ Value op_topk(const Value& value) {
   return Value(out);
 }
 
+// ---- non-maximum suppression (plaidml/op/lib/ops.cc:2034-2417) ------------------------------------------
+using plaidml::op::BoxesDecodeMode;
+using plaidml::op::NmsStyle;
+
+Tensor larger_of(const Tensor& a, const Tensor& b) { return op_maximum(make_tuple(Value{a}, Value{b})).as_tensor(); }
+Tensor smaller_of(const Tensor& a, const Tensor& b) { return op_minimum(make_tuple(Value{a}, Value{b})).as_tensor(); }
+Tensor unit_clip(const Tensor& t) {
+  return op_clip(make_tuple(Value{t}, Value{cast(Tensor(0.0), DType::FLOAT32)}, Value{cast(Tensor(1.0), DType::FLOAT32)})).as_tensor();
+}
+Tensor squeeze_at(const Tensor& t, int64_t axis) { return op_squeeze(make_tuple(Value{t}, int_tuple({axis}))).as_tensor(); }
+
+// The four edges {y1, x1, y2, x2} of every box, each shaped like `boxes` with a last dimension of 1
+// (ops.cc:2034-2117).  NMS boxes are corners in either order or centre + size; SSD boxes are priors in pixels that
+// the location deltas, scaled by the variances, move and stretch.
+std::vector<Tensor> box_edges(Tensor boxes, const Tensor& variances, const Tensor& location, BoxesDecodeMode decode, int64_t in_h,
+                              int64_t in_w, bool clip_boxes, bool centered) {
+  auto col = [](const Tensor& t, int k) -> Tensor { return gather(t, k).axis(3); };
+  Tensor y1, x1, y2, x2;
+  if (centered) {
+    Tensor xc, yc, half_w, half_h;
+    if (decode == BoxesDecodeMode::NMS) {
+      xc = col(boxes, 0);
+      yc = col(boxes, 1);
+      half_w = col(boxes, 2) / 2.0;
+      half_h = col(boxes, 3) / 2.0;
+    } else if (decode == BoxesDecodeMode::SSD) {
+      Tensor px1 = col(boxes, 0) / in_w, py1 = col(boxes, 1) / in_h, px2 = col(boxes, 2) / in_w, py2 = col(boxes, 3) / in_h;
+      Tensor pw = px2 - px1, ph = py2 - py1;
+      xc = col(variances, 0) * col(location, 0) * pw + (px1 + px2) / 2.0;
+      yc = col(variances, 1) * col(location, 1) * ph + (py1 + py2) / 2.0;
+      half_w = exp(col(variances, 2) * col(location, 2)) * pw / 2.0;
+      half_h = exp(col(variances, 3) * col(location, 3)) * ph / 2.0;
+    } else {
+      throw std::runtime_error("Unrecognized boxes decode mode");
+    }
+    x1 = xc - half_w, x2 = xc + half_w, y1 = yc - half_h, y2 = yc + half_h;
+  } else if (decode == BoxesDecodeMode::NMS) {
+    Tensor ya = col(boxes, 0), xa = col(boxes, 1), yb = col(boxes, 2), xb = col(boxes, 3);
+    y1 = smaller_of(ya, yb), x1 = smaller_of(xa, xb), y2 = larger_of(ya, yb), x2 = larger_of(xa, xb);
+  } else if (decode == BoxesDecodeMode::SSD) {
+    boxes = boxes / in_w + variances * location;
+    x1 = col(boxes, 0), y1 = col(boxes, 1), x2 = col(boxes, 2), y2 = col(boxes, 3);
+  } else {
+    throw std::runtime_error("Unrecognized boxes decode mode");
+  }
+  if (clip_boxes) y1 = unit_clip(y1), x1 = unit_clip(x1), y2 = unit_clip(y2), x2 = unit_clip(x2);
+  return {y1, x1, y2, x2};
+}
+
+// intersection over union of every pair of boxes: [batch, location class, box, box]; 0 where the union is empty
+Tensor pairwise_iou(const std::vector<Tensor>& edges, const TensorDim& nb, const TensorDim& nbox, const TensorDim& nloc) {
+  TensorDim one(1);
+  Tensor zero = cast(index({one}, 0), edges[0].dtype());
+  auto flat = [&](const Tensor& t) { return reshape(t, {nb, nloc, nbox}); };
+  Tensor y1 = flat(edges[0]), x1 = flat(edges[1]), y2 = flat(edges[2]), x2 = flat(edges[3]);
+  Tensor area = (y2 - y1) * (x2 - x1);
+  auto rows = [&](const Tensor& t) { return reshape(t, {nb, nloc, nbox, one}); };
+  auto cols = [&](const Tensor& t) { return reshape(t, {nb, nloc, one, nbox}); };
+  Tensor ygap = smaller_of(rows(y2), cols(y2)) - larger_of(rows(y1), cols(y1));
+  Tensor xgap = smaller_of(rows(x2), cols(x2)) - larger_of(rows(x1), cols(x1));
+  Tensor inter = select(ygap > 0.0, ygap, zero) * select(xgap > 0.0, xgap, zero);
+  Tensor uni = unsqueeze_at(area, -1) + unsqueeze_at(area, -2) - inter;
+  return inter * select(uni <= 0.0, zero, 1.0 / uni);
+}
+
+// Greedy suppression unrolled max_output_boxes_per_class times over Scores [batch, class, box]: each round takes
+// every (batch, class)'s best remaining box, records it, and zeroes the scores of the boxes overlapping it.
+// Returns {selected (batch, class, box) triples, (batch, class, score) triples, number of valid selections};
+// unused rows hold -1.
+Value op_nms(const Value& value) {
+  auto args = value.as_tuple();
+  if (args.size() != 21) throw std::runtime_error("nms expects 21 arguments");
+  auto Boxes = args[0].as_tensor();
+  auto Scores = args[1].as_tensor();
+  auto iou_threshold = args[2].as_tensor();
+  auto score_threshold = args[3].as_tensor();
+  const int64_t max_per_class = args[4].as_int();
+  const double sigma = args[5].as_float();
+  const bool centered = args[6].as_bool();
+  const bool sort_descending = args[7].as_bool();
+  const auto out_type = validate<DType>(args[8].as_int());
+  const auto decode = validate<BoxesDecodeMode>(args[9].as_int());
+  const bool clip_before = args[10].as_bool(), clip_after = args[11].as_bool();
+  const int64_t in_h = args[12].as_int(), in_w = args[13].as_int();
+  const DType in_type = Boxes.dtype(), thr_type = iou_threshold.dtype();
+  Tensor variances, location, arm_location;
+  if (decode == BoxesDecodeMode::SSD) variances = args[14].as_tensor(), location = args[15].as_tensor();
+  const bool with_arm = args[16].as_bool();
+  if (with_arm) arm_location = args[17].as_tensor();
+  const auto style = validate<NmsStyle>(args[18].as_int());
+  const bool share_location = args[19].as_bool();
+  const bool hard = args[20].as_bool();
+
+  const int64_t boxes_count = Scores.compute_shape().sizes().at(2);
+  std::vector<TensorDim> sd(Scores.rank());
+  Scores.bind_dims(sd);
+  TensorDim nb = sd[0], nc = sd[1], nbox = sd[2], one_dim(1);
+  TensorDim nloc = share_location ? one_dim : nc;
+
+  Tensor zero = cast(index({one_dim}, 0), in_type);
+  Tensor zero_int = cast(zero, DType::INT32);
+  Tensor one = zero + 1;
+  Tensor neg1 = -one;
+  Tensor neg1_out = cast(neg1, out_type);
+  Tensor valid_outputs = zero;
+
+  Boxes = unsqueeze_at(Boxes, 1);
+  std::vector<Tensor> edges;
+  if (with_arm) {
+    variances = unsqueeze_at(variances, 1);
+    auto p = box_edges(Boxes, variances, arm_location, decode, in_h, in_w, clip_before, centered);
+    Tensor priors = concatenate({p[1], p[0], p[3], p[2]}, -1);
+    edges = box_edges(priors, variances, location, decode, in_h, in_w, clip_before, centered);
+  } else {
+    if (decode == BoxesDecodeMode::SSD) variances = unsqueeze_at(variances, 1);
+    edges = box_edges(Boxes, variances, location, decode, in_h, in_w, clip_before, centered);
+  }
+  Tensor iou = pairwise_iou(edges, nb, nbox, nloc);
+  const double weight = sigma != 0 ? -0.5 / static_cast<float>(sigma) : 0.0;
+
+  const float minus_ones[2] = {-1.f, -1.f};
+  Buffer invalid_buf(TensorShape(DType::FLOAT32, {1, 1, 2}));
+  invalid_buf.copy_from(minus_ones);
+  Tensor invalid_node = cast(Constant(invalid_buf, "invalid_node"), out_type);
+
+  const int64_t per_class = max_per_class != 0 ? std::min(boxes_count, max_per_class) : boxes_count;
+  Tensor index_bc = cast(concatenate({index({nb, nc, one_dim}, 0), index({nb, nc, one_dim}, 1)}, 2), out_type);
+  Tensor score_thr = cast(score_threshold, in_type);
+  Tensor iou_thr = cast(iou_threshold, in_type);
+  Tensor new_scores = select(Scores > score_thr, Scores, zero);
+
+  auto zeros = [&](const std::vector<TensorDim>& dims) -> Tensor {
+    std::vector<TensorIndex> idxs(3);
+    return Contraction(dims, idxs, "nms").assign(zero(0));
+  };
+  auto top_k = [](const Tensor& t, int64_t k, int64_t axis, plaidml::op::TopKSortType type) {
+    return op_topk(make_tuple(Value{t}, Value{k}, Value{axis}, Value{static_cast<int64_t>(SortDirection::DESC)},
+                              Value{static_cast<int64_t>(type)}, Value{static_cast<int64_t>(DType::INT32)}))
+        .as_tuple();
+  };
+  auto gather_nd = [](const Tensor& t, const Tensor& at, int64_t batch_dims) {
+    return gatherBuilder(t, at, static_cast<uint64_t>(batch_dims), InterpolationMode::NONE).build();
+  };
+  auto sorted_desc = [](const Tensor& t, int64_t axis) { return sorted_by(t, argsort(t, static_cast<int>(axis), SortDirection::DESC), axis); };
+
+  if (style == NmsStyle::CAFFE) {
+    // only the top scores of each class take part
+    auto top = top_k(new_scores, per_class, 2, plaidml::op::TopKSortType::VALUE);
+    new_scores = scatter(zeros({nb, nc, nbox}), top[1].as_tensor(), top[0].as_tensor()).axis(2).mode(ScatterMode::UPDATE_ELT);
+  } else if (style == NmsStyle::MXNET) {
+    // every box competes in its best class only, and only the top boxes of a batch do
+    Tensor best_class = squeeze_at(gather(argsort(new_scores, 1, SortDirection::DESC), 0).axis(1), 1);
+    Tensor best_score = squeeze_at(gather(sorted_desc(new_scores, 1), 0).axis(1), 1);
+    auto top = top_k(best_score, per_class, 1, plaidml::op::TopKSortType::INDEX);
+    Tensor top_scores = top[0].as_tensor(), top_boxes = top[1].as_tensor();
+    Tensor top_classes = gather_nd(best_class, unsqueeze_at(top_boxes, -1), 1);
+    std::vector<TensorDim> dims(2);
+    top_classes.bind_dims(dims);
+    Tensor where = concatenate({unsqueeze_at(index(dims, 0), -1), unsqueeze_at(top_classes, -1), unsqueeze_at(top_boxes, -1)}, -1);
+    new_scores = scatter(zeros({nb, nc, nbox}), where, top_scores).mode(ScatterMode::UPDATE_ND);
+  }
+
+  Tensor zero_cell = zeros({nb, nc, one_dim});
+  std::vector<Tensor> box_parts, score_parts;
+  for (int64_t k = 0; k < per_class; ++k) {
+    Tensor candidate = gather(argsort(new_scores, 2, SortDirection::DESC), 0).axis(2);
+    Tensor score = reshape(reduce(make_tuple(Value{new_scores}, Value{int64_t{2}}, Value{false}), "max", PLAIDML_AGG_OP_MAX).as_tensor(),
+                           {nb, nc, one_dim});
+    Tensor node = select(score > 0.0, index_bc, invalid_node);
+    Tensor counted = reduce(make_tuple(Value{select(score != 0.0, one, zero)}, Value(), Value{false}), "sum", PLAIDML_AGG_OP_SUM).as_tensor();
+    valid_outputs = valid_outputs + counted;
+    score_parts.push_back(cast(node, thr_type));
+    score = select(score > 0.0, score, neg1);
+    score_parts.push_back(cast(score, thr_type));
+    // the winner itself goes to zero by position (equal scores may exist), its neighbours by overlap
+    Tensor cleared = scatter(new_scores, candidate, zero_cell).axis(2).mode(ScatterMode::UPDATE_ELT);
+    new_scores = reshape(cleared, {nb, nc, nbox});
+    Tensor class_idx;
+    if (share_location) {
+      class_idx = op_broadcast(make_tuple(Value{zero_int}, int_tuple(candidate.compute_shape().sizes()), int_tuple({1}))).as_tensor();
+    } else {
+      std::vector<TensorDim> cd(candidate.rank());
+      candidate.bind_dims(cd);
+      class_idx = index(cd, 1);
+    }
+    Tensor overlap = gather_nd(iou, concatenate({class_idx, candidate}, 2), 1);
+    new_scores = select(hard ? overlap >= iou_thr : overlap > iou_thr, zero, new_scores);
+    Tensor box_index = select(score > 0.0, cast(candidate, out_type), neg1_out);
+    box_parts.push_back(node);
+    box_parts.push_back(reshape(box_index, {nb, nc, one_dim}));
+    if (sigma != 0) {
+      new_scores = new_scores * exp(overlap * overlap * weight);
+      new_scores = select(new_scores > score_thr, new_scores, zero);
+    }
+  }
+
+  valid_outputs = cast(valid_outputs, out_type);
+  TensorDim rows = nb * nc * per_class;
+  Tensor scores_result = reshape(concatenate(score_parts, 2), {rows, TensorDim(3)});
+  Tensor boxes_result = reshape(concatenate(box_parts, 2), {rows, TensorDim(3)});
+  if (sort_descending) {
+    Tensor key = reshape(gather(scores_result, 2).axis(1), {rows});
+    Tensor order = argsort(key, 0, SortDirection::DESC);
+    scores_result = gather(scores_result, order).axis(0);
+    boxes_result = gather(boxes_result, order).axis(0);
+  } else {
+    // a stable sort on "own position, or past-the-end for a -1" moves the unused entries to the back
+    TensorDim n = rows * 3;
+    Tensor flat_scores = reshape(scores_result, {n}), flat_boxes = reshape(boxes_result, {n});
+    Tensor key = select(flat_scores != cast(Tensor(-1), thr_type), index({n}, 0), cast(Tensor{n}, DType::INT32));
+    Tensor order = argsort(cast(key, DType::FLOAT32), 0);
+    scores_result = reshape(gather(flat_scores, order).axis(0), {rows, TensorDim(3)});
+    boxes_result = reshape(gather(flat_boxes, order).axis(0), {rows, TensorDim(3)});
+    if (decode == BoxesDecodeMode::SSD) {
+      Tensor decoded = concatenate({edges[1], edges[0], edges[3], edges[2]}, -1);
+      if (clip_after) decoded = unit_clip(decoded);
+      Tensor out_boxes;
+      if (share_location) {
+        Tensor pick = gather(boxes_result, concatenate({zero_int, zero_int + 2}, 0)).axis(1);
+        out_boxes = gather_nd(squeeze_at(decoded, 0), pick, 0);
+      } else {
+        out_boxes = gather_nd(decoded, boxes_result, 0);
+      }
+      if (style == NmsStyle::MXNET) {
+        Tensor classes = gather(boxes_result, 1).axis(1) - 1;  // drops the background class
+        Tensor one_int = zero_int + 1;
+        scores_result = scatter(scores_result, one_int, cast(classes, scores_result.dtype())).mode(ScatterMode::UPDATE_SLICE).axis(1);
+        boxes_result = scatter(boxes_result, one_int, classes).mode(ScatterMode::UPDATE_SLICE).axis(1);
+      }
+      scores_result = concatenate({scores_result, out_boxes}, 1);
+    }
+  }
+  return make_tuple(boxes_result, scores_result, valid_outputs);
+}
+
 // plaidml/op/lib/ops.cc:1822-1918: both spatial dimensions of an image grow by integer factors.  NEAREST repeats
 // pixels; BILINEAR spreads every pixel with a (2f-1) x (2f-1) tent kernel, which aligns the corners to 0 and
 // f * (dim - 1) and treats the outside as zero.
@@ -1473,6 +1708,7 @@ const std::map<std::string, OpFn>& registry() {
       {"mean", [](const Value& v) { return reduce(v, "mean", PLAIDML_AGG_OP_SUM); }},
       {"min", [](const Value& v) { return reduce(v, "min", PLAIDML_AGG_OP_MIN); }},
       {"minimum", op_minimum},
+      {"nms", op_nms},
       {"mvn", op_mvn},
       {"pool", op_pool},
       {"prod", op_prod},

@@ -243,6 +243,26 @@ def topk(I, k, axis=-1, sort_direction=E.SORT_DESC, sort_type=TOPK_VALUE, index_
     return r[0].as_tensor(), r[1].as_tensor()
 
 
+BOXES_NMS, BOXES_SSD = range(2)
+NMS_CAFFE, NMS_MXNET, NMS_OV = range(3)
+
+
+def nms(Boxes, Scores, iou_threshold, score_threshold, max_output_boxes_per_class, soft_nms_sigma=0.0,
+        center_point_box=False, sort_result_descending=False, box_output_type=E.DType.INT32,
+        boxes_decode_mode=BOXES_NMS, clip_before_nms=False, clip_after_nms=False, ssd_input_height=0,
+        ssd_input_width=0, ssd_variances=None, ssd_location=None, ssd_with_arm_loc=False, ssd_arm_location=None,
+        nms_style=NMS_OV, share_location=True, hard_suppression=True):
+    """Non-maximum suppression; the arguments and defaults of the C++ builder plaidml::op::nms.  Returns
+    [selected (batch, class, box) triples, (batch, class, score) triples, number of valid selections]."""
+    r = E.op_make('nms', [Boxes, Scores, iou_threshold, score_threshold, int(max_output_boxes_per_class),
+                          float(soft_nms_sigma), bool(center_point_box), bool(sort_result_descending),
+                          int(box_output_type), int(boxes_decode_mode), bool(clip_before_nms), bool(clip_after_nms),
+                          int(ssd_input_height), int(ssd_input_width), ssd_variances, ssd_location,
+                          bool(ssd_with_arm_loc), ssd_arm_location, int(nms_style), bool(share_location),
+                          bool(hard_suppression)]).as_tuple()
+    return [v.as_tensor() for v in r]
+
+
 RESIZE_NEAREST, RESIZE_BILINEAR = range(2)
 
 

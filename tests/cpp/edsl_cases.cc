@@ -315,6 +315,21 @@ void caseOpBuilders() {
     expectClose("mvn", readBuffer<float>(out[2]), {-1.5, -.5, .5, 1.5, -1.5, -.5, .5, 1.5, -1.5, -.5, .5, 1.5}, 1e-6f, 1e-6f);
   }
   {
+    // three boxes of one class: the second overlaps the first (IoU 0.9 / 1.1) and loses, the third stands alone
+    auto Bx = Placeholder(DType::FLOAT32, {1, 3, 4});
+    auto Sc = Placeholder(DType::FLOAT32, {1, 1, 3});
+    auto It = Placeholder(DType::FLOAT32, {1});
+    auto St = Placeholder(DType::FLOAT32, {1});
+    auto R = op::nms(Bx, Sc, It, St, 3).build();
+    auto out = run(buildProgram("nms", {Bx, Sc, It, St}, R),
+                   {makeBuffer<float>(DType::FLOAT32, {1, 3, 4}, {0, 0, 1, 1, 0, 0.1f, 1, 1.1f, 2, 2, 3, 3}),
+                    makeBuffer<float>(DType::FLOAT32, {1, 1, 3}, {0.9f, 0.8f, 0.7f}), makeBuffer<float>(DType::FLOAT32, {1}, {0.5f}),
+                    makeBuffer<float>(DType::FLOAT32, {1}, {0.0f})});
+    expectEq<int32_t>("nms_boxes", readBuffer<int32_t>(out[0]), {0, 0, 0, 0, 0, 2, -1, -1, -1});
+    expectEq<float>("nms_scores", readBuffer<float>(out[1]), {0, 0, 0.9f, 0, 0, 0.7f, -1, -1, -1});
+    expectEq<int32_t>("nms_valid", readBuffer<int32_t>(out[2]), {2});
+  }
+  {
     auto I = Placeholder(DType::INT64, {1, 4, 6, 6});
     Tensor O = op::reorg_yolo(I, 2, /*decrease=*/false);
     auto dims = O.compute_shape().sizes();
