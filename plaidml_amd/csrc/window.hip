@@ -417,12 +417,99 @@ hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
   return hipGetLastError();
 }
 
+namespace {
+
+// Whole-image pooling (one output pixel per image): the outputs alone are too few threads to keep HBM
+// busy, so eight threads share the taps of one 16-byte channel vector -- thread g takes taps g, g + 8,
+// ... with all of its loads in flight at once -- and the eight partial results are folded through LDS in a
+// fixed order.  A workgroup covers 32 channel vectors of one image.
+template <int ES>
+__global__ __launch_bounds__(256) void pool_whole_kernel(PoolArgs a, int64_t chunks) {
+  constexpr int V = VecIO<ES>::V;
+  constexpr int kShare = 8, kMine = 8;  // up to kShare * kMine taps per pass
+  const pml_hip_pool2d_desc& d = a.d;
+  __shared__ float part[kShare][32][V + 1];
+  const int64_t cvecs = d.c / V;
+  const int64_t n = blockIdx.x / chunks;
+  const int64_t cv = (blockIdx.x % chunks) * 32 + (threadIdx.x & 31);
+  const int g = (int)(threadIdx.x >> 5);
+  const bool live = cv < cvecs;
+  const int64_t taps = d.h * d.w;
+  const float ident = d.agg == PML_HIP_AGG_MAX ? -INFINITY : (d.agg == PML_HIP_AGG_MIN ? INFINITY : 0.f);
+  float acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = ident;
+  const int64_t base = n * taps * d.c + (live ? cv : 0) * V;
+  for (int64_t t0 = g; t0 < taps; t0 += kShare * kMine) {
+    float x[kMine][V];
+#pragma unroll
+    for (int u = 0; u < kMine; ++u) {
+      const int64_t t = t0 + (int64_t)u * kShare;
+      VecIO<ES>::load(a.in, base + (t < taps ? t : 0) * d.c, x[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kMine; ++u) {
+      if (t0 + (int64_t)u * kShare >= taps) break;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        if (d.agg == PML_HIP_AGG_MAX)
+          acc[i] = (x[u][i] > acc[i]) ? x[u][i] : acc[i];
+        else if (d.agg == PML_HIP_AGG_MIN)
+          acc[i] = (x[u][i] < acc[i]) ? x[u][i] : acc[i];
+        else
+          acc[i] += x[u][i];
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < V; ++i) part[g][threadIdx.x & 31][i] = acc[i];
+  __syncthreads();
+  if (g != 0 || !live) return;
+  for (int k = 1; k < kShare; ++k) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float y = part[k][threadIdx.x][i];
+      if (d.agg == PML_HIP_AGG_MAX)
+        acc[i] = (y > acc[i]) ? y : acc[i];
+      else if (d.agg == PML_HIP_AGG_MIN)
+        acc[i] = (y < acc[i]) ? y : acc[i];
+      else
+        acc[i] += y;
+    }
+  }
+  const int64_t o0 = n * d.c + cv * V;
+  if constexpr (ES == 2) {
+    i32x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[2 * i + 1]) << 16));
+    *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+  } else {
+    const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
+    *(f32x4_t*)((float*)a.out + o0) = o;
+  }
+}
+
+}  // namespace
+
 hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s) {
   const pml_hip_pool2d_desc& d = a.d;
   const int es = dt_size(d.dtype);
   const int V = 16 / es;
   const int64_t total = d.n * d.oh * d.ow * (d.c / V);
   if (total == 0) return hipSuccess;
+  const bool whole = d.oh == 1 && d.ow == 1 && d.kh == d.h && d.kw == d.w && d.pad_h == 0 && d.pad_w == 0 && !d.with_index &&
+                     (d.dtype == PML_HIP_BF16 || d.dtype == PML_HIP_F32) && d.h * d.w >= 16;
+  if (whole) {
+    const int64_t chunks = (d.c / V + 31) / 32;
+    if (d.n * chunks <= 0x7fffffff) {
+      if (es == 2)
+        hipLaunchKernelGGL((pool_whole_kernel<2>), dim3((unsigned)(d.n * chunks)), dim3(256), 0, s, a, chunks);
+      else
+        hipLaunchKernelGGL((pool_whole_kernel<4>), dim3((unsigned)(d.n * chunks)), dim3(256), 0, s, a, chunks);
+      return hipGetLastError();
+    }
+  }
   if (es == 2 && d.with_index)
     hipLaunchKernelGGL((pool2d_kernel<2, true>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
   else if (es == 2)

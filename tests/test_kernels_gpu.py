@@ -484,3 +484,37 @@ def test_dwconv_pool_bf16():
     np.testing.assert_array_equal(ix, ao)
     hk.lib().pml_hip_plan_free(plan)
     hk.lib().pml_hip_plan_free(plan2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('kind,agg,N,H,W,C', [
+    ('bf16', 'add', 3, 7, 7, 2048), ('bf16', 'max', 2, 7, 7, 264), ('bf16', 'min', 2, 10, 13, 64),
+    ('f32', 'add', 2, 7, 7, 516), ('f32', 'max', 1, 9, 8, 128), ('f32', 'add', 2, 4, 4, 36), ('bf16', 'add', 2, 3, 3, 64)])
+def test_pool_whole_image(kind, agg, N, H, W, C):
+    """Pooling over the whole image (taps shared by eight threads when there are at least 16; the plain window
+    kernel below that) against numpy: max / min exactly, sums to the accumulation tolerance."""
+    print('whole-image pool', kind, agg, N, H, W, C, flush=True)
+    rng = np.random.default_rng(N * 1000 + C)
+    Iv = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    if kind == 'bf16':
+        Iv = E.round_bf16(Iv)
+    p = hk.Pool2dDesc()
+    p.dtype = hk.BF16 if kind == 'bf16' else hk.F32
+    p.agg = {'add': hk.AGG_ADD, 'max': hk.AGG_MAX, 'min': hk.AGG_MIN}[agg]
+    p.n, p.h, p.w, p.c, p.kh, p.kw, p.oh, p.ow = N, H, W, C, H, W, 1, 1
+    p.stride_h = p.stride_w = 1
+    plan = hk.lib().pml_hip_pool2d_dispatch(ctypes.byref(p))
+    assert plan, hk.lib().pml_hip_last_error()
+    es = 2 if kind == 'bf16' else 4
+    dI = hk.DeviceBuffer.from_numpy(bf16(Iv) if kind == 'bf16' else Iv)
+    dO = hk.DeviceBuffer(N * C * es)
+    hk.check(hk.lib().pml_hip_pool2d_invoke(plan, dI.ptr, dO.ptr, None, None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    out = E.bf16_from_bits(dO.to_numpy(np.uint16, (N, C))) if kind == 'bf16' else dO.to_numpy(np.float32, (N, C))
+    flat = Iv.reshape(N, H * W, C)
+    if agg == 'add':
+        ref = flat.astype(np.float64).sum(1)
+        np.testing.assert_allclose(out, ref, rtol=BF16_RTOL if kind == 'bf16' else 1e-5, atol=2e-2 if kind == 'bf16' else 1e-5)
+    else:
+        np.testing.assert_array_equal(out, flat.max(1) if agg == 'max' else flat.min(1))
+    hk.lib().pml_hip_plan_free(plan)
