@@ -861,7 +861,7 @@ def min(x, y):  # noqa: A001
 class Contraction:
     def __init__(self, name=''):
         self.name = name
-        self._dims = self._idxs = None
+        self._dims, self._idxs = [], []  # no outShape / outAccess: a scalar result
         self._agg = None
         self._rhs = None
         self._init = None

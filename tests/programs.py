@@ -215,6 +215,117 @@ def float_chains(E, op, dtype_name='FLOAT32', inner=40):
     return E.Program('float_chains', [A, B, col, row, one], outs), vals, FP32 if dtype_name == 'FLOAT32' else BF16
 
 
+def batched_dots(E, op):
+    """CppEdsl.HighDimDot / OuterDimDot, plaidml/edsl/tests/edsl_test.cc:418-446: a dot under three batch
+    dimensions, once with the contracted dimension innermost and once with it second."""
+    M, N, K, X, Y, Z = 8, 32, 16, 5, 4, 4
+    A = E.Placeholder(E.DType.FLOAT32, [X, Y, Z, M, K])
+    B = E.Placeholder(E.DType.FLOAT32, [X, Y, Z, K, N])
+    A2 = E.Placeholder(E.DType.FLOAT32, [X, K, Y, Z, M])
+    B2 = E.Placeholder(E.DType.FLOAT32, [X, K, Y, Z, N])
+    m, n, k, x, y, z = E.TensorIndexes(6)
+    C = E.Contraction().outShape(X, Y, Z, M, N).outAccess(x, y, z, m, n).sum(A[x, y, z, m, k] * B[x, y, z, k, n]).build()
+    C2 = E.Contraction().outShape(X, Y, Z, M, N).outAccess(x, y, z, m, n).sum(A2[x, k, y, z, m] * B2[x, k, y, z, n]).build()
+    r = _rng(41)
+    vals = [r.standard_normal(s).astype(np.float32) for s in ((X, Y, Z, M, K), (X, Y, Z, K, N), (X, K, Y, Z, M), (X, K, Y, Z, N))]
+    return E.Program('batched_dots', [A, B, A2, B2], [C, C2]), vals, FP32
+
+
+def double_dot_dup_out(E, op):
+    """CppEdsl.DoubleDot / DupOut, edsl_test.cc:547-563, 1084-1100: dot(dot(A, B), C) returned three times."""
+    A = E.Placeholder(E.DType.FLOAT32, [10, 20])
+    B = E.Placeholder(E.DType.FLOAT32, [20, 30])
+    C = E.Placeholder(E.DType.FLOAT32, [30, 40])
+    R = op.dot(op.dot(A, B), C)
+    r = _rng(42)
+    return E.Program('dup_out', [A, B, C], [R, R, R]), [r.standard_normal(s).astype(np.float32)
+                                                        for s in ((10, 20), (20, 30), (30, 40))], FP32
+
+
+def mnist_mlp(E, op):
+    """CppEdsl.MnistMlp, edsl_test.cc:645-662: 784 -> 512 -> 512 -> 10, relu, relu, softmax."""
+    f32 = E.DType.FLOAT32
+    shapes = [(1, 784), (784, 512), (512,), (512, 512), (512,), (512, 10), (10,)]
+    X, K1, b1, K2, b2, K3, b3 = [E.Placeholder(f32, list(s)) for s in shapes]
+    d1 = op.relu(op.dot(X, K1) + b1)
+    d2 = op.relu(op.dot(d1, K2) + b2)
+    Y = op.softmax(op.dot(d2, K3) + b3, 1)
+    r = _rng(43)
+    vals = [(r.standard_normal(s) * (0.05 if len(s) == 2 and s[0] > 1 else 1.0)).astype(np.float32) for s in shapes]
+    return E.Program('mnist_mlp', [X, K1, b1, K2, b2, K3, b3], [Y]), vals, FP32
+
+
+def mnist_cnn(E, op, side=28):
+    """CppEdsl.MnistCnn, edsl_test.cc:664-769, at 28 x 28 (the reference builds it at 224 x 224 and only runs it):
+    two SAME 3x3 convolutions written as contractions, the 2x2 max pool with its two constraints, flatten by
+    reshape, two dense layers, softmax."""
+    f32 = E.DType.FLOAT32
+
+    def conv(I, K):
+        N, X0, X1, CI = I.shape if not callable(getattr(I, 'shape', None)) else I.compute_shape().sizes
+        K0, K1, _, CO = K.shape if not callable(getattr(K, 'shape', None)) else K.compute_shape().sizes
+        n, x0, x1, co, ci, k0, k1 = E.TensorIndexes(7)
+        return E.Contraction().outShape(N, X0, X1, CO).outAccess(n, x0, x1, co).sum(
+            I[n, x0 + k0 - (K0 // 2), x1 + k1 - (K1 // 2), ci] * K[k0, k1, ci, co]).build()
+
+    def pool(I):
+        N, X0, X1, C = I.shape if not callable(getattr(I, 'shape', None)) else I.compute_shape().sizes
+        n, x0, x1, i, j, c = E.TensorIndexes(6)
+        return E.Contraction().outShape(N, (X0 + 1) // 2, (X1 + 1) // 2, C).outAccess(n, x0, x1, c).max(
+            I[n, 2 * x0 + i, 2 * x1 + j, c]).add_constraint(i < 2).add_constraint(j < 2).build()
+
+    flat = (side // 2) * (side // 2) * 64
+    shapes = [(1, side, side, 1), (3, 3, 1, 32), (32,), (3, 3, 32, 64), (64,), (flat, 128), (128,), (128, 100), (100,)]
+    X, K1, b1, K2, b2, K3, b3, K4, b4 = [E.Placeholder(f32, list(s)) for s in shapes]
+    c1 = op.relu(conv(X, K1) + b1)
+    c2 = op.relu(conv(c1, K2) + b2)
+    p1 = pool(c2)
+    fl = E.reshape(p1, [1, flat])
+    d1 = op.relu(op.dot(fl, K3) + b3)
+    Y = op.softmax(op.dot(d1, K4) + b4, 1)
+    r = _rng(44)
+    vals = [(r.standard_normal(s) * (0.1 if len(s) > 1 and s != shapes[0] else 1.0)).astype(np.float32) for s in shapes]
+    vals[5] = (vals[5] * 0.1).astype(np.float32)
+    return E.Program('mnist_cnn', [X, K1, b1, K2, b2, K3, b3, K4, b4], [Y]), vals, FP32
+
+
+def lars_momentum4d(E, op):
+    """CppEdsl.LarsMomentum4d, edsl_test.cc:796-830: two whole-tensor norms (contractions into a scalar) steer an
+    elementwise update; the learning rate is a rank-0 input."""
+    f32 = E.DType.FLOAT32
+    shape = [4, 7, 3, 9]
+    X, G, V = [E.Placeholder(f32, shape) for _ in range(3)]
+    LR = E.Placeholder(f32, [])
+
+    def norm(T):
+        idxs = E.TensorIndexes(4)
+        return E.sqrt(E.Contraction().sum((T * T)[idxs]).build())
+
+    coeff, decay, momentum = 1. / 1024., 1. / 2048., 1. / 8.
+    xn, gn = norm(X), norm(G)
+    loc = LR * coeff * xn / (gn + decay * xn)
+    nv = momentum * V + loc * (G + decay * X)
+    r = _rng(45)
+    vals = [r.standard_normal(shape).astype(np.float32) for _ in range(3)] + [np.array(0.5, np.float32)]
+    return E.Program('lars_momentum4d', [X, G, V, LR], [X - nv, nv]), vals, FP32
+
+
+def repeat_and_global_min(E, op):
+    """CppEdsl.RepeatElements (edsl_test.cc:856-875: out[n0, 3 n1 + k, n2] = in[n0, n1, n2], k < 3), GlobalMin
+    (:895-907: -max(-I) over everything) and UniqueNames (:877-893: two inputs share a name)."""
+    f32 = E.DType.FLOAT32
+    I = E.Placeholder(f32, [10, 10, 10])
+    n0, n1, n2, k = E.TensorIndexes(4)
+    O = E.Contraction().outShape(10, 30, 10).outAccess(n0, 3 * n1 + k, n2).assign(I[n0, n1, n2]).add_constraint(k < 3).build()
+    i, j, l = E.TensorIndexes(3)
+    M = -(E.Contraction().max((-I)[i, j, l]).build())
+    A, B = E.Placeholder(f32, [1], name='A'), E.Placeholder(f32, [1], name='B')
+    C0, C1 = E.Placeholder(f32, [1], name='C'), E.Placeholder(f32, [1], name='C')
+    r = _rng(46)
+    vals = [r.standard_normal((10, 10, 10)).astype(np.float32)] + [np.array([v], np.float32) for v in (1, 2, 4, 8)]
+    return E.Program('repeat_min_names', [I, A, B, C0, C1], [O, M, A + B + C0 + C1]), vals, EXACT
+
+
 def u64_add(E, op):
     """CppEdsl.Add, plaidml/edsl/tests/edsl_test.cc:335-374 (64-bit integer elementwise)."""
     A = E.Placeholder(E.DType.UINT64, [3, 3])
@@ -392,6 +503,12 @@ ALL = {
     'float_chains_f32': float_chains,
     'float_chains_bf16': lambda E, op: float_chains(E, op, 'BFLOAT16'),
     'float_chains_f32_ragged': lambda E, op: float_chains(E, op, 'FLOAT32', inner=37),
+    'batched_dots': batched_dots,
+    'double_dot_dup_out': double_dot_dup_out,
+    'mnist_mlp': mnist_mlp,
+    'mnist_cnn': mnist_cnn,
+    'lars_momentum4d': lars_momentum4d,
+    'repeat_and_global_min': repeat_and_global_min,
     'u64_add': u64_add,
     'higher_precision_constants': higher_precision_constants,
     'config0_gemm_f32': config0_gemm_f32,
