@@ -662,7 +662,9 @@ inline std::ostream& operator<<(std::ostream& os, const Value& x) { return os <<
 
 using Dictionary = std::unordered_map<std::string, Value>;
 
-// Layers group operations for readers of the program text; this backend inlines them.
+// Layers group operations for readers of the program text; this backend inlines them.  The operand list is
+// not checked: a body that reads a tensor missing from it builds here, where the reference rejects the
+// program (plaidml/edsl/tests/edsl_test.cc:2200-2205).
 inline Tensor layer(const std::string&, const TensorVec&, const Dictionary&, const std::function<Tensor()>& fn) { return fn(); }
 inline Tensor layer(const std::string&, const TensorVec&, const std::function<Tensor()>& fn) { return fn(); }
 inline TensorVec layer(const std::string&, const TensorVec&, const Dictionary&, const std::function<TensorVec()>& fn) { return fn(); }

@@ -433,6 +433,70 @@ void caseErrors() {
   fail("arity_error", "no exception");
 }
 
+template <typename F>
+void expectThrows(const char* name, F&& fn) {
+  try {
+    fn();
+  } catch (const std::exception&) {
+    std::printf("ok %s\n", name);
+    return;
+  }
+  fail(name, "no exception");
+}
+
+// The misuse cases of plaidml/edsl/tests/edsl_test.cc:2274-2398 and its layer / trace cases (:2110-2345).
+void caseReferenceErrors() {
+  expectThrows("bad_data_type", [] { auto A = Placeholder(DType::INVALID, {10, 20}); });
+  expectThrows("index_without_dims", [] { plaidml::edsl::index(std::vector<TensorDim>{}, 0); });
+  expectThrows("index_unbound_dim", [] {
+    TensorDim X0;
+    plaidml::edsl::index({X0}, 0);
+  });
+  {
+    TensorDim X0, X1;
+    auto I = Placeholder(DType::FLOAT32, {10, 3});
+    I.bind_dims(X0, X1);
+    Tensor O = plaidml::edsl::index({X0}, 0);
+    auto out = run(buildProgram("IndexOp", {}, {O}), {});
+    expectEq<int32_t>("index_op", readBuffer<int32_t>(out[0]), {0, 1, 2, 3, 4, 5, 6, 7, 8, 9});
+  }
+  expectThrows("bind_bad_dims", [] {
+    auto X = Placeholder(DType::FLOAT32, {10, 10});
+    auto Y = Placeholder(DType::FLOAT32, {12, 10});
+    TensorDim I, J, K;
+    X.bind_dims({I, K});
+    Y.bind_dims({K, J});
+  });
+  expectThrows("eltwise_mismatch", [] {
+    auto X = Placeholder(DType::FLOAT32, {10, 10});
+    auto Y = Placeholder(DType::FLOAT32, {12, 10});
+    auto O = X + Y;
+  });
+  expectThrows("op_operators", [] {
+    auto X = Placeholder(DType::FLOAT32, {10, 10});
+    auto Y = Placeholder(DType::FLOAT32, {12, 12});
+    auto O = op::relu(X) + op::relu(Y);
+  });
+  {
+    auto A = Placeholder(DType::FLOAT32, {2, 2});
+    expectThrows("layer_exception", [&] { layer("sum", {A}, [&]() -> Tensor { throw std::runtime_error("exception"); }); });
+    Tensor B = layer("sum", {A}, [&]() { return A + Constant(makeBuffer<float>(DType::FLOAT32, {2, 2}, {1, 2, 3, 4}), "C"); });
+    Tensor O = layer("sum", {B}, [&]() { return trace(B, "msg") + Constant(makeBuffer<float>(DType::FLOAT32, {2, 2}, {1, 2, 3, 4}), "C"); });
+    auto out = run(buildProgram("LayerMulti", {A}, {O}), {makeBuffer<float>(DType::FLOAT32, {2, 2}, {10, 20, 30, 40})});
+    expectEq<float>("layer_multi", readBuffer<float>(out[0]), {12, 24, 36, 48});
+  }
+  {
+    auto A = Placeholder(DType::FLOAT32, {3, 2});
+    TensorVec both = layer("two_output", {A}, {}, [&]() {
+      Tensor idxs = argsort(A, 0);
+      Tensor vals = gather(A, idxs);
+      return TensorVec{vals, idxs};
+    });
+    auto out = run(buildProgram("LayerMultipleReturnValues", {A}, both), {makeBuffer<float>(DType::FLOAT32, {3, 2}, {3, 9, 1, 8, 2, 7})});
+    expectEq<int32_t>("layer_two_outputs_positions", readBuffer<int32_t>(out[1]), {1, 2, 2, 1, 0, 0});
+  }
+}
+
 }  // namespace
 
 int main() {
@@ -456,6 +520,7 @@ int main() {
     caseSpecialOps();
     caseLens();
     caseErrors();
+    caseReferenceErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAILED with exception: %s\n", e.what());
     return 1;
