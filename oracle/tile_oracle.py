@@ -360,6 +360,8 @@ class Tensor:
             dims = dims[0]
         if len(dims) != len(self.shape):
             raise ValueError('Rank mismatch in bind_dims')
+        if self._lens is not None:
+            dims = self._lens.apply(list(dims))
         for d, s in zip(dims, self.shape):
             if d.value is None:
                 d.value = s
@@ -376,9 +378,18 @@ class Tensor:
     def rank(self):
         return len(self.shape)
 
+    _lens = None  # a TensorLens set by use(): dimensions and indexes are then given in the lens's source order
+
+    def use(self, lens):
+        """The same values seen through `lens` (plaidml/edsl/__init__.py:645-646)."""
+        t = intrinsic('ident', self)
+        t._lens = lens
+        return t
+
     def __getitem__(self, key):
         if not isinstance(key, (tuple, list)):
             key = (key,)
+        key = list(key) if self._lens is None else self._lens.apply(list(key))
         return IndexedTensor('none', ref=self, idxs=[TensorIndex._wrap(k) for k in key])
 
     # --- eltwise operators ---
@@ -858,8 +869,37 @@ def min(x, y):  # noqa: A001
     return select(_literal(x) < y, x, y)
 
 
+class TensorLens:
+    """plaidml/edsl/__init__.py:292-309: position i of what the user writes (in `source` order) lands where the
+    letter source[i] stands in `target`."""
+
+    def __init__(self, source='', target=''):
+        if len(source) != len(target):
+            raise ValueError('source and target rank mismatch')
+        self.map = []
+        for ch in source:
+            pos = target.find(ch)
+            if pos == -1:
+                raise ValueError('source and target dims mismatch')
+            self.map.append(pos)
+
+    def apply(self, items):
+        if not self.map:
+            return items
+        if len(items) != len(self.map):
+            raise ValueError('rank mismatch in TensorLens apply')
+        return [items[x] for x in self.map]
+
+
+def trace(x, msg):
+    return x
+
+
 class Contraction:
-    def __init__(self, name=''):
+    def __init__(self, lens=None, name=''):
+        if isinstance(lens, str):
+            lens, name = None, lens
+        self._lens = lens
         self.name = name
         self._dims, self._idxs = [], []  # no outShape / outAccess: a scalar result
         self._agg = None
@@ -928,8 +968,10 @@ class Contraction:
         for o in operands:
             if len(o.idxs) != len(o.ref.shape):
                 raise ValueError('rank mismatch in contraction operand')
-        return Tensor('contraction', dt, self._dims, srcs,
-                      {'agg': self._agg, 'combo': combo, 'sink': self._idxs,
+        dims = self._dims if self._lens is None else self._lens.apply(list(self._dims))
+        sink = self._idxs if self._lens is None else self._lens.apply(list(self._idxs))
+        return Tensor('contraction', dt, dims, srcs,
+                      {'agg': self._agg, 'combo': combo, 'sink': sink,
                        'accs': [o.idxs for o in operands], 'cons': list(self._cons),
                        'init': self._init, 'name': self.name})
 

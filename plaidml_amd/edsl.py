@@ -466,9 +466,18 @@ class Tensor(_Handle):
         p, self._ptr = self._ptr, None
         return p
 
+    _lens = None  # a TensorLens set by use(): dimensions and indexes are then given in the lens's source order
+
+    def use(self, lens):
+        """The same tensor seen through `lens` (plaidml/edsl/__init__.py:645-646)."""
+        t = Tensor(ptr=call('plaidml_expr_clone', self._ptr))
+        t._lens = lens
+        return t
+
     def __getitem__(self, key):
         if not isinstance(key, (tuple, list)):
             key = (key,)
+        key = list(key) if self._lens is None else self._lens.apply(list(key))
         return IndexedTensor('none', ref=self, idxs=[_wrap_poly(k) for k in key])
 
     def __neg__(self):
@@ -577,14 +586,40 @@ class Tensor(_Handle):
     def bind_dims(self, *dims):
         if len(dims) == 1 and isinstance(dims[0], (list, tuple)):
             dims = dims[0]
+        dims = list(dims) if self._lens is None else self._lens.apply(list(dims))
         call('plaidml_expr_bind_dims', self._ptr, len(dims), _ptr_array([d.as_ptr() for d in dims]))
 
     def __str__(self):
         return _take_str(call('plaidml_expr_repr', self._ptr))
 
 
+class TensorLens:
+    """A change of dimension order: position i of what the user writes (in `source` order) lands where the
+    letter source[i] stands in `target` (plaidml/edsl/__init__.py:292-309)."""
+
+    def __init__(self, source='', target=''):
+        if len(source) != len(target):
+            raise ValueError('source and target rank mismatch')
+        self.map = []
+        for ch in source:
+            pos = target.find(ch)
+            if pos == -1:
+                raise ValueError('source and target dims mismatch')
+            self.map.append(pos)
+
+    def apply(self, items):
+        if not self.map:
+            return items
+        if len(items) != len(self.map):
+            raise ValueError('rank mismatch in TensorLens apply')
+        return [items[x] for x in self.map]
+
+
 class Contraction:
-    def __init__(self, name=''):
+    def __init__(self, lens=None, name=''):
+        if isinstance(lens, str):  # Contraction('name')
+            lens, name = None, lens
+        self._lens = lens
         self._name = name
         self._dims, self._idxs, self._agg, self._rhs, self._init, self._cons = [], [], None, None, None, []
 
@@ -635,8 +670,10 @@ class Contraction:
         rhs = self._rhs
         if isinstance(rhs, Tensor):
             rhs = IndexedTensor('none', ref=rhs, idxs=[])
-        t = Tensor(ptr=call('plaidml_expr_contraction', _AGG[self._agg], _COMBO[rhs._op], len(self._idxs),
-                            _ptr_array([i.as_ptr() for i in self._idxs]), _ptr_array([d.as_ptr() for d in self._dims]),
+        idxs = self._idxs if self._lens is None else self._lens.apply(self._idxs)
+        dims = self._dims if self._lens is None else self._lens.apply(self._dims)
+        t = Tensor(ptr=call('plaidml_expr_contraction', _AGG[self._agg], _COMBO[rhs._op], len(idxs),
+                            _ptr_array([i.as_ptr() for i in idxs]), _ptr_array([d.as_ptr() for d in dims]),
                             self._init.as_ptr() if self._init is not None else None, self._name.encode()))
         operands = [rhs] if rhs._op == 'none' else rhs._args
         for o in operands:
@@ -777,6 +814,11 @@ def gather(x, y, axis=0, interpolation_mode=INTERP_NONE, nearest_mode=NEAREST_RO
         axis += x.rank
     return intrinsic('gather', x, y, _uint(axis), _uint(interpolation_mode), _uint(nearest_mode), _float(cube_coeff), _uint(mode),
                      _uint(batch_dims), _uint(out_of_bounds_mode))
+
+
+def trace(x, msg):
+    """A trace marker passes its tensor through (the reference prints `msg` when the value is computed)."""
+    return x
 
 
 def scatter(x, y, z, axis=0, mode=SCATTER_NORMAL):

@@ -326,6 +326,72 @@ def repeat_and_global_min(E, op):
     return E.Program('repeat_min_names', [I, A, B, C0, C1], [O, M, A + B + C0 + C1]), vals, EXACT
 
 
+def python_front_end_cases(E, op):
+    """The small cases of plaidml/edsl/tests/edsl_test.py: test_cast_scalar (:265, a rank-0 input), test_cast_folder
+    (:271, a cast to the same type), test_funky_names (:462, a program name that is no identifier), test_identity and
+    test_two_outputs (:482, :513: an input returned as is, twice), test_trace (:573)."""
+    S = E.Placeholder(E.DType.INT32, [])
+    V = E.Placeholder(E.DType.INT32, [3])
+    I = E.Placeholder(E.DType.FLOAT32, [3], name='I')
+    K = E.Placeholder(E.DType.FLOAT32, [3], name='K')
+    i, j = E.TensorIndexes(2)
+    F = E.Contraction().outShape(5).outAccess(i).sum(I[(i - j + 1) // 2] * K[j]).build()
+    outs = [E.cast(S, E.DType.FLOAT32), E.cast(V, E.DType.INT32), F, I, I, E.trace(K, 'msg')]
+    vals = [np.array(3, np.int32), np.array([1, 2, 3], np.int32), np.array([1, 2, 3], np.float32), np.array([1, 2, 3], np.float32)]
+    return E.Program('this-is-not an identifier', [S, V, I, K], outs), vals, EXACT
+
+
+def python_conv_cases(E, op):
+    """test_conv_1d (:277), test_conv_2d_dilated (:284), test_complex_conv_2d (:291, grouped, strided, dilated,
+    SAME_LOWER; its first spatial access reads x1 where x0 is meant, and so does this restatement) and test_lens
+    (:578, the same convolution written through NHWC/HWCK and NCHW/CKHW lenses), at reduced image sizes."""
+    f32 = E.DType.FLOAT32
+
+    def conv_1d(I, K):
+        N, X, KX, CI, CO = E.TensorDims(5)
+        n, x, k, ci, co = E.TensorIndexes(5)
+        I.bind_dims(N, X, CI)
+        K.bind_dims(KX, CI, CO)
+        return E.Contraction().outShape(N, X - KX + 1, CO).outAccess(n, x, co).sum(I[n, x + k, ci] * K[k, ci, co]).build()
+
+    def conv_2d_dilated(I, K):
+        N, X, Y, KX, KY, CI, CO = E.TensorDims(7)
+        n, x, y, kx, ky, ci, co = E.TensorIndexes(7)
+        I.bind_dims(N, X, Y, CI)
+        K.bind_dims(KX, KY, CI, CO)
+        return E.Contraction().outShape(N, X - 2 * (KX - 1), Y - 3 * (KY - 1), CO).outAccess(n, x, y, co).sum(
+            I[n, x + 2 * kx, y + 3 * ky, ci] * K[kx, ky, ci, co]).build()
+
+    def complex_conv_2d(I, K, s0, s1, d0, d1):
+        N, G, GCI, GCO, X0, X1, K0, K1 = E.TensorDims(8)
+        n, g, gci, gco, x0, x1, k0, k1 = E.TensorIndexes(8)
+        I.bind_dims(N, X0, X1, G, GCI)
+        K.bind_dims(K0, K1, G, GCI, GCO)
+        Y0, Y1 = (X0 + s0 - 1) // s0, (X1 + s1 - 1) // s1
+        EK0, EK1 = d0 * (K0 - 1) + 1, d1 * (K1 - 1) + 1
+        P0, P1 = ((Y0 - 1) * s0 + EK0 - X0) // 2, ((Y1 - 1) * s1 + EK1 - X1) // 2
+        return E.Contraction().outShape(N, Y0, Y1, G, GCO).outAccess(n, x0, x1, g, gco).sum(
+            I[n, s0 * x1 + d0 * k0 - P0, s1 * x1 + d1 * k1 - P1, g, gci] * K[k0, k1, g, gci, gco]).build()
+
+    def conv_2d(I, K, I_layout, K_layout):
+        I_lens, K_lens = E.TensorLens(I_layout, 'NHWC'), E.TensorLens(K_layout, 'HWCK')
+        I, K = I.use(I_lens), K.use(K_lens)
+        CI, CO, K0, K1, N, X0, X1 = E.TensorDims(7)
+        n, x0, x1, k0, k1, ci, co = E.TensorIndexes(7)
+        I.bind_dims(N, X0, X1, CI)
+        K.bind_dims(K0, K1, CI, CO)
+        return E.Contraction(I_lens).outShape(N, X0 - (K0 - 1), X1 - (K1 - 1), CO).outAccess(n, x0, x1, co).sum(
+            I[n, x0 + k0 - (K0 // 2), x1 + k1 - (K1 // 2), ci] * K[k0, k1, ci, co]).build()
+
+    shapes = [(1, 24, 3), (3, 3, 1), (1, 20, 22, 1), (3, 3, 1, 8), (1, 12, 14, 3, 3), (3, 3, 3, 3, 8), (1, 1, 1, 1, 1),
+              (1, 1, 1, 1, 1), (1, 12, 12, 3), (3, 3, 3, 8), (1, 3, 12, 12), (3, 8, 5, 5)]
+    P = [E.Placeholder(f32, list(s)) for s in shapes]
+    outs = [conv_1d(P[0], P[1]), conv_2d_dilated(P[2], P[3]), complex_conv_2d(P[4], P[5], 1, 2, 1, 2),
+            complex_conv_2d(P[6], P[7], 1, 2, 1, 2), conv_2d(P[8], P[9], 'NHWC', 'HWCK'), conv_2d(P[10], P[11], 'NCHW', 'CKHW')]
+    r = _rng(47)
+    return E.Program('python_convs', P, outs), [r.standard_normal(s).astype(np.float32) for s in shapes], FP32
+
+
 def u64_add(E, op):
     """CppEdsl.Add, plaidml/edsl/tests/edsl_test.cc:335-374 (64-bit integer elementwise)."""
     A = E.Placeholder(E.DType.UINT64, [3, 3])
@@ -509,6 +575,8 @@ ALL = {
     'mnist_cnn': mnist_cnn,
     'lars_momentum4d': lars_momentum4d,
     'repeat_and_global_min': repeat_and_global_min,
+    'python_front_end_cases': python_front_end_cases,
+    'python_conv_cases': python_conv_cases,
     'u64_add': u64_add,
     'higher_precision_constants': higher_precision_constants,
     'config0_gemm_f32': config0_gemm_f32,
