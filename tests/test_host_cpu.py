@@ -124,3 +124,27 @@ def test_cpp_cases_fail_loudly_without_a_device():
     res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert res.returncode != 0
     assert 'hip' in res.stderr.lower()
+
+
+def test_placeholder_shapes_and_collected_passes():
+    """test_placeholder and test_collect_passes, plaidml/edsl/tests/edsl_test.py:534-571."""
+    from plaidml_amd import edsl as E, op
+    assert str(E.Placeholder(E.DType.INT32).compute_shape()) == 'si32'
+    assert str(E.Placeholder(E.DType.INT32, [1, 1]).compute_shape()) == '1x1xsi32'
+    assert str(E.Placeholder(E.DType.INT32, [1, 1], name='I').compute_shape()) == '1x1xsi32'
+    A, B = E.Placeholder(E.DType.FLOAT32, [10, 10]), E.Placeholder(E.DType.FLOAT32, [10, 10])
+    program = E.Program('collect_passes', [A, B], [op.dot(A, B)])
+    program.compile(debug=True)
+    assert program.passes[0][0] == 'tile'
+
+
+def test_lens_rejects_mismatched_layouts():
+    """TensorLens, plaidml/edsl/__init__.py:292-309."""
+    from plaidml_amd import edsl as E
+    with pytest.raises(ValueError):
+        E.TensorLens('NHWC', 'NCH')
+    with pytest.raises(ValueError):
+        E.TensorLens('NHWC', 'NCHX')
+    assert E.TensorLens('NCHW', 'NHWC').apply(list('abcd')) == ['a', 'd', 'b', 'c']
+    with pytest.raises(ValueError):
+        E.TensorLens('MN', 'MN').apply([1, 2, 3])
