@@ -39,6 +39,7 @@ for float16, which this oracle treats like bfloat16 (fp32 compute, one rounding)
 
 Pinned by tests/test_oracle_golden.py against these reference-held vectors:
   GEMM_{INT64,UINT64,INT32,INT8,FLOAT32} (plaidml/edsl/examples/gemm.cc:27-90),
+  GEMV_{INT64,UINT64,INT32,INT8,FLOAT32} and GEMVC_INT64 (plaidml/edsl/examples/gemv.cc:39-139),
   FunkySum (plaidml/edsl/tests/edsl_test.cc:2709-2719), test_defract,
   test_defract_short, test_defract_long (plaidml/edsl/tests/edsl_test.py:408-460),
   Max (edsl_test.cc:576-590), Quantize (plaidml/edsl/examples/quantize.cc:25-32),

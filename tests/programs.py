@@ -46,6 +46,28 @@ def gemm_int(E, op, dtype_name='INT32'):
     return E.Program('gemm', [A, B, C], [O]), [a, b, np.ones((3, 3), npdt)], EXACT
 
 
+GEMV_ANSWERS = {  # dtype -> (A, answer); x = y = ones: plaidml/edsl/examples/gemv.cc:56-139
+    'INT64': ([1] * 9, [4, 4, 4]), 'UINT64': ([1] * 9, [4, 4, 4]), 'INT32': ([1] * 9, [4, 4, 4]),
+    'INT8': ([1] * 9, [4, 4, 4]), 'FLOAT32': ([1, 0.5, 1, 1, 1, 1, 1, 0.6, 1], [3.5, 4, 3.6]),
+}
+
+
+def gemv(E, op, dtype_name='INT32'):
+    """ExampleCppEdsl.GEMV_* and GEMVC_INT64, plaidml/edsl/examples/gemv.cc:14-139: A x + y, and (5 A) x + 4 y
+    (answer 19 19 19 on all-ones inputs); plus MaxPool1D on three elements (max_pool_1d.cc:30-35, :65-68)."""
+    dt = getattr(E.DType, dtype_name)
+    npdt = np.dtype(dtype_name.lower())
+    A, x, y = E.Placeholder(dt, [3, 3]), E.Placeholder(dt, [3]), E.Placeholder(dt, [3])
+    i, j = E.TensorIndexes(2)
+    O = E.Contraction().outShape(3).outAccess(i).sum(A[i, j] * x[j]).build() + y
+    i2, j2 = E.TensorIndexes(2)
+    O2 = E.Contraction().outShape(3).outAccess(i2).sum((A * 5)[i2, j2] * x[j2]).build() + y * 4
+    i3, j3 = E.TensorIndexes(2)
+    P = E.Contraction().outShape(1).outAccess(i3).max(y[2 * i3 + j3]).add_constraint(j3 < 2).build()
+    a = np.array(GEMV_ANSWERS[dtype_name][0], npdt).reshape(3, 3)
+    return E.Program('gemv', [A, x, y], [O, O2, P]), [a, np.ones(3, npdt), np.ones(3, npdt)], EXACT
+
+
 def funky_sum(E, op):
     """CppEdsl.FunkySum, plaidml/edsl/tests/edsl_test.cc:2709-2719: fractional index polynomial."""
     I = E.Placeholder(E.DType.FLOAT32, [3])
@@ -552,6 +574,11 @@ ALL = {
     'gemm_int64': lambda E, op: gemm_int(E, op, 'INT64'),
     'gemm_uint64': lambda E, op: gemm_int(E, op, 'UINT64'),
     'gemm_int8': lambda E, op: gemm_int(E, op, 'INT8'),
+    'gemv_int64': lambda E, op: gemv(E, op, 'INT64'),
+    'gemv_uint64': lambda E, op: gemv(E, op, 'UINT64'),
+    'gemv_int32': lambda E, op: gemv(E, op, 'INT32'),
+    'gemv_int8': lambda E, op: gemv(E, op, 'INT8'),
+    'gemv_float32': lambda E, op: gemv(E, op, 'FLOAT32'),
     'funky_sum': funky_sum,
     'defract_long': defract_long,
     'max_rows': max_rows,

@@ -329,3 +329,17 @@ def test_bf16_rounding_is_nearest_even():
     assert r[0] == 1.0 and r[1] == 1.0 and r[2] == np.float32(1.015625) and r[3] == -2.5
     assert np.isinf(r[4])
     np.testing.assert_array_equal(E.bf16_from_bits(E.bf16_bits(r[:4])), r[:4])
+
+
+@pytest.mark.parametrize('dtype_name', ['INT64', 'UINT64', 'INT32', 'INT8', 'FLOAT32'])
+def test_gemv_known_answers(dtype_name):
+    """plaidml/edsl/examples/gemv.cc:39-139: A x + y for five element types, and (5 A) x + 4 y = 19 19 19."""
+    import programs
+    from oracle import tile_oplib as Oop
+    prog, vals, _ = programs.gemv(E, Oop, dtype_name)
+    o, o2, p = E.run(prog, vals)
+    want = np.array(programs.GEMV_ANSWERS[dtype_name][1], o.dtype)
+    np.testing.assert_array_equal(o, want)
+    if dtype_name == 'INT64':
+        np.testing.assert_array_equal(o2, [19, 19, 19])
+    np.testing.assert_array_equal(p, [1])
