@@ -148,3 +148,32 @@ def test_cpp_header_api_cases():
     print(res.stdout, res.stderr, flush=True)
     assert res.returncode == 0, res.stderr
     assert 'all cases passed' in res.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype_name', ['FLOAT32', 'BFLOAT16'])
+def test_row_reductions_at_size(dtype_name):
+    """Row sum / max / min of a 2048 x 3000 matrix and the sum of everything, against numpy: the maxima exactly, the
+    sums to the accumulation tolerance (fp32 partial sums per lane, folded across the wavefront)."""
+    print('row reductions at size', dtype_name, flush=True)
+    from oracle.tile_oracle import round_bf16
+    rows, cols = 2048, 3000
+    x = np.random.default_rng(51).standard_normal((rows, cols)).astype(np.float32)
+    if dtype_name == 'BFLOAT16':
+        x = round_bf16(x)
+    X = E.Placeholder(getattr(E.DType, dtype_name), [rows, cols])
+    i, j = E.TensorIndexes(2)
+    outs = [E.Contraction().outShape(rows).outAccess(i).sum(X[i, j]).build(),
+            E.Contraction().outShape(rows).outAccess(i).max(X[i, j]).build(),
+            E.Contraction().outShape(rows).outAccess(i).min(X[i, j]).build(),
+            E.Contraction().sum(X[i, j]).build()]
+    s, mx, mn, total = E.run(E.Program('rows', [X], outs), [x], target='hip')
+    np.testing.assert_array_equal(mx, x.max(1))
+    np.testing.assert_array_equal(mn, x.min(1))
+    exact = x.astype(np.float64).sum(1)
+    if dtype_name == 'BFLOAT16':
+        np.testing.assert_allclose(s, exact, rtol=1e-2, atol=0.5)      # one bf16 rounding of a sum of magnitude ~55
+        np.testing.assert_allclose(total, exact.sum(), rtol=1e-2, atol=16)
+    else:
+        np.testing.assert_allclose(s, exact, rtol=1e-4, atol=1e-3)
+        np.testing.assert_allclose(total, exact.sum(), rtol=1e-4, atol=0.5)
