@@ -378,6 +378,7 @@ int pml_hip_scatter(const pml_hip_scatter_desc* desc, const void* data, const vo
 /* argsort along `axis`: out (si32, shape of the input) holds the positions of the input's elements in
  * ascending (direction 0) or descending (1) order; equal elements keep their input order (the reference's
  * stable selection sort with strict ordered compares). */
+#define PML_HIP_MAX_SORT_LINE 16384 /* every element's rank is counted against the whole line: O(n^2) per line */
 typedef struct {
   int32_t dtype;
   int32_t rank, axis, direction;
@@ -425,7 +426,7 @@ typedef struct {
   int32_t n_out_idx;
   int32_t n_src;
   int32_t n_forms;
-  int32_t cmp_dtype; /* COMBO_COND: element type the two comparands are compared in */
+  int32_t cmp_dtype; /* COMBO_COND, COMBO_EQ: element type the two comparands are compared in */
   int32_t src_dtype[3];
   int32_t has_init;  /* output buffer already holds the initial value; else the identity is used */
   int64_t lo[PML_HIP_MAX_IDX], hi[PML_HIP_MAX_IDX]; /* inclusive box */

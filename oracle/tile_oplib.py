@@ -23,8 +23,9 @@ Pinned by tests/test_oplib_ops.py, tests/test_conv_general.py and the op-level
 cases of tests/test_oracle_golden.py (numpy closed forms, the exact cases of
 plaidml/op/op_test.cc, direct numpy evaluations of the definitions).
 nms has no test in the reference: tests/test_nms.py pins it against a loop-written
-greedy suppression for the NMS box formats and the three styles; its SSD box
-decoding (_box_corners, SSD branches) has no independent check: PARITY UNPINNED.
+greedy suppression for the NMS box formats and the three styles, its SSD box
+decoding (_box_corners) against boxes worked out by hand from ops.cc:2034-2117 and the
+box columns of whole SSD results against a box-by-box scalar decoding.
 
 Nothing in the shipped package imports this module.
 """

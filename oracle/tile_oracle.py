@@ -33,9 +33,17 @@ computes for a Tile program:
 bfloat16 does not exist in the reference (plaidml/core/ffi.h:139-156 stops at
 FLOAT64).  Its semantics here are DECLARED, not inherited: values are stored as
 bf16, every operation computes in fp32 and rounds its result to bf16 with
-round-to-nearest-even; a contraction accumulates in fp32 and rounds once at the
-end.  PARITY UNPINNED for bf16 (no reference vector exists).  The same holds
-for float16, which this oracle treats like bfloat16 (fp32 compute, one rounding).
+round-to-nearest-even; a contraction accumulates in fp32 (its initial value
+included) and rounds once at the end.  No reference vector can exist for bf16;
+what the declaration fixes is pinned by sums that fp32 holds and bf16 does not
+(tests/test_oracle_golden.py: rounding per tap, per partial sum or before the
+initial value goes in gives a different, stated answer), and the scalar
+conversion by its ties.  float16 is treated like bfloat16 (fp32 compute, one
+rounding) and pinned the same way.
+
+The `eq` combination (plaidml/edsl/edsl.h:421; i1 result pmlc/ast/eval.cc:25;
+tile_to_linalg.cc:1257-1262) has no test in the reference: pinned by numpy any /
+all / parity of the match table (test_eq_combination_closed_forms).
 
 Pinned by tests/test_oracle_golden.py against these reference-held vectors:
   GEMM_{INT64,UINT64,INT32,INT8,FLOAT32} (plaidml/edsl/examples/gemm.cc:27-90),
@@ -1047,14 +1055,20 @@ def contract(agg, combo, out_dt, out_shape, sink, srcs, accs, cons=(), init=None
     # sources in compute type
     bufs = []
     cmp_float = 0
+    if combo == 'eq':
+        # (a == b) as a one-bit value aggregated in one-bit arithmetic (tile_to_linalg.cc:1257-1262, :485-544:
+        # addi / muli on i1, unsigned compares for max / min): the low bit of the same aggregation over
+        # select(a == b, 1, 0) in eight bits -- a sum's low bit is its parity, max / min / mul of 0s and 1s
+        # never leave {0, 1}, and the identities 0, 1, 0xff, 0 keep their low bit
+        srcs = list(srcs) + [(np.ones((), np.uint8), DType.BOOLEAN)]
+        accs = list(accs) + [[]]
+        combo = 'cond'
     if combo == 'cond':
         (a, adt), (b, bdt), (c, cdt_) = srcs
         cmp_float = 1 if (is_float(adt) or is_float(bdt)) else 0
         t = np.float64 if cmp_float else np.int64
         bufs = [np.ascontiguousarray(a, dtype=t), np.ascontiguousarray(b, dtype=t),
                 np.ascontiguousarray(convert(c, cdt_, cdt) if cdt_ != out_dt else c).astype(npdt)]
-    elif combo == 'eq':
-        raise NotImplementedError('eq combination')
     else:
         for a, adt in srcs:
             if adt != out_dt:
@@ -1102,7 +1116,7 @@ def contract(agg, combo, out_dt, out_shape, sink, srcs, accs, cons=(), init=None
     if n < 0:
         raise ValueError('malformed contraction')
     if cdt == DType.BOOLEAN:
-        out = out.astype(np.bool_)
+        out = (out & 1).astype(np.bool_)
     out = _store(out, out_dt)
     if return_box:
         return out, dict(zip(names, zip(lo.tolist(), hi.tolist()))), int(n)
@@ -1330,7 +1344,10 @@ def evaluate(outputs, feeds):
 
     seen = set()
     for o in outputs:
-        count(o, seen)
+        uses[id(o)] = uses.get(id(o), 0) + 1  # the function's return is a use as well (hasOneUse)
+        if id(o) not in seen:
+            seen.add(id(o))
+            count(o, seen)
 
     rewritten = {}
 

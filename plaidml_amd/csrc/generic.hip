@@ -42,6 +42,9 @@ __device__ inline Scalar<FT, IT> combine(int combo, int dt, int cmp_dt, const Sc
       if (eq) r = x[2];
       break;
     }
+    case PML_HIP_COMBO_EQ:  // a one-bit result; its aggregation wraps to one bit as well
+      r.i = (dt_is_float(cmp_dt) ? (x[0].f == x[1].f) : (x[0].i == x[1].i)) ? 1 : 0;
+      break;
     default:
       break;
   }
@@ -113,7 +116,7 @@ __device__ inline void accumulate_point(const pml_hip_contract_desc& d, const Co
     for (int q = 0; q < d.n_src; ++q) {
       const int sd = d.src_dtype[q];
       Scalar<FT, IT> raw = load_scalar<FT, IT>(a.srcs[q], off[q + 1], sd);
-      if (d.combo == PML_HIP_COMBO_COND && q < 2) {
+      if ((d.combo == PML_HIP_COMBO_COND || d.combo == PML_HIP_COMBO_EQ) && q < 2) {
         x[q] = convert_scalar<FT, IT>(raw, sd, d.cmp_dtype);
       } else if (!dt_is_float(sd) && !dt_is_float(acc_dt) && sd != PML_HIP_BOOL && dt_size(sd) < dt_size(acc_dt) &&
                  d.combo != PML_HIP_COMBO_COND) {

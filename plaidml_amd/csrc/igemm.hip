@@ -24,6 +24,8 @@
 // once per element in row-major order and stores are contiguous 8/16-byte pieces.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "device_common.h"
 #include "igemm_tail.h"
 #include "plans.h"
@@ -50,49 +52,90 @@ constexpr unsigned kOutside = 0x80000000u;     // ... and this one reads as zero
 // Sum of two byte offsets, each of which may be the "outside" mark.
 __device__ inline unsigned join_offsets(unsigned x, unsigned y) { return ((x | y) & kOutside) ? kOutside : x + y; }
 
-// XCD-aware tile order: hardware deals consecutive workgroup ids round-robin to
-// the 8 XCDs, each with its own L2.  Re-number so that one XCD works on a
-// contiguous run of tiles (neighbouring tiles share A rows / Bt rows in L2).
-__device__ inline int xcd_remap(int bid, int nblocks) {
-  constexpr int kXcds = 8;
-  if (nblocks % kXcds != 0) return bid;
-  const int per = nblocks / kXcds;
-  return (bid % kXcds) * per + (bid / kXcds);
+// XCD-aware tile order.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its
+// own L2, and a CU takes the next id of its XCD when it falls free: the workgroups resident on an XCD at any
+// time are a run of about 32 consecutive "local" numbers bid / 8.  What such a run costs the L2 is the
+// number of distinct A rows plus Bt rows under its tiles, so a run should be a compact block, not a strip:
+// the tile grid is cut into blocks of TH x TW tiles (32 tiles, as square as the grid allows), blocks are
+// numbered row-major, XCD x owns the blocks x*per/32 ... and walks each block row-major.  (4096^2 with
+// 256x256 tiles: 2 x 16 strips fetch 576 KB per K-slab and XCD, 4 x 8 blocks 384 KB; what misses L2 comes
+// over the fabric from the last-level cache, whose bandwidth is the scarce one.)
+__device__ inline void xcd_tile(int bid, int tiles_m, int tiles_n, int* tm, int* tn) {
+  constexpr int kXcds = 8, kRun = 32;
+  const int nblocks = tiles_m * tiles_n;
+  int t = bid;
+  if (nblocks % kXcds == 0) {
+    const int per = nblocks / kXcds;
+    t = (bid % kXcds) * per + (bid / kXcds);  // contiguous run per XCD
+    int th = 0, tw = 0;
+    if (tiles_m % 4 == 0 && tiles_n % 8 == 0) { th = 4; tw = 8; }
+    else if (tiles_m % 8 == 0 && tiles_n % 4 == 0) { th = 8; tw = 4; }
+    else if (tiles_m % 16 == 0 && tiles_n % 2 == 0) { th = 16; tw = 2; }
+    else if (tiles_m % 2 == 0 && tiles_n % 16 == 0) { th = 2; tw = 16; }
+    if (th && per % kRun == 0) {
+      const int blk = t / kRun, in = t % kRun;
+      const int blocks_n = tiles_n / tw;
+      *tm = (blk / blocks_n) * th + in / tw;
+      *tn = (blk % blocks_n) * tw + in % tw;
+      return;
+    }
+  }
+  *tm = t / tiles_n;
+  *tn = t % tiles_n;
 }
 
 // STAGES = 0: as many as pay for the tile; 2: two, and LDS rounded up to what staging the whole result
 // tile needs (a short-K, bandwidth-bound GEMM gains more from a second workgroup on the CU than from a
 // third slab in flight)
-template <int BM, int BN, int STAGES = 0>
+template <int I, int N, int STEP, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + STEP, N, STEP>(f);
+  }
+}
+
+template <int BM, int BN, int STAGES = 0, int SLAB = 128>
 struct Ring {
-  static constexpr int kStage = (BM + BN) * kSlabBytes;                 // A rows then Bt rows
+  static constexpr int kStage = (BM + BN) * SLAB;                       // A rows then Bt rows
   // 64x64 tiles run two stages: 32 KB of LDS lets five workgroups share a CU, and for this tile
   // residency hides more latency than a third slab in flight does
   static constexpr int kStages = STAGES ? STAGES : ((BM * BN <= 64 * 64) ? 2 : (3 * kStage <= kLdsBytes ? 3 : 2));
   static constexpr int kTileBytes = BM * (BN + 4) * 4;
-  static constexpr int kBytes = (STAGES && kTileBytes > kStages * kStage) ? kTileBytes : kStages * kStage;
+  static constexpr int kBytes = (STAGES && kTileBytes > kStages * kStage && kTileBytes <= kLdsBytes) ? kTileBytes : kStages * kStage;
+  static_assert(kBytes <= kLdsBytes, "the ring must fit the CU's LDS");
 };
 
 // BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4, 8 or 16 wavefronts (one, two or four
 // per SIMD).  WAVES_K = 2: two such grids, each multiplying one half of the K-blocks of every slab; their
 // partial results meet in LDS before the tail (more wavefronts for problems with few tiles and a long K).
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1>
-__global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
-  typedef Ring<BM, BN, STAGES> ring_t;
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
+__global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
+  // The argument block is read where the dispatcher put it (the kernel-argument segment, scalar loads),
+  // through a reference: taking the by-value parameter's address instead makes the compiler copy all of
+  // it to scratch memory as soon as one field is indexed with a run-time value.
+  const IgemmArgs& p = *(const IgemmArgs*)(const __attribute__((address_space(4))) void*)__builtin_amdgcn_kernarg_segment_ptr();
+  typedef Ring<BM, BN, STAGES, SLAB> ring_t;
+  // bytes of K per LDS row and ring stage: 128 (four 32-byte K-blocks), or 64 for the large tiles, whose
+  // 160 KB of LDS then hold five stages instead of two -- what a CU has in flight is what hides memory latency
+  constexpr int kSlabBytes = SLAB;
+  constexpr int CPR = SLAB / 16;                      // 16-byte chunks per row
+  constexpr int kSwzShift = SLAB == 128 ? 1 : 2;      // chunk u of row r sits in slot u ^ ((r >> shift) & (CPR - 1))
+  static_assert(SLAB == 128 || SLAB == 64, "rows of 128 or 64 bytes");
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
   constexpr int kWaves = NT / 64;
-  constexpr int kRowsPerPass = NT / 8;  // operand rows one load of all threads covers (8 lanes per 128-byte row)
+  constexpr int kRowsPerPass = NT / CPR;  // operand rows one load of all threads covers
   constexpr int WAVES_N = kWaves / WAVES_M / WAVES_K;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int MI = WM / 32, NI = WN / 32;
-  constexpr int A_VECS = BM * 8 / NT;  // 16-byte vectors per thread per slab
-  constexpr int B_VECS = BN * 8 / NT;
+  constexpr int A_VECS = BM * CPR / NT;  // 16-byte vectors per thread per slab
+  constexpr int B_VECS = BN * CPR / NT;
   static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0, "tile sides are whole load passes");
   constexpr int kStage = ring_t::kStage;
   constexpr int kStages = ring_t::kStages;
-  constexpr int kAhead = kStages - 1;              // slabs in flight ahead of the one being multiplied
   constexpr int kLoads = A_VECS + B_VECS;          // loads a thread issues per slab
-  static_assert(kAhead * kLoads <= 63, "the vmcnt field counts at most 63 loads");
+  static_assert((kStages - 1) * kLoads <= 63, "the vmcnt field counts at most 63 loads");
+  static_assert((kSlabBytes / 32 / WAVES_K) % 2 == 0, "fragment buffers alternate per K-block and must line up across slabs");
   // (The vmcnt arithmetic below counts this kernel's own requests: a configuration whose registers spill
   // puts scratch loads and stores into the same counter and is wrong, not just slow -- 256x256 with 16
   // wavefronts needs 198 registers of the 128 it may have and failed its tests for that reason.)
@@ -110,17 +153,18 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
 
   const int tiles_n = (int)((p.N + BN - 1) / BN);
   const int tiles_m = (int)((p.M + BM - 1) / BM);
-  const int tile = xcd_remap(blockIdx.x, tiles_m * tiles_n);
-  const int64_t m0 = (int64_t)(tile / tiles_n) * BM;
-  const int64_t n0 = (int64_t)(tile % tiles_n) * BN;
+  int tile_m, tile_n;
+  xcd_tile(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
+  const int64_t m0 = (int64_t)tile_m * BM;
+  const int64_t n0 = (int64_t)tile_n * BN;
 
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)kBufRange, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.Bt, 0, (int)kBufRange, kRsrcFlags);
 
   // ---- per-thread load assignments (fixed across slabs): slot lv of rows lr + kRowsPerPass*i ----
-  const int lv = tid & 7;
-  const int lr = tid >> 3;
-  const int lc = lv ^ ((lr >> 1) & 7);                        // the chunk of its row this thread fetches
+  const int lv = tid % CPR;
+  const int lr = tid / CPR;
+  const int lc = lv ^ ((lr >> kSwzShift) & (CPR - 1));        // the chunk of its row this thread fetches
   const int kbytes_row = (int)(CONV ? p.CI * ES : p.K * ES);  // valid bytes per (tap) row
 
   unsigned a_off[A_VECS];  // GEMM: byte offset of the row; CONV: of the image; kOutside for rows past M
@@ -166,7 +210,7 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   int req_dh = 0, req_dw = 0, req_px = 0;  // req_px: pixels the chunk lies beyond the tap's first one (pitch < run)
   bool req_ok = false;
   auto prepare_slab = [&](int s, int stage) {
-    req_base = smem + stage * kStage + wave * (8 * kSlabBytes);
+    req_base = smem + stage * kStage + wave * 1024;  // one request of a wavefront fills 1 KB
     const bool live = s < n_slabs;
     if (CONV) {
       const int tap = s / slabs_per_tap;
@@ -214,8 +258,9 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
+  // Every ring stage is requested before the first multiply: kStages slabs in flight.
 #pragma unroll
-  for (int s = 0; s < kAhead; ++s) {
+  for (int s = 0; s < kStages; ++s) {
     prepare_slab(s, s);
 #pragma unroll
     for (int l = 0; l < kLoads; ++l) issue_load(l);
@@ -226,51 +271,83 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
   constexpr int kBlocks = kSlabBytes / 32 / WAVES_K;
   int fslot[kBlocks];
 #pragma unroll
-  for (int kb = 0; kb < kBlocks; ++kb) fslot[kb] = (((wk * kBlocks + kb) * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
+  for (int kb = 0; kb < kBlocks; ++kb) fslot[kb] = (((wk * kBlocks + kb) * 2 + (lane >> 5)) ^ ((lane >> kSwzShift) & (CPR - 1))) * 16;
+
+  // The loop is rotated by one K-block: the one synchronisation point of a slab sits before its LAST
+  // K-block, whose fragments are in registers by then.  Past it every wavefront is done reading this
+  // slab's stage, and the next slab has landed (vmcnt leaves only the younger slabs outstanding); so the
+  // last K-block's MFMAs cover the first fragment reads of the next slab and the requests that refill this
+  // stage with slab s + kStages, and no MFMA ever waits behind a barrier for LDS or memory.
+  constexpr int kOutstanding = (kStages - 2) * kLoads;  // requests that may still be in flight at the sync point
+  constexpr int kSlots = MI * NI;
+  i32x4_t fa[2][MI], fb[2][NI];
+  const unsigned char* a_base = smem + (wm * WM + frow) * kSlabBytes;
+  const unsigned char* b_base = smem + (BM + wn * WN + frow) * kSlabBytes;
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (((kStages - 1) * kLoads) & 15) | ((((kStages - 1) * kLoads) >> 4) << 14));
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(a_base + i * 32 * kSlabBytes + fslot[0]);
+#pragma unroll
+  for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(b_base + j * 32 * kSlabBytes + fslot[0]);
 
   int stage = 0;  // ring stage of slab s
   for (int s = 0; s < n_slabs; ++s) {
-    // slab s has landed once at most (kAhead - 1) later slabs of this thread are outstanding;
-    // the barrier extends that to every thread and also says: everyone is done with slab s - 1
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (((kAhead - 1) * kLoads) & 15) | ((((kAhead - 1) * kLoads) >> 4) << 14));
-    __builtin_amdgcn_s_barrier();
-    int free_stage = stage - 1;
-    if (free_stage < 0) free_stage = kStages - 1;
-    prepare_slab(s + kAhead, free_stage);
-    const unsigned char* a_base = smem + stage * kStage + (wm * WM + frow) * kSlabBytes;
-    const unsigned char* b_base = smem + stage * kStage + (BM + wn * WN + frow) * kSlabBytes;
-    // Per K-block: MI*NI MFMA groups in program order; behind the m-th one sit one request of the
-    // slab two ahead and one fragment read of K-block kb + 1, so that neither the texture path nor
-    // LDS latency ever holds up the matrix pipe.  sched_barrier pins that order.
-    i32x4_t fa[2][MI], fb[2][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(a_base + i * 32 * kSlabBytes + fslot[0]);
-#pragma unroll
-    for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(b_base + j * 32 * kSlabBytes + fslot[0]);
+    int next_stage = stage + 1;
+    if (next_stage == kStages) next_stage = 0;
+    const unsigned char* a_next = smem + next_stage * kStage + (wm * WM + frow) * kSlabBytes;
+    const unsigned char* b_next = smem + next_stage * kStage + (BM + wn * WN + frow) * kSlabBytes;
 #pragma unroll
     for (int kb = 0; kb < kBlocks; ++kb) {
       const int cur = kb & 1, nxt = cur ^ 1;
-      const int l0 = kb * kLoads / kBlocks, l1 = (kb + 1) * kLoads / kBlocks;
-      constexpr int kSlots = MI * NI;
+      const bool last = kb + 1 == kBlocks;
+      if (last) {
+        // fragments of this K-block are in registers (lgkmcnt 0), slab s + 1 has landed
+#ifdef PML_TRACE
+        const uint64_t t0 = __builtin_amdgcn_s_memtime();
+        __builtin_amdgcn_s_waitcnt(0x0F7F & ~0x0F00);  // lgkmcnt(0) only
+        const uint64_t t1 = __builtin_amdgcn_s_memtime();
+#endif
+        __builtin_amdgcn_s_waitcnt(0x0070 | (kOutstanding & 15) | ((kOutstanding >> 4) << 14));
+#ifdef PML_TRACE
+        const uint64_t t2 = __builtin_amdgcn_s_memtime();
+#endif
+        if constexpr (!(ABL & 8)) __builtin_amdgcn_s_barrier();
+#ifdef PML_TRACE
+        if (p.outs[5] && blockIdx.x == 37 && lane == 0 && s < 60) {
+          uint64_t* tr = (uint64_t*)p.outs[5] + (wave * 64 + s) * 4;
+          tr[0] = t0; tr[1] = t1; tr[2] = t2; tr[3] = __builtin_amdgcn_s_memtime();
+          if (wave == 15 || (wave == 7 && NT == 512)) tr[1] = __builtin_amdgcn_s_memrealtime();  // the 100 MHz clock, to calibrate
+        }
+#endif
+        prepare_slab(s + kStages, stage);
+      }
+      const unsigned char* ra_ = last ? a_next : a_base;
+      const unsigned char* rb_ = last ? b_next : b_base;
+      const int fs = fslot[last ? 0 : kb + 1];
 #pragma unroll
       for (int m = 0; m < kSlots; ++m) {
-        mma_block<KIND>(acc[m / NI][m % NI], fb[cur][m % NI], fa[cur][m / NI]);
-        // requests and fragment reads of this K-block, dealt over its MFMA slots
+        if constexpr (ABL & 4) {
+          asm volatile("" ::"v"(fb[cur][m % NI]), "v"(fa[cur][m / NI]));
+        } else {
+          mma_block<KIND>(acc[m / NI][m % NI], fb[cur][m % NI], fa[cur][m / NI]);
+        }
+        if (last && !(ABL & 1)) {
 #pragma unroll
-        for (int l = l0 + m; l < l1; l += kSlots) issue_load(l);
-        if (kb + 1 < kBlocks) {
+          for (int l = m; l < kLoads; l += kSlots) issue_load(l);
+        }
 #pragma unroll
-          for (int d = m; d < MI + NI; d += kSlots) {
-            if (d < MI)
-              fa[nxt][d] = *(const i32x4_t*)(a_base + d * 32 * kSlabBytes + fslot[kb + 1]);
-            else
-              fb[nxt][d - MI] = *(const i32x4_t*)(b_base + (d - MI) * 32 * kSlabBytes + fslot[kb + 1]);
-          }
+        for (int d = m; d < ((ABL & 2) ? 0 : MI + NI); d += kSlots) {
+          if (d < MI)
+            fa[nxt][d] = *(const i32x4_t*)(ra_ + d * 32 * kSlabBytes + fs);
+          else
+            fb[nxt][d - MI] = *(const i32x4_t*)(rb_ + (d - MI) * 32 * kSlabBytes + fs);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if (++stage == kStages) stage = 0;
+    stage = next_stage;
+    a_base = a_next;
+    b_base = b_next;
   }
   // drain the (all-outside) requests still in flight before LDS is reused
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -316,8 +393,10 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
     constexpr int RB = kFit >= MI ? MI : (kFit >= 4 ? 4 : (kFit >= 2 ? 2 : 1));  // MI is a power of two
     static_assert(RB >= 1 && MI % RB == 0, "row blocks must stage evenly");
     accs_t* wtile = (accs_t*)(smem + wave * kBudget);
-#pragma unroll
-    for (int i0 = 0; i0 < MI; i0 += RB) {
+    // (a compile-time loop: with a run-time row-block number the accumulators would be indexed
+    // dynamically and live in scratch memory)
+    static_for<0, MI, RB>([&](auto i0c) {
+      constexpr int i0 = decltype(i0c)::value;
 #pragma unroll
       for (int i = 0; i < RB; ++i)
 #pragma unroll
@@ -329,10 +408,15 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p) {
             for (int e = 0; e < 4; ++e) q[e] = acc[i0 + i][j][4 * g + e];
             *(acc4_t*)&wtile[(i * 32 + crow) * CS + j * 32 + 8 * g + ccol] = q;
           }
-      __syncthreads();
+      // the staging region is private to the wavefront: its own LDS counter orders stores and reads
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       tile_tail<KIND, RB * 32, WN, 64>(p, wtile, m0 + wm * WM + i0 * 32, n0 + wn * WN, lane);
-      __syncthreads();
-    }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    });
   }
 }
 
@@ -413,11 +497,11 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
   }
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  const size_t lds = Ring<BM, BN, STAGES>::kBytes;
-  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K>;
+  const size_t lds = Ring<BM, BN, STAGES, SLAB>::kBytes;
+  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -430,6 +514,10 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
 
 template <int KIND, bool CONV>
 hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
+#ifdef PML_DEV_CFG  // development builds: one configuration, given as the template arguments after KIND
+  if constexpr (!CONV && KIND == PML_KIND) return launch_cfg<KIND, PML_DEV_CFG>(a, s);
+  return hipErrorInvalidValue;
+#else
   switch (cfg) {
     case TILE_64x64: return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);
     case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
@@ -439,8 +527,12 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_256x128_W16: return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
     case TILE_128x128_W8_S2: return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
     case TILE_64x64_W8_K2: return launch_cfg<KIND, 64, 64, 2, CONV, 512, 0, 2>(a, s);
+    case TILE_256x256_W8: return launch_cfg<KIND, 256, 256, 2, CONV, 512>(a, s);
+    case TILE_256x256_W8T: return launch_cfg<KIND, 256, 256, 4, CONV, 512>(a, s);
+    case TILE_256x256_W4: return launch_cfg<KIND, 256, 256, 2, CONV, 256>(a, s);
   }
   return hipErrorInvalidValue;
+#endif
 }
 
 }  // namespace

@@ -80,6 +80,9 @@ const char* tile_name(int t) {
     case TILE_128x128_W8: return "128x128 (8 wavefronts)";
     case TILE_256x128_W16: return "256x128 (16 wavefronts)";
     case TILE_64x64_W8_K2: return "64x64 (8 wavefronts, K split in two)";
+    case TILE_256x256_W8: return "256x256 (8 wavefronts of 128x64)";
+    case TILE_256x256_W8T: return "256x256 (8 wavefronts of 64x128)";
+    case TILE_256x256_W4: return "256x256 (4 wavefronts of 128x128)";
     case TILE_128x128_W8_S2: return "128x128 (8 wavefronts, 2 stages)";
   }
   return "?";
@@ -122,6 +125,9 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
     if (v == "128x128w8s2") return TILE_128x128_W8_S2;
     if (v == "256x128w16") return TILE_256x128_W16;
     if (v == "64x64w8k2") return TILE_64x64_W8_K2;
+    if (v == "256x256w8") return TILE_256x256_W8;
+    if (v == "256x256w8t") return TILE_256x256_W8T;
+    if (v == "256x256w4") return TILE_256x256_W4;
   }
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (n <= 64) return TILE_64x64;  // (the 7x7 stem of ResNet-50 over 2x2 pixel blocks: 191 us against 207 us with 128x64w8)
@@ -993,7 +999,8 @@ int pml_hip_argsort(const pml_hip_argsort_desc* d, const void* tensor, void* out
   if (d->axis < 0 || d->axis >= d->rank) return fail("argsort: axis out of range");
   if (d->direction != 0 && d->direction != 1) return fail("argsort: bad direction");
   if (dt_size(d->dtype) == 0 || d->dtype == PML_HIP_BOOL) return fail("argsort: bad element type");
-  if (d->sizes[d->axis] > INT32_MAX) return fail("argsort: axis too long for si32 positions");
+  if (d->sizes[d->axis] > PML_HIP_MAX_SORT_LINE)
+    return fail("argsort: more than PML_HIP_MAX_SORT_LINE (16384) elements along the sorted axis");
   if (count_of(d->sizes, d->rank) == 0) return 0;
   return check(argsort_launch(*d, tensor, out, (hipStream_t)s), "argsort_launch");
 }
@@ -1030,8 +1037,8 @@ int64_t pml_hip_contract_dispatch(const pml_hip_contract_desc* d) {
       return 0;
     }
   }
-  if (d->combo == PML_HIP_COMBO_EQ) {
-    fail("contract: the eq combination is not supported");
+  if (d->combo == PML_HIP_COMBO_EQ && (d->dtype != PML_HIP_BOOL || d->n_src != 2)) {
+    fail("contract: the eq combination takes two operands and gives a boolean result");
     return 0;
   }
   Plan* p = new Plan();

@@ -687,6 +687,9 @@ class Planner {
       int64_t axis = param(0);
       if (axis < 0) axis += d.rank;
       if (axis < 0 || axis >= d.rank) throw std::runtime_error("'argsort' axis out of range");
+      if (d.sizes[axis] > PML_HIP_MAX_SORT_LINE)
+        throw std::runtime_error("'argsort' over more than " + std::to_string(PML_HIP_MAX_SORT_LINE) +
+                                 " elements along the axis is not supported by the hip target");
       d.axis = static_cast<int32_t>(axis);
       d.direction = static_cast<int32_t>(param(1));
       s.text = std::string("argsort axis=") + std::to_string(d.axis) + (d.direction ? " desc" : " asc") + " -> " + op.result->shape.str();
@@ -736,7 +739,14 @@ class Planner {
     TailBuild tb;
     ValuePtr main;
     int main_pos = -1;
-    for (size_t k = 0; k < op.operands.size(); ++k) {
+    // max / min keep the first comparand as the running value (their NaN behaviour is not symmetric); it is
+    // read through zero strides where it is broadcast
+    const bool ordered = op.kind == Op::Eltwise && (op.fn == "max" || op.fn == "min" || op.fn == "maxgt");
+    if (ordered && op.operands.size() == 2 && op.operands[0]->kind != Value::Literal) {
+      main = op.operands[0];
+      main_pos = 0;
+    }
+    for (size_t k = 0; !main && k < op.operands.size(); ++k) {
       const ValuePtr& v = op.operands[k];
       if (v->kind != Value::Literal && v->shape.sizes == out.sizes) {
         main = v;
@@ -960,6 +970,9 @@ class Planner {
     for (const Idx& x : M) m *= x.range;
     for (const Idx& x : N) nn *= x.range;
     for (const Idx& x : K) kk *= x.range;
+    // the m x n block must be the whole result: elements the contraction never reaches hold the
+    // aggregation identity (or the initial value), which only the general path writes
+    if (bo != 0 || m * nn != op.result->shape.elements()) return false;
     if (N.empty()) { ncs = 1; nbs = 1; }   // matrix-vector: one column
     if (M.empty()) { ldc = nn; lda = kk; }  // vector-matrix: one row
     if (ncs != 1 || kas != 1) return false;
@@ -1439,7 +1452,6 @@ class Planner {
 
   void emitGeneral(size_t i) {
     const Op& op = prog_->ops[i];
-    if (op.combo == ComboKind::eq) throw std::runtime_error("the 'eq' combination is not supported by the hip target");
     const size_t nIdx = op.idxNames.size();
     const TensorShape& os = op.result->shape;
     // output indices: each output dimension is exactly one distinct index (coef 1 or more), den 1
@@ -1490,7 +1502,7 @@ class Planner {
     d.combo = hipCombo(op.combo);
     d.n_src = static_cast<int>(op.operands.size());
     for (size_t k = 0; k < op.operands.size(); ++k) d.src_dtype[k] = hipType(op.operands[k]->shape.elementType);
-    if (op.combo == ComboKind::cond)
+    if (op.combo == ComboKind::cond || op.combo == ComboKind::eq)
       d.cmp_dtype = hipType(util::promoteTypes(op.operands[0]->shape.elementType, op.operands[1]->shape.elementType));
     tile::aggregationIdentity(op.agg, os.elementType, &d.identity_f, &d.identity_i);
     // positions: fresh output indices first (non-injective case), then `order`

@@ -1,8 +1,8 @@
 """Non-maximum suppression cases, built twice like tests/programs.py: with the oracle's op library and with
 the product's.  The reference holds no test of plaidml::op::nms (plaidml/op/lib/ops.cc:2157-2417), so the
 oracle's restatement is pinned here against an independent, loop-written greedy suppression -- the textbook
-algorithm the operation unrolls -- for the NMS box formats and the three styles; the SSD box decoding has no
-independent check (parity unpinned) and is compared product-against-oracle only."""
+algorithm the operation unrolls -- for the NMS box formats and the three styles; the SSD box decoding is pinned
+in tests/test_nms.py by hand-computed boxes."""
 import numpy as np
 
 CAFFE, MXNET, OV = range(3)

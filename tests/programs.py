@@ -432,6 +432,121 @@ def higher_precision_constants(E, op):
 
 # ---- the five workload configurations, reduced ---------------------------------------------------------
 
+
+def eq_combination(E, op):
+    """The `eq` combination (plaidml/edsl/edsl.h:421, result type i1: pmlc/ast/eval.cc:25; lowered as a compare
+    aggregated in one-bit arithmetic: tile_to_linalg.cc:1257-1262, :485-544).  any / all / parity of matches per
+    output point, integer comparands and mixed float / integer ones, one output with uncovered elements."""
+    r = _rng(31)
+    a = r.integers(0, 3, (6, 8)).astype(np.int32)
+    b = r.integers(0, 3, (8, 5)).astype(np.int32)
+    f = r.integers(0, 3, (6, 8)).astype(np.float32)
+    f[0, 0] = np.nan
+    A = E.Placeholder(E.DType.INT32, a.shape)
+    B = E.Placeholder(E.DType.INT32, b.shape)
+    F = E.Placeholder(E.DType.FLOAT32, f.shape)
+    outs = []
+    for agg in ('max', 'min', 'sum', 'product'):
+        i, j, k = E.TensorIndexes(3)
+        outs.append(getattr(E.Contraction().outShape(6, 5).outAccess(i, j), agg)(A[i, k] == B[k, j]).build())
+    i, j, k = E.TensorIndexes(3)
+    outs.append(E.Contraction().outShape(6, 5).outAccess(i, j).sum(F[i, k] == B[k, j]).build())
+    i, j, k = E.TensorIndexes(3)
+    outs.append(E.Contraction().outShape(7, 6).outAccess(i, j).min(A[i, k] == B[k, j]).build())
+    return E.Program('eq_combination', [A, B, F], outs), [a, b, f], EXACT
+
+
+def eq_combination_answers(a, b, f):
+    """What the mathematics fixes for eq_combination: numpy any / all / parity of the match table."""
+    m = a[:, :, None] == b[None, :, :]
+    mf = f[:, :, None] == b[None, :, :].astype(np.float32)
+    part = np.ones((7, 6), bool)   # elements the contraction never reaches keep min's identity: true
+    part[:6, :5] = m.all(1)
+    return [m.any(1), m.all(1), (m.sum(1) % 2).astype(bool), m.all(1), (mf.sum(1) % 2).astype(bool), part]
+
+
+def partial_cover_gemm(E, op):
+    """A matrix product that writes only part of its result (a larger outShape, a shifted outAccess): the
+    rest holds the aggregation identity, also under a fused elementwise tail (exp(0) = 1)."""
+    r = _rng(32)
+    a = r.standard_normal((8, 16)).astype(np.float32) * 0.25
+    b = r.standard_normal((16, 8)).astype(np.float32) * 0.25
+    A = E.Placeholder(E.DType.FLOAT32, a.shape)
+    B = E.Placeholder(E.DType.FLOAT32, b.shape)
+    outs = []
+    for shape, dj in (((16, 8), 0), ((16, 12), 0), ((8, 12), 4)):
+        i, j, k = E.TensorIndexes(3)
+        outs.append(E.exp(E.Contraction().outShape(*shape).outAccess(i, j + dj).sum(A[i, k] * B[k, j]).build()))
+    return E.Program('partial_cover_gemm', [A, B], outs), [a, b], FP32
+
+
+def broadcast_first_min_max(E, op):
+    """maximum / minimum / select-as-max whose first operand is the broadcast one (X[8] against Y[4,8])."""
+    r = _rng(33)
+    x = r.standard_normal(8).astype(np.float32)
+    y = r.standard_normal((4, 8)).astype(np.float32)
+    y[1, 2] = np.nan
+    x[5] = np.nan
+    X = E.Placeholder(E.DType.FLOAT32, x.shape)
+    Y = E.Placeholder(E.DType.FLOAT32, y.shape)
+    outs = [op.maximum(X, Y), op.minimum(X, Y), E.select(X < Y, Y, X), E.select(X > Y, X, Y),
+            op.maximum(Y, X), op.minimum(Y, X)]
+    return E.Program('broadcast_first_min_max', [X, Y], outs), [x, y], FP32
+
+
+
+def bf16_rounding_placement(E, op):
+    """bf16 contractions accumulate in fp32 and round once, to nearest even, after the last tap and after the
+    initial value went in.  Integer-valued inputs whose exact sums fp32 holds and bf16 does not:
+    256 + 1 + 1 + 1 = 259 -> 260 (rounding after every tap gives 256, after pairs 258);
+    2 (initial value) + 256 + 1 = 259 -> 260 (rounding the sum before the initial value goes in gives 258);
+    columns 1: 128 + 0.5 + 0.5 + 0.5 = 129.5 -> 130 (per tap: 128)."""
+    a = np.array([[256, 1, 1, 1], [128, 0.5, 0.5, 0.5]], np.float32)
+    b = np.ones((4, 2), np.float32)
+    a2 = np.array([[256, 1, 0, 0]], np.float32)
+    c = np.full((1, 2), 2, np.float32)
+    A = E.Placeholder(E.DType.BFLOAT16, a.shape)
+    B = E.Placeholder(E.DType.BFLOAT16, b.shape)
+    A2 = E.Placeholder(E.DType.BFLOAT16, a2.shape)
+    C = E.Placeholder(E.DType.BFLOAT16, c.shape)
+    i, j, k = E.TensorIndexes(3)
+    O = E.Contraction().outShape(2, 2).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    i, j, k = E.TensorIndexes(3)
+    O2 = E.Contraction().outShape(1, 2).outAccess(i, j).sum(A2[i, k] * B[k, j]).init(C).build()
+    i, j, k = E.TensorIndexes(3)
+    O3 = E.Contraction().outShape(1, 2).outAccess(i, j).sum(A2[i, k] * B[k, j]).build() + C
+    # the same sums at a size the matrix-core kernels take: rows of 256, 1, 1, 1, 0 ... and 128, .5, .5, .5, 0 ...
+    a4 = np.zeros((64, 64), np.float32)
+    a4[0::2, :4] = a[0]
+    a4[1::2, 20:24] = a[1]
+    c4 = np.zeros((64, 64), np.float32)
+    c4[:, 1::2] = 2
+    a4[2, 3] = 0  # row 2 with the initial value 2: 2 + 256 + 1 + 1 = 260 exactly; without: 258
+    A4 = E.Placeholder(E.DType.BFLOAT16, a4.shape)
+    B4 = E.Placeholder(E.DType.BFLOAT16, [64, 64])
+    C4 = E.Placeholder(E.DType.BFLOAT16, c4.shape)
+    i, j, k = E.TensorIndexes(3)
+    O4 = E.Contraction().outShape(64, 64).outAccess(i, j).sum(A4[i, k] * B4[k, j]).build()
+    O5 = O4 + C4
+    return (E.Program('bf16_rounding_placement', [A, B, A2, C, A4, B4, C4], [O, O2, O3, O4, O5]),
+            [a, b, a2, c, a4, np.ones((64, 64), np.float32), c4], EXACT)
+
+
+def _bf16_rounding_answers():
+    o4 = np.zeros((64, 64), np.float32)
+    o4[0::2] = 260
+    o4[1::2] = 130
+    o4[2] = 258
+    o5 = o4.copy()
+    o5[0::2, 1::2] = 262   # 2 + 259 = 261 -> 262 (tie to even; 260 + 2 after an early rounding is 262 as well)
+    o5[1::2, 1::2] = 132   # 2 + 129.5 = 131.5 -> 132 (130 + 2 = 132 as well)
+    o5[2, 1::2] = 260      # 2 + 258 = 260 exactly
+    return [np.array([[260, 260], [130, 130]], np.float32), np.array([[260, 260]], np.float32),
+            np.array([[260, 260]], np.float32), o4, o5]
+
+
+BF16_ROUNDING_ANSWERS = _bf16_rounding_answers()
+
 def config0_gemm_f32(E, op, n=128, seed=1):
     """configs[0]: C[M,N] += A[M,K] * B[K,N], fp32, U(-1,1)."""
     A = E.Placeholder(E.DType.FLOAT32, [n, n])
@@ -475,7 +590,7 @@ def config2_int8_gemm(E, op, M=64, N=48, K=32):
                                                        r6.uniform(0.001, 0.01, N).astype(np.float32)], EXACT
 
 
-def config3_xception_block(E, op, N=2, H=19, W=19, C=32, dtype_name='BFLOAT16'):
+def config3_xception_block(E, op, N=2, H=19, W=19, C=32, dtype_name='BFLOAT16', with_pool_input=False):
     """configs[3]: depthwise 3x3 -> pointwise 1x1 -> scale/shift + ReLU -> maxpool 3x3/2 with window argmax."""
     dt = getattr(E.DType, dtype_name)
     I = E.Placeholder(dt, [N, H, W, C])
@@ -499,7 +614,24 @@ def config3_xception_block(E, op, N=2, H=19, W=19, C=32, dtype_name='BFLOAT16'):
     vals = [Iv, Fd, Fp, sc, sh]
     if dtype_name == 'BFLOAT16':
         vals = [_bf16(v) for v in vals]
-    return E.Program('xception_block', [I, Fdw, Fpw, scale, shift], [M, AM]), vals, BF16 if dtype_name == 'BFLOAT16' else FP32
+    outs = [M, AM, R] if with_pool_input else [M, AM]
+    return E.Program('xception_block', [I, Fdw, Fpw, scale, shift], outs), vals, BF16 if dtype_name == 'BFLOAT16' else FP32
+
+
+def window_argmax_of(R, M):
+    """The window argmax of config3_xception_block worked out in numpy from the pool's own input R and result M:
+    the largest tap number 3 * k0 + k1 whose element equals the window maximum (taps outside the image never
+    match), 0 where none does."""
+    N, H, W, C = R.shape
+    OH, OW = M.shape[1], M.shape[2]
+    padded = np.full((N, 2 * OH + 1, 2 * OW + 1, C), np.nan, np.float32)  # NaN never equals
+    padded[:, 1:H + 1, 1:W + 1] = R
+    best = np.zeros(M.shape, np.int32)
+    for k0 in range(3):
+        for k1 in range(3):
+            tap = padded[:, k0:k0 + 2 * OH:2, k1:k1 + 2 * OW:2]
+            best = np.where(tap == M, np.int32(3 * k0 + k1), best)
+    return best
 
 
 def classifier_tail(E, op, N=4, C=64, K=10, dtype_name='FLOAT32'):
@@ -606,6 +738,10 @@ ALL = {
     'python_conv_cases': python_conv_cases,
     'u64_add': u64_add,
     'higher_precision_constants': higher_precision_constants,
+    'eq_combination': eq_combination,
+    'partial_cover_gemm': partial_cover_gemm,
+    'broadcast_first_min_max': broadcast_first_min_max,
+    'bf16_rounding_placement': bf16_rounding_placement,
     'config0_gemm_f32': config0_gemm_f32,
     'config1_conv_bf16': lambda E, op: config1_conv(E, op, 'BFLOAT16'),
     'config1_conv_f32': lambda E, op: config1_conv(E, op, 'FLOAT32', CI=32, CO=48),

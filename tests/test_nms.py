@@ -103,3 +103,69 @@ def test_device_matches_oracle_ssd(with_arm, share, style):
     np.testing.assert_array_equal(gb, rb)
     np.testing.assert_array_equal(gv, rv)
     np.testing.assert_allclose(gs, rs, rtol=1e-4, atol=1e-6)
+
+
+# --- SSD box decoding (decode_boxes, plaidml/op/lib/ops.cc:2034-2117) pinned by hand-computed boxes -------------
+# Two priors in pixels of a 100 (wide) x 200 (high) image, variances (0.1, 0.1, 0.2, 0.2).  The numbers below
+# were worked out by hand from the reference's formulas, not produced by this repository's code:
+#   centred form, prior (20, 30, 60, 50), location (1, -2, 0.5, -0.5):
+#     normalised prior x 0.2 .. 0.6, y 0.15 .. 0.25 (x by the width, y by the height), size 0.4 x 0.1
+#     centre x = 0.1 * 1 * 0.4 + 0.4 = 0.44, centre y = 0.1 * -2 * 0.1 + 0.2 = 0.18
+#     half width = exp(0.2 * 0.5) * 0.4 / 2 = 0.2210342, half height = exp(0.2 * -0.5) * 0.1 / 2 = 0.0452419
+#   centred form, location 0: the normalised prior itself
+#   corner form: every coordinate is divided by the WIDTH (also y), then + variance * location
+_SSD_PRIORS = np.array([[[[20, 30, 60, 50], [10, 10, 30, 90], [70, 20, 95, 40]]]], np.float32)
+_SSD_VAR = np.array([[[[0.1, 0.1, 0.2, 0.2]] * 3]], np.float32)
+_SSD_LOC = np.array([[[[1, -2, 0.5, -0.5], [0, 0, 0, 0], [-9, -3, 1, 2]]]], np.float32)
+_SSD_WANT = {  # (centred, clip) -> rows of (y1, x1, y2, x2)
+    (True, False): [[0.1347581, 0.2189658, 0.2252419, 0.6610342], [0.05, 0.1, 0.45, 0.3],
+                    [0.12 - 0.0745912, 0.6 - 0.1526753, 0.12 + 0.0745912, 0.6 + 0.1526753]],
+    (False, False): [[0.1, 0.3, 0.4, 0.7], [0.1, 0.1, 0.9, 0.3], [-0.1, -0.2, 0.8, 1.15]],
+    (False, True): [[0.1, 0.3, 0.4, 0.7], [0.1, 0.1, 0.9, 0.3], [0.0, 0.0, 0.8, 1.0]],
+}
+# third prior, centred: x 0.7 .. 0.95 (size 0.25), y 0.1 .. 0.2 (size 0.1); centre x = 0.1 * -9 * 0.25 + 0.825 = 0.6,
+# centre y = 0.1 * -3 * 0.1 + 0.15 = 0.12; half width exp(0.2) * 0.125 = 0.1526753, half height exp(0.4) * 0.05 = 0.0745912
+
+
+@pytest.mark.parametrize('centered,clip', sorted(_SSD_WANT))
+def test_ssd_box_decoding_hand_computed(centered, clip):
+    f32 = OE.DType.FLOAT32
+    Bx, Va, Lo = (OE.Placeholder(f32, [1, 1, 3, 4]) for _ in range(3))
+    corners = Oop._box_corners(Bx, Va, Lo, Oop.BOXES_SSD, 200, 100, clip, centered)
+    got = OE.run(OE.Program('decode', [Bx, Va, Lo], corners), [_SSD_PRIORS, _SSD_VAR, _SSD_LOC])
+    got = np.stack([g.reshape(3) for g in got], axis=1)  # rows of (y1, x1, y2, x2)
+    np.testing.assert_allclose(got, np.array(_SSD_WANT[(centered, clip)], np.float32), rtol=2e-6, atol=2e-7)
+
+
+@pytest.mark.parametrize('with_arm,share,style', [(False, True, 2), (True, True, 2), (False, False, 2), (False, True, 1)])
+def test_ssd_result_rows_carry_the_decoded_boxes(with_arm, share, style):
+    """The four extra columns of the score rows are (x1, y1, x2, y2) of the selected box, decoded here box by box
+    with scalar arithmetic (twice for the refined priors of the ARM variant) and clipped to the unit square."""
+    prog, vals = _ssd_case(OE, Oop, with_arm, share, style)
+    rb, rs, rv = OE.run(prog, vals)
+    priors, var, loc = vals[0], vals[4], vals[5]
+    arm = vals[6] if with_arm else None
+    W = H = np.float32(100)
+    f = np.float32
+
+    def decode(box, v, l, centred):  # -> (x1, y1, x2, y2)
+        if centred:
+            x1, y1, x2, y2 = box[0] / W, box[1] / H, box[2] / W, box[3] / H
+            pw, ph = x2 - x1, y2 - y1
+            xc, yc = v[0] * l[0] * pw + (x1 + x2) / f(2), v[1] * l[1] * ph + (y1 + y2) / f(2)
+            hw, hh = np.exp(v[2] * l[2]) * pw / f(2), np.exp(v[3] * l[3]) * ph / f(2)
+            out = [xc - hw, yc - hh, xc + hw, yc + hh]
+        else:
+            out = [box[k] / W + v[k] * l[k] for k in range(4)]
+        return [min(max(t, f(0)), f(1)) for t in out]  # clip_before_nms
+
+    for row in range(int(rv[0])):
+        b, c, j = (int(t) for t in rb[row])
+        cls = c + 1 if style == 1 else c  # the MXNET style reports the class without the background id
+        lc = 0 if share else cls
+        if with_arm:
+            refined = decode(priors[b, j], var[b, j], arm[b, lc, j], True)
+            want = decode(refined, var[b, j], loc[b, lc, j], True)
+        else:
+            want = decode(priors[b, j], var[b, j], loc[b, lc, j], False)
+        np.testing.assert_allclose(rs[row, 3:], np.array(want, np.float32), rtol=1e-5, atol=1e-6, err_msg=str((row, b, c, j)))

@@ -343,3 +343,39 @@ def test_gemv_known_answers(dtype_name):
     if dtype_name == 'INT64':
         np.testing.assert_array_equal(o2, [19, 19, 19])
     np.testing.assert_array_equal(p, [1])
+
+
+def test_bf16_contractions_round_once_after_the_last_tap():
+    """What the declared bf16 semantics fix (fp32 accumulation, one rounding to nearest even at the end, the
+    initial value inside the accumulator), on sums that fp32 holds exactly and bf16 does not: rounding after
+    every tap, after partial sums, or before the initial value goes in gives 256 / 258 / 128 instead."""
+    import programs
+    from oracle import tile_oplib as Oop
+    prog, vals, _ = programs.bf16_rounding_placement(E, Oop)
+    for got, want in zip(E.run(prog, vals), programs.BF16_ROUNDING_ANSWERS):
+        np.testing.assert_array_equal(got, want)
+
+
+def test_f16_contraction_rounds_once():
+    """The same for fp16 (11 significant bits): 2048 + 1 + 1 + 1 = 2051 -> 2052 (per tap: 2048)."""
+    A = E.Placeholder(D.FLOAT16, [1, 4])
+    B = E.Placeholder(D.FLOAT16, [4, 1])
+    i, j, k = E.TensorIndexes(3)
+    O = E.Contraction().outShape(1, 1).outAccess(i, j).sum(A[i, k] * B[k, j]).build()
+    out, = E.run(E.Program('f16', [A, B], [O]), [np.array([[2048, 1, 1, 1]], np.float16), np.ones((4, 1), np.float16)])
+    assert float(out[0, 0]) == 2052.0
+
+
+def test_eq_combination_closed_forms():
+    """`eq` (edsl.h:421; i1 result: eval.cc:25; tile_to_linalg.cc:1257-1262): any / all / parity of the match
+    table by numpy, NaN never equal, uncovered elements hold min's identity (true)."""
+    import programs
+    from oracle import tile_oplib as Oop
+    prog, vals, _ = programs.eq_combination(E, Oop)
+    outs = E.run(prog, vals)
+    want = programs.eq_combination_answers(*vals)
+    assert len(outs) == len(want)
+    for k, (g, w) in enumerate(zip(outs, want)):
+        assert g.dtype == np.bool_ and g.shape == w.shape, k
+        np.testing.assert_array_equal(g, w, err_msg=str(k))
+    assert outs[0].any() and not outs[1].all() and outs[2].any() and not outs[2].all()  # the case is telling

@@ -37,7 +37,15 @@ def test_program_matches_oracle(name, target):
     prog, vals, _ = programs.ALL[name](E, op)
     got = E.run(prog, vals, target=target)
     if name.startswith('config3') and tol == programs.BF16:
-        # the window argmax is exact given the pooled values; compare it where the bf16 pooled values agree
+        # The pooled bf16 values may differ from the oracle's by one rounding step upstream, and with them the
+        # winning tap.  Every index is therefore checked, bit for bit, against the device's own pool input (a
+        # third program output); the comparison with the oracle's indices covers the positions whose pooled values
+        # agree.
+        prog3, vals3, _ = programs.config3_xception_block(E, op, with_pool_input=True)
+        M3, AM3, R3 = E.run(prog3, vals3, target=target)
+        np.testing.assert_array_equal(M3, got[0])
+        np.testing.assert_array_equal(AM3, got[1])
+        np.testing.assert_array_equal(AM3, programs.window_argmax_of(R3, M3))
         same = got[0] == ref[0]
         assert same.mean() > 0.98
         np.testing.assert_array_equal(got[1][same], ref[1][same])
@@ -72,9 +80,17 @@ def test_config3_full_size_against_oracle_on_a_slice():
     """BASELINE configs[3] at full size (N64 19x19x728 bf16: depthwise 3x3 -> pointwise -> scale/shift + ReLU ->
     max-pool 3x3/2 + window argmax) through the plaidml API.  Images do not interact, so the first two images of the
     batch-64 run must equal what the oracle computes for a batch of those two with the same weights."""
-    prog, vals, _ = programs.config3_xception_block(E, op, N=64, C=728)
-    M, AM = E.run(prog, vals, target='hip')
-    assert M.shape == (64, 10, 10, 728) and AM.shape == (64, 10, 10, 728)
+    prog, vals, _ = programs.config3_xception_block(E, op, N=64, C=728, with_pool_input=True)
+    M, AM, R = E.run(prog, vals, target='hip')
+    assert M.shape == (64, 10, 10, 728) and AM.shape == (64, 10, 10, 728) and R.shape == (64, 19, 19, 728)
+    # every index of the whole batch, bit for bit, from the device's own pool input; and the pooled values exactly
+    np.testing.assert_array_equal(AM, programs.window_argmax_of(R, M))
+    padded = np.zeros((64, 21, 21, 728), np.float32)   # ReLU outputs: zero padding never wins over a window's maximum
+    padded[:, 1:20, 1:20] = R
+    np.testing.assert_array_equal(M, np.max([padded[:, a:a + 20:2, b:b + 20:2] for a in range(3) for b in range(3)], axis=0))
+    M2, AM2 = E.run(programs.config3_xception_block(E, op, N=64, C=728)[0], vals, target='hip')
+    np.testing.assert_array_equal(M2, M)               # the two-output program of the benchmark gives the same
+    np.testing.assert_array_equal(AM2, AM)
     oprog, ovals, _ = programs.config3_xception_block(OE, Oop, N=2, C=728)
     ovals[0] = vals[0][:2]
     for a, b in zip(ovals[1:], vals[1:]):
@@ -89,6 +105,49 @@ def test_config3_full_size_against_oracle_on_a_slice():
     # structural facts that hold for every image
     assert AM.min() >= 0 and AM.max() <= 8
     assert (M >= 0).all()                             # max over ReLU outputs
+
+
+def test_config0_full_size_against_float64():
+    """BASELINE configs[0] at full size through the plaidml API: fp32 1024^3, U(-1, 1), against float64 numpy."""
+    prog, vals, _ = programs.config0_gemm_f32(E, op, n=1024)
+    C, = E.run(prog, vals, target='hip')
+    want = vals[0].astype(np.float64) @ vals[1].astype(np.float64)
+    # rtol 1e-3 on the scale of a result row (entries are sums of 1024 terms of either sign: those near zero are
+    # compared through atol = 1e-3 x the typical magnitude sqrt(1024 / 9))
+    np.testing.assert_allclose(C, want, rtol=1e-3, atol=1e-3 * np.sqrt(1024 / 9.0))
+    assert np.abs(C - want).max() < 1e-3                  # measured: a few 1e-5 (fp32 accumulation over 1024 terms)
+
+
+@pytest.mark.parametrize('dtype_name', ['FLOAT32', 'BFLOAT16'])
+def test_config1_full_size_through_exec(dtype_name):
+    """BASELINE configs[1] at full size (N128 56x56x64, 3x3x64x64, SAME, + bias + ReLU) through the plaidml API, in
+    fp32 and in bf16: images do not interact, so images 0 and 127 must equal the oracle's result for a batch of
+    those two; sampled pixels of every image are checked against float64 arithmetic on the same values."""
+    print('configs[1] full size', dtype_name, flush=True)
+    prog, vals, tol = programs.config1_conv(E, op, dtype_name, N=128, H=56, W=56)
+    O, = E.run(prog, vals, target='hip')
+    assert O.shape == (128, 56, 56, 64)
+    plan = dict(prog.passes)['hip-plan']
+    assert 'conv2d' in plan and 'contract (general)' not in plan, plan
+    oprog, ovals, _ = programs.config1_conv(OE, Oop, dtype_name, N=2, H=56, W=56)
+    ovals[0] = vals[0][[0, 127]]
+    np.testing.assert_array_equal(ovals[1], vals[1])
+    ref, = OE.run(oprog, ovals)
+    rtol, atol = (2e-2, 2e-2) if dtype_name == 'BFLOAT16' else (1e-3, 1e-5)
+    np.testing.assert_allclose(O[[0, 127]], ref, rtol=rtol, atol=atol)
+    Iv, Fv, Bv = (v.astype(np.float64) for v in vals)
+    r = np.random.default_rng(12)
+    pix = [(int(n), int(y), int(x)) for n, y, x in zip(r.integers(0, 128, 300), r.integers(0, 56, 300), r.integers(0, 56, 300))]
+    pix += [(n, y, x) for n in (0, 64, 127) for y in (0, 55) for x in (0, 55)]     # corners: padding on two sides
+    for n, y, x in pix:
+        acc = Bv.copy()
+        for ky in range(3):
+            for kx in range(3):
+                yy, xx = y + ky - 1, x + kx - 1
+                if 0 <= yy < 56 and 0 <= xx < 56:
+                    acc += Iv[n, yy, xx] @ Fv[ky, kx]
+        np.testing.assert_allclose(O[n, y, x], np.maximum(acc, 0), rtol=rtol, atol=atol if dtype_name == 'BFLOAT16' else 1e-4,
+                                   err_msg=str((n, y, x)))
 
 
 def test_config4_full_size_image_against_golden():
