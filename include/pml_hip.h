@@ -214,6 +214,19 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
  * (pmlc/rt/jit_executable.cc:404-418): after pack_b, invoke may be given b == NULL. */
 int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s);
 
+/* The GEMM above in one call that allocates nothing, neither on the host heap of the device runtime nor in
+ * device memory: dispatch + invoke without a plan object.  It has no counterpart in the reference; it is for
+ * callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  The transposed copy of a [K][N] right-hand side (b_layout 0), which a plan keeps in memory of its
+ * own, lives in a fixed array in the library's device image instead: n * k * element size must not exceed
+ * PML_HIP_STATIC_SCRATCH_BYTES, larger right-hand sides are rejected with an error text that says so
+ * (b_layout 1 needs no copy and has no such limit).  Each GPU holds one such array for the life of the process and
+ * every call on that GPU uses it: calls that overlap on one GPU (two streams, two threads) race on it.  The
+ * result equals pml_hip_gemm_dispatch + pml_hip_gemm_invoke bit for bit (same tile choice, same kernels). */
+#define PML_HIP_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int pml_hip_gemm_run_static(const pml_hip_gemm_desc* desc, const void* a, const void* b, void* c, const void* init,
+                            const void* const* operands, void* const* outs, pml_hip_stream s);
+
 /* ---- dense contraction: 2-D convolution, NHWC (x) HWCK ------------------------
  * O[n,y,x,co] = tail( init + sum_{ky,kx,ci} I[n, sy*y + dy*ky - py, sx*x + dx*kx - px, ci] * F[ky,kx,ci,co] )
  * over the taps that fall inside the input (out-of-range taps are not part of

@@ -253,6 +253,32 @@ int device_cus() {
   return cached[dev];
 }
 
+// Device memory of the entry point that allocates nothing (pml_hip_gemm_run_static): the transposed
+// right-hand side Bt[N][K].  Every GPU the library runs on holds its own copy of the array until the process
+// ends.  In host code the array's name is only a handle: the address kernels and copies use is looked up once
+// per device, with that device current, and kept here.
+static __device__ __align__(256) unsigned char scratch[PML_HIP_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+std::mutex g_scratch_mutex;
+
+// Address of `scratch` on the current device; null (and the error text set) on failure.
+void* scratch_of_current_device() {
+  int dev = 0;
+  if (check(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+  if (dev < 0 || dev >= kMaxDevices) {
+    fail("device ordinal beyond the per-device table");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (check(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
 // Everything of the kernel arguments that the descriptor fixes (no operand pointers).
 void conv_args(const Plan* p, IgemmArgs& g) {
   const pml_hip_conv2d_desc& d = p->conv;
@@ -354,7 +380,8 @@ int pml_hip_init(int device_ordinal) {
   int n = pml_hip_device_count();
   if (n <= 0) return fail("no HIP device is visible");
   if (device_ordinal < 0 || device_ordinal >= n) return fail("device ordinal out of range");
-  return check(hipSetDevice(device_ordinal), "hipSetDevice");
+  if (check(hipSetDevice(device_ordinal), "hipSetDevice")) return 1;
+  return scratch_of_current_device() ? 0 : 1;
 }
 
 int pml_hip_device_name(char* buf, size_t buf_len) {
@@ -425,36 +452,44 @@ int pml_hip_event_elapsed_ms(pml_hip_event start, pml_hip_event stop, float* ms)
 // GEMM
 // ---------------------------------------------------------------------------
 
-int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
+// Checks a GEMM descriptor; the MFMA kind (>= 0) or -1 with the error text set.
+static int gemm_desc_kind(const pml_hip_gemm_desc* d) {
   if (!d) {
     fail("null descriptor");
-    return 0;
+    return -1;
   }
   const int kind = mfma_kind_of(d->in_dtype);
   if (kind < 0) {
     fail("gemm: in_dtype must be F32, BF16 or I8");
-    return 0;
+    return -1;
   }
   const bool out_ok = (kind == KIND_I8) ? d->out_dtype == PML_HIP_I32
                                         : (d->out_dtype == PML_HIP_F32 || (kind == KIND_BF16 && d->out_dtype == PML_HIP_BF16));
   if (!out_ok) {
     fail("gemm: out_dtype does not fit in_dtype");
-    return 0;
+    return -1;
   }
   if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->lda < d->k || d->ldb < (d->b_layout ? d->k : d->n) || d->ldc < d->n ||
       (d->b_layout != 0 && d->b_layout != 1)) {
     fail("gemm: bad sizes or leading dimensions");
-    return 0;
+    return -1;
   }
   const int es = dt_size(d->in_dtype);
   if ((d->k * es) % 16 != 0 || (d->lda * es) % 16 != 0 || (d->b_layout && (d->ldb * es) % 16 != 0)) {
     fail("gemm: K and the K-contiguous leading dimensions must cover whole 16-byte vectors");
-    return 0;
+    return -1;
   }
   if (!valid_tail(d->tail)) {
     fail("gemm: malformed tail");
-    return 0;
+    return -1;
   }
+  return kind;
+}
+
+int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
+  const int kind = gemm_desc_kind(d);
+  if (kind < 0) return 0;
+  const int es = dt_size(d->in_dtype);
   Plan* p = new Plan();
   p->kind = PLAN_GEMM;
   p->mfma_kind = kind;
@@ -475,18 +510,19 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   return (int64_t)(intptr_t)p;
 }
 
-int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, const void* init,
-                        const void* const* operands, void* const* outs, pml_hip_stream s) {
-  Plan* p = (Plan*)(intptr_t)plan;
-  if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
-  const pml_hip_gemm_desc& d = p->gemm;
+// One GEMM launch sequence: the per-run transposition of a [K][N] right-hand side into `bt` (device memory of
+// n x bt_ld elements; skipped when b is null, i.e. packed earlier, or already [N][K]), then the MFMA kernel.
+// Shared by the plan-based entry point and by the one that allocates nothing.
+static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* bt, int64_t bt_ld, bool packed,
+                    const void* a, const void* b, void* c, const void* init, const void* const* operands,
+                    void* const* outs, pml_hip_stream s) {
   if (!a || !c) return fail("gemm_invoke: null operand");
-  if (!b && (!p->packed || d.b_layout)) return fail("gemm_invoke: b is null and no packed right-hand side exists");
+  if (!b && (!packed || d.b_layout)) return fail("gemm_invoke: b is null and no packed right-hand side exists");
   if (d.b_layout && ((uintptr_t)b & 15) != 0) return fail("gemm_invoke: an [N][K] right-hand side must be 16-byte aligned");
   if (((uintptr_t)a & 15) != 0) return fail("gemm_invoke: A must be 16-byte aligned");
   if (d.init_kind && !init) return fail("gemm_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
-  if (b && !d.b_layout && check(transpose_pack(es, b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack"))
+  if (b && !d.b_layout && check(transpose_pack(es, b, bt, d.k, d.n, d.ldb, bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   IgemmArgs g;
   std::memset(&g, 0, sizeof g);
@@ -495,8 +531,8 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   g.K = d.k;
   g.A = a;
   g.lda = d.lda;
-  g.Bt = d.b_layout ? b : p->bt;
-  g.ldbt = d.b_layout ? d.ldb : p->bt_ld;
+  g.Bt = d.b_layout ? b : bt;
+  g.ldbt = d.b_layout ? d.ldb : bt_ld;
   g.C = c;
   g.ldc = d.ldc;
   g.out_dtype = d.out_dtype;
@@ -524,7 +560,32 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("gemm_invoke: missing extra output");
-  return check(igemm_launch(p->mfma_kind, p->tile, false, g, (hipStream_t)s), "igemm_launch");
+  return check(igemm_launch(mfma_kind, tile, false, g, (hipStream_t)s), "igemm_launch");
+}
+
+int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, const void* init,
+                        const void* const* operands, void* const* outs, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
+  return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s);
+}
+
+int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const void* b, void* c, const void* init,
+                            const void* const* operands, void* const* outs, pml_hip_stream s) {
+  const int kind = gemm_desc_kind(d);
+  if (kind < 0) return 1;
+  if (!b) return fail("gemm_run_static: b is null");
+  void* bt = nullptr;
+  if (!d->b_layout) {
+    // n and k are positive and each below 2^31 by the check below, so the product cannot overflow
+    if (d->n > PML_HIP_STATIC_SCRATCH_BYTES || d->k > PML_HIP_STATIC_SCRATCH_BYTES ||
+        (uint64_t)d->n * (uint64_t)d->k * (uint64_t)dt_size(d->in_dtype) > (uint64_t)PML_HIP_STATIC_SCRATCH_BYTES)
+      return fail("gemm_run_static: the transposed right-hand side (n x k elements) exceeds PML_HIP_STATIC_SCRATCH_BYTES (32 MiB)");
+    bt = scratch_of_current_device();
+    if (!bt) return 1;
+  }
+  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype));
+  return gemm_run(*d, kind, tile, bt, d->k, false, a, b, c, init, operands, outs, s);
 }
 
 // ---------------------------------------------------------------------------
