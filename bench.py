@@ -194,7 +194,7 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):
 def resnet50_leg(E, batch=128, runs=5):
     """Whole-network forward through libplaidml.so: device time between the first and the last kernel of a run."""
     from plaidml_amd import edsl as P, op as Pop, resnet50
-    prog, _, flops_full_box = resnet50.build(P, Pop, batch=batch, round_fn=E.round_bf16)
+    prog, _, flops_full_box = resnet50.build(P, Pop, batch=batch, round_fn=P.round_bf16)
     runner = P.Runner(prog, target='hip')
     x = np.random.default_rng(11).uniform(0, 1, (batch, 224, 224, 3)).astype(np.float32)
     times = []

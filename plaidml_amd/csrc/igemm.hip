@@ -165,9 +165,29 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
   const int lv = tid % CPR;
   const int lr = tid / CPR;
   const int lc = lv ^ ((lr >> kSwzShift) & (CPR - 1));        // the chunk of its row this thread fetches
-  const int kbytes_row = (int)(CONV ? p.CI * ES : p.K * ES);  // valid bytes per (tap) row
+  int kbytes_row = __builtin_amdgcn_readfirstlane((int)(CONV ? p.CI * ES : p.K * ES));  // valid bytes per (tap) row
+  asm volatile("" : "+s"(kbytes_row));
 
-  unsigned a_off[A_VECS];  // GEMM: byte offset of the row; CONV: of the image; kOutside for rows past M
+  // Loop-invariant scalars of the geometry, pinned to scalar registers: read through the argument block inside
+  // the K loop they would be re-fetched there (a scalar load and a wait that also drains the LDS reads).
+  auto pinned = [](int v) {
+    v = __builtin_amdgcn_readfirstlane(v);
+    asm volatile("" : "+s"(v));
+    return v;
+  };
+  const int cH = pinned(CONV ? p.H : 0), cW = pinned(CONV ? p.W : 0);
+  const int cKW = pinned(CONV ? p.KW : 1), cKH = pinned(CONV ? p.KH : 1);
+  const int cDH = pinned(CONV ? p.DH : 0), cDW = pinned(CONV ? p.DW : 0);
+  const int pix_bytes = pinned(p.CI * ES);                               // bytes of one tap's K-run
+  const int pix_pitch = pinned(p.pix_pitch ? p.pix_pitch : p.CI * ES);   // bytes between neighbouring input pixels
+  // a K-run that spans several pixels (pitch < run): chunk byte -> pixel as multiply-and-shift, exact for the
+  // few thousand bytes a run can have; otherwise every chunk lies in the tap's own pixel
+  const unsigned pitch_magic = (CONV && p.pix_pitch) ? (unsigned)pinned((int)(((1u << 20) + (unsigned)p.pix_pitch - 1) / (unsigned)p.pix_pitch)) : 0u;
+
+  // GEMM: byte offset of the row, kOutside for rows past M.  CONV: byte offset of input pixel (ih0, iw0) of the
+  // row's output pixel, the one its tap (0, 0) reads -- possibly before the image's first byte, which is why it
+  // is only ever used together with the bounds check on (ih0 + dh, iw0 + dw); rows past M fail that check.
+  unsigned a_off[A_VECS];
   int a_ih0[A_VECS], a_iw0[A_VECS];
 #pragma unroll
   for (int i = 0; i < A_VECS; ++i) {
@@ -181,9 +201,9 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
       const unsigned rem = mu - nb * (unsigned)(p.OH * p.OW);
       const unsigned ohu = fast_div(rem, p.div_ow_magic, p.div_ow_shift);
       const int oh = (int)ohu, ow = (int)(rem - ohu * (unsigned)p.OW);
-      a_ih0[i] = oh * p.SH - p.PH;
+      a_ih0[i] = ok ? oh * p.SH - p.PH : -(1 << 28);
       a_iw0[i] = ow * p.SW - p.PW;
-      a_off[i] = ok ? (unsigned)((int64_t)nb * ((int64_t)p.H * p.W * (p.pix_pitch ? p.pix_pitch : p.CI * ES))) : kOutside;
+      a_off[i] = (unsigned)((int64_t)nb * ((int64_t)cH * cW * pix_pitch)) + (unsigned)((a_ih0[i] * cW + a_iw0[i]) * pix_pitch);
     } else {
       a_ih0[i] = a_iw0[i] = 0;
       a_off[i] = ok ? (unsigned)(mm * p.lda * ES) : kOutside;
@@ -196,45 +216,53 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
     b_off[i] = n < p.N ? (unsigned)(n * p.ldbt * ES) : kOutside;
   }
 
-  const int slabs_per_tap = (kbytes_row + kSlabBytes - 1) / kSlabBytes;
+  const int slabs_per_tap = pinned((kbytes_row + kSlabBytes - 1) / kSlabBytes);
   const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : slabs_per_tap;
-  const int pix_bytes = p.CI * ES;                              // bytes of one tap's K-run
-  const int pix_pitch = p.pix_pitch ? p.pix_pitch : pix_bytes;  // bytes between neighbouring input pixels
 
-  // Requests of slab s into ring stage `stage`, one 16-byte-per-lane load at a time (index l: the A
-  // rows first, then the Bt rows) so that they can be spread between the MFMAs.  Past the last slab
-  // every offset is outside: the request count per slab stays constant, which is what the vmcnt
-  // arithmetic below relies on.
+  // Requests of the next slab into ring stage `stage`, one 16-byte-per-lane load at a time (index l: the A
+  // rows first, then the Bt rows) so that they can be spread between the MFMAs.  Slabs are prepared in order,
+  // one per call, so the filter tap and the position inside its channel run are counters, not quotients.
+  // Past the last slab every offset is outside: the request count per slab stays constant, which is what
+  // the vmcnt arithmetic below relies on.
   unsigned char* req_base = smem;
-  unsigned req_a = 0, req_b = 0;  // slab-dependent part of the A / Bt offsets (CONV: A adds the tap per row)
-  int req_dh = 0, req_dw = 0, req_px = 0;  // req_px: pixels the chunk lies beyond the tap's first one (pitch < run)
+  unsigned req_a = 0, req_b = 0;  // slab-dependent part of the A / Bt offsets
+  int req_dh = 0, req_dw = 0;     // CONV: the tap's displacement in input rows / columns (columns: plus the chunk's pixel)
   bool req_ok = false;
-  auto prepare_slab = [&](int s, int stage) {
+  int nx_kh = 0, nx_kw = 0, nx_cs = 0, nx_dh = 0, nx_dw = 0, nx_tap = 0;  // CONV: tap and slab-in-tap of the next slab
+  int nx_kbo = 0;                                                          // GEMM: its first byte of K
+  auto prepare_slab = [&](int stage) {
     req_base = smem + stage * kStage + wave * 1024;  // one request of a wavefront fills 1 KB
-    const bool live = s < n_slabs;
     if (CONV) {
-      const int tap = s / slabs_per_tap;
-      const int cs = s - tap * slabs_per_tap;
-      const int kh = tap / p.KW, kw = tap - kh * p.KW;
-      const int cb = cs * kSlabBytes + lc * 16;  // byte offset inside the channel vector
-      req_ok = live && cb < kbytes_row;
-      req_dh = kh * p.DH;
-      req_dw = kw * p.DW;
-      req_px = cb / pix_pitch;
-      req_a = (unsigned)cb;
-      req_b = req_ok ? (unsigned)(tap * pix_bytes + cb) : kOutside;  // Bt row: tap-major, channel-minor
+      const int cb = nx_cs * kSlabBytes + lc * 16;  // byte offset inside the tap's K-run
+      req_ok = (nx_kh < cKH) & (cb < kbytes_row);
+      const int px = (int)(((unsigned)cb * pitch_magic) >> 20);
+      req_dh = nx_dh;
+      req_dw = nx_dw + px;
+      req_a = (unsigned)((nx_dh * cW + nx_dw) * pix_pitch + cb);
+      req_b = req_ok ? (unsigned)(nx_tap + cb) : kOutside;  // Bt row: tap-major, channel-minor
+      if (++nx_cs == slabs_per_tap) {
+        nx_cs = 0;
+        nx_tap += pix_bytes;
+        nx_dw += cDW;
+        if (++nx_kw == cKW) {
+          nx_kw = 0;
+          nx_dw = 0;
+          ++nx_kh;
+          nx_dh += cDH;
+        }
+      }
     } else {
-      const int kbo = s * kSlabBytes + lc * 16;
-      req_a = req_b = (live && kbo < kbytes_row) ? (unsigned)kbo : kOutside;
+      const int kbo = nx_kbo + lc * 16;
+      req_a = req_b = kbo < kbytes_row ? (unsigned)kbo : kOutside;
+      nx_kbo += kSlabBytes;
     }
   };
   auto issue_load = [&](int l) {
     if (l < A_VECS) {
       unsigned off;
       if (CONV) {
-        const int ih = a_ih0[l] + req_dh, iw = a_iw0[l] + req_dw;
-        const bool ok = req_ok && (unsigned)ih < (unsigned)p.H && (unsigned)(iw + req_px) < (unsigned)p.W;
-        off = ok ? join_offsets(a_off[l], (unsigned)((ih * p.W + iw) * pix_pitch + (int)req_a)) : kOutside;
+        const bool ok = req_ok & ((unsigned)(a_ih0[l] + req_dh) < (unsigned)cH) & ((unsigned)(a_iw0[l] + req_dw) < (unsigned)cW);
+        off = ok ? a_off[l] + req_a : kOutside;
       } else {
         off = join_offsets(a_off[l], req_a);
       }
@@ -261,7 +289,7 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
   // Every ring stage is requested before the first multiply: kStages slabs in flight.
 #pragma unroll
   for (int s = 0; s < kStages; ++s) {
-    prepare_slab(s, s);
+    prepare_slab(s);
 #pragma unroll
     for (int l = 0; l < kLoads; ++l) issue_load(l);
   }
@@ -319,7 +347,7 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
           if (wave == 15 || (wave == 7 && NT == 512)) tr[1] = __builtin_amdgcn_s_memrealtime();  // the 100 MHz clock, to calibrate
         }
 #endif
-        prepare_slab(s + kStages, stage);
+        prepare_slab(stage);
       }
       const unsigned char* ra_ = last ? a_next : a_base;
       const unsigned char* rb_ = last ? b_next : b_base;
@@ -515,7 +543,7 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
 template <int KIND, bool CONV>
 hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
 #ifdef PML_DEV_CFG  // development builds: one configuration, given as the template arguments after KIND
-  if constexpr (!CONV && KIND == PML_KIND) return launch_cfg<KIND, PML_DEV_CFG>(a, s);
+  if constexpr (CONV == PML_DEV_CONV && KIND == PML_KIND) return launch_cfg<KIND, PML_DEV_CFG>(a, s);
   return hipErrorInvalidValue;
 #else
   switch (cfg) {

@@ -96,7 +96,8 @@ _SIGS = {
     'plaidml_executable_run': (f64, [vp, sz, ctypes.POINTER(vp), sz, ctypes.POINTER(vp)]),
 }
 # the two functions that take no plaidml_error, and the statistics helper
-EXPORTS = sorted(list(_SIGS) + ['plaidml_string_ptr', 'plaidml_string_free', 'plaidml_hip_last_run_stats'])
+EXPORTS = sorted(list(_SIGS) + ['plaidml_string_ptr', 'plaidml_string_free', 'plaidml_hip_last_run_stats',
+                               'plaidml_hip_last_run_memory', 'plaidml_hip_last_run_step_ms'])
 
 _lib = None
 
@@ -118,6 +119,10 @@ def lib():
         L.plaidml_string_free.argtypes = [vp]
         L.plaidml_hip_last_run_stats.restype = None
         L.plaidml_hip_last_run_stats.argtypes = [ctypes.POINTER(f64), ctypes.POINTER(f64), ctypes.POINTER(f64), ctypes.POINTER(sz)]
+        L.plaidml_hip_last_run_memory.restype = None
+        L.plaidml_hip_last_run_memory.argtypes = [ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]
+        L.plaidml_hip_last_run_step_ms.restype = sz
+        L.plaidml_hip_last_run_step_ms.argtypes = [sz, ctypes.POINTER(f64)]
         _lib = L
         call('plaidml_init')
         call('plaidml_edsl_init')
@@ -938,7 +943,7 @@ class Executable(_Handle):
         super().__init__(call('plaidml_jit', program.as_ptr(), device.encode()))
 
     def run(self, inputs, outputs):
-        """inputs / outputs: lists of Buffer.  Returns the device execution time in ms."""
+        """inputs / outputs: lists of Buffer.  Returns the wall time of the run in ms, transfers included."""
         return call('plaidml_executable_run', self._ptr, len(inputs), _ptr_array([b.as_ptr() for b in inputs]), len(outputs),
                     _ptr_array([b.as_ptr() for b in outputs]))
 
@@ -946,7 +951,12 @@ class Executable(_Handle):
 def last_run_stats():
     k, h, d, n = f64(), f64(), f64(), sz()
     lib().plaidml_hip_last_run_stats(ctypes.byref(k), ctypes.byref(h), ctypes.byref(d), ctypes.byref(n))
-    return {'kernel_ms': k.value, 'h2d_ms': h.value, 'd2h_ms': d.value, 'launches': n.value}
+    a, u, t = sz(), sz(), sz()
+    lib().plaidml_hip_last_run_memory(ctypes.byref(a), ctypes.byref(u), ctypes.byref(t))
+    steps = (f64 * (n.value or 1))()
+    got = lib().plaidml_hip_last_run_step_ms(n.value, steps)  # per launch; empty unless PLAIDML_PROFILE=1 was set
+    return {'kernel_ms': k.value, 'h2d_ms': h.value, 'd2h_ms': d.value, 'launches': n.value, 'arena_bytes': a.value,
+            'unshared_temp_bytes': u.value, 'device_bytes': t.value, 'step_ms': [steps[i] for i in range(got if got < n.value else n.value)]}
 
 
 def to_bf16_bits(a):
@@ -960,6 +970,11 @@ def to_bf16_bits(a):
 
 def from_bf16_bits(b):
     return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def round_bf16(a):
+    """float32 -> the nearest bfloat16 value (ties to even), as float32."""
+    return from_bf16_bits(to_bf16_bits(a))
 
 
 class Runner:

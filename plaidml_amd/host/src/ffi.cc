@@ -822,4 +822,21 @@ void plaidml_hip_last_run_stats(double* kernel_ms, double* h2d_ms, double* d2h_m
   if (launches) *launches = s.launches;
 }
 
+// Device memory of the executable behind the calling thread's most recent run: the arena its temporaries share,
+// what they would take unshared, and everything it holds on the device (arena + inputs + outputs + constants).
+void plaidml_hip_last_run_memory(size_t* arena_bytes, size_t* unshared_temp_bytes, size_t* device_bytes) {
+  rt::InvokeStats s = rt::lastInvokeStats();
+  if (arena_bytes) *arena_bytes = s.arena_bytes;
+  if (unshared_temp_bytes) *unshared_temp_bytes = s.unshared_temp_bytes;
+  if (device_bytes) *device_bytes = s.device_bytes;
+}
+
+// Per-launch device milliseconds of that run (filled only when PLAIDML_PROFILE=1 was set during it): copies up
+// to `capacity` values to `ms` and returns how many launches the run had timed.
+size_t plaidml_hip_last_run_step_ms(size_t capacity, double* ms) {
+  rt::InvokeStats s = rt::lastInvokeStats();
+  for (size_t i = 0; i < s.step_ms.size() && i < capacity && ms; ++i) ms[i] = s.step_ms[i];
+  return s.step_ms.size();
+}
+
 }  // extern "C"

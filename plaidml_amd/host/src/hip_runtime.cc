@@ -1,6 +1,9 @@
 #include "hip_runtime.h"
 
+#include <algorithm>
 #include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <regex>
@@ -18,6 +21,14 @@ namespace {
 
 thread_local InvokeStats g_stats;
 
+constexpr size_t kAlign = 256;  // arena offsets; also the slack behind every value (kernels read whole 16-byte vectors)
+size_t padded(size_t bytes) { return (bytes + 16 + kAlign - 1) / kAlign * kAlign; }
+
+bool profileRequested() {
+  const char* e = std::getenv("PLAIDML_PROFILE");
+  return e && std::string(e) == "1";
+}
+
 void hipCheck(int status, const char* what) {
   if (status != 0) throw std::runtime_error(std::string(what) + ": " + pml_hip_last_error());
 }
@@ -33,10 +44,22 @@ class HipExecutable final : public Executable {
       : program_(std::move(program)), plan_(std::move(plan)), ordinal_(ordinal) {
     hipCheck(pml_hip_init(ordinal_), "pml_hip_init");
     device_.assign(plan_->buffers.size(), nullptr);
+    owned_.assign(plan_->buffers.size(), false);
     try {
+      // Inputs, outputs and constants keep memory of their own for the life of the executable; temporaries
+      // share one arena, each placed by the span of steps in which it is live (what the reference's
+      // resize-tmps / dealloc placement does for its heap temporaries, pmlc/target/x86/pipeline.cc:289-360).
+      const std::vector<size_t> offsets = placeTemporaries();
+      if (arena_bytes_) hipCheck(pml_hip_malloc(&arena_, arena_bytes_), "pml_hip_malloc (arena)");
       for (size_t i = 0; i < plan_->buffers.size(); ++i) {
         const BufferInfo& b = plan_->buffers[i];
+        if (b.kind == BufferInfo::Temp) {
+          device_[i] = static_cast<char*>(arena_) + offsets[i];
+          continue;
+        }
         hipCheck(pml_hip_malloc(&device_[i], b.bytes + 16), "pml_hip_malloc");
+        owned_[i] = true;
+        fixed_bytes_ += padded(b.bytes);
         if (b.kind == BufferInfo::Constant)
           hipCheck(pml_hip_memcpy_h2d(device_[i], b.constant->data(), b.constant->size(), nullptr), "upload constant");
       }
@@ -58,21 +81,51 @@ class HipExecutable final : public Executable {
     if (inputs.size() != plan_->input_buffers.size() || outputs.size() != plan_->output_buffers.size())
       throw std::runtime_error("executable invoked with the wrong number of buffers");
     InvokeStats st;
-    double t0 = nowMs();
+    const double start = nowMs();
+    double t0 = start;
+    const bool profile = profileRequested();
     for (size_t i = 0; i < inputs.size(); ++i) {
       const BufferInfo& b = plan_->buffers[plan_->input_buffers[i]];
       if (inputs[i]->size() < b.bytes) throw std::runtime_error("input buffer #" + std::to_string(i) + " is too small");
       hipCheck(pml_hip_memcpy_h2d(device_[plan_->input_buffers[i]], inputs[i]->data(), b.bytes, nullptr), "h2d");
     }
     st.h2d_ms = nowMs() - t0;
+    if (profile && step_events_.size() != plan_->steps.size() + 1) {
+      step_events_.assign(plan_->steps.size() + 1, nullptr);
+      for (auto& e : step_events_) hipCheck(pml_hip_event_create(&e), "event");
+    }
     hipCheck(pml_hip_event_record(ev0_, nullptr), "event record");
-    for (size_t i = 0; i < plan_->steps.size(); ++i) launch(i);
+    for (size_t i = 0; i < plan_->steps.size(); ++i) {
+      if (profile) hipCheck(pml_hip_event_record(step_events_[i], nullptr), "event record");
+      launch(i);
+    }
+    if (profile) hipCheck(pml_hip_event_record(step_events_.back(), nullptr), "event record");
     hipCheck(pml_hip_event_record(ev1_, nullptr), "event record");
     hipCheck(pml_hip_event_sync(ev1_), "event sync");
     float ms = 0;
     hipCheck(pml_hip_event_elapsed_ms(ev0_, ev1_, &ms), "event elapsed");
     st.kernel_ms = ms;
     st.launches = plan_->steps.size();
+    st.arena_bytes = arena_bytes_;
+    st.unshared_temp_bytes = unshared_temp_bytes_;
+    st.device_bytes = arena_bytes_ + fixed_bytes_;
+    if (profile) {
+      // One row per launch, in the reference's format (pmlc/rt/instrument.cc:22-43: id, loc, tag, seconds since
+      // the previous point, seconds since the start); loc is the plan's line for the step, tag its kind.
+      std::printf("\"id\",\"loc\",\"tag\",\"elapsed\",\"accumulated\"\n");
+      double total = 0;
+      st.step_ms.resize(plan_->steps.size());
+      for (size_t i = 0; i < plan_->steps.size(); ++i) {
+        float step = 0;
+        hipCheck(pml_hip_event_elapsed_ms(step_events_[i], step_events_[i + 1], &step), "event elapsed");
+        st.step_ms[i] = step;
+        total += step;
+        std::printf("%03d,\"%s\",%d,%7.6f,%7.6f\n", static_cast<int>(i), plan_->steps[i].text.c_str(),
+                    static_cast<int>(plan_->steps[i].kind), step * 1e-3, total * 1e-3);
+      }
+      std::printf("%03d,%s,%d,%7.6f,%7.6f\n", 9999, "endTime", 9999, 0.0, total * 1e-3);
+      std::fflush(stdout);
+    }
     t0 = nowMs();
     for (size_t i = 0; i < outputs.size(); ++i) {
       const BufferInfo& b = plan_->buffers[plan_->output_buffers[i]];
@@ -80,8 +133,11 @@ class HipExecutable final : public Executable {
       hipCheck(pml_hip_memcpy_d2h(outputs[i]->data(), device_[plan_->output_buffers[i]], b.bytes, nullptr), "d2h");
     }
     st.d2h_ms = nowMs() - t0;
+    st.wall_ms = nowMs() - start;
     g_stats = st;
-    return st.kernel_ms;
+    // wall time of the whole run, transfers included, as the reference returns the time around its jitted main
+    // (pmlc/rt/jit_executable.cc:484-490); the device time alone is in the statistics
+    return st.wall_ms;
   }
 
  private:
@@ -89,16 +145,95 @@ class HipExecutable final : public Executable {
   std::shared_ptr<Plan> plan_;
   int ordinal_;
   std::vector<void*> device_;
+  std::vector<bool> owned_;
+  void* arena_ = nullptr;
+  size_t arena_bytes_ = 0, fixed_bytes_ = 0, unshared_temp_bytes_ = 0;
   std::vector<int64_t> handles_;
   pml_hip_event ev0_ = nullptr, ev1_ = nullptr;
+  std::vector<pml_hip_event> step_events_;
+
+  // Offsets of the temporaries in the arena.  A temporary is live from the first to the last step that names
+  // it; steps run in order on one stream, so two temporaries whose spans do not overlap may share bytes.  A
+  // value freed by step i is not handed to a value that step i itself defines (kernels read while they write).
+  std::vector<size_t> placeTemporaries() {
+    const size_t nb = plan_->buffers.size(), ns = plan_->steps.size();
+    std::vector<int> first(nb, -1), last(nb, -1);
+    auto touch = [&](int buf, size_t step) {
+      if (buf < 0 || static_cast<size_t>(buf) >= nb) return;
+      if (first[buf] < 0) first[buf] = static_cast<int>(step);
+      last[buf] = static_cast<int>(step);
+    };
+    for (size_t i = 0; i < ns; ++i) {
+      const Step& s = plan_->steps[i];
+      for (int b : {s.a, s.b, s.c, s.init, s.out2}) touch(b, i);
+      for (int b : s.operands) touch(b, i);
+      for (int b : s.outs) touch(b, i);
+    }
+    std::vector<size_t> offsets(nb, 0);
+    struct Block { size_t off, size; };
+    std::vector<Block> free_blocks;
+    std::vector<std::vector<int>> starts(ns + 1), ends(ns + 1);
+    for (size_t b = 0; b < nb; ++b) {
+      if (plan_->buffers[b].kind != BufferInfo::Temp) continue;
+      unshared_temp_bytes_ += padded(plan_->buffers[b].bytes);
+      const size_t f = first[b] < 0 ? 0 : static_cast<size_t>(first[b]);
+      const size_t l = last[b] < 0 ? 0 : static_cast<size_t>(last[b]);
+      starts[f].push_back(static_cast<int>(b));
+      ends[l].push_back(static_cast<int>(b));
+    }
+    auto release_block = [&](size_t off, size_t size) {
+      free_blocks.push_back({off, size});
+      std::sort(free_blocks.begin(), free_blocks.end(), [](const Block& x, const Block& y) { return x.off < y.off; });
+      for (size_t k = 0; k + 1 < free_blocks.size();) {
+        if (free_blocks[k].off + free_blocks[k].size == free_blocks[k + 1].off) {
+          free_blocks[k].size += free_blocks[k + 1].size;
+          free_blocks.erase(free_blocks.begin() + static_cast<long>(k) + 1);
+        } else {
+          ++k;
+        }
+      }
+    };
+    for (size_t i = 0; i <= ns; ++i) {
+      // larger values first: they are the hard ones to place
+      std::sort(starts[i].begin(), starts[i].end(),
+                [&](int x, int y) { return plan_->buffers[x].bytes > plan_->buffers[y].bytes; });
+      for (int b : starts[i]) {
+        const size_t need = padded(plan_->buffers[b].bytes);
+        size_t best = free_blocks.size();
+        for (size_t k = 0; k < free_blocks.size(); ++k)
+          if (free_blocks[k].size >= need && (best == free_blocks.size() || free_blocks[k].size < free_blocks[best].size)) best = k;
+        if (best < free_blocks.size()) {
+          offsets[b] = free_blocks[best].off;
+          free_blocks[best].off += need;
+          free_blocks[best].size -= need;
+          if (!free_blocks[best].size) free_blocks.erase(free_blocks.begin() + static_cast<long>(best));
+        } else if (!free_blocks.empty() && free_blocks.back().off + free_blocks.back().size == arena_bytes_) {
+          // grow the free block at the end of the arena
+          offsets[b] = free_blocks.back().off;
+          arena_bytes_ = offsets[b] + need;
+          free_blocks.pop_back();
+        } else {
+          offsets[b] = arena_bytes_;
+          arena_bytes_ += need;
+        }
+      }
+      for (int b : ends[i]) release_block(offsets[b], padded(plan_->buffers[b].bytes));
+    }
+    return offsets;
+  }
 
   void release() {
     for (int64_t h : handles_)
       if (h) pml_hip_plan_free(h);
     handles_.clear();
-    for (void* p : device_)
-      if (p) pml_hip_free(p);
+    for (size_t i = 0; i < device_.size(); ++i)
+      if (device_[i] && owned_[i]) pml_hip_free(device_[i]);
     device_.clear();
+    if (arena_) pml_hip_free(arena_);
+    arena_ = nullptr;
+    for (auto& e : step_events_)
+      if (e) pml_hip_event_destroy(e);
+    step_events_.clear();
     if (ev0_) pml_hip_event_destroy(ev0_);
     if (ev1_) pml_hip_event_destroy(ev1_);
     ev0_ = ev1_ = nullptr;

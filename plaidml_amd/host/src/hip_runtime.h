@@ -22,7 +22,7 @@ namespace pmlc::rt {
 class Executable {
  public:
   virtual ~Executable() = default;
-  // returns the device execution time in milliseconds (first launch to last launch)
+  // returns the wall time of the run in milliseconds, host-device transfers included
   virtual double invoke(const std::vector<util::BufferPtr>& inputs, const std::vector<util::BufferPtr>& outputs) = 0;
 };
 
@@ -51,6 +51,11 @@ struct InvokeStats {
   double h2d_ms = 0;
   double d2h_ms = 0;
   size_t launches = 0;
+  double wall_ms = 0;              // the whole run, transfers included (what invoke returns)
+  size_t arena_bytes = 0;          // device memory shared by the temporaries
+  size_t unshared_temp_bytes = 0;  // what the temporaries would take with memory of their own
+  size_t device_bytes = 0;         // arena + inputs + outputs + constants
+  std::vector<double> step_ms;     // per launch, only with PLAIDML_PROFILE=1
 };
 InvokeStats lastInvokeStats();
 
