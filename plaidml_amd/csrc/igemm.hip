@@ -109,8 +109,15 @@ struct Ring {
 // BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4, 8 or 16 wavefronts (one, two or four
 // per SIMD).  WAVES_K = 2: two such grids, each multiplying one half of the K-blocks of every slab; their
 // partial results meet in LDS before the tail (more wavefronts for problems with few tiles and a long K).
+// Wavefronts per SIMD the register allocation has to leave room for: those of as many workgroups as the LDS
+// footprint lets a CU hold (at most two are counted on).
+template <int BM, int BN, int STAGES, int SLAB, int NT>
+constexpr int igemm_waves_per_simd() {
+  return (NT / 256) * (2 * Ring<BM, BN, STAGES, SLAB>::kBytes <= kLdsBytes ? 2 : 1);
+}
+
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
-__global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
+__global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>())) void igemm_kernel(IgemmArgs p_by_value) {
   // The argument block is read where the dispatcher put it (the kernel-argument segment, scalar loads),
   // through a reference: taking the by-value parameter's address instead makes the compiler copy all of
   // it to scratch memory as soon as one field is indexed with a run-time value.
@@ -276,7 +283,9 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
 
   // a residual tensor of the tail is requested now, so that it arrives under the K loop
   TailPrefetch<KIND, BM, BN, NT> pre;
-  tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
+  const bool direct = WAVES_K == 1 && direct_tail_ok<KIND>(p, n0, BN);
+  pre.valid = false;
+  if (!direct) tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
 
   acc_t acc[MI][NI];
 #pragma unroll
@@ -379,6 +388,17 @@ __global__ __launch_bounds__(NT) void igemm_kernel(IgemmArgs p_by_value) {
   }
   // drain the (all-outside) requests still in flight before LDS is reused
   __builtin_amdgcn_s_waitcnt(0x0F70);
+  // the common bf16 tails go straight from the accumulators to memory
+  if constexpr (KIND == KIND_BF16 && WAVES_K == 1) {
+    if (direct) {
+      // (the lane number through an opaque move: the tail's addresses are then worked out here, after the K loop,
+      // instead of being carried through it in registers the loop needs)
+      int lane_now = lane;
+      asm volatile("" : "+v"(lane_now));
+      direct_tail_bf16<MI, NI>(p, acc, m0 + wm * WM, n0 + wn * WN, lane_now);
+      return;
+    }
+  }
   __syncthreads();
 
   // ---- stage accumulators in LDS and run the tail ----

@@ -57,7 +57,9 @@ struct TailPrefetch {
   static constexpr int TPR = BN / 4;
   static constexpr int RPP = NTHREADS / TPR;
   static constexpr int kIters = (BM + RPP - 1) / RPP;
-  static constexpr bool kFits = kIters <= 8;
+  // (bf16 results take the direct tail, which prefetches in its own layout: the staged tail of the remaining
+  // edge tiles loads its residual rows when it gets there)
+  static constexpr bool kFits = kIters <= 8 && KIND != KIND_BF16;
   i32x4_t res[kFits ? kIters : 1];
   bool valid;
 };
@@ -85,6 +87,107 @@ __device__ __forceinline__ void tail_prefetch(const IgemmArgs& p, int64_t m0, in
         } else {
           pre.res[c] = *(const i32x4_t*)((const int*)p.operands[0] + m * res_rs + n);
         }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The common bf16 tails straight from the accumulators, without the trip through LDS: relu?(acc + bias)
+// and relu?(bf16(acc + bias) + residual).  A lane of a 32x32 block holds, for its row (lane & 31), the
+// four columns 8g + 4 * (lane >> 5) ... of each group g; exchanging the upper half of group 2q with the
+// lower half of group 2q + 1 (v_permlane32_swap) leaves every lane with eight neighbouring columns of its
+// row -- columns 16q + 8 * (lane >> 5) ... -- which is one 16-byte store (8-byte stores measured a third
+// slower).  The stores of a row's 64-byte run leave the wavefront within a few instructions of each other
+// and meet again in L2.
+// ---------------------------------------------------------------------------------------------------
+
+// Whether the tile can take the direct tail (uniform over the workgroup).
+template <int KIND>
+__device__ __forceinline__ bool direct_tail_ok(const IgemmArgs& p, int64_t n0, int bn) {
+  if constexpr (KIND != KIND_BF16) return false;
+  if (p.out_dtype != PML_HIP_BF16 || (p.tail_mode != 1 && p.tail_mode != 2)) return false;
+  if (n0 + bn > p.N || (p.ldc & 7) != 0 || ((uintptr_t)p.C & 15) != 0) return false;
+  if (p.init != nullptr && !(p.init_rs == 0 && p.init_cs == 1 && p.init_dtype == PML_HIP_BF16 && ((uintptr_t)p.init & 15) == 0)) return false;
+  if (p.tail_mode == 2 && ((p.tail.operand_row_stride[0] & 7) != 0 || ((uintptr_t)p.operands[0] & 15) != 0)) return false;
+  return true;
+}
+
+__device__ __forceinline__ void unpack_bf16x8(const i32x4_t& w, float* f) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    f[2 * q] = __uint_as_float((uint32_t)w[q] << 16);
+    f[2 * q + 1] = __uint_as_float((uint32_t)w[q] & 0xffff0000u);
+  }
+}
+
+__device__ __forceinline__ i32x4_t pack_bf16x8(const float* v) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  i32x4_t o;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const bf16x2 h = __builtin_convertvector(f32x2{v[2 * q], v[2 * q + 1]}, bf16x2);  // round to nearest even
+    uint32_t w;
+    __builtin_memcpy(&w, &h, 4);
+    o[q] = (int)w;
+  }
+  return o;
+}
+
+// mw, nw: first row / column of the wavefront's MI x NI blocks.
+template <int MI, int NI>
+__device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&acc)[MI][NI], int64_t mw, int64_t nw, int lane) {
+  const int hi = lane >> 5;
+  const bool residual = p.tail_mode == 2;
+  const int64_t rs = p.tail.operand_row_stride[0];
+  // the last MFMAs must have written the accumulators before the lane exchange below reads them: the compiler
+  // cannot see that read (it is assembler text), so the longest MFMA's passes are waited out here, once
+  asm volatile("s_nop 15\n\ts_nop 3");
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    i32x4_t bias_bits[2];  // kept packed: registers are the scarce thing here
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      bias_bits[q] = p.init != nullptr ? *(const i32x4_t*)((const uint16_t*)p.init + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int64_t m = mw + i * 32 + (lane & 31);
+      const bool row_ok = m < p.M;
+      i32x4_t res[2] = {i32x4_t{0, 0, 0, 0}, i32x4_t{0, 0, 0, 0}};
+      if (residual && row_ok) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) res[q] = *(const i32x4_t*)((const uint16_t*)p.operands[0] + m * rs + nw + j * 32 + 16 * q + 8 * hi);
+      }
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        float v[8], bias[8];
+        unpack_bf16x8(bias_bits[q], bias);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // x: group 2q, y: group 2q + 1; afterwards lanes 0..31 hold group 2q whole, lanes 32..63 group 2q + 1.
+          // (As an instruction on the accumulator registers themselves: the builtin made the compiler copy all
+          // accumulators first, which cost the second workgroup of a CU its registers.)
+          float x = acc[i][j][4 * (2 * q) + e], y = acc[i][j][4 * (2 * q + 1) + e];
+          // (the waits: the compiler does not see through the text, so it cannot insert the idle cycles this
+          // instruction needs after a vector write of its operands and before a vector read of its results)
+          asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+          v[e] = x + bias[e];
+          v[4 + e] = y + bias[4 + e];
+        }
+        if (residual) {
+          // the contraction result is rounded first, then the bf16 addition rounds again
+          float c[8], r[8];
+          unpack_bf16x8(pack_bf16x8(v), c);
+          unpack_bf16x8(res[q], r);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = c[e] + r[e];
+        }
+        if (p.tail_relu) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = v[e] < 0.f ? 0.f : v[e];
+        }
+        if (row_ok) *(i32x4_t*)((uint16_t*)p.C + m * p.ldc + nw + j * 32 + 16 * q + 8 * hi) = pack_bf16x8(v);
       }
     }
   }
