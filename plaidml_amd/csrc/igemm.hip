@@ -87,14 +87,6 @@ __device__ inline void xcd_tile(int bid, int tiles_m, int tiles_n, int* tm, int*
 // STAGES = 0: as many as pay for the tile; 2: two, and LDS rounded up to what staging the whole result
 // tile needs (a short-K, bandwidth-bound GEMM gains more from a second workgroup on the CU than from a
 // third slab in flight)
-template <int I, int N, int STEP, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + STEP, N, STEP>(f);
-  }
-}
-
 template <int BM, int BN, int STAGES = 0, int SLAB = 128>
 struct Ring {
   static constexpr int kStage = (BM + BN) * SLAB;                       // A rows then Bt rows
@@ -284,6 +276,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   // a residual tensor of the tail is requested now, so that it arrives under the K loop
   TailPrefetch<KIND, BM, BN, NT> pre;
   const bool direct = WAVES_K == 1 && direct_tail_ok<KIND>(p, n0, BN);
+
   pre.valid = false;
   if (!direct) tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
 
@@ -439,6 +432,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
     constexpr int kBudget = ring_t::kBytes / kWaves / 16 * 16;  // bytes per wavefront
     constexpr int kFit = kBudget / (32 * CS * 4);
     constexpr int RB = kFit >= MI ? MI : (kFit >= 4 ? 4 : (kFit >= 2 ? 2 : 1));  // MI is a power of two
+    static_assert(kFit >= 1, "one 32-row block of a wavefront's columns must fit its share of LDS");
     static_assert(RB >= 1 && MI % RB == 0, "row blocks must stage evenly");
     accs_t* wtile = (accs_t*)(smem + wave * kBudget);
     // (a compile-time loop: with a run-time row-block number the accumulators would be indexed
@@ -576,8 +570,6 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_128x128_W8_S2: return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
     case TILE_64x64_W8_K2: return launch_cfg<KIND, 64, 64, 2, CONV, 512, 0, 2>(a, s);
     case TILE_256x256_W8: return launch_cfg<KIND, 256, 256, 2, CONV, 512>(a, s);
-    case TILE_256x256_W8T: return launch_cfg<KIND, 256, 256, 4, CONV, 512>(a, s);
-    case TILE_256x256_W4: return launch_cfg<KIND, 256, 256, 2, CONV, 256>(a, s);
   }
   return hipErrorInvalidValue;
 #endif

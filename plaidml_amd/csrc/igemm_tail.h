@@ -8,7 +8,18 @@
 #include "device_common.h"
 #include "plans.h"
 
+#include <type_traits>
+
 namespace pml {
+
+// A loop whose counter is a compile-time constant in the body (accumulator registers can only be named, not indexed).
+template <int I, int N, int STEP, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + STEP, N, STEP>(f);
+  }
+}
 
 template <int KIND>
 struct Acc;

@@ -13,7 +13,7 @@ namespace pml {
 
 enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2 };
 // _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages; _K2: two wavefront grids share the K-blocks of every slab
-enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2, TILE_64x64_W8_K2, TILE_256x256_W8, TILE_256x256_W8T, TILE_256x256_W4 };
+enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2, TILE_64x64_W8_K2, TILE_256x256_W8 };
 
 struct TailPtrs {
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];

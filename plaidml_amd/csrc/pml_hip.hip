@@ -81,8 +81,6 @@ const char* tile_name(int t) {
     case TILE_256x128_W16: return "256x128 (16 wavefronts)";
     case TILE_64x64_W8_K2: return "64x64 (8 wavefronts, K split in two)";
     case TILE_256x256_W8: return "256x256 (8 wavefronts of 128x64)";
-    case TILE_256x256_W8T: return "256x256 (8 wavefronts of 64x128)";
-    case TILE_256x256_W4: return "256x256 (4 wavefronts of 128x128)";
     case TILE_128x128_W8_S2: return "128x128 (8 wavefronts, 2 stages)";
   }
   return "?";
@@ -113,8 +111,8 @@ const char* tile_name(int t) {
 // wavefronts, two to a CU if that still gives every CU a workgroup, one to a CU (three stages) below
 // that; and for small problems the smaller of 64x64 and 128x64 by (rounds of resident workgroups) x
 // (tile area), the larger tile on a tie.
-int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
-  // PML_HIP_TILE=64x64|64x64w8k2|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16 overrides the table (for tuning runs)
+int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, bool plain_tail = true) {
+  // PML_HIP_TILE=64x64|64x64w8k2|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16|256x256w8 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
     const std::string v(e);
     if (v == "64x64") return TILE_64x64;
@@ -126,11 +124,16 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes) {
     if (v == "256x128w16") return TILE_256x128_W16;
     if (v == "64x64w8k2") return TILE_64x64_W8_K2;
     if (v == "256x256w8") return TILE_256x256_W8;
-    if (v == "256x256w8t") return TILE_256x256_W8T;
-    if (v == "256x256w4") return TILE_256x256_W4;
   }
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (n <= 64) return TILE_64x64;  // (the 7x7 stem of ResNet-50 over 2x2 pixel blocks: 191 us against 207 us with 128x64w8)
+  // Long K, at least three quarters of a round of 256x256 tiles and little of them hanging over the edges:
+  // eight wavefronts of 128x64 (0.75 KB of LDS fragment reads per MFMA instead of 1.5).  Measured with N(0,1) /
+  // uniform int8 data, 4096^3: bf16 121 us against 139 (256x128, 16 wavefronts), int8 73 against 84.
+  // (Not under a tail that runs in steps -- requantisation chains: a wavefront stages its 128x64 part through a
+  // 16 KB share of LDS in four rounds, 4096^3 int8 with that tail 132 us against 106 with 256x128.)
+  if (kind != KIND_F32 && plain_tail && k_bytes >= 2048 && tiles(256, 256) >= 192 && tiles(256, 256) * 65536 * 10 <= m * n * 11)
+    return TILE_256x256_W8;
   if (k_bytes >= 4096 && tiles(256, 128) >= 512) return TILE_256x128_W16;
   if (tiles(128, 128) >= 256) return TILE_128x128_W8_S2;
   if (tiles(128, 128) >= 128) return TILE_128x128_W8;
@@ -494,7 +497,11 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   p->kind = PLAN_GEMM;
   p->mfma_kind = kind;
   p->gemm = *d;
-  p->tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype));
+  {
+    int mode = 0, relu = 0;
+    classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
+    p->tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, mode == 1 || mode == 2);
+  }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
   if (!d->b_layout && hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
@@ -584,7 +591,9 @@ int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const voi
     bt = scratch_of_current_device();
     if (!bt) return 1;
   }
-  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype));
+  int mode = 0, relu = 0;
+  classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
+  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, mode == 1 || mode == 2);
   return gemm_run(*d, kind, tile, bt, d->k, false, a, b, c, init, operands, outs, s);
 }
 

@@ -85,6 +85,48 @@ def test_gemm_f32_matches_oracle_contraction():
     np.testing.assert_allclose(run_gemm(Av, Bv, hk.F32, hk.F32), ref, rtol=FP32_RTOL, atol=1e-5)
 
 
+TILE_NAMES = ['64x64', '128x64', '128x128', '128x64w8', '128x128w8', '128x128w8s2', '256x128w16', '64x64w8k2', '256x256w8']
+
+
+@pytest.mark.parametrize('tile', TILE_NAMES)
+def test_every_tile_configuration(tile, monkeypatch):
+    """Every tiling the library holds (selected with the tuning override PML_HIP_TILE), on a problem that is ragged
+    in M, N and K and spans several tiles: int8 bit for bit, bf16 (+ bias + relu, the direct tail where the tile is
+    interior) and fp32 against float64."""
+    monkeypatch.setenv('PML_HIP_TILE', tile)
+    print('tile', tile, flush=True)
+    rng = np.random.default_rng(7)
+    M, N, K = 600, 520, 336
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    np.testing.assert_array_equal(run_gemm(A, B, hk.I8, hk.I32), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.int32))
+    Af = E.round_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    Bf = E.round_bf16(rng.standard_normal((K, N)).astype(np.float32))
+    bias = E.round_bf16(rng.standard_normal(N).astype(np.float32))
+    tail = hk.make_tail(ops=[(hk.EPI_RELU, hk.BF16, 0, 0, 0.0)])
+    C = E.bf16_from_bits(run_gemm(bf16(Af), bf16(Bf), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16, tail=tail))
+    ref = np.maximum(Af.astype(np.float64) @ Bf.astype(np.float64) + bias, 0)
+    np.testing.assert_allclose(C, ref, rtol=BF16_RTOL, atol=BF16_RTOL * np.sqrt(K))
+    A32 = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B32 = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    np.testing.assert_allclose(run_gemm(A32, B32, hk.F32, hk.F32), A32.astype(np.float64) @ B32.astype(np.float64),
+                               rtol=FP32_RTOL, atol=1e-3)
+
+
+def test_gemm_bf16_4096_sampled():
+    """bf16 4096^3 with N(0,1) inputs (the large-tile path): sampled rows and columns against float64."""
+    rng = np.random.default_rng(9)
+    n = 4096
+    A = E.round_bf16(rng.standard_normal((n, n)).astype(np.float32))
+    B = E.round_bf16(rng.standard_normal((n, n)).astype(np.float32))
+    C = E.bf16_from_bits(run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16))
+    rows = rng.choice(n, 16, replace=False)
+    ref = A[rows].astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_allclose(C[rows], ref, rtol=BF16_RTOL, atol=BF16_RTOL * 64)   # results are ~N(0, 64^2)
+    cols = rng.choice(n, 16, replace=False)
+    np.testing.assert_allclose(C[:, cols], A.astype(np.float64) @ B[:, cols].astype(np.float64), rtol=BF16_RTOL, atol=BF16_RTOL * 64)
+
+
 @pytest.mark.parametrize('M,N,K', [(512, 512, 512), (100, 72, 48), (4096, 4096, 4096)])
 def test_gemm_i8_bit_exact(M, N, K):
     rng = np.random.default_rng(4)
