@@ -204,6 +204,18 @@ typedef struct {
   int32_t c_dtype;  /* element type stored to C (type after the tail) */
   int32_t b_layout; /* 0: B is [K][N] with leading dimension ldb; 1: B is [N][K] (K contiguous, ldb >= k) */
   pml_hip_epilogue tail;
+  /* Optional second product summed into the same accumulators before the tail, C = tail(init + init2 + A.B + A2.B2):
+   * what a residual block's projection shortcut and its main path's last 1x1 convolution compute together (the
+   * reference fuses producer and consumer loop nests, pmlc/target/x86/pipeline.cc:304-322; here the two
+   * contractions share one result tile).  k2 = 0: none.  A2 is [M][k2] with leading dimension lda2, or, with
+   * a2_stride > 0, the rows a 1x1 convolution with that stride (no padding) reads from an NHWC image of
+   * a2_h x a2_w pixels of lda2 elements each: row m = (image, oy, ox) of an a2_oh x a2_ow result starts at pixel
+   * (oy * a2_stride, ox * a2_stride).  B2 is [k2][N] (leading dimension ldb2) or [N][k2] like B (b_layout).
+   * init2_kind 1: a second per-column initial value, a contiguous vector of out_dtype.  bf16 GEMMs only. */
+  int64_t k2, lda2, ldb2;
+  int32_t a2_stride;
+  int32_t init2_kind;
+  int64_t a2_h, a2_w, a2_oh, a2_ow;
 } pml_hip_gemm_desc;
 
 int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* desc); /* 0 on failure */
@@ -213,6 +225,11 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
  * reference runs its `init` closure once when the executable is built
  * (pmlc/rt/jit_executable.cc:404-418): after pack_b, invoke may be given b == NULL. */
 int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s);
+/* The same pair for a plan with a second product (k2 > 0): invoke2 also takes its operands, pack_b2 re-lays-out a
+ * constant B2 once (invoke2 may then be given b2 == NULL). */
+int pml_hip_gemm_invoke2(int64_t plan, const void* a, const void* b, void* c, const void* init, const void* a2, const void* b2,
+                         const void* init2, const void* const* operands, void* const* outs, pml_hip_stream s);
+int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s);
 
 /* The GEMM above in one call that allocates nothing, neither on the host heap of the device runtime nor in
  * device memory: dispatch + invoke without a plan object.  It has no counterpart in the reference; it is for

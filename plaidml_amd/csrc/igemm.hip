@@ -159,6 +159,10 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
 
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, (int)kBufRange, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.Bt, 0, (int)kBufRange, kRsrcFlags);
+  // the second product of a two-product GEMM (the first one's operands again when there is none)
+  const bool two = !CONV && p.K2 > 0;
+  const __amdgpu_buffer_rsrc_t ra2 = __builtin_amdgcn_make_buffer_rsrc((void*)(two ? p.A2 : p.A), 0, (int)kBufRange, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t rb2 = __builtin_amdgcn_make_buffer_rsrc((void*)(two ? p.Bt2 : p.Bt), 0, (int)kBufRange, kRsrcFlags);
 
   // ---- per-thread load assignments (fixed across slabs): slot lv of rows lr + kRowsPerPass*i ----
   const int lv = tid % CPR;
@@ -214,9 +218,33 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
     const int64_t n = n0 + lr + kRowsPerPass * i;
     b_off[i] = n < p.N ? (unsigned)(n * p.ldbt * ES) : kOutside;
   }
+  unsigned a2_off[CONV ? 1 : A_VECS], b2_off[CONV ? 1 : B_VECS];
+  if constexpr (!CONV) {
+#pragma unroll
+    for (int i = 0; i < A_VECS; ++i) {
+      const int64_t m = m0 + lr + kRowsPerPass * i;
+      int64_t row = m;
+      if (two && p.g2_stride > 0) {
+        const unsigned mu = (unsigned)(m < p.M ? m : 0);
+        const unsigned nb = fast_div(mu, p.g2_ohw_magic, p.g2_ohw_shift);
+        const unsigned rem = mu - nb * (unsigned)p.g2_ohw;
+        const unsigned oy = fast_div(rem, p.g2_ow_magic, p.g2_ow_shift);
+        const unsigned ox = rem - oy * (unsigned)p.g2_ow;
+        row = ((int64_t)nb * p.g2_h + (int64_t)oy * p.g2_stride) * p.g2_w + (int64_t)ox * p.g2_stride;
+      }
+      a2_off[i] = (two && m < p.M) ? (unsigned)(row * p.lda2 * ES) : kOutside;
+    }
+#pragma unroll
+    for (int i = 0; i < B_VECS; ++i) {
+      const int64_t n = n0 + lr + kRowsPerPass * i;
+      b2_off[i] = (two && n < p.N) ? (unsigned)(n * p.ldbt2 * ES) : kOutside;
+    }
+  }
 
   const int slabs_per_tap = pinned((kbytes_row + kSlabBytes - 1) / kSlabBytes);
-  const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : slabs_per_tap;
+  const int k2_bytes = pinned(two ? (int)(p.K2 * ES) : 0);
+  const int first_bytes = slabs_per_tap * kSlabBytes;  // where the second product's slabs begin on the slab axis
+  const int n_slabs = CONV ? p.KH * p.KW * slabs_per_tap : slabs_per_tap + (k2_bytes + kSlabBytes - 1) / kSlabBytes;
 
   // Requests of the next slab into ring stage `stage`, one 16-byte-per-lane load at a time (index l: the A
   // rows first, then the Bt rows) so that they can be spread between the MFMAs.  Slabs are prepared in order,
@@ -227,6 +255,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   unsigned req_a = 0, req_b = 0;  // slab-dependent part of the A / Bt offsets
   int req_dh = 0, req_dw = 0;     // CONV: the tap's displacement in input rows / columns (columns: plus the chunk's pixel)
   bool req_ok = false;
+  bool req_second = false;        // GEMM: the slab belongs to the second product
   int nx_kh = 0, nx_kw = 0, nx_cs = 0, nx_dh = 0, nx_dw = 0, nx_tap = 0;  // CONV: tap and slab-in-tap of the next slab
   int nx_kbo = 0;                                                          // GEMM: its first byte of K
   auto prepare_slab = [&](int stage) {
@@ -251,8 +280,9 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
         }
       }
     } else {
-      const int kbo = nx_kbo + lc * 16;
-      req_a = req_b = kbo < kbytes_row ? (unsigned)kbo : kOutside;
+      req_second = nx_kbo >= first_bytes;
+      const int kbo = (req_second ? nx_kbo - first_bytes : nx_kbo) + lc * 16;
+      req_a = req_b = kbo < (req_second ? k2_bytes : kbytes_row) ? (unsigned)kbo : kOutside;
       nx_kbo += kSlabBytes;
     }
   };
@@ -262,14 +292,20 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       if (CONV) {
         const bool ok = req_ok & ((unsigned)(a_ih0[l] + req_dh) < (unsigned)cH) & ((unsigned)(a_iw0[l] + req_dw) < (unsigned)cW);
         off = ok ? a_off[l] + req_a : kOutside;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, PML_LDS(req_base + l * kRowsPerPass * kSlabBytes), 16, (int)off, 0, 0, 0);
       } else {
-        off = join_offsets(a_off[l], req_a);
+        off = join_offsets(req_second ? a2_off[l] : a_off[l], req_a);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(req_second ? ra2 : ra, PML_LDS(req_base + l * kRowsPerPass * kSlabBytes), 16, (int)off, 0, 0, 0);
       }
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, PML_LDS(req_base + l * kRowsPerPass * kSlabBytes), 16, (int)off, 0, 0, 0);
     } else {
       const int i = l - A_VECS;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16,
-                                               (int)join_offsets(b_off[i], req_b), 0, 0, 0);
+      if (CONV) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16,
+                                                 (int)join_offsets(b_off[i], req_b), 0, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(req_second ? rb2 : rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16,
+                                                 (int)join_offsets(req_second ? b2_off[i] : b_off[i], req_b), 0, 0, 0);
+      }
     }
   };
 

@@ -121,6 +121,7 @@ __device__ __forceinline__ bool direct_tail_ok(const IgemmArgs& p, int64_t n0, i
   if (n0 + bn > p.N || (p.ldc & 7) != 0 || ((uintptr_t)p.C & 15) != 0) return false;
   if (p.init != nullptr && !(p.init_rs == 0 && p.init_cs == 1 && p.init_dtype == PML_HIP_BF16 && ((uintptr_t)p.init & 15) == 0)) return false;
   if (p.tail_mode == 2 && ((p.tail.operand_row_stride[0] & 7) != 0 || ((uintptr_t)p.operands[0] & 15) != 0)) return false;
+  if (p.init2 != nullptr && ((uintptr_t)p.init2 & 15) != 0) return false;
   return true;
 }
 
@@ -161,6 +162,10 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
 #pragma unroll
     for (int q = 0; q < 2; ++q)
       bias_bits[q] = p.init != nullptr ? *(const i32x4_t*)((const uint16_t*)p.init + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+    i32x4_t bias2_bits[2];  // the second product's bias (zeros when there is none)
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      bias2_bits[q] = p.init2 != nullptr ? *(const i32x4_t*)((const uint16_t*)p.init2 + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int64_t m = mw + i * 32 + (lane & 31);
@@ -172,8 +177,11 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
       }
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        float v[8], bias[8];
+        float v[8], bias[8], bias2[8];
         unpack_bf16x8(bias_bits[q], bias);
+        unpack_bf16x8(bias2_bits[q], bias2);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bias[e] += bias2[e];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           // x: group 2q, y: group 2q + 1; afterwards lanes 0..31 hold group 2q whole, lanes 32..63 group 2q + 1.
@@ -255,6 +263,16 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
           Scalar<float, int> b = load_scalar<float, int>(p.init, (n + q) * p.init_cs, p.init_dtype);
           cinit[q] = KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
         }
+      }
+    }
+  }
+  // the per-column start value of a second product (a contiguous vector of the result type)
+  if (p.init2 != nullptr) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (n + q < p.N) {
+        Scalar<float, int> b = load_scalar<float, int>(p.init2, n + q, KIND == KIND_I8 ? PML_HIP_I32 : p.out_dtype);
+        cinit[q] += KIND == KIND_I8 ? (accs_t)b.i : (accs_t)b.f;
       }
     }
   }
@@ -601,10 +619,11 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
     accs_t v4[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) v4[q] = ctile[row * CS + c4 + q];
-    if (col_init) {
+    if (col_init || p.init2 != nullptr) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) v4[q] += cinit[q];
-    } else if (p.init) {
+    }
+    if (p.init && !col_init) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         if (n + q < p.N) {

@@ -67,6 +67,17 @@ struct IgemmArgs {
   pml_hip_epilogue tail;
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
   void* outs[PML_HIP_MAX_EPI_OPERANDS];
+  // A second product summed into the same result, C = A . Bt^T + A2 . Bt2^T (GEMM instantiations only; K2 = 0: none).
+  // Row m of A2 starts at element lda2 * m, or, with g2_stride > 0, at the pixel the output pixel m reads in an
+  // NHWC image walked with that stride (a 1x1 convolution): ((n * g2_h + oy * stride) * g2_w + ox * stride) * lda2
+  // with n, oy, ox from m by g2_ohw / g2_ow.  init2: a second per-column initial value of the result type or null.
+  const void* A2;
+  const void* Bt2;
+  const void* init2;
+  int64_t K2, lda2, ldbt2;
+  int g2_stride, g2_h, g2_w, g2_ohw, g2_ow;
+  unsigned g2_ohw_magic, g2_ow_magic;
+  int g2_ohw_shift, g2_ow_shift;
 };
 
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);

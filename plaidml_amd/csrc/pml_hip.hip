@@ -44,6 +44,9 @@ struct Plan {
   int64_t bt_ld = 0;
   size_t bt_bytes = 0;
   bool packed = false;
+  // second product of a GEMM: its packed right-hand side Bt2[N][K2]
+  void* bt2 = nullptr;
+  bool packed2 = false;
   // convolution whose channels do not fill 16-byte vectors: patch matrix [M][kpad] + GEMM
   void* patches = nullptr;
   int64_t kpad = 0;
@@ -57,6 +60,7 @@ struct Plan {
   std::string text;
   ~Plan() {
     if (bt) (void)hipFree(bt);
+    if (bt2) (void)hipFree(bt2);
     if (patches) (void)hipFree(patches);
     if (s2d) (void)hipFree(s2d);
   }
@@ -486,6 +490,25 @@ static int gemm_desc_kind(const pml_hip_gemm_desc* d) {
     fail("gemm: malformed tail");
     return -1;
   }
+  if (d->k2 != 0) {
+    if (kind != KIND_BF16 || d->k2 < 0 || (d->k2 * es) % 16 != 0 || (d->lda2 * es) % 16 != 0 || d->lda2 < d->k2 ||
+        d->ldb2 < (d->b_layout ? d->k2 : d->n) || (d->b_layout && (d->ldb2 * es) % 16 != 0) || d->a2_stride < 0 ||
+        (d->init2_kind != 0 && d->init2_kind != 1)) {
+      fail("gemm: malformed second product (bf16 only; k2 and lda2 must cover whole 16-byte vectors)");
+      return -1;
+    }
+    if (d->a2_stride > 0) {
+      // rows of a strided 1x1 convolution: the result rows are the pixels of whole images
+      if (d->a2_oh <= 0 || d->a2_ow <= 0 || d->m % (d->a2_oh * d->a2_ow) != 0 || (d->a2_oh - 1) * d->a2_stride >= d->a2_h ||
+          (d->a2_ow - 1) * d->a2_stride >= d->a2_w || d->a2_oh * d->a2_ow > INT32_MAX || d->a2_h > INT32_MAX || d->a2_w > INT32_MAX) {
+        fail("gemm: the second product's pixel rows do not fit its image");
+        return -1;
+      }
+    }
+  } else if (d->init2_kind != 0) {
+    fail("gemm: a second initial value needs a second product");
+    return -1;
+  }
   return kind;
 }
 
@@ -500,7 +523,7 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   {
     int mode = 0, relu = 0;
     classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
-    p->tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, mode == 1 || mode == 2);
+    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, mode == 1 || mode == 2);
   }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
@@ -509,20 +532,34 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
     fail("gemm: cannot allocate the packed right-hand side");
     return 0;
   }
+  if (d->k2 > 0 && !d->b_layout && hipMalloc(&p->bt2, (size_t)d->n * d->k2 * es) != hipSuccess) {
+    delete p;
+    fail("gemm: cannot allocate the second packed right-hand side");
+    return 0;
+  }
   char buf[256];
   std::snprintf(buf, sizeof buf, "gemm %s m=%lld n=%lld k=%lld tile=%s mfma=%s", d->in_dtype == PML_HIP_F32 ? "f32" : d->in_dtype == PML_HIP_BF16 ? "bf16" : "i8",
                 (long long)d->m, (long long)d->n, (long long)d->k, tile_name(p->tile),
                 kind == KIND_F32 ? "f32_32x32x2" : kind == KIND_BF16 ? "f32_32x32x16_bf16" : "i32_32x32x32_i8");
   p->text = buf;
+  if (d->k2 > 0) p->text += " + second product k2=" + std::to_string(d->k2) + (d->a2_stride > 0 ? " over pixel rows of stride " + std::to_string(d->a2_stride) : "");
   return (int64_t)(intptr_t)p;
 }
 
 // One GEMM launch sequence: the per-run transposition of a [K][N] right-hand side into `bt` (device memory of
 // n x bt_ld elements; skipped when b is null, i.e. packed earlier, or already [N][K]), then the MFMA kernel.
 // Shared by the plan-based entry point and by the one that allocates nothing.
+struct SecondProduct {
+  const void* a2 = nullptr;
+  const void* b2 = nullptr;
+  const void* init2 = nullptr;
+  void* bt2 = nullptr;
+  bool packed2 = false;
+};
+
 static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* bt, int64_t bt_ld, bool packed,
                     const void* a, const void* b, void* c, const void* init, const void* const* operands,
-                    void* const* outs, pml_hip_stream s) {
+                    void* const* outs, pml_hip_stream s, const SecondProduct* second = nullptr) {
   if (!a || !c) return fail("gemm_invoke: null operand");
   if (!b && (!packed || d.b_layout)) return fail("gemm_invoke: b is null and no packed right-hand side exists");
   if (d.b_layout && ((uintptr_t)b & 15) != 0) return fail("gemm_invoke: an [N][K] right-hand side must be 16-byte aligned");
@@ -531,8 +568,34 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   const int es = dt_size(d.in_dtype);
   if (b && !d.b_layout && check(transpose_pack(es, b, bt, d.k, d.n, d.ldb, bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
+  if (d.k2 > 0) {
+    if (!second || !second->a2) return fail("gemm_invoke: the plan has a second product: use pml_hip_gemm_invoke2");
+    if (!second->b2 && (!second->packed2 || d.b_layout)) return fail("gemm_invoke2: b2 is null and no packed right-hand side exists");
+    if (((uintptr_t)second->a2 & 15) != 0 || (d.b_layout && ((uintptr_t)second->b2 & 15) != 0)) return fail("gemm_invoke2: the second product's operands must be 16-byte aligned");
+    if (d.init2_kind && !second->init2) return fail("gemm_invoke2: the plan expects a second initial value");
+    if (second->b2 && !d.b_layout &&
+        check(transpose_pack(es, second->b2, second->bt2, d.k2, d.n, d.ldb2, d.k2, (hipStream_t)s), "transpose_pack"))
+      return 1;
+  }
   IgemmArgs g;
   std::memset(&g, 0, sizeof g);
+  if (d.k2 > 0) {
+    g.K2 = d.k2;
+    g.A2 = second->a2;
+    g.lda2 = d.lda2;
+    g.Bt2 = d.b_layout ? second->b2 : second->bt2;
+    g.ldbt2 = d.b_layout ? d.ldb2 : d.k2;
+    g.init2 = d.init2_kind ? second->init2 : nullptr;
+    g.g2_stride = d.a2_stride;
+    if (d.a2_stride > 0) {
+      g.g2_h = (int)d.a2_h;
+      g.g2_w = (int)d.a2_w;
+      g.g2_ohw = (int)(d.a2_oh * d.a2_ow);
+      g.g2_ow = (int)d.a2_ow;
+      fast_div_magic((unsigned)g.g2_ohw, &g.g2_ohw_magic, &g.g2_ohw_shift);
+      fast_div_magic((unsigned)g.g2_ow, &g.g2_ow_magic, &g.g2_ow_shift);
+    }
+  }
   g.M = d.m;
   g.N = d.n;
   g.K = d.k;
@@ -577,10 +640,25 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s);
 }
 
+int pml_hip_gemm_invoke2(int64_t plan, const void* a, const void* b, void* c, const void* init, const void* a2, const void* b2,
+                         const void* init2, const void* const* operands, void* const* outs, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke2: not a gemm plan");
+  if (p->gemm.k2 <= 0) return fail("gemm_invoke2: the plan has no second product");
+  SecondProduct sp;
+  sp.a2 = a2;
+  sp.b2 = b2;
+  sp.init2 = init2;
+  sp.bt2 = p->bt2;
+  sp.packed2 = p->packed2;
+  return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s, &sp);
+}
+
 int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const void* b, void* c, const void* init,
                             const void* const* operands, void* const* outs, pml_hip_stream s) {
   const int kind = gemm_desc_kind(d);
   if (kind < 0) return 1;
+  if (d->k2 != 0) return fail("gemm_run_static: a second product is not supported by this entry point");
   if (!b) return fail("gemm_run_static: b is null");
   void* bt = nullptr;
   if (!d->b_layout) {
@@ -790,6 +868,16 @@ int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s) {
   if (check(transpose_pack(dt_size(d.in_dtype), b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   p->packed = true;
+  return 0;
+}
+
+int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_GEMM || !b2 || p->gemm.k2 <= 0) return fail("gemm_pack_b2: bad argument");
+  const pml_hip_gemm_desc& d = p->gemm;
+  if (d.b_layout) return fail("gemm_pack_b2: an [N][K] right-hand side needs no packing");
+  if (check(transpose_pack(dt_size(d.in_dtype), b2, p->bt2, d.k2, d.n, d.ldb2, d.k2, (hipStream_t)s), "transpose_pack")) return 1;
+  p->packed2 = true;
   return 0;
 }
 

@@ -28,7 +28,7 @@ EXPORTS = [
     'pml_hip_memcpy_d2d', 'pml_hip_fill_u32', 'pml_hip_stream_create', 'pml_hip_stream_destroy',
     'pml_hip_stream_sync', 'pml_hip_event_create', 'pml_hip_event_destroy', 'pml_hip_event_record',
     'pml_hip_event_sync', 'pml_hip_event_elapsed_ms', 'pml_hip_gemm_dispatch', 'pml_hip_gemm_invoke',
-    'pml_hip_gemm_run_static',
+    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2',
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
@@ -52,7 +52,9 @@ class Epilogue(ctypes.Structure):
 class GemmDesc(ctypes.Structure):
     _fields_ = [('in_dtype', i32), ('out_dtype', i32), ('m', i64), ('n', i64), ('k', i64), ('lda', i64), ('ldb', i64),
                 ('ldc', i64), ('init_kind', i32), ('init_dtype', i32), ('init_row_stride', i64),
-                ('init_col_stride', i64), ('c_dtype', i32), ('b_layout', i32), ('tail', Epilogue)]
+                ('init_col_stride', i64), ('c_dtype', i32), ('b_layout', i32), ('tail', Epilogue),
+                ('k2', i64), ('lda2', i64), ('ldb2', i64), ('a2_stride', i32), ('init2_kind', i32),
+                ('a2_h', i64), ('a2_w', i64), ('a2_oh', i64), ('a2_ow', i64)]
 
 
 class Conv2dDesc(ctypes.Structure):
@@ -147,6 +149,8 @@ def lib():
         pp = ctypes.POINTER(vp)
         L.pml_hip_gemm_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp, pp, pp, vp]
         L.pml_hip_gemm_run_static.argtypes = [ctypes.POINTER(GemmDesc), vp, vp, vp, vp, pp, pp, vp]
+        L.pml_hip_gemm_invoke2.argtypes = [ctypes.c_int64, vp, vp, vp, vp, vp, vp, vp, pp, pp, vp]
+        L.pml_hip_gemm_pack_b2.argtypes = [ctypes.c_int64, vp, vp]
         L.pml_hip_conv2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp, pp, pp, vp]
         L.pml_hip_dwconv2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, pp, pp, vp]
         L.pml_hip_pool2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp]

@@ -186,8 +186,146 @@ class Planner {
       s.text = "copy -> output #" + std::to_string(c.first);
       plan_->steps.push_back(s);
     }
+    if (opt_.fuse && opt_.specialise) fuseSecondProducts();
     pruneDeadSteps();
     return plan_;
+  }
+
+  // Two matrix products that are added -- a residual block's projection shortcut and the last 1x1 convolution
+  // of its main path -- become one launch that accumulates both into the same result tile: the sum is never
+  // written and read back (the reference reaches the same by fusing the loop nests of producer and consumer,
+  // pmlc/target/x86/pipeline.cc:304-322).  Works on finished steps: Y = gemm / 1x1 convolution whose tail starts
+  // with "+ result of X", X = earlier gemm / 1x1 convolution without a tail whose result nobody else reads.
+  void fuseSecondProducts() {
+    auto pointwise = [](const Step& s) {
+      const pml_hip_conv2d_desc& c = s.conv;
+      return s.kind == Step::Conv2d && c.kh == 1 && c.kw == 1 && c.pad_h == 0 && c.pad_w == 0 && c.dil_h == 1 && c.dil_w == 1 &&
+             c.stride_h == c.stride_w && c.in_dtype == PML_HIP_BF16 && c.out_dtype == PML_HIP_BF16;
+    };
+    auto plainGemm = [](const Step& s) {
+      return s.kind == Step::Gemm && s.gemm.k2 == 0 && s.gemm.in_dtype == PML_HIP_BF16 && s.gemm.out_dtype == PML_HIP_BF16 &&
+             s.gemm.ldc == s.gemm.n && s.c_off == 0;
+    };
+    auto columnInit = [](int32_t kind, int32_t dtype, int64_t rs, int64_t cs) {
+      return kind == 0 || (kind == 1 && dtype == PML_HIP_BF16 && rs == 0 && cs == 1);
+    };
+    for (size_t y = 0; y < plan_->steps.size(); ++y) {
+      Step& Y = plan_->steps[y];
+      if (!plainGemm(Y) && !pointwise(Y)) continue;
+      const pml_hip_epilogue& ty = Y.kind == Step::Gemm ? Y.gemm.tail : Y.conv.tail;
+      if (ty.n_ops < 1 || ty.ops[0].opcode != PML_HIP_EPI_ADD || ty.ops[0].operand_kind != PML_HIP_OPND_TENSOR ||
+          ty.ops[0].dtype != PML_HIP_BF16)
+        continue;
+      const int q = ty.ops[0].operand;
+      const int64_t n_cols = Y.kind == Step::Gemm ? Y.gemm.n : Y.conv.co;
+      if (q < 0 || q >= ty.n_operands || ty.operand_dtype[q] != PML_HIP_BF16 || ty.operand_col_stride[q] != 1 ||
+          ty.operand_row_stride[q] != n_cols || static_cast<size_t>(q) >= Y.operands.size() || Y.operand_off[q] != 0)
+        continue;
+      bool reused = false;  // the operand must not be used again further down the tail
+      for (int k = 1; k < ty.n_ops; ++k) reused = reused || (ty.ops[k].operand_kind == PML_HIP_OPND_TENSOR && ty.ops[k].operand == q);
+      if (reused) continue;
+      const int xbuf = Y.operands[q];
+      if (plan_->buffers[xbuf].kind != BufferInfo::Temp) continue;
+      // X: the last earlier writer of that buffer; readers: only Y's tail
+      int x = -1;
+      for (size_t k = 0; k < y; ++k)
+        if (plan_->steps[k].c == xbuf) x = static_cast<int>(k);
+      if (x < 0) continue;
+      int readers = 0;
+      for (const Step& s : plan_->steps) {
+        for (int r : {s.a, s.b, s.init, s.a2, s.b2, s.init2}) readers += r == xbuf;
+        for (int r : s.operands) readers += r == xbuf;
+      }
+      if (readers != 1) continue;
+      const Step& X = plan_->steps[x];
+      if (!plainGemm(X) && !pointwise(X)) continue;
+      const pml_hip_epilogue& tx = X.kind == Step::Gemm ? X.gemm.tail : X.conv.tail;
+      if (tx.n_ops != 0 || !X.outs.empty()) continue;
+      // one of the two must be a plain GEMM (the kernel's first product walks plain rows)
+      const Step& P = plainGemm(Y) ? Y : X;   // first product
+      const Step& S = plainGemm(Y) ? X : Y;   // second product
+      if (!plainGemm(P) || &P == &S) continue;
+      if (P.gemm.b_layout != 0 || P.b_is_nk) continue;
+      const pml_hip_gemm_desc& pg = P.gemm;
+      Step F = P;
+      pml_hip_gemm_desc& g = F.gemm;
+      if (S.kind == Step::Gemm) {
+        const pml_hip_gemm_desc& sg = S.gemm;
+        if (sg.m != pg.m || sg.n != pg.n || sg.b_layout != 0 || S.b_is_nk) continue;
+        if (!columnInit(sg.init_kind, sg.init_dtype, sg.init_row_stride, sg.init_col_stride) || S.init_off != 0) continue;
+        g.k2 = sg.k;
+        g.lda2 = sg.lda;
+        g.ldb2 = sg.ldb;
+        g.a2_stride = 0;
+        g.init2_kind = sg.init_kind;
+      } else {
+        const pml_hip_conv2d_desc& sc = S.conv;
+        if (sc.n * sc.oh * sc.ow != pg.m || sc.co != pg.n) continue;
+        if (!columnInit(sc.init_kind, sc.init_dtype, sc.init_row_stride, sc.init_col_stride) || S.init_off != 0) continue;
+        g.k2 = sc.ci;
+        g.lda2 = sc.ci;
+        g.ldb2 = sc.co;
+        const bool plain_rows = sc.stride_h == 1 && sc.oh == sc.h && sc.ow == sc.w;
+        g.a2_stride = plain_rows ? 0 : static_cast<int32_t>(sc.stride_h);
+        g.a2_h = sc.h;
+        g.a2_w = sc.w;
+        g.a2_oh = sc.oh;
+        g.a2_ow = sc.ow;
+        g.init2_kind = sc.init_kind;
+      }
+      if ((g.k2 * 2) % 16 != 0 || (g.lda2 * 2) % 16 != 0) continue;
+      if (!columnInit(pg.init_kind, pg.init_dtype, pg.init_row_stride, pg.init_col_stride)) continue;
+      // the tail is Y's without its first step; operand q goes, later operands move down
+      pml_hip_epilogue t{};
+      t.n_ops = ty.n_ops - 1;
+      for (int k = 1; k < ty.n_ops; ++k) {
+        t.ops[k - 1] = ty.ops[k];
+        if (t.ops[k - 1].operand_kind == PML_HIP_OPND_TENSOR && t.ops[k - 1].operand > q) t.ops[k - 1].operand -= 1;
+      }
+      t.n_operands = ty.n_operands - 1;
+      for (int k = 0, w = 0; k < ty.n_operands; ++k) {
+        if (k == q) continue;
+        t.operand_dtype[w] = ty.operand_dtype[k];
+        t.operand_row_stride[w] = ty.operand_row_stride[k];
+        t.operand_col_stride[w] = ty.operand_col_stride[k];
+        ++w;
+      }
+      g.tail = t;
+      g.c_dtype = Y.kind == Step::Gemm ? Y.gemm.c_dtype : Y.conv.c_dtype;
+      F.c = Y.c;
+      F.c_off = 0;
+      F.operands.clear();
+      F.operand_off.clear();
+      for (size_t k = 0; k < Y.operands.size(); ++k) {
+        if (static_cast<int>(k) == q) continue;
+        F.operands.push_back(Y.operands[k]);
+        F.operand_off.push_back(k < Y.operand_off.size() ? Y.operand_off[k] : 0);
+      }
+      F.outs = Y.outs;
+      F.out2 = Y.out2;
+      F.a2 = S.a;
+      F.b2 = S.b;
+      F.init2 = S.init;
+      F.a2_off = S.a_off;
+      F.b2_off = S.b_off;
+      F.b2_constant = S.b_constant;
+      F.flops = X.flops + Y.flops;
+      F.bytes = X.bytes + Y.bytes - 2.0 * static_cast<double>(pg.m * pg.n) * 2;  // the sum is neither written nor read
+      {
+        TailBuild shown;
+        shown.tail = t;
+        std::stringstream ss;
+        ss << "gemm bf16 m=" << g.m << " n=" << g.n << " k=" << g.k << " + second product k2=" << g.k2;
+        if (S.kind == Step::Conv2d) ss << " (pixel rows of a 1x1 convolution, stride " << S.conv.stride_h << ")";
+        ss << " B=[k][n]" << ((F.b_constant && F.b2_constant) ? " (constants, packed once)" : "") << (g.init_kind ? " +init" : "")
+           << (g.init2_kind ? " +init2" : "") << tailText(shown);
+        const std::string& ytext = Y.text;
+        const size_t arrow = ytext.rfind(" -> ");
+        ss << (arrow == std::string::npos ? "" : ytext.substr(arrow));
+        F.text = ss.str();
+      }
+      plan_->steps[y] = F;  // X is left without readers and is dropped by pruneDeadSteps
+    }
   }
 
   // A kernel that took over the work of earlier operations (the int8 GEMM reads the un-cast operands, a pool
@@ -208,7 +346,7 @@ class Planner {
       const bool accumulates = s.kind == Step::Contract && s.con.has_init;
       if (!accumulates)
         for (int w : writes) needed.erase(w);
-      for (int r : {s.a, s.b, s.init}) {
+      for (int r : {s.a, s.b, s.init, s.a2, s.b2, s.init2}) {
         if (r >= 0) needed.insert(r);
       }
       for (int r : s.operands) needed.insert(r);

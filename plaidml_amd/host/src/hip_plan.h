@@ -46,6 +46,10 @@ struct Step {
   // buffer ids (-1 = none) and element offsets applied to the base pointers
   int a = -1, b = -1, c = -1, init = -1, out2 = -1;
   int64_t a_off = 0, b_off = 0, c_off = 0, init_off = 0;
+  // Gemm with a second product (gemm.k2 > 0): its left- and right-hand side and per-column initial value
+  int a2 = -1, b2 = -1, init2 = -1;
+  int64_t a2_off = 0, b2_off = 0;
+  bool b2_constant = false;
   std::vector<int> operands;       // tail operands / contraction sources / select inputs
   std::vector<int64_t> operand_off;
   std::vector<int> outs;           // extra outputs of STORE steps (index = STORE's operand field)

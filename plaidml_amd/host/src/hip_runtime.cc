@@ -165,7 +165,7 @@ class HipExecutable final : public Executable {
     };
     for (size_t i = 0; i < ns; ++i) {
       const Step& s = plan_->steps[i];
-      for (int b : {s.a, s.b, s.c, s.init, s.out2}) touch(b, i);
+      for (int b : {s.a, s.b, s.c, s.init, s.out2, s.a2, s.b2, s.init2}) touch(b, i);
       for (int b : s.operands) touch(b, i);
       for (int b : s.outs) touch(b, i);
     }
@@ -175,6 +175,7 @@ class HipExecutable final : public Executable {
     std::vector<std::vector<int>> starts(ns + 1), ends(ns + 1);
     for (size_t b = 0; b < nb; ++b) {
       if (plan_->buffers[b].kind != BufferInfo::Temp) continue;
+      if (first[b] < 0) continue;  // a value no launch touches (its producer was fused away) takes no memory
       unshared_temp_bytes_ += padded(plan_->buffers[b].bytes);
       const size_t f = first[b] < 0 ? 0 : static_cast<size_t>(first[b]);
       const size_t l = last[b] < 0 ? 0 : static_cast<size_t>(last[b]);
@@ -272,6 +273,8 @@ class HipExecutable final : public Executable {
     // constant right-hand sides are re-laid-out once, here
     if (s.kind == Step::Gemm && s.b_constant && !s.b_is_nk)
       hipCheck(pml_hip_gemm_pack_b(h, ptr(s.b, s.b_off, elemSize(s.gemm.in_dtype)), nullptr), "pack_b");
+    if (s.kind == Step::Gemm && s.gemm.k2 > 0 && s.b2_constant && !s.b_is_nk)
+      hipCheck(pml_hip_gemm_pack_b2(h, ptr(s.b2, s.b2_off, elemSize(s.gemm.in_dtype)), nullptr), "pack_b2");
     if (s.kind == Step::Conv2d && s.b_constant) hipCheck(pml_hip_conv2d_pack_filter(h, ptr(s.b), nullptr), "pack_filter");
   }
 
@@ -286,6 +289,14 @@ class HipExecutable final : public Executable {
         const size_t es = elemSize(s.gemm.in_dtype);
         const void* b = ptr(s.b, s.b_off, es);
         if (s.b_constant && !s.b_is_nk) b = nullptr;  // packed when the executable was built
+        if (s.gemm.k2 > 0) {
+          const void* b2 = ptr(s.b2, s.b2_off, es);
+          if (s.b2_constant && !s.b_is_nk) b2 = nullptr;
+          hipCheck(pml_hip_gemm_invoke2(handles_[i], ptr(s.a, s.a_off, es), b, ptr(s.c, s.c_off, elemSize(s.gemm.c_dtype)), ptr(s.init),
+                                        ptr(s.a2, s.a2_off, es), b2, ptr(s.init2), operands, outs, nullptr),
+                   s.text.c_str());
+          break;
+        }
         hipCheck(pml_hip_gemm_invoke(handles_[i], ptr(s.a, s.a_off, es), b, ptr(s.c, s.c_off, elemSize(s.gemm.c_dtype)),
                                      ptr(s.init), operands, outs, nullptr),
                  s.text.c_str());

@@ -46,6 +46,17 @@ def test_plan_choices_for_the_workload_configs():
     assert t.count('conv2d bf16') + t.count('gemm bf16') == 2 and 'constant' in t and 'add(t' in t, t
 
 
+def test_projection_shortcut_and_main_path_share_one_launch():
+    """relu(conv1x1(y) + b + conv1x1(x) + b') of a residual block with a projection shortcut is one GEMM with two
+    products (plain rows, or the pixel rows of the stride-2 shortcut); `fuse=0` keeps the contractions apart."""
+    prog = programs.resnet50_tiny(E, op)[0]
+    t = plan_of(prog)
+    assert t.count('+ second product') == 4 and t.count('pixel rows of a 1x1 convolution, stride 2') == 2, t
+    assert '+init +init2 tail=[relu]' in t
+    prog = programs.resnet50_tiny(E, op)[0]
+    assert 'second product' not in plan_of(prog, 'hip{fuse=0}')
+
+
 def test_target_options_switch_specialisation_off():
     prog = programs.config1_conv(E, op, 'BFLOAT16')[0]
     t = plan_of(prog, 'hip{specialise=0,fuse=0}')

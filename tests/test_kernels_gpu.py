@@ -113,6 +113,52 @@ def test_every_tile_configuration(tile, monkeypatch):
                                rtol=FP32_RTOL, atol=1e-3)
 
 
+@pytest.mark.parametrize('stride', [0, 2])
+def test_gemm_two_products(stride):
+    """C = relu(A.B + b + A2.B2 + b2) in one launch: the second left-hand side as plain rows, and as the pixel rows a
+    1x1 convolution with stride 2 reads from an NHWC image (a residual block's projection shortcut)."""
+    rng = np.random.default_rng(21)
+    NB, OH, OW, K1, K2, N = 3, 7, 9, 72, 40, 136
+    M = NB * OH * OW
+    A = E.round_bf16(rng.standard_normal((M, K1)).astype(np.float32))
+    B = E.round_bf16(rng.standard_normal((K1, N)).astype(np.float32) * 0.2)
+    B2 = E.round_bf16(rng.standard_normal((K2, N)).astype(np.float32) * 0.2)
+    b1 = E.round_bf16(rng.standard_normal(N).astype(np.float32))
+    b2 = E.round_bf16(rng.standard_normal(N).astype(np.float32))
+    if stride:
+        H2, W2 = (OH - 1) * stride + 2, (OW - 1) * stride + 1
+        img = E.round_bf16(rng.standard_normal((NB, H2, W2, K2)).astype(np.float32))
+        A2 = img[:, :(OH - 1) * stride + 1:stride, :(OW - 1) * stride + 1:stride].reshape(M, K2)
+        a2_dev = img
+    else:
+        A2 = E.round_bf16(rng.standard_normal((M, K2)).astype(np.float32))
+        a2_dev = A2
+    d = hk.GemmDesc()
+    d.in_dtype = d.out_dtype = d.c_dtype = hk.BF16
+    d.m, d.n, d.k, d.lda, d.ldb, d.ldc = M, N, K1, K1, N, N
+    d.init_kind, d.init_dtype, d.init_row_stride, d.init_col_stride = 1, hk.BF16, 0, 1
+    d.tail = hk.make_tail(ops=[(hk.EPI_RELU, hk.BF16, 0, 0, 0.0)])
+    d.k2, d.lda2, d.ldb2, d.init2_kind = K2, K2, N, 1
+    if stride:
+        d.a2_stride, d.a2_h, d.a2_w, d.a2_oh, d.a2_ow = stride, H2, W2, OH, OW
+    L = hk.lib()
+    plan = L.pml_hip_gemm_dispatch(ctypes.byref(d))
+    assert plan, L.pml_hip_last_error()
+    print('plan:', hk.describe(plan), flush=True)
+    bufs = [hk.DeviceBuffer.from_numpy(bf16(x)) for x in (A, B, b1, a2_dev, B2, b2)]
+    dC = hk.DeviceBuffer(M * N * 2)
+    none = hk.ptr_array([])
+    # the plain entry point refuses a plan with a second product
+    assert L.pml_hip_gemm_invoke(plan, bufs[0].ptr, bufs[1].ptr, dC.ptr, bufs[2].ptr, none, none, None) != 0
+    hk.check(L.pml_hip_gemm_pack_b2(plan, bufs[4].ptr, None))
+    hk.check(L.pml_hip_gemm_invoke2(plan, bufs[0].ptr, bufs[1].ptr, dC.ptr, bufs[2].ptr, bufs[3].ptr, None, bufs[5].ptr, none, none, None))
+    hk.check(L.pml_hip_stream_sync(None))
+    C = E.bf16_from_bits(dC.to_numpy(np.uint16, (M, N)))
+    ref = np.maximum(A.astype(np.float64) @ B + A2.astype(np.float64) @ B2 + b1 + b2, 0)
+    np.testing.assert_allclose(C, ref, rtol=BF16_RTOL, atol=BF16_RTOL)
+    L.pml_hip_plan_free(plan)
+
+
 def test_gemm_bf16_4096_sampled():
     """bf16 4096^3 with N(0,1) inputs (the large-tile path): sampled rows and columns against float64."""
     rng = np.random.default_rng(9)
