@@ -13,7 +13,10 @@ dominant kernel (the convolution kernel with a pre-packed filter) timed with HIP
 launch stream; `roofline.traffic` is the HBM bytes per launch taken from the committed rocprofv3
 counter summary (profiles/), null when that file is absent; `cpu_baseline` is the
 OpenMP restatement (oracle/cpu_baseline.c) on a bounded sample of the same workload.
-`extra` carries the other single-kernel configs for information only.
+`extra` carries the other configs (each kernel alone, and the whole programs through the plaidml API), all on
+the data the configs name (N(0,1) activations, uniform int8), and the rate the matrix cores sustain on LDS-resident
+operands with constant and with random values (the clock the chip holds under real data bounds every GEMM here).
+`--only a,b` runs just those legs of `extra` (for profiling runs); ResNet-50 img/s is repeated at the top level.
 
 `--copy-calibration` runs only a plain device copy of a known size (the factor that scales the
 FETCH_SIZE / WRITE_SIZE counters) and prints its byte count.
@@ -69,7 +72,9 @@ def valid_taps(size, k, pad):
     return sum(1 for x in range(size) for t in range(k) if 0 <= x + t - pad < size)
 
 
-def cpu_baseline_conv(E, N_sample, H, W, CI, CO, seed_i, seed_f, flops_per_image):
+def cpu_baseline_conv(N_sample, H, W, CI, CO, seed_i, seed_f, flops_per_image):
+    """The only leg that touches oracle/: the OpenMP restatement, timed on a bounded sample."""
+    from oracle import tile_oracle as E  # checker (test infrastructure), never the thing measured
     lib = ctypes.CDLL(os.path.join(ROOT, 'oracle', 'libcpu_baseline.so'))
     lib.cpu_baseline_threads.restype = ctypes.c_int
     threads = lib.cpu_baseline_threads()
@@ -140,12 +145,14 @@ def int8_program_leg(n=4096, runs=5):
             'd2h_ms': round(best['d2h_ms'], 3)}
 
 
-def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):
+def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):  # noqa: C901
     """Depthwise 3x3, pointwise 728->728 with the fused scale/shift + ReLU tail, max-pool 3x3/2 with window argmax."""
     out = {}
     px = N * H * W
-    dI, dD, dP = hk.DeviceBuffer(px * C * 2), hk.DeviceBuffer(px * C * 2), hk.DeviceBuffer(px * C * 2)
-    dI.fill_u32(0x3f803f80)
+    from plaidml_amd import edsl as P
+    rng = np.random.default_rng(7)
+    dI = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(rng.standard_normal((N, H, W, C)).astype(np.float32)))  # N(0,1) as the config says
+    dD, dP = hk.DeviceBuffer(px * C * 2), hk.DeviceBuffer(px * C * 2)
     # depthwise
     d = hk.Dwconv2dDesc()
     d.dtype = hk.BF16
@@ -153,8 +160,7 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):
     d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
     d.pad_h = d.pad_w = 1
     plan = L.pml_hip_dwconv2d_dispatch(ctypes.byref(d))
-    dF = hk.DeviceBuffer(9 * C * 2)
-    dF.fill_u32(0x3c003c00)
+    dF = hk.DeviceBuffer.from_numpy(P.to_bf16_bits((rng.standard_normal((3, 3, C, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)))
     ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_dwconv2d_invoke(plan, dI.ptr, dF.ptr, dD.ptr, none, none, None)), 20, 3)
     nbytes = 2 * px * C * 2
     out['depthwise3x3'] = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms / 1e6, 1), 'frac_hbm': round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
@@ -165,9 +171,9 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):
     g.tail = hk.make_tail(ops=[(hk.EPI_MUL, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 1, 0.0),
                                (hk.EPI_RELU, hk.BF16, 0, 0, 0.0)], operands=[(hk.BF16, 0, 1), (hk.BF16, 0, 1)])
     pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
-    dW, dS, dT = hk.DeviceBuffer(C * C * 2), hk.DeviceBuffer(C * 2), hk.DeviceBuffer(C * 2)
-    for b in (dW, dS, dT):
-        b.fill_u32(0x3c003c00)
+    dW = hk.DeviceBuffer.from_numpy(P.to_bf16_bits((rng.standard_normal((C, C)) * np.sqrt(2.0 / C)).astype(np.float32)))
+    dS = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(rng.uniform(0.5, 1.5, C).astype(np.float32)))
+    dT = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(rng.uniform(-0.5, 0.5, C).astype(np.float32)))
     hk.check(L.pml_hip_gemm_pack_b(pg, dW.ptr, None))
     ops = hk.ptr_array([dS.ptr, dT.ptr])
     ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dD.ptr, None, dP.ptr, None, ops, none, None)), 20, 3)
@@ -191,7 +197,7 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):
     return out
 
 
-def resnet50_leg(E, batch=128, runs=5):
+def resnet50_leg(batch=128, runs=5):
     """Whole-network forward through libplaidml.so: device time between the first and the last kernel of a run."""
     from plaidml_amd import edsl as P, op as Pop, resnet50
     prog, _, flops_full_box = resnet50.build(P, Pop, batch=batch, round_fn=P.round_bf16)
@@ -206,6 +212,8 @@ def resnet50_leg(E, batch=128, runs=5):
     best = min(times[1:], key=lambda t: t['kernel_ms'])
     return {'img_per_s': round(batch / (best['kernel_ms'] * 1e-3), 1), 'kernel_ms': round(best['kernel_ms'], 3),
             'h2d_ms': round(best['h2d_ms'], 3), 'd2h_ms': round(best['d2h_ms'], 3), 'launches': int(best['launches']),
+            'device_MB': round(best['device_bytes'] / 1e6, 1), 'arena_MB': round(best['arena_bytes'] / 1e6, 1),
+            'temporaries_unshared_MB': round(best['unshared_temp_bytes'] / 1e6, 1),
             'TFLOP/s_full_box': round(flops_full_box / (best['kernel_ms'] * 1e-3) / 1e12, 1),
             'frac_mfma_bf16': round(flops_full_box / (best['kernel_ms'] * 1e-3) / 1e12 / PEAK['bf16'], 4)}
 
@@ -222,6 +230,62 @@ def committed_traffic():
     return None
 
 
+def gemm_leg(hk, kind, n=4096):
+    """A square GEMM on the data its config names: int8 uniform in [-127, 127], bf16 N(0,1); B given as [N][K]."""
+    from plaidml_amd import edsl as P
+    L, none = hk.lib(), hk.ptr_array([])
+    g = hk.GemmDesc()
+    rng = np.random.default_rng(4)
+    if kind == 'i8':
+        g.in_dtype, g.out_dtype, g.c_dtype = hk.I8, hk.I32, hk.I32
+        a, b = rng.integers(-127, 128, (n, n), dtype=np.int8), rng.integers(-127, 128, (n, n), dtype=np.int8)
+        out_bytes, peak, unit = 4, PEAK['i8'], 'TOP/s'
+    else:
+        g.in_dtype = g.out_dtype = g.c_dtype = hk.BF16
+        a, b = (P.to_bf16_bits(rng.standard_normal((n, n)).astype(np.float32)) for _ in range(2))
+        out_bytes, peak, unit = 2, PEAK['bf16'], 'TFLOP/s'
+    g.m = g.n = g.k = g.lda = g.ldb = g.ldc = n
+    g.b_layout = 1
+    plan = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+    dA, dB, dC = hk.DeviceBuffer.from_numpy(a), hk.DeviceBuffer.from_numpy(b), hk.DeviceBuffer(n * n * out_bytes)
+    ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, None, none, none, None)), 20, 5)
+    res = {'ms': round(ms, 4), unit: round(2.0 * n ** 3 / ms / 1e9, 2), 'frac_mfma': round(2.0 * n ** 3 / ms / 1e9 / peak, 4),
+           'plan': hk.describe(plan), 'data': 'uniform int8 [-127, 127]' if kind == 'i8' else 'N(0,1) bf16'}
+    for buf in (dA, dB, dC):
+        buf.free()
+    L.pml_hip_plan_free(plan)
+    return res
+
+
+def mfma_ceiling_leg(hk):
+    """pml_hip_probe_mfma: bf16 MFMA stream on LDS-resident operands, constant against random operand values."""
+    out = {}
+    for name, rnd in (('constant_operands', 0), ('random_operands', 1)):
+        tf, mhz = ctypes.c_double(), ctypes.c_double()
+        hk.check(hk.lib().pml_hip_probe_mfma(rnd, 2000, ctypes.byref(tf), ctypes.byref(mhz)))
+        out[name] = {'TFLOP/s': round(tf.value, 1), 'frac_of_2500': round(tf.value / PEAK['bf16'], 4), 'core_clock_MHz': round(mhz.value)}
+    return out
+
+
+def conv_through_exec(N, H, W, CI, CO, Iv, Fv, runs=6):
+    """configs[1] bf16 as a Tile program through plaidml::exec: the planner's own choice of kernel, device ms per run."""
+    from plaidml_amd import edsl as P, op as Pop
+    I = P.Placeholder(P.DType.BFLOAT16, [N, H, W, CI])
+    F = P.Placeholder(P.DType.BFLOAT16, [3, 3, CI, CO])
+    B = P.Placeholder(P.DType.BFLOAT16, [CO])
+    prog = P.Program('conv', [I, F, B], [Pop.relu(Pop.convolution(I, F) + B)])
+    runner = P.Runner(prog, target='hip')
+    bias = np.zeros(CO, np.float32)
+    times = []
+    for _ in range(runs):
+        runner.run([Iv, Fv, bias])
+        times.append(P.last_run_stats())
+    best = min(times[1:], key=lambda t: t['kernel_ms'])
+    plan = [v for k, v in prog.passes if k == 'hip-plan']
+    return {'kernel_ms': round(best['kernel_ms'], 5), 'launches': int(best['launches']), 'h2d_ms': round(best['h2d_ms'], 3),
+            'd2h_ms': round(best['d2h_ms'], 3), 'plan': plan[0].splitlines()[1].strip() if plan else ''}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -230,12 +294,13 @@ def main():
     ap.add_argument('--no-extra', action='store_true')
     ap.add_argument('--no-cpu', action='store_true')
     ap.add_argument('--copy-calibration', action='store_true')
+    ap.add_argument('--only', default='', help='comma-separated legs of `extra` to run (default: all)')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus, file=sys.stderr)
         sys.exit(2)
 
-    from oracle import tile_oracle as E  # checker: used only for the cpu_baseline leg and the spot check
+    from plaidml_amd import edsl as P
     from plaidml_amd import hipkernels as hk
 
     hk.init(0)
@@ -250,10 +315,10 @@ def main():
     bytes_alg = (N * H * W * CI + N * H * W * CO) * 2 + 9 * CI * CO * 2 + CO * 2
 
     rng = np.random.default_rng(2)
-    Iv = E.round_bf16(rng.standard_normal((N, H, W, CI)).astype(np.float32))
-    Fv = E.round_bf16((np.random.default_rng(3).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32))
-    dI = hk.DeviceBuffer.from_numpy(E.bf16_bits(Iv))
-    dF = hk.DeviceBuffer.from_numpy(E.bf16_bits(Fv))
+    Iv = P.round_bf16(rng.standard_normal((N, H, W, CI)).astype(np.float32))
+    Fv = P.round_bf16((np.random.default_rng(3).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32))
+    dI = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(Iv))
+    dF = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(Fv))
     dB = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.uint16))
     dO = hk.DeviceBuffer(N * H * W * CO * 2)
     plan = conv_plan(hk, hk.BF16, N, H, W, CI, CO, 3, 3)
@@ -291,8 +356,8 @@ def main():
     # spot check of the timed output against the CPU baseline on the sampled images
     if not args.no_cpu:
         n_s = 4
-        cb, ref, _, _ = cpu_baseline_conv(E, n_s, H, W, CI, CO, 2, 3, flops / N)
-        got = E.bf16_from_bits(dO.to_numpy(np.uint16, (N, H, W, CO)))[:n_s]
+        cb, ref, _, _ = cpu_baseline_conv(n_s, H, W, CI, CO, 2, 3, flops / N)
+        got = P.from_bf16_bits(dO.to_numpy(np.uint16, (N, H, W, CO)))[:n_s]
         if not np.allclose(got, ref, rtol=2e-2, atol=2e-2):
             raise SystemExit('bench: GPU output disagrees with the CPU baseline on the sampled images')
         result['cpu_baseline'] = cb
@@ -300,65 +365,70 @@ def main():
         result['cpu_baseline'] = None
 
     if not args.no_extra:
+        only = set(x for x in args.only.split(',') if x)
+        want = lambda name: not only or name in only  # noqa: E731
         extra = {}
-        # configs[1] bf16 again, over five input / output pairs in turn (514 MB): the timed loop above re-reads one
-        # 51 MB input, which the 256 MB last-level cache in front of HBM can hold; here every launch reads from HBM
-        pairs = [(dI, dO)] + [(hk.DeviceBuffer.from_numpy(E.bf16_bits(Iv)), hk.DeviceBuffer(N * H * W * CO * 2)) for _ in range(4)]
-        turn = {'k': 0}
+        if want('conv_rotating'):
+            # configs[1] bf16 again, over five input / output pairs in turn (514 MB): the timed loop above re-reads one
+            # 51 MB input, which the 256 MB last-level cache in front of HBM can hold; here every launch reads from HBM
+            pairs = [(dI, dO)] + [(hk.DeviceBuffer.from_numpy(P.to_bf16_bits(Iv)), hk.DeviceBuffer(N * H * W * CO * 2)) for _ in range(4)]
+            turn = {'k': 0}
 
-        def rotating():
-            turn['k'] = (turn['k'] + 1) % len(pairs)
-            i_buf, o_buf = pairs[turn['k']]
-            hk.check(L.pml_hip_conv2d_invoke(plan, i_buf.ptr, None, o_buf.ptr, dB.ptr, none, none, None))
+            def rotating():
+                turn['k'] = (turn['k'] + 1) % len(pairs)
+                i_buf, o_buf = pairs[turn['k']]
+                hk.check(L.pml_hip_conv2d_invoke(plan, i_buf.ptr, None, o_buf.ptr, dB.ptr, none, none, None))
 
-        ms, _ = time_loop(hk, rotating, args.steps, args.warmup)
-        extra['conv_bf16_configs1_rotating_buffers'] = {
-            'ms': round(ms, 5), 'TFLOP/s': round(flops / ms / 1e9, 2), 'frac_mfma_bf16': round(flops / ms / 1e9 / PEAK['bf16'], 4),
-            'hbm_GBps_at_algorithmic_bytes': round(bytes_alg / (ms * 1e-3) / 1e9, 1), 'pairs': len(pairs)}
-        for i_buf, o_buf in pairs[1:]:
-            i_buf.free()
-            o_buf.free()
-        # configs[1], fp32 variant
-        dI32 = hk.DeviceBuffer.from_numpy(Iv)
-        dF32 = hk.DeviceBuffer.from_numpy(Fv)
-        dB32 = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.float32))
-        dO32 = hk.DeviceBuffer(N * H * W * CO * 4)
-        p32 = conv_plan(hk, hk.F32, N, H, W, CI, CO, 3, 3)
-        ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_conv2d_invoke(p32, dI32.ptr, dF32.ptr, dO32.ptr, dB32.ptr, none, none, None)),
-                          max(5, args.steps // 5), 3)
-        extra['conv_f32_configs1'] = {'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2),
-                                      'frac_mfma_f32': round(flops / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(p32)}
-        for b in (dI32, dF32, dB32, dO32):
-            b.free()
-        # configs[0]: fp32 GEMM 1024^3
-        g = hk.GemmDesc()
-        g.in_dtype = g.out_dtype = g.c_dtype = hk.F32
-        g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 1024
-        pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
-        A = np.random.default_rng(1).uniform(-1, 1, (1024, 1024)).astype(np.float32)
-        dA, dBm, dC = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(A.T.copy()), hk.DeviceBuffer(4 << 20)
-        ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dA.ptr, dBm.ptr, dC.ptr, None, none, none, None)), 50, 10)
-        extra['gemm_f32_1024_configs0'] = {'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2),
-                                           'frac_mfma_f32': round(2 * 1024 ** 3 / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(pg)}
-        # configs[2]: int8 GEMM 4096^3 -> int32
-        g = hk.GemmDesc()
-        g.in_dtype, g.out_dtype, g.c_dtype = hk.I8, hk.I32, hk.I32
-        g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 4096
-        pi = L.pml_hip_gemm_dispatch(ctypes.byref(g))
-        Ai = np.random.default_rng(4).integers(-127, 128, (4096, 4096), dtype=np.int8)
-        dAi, dBi, dCi = hk.DeviceBuffer.from_numpy(Ai), hk.DeviceBuffer.from_numpy(Ai.T.copy()), hk.DeviceBuffer(4096 * 4096 * 4)
-        hk.check(L.pml_hip_gemm_pack_b(pi, dBi.ptr, None))
-        ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pi, dAi.ptr, None, dCi.ptr, None, none, none, None)), 20, 5)
-        extra['gemm_i8_4096_configs2'] = {'ms': round(ms, 4), 'TOP/s': round(2 * 4096 ** 3 / ms / 1e9, 2),
-                                          'frac_mfma_i8': round(2 * 4096 ** 3 / ms / 1e9 / PEAK['i8'], 4), 'plan': hk.describe(pi),
-                                          'note': 'right-hand side packed once; the GEMM kernel alone'}
-        # configs[2] as a Tile program through the plaidml API: cast -> contraction (si32, first output) with the
-        # fused per-column requantisation tail (si8, second output); B is a program input, so it is re-laid per run
-        extra['int8_gemm_requant_program_configs2'] = int8_program_leg()
-        # configs[3]: Xception block pieces at full size (N64 19x19x728 bf16), each kernel alone
-        extra['xception_block_configs3'] = xception_leg(hk, L, none)
-        # configs[4]: ResNet-50 v1.5, batch 128, bf16, through the plaidml API (weights are program constants)
-        extra['resnet50_v1_5_b128_bf16'] = resnet50_leg(E)
+            ms, _ = time_loop(hk, rotating, args.steps, args.warmup)
+            extra['conv_bf16_configs1_rotating_buffers'] = {
+                'ms': round(ms, 5), 'TFLOP/s': round(flops / ms / 1e9, 2), 'frac_mfma_bf16': round(flops / ms / 1e9 / PEAK['bf16'], 4),
+                'hbm_GBps_at_algorithmic_bytes': round(bytes_alg / (ms * 1e-3) / 1e9, 1), 'pairs': len(pairs)}
+            for i_buf, o_buf in pairs[1:]:
+                i_buf.free()
+                o_buf.free()
+        if want('conv_exec'):
+            extra['conv_bf16_configs1_through_exec'] = conv_through_exec(N, H, W, CI, CO, Iv, Fv)
+            e = extra['conv_bf16_configs1_through_exec']
+            e['TFLOP/s'] = round(flops / e['kernel_ms'] / 1e9, 2)
+        if want('conv_f32'):
+            dI32 = hk.DeviceBuffer.from_numpy(Iv)
+            dF32 = hk.DeviceBuffer.from_numpy(Fv)
+            dB32 = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.float32))
+            dO32 = hk.DeviceBuffer(N * H * W * CO * 4)
+            p32 = conv_plan(hk, hk.F32, N, H, W, CI, CO, 3, 3)
+            ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_conv2d_invoke(p32, dI32.ptr, dF32.ptr, dO32.ptr, dB32.ptr, none, none, None)),
+                              max(5, args.steps // 5), 3)
+            extra['conv_f32_configs1'] = {'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2),
+                                          'frac_mfma_f32': round(flops / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(p32)}
+            for b in (dI32, dF32, dB32, dO32):
+                b.free()
+        if want('gemm_f32'):
+            # configs[0]: fp32 GEMM 1024^3, B as the program gives it ([K][N], re-laid per run)
+            g = hk.GemmDesc()
+            g.in_dtype = g.out_dtype = g.c_dtype = hk.F32
+            g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 1024
+            pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+            A = np.random.default_rng(1).uniform(-1, 1, (1024, 1024)).astype(np.float32)
+            dA, dBm, dC = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(A.T.copy()), hk.DeviceBuffer(4 << 20)
+            ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dA.ptr, dBm.ptr, dC.ptr, None, none, none, None)), 50, 10)
+            extra['gemm_f32_1024_configs0'] = {'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2),
+                                               'frac_mfma_f32': round(2 * 1024 ** 3 / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(pg)}
+        if want('gemm_i8'):
+            extra['gemm_i8_4096_configs2'] = gemm_leg(hk, 'i8')
+        if want('gemm_bf16'):
+            extra['gemm_bf16_4096'] = gemm_leg(hk, 'bf16')
+        if want('mfma_ceiling'):
+            extra['mfma_ceiling_bf16'] = mfma_ceiling_leg(hk)
+        if want('int8_program'):
+            # configs[2] as a Tile program through the plaidml API: cast -> contraction (si32, first output) with the
+            # fused per-column requantisation tail (si8, second output); B is a program input, so it is re-laid per run
+            extra['int8_gemm_requant_program_configs2'] = int8_program_leg()
+        if want('xception'):
+            extra['xception_block_configs3'] = xception_leg(hk, L, none)
+        if want('resnet50'):
+            # configs[4]: ResNet-50 v1.5, batch 128, bf16, through the plaidml API (weights are program constants)
+            extra['resnet50_v1_5_b128_bf16'] = resnet50_leg()
+            result['resnet50_b128_img_per_s'] = extra['resnet50_v1_5_b128_bf16']['img_per_s']
         result['extra'] = extra
 
     print(json.dumps(result))

@@ -231,6 +231,12 @@ int pml_hip_gemm_invoke2(int64_t plan, const void* a, const void* b, void* c, co
                          const void* init2, const void* const* operands, void* const* outs, pml_hip_stream s);
 int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s);
 
+/* Measurement aid (no counterpart in the reference): the bf16 rate the matrix cores of the current device sustain on
+ * operands that stay in LDS -- the instruction mix of the large GEMM tile, no global memory -- with constant operand
+ * values (random_data 0) or random ones of magnitude about 1 (random_data 1), and the core clock during the run.
+ * Random values make the chip lower its clock: the second figure is the ceiling a GEMM on N(0,1) data can reach. */
+int pml_hip_probe_mfma(int random_data, int iters, double* tflops, double* core_mhz);
+
 /* The GEMM above in one call that allocates nothing, neither on the host heap of the device runtime nor in
  * device memory: dispatch + invoke without a plan object.  It has no counterpart in the reference; it is for
  * callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid

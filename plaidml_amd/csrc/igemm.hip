@@ -55,24 +55,28 @@ __device__ inline unsigned join_offsets(unsigned x, unsigned y) { return ((x | y
 // XCD-aware tile order.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its
 // own L2, and a CU takes the next id of its XCD when it falls free: the workgroups resident on an XCD at any
 // time are a run of about 32 consecutive "local" numbers bid / 8.  What such a run costs the L2 is the
-// number of distinct A rows plus Bt rows under its tiles, so a run should be a compact block, not a strip:
-// the tile grid is cut into blocks of TH x TW tiles (32 tiles, as square as the grid allows), blocks are
-// numbered row-major, XCD x owns the blocks x*per/32 ... and walks each block row-major.  (4096^2 with
-// 256x256 tiles: 2 x 16 strips fetch 576 KB per K-slab and XCD, 4 x 8 blocks 384 KB; what misses L2 comes
-// over the fabric from the last-level cache, whose bandwidth is the scarce one.)
+// number of distinct A rows plus Bt rows under its tiles, so a run should be a compact block, not a strip,
+// and above all the tiles that share an A row block must not be dealt to eight different L2s (a 181 x 6
+// grid in workgroup-id order fetched A 6.5 times from memory).  XCD x therefore owns a contiguous range of
+// tile numbers t (the ranges differ by at most one tile when the count is no multiple of 8), and t walks
+// the grid in blocks of TH x TW tiles (32 tiles, as square as the grid allows).  When the grid divides into
+// whole blocks, blocks are numbered row-major and walked row-major; otherwise t walks groups of TH tile rows
+// column by column, the last group being as short as the grid leaves it.  (4096^2 with 256x256 tiles: 2 x 16
+// strips fetch 576 KB per K-slab and XCD, 4 x 8 blocks 384 KB; what misses L2 comes over the fabric from the
+// last-level cache, whose bandwidth is the scarce one.)
 __device__ inline void xcd_tile(int bid, int tiles_m, int tiles_n, int* tm, int* tn) {
   constexpr int kXcds = 8, kRun = 32;
   const int nblocks = tiles_m * tiles_n;
-  int t = bid;
-  if (nblocks % kXcds == 0) {
-    const int per = nblocks / kXcds;
-    t = (bid % kXcds) * per + (bid / kXcds);  // contiguous run per XCD
+  const int per = nblocks / kXcds, rem = nblocks % kXcds;
+  const int x = bid % kXcds;
+  const int t = x * per + (x < rem ? x : rem) + bid / kXcds;  // contiguous range per XCD
+  if (rem == 0 && per % kRun == 0) {
     int th = 0, tw = 0;
     if (tiles_m % 4 == 0 && tiles_n % 8 == 0) { th = 4; tw = 8; }
     else if (tiles_m % 8 == 0 && tiles_n % 4 == 0) { th = 8; tw = 4; }
     else if (tiles_m % 16 == 0 && tiles_n % 2 == 0) { th = 16; tw = 2; }
     else if (tiles_m % 2 == 0 && tiles_n % 16 == 0) { th = 2; tw = 16; }
-    if (th && per % kRun == 0) {
+    if (th) {
       const int blk = t / kRun, in = t % kRun;
       const int blocks_n = tiles_n / tw;
       *tm = (blk / blocks_n) * th + in / tw;
@@ -80,8 +84,14 @@ __device__ inline void xcd_tile(int bid, int tiles_m, int tiles_n, int* tm, int*
       return;
     }
   }
-  *tm = t / tiles_n;
-  *tn = t % tiles_n;
+  const int tw = tiles_n < 8 ? tiles_n : 8;
+  const int th = kRun / tw;
+  const int group = th * tiles_n;                      // tiles in a group of th tile rows
+  const int first_m = (t / group) * th;
+  const int rows = tiles_m - first_m < th ? tiles_m - first_m : th;
+  const int in = t % group;
+  *tm = first_m + in % rows;
+  *tn = in / rows;
 }
 
 // STAGES = 0: as many as pay for the tile; 2: two, and LDS rounded up to what staging the whole result
@@ -621,6 +631,83 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
 hipError_t PML_CAT(igemm_launch_kind_, PML_KIND)(int cfg, bool conv, const IgemmArgs& a, hipStream_t s) {
   return conv ? launch_kind<PML_KIND, true>(cfg, a, s) : launch_kind<PML_KIND, false>(cfg, a, s);
 }
+
+#if PML_KIND == 1
+// Measurement aid, not part of any contraction: what the matrix cores sustain on operands that never leave LDS
+// (no global traffic, no barriers), 8 wavefronts per CU with 128x64 tiles' instruction mix -- 8 MFMAs and 6
+// fragment reads per K-block.  With `random` the LDS holds random bf16 values of magnitude about 1, otherwise a
+// constant: the difference is what the switching activity of real data costs in clock frequency, i.e. the ceiling
+// a GEMM on N(0,1) data can reach on this device.  clk[0]: core clock ticks, clk[1]: 100 MHz ticks.
+__global__ __launch_bounds__(512) void mfma_probe_kernel(int iters, int random, float* sink, unsigned long long* clk) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  for (int o = tid * 4; o < 128 * 1024; o += 512 * 4) {
+    unsigned h = (o + blockIdx.x * 7919u) * 2654435761u;
+    h ^= h >> 15;
+    h *= 2246822519u;
+    h ^= h >> 13;
+    const unsigned lo = (h & 0x807f) | (0x3f00 + ((h >> 8) & 0x0180)), hi = ((h >> 16) & 0x807f) | (0x3f00 + ((h >> 24) & 0x0180));
+    *(unsigned*)(smem + o) = random ? (lo | (hi << 16)) : 0x3f803f80u;
+  }
+  __syncthreads();
+  unsigned long long t0 = 0, r0 = 0;
+  if (tid == 0 && blockIdx.x == 0) {
+    t0 = __builtin_amdgcn_s_memtime();
+    r0 = __builtin_amdgcn_s_memrealtime();
+  }
+  f32x16_t acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  i32x4_t fa[2][4], fb[2][2];
+  const unsigned char* base = smem + (wave & 3) * 16384 + ((lane & 31) * 128) + (((lane >> 5) ^ ((lane >> 1) & 7)) * 16);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) fa[0][i] = *(const i32x4_t*)(base + i * 4096);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) fb[0][j] = *(const i32x4_t*)(base + 65536 + j * 4096);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int cur = kb & 1, nxt = cur ^ 1;
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        mma_block<KIND_BF16>(acc[m / 2][m % 2], fb[cur][m % 2], fa[cur][m / 2]);
+        if (m < 4) fa[nxt][m] = *(const i32x4_t*)(base + m * 4096 + (it & 1) * 64);
+        else if (m < 6) fb[nxt][m - 4] = *(const i32x4_t*)(base + 65536 + (m - 4) * 4096 + (it & 1) * 64);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  if (tid == 0 && blockIdx.x == 0) {
+    clk[0] = __builtin_amdgcn_s_memtime() - t0;
+    clk[1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+  float total = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) total += acc[i][j][e];
+  if (total == 123.456f) sink[0] = total;  // keeps the accumulators alive
+}
+
+// MFMAs (32x32x16 bf16) issued by one launch of `iters` rounds on `blocks` workgroups.
+hipError_t mfma_probe_launch(int blocks, int iters, int random, float* sink, unsigned long long* clk, hipStream_t s) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)mfma_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)blocks), dim3(512), 128 * 1024, s, iters, random, sink, clk);
+  return hipGetLastError();
+}
+#endif
 
 #if PML_KIND == 0
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s) {

@@ -85,6 +85,7 @@ hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStr
 // shape does not qualify; `a.halo_rows` and `a.n_tiles` are filled in by conv_halo_prepare.
 size_t conv_halo_prepare(int kind, IgemmArgs* a);
 hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s);
+hipError_t mfma_probe_launch(int blocks, int iters, int random, float* sink, unsigned long long* clk, hipStream_t s);
 hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int64_t N, int64_t ldb, int64_t ldbt,
                           hipStream_t s);
 

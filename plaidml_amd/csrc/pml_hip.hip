@@ -871,6 +871,36 @@ int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s) {
   return 0;
 }
 
+int pml_hip_probe_mfma(int random_data, int iters, double* tflops, double* core_mhz) {
+  if (iters <= 0 || iters > 100000) return fail("probe_mfma: iters out of range");
+  const int blocks = device_cus();
+  float* sink = nullptr;
+  unsigned long long* clk = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int rc = 1;
+  do {
+    if (check(hipMalloc((void**)&sink, 64), "hipMalloc") || check(hipMalloc((void**)&clk, 64), "hipMalloc")) break;
+    if (check(hipEventCreate(&e0), "hipEventCreate") || check(hipEventCreate(&e1), "hipEventCreate")) break;
+    if (check(mfma_probe_launch(blocks, 16, random_data, sink, clk, nullptr), "mfma_probe_launch")) break;  // warm-up
+    if (check(hipEventRecord(e0, nullptr), "hipEventRecord")) break;
+    if (check(mfma_probe_launch(blocks, iters, random_data, sink, clk, nullptr), "mfma_probe_launch")) break;
+    if (check(hipEventRecord(e1, nullptr), "hipEventRecord") || check(hipEventSynchronize(e1), "hipEventSynchronize")) break;
+    float ms = 0;
+    if (check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime")) break;
+    unsigned long long host_clk[2] = {0, 0};
+    if (check(hipMemcpy(host_clk, clk, sizeof host_clk, hipMemcpyDeviceToHost), "hipMemcpy")) break;
+    const double mfmas = (double)iters * 4 * 8 * 8 * blocks;  // rounds x K-blocks x MFMAs per wavefront x wavefronts x workgroups
+    if (tflops) *tflops = mfmas * 32768.0 / (ms * 1e-3) / 1e12;
+    if (core_mhz) *core_mhz = host_clk[1] ? (double)host_clk[0] / ((double)host_clk[1] / 100.0) : 0.0;
+    rc = 0;
+  } while (false);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (sink) (void)hipFree(sink);
+  if (clk) (void)hipFree(clk);
+  return rc;
+}
+
 int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s) {
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_GEMM || !b2 || p->gemm.k2 <= 0) return fail("gemm_pack_b2: bad argument");
