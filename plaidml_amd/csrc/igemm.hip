@@ -23,6 +23,7 @@
 // After the K loop the accumulators are staged through LDS so that the tail runs
 // once per element in row-major order and stores are contiguous 8/16-byte pieces.
 #include <hip/hip_runtime.h>
+#include <atomic>
 
 #include <type_traits>
 
@@ -105,7 +106,12 @@ struct Ring {
   static constexpr int kStages = STAGES ? STAGES : ((BM * BN <= 64 * 64) ? 2 : (3 * kStage <= kLdsBytes ? 3 : 2));
   static constexpr int kTileBytes = BM * (BN + 4) * 4;
   static constexpr int kBytes = (STAGES && kTileBytes > kStages * kStage && kTileBytes <= kLdsBytes) ? kTileBytes : kStages * kStage;
-  static_assert(kBytes <= kLdsBytes, "the ring must fit the CU's LDS");
+  // 256 bytes behind the ring take what the "touch" loads of a residual tensor bring (their only purpose is to
+  // pull the rows into the caches; a load that writes LDS needs no register to land in).  Not for 64x64 tiles:
+  // five of their 32 KB rings fill a CU's LDS exactly.
+  static constexpr int kDump = BM * BN > 64 * 64 ? 256 : 0;
+  static constexpr int kAlloc = kBytes + kDump;
+  static_assert(kAlloc <= kLdsBytes, "the ring must fit the CU's LDS");
 };
 
 // BM x BN output tile, WAVES_M x WAVES_N wavefront grid; NT threads = 4, 8 or 16 wavefronts (one, two or four
@@ -115,7 +121,7 @@ struct Ring {
 // footprint lets a CU hold (at most two are counted on).
 template <int BM, int BN, int STAGES, int SLAB, int NT>
 constexpr int igemm_waves_per_simd() {
-  return (NT / 256) * (2 * Ring<BM, BN, STAGES, SLAB>::kBytes <= kLdsBytes ? 2 : 1);
+  return (NT / 256) * (2 * Ring<BM, BN, STAGES, SLAB>::kAlloc <= kLdsBytes ? 2 : 1);
 }
 
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
@@ -325,6 +331,28 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
 
   pre.valid = false;
   if (!direct) tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
+  // The direct tail reads its residual rows only after the K loop.  One 4-byte load per lane and 32x32 block,
+  // issued here and landing in the dump area of LDS, brings the 64 bytes a row contributes to the block into the
+  // caches: a short-K GEMM then waits for operands and residual together instead of one after the other.
+  // (Holding the rows in registers from here on -- 8 per block -- made the 128-register configurations spill.)
+  if constexpr (KIND == KIND_BF16 && WAVES_K == 1 && ring_t::kDump > 0 && MI * NI <= 4) {
+    if (direct && p.tail_mode == 2) {
+      const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc((void*)p.operands[0], 0, (int)kBufRange, kRsrcFlags);
+      const int64_t rs = p.tail.operand_row_stride[0];
+      // (the lane number through an opaque move, so that nothing worked out here is kept for the tail)
+      int lane_t = lane;
+      asm volatile("" : "+v"(lane_t));
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+          const int64_t m = m0 + wm * WM + i * 32 + (lane_t & 31);
+          const int64_t off = (m * rs + n0 + wn * WN + j * 32 + 16 * (lane_t >> 5)) * 2;
+          const unsigned voff = (m < p.M && off < (int64_t)kBufRange) ? (unsigned)off : kOutside;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rr, PML_LDS(smem + ring_t::kBytes), 4, (int)voff, 0, 0, 0);
+        }
+    }
+  }
 
   acc_t acc[MI][NI];
 #pragma unroll
@@ -588,13 +616,18 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  const size_t lds = Ring<BM, BN, STAGES, SLAB>::kBytes;
+  const size_t lds = Ring<BM, BN, STAGES, SLAB>::kAlloc;
   auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB>;
-  static bool attr_set = false;
-  if (!attr_set) {
+  // the attribute belongs to the kernel on one device: set once per device, from whichever thread comes first
+  // (two threads setting it at the same time set the same value)
+  static std::atomic<uint32_t> attr_set{0};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  const uint32_t bit = 1u << (dev & 31);
+  if (!(attr_set.load(std::memory_order_acquire) & bit)) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    attr_set = true;
+    attr_set.fetch_or(bit, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), lds, s, a);
   return hipGetLastError();

@@ -104,8 +104,9 @@ __device__ __forceinline__ void tail_prefetch(const IgemmArgs& p, int64_t m0, in
 }
 
 // ---------------------------------------------------------------------------------------------------
-// The common bf16 tails straight from the accumulators, without the trip through LDS: relu?(acc + bias)
-// and relu?(bf16(acc + bias) + residual).  A lane of a 32x32 block holds, for its row (lane & 31), the
+// The common bf16 tails straight from the accumulators, without the trip through LDS: relu?(acc + bias),
+// relu?(bf16(acc + bias) + residual) and the folded batch normalisation relu?(bf16(bf16(acc + bias) * scale) + shift),
+// every step rounded to bf16 as the step-wise tail does.  A lane of a 32x32 block holds, for its row (lane & 31), the
 // four columns 8g + 4 * (lane >> 5) ... of each group g; exchanging the upper half of group 2q with the
 // lower half of group 2q + 1 (v_permlane32_swap) leaves every lane with eight neighbouring columns of its
 // row -- columns 16q + 8 * (lane >> 5) ... -- which is one 16-byte store (8-byte stores measured a third
@@ -117,7 +118,8 @@ __device__ __forceinline__ void tail_prefetch(const IgemmArgs& p, int64_t m0, in
 template <int KIND>
 __device__ __forceinline__ bool direct_tail_ok(const IgemmArgs& p, int64_t n0, int bn) {
   if constexpr (KIND != KIND_BF16) return false;
-  if (p.out_dtype != PML_HIP_BF16 || (p.tail_mode != 1 && p.tail_mode != 2)) return false;
+  const bool scale_shift = p.tail_mode == 3 && p.tail_ssr != 0 && p.init2 == nullptr;
+  if (p.out_dtype != PML_HIP_BF16 || (p.tail_mode != 1 && p.tail_mode != 2 && !scale_shift)) return false;
   if (n0 + bn > p.N || (p.ldc & 7) != 0 || ((uintptr_t)p.C & 15) != 0) return false;
   if (p.init != nullptr && !(p.init_rs == 0 && p.init_cs == 1 && p.init_dtype == PML_HIP_BF16 && ((uintptr_t)p.init & 15) == 0)) return false;
   if (p.tail_mode == 2 && ((p.tail.operand_row_stride[0] & 7) != 0 || ((uintptr_t)p.operands[0] & 15) != 0)) return false;
@@ -152,7 +154,11 @@ template <int MI, int NI>
 __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&acc)[MI][NI], int64_t mw, int64_t nw, int lane) {
   const int hi = lane >> 5;
   const bool residual = p.tail_mode == 2;
+  const bool scale_shift = p.tail_mode == 3;
   const int64_t rs = p.tail.operand_row_stride[0];
+  const uint16_t* const scale = scale_shift ? (const uint16_t*)p.operands[p.tail.ops[0].operand] : nullptr;
+  const uint16_t* const shift = scale_shift ? (const uint16_t*)p.operands[p.tail.ops[1].operand] : nullptr;
+  const bool relu = scale_shift ? p.tail_ssr == 2 : p.tail_relu != 0;
   // the last MFMAs must have written the accumulators before the lane exchange below reads them: the compiler
   // cannot see that read (it is assembler text), so the longest MFMA's passes are waited out here, once
   asm volatile("s_nop 15\n\ts_nop 3");
@@ -162,10 +168,17 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
 #pragma unroll
     for (int q = 0; q < 2; ++q)
       bias_bits[q] = p.init != nullptr ? *(const i32x4_t*)((const uint16_t*)p.init + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
-    i32x4_t bias2_bits[2];  // the second product's bias (zeros when there is none)
+    // the second product's bias, or the scale vector of a scale / shift chain (which excludes a second product)
+    i32x4_t second_bits[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const uint16_t* src = scale_shift ? scale : (const uint16_t*)p.init2;
+      second_bits[q] = src != nullptr ? *(const i32x4_t*)(src + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+    }
+    i32x4_t shift_bits[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q)
-      bias2_bits[q] = p.init2 != nullptr ? *(const i32x4_t*)((const uint16_t*)p.init2 + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+      shift_bits[q] = scale_shift ? *(const i32x4_t*)(shift + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int64_t m = mw + i * 32 + (lane & 31);
@@ -177,11 +190,13 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
       }
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        float v[8], bias[8], bias2[8];
+        float v[8], bias[8], second[8];
         unpack_bf16x8(bias_bits[q], bias);
-        unpack_bf16x8(bias2_bits[q], bias2);
+        unpack_bf16x8(second_bits[q], second);
+        if (!scale_shift) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) bias[e] += bias2[e];
+          for (int e = 0; e < 8; ++e) bias[e] += second[e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           // x: group 2q, y: group 2q + 1; afterwards lanes 0..31 hold group 2q whole, lanes 32..63 group 2q + 1.
@@ -202,7 +217,18 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = c[e] + r[e];
         }
-        if (p.tail_relu) {
+        if (scale_shift) {
+          // three roundings: the contraction result, the product, the sum
+          float c[8], sh[8];
+          unpack_bf16x8(pack_bf16x8(v), c);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = c[e] * second[e];
+          unpack_bf16x8(pack_bf16x8(v), c);
+          unpack_bf16x8(shift_bits[q], sh);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = c[e] + sh[e];
+        }
+        if (relu) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = v[e] < 0.f ? 0.f : v[e];
         }

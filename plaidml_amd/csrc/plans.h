@@ -63,6 +63,7 @@ struct IgemmArgs {
   // fast tail: 0 = interpret `tail`; 1 = (optional relu) then store as c_dtype
   int tail_mode;
   int tail_relu;
+  int tail_ssr;  // tail_mode 3 only: 1 = result * column vector + column vector, 2 = the same and relu (all in the bf16 result type)
   int c_dtype;
   pml_hip_epilogue tail;
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];

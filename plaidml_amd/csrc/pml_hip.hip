@@ -235,6 +235,21 @@ void classify_tail(const pml_hip_epilogue& t, int out_dtype, int c_dtype, int* m
   }
 }
 
+// The scale / shift (/ relu) chain of a folded batch normalisation, bf16 throughout: result * v0[col] + v1[col].
+// 0: the chain is something else; 1: without relu; 2: with relu.
+int tail_scale_shift(const pml_hip_epilogue& t, int out_dtype, int mode) {
+  if (mode != 3 || out_dtype != PML_HIP_BF16 || (t.n_ops != 2 && t.n_ops != 3)) return 0;
+  const int want[3] = {PML_HIP_EPI_MUL, PML_HIP_EPI_ADD, PML_HIP_EPI_RELU};
+  for (int i = 0; i < t.n_ops; ++i) {
+    const pml_hip_epi_op& op = t.ops[i];
+    if (op.opcode != want[i] || op.dtype != PML_HIP_BF16) return 0;
+    if (i < 2 && (op.operand_kind != PML_HIP_OPND_TENSOR || t.operand_col_stride[op.operand] != 1 || t.operand_row_stride[op.operand] != 0 ||
+                  t.operand_dtype[op.operand] != PML_HIP_BF16))
+      return 0;
+  }
+  return t.n_ops - 1;
+}
+
 bool valid_tail(const pml_hip_epilogue& t) {
   if (t.n_ops < 0 || t.n_ops > PML_HIP_MAX_EPI_OPS) return false;
   if (t.n_operands < 0 || t.n_operands > PML_HIP_MAX_EPI_OPERANDS) return false;
@@ -319,6 +334,7 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.init_cs = d.init_col_stride;
   g.c_dtype = d.c_dtype;
   classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
+  g.tail_ssr = tail_scale_shift(d.tail, d.out_dtype, g.tail_mode);
   g.tail = d.tail;
   g.NB = (int)d.n;
   g.n_cus = device_cus();
@@ -613,6 +629,7 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   g.c_dtype = d.c_dtype;
   g.n_cus = device_cus();
   classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
+  g.tail_ssr = tail_scale_shift(d.tail, d.out_dtype, g.tail_mode);
   g.tail = d.tail;
   for (int i = 0; i < d.tail.n_operands; ++i) {
     if (!operands || !operands[i]) return fail("gemm_invoke: missing tail operand");

@@ -159,6 +159,39 @@ def test_gemm_two_products(stride):
     L.pml_hip_plan_free(plan)
 
 
+@pytest.mark.parametrize('tile', ['', '128x128w8s2', '128x64w8', '256x128w16', '256x256w8'])
+def test_gemm_bf16_step_tails_bit_exact(tile, monkeypatch):
+    """The bf16 tails that leave the accumulators directly (interior tiles) and through LDS (the ragged last column
+    tile) must round alike: small-integer operands make the fp32 accumulation exact, so the expected result is
+    fixed bit for bit by the declared step semantics -- each step rounds to bf16 -- for the folded batch
+    normalisation relu(x * scale + shift) and for relu(x + residual)."""
+    rng = np.random.default_rng(33)
+    M, N, K = 300, 392, 72
+    A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    bias = E.round_bf16(rng.standard_normal(N).astype(np.float32) * 8)
+    scale = E.round_bf16(rng.uniform(0.5, 1.5, N).astype(np.float32))
+    shift = E.round_bf16(rng.standard_normal(N).astype(np.float32) * 20)
+    res = E.round_bf16(rng.standard_normal((M, N)).astype(np.float32) * 30)
+    x = E.round_bf16((A @ B + bias).astype(np.float32))  # exact sum, one rounding
+    for relu in (False, True):
+        ops = [(hk.EPI_MUL, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 1, 0.0)]
+        ops += [(hk.EPI_RELU, hk.BF16, 0, 0, 0.0)] if relu else []
+        tail = hk.make_tail(ops=ops, operands=[(hk.BF16, 0, 1), (hk.BF16, 0, 1)])
+        C = run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16, tail=tail,
+                     operands=(bf16(scale), bf16(shift)))
+        want = E.round_bf16(E.round_bf16(x * scale) + shift)
+        want = np.maximum(want, 0) if relu else want
+        np.testing.assert_array_equal(C, bf16(want))
+        ops = [(hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 0, 0.0)] + ([(hk.EPI_RELU, hk.BF16, 0, 0, 0.0)] if relu else [])
+        tail = hk.make_tail(ops=ops, operands=[(hk.BF16, N, 1)])
+        C = run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16, tail=tail,
+                     operands=(bf16(res),))
+        want = E.round_bf16(x + res)
+        want = np.maximum(want, 0) if relu else want
+        np.testing.assert_array_equal(C, bf16(want))
+
+
 def test_gemm_bf16_4096_sampled():
     """bf16 4096^3 with N(0,1) inputs (the large-tile path): sampled rows and columns against float64."""
     rng = np.random.default_rng(9)
