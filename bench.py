@@ -3,9 +3,10 @@
 
 Workload (BASELINE.json configs[1]): conv2d NHWC via the contraction
   O[n,y,x,co] += I[n,y+ky-1,x+kx-1,ci] * F[ky,kx,ci,co]   (N128, 56x56x64, 3x3x64x64, stride 1, SAME)
-followed by the fused bias + ReLU tail, bf16 (fp32 accumulate).  One step = one pass over the
+followed by the fused bias + ReLU tail, bf16 (fp32 accumulate).  One step = one pass over one
 batch, inputs (image, HWCK filter, bias) resident in HBM: a single launch of the resident-filter
-convolution kernel, which re-lays the filter out on its way into LDS.
+convolution kernel, which re-lays the filter out on its way into LDS.  Consecutive steps take five
+input / output buffer pairs in turn, so that no step finds its input in the last-level cache.
 
 Prints ONE JSON line.  `value` is TFLOP/s over the algorithmic FLOPs (2 x valid index tuples:
 SAME-padding taps that fall outside the image are not counted).  `roofline` describes the
@@ -317,17 +318,29 @@ def main():
     rng = np.random.default_rng(2)
     Iv = P.round_bf16(rng.standard_normal((N, H, W, CI)).astype(np.float32))
     Fv = P.round_bf16((np.random.default_rng(3).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32))
-    dI = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(Iv))
+    # Five input / output pairs taken in turn (514 MB): a loop over one pair re-reads a 51 MB input that the 256 MB
+    # last-level cache in front of HBM can hold between launches; in turn, every launch reads from HBM.
+    n_pairs = 5
+    bits = P.to_bf16_bits(Iv)
+    pairs = [(hk.DeviceBuffer.from_numpy(bits), hk.DeviceBuffer(N * H * W * CO * 2)) for _ in range(n_pairs)]
+    dI, dO = pairs[0]
     dF = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(Fv))
     dB = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.uint16))
-    dO = hk.DeviceBuffer(N * H * W * CO * 2)
     plan = conv_plan(hk, hk.BF16, N, H, W, CI, CO, 3, 3)
     none = hk.ptr_array([])
+    turn = {'k': 0}
 
-    def step():
-        hk.check(L.pml_hip_conv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, dB.ptr, none, none, None))
+    def step():  # one batch through the convolution, filter as the caller holds it (HWCK)
+        turn['k'] = (turn['k'] + 1) % n_pairs
+        i_buf, o_buf = pairs[turn['k']]
+        hk.check(L.pml_hip_conv2d_invoke(plan, i_buf.ptr, dF.ptr, o_buf.ptr, dB.ptr, none, none, None))
 
-    def kernel_only():
+    def kernel_only():  # the same with the filter packed once, as a network's constant weights are
+        turn['k'] = (turn['k'] + 1) % n_pairs
+        i_buf, o_buf = pairs[turn['k']]
+        hk.check(L.pml_hip_conv2d_invoke(plan, i_buf.ptr, None, o_buf.ptr, dB.ptr, none, none, None))
+
+    def one_pair():
         hk.check(L.pml_hip_conv2d_invoke(plan, dI.ptr, None, dO.ptr, dB.ptr, none, none, None))
 
     ms_step, wall_step = time_loop(hk, step, args.steps, args.warmup)
@@ -344,7 +357,7 @@ def main():
         'dtype': 'bf16', 'data': 'synthetic',
         'config': {'workload': 'configs[1]: conv2d NHWC N128 56x56x64 (*) 3x3x64x64 stride 1 SAME + bias + ReLU, bf16, fp32 accumulate',
                    'plan': hk.describe(plan), 'device': hk.device_name(),
-                   'algorithmic_gflop': round(flops / 1e9, 3), 'full_box_gflop': round(flops_full_box / 1e9, 3),
+                   'input_output_pairs_in_turn': n_pairs, 'algorithmic_gflop': round(flops / 1e9, 3), 'full_box_gflop': round(flops_full_box / 1e9, 3),
                    'host_wall_ms_per_step': round(wall_step, 5)},
         'roofline': {'bound': 'mfma', 'achieved': round(flops / (ms_kernel * 1e-3) / 1e12, 3), 'peak': PEAK['bf16'],
                      'unit': 'TFLOP/s', 'frac': round(flops / (ms_kernel * 1e-3) / 1e12 / PEAK['bf16'], 4),
@@ -368,24 +381,12 @@ def main():
         only = set(x for x in args.only.split(',') if x)
         want = lambda name: not only or name in only  # noqa: E731
         extra = {}
-        if want('conv_rotating'):
-            # configs[1] bf16 again, over five input / output pairs in turn (514 MB): the timed loop above re-reads one
-            # 51 MB input, which the 256 MB last-level cache in front of HBM can hold; here every launch reads from HBM
-            pairs = [(dI, dO)] + [(hk.DeviceBuffer.from_numpy(P.to_bf16_bits(Iv)), hk.DeviceBuffer(N * H * W * CO * 2)) for _ in range(4)]
-            turn = {'k': 0}
-
-            def rotating():
-                turn['k'] = (turn['k'] + 1) % len(pairs)
-                i_buf, o_buf = pairs[turn['k']]
-                hk.check(L.pml_hip_conv2d_invoke(plan, i_buf.ptr, None, o_buf.ptr, dB.ptr, none, none, None))
-
-            ms, _ = time_loop(hk, rotating, args.steps, args.warmup)
-            extra['conv_bf16_configs1_rotating_buffers'] = {
+        if want('conv_one_pair'):
+            # the same kernel over ONE input / output pair (what the last-level cache can hold): the cache-resident figure
+            ms, _ = time_loop(hk, one_pair, args.steps, args.warmup)
+            extra['conv_bf16_configs1_one_buffer_pair'] = {
                 'ms': round(ms, 5), 'TFLOP/s': round(flops / ms / 1e9, 2), 'frac_mfma_bf16': round(flops / ms / 1e9 / PEAK['bf16'], 4),
-                'hbm_GBps_at_algorithmic_bytes': round(bytes_alg / (ms * 1e-3) / 1e9, 1), 'pairs': len(pairs)}
-            for i_buf, o_buf in pairs[1:]:
-                i_buf.free()
-                o_buf.free()
+                'hbm_GBps_at_algorithmic_bytes': round(bytes_alg / (ms * 1e-3) / 1e9, 1)}
         if want('conv_exec'):
             extra['conv_bf16_configs1_through_exec'] = conv_through_exec(N, H, W, CI, CO, Iv, Fv)
             e = extra['conv_bf16_configs1_through_exec']
