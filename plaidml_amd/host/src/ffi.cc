@@ -301,7 +301,18 @@ uint64_t plaidml_shape_get_nbytes(plaidml_error* err, plaidml_shape* shape) {
 
 plaidml_buffer* plaidml_buffer_alloc(plaidml_error* err, plaidml_shape* shape) {
   return ffi_wrap<plaidml_buffer*>(err, nullptr,
-                                   [&] { return new plaidml_buffer{std::make_shared<util::SimpleBuffer>(shape->shape)}; });
+                                   [&] {
+                                     // large buffers in page-locked memory when a GPU is visible: exec copies to and
+                                     // from them at the link's rate (65536: below that the copy's set-up dominates)
+                                     if (shape->shape.getByteSize() >= 65536) {
+                                       try {
+                                         return new plaidml_buffer{
+                                             std::make_shared<util::ForeignBuffer>(shape->shape, rt::pinnedAlloc, rt::pinnedFree)};
+                                       } catch (const std::bad_alloc&) {
+                                       }
+                                     }
+                                     return new plaidml_buffer{std::make_shared<util::SimpleBuffer>(shape->shape)};
+                                   });
 }
 plaidml_buffer* plaidml_buffer_adopt(plaidml_error* err, plaidml_shape* shape, char* data, size_t size) {
   return ffi_wrap<plaidml_buffer*>(

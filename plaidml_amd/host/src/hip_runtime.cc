@@ -390,6 +390,19 @@ void registerRuntime(const std::string& id, std::shared_ptr<Runtime> runtime) {
   registry()[id] = std::move(runtime);
 }
 
+void* pinnedAlloc(size_t bytes) {
+  initRuntimes();
+  if (listDevices().empty()) return nullptr;
+  void* p = nullptr;
+  if (pml_hip_host_alloc(&p, bytes) != 0 || !p) return nullptr;
+  std::memset(p, 0, bytes);
+  return p;
+}
+
+void pinnedFree(void* p) {
+  if (p) pml_hip_host_free(p);
+}
+
 void initRuntimes() {
   static bool done = false;
   if (done) return;

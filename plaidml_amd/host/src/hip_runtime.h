@@ -45,6 +45,12 @@ void initRuntimes();
 std::vector<std::string> listDevices();
 std::shared_ptr<Device> getDevice(const std::string& deviceID);
 
+// Host memory the GPU can read and write directly (page-locked), for buffers the library allocates itself: a
+// copy to or from it runs at the link's rate instead of being staged through the driver's own bounce buffers.
+// Zero-initialised.  nullptr when no GPU is visible (the caller falls back to ordinary memory).
+void* pinnedAlloc(size_t bytes);
+void pinnedFree(void* p);
+
 // statistics of the most recent invoke of any hip executable in this thread (for benchmarks)
 struct InvokeStats {
   double kernel_ms = 0;  // first launch -> last launch, HIP events

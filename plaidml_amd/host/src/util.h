@@ -8,6 +8,7 @@
 #include <cstring>
 #include <map>
 #include <memory>
+#include <new>
 #include <sstream>
 #include <stdexcept>
 #include <string>
@@ -175,6 +176,36 @@ class SimpleBuffer : public Buffer, public std::enable_shared_from_this<SimpleBu
 
  private:
   std::vector<char> data_;
+};
+
+// owns zero-initialised storage obtained from (and returned to) a caller-given pair of functions: page-locked
+// host memory when a GPU is present
+class ForeignBuffer : public Buffer {
+ public:
+  typedef void* (*AllocFn)(size_t);
+  typedef void (*FreeFn)(void*);
+  // throws std::bad_alloc when `alloc` returns nullptr
+  ForeignBuffer(const TensorShape& shape, AllocFn alloc, FreeFn release)
+      : Buffer(shape), size_(shape.getByteSize()), alloc_(alloc), release_(release) {
+    data_ = static_cast<char*>(alloc_(size_ ? size_ : 1));
+    if (!data_) throw std::bad_alloc();
+  }
+  ~ForeignBuffer() override { release_(data_); }
+  ForeignBuffer(const ForeignBuffer&) = delete;
+  ForeignBuffer& operator=(const ForeignBuffer&) = delete;
+  char* data() final { return data_; }
+  size_t size() const final { return size_; }
+  BufferPtr clone() final {
+    auto copy = std::make_shared<ForeignBuffer>(shape_, alloc_, release_);
+    std::memcpy(copy->data_, data_, size_);
+    return copy;
+  }
+
+ private:
+  char* data_ = nullptr;
+  size_t size_;
+  AllocFn alloc_;
+  FreeFn release_;
 };
 
 // aliases caller memory: no copy, no ownership
