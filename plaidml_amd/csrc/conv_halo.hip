@@ -1070,12 +1070,8 @@ template <int KIND, int WV>
 hipError_t launch_regfilter(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
   constexpr int NI = 1;  // measured on the 128 x 56 x 56 x 64 case: 33.7 us against 42.7 us with NI = 2
   auto kern = conv_regfilter3x3_kernel<KIND, WV, NI>;
-  static size_t attr_lds = 0;
-  if (lds > attr_lds) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    attr_lds = lds;
-  }
+  static DynamicLdsLimit limit;
+  if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
   const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512 / NI), lds, s, a);
   return hipGetLastError();
@@ -1084,12 +1080,8 @@ hipError_t launch_regfilter(const IgemmArgs& a, size_t lds, int n_cus, hipStream
 template <int KIND, int NCH>
 hipError_t launch3x3(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
   auto kern = conv_halo3x3_kernel<KIND, NCH>;
-  static size_t attr_lds = 0;
-  if (lds > attr_lds) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    attr_lds = lds;
-  }
+  static DynamicLdsLimit limit;
+  if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
   const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), lds, s, a);
   return hipGetLastError();
@@ -1098,12 +1090,8 @@ hipError_t launch3x3(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
 template <int KIND>
 hipError_t launch(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
   auto kern = conv_halo_kernel<KIND>;
-  static size_t attr_lds = 0;
-  if (lds > attr_lds) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    attr_lds = lds;
-  }
+  static DynamicLdsLimit limit;
+  if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
   const int grid = a.n_tiles < n_cus ? a.n_tiles : n_cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), lds, s, a);
   return hipGetLastError();

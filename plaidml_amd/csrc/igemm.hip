@@ -23,7 +23,6 @@
 // After the K loop the accumulators are staged through LDS so that the tail runs
 // once per element in row-major order and stores are contiguous 8/16-byte pieces.
 #include <hip/hip_runtime.h>
-#include <atomic>
 
 #include <type_traits>
 
@@ -618,17 +617,8 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const size_t lds = Ring<BM, BN, STAGES, SLAB>::kAlloc;
   auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB>;
-  // the attribute belongs to the kernel on one device: set once per device, from whichever thread comes first
-  // (two threads setting it at the same time set the same value)
-  static std::atomic<uint32_t> attr_set{0};
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-  const uint32_t bit = 1u << (dev & 31);
-  if (!(attr_set.load(std::memory_order_acquire) & bit)) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    attr_set.fetch_or(bit, std::memory_order_release);
-  }
+  static DynamicLdsLimit limit;
+  if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), lds, s, a);
   return hipGetLastError();
 }

@@ -3,6 +3,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <mutex>
 #include <stdint.h>
 
 #include <string>
@@ -10,6 +12,24 @@
 #include "pml_hip.h"
 
 namespace pml {
+
+// The dynamic-LDS ceiling of a kernel (hipFuncAttributeMaxDynamicSharedMemorySize) belongs to the kernel on one
+// device.  One of these per kernel instantiation remembers, per device, the largest size already set.
+struct DynamicLdsLimit {
+  std::mutex lock;
+  size_t set[32] = {};
+  hipError_t ensure(const void* kernel, size_t bytes) {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    std::lock_guard<std::mutex> hold(lock);
+    size_t& have = set[dev & 31];
+    if (bytes <= have) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes); e != hipSuccess) return e;
+    have = bytes;
+    return hipSuccess;
+  }
+};
+
 
 enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2 };
 // _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages; _K2: two wavefront grids share the K-blocks of every slab

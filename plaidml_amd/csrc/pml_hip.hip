@@ -1057,6 +1057,10 @@ int64_t pml_hip_eltwise_dispatch(const pml_hip_eltwise_desc* d) {
     fail("eltwise: malformed tail");
     return 0;
   }
+  if (!valid_tail(t)) {
+    fail("eltwise: a step of the chain names an unknown operation or an operand outside the operand list");
+    return 0;
+  }
   Plan* p = new Plan();
   p->kind = PLAN_ELTWISE;
   p->elt = *d;

@@ -1016,6 +1016,9 @@ class Planner {
     *a = op.operands[0];
     *b = op.operands[1];
     const DataType adt = (*a)->shape.elementType, bdt = (*b)->shape.elementType;
+    // the matrix-core kernels address an operand with 32-bit byte offsets: larger ones take the general kernel
+    const size_t kOffsetLimit = size_t(1) << 31;
+    if ((*a)->shape.getByteSize() >= kOffsetLimit || (*b)->shape.getByteSize() >= kOffsetLimit) return false;
     if (adt == bdt && adt == rdt && (rdt == DataType::f32 || rdt == DataType::bf16)) {
       *in_dt = hipType(rdt);
       *out_dt = hipType(rdt);

@@ -50,3 +50,9 @@ def test_dispatch_rejects_bad_descriptors_without_a_gpu():
     sc.rank, sc.idx_rank, sc.upd_rank, sc.dtype, sc.idx_dtype = 1, 1, 1, hk.F32, hk.F32
     assert L.pml_hip_scatter(ctypes.byref(sc), one, ctypes.c_void_p(2), one, ctypes.c_void_p(3), None) != 0
     assert b'si32 or ui32' in L.pml_hip_last_error()
+    # an elementwise chain whose step names an operand outside the operand list
+    e = hk.EltwiseDesc()
+    e.rank = 1
+    e.tail = hk.make_tail(ops=[(hk.EPI_ADD, hk.F32, hk.OPND_TENSOR, 3, 0.0)], operands=[(hk.F32, 0, 1)])
+    assert L.pml_hip_eltwise_dispatch(ctypes.byref(e)) == 0
+    assert b'outside the operand list' in L.pml_hip_last_error()

@@ -57,6 +57,18 @@ def test_projection_shortcut_and_main_path_share_one_launch():
     assert 'second product' not in plan_of(prog, 'hip{fuse=0}')
 
 
+def test_operand_of_two_gib_takes_the_general_kernel():
+    """The matrix-core kernels address an operand with 32-bit byte offsets; a contraction over a larger one must
+    be planned onto the general kernel at compile time instead of failing at every run."""
+    A = E.Placeholder(D.FLOAT32, [32768, 16384], name='A')      # exactly 2 GiB
+    B = E.Placeholder(D.FLOAT32, [16384, 8], name='B')
+    t = plan_of(E.Program('big_dot', [A, B], [op.dot(A, B)]))
+    assert 'contract (general)' in t and 'gemm' not in t, t
+    A = E.Placeholder(D.FLOAT32, [32768, 8192], name='A')       # 1 GiB: the GEMM kernel
+    B = E.Placeholder(D.FLOAT32, [8192, 8], name='B')
+    assert 'gemm f32' in plan_of(E.Program('dot', [A, B], [op.dot(A, B)]))
+
+
 def test_target_options_switch_specialisation_off():
     prog = programs.config1_conv(E, op, 'BFLOAT16')[0]
     t = plan_of(prog, 'hip{specialise=0,fuse=0}')
