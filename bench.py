@@ -38,9 +38,10 @@ PEAK = {'bf16': 2500.0, 'f32': 157.3, 'i8': 5000.0}  # dense MFMA TFLOP/s (TOP/s
 HBM_PEAK_GBS = 8000.0
 
 
-def conv_plan(hk, in_dt, N, H, W, CI, CO, KH, KW, relu=True):
+def conv_plan(hk, in_dt, N, H, W, CI, CO, KH, KW, relu=True, flags=0):
     d = hk.Conv2dDesc()
     d.in_dtype, d.out_dtype, d.c_dtype = in_dt, in_dt, in_dt
+    d.flags = flags
     d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, KH, KW, CO, H, W
     d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
     d.pad_h, d.pad_w = (KH - 1) // 2, (KW - 1) // 2
@@ -392,28 +393,37 @@ def main():
             e = extra['conv_bf16_configs1_through_exec']
             e['TFLOP/s'] = round(flops / e['kernel_ms'] / 1e9, 2)
         if want('conv_f32'):
+            # configs[1] in fp32: with fp32 MFMAs, and with every operand value split into a bf16 head + remainder in
+            # registers (three bf16 MFMAs per term, rtol 1e-3 kept: tests/test_kernels_gpu.py)
             dI32 = hk.DeviceBuffer.from_numpy(Iv)
             dF32 = hk.DeviceBuffer.from_numpy(Fv)
             dB32 = hk.DeviceBuffer.from_numpy(np.zeros(CO, np.float32))
             dO32 = hk.DeviceBuffer(N * H * W * CO * 4)
-            p32 = conv_plan(hk, hk.F32, N, H, W, CI, CO, 3, 3)
-            ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_conv2d_invoke(p32, dI32.ptr, dF32.ptr, dO32.ptr, dB32.ptr, none, none, None)),
-                              max(5, args.steps // 5), 3)
-            extra['conv_f32_configs1'] = {'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2),
-                                          'frac_mfma_f32': round(flops / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(p32)}
+            for name, flags in (('conv_f32_configs1', 0), ('conv_f32_as_bf16x3_configs1', hk.FP32_AS_BF16X3)):
+                p32 = conv_plan(hk, hk.F32, N, H, W, CI, CO, 3, 3, flags=flags)
+                ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_conv2d_invoke(p32, dI32.ptr, dF32.ptr, dO32.ptr, dB32.ptr, none, none, None)),
+                                  max(5, args.steps // 5), 3)
+                extra[name] = {'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2),
+                               'frac_mfma_f32': round(flops / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(p32)}
+                L.pml_hip_plan_free(p32)
             for b in (dI32, dF32, dB32, dO32):
                 b.free()
         if want('gemm_f32'):
-            # configs[0]: fp32 GEMM 1024^3, B as the program gives it ([K][N], re-laid per run)
-            g = hk.GemmDesc()
-            g.in_dtype = g.out_dtype = g.c_dtype = hk.F32
-            g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 1024
-            pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+            # configs[0]: fp32 GEMM 1024^3, B as the program gives it ([K][N], re-laid per run); both fp32 modes
             A = np.random.default_rng(1).uniform(-1, 1, (1024, 1024)).astype(np.float32)
             dA, dBm, dC = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(A.T.copy()), hk.DeviceBuffer(4 << 20)
-            ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dA.ptr, dBm.ptr, dC.ptr, None, none, none, None)), 50, 10)
-            extra['gemm_f32_1024_configs0'] = {'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2),
-                                               'frac_mfma_f32': round(2 * 1024 ** 3 / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(pg)}
+            for name, flags in (('gemm_f32_1024_configs0', 0), ('gemm_f32_as_bf16x3_1024_configs0', hk.FP32_AS_BF16X3)):
+                g = hk.GemmDesc()
+                g.in_dtype = g.out_dtype = g.c_dtype = hk.F32
+                g.m = g.n = g.k = g.lda = g.ldb = g.ldc = 1024
+                g.flags = flags
+                pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
+                ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dA.ptr, dBm.ptr, dC.ptr, None, none, none, None)), 50, 10)
+                extra[name] = {'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2),
+                               'frac_mfma_f32': round(2 * 1024 ** 3 / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(pg)}
+                L.pml_hip_plan_free(pg)
+            for b in (dA, dBm, dC):
+                b.free()
         if want('gemm_i8'):
             extra['gemm_i8_4096_configs2'] = gemm_leg(hk, 'i8')
         if want('gemm_bf16'):

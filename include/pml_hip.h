@@ -157,6 +157,9 @@ enum {
 #define PML_HIP_MAX_EPI_OPERANDS 6
 #define PML_HIP_MAX_RANK 6
 
+/* descriptor flag of gemm and conv2d (in_dtype F32 only): multiply fp32 operands as three bf16 products */
+#define PML_HIP_FP32_AS_BF16X3 1
+
 typedef struct {
   int32_t opcode;
   int32_t dtype;        /* result element type of this step */
@@ -184,7 +187,10 @@ typedef struct {
  * Replaces plaidml_rt_xsmm_gemm_dispatch_f32 / _invoke_f32 and the bias / relu
  * variants (pmlc/rt/xsmm.cc:17-233), and the strided batch-reduce
  * plaidml_rt_xsmm_brgemm_* (:235-287).
- *   in_dtype F32  -> fp32 MFMA, fp32 accumulate
+ *   in_dtype F32  -> fp32 MFMA, fp32 accumulate; with PML_HIP_FP32_AS_BF16X3 in `flags` every operand value is
+ *                    split into a bf16 head and a bf16 remainder in registers and each product is formed as
+ *                    head*head + remainder*head + head*remainder on the bf16 matrix cores (fp32 accumulate):
+ *                    about 2^-16 relative error per product instead of 2^-24, at several times the fp32 MFMA rate
  *   in_dtype BF16 -> bf16 MFMA, fp32 accumulate, result rounded once to acc_dtype's storage
  *   in_dtype I8   -> int8 MFMA, int32 accumulate (this is the `cast(A, INT32)` then
  *                    contract pattern of plaidml/edsl/tests/edsl_test.cc:509-545 applied to int8)
@@ -216,6 +222,8 @@ typedef struct {
   int32_t a2_stride;
   int32_t init2_kind;
   int64_t a2_h, a2_w, a2_oh, a2_ow;
+  int32_t flags; /* PML_HIP_FP32_AS_BF16X3 or 0 */
+  int32_t reserved;
 } pml_hip_gemm_desc;
 
 int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* desc); /* 0 on failure */
@@ -271,7 +279,7 @@ typedef struct {
   int32_t init_dtype;
   int64_t init_row_stride, init_col_stride;
   int32_t c_dtype;
-  int32_t reserved;
+  int32_t flags; /* PML_HIP_FP32_AS_BF16X3 or 0 (see the GEMM descriptor) */
   pml_hip_epilogue tail;
 } pml_hip_conv2d_desc;
 

@@ -37,6 +37,7 @@ namespace pml {
 hipError_t igemm_launch_kind_0(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 hipError_t igemm_launch_kind_1(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 hipError_t igemm_launch_kind_2(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
+hipError_t igemm_launch_kind_3(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 
 namespace {
 
@@ -384,6 +385,10 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   constexpr int kOutstanding = (kStages - 2) * kLoads;  // requests that may still be in flight at the sync point
   constexpr int kSlots = MI * NI;
   i32x4_t fa[2][MI], fb[2][NI];
+  // fp32 as three bf16 products: a pair of K-blocks (8 fp32 values per lane and fragment) is split into bf16 heads
+  // and remainders at its second block and multiplied there; the first block of a pair only fetches
+  i32x4_t xa_head[KIND == KIND_F32X3 ? MI : 1], xa_rem[KIND == KIND_F32X3 ? MI : 1];
+  i32x4_t xb_head[KIND == KIND_F32X3 ? NI : 1], xb_rem[KIND == KIND_F32X3 ? NI : 1];
   const unsigned char* a_base = smem + (wm * WM + frow) * kSlabBytes;
   const unsigned char* b_base = smem + (BM + wn * WN + frow) * kSlabBytes;
   __builtin_amdgcn_s_waitcnt(0x0F70 | (((kStages - 1) * kLoads) & 15) | ((((kStages - 1) * kLoads) >> 4) << 14));
@@ -427,10 +432,21 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       const unsigned char* ra_ = last ? a_next : a_base;
       const unsigned char* rb_ = last ? b_next : b_base;
       const int fs = fslot[last ? 0 : kb + 1];
+      if constexpr (KIND == KIND_F32X3) {
+        if (cur == 1) {
+#pragma unroll
+          for (int i = 0; i < MI; ++i) split_f32x8(fa[0][i], fa[1][i], xa_head[i], xa_rem[i]);
+#pragma unroll
+          for (int j = 0; j < NI; ++j) split_f32x8(fb[0][j], fb[1][j], xb_head[j], xb_rem[j]);
+        }
+      }
 #pragma unroll
       for (int m = 0; m < kSlots; ++m) {
         if constexpr (ABL & 4) {
           asm volatile("" ::"v"(fb[cur][m % NI]), "v"(fa[cur][m / NI]));
+        } else if constexpr (KIND == KIND_F32X3) {
+          // (Bt's fragment is the row operand, as in mma_block)
+          if (cur == 1) mma_split(acc[m / NI][m % NI], xb_head[m % NI], xb_rem[m % NI], xa_head[m / NI], xa_rem[m / NI]);
         } else {
           mma_block<KIND>(acc[m / NI][m % NI], fb[cur][m % NI], fa[cur][m / NI]);
         }
@@ -635,10 +651,24 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_128x128: return launch_cfg<KIND, 128, 128, 2, CONV>(a, s);
     case TILE_128x64_W8: return launch_cfg<KIND, 128, 64, 4, CONV, 512>(a, s);
     case TILE_128x128_W8: return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
-    case TILE_256x128_W16: return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
-    case TILE_128x128_W8_S2: return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
+    case TILE_128x128_W8_S2:
+      // (128 registers do not hold the split kind's fragments: it takes the one-workgroup-per-CU form)
+      if constexpr (KIND == KIND_F32X3) {
+        return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
+      } else {
+        return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
+      }
     case TILE_64x64_W8_K2: return launch_cfg<KIND, 64, 64, 2, CONV, 512, 0, 2>(a, s);
-    case TILE_256x256_W8: return launch_cfg<KIND, 256, 256, 2, CONV, 512>(a, s);
+    case TILE_256x128_W16:
+    case TILE_256x256_W8:
+      // (the split fp32 kind keeps heads and remainders of every fragment in registers beside the raw values:
+      // the largest tiles are not built for it)
+      if constexpr (KIND == KIND_F32X3) {
+        return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
+      } else {
+        if (cfg == TILE_256x128_W16) return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
+        return launch_cfg<KIND, 256, 256, 2, CONV, 512>(a, s);
+      }
   }
   return hipErrorInvalidValue;
 #endif
@@ -647,7 +677,7 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
 }  // namespace
 
 #ifndef PML_KIND
-#error "compile with -DPML_KIND=0|1|2 (fp32 | bf16 | int8); -DPML_KIND=0 also emits the shared entry points"
+#error "compile with -DPML_KIND=0|1|2|3 (fp32 | bf16 | int8 | fp32 as three bf16 products); -DPML_KIND=0 also emits the shared entry points"
 #endif
 
 // One translation unit per element kind keeps each compile short and lets make run them in parallel.
@@ -743,6 +773,7 @@ hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStr
     case KIND_F32: return igemm_launch_kind_0(cfg, conv, a, s);
     case KIND_BF16: return igemm_launch_kind_1(cfg, conv, a, s);
     case KIND_I8: return igemm_launch_kind_2(cfg, conv, a, s);
+    case KIND_F32X3: return igemm_launch_kind_3(cfg, conv, a, s);
   }
   return hipErrorInvalidValue;
 }

@@ -38,6 +38,11 @@ struct Acc<KIND_I8> {
   typedef i32x16_t type;
   typedef int scalar;
 };
+template <>
+struct Acc<KIND_F32X3> {
+  typedef f32x16_t type;
+  typedef float scalar;
+};
 
 template <int KIND>
 __device__ inline void mma_block(typename Acc<KIND>::type& acc, const i32x4_t& a, const i32x4_t& b);
@@ -59,6 +64,41 @@ __device__ inline void mma_block<KIND_F32>(f32x16_t& acc, const i32x4_t& a, cons
   for (int j = 0; j < 4; ++j) {
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[j]), __int_as_float(b[j]), acc, 0, 0, 0);
   }
+}
+
+// fp32 on the bf16 matrix pipe.  Eight fp32 values (two 16-byte fragments) become a bf16 "head" (round to nearest
+// even) and a bf16 "remainder" (the rounded difference): x = head + remainder to about 2^-17 |x|.
+__device__ __forceinline__ void split_f32x8(const i32x4_t& r0, const i32x4_t& r1, i32x4_t& head, i32x4_t& rem) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float x0 = __int_as_float(q < 2 ? r0[2 * q] : r1[2 * q - 4]);
+    const float x1 = __int_as_float(q < 2 ? r0[2 * q + 1] : r1[2 * q - 3]);
+    const bf16x2 h = __builtin_convertvector(f32x2{x0, x1}, bf16x2);
+    uint32_t hb;
+    __builtin_memcpy(&hb, &h, 4);
+    head[q] = (int)hb;
+    const float d0 = x0 - __uint_as_float(hb << 16), d1 = x1 - __uint_as_float(hb & 0xffff0000u);
+    const bf16x2 l = __builtin_convertvector(f32x2{d0, d1}, bf16x2);
+    uint32_t lb;
+    __builtin_memcpy(&lb, &l, 4);
+    rem[q] = (int)lb;
+  }
+}
+
+// acc += a . b with a = a_head + a_rem, b = b_head + b_rem, the product of the two remainders dropped (2^-16 of the
+// term).  The small products go first.
+__device__ __forceinline__ void mma_split(f32x16_t& acc, const i32x4_t& a_head, const i32x4_t& a_rem, const i32x4_t& b_head,
+                                          const i32x4_t& b_rem) {
+  bf16x8_t ah, ar, bh, br;
+  __builtin_memcpy(&ah, &a_head, 16);
+  __builtin_memcpy(&ar, &a_rem, 16);
+  __builtin_memcpy(&bh, &b_head, 16);
+  __builtin_memcpy(&br, &b_rem, 16);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ar, bh, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, br, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh, acc, 0, 0, 0);
 }
 
 // Residual rows of a tile requested ahead of its K loop (tail_mode 2, at most 8 rows per thread):

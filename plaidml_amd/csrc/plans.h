@@ -31,7 +31,9 @@ struct DynamicLdsLimit {
 };
 
 
-enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2 };
+// KIND_F32X3: fp32 operands in memory and in LDS, each split in registers into a bf16 head and a bf16 remainder and
+// multiplied as three bf16 products (head x head + remainder x head + head x remainder), fp32 accumulation
+enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2, KIND_F32X3 = 3 };
 // _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages; _K2: two wavefront grids share the K-blocks of every slab
 enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2, TILE_64x64_W8_K2, TILE_256x256_W8 };
 

@@ -66,9 +66,9 @@ struct Plan {
   }
 };
 
-int mfma_kind_of(int in_dtype) {
+int mfma_kind_of(int in_dtype, int flags = 0) {
   switch (in_dtype) {
-    case PML_HIP_F32: return KIND_F32;
+    case PML_HIP_F32: return (flags & PML_HIP_FP32_AS_BF16X3) ? KIND_F32X3 : KIND_F32;
     case PML_HIP_BF16: return KIND_BF16;
     case PML_HIP_I8: return KIND_I8;
   }
@@ -130,6 +130,14 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, boo
     if (v == "256x256w8") return TILE_256x256_W8;
   }
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+  if (kind == KIND_F32X3) {
+    // Every fragment costs 24 vector instructions to split, whatever it is multiplied with: the tile a wavefront
+    // holds decides how many MFMAs share that cost.  128x128 with four wavefronts (64x64 each: 4 fragments, 12
+    // MFMAs per pair of K-blocks) where it still fills the chip, 128x64 (3 fragments, 6 MFMAs) below that.
+    if (n > 64 && tiles(128, 128) >= 192) return TILE_128x128;
+    if (tiles(128, 64) >= 192) return TILE_128x64;
+    return TILE_64x64;
+  }
   if (n <= 64) return TILE_64x64;  // (the 7x7 stem of ResNet-50 over 2x2 pixel blocks: 191 us against 207 us with 128x64w8)
   // Long K, at least three quarters of a round of 256x256 tiles and little of them hanging over the edges:
   // eight wavefronts of 128x64 (0.75 KB of LDS fragment reads per MFMA instead of 1.5).  Measured with N(0,1) /
@@ -250,7 +258,8 @@ int tail_scale_shift(const pml_hip_epilogue& t, int out_dtype, int mode) {
   return t.n_ops - 1;
 }
 
-bool valid_tail(const pml_hip_epilogue& t) {
+// allow64: the standalone elementwise kernel also runs 64-bit steps; the tails of the contraction kernels do not
+bool valid_tail(const pml_hip_epilogue& t, bool allow64 = false) {
   if (t.n_ops < 0 || t.n_ops > PML_HIP_MAX_EPI_OPS) return false;
   if (t.n_operands < 0 || t.n_operands > PML_HIP_MAX_EPI_OPERANDS) return false;
   for (int i = 0; i < t.n_ops; ++i) {
@@ -258,7 +267,7 @@ bool valid_tail(const pml_hip_epilogue& t) {
     if (op.opcode < PML_HIP_EPI_ADD || op.opcode > PML_HIP_EPI_LAST_) return false;
     if (op.operand_kind == PML_HIP_OPND_TENSOR && (op.operand < 0 || op.operand >= t.n_operands)) return false;
     if (op.opcode == PML_HIP_EPI_STORE && (op.operand < 0 || op.operand >= PML_HIP_MAX_EPI_OPERANDS)) return false;
-    if (dt_size(op.dtype) == 8 && op.opcode != PML_HIP_EPI_STORE) return false;  // 64-bit steps: general path only
+    if (!allow64 && dt_size(op.dtype) == 8 && op.opcode != PML_HIP_EPI_STORE) return false;  // 64-bit steps: general path only
   }
   return true;
 }
@@ -481,7 +490,7 @@ static int gemm_desc_kind(const pml_hip_gemm_desc* d) {
     fail("null descriptor");
     return -1;
   }
-  const int kind = mfma_kind_of(d->in_dtype);
+  const int kind = mfma_kind_of(d->in_dtype, d->flags);
   if (kind < 0) {
     fail("gemm: in_dtype must be F32, BF16 or I8");
     return -1;
@@ -490,6 +499,10 @@ static int gemm_desc_kind(const pml_hip_gemm_desc* d) {
                                         : (d->out_dtype == PML_HIP_F32 || (kind == KIND_BF16 && d->out_dtype == PML_HIP_BF16));
   if (!out_ok) {
     fail("gemm: out_dtype does not fit in_dtype");
+    return -1;
+  }
+  if ((d->flags & ~PML_HIP_FP32_AS_BF16X3) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32)) {
+    fail("gemm: flags may only hold PML_HIP_FP32_AS_BF16X3, and only with in_dtype F32");
     return -1;
   }
   if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->lda < d->k || d->ldb < (d->b_layout ? d->k : d->n) || d->ldc < d->n ||
@@ -556,7 +569,7 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   char buf[256];
   std::snprintf(buf, sizeof buf, "gemm %s m=%lld n=%lld k=%lld tile=%s mfma=%s", d->in_dtype == PML_HIP_F32 ? "f32" : d->in_dtype == PML_HIP_BF16 ? "bf16" : "i8",
                 (long long)d->m, (long long)d->n, (long long)d->k, tile_name(p->tile),
-                kind == KIND_F32 ? "f32_32x32x2" : kind == KIND_BF16 ? "f32_32x32x16_bf16" : "i32_32x32x32_i8");
+                kind == KIND_F32 ? "f32_32x32x2" : kind == KIND_BF16 ? "f32_32x32x16_bf16" : kind == KIND_I8 ? "i32_32x32x32_i8" : "3 x f32_32x32x16_bf16 (fp32 split into bf16 head + remainder)");
   p->text = buf;
   if (d->k2 > 0) p->text += " + second product k2=" + std::to_string(d->k2) + (d->a2_stride > 0 ? " over pixel rows of stride " + std::to_string(d->a2_stride) : "");
   return (int64_t)(intptr_t)p;
@@ -701,7 +714,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     fail("null descriptor");
     return 0;
   }
-  const int kind = mfma_kind_of(d->in_dtype);
+  const int kind = mfma_kind_of(d->in_dtype, d->flags);
   if (kind < 0) {
     fail("conv2d: in_dtype must be F32, BF16 or I8");
     return 0;
@@ -710,6 +723,10 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
                                         : (d->out_dtype == PML_HIP_F32 || (kind == KIND_BF16 && d->out_dtype == PML_HIP_BF16));
   if (!out_ok) {
     fail("conv2d: out_dtype does not fit in_dtype");
+    return 0;
+  }
+  if ((d->flags & ~PML_HIP_FP32_AS_BF16X3) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32)) {
+    fail("conv2d: flags may only hold PML_HIP_FP32_AS_BF16X3, and only with in_dtype F32");
     return 0;
   }
   if (d->n <= 0 || d->h <= 0 || d->w <= 0 || d->ci <= 0 || d->co <= 0 || d->kh <= 0 || d->kw <= 0 || d->oh <= 0 ||
@@ -739,7 +756,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   p->conv = *d;
   const int64_t M = d->n * d->oh * d->ow;
   const int64_t K = d->kh * d->kw * d->ci;
-  p->tile = choose_tile(M, d->co, K * es);
+  p->tile = choose_tile(M, d->co, K * es, kind, false);
   p->bt_ld = K;
   if (via_s2d) {
     const int v = 16 / es;
@@ -749,7 +766,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     p->s2d_ka = (int)(d->kh + (d->pad_h & 1) + 1) / 2;
     p->s2d_kaw = (int)(d->kw + (d->pad_w & 1) + 1) / 2;
     const int64_t k2 = (int64_t)p->s2d_ka * p->s2d_kaw * p->s2d_ch;
-    p->tile = choose_tile(M, d->co, k2 * es);
+    p->tile = choose_tile(M, d->co, k2 * es, kind, false);
     p->bt_ld = k2;
     // 256 spare bytes: a K-run that starts left of the image is addressed (never read) below the buffer's end only
     if (hipMalloc(&p->s2d, (size_t)d->n * p->s2d_h * p->s2d_w * p->s2d_ch * es + 256) != hipSuccess) {
@@ -780,7 +797,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     const char* e = std::getenv("PML_HIP_CONV");
     int dev = 0;
     hipDeviceProp_t prop;
-    if (!odd_channels && !(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
+    if (!odd_channels && kind != KIND_F32X3 && !(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
         hipGetDeviceProperties(&prop, dev) == hipSuccess) {
       IgemmArgs g;
       conv_args(p, g);
@@ -800,6 +817,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
                 (long long)d->h, (long long)d->w, (long long)d->ci, (long long)d->kh, (long long)d->kw, (long long)d->co,
                 (long long)d->oh, (long long)d->ow, (long long)M, (long long)d->co, (long long)K, p->halo_lds ? (p->halo_variant == 3 ? "256x64 resident filter, in registers" : p->halo_variant ? "256x64 resident filter, pipelined 3x3" : "256x64 resident filter") : tile_name(p->tile));
   p->text = buf;
+  if (kind == KIND_F32X3) p->text += " mfma=3 x f32_32x32x16_bf16 (fp32 split into bf16 head + remainder)";
   if (via_patches) p->text += " via patch matrix (k padded to " + std::to_string(p->kpad) + ")";
   if (via_s2d)
     p->text += " over 2x2 pixel blocks (" + std::to_string(p->s2d_ka) + "x" + std::to_string(p->s2d_kaw) + " block taps of " +
@@ -1057,7 +1075,7 @@ int64_t pml_hip_eltwise_dispatch(const pml_hip_eltwise_desc* d) {
     fail("eltwise: malformed tail");
     return 0;
   }
-  if (!valid_tail(t)) {
+  if (!valid_tail(t, /*allow64=*/true)) {
     fail("eltwise: a step of the chain names an unknown operation or an operand outside the operand list");
     return 0;
   }

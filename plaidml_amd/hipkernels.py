@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libpml_hip.so')
 
 # element types (values of plaidml_datatype, bfloat16 appended)
 BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, F32, F64, BF16 = 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16
+FP32_AS_BF16X3 = 1  # descriptor flag of gemm / conv2d: fp32 operands multiplied as three bf16 products
 AGG_ASSIGN, AGG_ADD, AGG_MAX, AGG_MIN, AGG_MUL = 0, 1, 2, 3, 4
 COMBO_NONE, COMBO_ADD, COMBO_COND, COMBO_EQ, COMBO_MUL = 0, 1, 2, 3, 4
 (EPI_ADD, EPI_SUB, EPI_RSUB, EPI_MUL, EPI_DIV, EPI_RDIV, EPI_MAX, EPI_MIN, EPI_RELU, EPI_NEG, EPI_EXP, EPI_LOG,
@@ -54,7 +55,7 @@ class GemmDesc(ctypes.Structure):
                 ('ldc', i64), ('init_kind', i32), ('init_dtype', i32), ('init_row_stride', i64),
                 ('init_col_stride', i64), ('c_dtype', i32), ('b_layout', i32), ('tail', Epilogue),
                 ('k2', i64), ('lda2', i64), ('ldb2', i64), ('a2_stride', i32), ('init2_kind', i32),
-                ('a2_h', i64), ('a2_w', i64), ('a2_oh', i64), ('a2_ow', i64)]
+                ('a2_h', i64), ('a2_w', i64), ('a2_oh', i64), ('a2_ow', i64), ('flags', i32), ('reserved', i32)]
 
 
 class Conv2dDesc(ctypes.Structure):
@@ -62,7 +63,7 @@ class Conv2dDesc(ctypes.Structure):
                 ('kw', i64), ('co', i64), ('oh', i64), ('ow', i64), ('stride_h', i64), ('stride_w', i64),
                 ('dil_h', i64), ('dil_w', i64), ('pad_h', i64), ('pad_w', i64), ('init_kind', i32),
                 ('init_dtype', i32), ('init_row_stride', i64), ('init_col_stride', i64), ('c_dtype', i32),
-                ('reserved', i32), ('tail', Epilogue)]
+                ('flags', i32), ('tail', Epilogue)]
 
 
 class Dwconv2dDesc(ctypes.Structure):

@@ -172,6 +172,12 @@ void compileProgram(tile::Program* program, const std::string& requested, bool /
   if (opts.count("fuse")) options.fuse = truthy(opts["fuse"]);
   if (opts.count("specialise")) options.specialise = truthy(opts["specialise"]);
   if (opts.count("specialize")) options.specialise = truthy(opts["specialize"]);
+  if (opts.count("fp32")) {
+    if (opts["fp32"] == "bf16x3")
+      options.fp32_as_bf16x3 = true;
+    else if (opts["fp32"] != "mfma")
+      throw std::runtime_error("Invalid target option fp32=" + opts["fp32"] + " (mfma or bf16x3)");
+  }
   program->passes.resize(1);  // keep only the "tile" text when compiling again
   tile::foldAddIntoInit(program);
   program->passes.emplace_back("tile-algebraic-opt", program->str());

@@ -1147,6 +1147,7 @@ class Planner {
     d.ldb = ldb;
     d.ldc = ldc;
     d.b_layout = b_is_nk ? 1 : 0;
+    if (opt_.fp32_as_bf16x3 && in_dt == PML_HIP_F32) d.flags = PML_HIP_FP32_AS_BF16X3;
     if (!denseInit(op, &d.init_kind, &d.init_dtype, &d.init_row_stride, &d.init_col_stride, &s.init)) return false;
     // the tail and the row/col operand addressing assume a dense rows x cols output
     TailBuild tb;
@@ -1169,8 +1170,8 @@ class Planner {
     s.flops = 2.0 * m * nn * kk;
     s.bytes = static_cast<double>(m * kk + kk * nn) * es + static_cast<double>(m * nn) * util::byteSize(tb.final_dtype);
     std::stringstream ss;
-    ss << "gemm " << util::mnemonic(static_cast<DataType>(in_dt)) << " m=" << m << " n=" << nn << " k=" << kk
-       << (b_is_nk ? " B=[n][k]" : " B=[k][n]") << (s.b_constant ? " (constant, packed once)" : "")
+    ss << "gemm " << util::mnemonic(static_cast<DataType>(in_dt)) << (d.flags & PML_HIP_FP32_AS_BF16X3 ? " (as 3 bf16 products)" : "")
+       << " m=" << m << " n=" << nn << " k=" << kk << (b_is_nk ? " B=[n][k]" : " B=[k][n]") << (s.b_constant ? " (constant, packed once)" : "")
        << (d.init_kind ? " +init" : "") << tailText(tb) << " -> " << tb.final_value->shape.str();
     s.text = ss.str();
     plan_->steps.push_back(s);
@@ -1280,6 +1281,7 @@ class Planner {
     d.dil_w = sx.dil;
     d.pad_h = sy.pad;
     d.pad_w = sx.pad;
+    if (opt_.fp32_as_bf16x3 && in_dt == PML_HIP_F32) d.flags = PML_HIP_FP32_AS_BF16X3;
     if (os.sizes[0] != d.n) return false;
     if (!denseInit(op, &d.init_kind, &d.init_dtype, &d.init_row_stride, &d.init_col_stride, &s.init)) return false;
     TailBuild tb;
@@ -1305,7 +1307,7 @@ class Planner {
               d.ci * d.co;
     s.bytes = static_cast<double>(is.elements() + fs.elements()) * es + static_cast<double>(os.elements()) * util::byteSize(tb.final_dtype);
     std::stringstream ss;
-    ss << "conv2d " << util::mnemonic(static_cast<DataType>(in_dt)) << " " << is.str() << " (*) " << fs.str() << " stride=" << d.stride_h
+    ss << "conv2d " << util::mnemonic(static_cast<DataType>(in_dt)) << (d.flags & PML_HIP_FP32_AS_BF16X3 ? " (as 3 bf16 products) " : " ") << is.str() << " (*) " << fs.str() << " stride=" << d.stride_h
        << "x" << d.stride_w << " pad=" << d.pad_h << "," << d.pad_w << (s.b_constant ? " (constant filter, packed once)" : "")
        << (d.init_kind ? " +init" : "") << tailText(tb) << " -> " << tb.final_value->shape.str();
     s.text = ss.str();

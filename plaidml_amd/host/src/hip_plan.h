@@ -72,6 +72,9 @@ struct Plan {
 struct Options {
   bool fuse = true;        // fold elementwise consumers into kernel tails
   bool specialise = true;  // use the MFMA / window kernels; false = every contraction through the general kernel
+  // fp32 GEMMs and convolutions on the bf16 matrix cores, every operand value split into a bf16 head and a bf16
+  // remainder (three products per term, about 2^-16 relative error per product): `hip{fp32=bf16x3}`
+  bool fp32_as_bf16x3 = false;
 };
 
 // Runs the pipeline on a copy of the program's op list and returns the plan.

@@ -69,6 +69,19 @@ def test_operand_of_two_gib_takes_the_general_kernel():
     assert 'gemm f32' in plan_of(E.Program('dot', [A, B], [op.dot(A, B)]))
 
 
+def test_target_option_fp32_as_three_bf16_products():
+    prog = programs.config1_conv(E, op, 'FLOAT32')[0]
+    assert 'as 3 bf16 products' not in plan_of(prog)
+    prog = programs.config1_conv(E, op, 'FLOAT32')[0]
+    assert 'conv2d f32 (as 3 bf16 products)' in plan_of(prog, 'hip{fp32=bf16x3}')
+    prog = programs.config1_conv(E, op, 'BFLOAT16')[0]
+    assert 'as 3 bf16 products' not in plan_of(prog, 'hip{fp32=bf16x3}')   # bf16 programs are not touched
+    prog = programs.config0_gemm_f32(E, op)[0]
+    assert 'gemm f32 (as 3 bf16 products)' in plan_of(prog, 'hip{fp32=bf16x3}')
+    with pytest.raises(E.PlaidMLError, match='Invalid target option fp32'):
+        programs.config0_gemm_f32(E, op)[0].compile('hip{fp32=tf32}')
+
+
 def test_target_options_switch_specialisation_off():
     prog = programs.config1_conv(E, op, 'BFLOAT16')[0]
     t = plan_of(prog, 'hip{specialise=0,fuse=0}')

@@ -29,11 +29,12 @@ def bf16(a):
 
 
 def run_gemm(A, B, in_dt, out_dt, init=None, init_strides=(0, 0), init_dt=0, tail=None, operands=(), c_dt=None,
-             extra_out=None):
+             extra_out=None, flags=0):
     M, K = A.shape
     _, N = B.shape
     d = hk.GemmDesc()
     d.in_dtype, d.out_dtype = in_dt, out_dt
+    d.flags = flags
     d.m, d.n, d.k = M, N, K
     d.lda, d.ldb, d.ldc = K, N, N
     d.c_dtype = c_dt if c_dt is not None else out_dt
@@ -111,6 +112,29 @@ def test_every_tile_configuration(tile, monkeypatch):
     B32 = rng.uniform(-1, 1, (K, N)).astype(np.float32)
     np.testing.assert_allclose(run_gemm(A32, B32, hk.F32, hk.F32), A32.astype(np.float64) @ B32.astype(np.float64),
                                rtol=FP32_RTOL, atol=1e-3)
+    np.testing.assert_allclose(run_gemm(A32, B32, hk.F32, hk.F32, flags=hk.FP32_AS_BF16X3),
+                               A32.astype(np.float64) @ B32.astype(np.float64), rtol=FP32_RTOL, atol=1e-3)
+
+
+@pytest.mark.parametrize('M,N,K', [(1024, 1024, 1024), (257, 130, 68), (256, 384, 4096)])
+def test_gemm_f32_as_three_bf16_products(M, N, K):
+    """fp32 operands split into bf16 head + remainder in registers, three bf16 MFMAs per term.  U(-1, 1) operands make
+    every result a sum of K terms of both signs (K = 4096: results of size ~21 from terms of size ~1/3), the case
+    where a lost low part shows; the bar is fp32's own (rtol 1e-3).  What the split drops is bounded as well: the
+    largest deviation from float64 stays below 4 x 2^-16 x sqrt(K) x E|ab|."""
+    rng = np.random.default_rng(41)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tail = hk.make_tail(ops=[(hk.EPI_RELU, hk.F32, 0, 0, 0.0)])
+    C = run_gemm(A, B, hk.F32, hk.F32, init=bias, init_strides=(0, 1), init_dt=hk.F32, tail=tail, flags=hk.FP32_AS_BF16X3)
+    ref = np.maximum(A.astype(np.float64) @ B.astype(np.float64) + bias, 0)
+    np.testing.assert_allclose(C, ref, rtol=FP32_RTOL, atol=1e-3)
+    assert np.abs(C - ref).max() < 4 * 2.0 ** -16 * np.sqrt(K) * 0.25 + 1e-5
+    # values a bf16 holds exactly go through unchanged: small integers give the exact integer result
+    Ai = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    Bi = rng.integers(-8, 9, (K, N)).astype(np.float32)
+    np.testing.assert_array_equal(run_gemm(Ai, Bi, hk.F32, hk.F32, flags=hk.FP32_AS_BF16X3), Ai @ Bi)
 
 
 @pytest.mark.parametrize('stride', [0, 2])
@@ -266,7 +290,7 @@ def test_gemm_bf16(M, N, K):
 
 
 def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bias=None, relu=False, tail=None,
-             operands=()):
+             operands=(), flags=0):
     N, H, W, CI = I.shape
     KH, KW, _, CO = F.shape
     ph, OH = op.compute_padding_and_output_size(H, KH, stride, autopad)
@@ -276,6 +300,7 @@ def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bia
         OH, OW = (H + 2 * pad - KH) // stride + 1, (W + 2 * pad - KW) // stride + 1
     d = hk.Conv2dDesc()
     d.in_dtype, d.out_dtype, d.c_dtype = in_dt, out_dt, out_dt
+    d.flags = flags
     d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, KH, KW, CO, OH, OW
     d.stride_h = d.stride_w = stride
     d.dil_h = d.dil_w = 1
@@ -323,14 +348,31 @@ def oracle_conv(Iv, Fv, dt, stride, autopad, bias=None, relu=False, pad=None):
 
 @pytest.mark.parametrize('shape,k,stride,autopad', [((2, 12, 12, 32), 3, 1, op.SAME_UPPER), ((1, 9, 11, 64), 3, 2, op.SAME_UPPER),
                                                      ((2, 8, 8, 32), 1, 1, op.VALID), ((1, 14, 14, 32), 7, 2, op.SAME_UPPER)])
-def test_conv_f32(shape, k, stride, autopad):
+@pytest.mark.parametrize('flags', [0, hk.FP32_AS_BF16X3])
+def test_conv_f32(shape, k, stride, autopad, flags):
     rng = np.random.default_rng(7)
     Iv = rng.standard_normal(shape).astype(np.float32)
     Fv = (rng.standard_normal((k, k, shape[3], 48)) * 0.1).astype(np.float32)
     bias = rng.standard_normal(48).astype(np.float32)
-    out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, autopad=autopad, bias=bias, relu=True)
+    out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, autopad=autopad, bias=bias, relu=True, flags=flags)
     ref = oracle_conv(Iv, Fv, D.FLOAT32, stride, autopad, bias, True)
     np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4)
+
+
+def test_conv_f32_as_three_bf16_products_configs1_sampled():
+    """BASELINE configs[1] in fp32 at full size with the operands split into bf16 head + remainder: sampled pixels
+    against float64."""
+    rng = np.random.default_rng(2)
+    N, H, W, CI, CO = 128, 56, 56, 64, 64
+    Iv = rng.standard_normal((N, H, W, CI)).astype(np.float32)
+    Fv = (np.random.default_rng(3).standard_normal((3, 3, CI, CO)) * np.sqrt(2.0 / (9 * CI))).astype(np.float32)
+    bias = rng.standard_normal(CO).astype(np.float32)
+    out = run_conv(Iv, Fv, hk.F32, hk.F32, bias=bias, relu=True, flags=hk.FP32_AS_BF16X3)
+    Ip = np.pad(Iv, ((0, 0), (1, 1), (1, 1), (0, 0))).astype(np.float64)
+    for _ in range(200):
+        n, y, x = rng.integers(N), rng.integers(H), rng.integers(W)
+        ref = np.maximum(np.einsum('yxc,yxck->k', Ip[n, y:y + 3, x:x + 3], Fv.astype(np.float64)) + bias, 0)
+        np.testing.assert_allclose(out[n, y, x], ref, rtol=FP32_RTOL, atol=1e-4)
 
 
 @pytest.mark.parametrize('shape,k,stride,co', [((2, 14, 14, 64), 3, 1, 64), ((1, 10, 10, 128), 1, 2, 72), ((2, 7, 9, 64), 3, 2, 40)])

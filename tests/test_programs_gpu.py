@@ -107,10 +107,13 @@ def test_config3_full_size_against_oracle_on_a_slice():
     assert (M >= 0).all()                             # max over ReLU outputs
 
 
-def test_config0_full_size_against_float64():
-    """BASELINE configs[0] at full size through the plaidml API: fp32 1024^3, U(-1, 1), against float64 numpy."""
+@pytest.mark.parametrize('target', ['hip', 'hip{fp32=bf16x3}'])
+def test_config0_full_size_against_float64(target):
+    """BASELINE configs[0] at full size through the plaidml API: fp32 1024^3, U(-1, 1), against float64 numpy; with
+    fp32 MFMAs and with the operands split for the bf16 matrix cores (three products per term)."""
     prog, vals, _ = programs.config0_gemm_f32(E, op, n=1024)
-    C, = E.run(prog, vals, target='hip')
+    C, = E.run(prog, vals, target=target)
+    assert ('as 3 bf16 products' in dict(prog.passes)['hip-plan']) == ('bf16x3' in target)
     want = vals[0].astype(np.float64) @ vals[1].astype(np.float64)
     # rtol 1e-3 on the scale of a result row (entries are sums of 1024 terms of either sign: those near zero are
     # compared through atol = 1e-3 x the typical magnitude sqrt(1024 / 9))
@@ -118,14 +121,14 @@ def test_config0_full_size_against_float64():
     assert np.abs(C - want).max() < 1e-3                  # measured: a few 1e-5 (fp32 accumulation over 1024 terms)
 
 
-@pytest.mark.parametrize('dtype_name', ['FLOAT32', 'BFLOAT16'])
-def test_config1_full_size_through_exec(dtype_name):
+@pytest.mark.parametrize('dtype_name,target', [('FLOAT32', 'hip'), ('BFLOAT16', 'hip'), ('FLOAT32', 'hip{fp32=bf16x3}')])
+def test_config1_full_size_through_exec(dtype_name, target):
     """BASELINE configs[1] at full size (N128 56x56x64, 3x3x64x64, SAME, + bias + ReLU) through the plaidml API, in
     fp32 and in bf16: images do not interact, so images 0 and 127 must equal the oracle's result for a batch of
     those two; sampled pixels of every image are checked against float64 arithmetic on the same values."""
     print('configs[1] full size', dtype_name, flush=True)
     prog, vals, tol = programs.config1_conv(E, op, dtype_name, N=128, H=56, W=56)
-    O, = E.run(prog, vals, target='hip')
+    O, = E.run(prog, vals, target=target)
     assert O.shape == (128, 56, 56, 64)
     plan = dict(prog.passes)['hip-plan']
     assert 'conv2d' in plan and 'contract (general)' not in plan, plan
@@ -133,7 +136,7 @@ def test_config1_full_size_through_exec(dtype_name):
     ovals[0] = vals[0][[0, 127]]
     np.testing.assert_array_equal(ovals[1], vals[1])
     ref, = OE.run(oprog, ovals)
-    rtol, atol = (2e-2, 2e-2) if dtype_name == 'BFLOAT16' else (1e-3, 1e-5)
+    rtol, atol = (2e-2, 2e-2) if dtype_name == 'BFLOAT16' else (1e-3, 1e-4 if 'bf16x3' in target else 1e-5)
     np.testing.assert_allclose(O[[0, 127]], ref, rtol=rtol, atol=atol)
     Iv, Fv, Bv = (v.astype(np.float64) for v in vals)
     r = np.random.default_rng(12)
