@@ -38,6 +38,7 @@ hipError_t igemm_launch_kind_0(int cfg, bool conv, const IgemmArgs& a, hipStream
 hipError_t igemm_launch_kind_1(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 hipError_t igemm_launch_kind_2(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 hipError_t igemm_launch_kind_3(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
+hipError_t igemm_launch_kind_4(int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 
 namespace {
 
@@ -138,6 +139,8 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   constexpr int kSwzShift = SLAB == 128 ? 1 : 2;      // chunk u of row r sits in slot u ^ ((r >> shift) & (CPR - 1))
   static_assert(SLAB == 128 || SLAB == 64, "rows of 128 or 64 bytes");
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
+  constexpr bool kSplit = KIND == KIND_F32X3 || KIND == KIND_F32X3P;  // fp32 operands as three bf16 products
+  constexpr bool kSplitB = KIND == KIND_F32X3P;                       // ... the right-hand side split when it was packed
   constexpr int kWaves = NT / 64;
   constexpr int kRowsPerPass = NT / CPR;  // operand rows one load of all threads covers
   constexpr int WAVES_N = kWaves / WAVES_M / WAVES_K;
@@ -373,9 +376,22 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   const int frow = lane & 31;  // row of the 32x32 block this lane feeds
   // byte offset of its 16-byte half of each of the wavefront's 32-byte K-blocks, swizzled
   constexpr int kBlocks = kSlabBytes / 32 / WAVES_K;
-  int fslot[kBlocks];
+  // (fslot_b: the Bt fragment's; different only for the split fp32 kind.  That kind takes a pair of K-blocks as one
+  // bf16 MFMA step of 16 K-values, the lane's eight values being two neighbouring 16-byte chunks of the fp32 row;
+  // a right-hand side that was split when it was packed keeps, per 128 bytes of a row, the 32 bf16 heads in the
+  // first 64 bytes and the 32 remainders in the second, and the pair's two reads fetch one of each.)
+  int fslot[kBlocks], fslot_b[kBlocks];
 #pragma unroll
-  for (int kb = 0; kb < kBlocks; ++kb) fslot[kb] = (((wk * kBlocks + kb) * 2 + (lane >> 5)) ^ ((lane >> kSwzShift) & (CPR - 1))) * 16;
+  for (int kb = 0; kb < kBlocks; ++kb) {
+    const int gb = wk * kBlocks + kb, h = lane >> 5, key = (lane >> kSwzShift) & (CPR - 1);
+    if constexpr (kSplit) {
+      fslot[kb] = (((gb & ~1) * 2 + 2 * h + (gb & 1)) ^ key) * 16;
+      fslot_b[kb] = kSplitB ? ((((gb & 1) * 4 + (gb >> 1) * 2 + h) ^ key) * 16) : fslot[kb];
+    } else {
+      fslot[kb] = ((gb * 2 + h) ^ key) * 16;
+      fslot_b[kb] = fslot[kb];
+    }
+  }
 
   // The loop is rotated by one K-block: the one synchronisation point of a slab sits before its LAST
   // K-block, whose fragments are in registers by then.  Past it every wavefront is done reading this
@@ -387,8 +403,8 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   i32x4_t fa[2][MI], fb[2][NI];
   // fp32 as three bf16 products: a pair of K-blocks (8 fp32 values per lane and fragment) is split into bf16 heads
   // and remainders at its second block and multiplied there; the first block of a pair only fetches
-  i32x4_t xa_head[KIND == KIND_F32X3 ? MI : 1], xa_rem[KIND == KIND_F32X3 ? MI : 1];
-  i32x4_t xb_head[KIND == KIND_F32X3 ? NI : 1], xb_rem[KIND == KIND_F32X3 ? NI : 1];
+  i32x4_t xa_head[kSplit ? MI : 1], xa_rem[kSplit ? MI : 1];
+  i32x4_t xb_head[kSplit && !kSplitB ? NI : 1], xb_rem[kSplit && !kSplitB ? NI : 1];
   const unsigned char* a_base = smem + (wm * WM + frow) * kSlabBytes;
   const unsigned char* b_base = smem + (BM + wn * WN + frow) * kSlabBytes;
   __builtin_amdgcn_s_waitcnt(0x0F70 | (((kStages - 1) * kLoads) & 15) | ((((kStages - 1) * kLoads) >> 4) << 14));
@@ -396,7 +412,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
 #pragma unroll
   for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(a_base + i * 32 * kSlabBytes + fslot[0]);
 #pragma unroll
-  for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(b_base + j * 32 * kSlabBytes + fslot[0]);
+  for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(b_base + j * 32 * kSlabBytes + fslot_b[0]);
 
   int stage = 0;  // ring stage of slab s
   for (int s = 0; s < n_slabs; ++s) {
@@ -432,21 +448,31 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       const unsigned char* ra_ = last ? a_next : a_base;
       const unsigned char* rb_ = last ? b_next : b_base;
       const int fs = fslot[last ? 0 : kb + 1];
-      if constexpr (KIND == KIND_F32X3) {
+      const int fs_b = fslot_b[last ? 0 : kb + 1];
+      if constexpr (kSplit) {
         if (cur == 1) {
 #pragma unroll
           for (int i = 0; i < MI; ++i) split_f32x8(fa[0][i], fa[1][i], xa_head[i], xa_rem[i]);
+          if constexpr (!kSplitB) {
 #pragma unroll
-          for (int j = 0; j < NI; ++j) split_f32x8(fb[0][j], fb[1][j], xb_head[j], xb_rem[j]);
+            for (int j = 0; j < NI; ++j) split_f32x8(fb[0][j], fb[1][j], xb_head[j], xb_rem[j]);
+          }
         }
       }
 #pragma unroll
       for (int m = 0; m < kSlots; ++m) {
         if constexpr (ABL & 4) {
           asm volatile("" ::"v"(fb[cur][m % NI]), "v"(fa[cur][m / NI]));
-        } else if constexpr (KIND == KIND_F32X3) {
-          // (Bt's fragment is the row operand, as in mma_block)
-          if (cur == 1) mma_split(acc[m / NI][m % NI], xb_head[m % NI], xb_rem[m % NI], xa_head[m / NI], xa_rem[m / NI]);
+        } else if constexpr (kSplit) {
+          // (Bt's fragment is the row operand, as in mma_block; a packed right-hand side's two reads of the pair are
+          // its heads and its remainders)
+          if (cur == 1) {
+            if constexpr (kSplitB) {
+              mma_split(acc[m / NI][m % NI], fb[0][m % NI], fb[1][m % NI], xa_head[m / NI], xa_rem[m / NI]);
+            } else {
+              mma_split(acc[m / NI][m % NI], xb_head[m % NI], xb_rem[m % NI], xa_head[m / NI], xa_rem[m / NI]);
+            }
+          }
         } else {
           mma_block<KIND>(acc[m / NI][m % NI], fb[cur][m % NI], fa[cur][m / NI]);
         }
@@ -459,7 +485,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
           if (d < MI)
             fa[nxt][d] = *(const i32x4_t*)(ra_ + d * 32 * kSlabBytes + fs);
           else
-            fb[nxt][d - MI] = *(const i32x4_t*)(rb_ + (d - MI) * 32 * kSlabBytes + fs);
+            fb[nxt][d - MI] = *(const i32x4_t*)(rb_ + (d - MI) * 32 * kSlabBytes + fs_b);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -653,17 +679,25 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
     case TILE_128x128_W8: return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
     case TILE_128x128_W8_S2:
       // (128 registers do not hold the split kind's fragments: it takes the one-workgroup-per-CU form)
-      if constexpr (KIND == KIND_F32X3) {
+      if constexpr (KIND == KIND_F32X3 || KIND == KIND_F32X3P) {
         return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
       } else {
         return launch_cfg<KIND, 128, 128, 2, CONV, 512, 2>(a, s);
       }
     case TILE_64x64_W8_K2: return launch_cfg<KIND, 64, 64, 2, CONV, 512, 0, 2>(a, s);
+    case TILE_128x64_N2:
+      // four wavefronts side by side in M, each 32 rows x 64 columns: one left-hand fragment (the one that is split
+      // in registers) feeds six MFMAs.  Built for the split fp32 kind only.
+      if constexpr (KIND == KIND_F32X3 || KIND == KIND_F32X3P) {
+        return launch_cfg<KIND, 128, 64, 4, CONV>(a, s);
+      } else {
+        return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
+      }
     case TILE_256x128_W16:
     case TILE_256x256_W8:
       // (the split fp32 kind keeps heads and remainders of every fragment in registers beside the raw values:
       // the largest tiles are not built for it)
-      if constexpr (KIND == KIND_F32X3) {
+      if constexpr (KIND == KIND_F32X3 || KIND == KIND_F32X3P) {
         return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
       } else {
         if (cfg == TILE_256x128_W16) return launch_cfg<KIND, 256, 128, 4, CONV, 1024>(a, s);
@@ -677,7 +711,7 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
 }  // namespace
 
 #ifndef PML_KIND
-#error "compile with -DPML_KIND=0|1|2|3 (fp32 | bf16 | int8 | fp32 as three bf16 products); -DPML_KIND=0 also emits the shared entry points"
+#error "compile with -DPML_KIND=0|1|2|3|4 (fp32 | bf16 | int8 | fp32 as three bf16 products | the same, right-hand side split when packed); -DPML_KIND=0 also emits the shared entry points"
 #endif
 
 // One translation unit per element kind keeps each compile short and lets make run them in parallel.
@@ -774,8 +808,34 @@ hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStr
     case KIND_BF16: return igemm_launch_kind_1(cfg, conv, a, s);
     case KIND_I8: return igemm_launch_kind_2(cfg, conv, a, s);
     case KIND_F32X3: return igemm_launch_kind_3(cfg, conv, a, s);
+    case KIND_F32X3P: return igemm_launch_kind_4(cfg, conv, a, s);
   }
   return hipErrorInvalidValue;
+}
+
+// In place, per 32 fp32 values (128 bytes) of a row: their 32 bf16 heads (round to nearest even), then the 32 bf16
+// remainders (the rounded differences) -- the form the split fp32 kind reads a packed right-hand side in.
+__global__ __launch_bounds__(256) void split_rows_kernel(float* bt, int64_t rows, int64_t ld, int64_t chunks_per_row) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= rows * chunks_per_row) return;
+  i32x4_t* at = (i32x4_t*)(bt + (t / chunks_per_row) * ld + (t % chunks_per_row) * 32);
+  i32x4_t raw[8], head[4], rem[4];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) raw[u] = at[u];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) split_f32x8(raw[2 * u], raw[2 * u + 1], head[u], rem[u]);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    at[u] = head[u];
+    at[4 + u] = rem[u];
+  }
+}
+
+hipError_t split_rows_launch(void* bt, int64_t rows, int64_t ld, int64_t k, hipStream_t s) {
+  if (k % 32 != 0 || ld % 4 != 0 || ((uintptr_t)bt & 15) != 0) return hipErrorInvalidValue;
+  const int64_t chunks = k / 32, total = rows * chunks;
+  hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (float*)bt, rows, ld, chunks);
+  return hipGetLastError();
 }
 
 hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int64_t N, int64_t ldb, int64_t ldbt,

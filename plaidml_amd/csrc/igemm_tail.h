@@ -43,6 +43,11 @@ struct Acc<KIND_F32X3> {
   typedef f32x16_t type;
   typedef float scalar;
 };
+template <>
+struct Acc<KIND_F32X3P> {
+  typedef f32x16_t type;
+  typedef float scalar;
+};
 
 template <int KIND>
 __device__ inline void mma_block(typename Acc<KIND>::type& acc, const i32x4_t& a, const i32x4_t& b);

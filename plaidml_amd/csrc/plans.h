@@ -33,9 +33,11 @@ struct DynamicLdsLimit {
 
 // KIND_F32X3: fp32 operands in memory and in LDS, each split in registers into a bf16 head and a bf16 remainder and
 // multiplied as three bf16 products (head x head + remainder x head + head x remainder), fp32 accumulation
-enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2, KIND_F32X3 = 3 };
+// KIND_F32X3P: the same with a right-hand side that was split when it was packed (per 32 K-values of a row of Bt:
+// their 32 bf16 heads, then their 32 bf16 remainders), so that only the left-hand fragments are split in registers
+enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2, KIND_F32X3 = 3, KIND_F32X3P = 4 };
 // _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages; _K2: two wavefront grids share the K-blocks of every slab
-enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2, TILE_64x64_W8_K2, TILE_256x256_W8 };
+enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2, TILE_64x64_W8_K2, TILE_256x256_W8, TILE_128x64_N2 };
 
 struct TailPtrs {
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
@@ -109,6 +111,8 @@ hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStr
 size_t conv_halo_prepare(int kind, IgemmArgs* a);
 hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s);
 hipError_t mfma_probe_launch(int blocks, int iters, int random, float* sink, unsigned long long* clk, hipStream_t s);
+// splits a packed fp32 Bt[rows][ld] in place (k values per row, a multiple of 32) into the heads / remainders form
+hipError_t split_rows_launch(void* bt, int64_t rows, int64_t ld, int64_t k, hipStream_t s);
 hipError_t transpose_pack(int elem_size, const void* B, void* Bt, int64_t K, int64_t N, int64_t ldb, int64_t ldbt,
                           hipStream_t s);
 

@@ -44,6 +44,8 @@ struct Plan {
   int64_t bt_ld = 0;
   size_t bt_bytes = 0;
   bool packed = false;
+  bool b_split = false;  // split fp32 kind: a right-hand side packed once is kept as bf16 heads + remainders
+  bool bt_is_split = false;  // ... and `bt` holds that form now
   // second product of a GEMM: its packed right-hand side Bt2[N][K2]
   void* bt2 = nullptr;
   bool packed2 = false;
@@ -85,6 +87,7 @@ const char* tile_name(int t) {
     case TILE_256x128_W16: return "256x128 (16 wavefronts)";
     case TILE_64x64_W8_K2: return "64x64 (8 wavefronts, K split in two)";
     case TILE_256x256_W8: return "256x256 (8 wavefronts of 128x64)";
+    case TILE_128x64_N2: return "128x64 (4 wavefronts of 32x64)";
     case TILE_128x128_W8_S2: return "128x128 (8 wavefronts, 2 stages)";
   }
   return "?";
@@ -116,7 +119,7 @@ const char* tile_name(int t) {
 // that; and for small problems the smaller of 64x64 and 128x64 by (rounds of resident workgroups) x
 // (tile area), the larger tile on a tie.
 int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, bool plain_tail = true) {
-  // PML_HIP_TILE=64x64|64x64w8k2|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16|256x256w8 overrides the table (for tuning runs)
+  // PML_HIP_TILE=64x64|64x64w8k2|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16|256x256w8|128x64n2 overrides the table (for tuning runs)
   if (const char* e = std::getenv("PML_HIP_TILE")) {
     const std::string v(e);
     if (v == "64x64") return TILE_64x64;
@@ -128,14 +131,16 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, boo
     if (v == "256x128w16") return TILE_256x128_W16;
     if (v == "64x64w8k2") return TILE_64x64_W8_K2;
     if (v == "256x256w8") return TILE_256x256_W8;
+    if (v == "128x64n2" && kind == KIND_F32X3) return TILE_128x64_N2;
   }
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (kind == KIND_F32X3) {
-    // Every fragment costs 24 vector instructions to split, whatever it is multiplied with: the tile a wavefront
-    // holds decides how many MFMAs share that cost.  128x128 with four wavefronts (64x64 each: 4 fragments, 12
-    // MFMAs per pair of K-blocks) where it still fills the chip, 128x64 (3 fragments, 6 MFMAs) below that.
-    if (n > 64 && tiles(128, 128) >= 192) return TILE_128x128;
-    if (tiles(128, 64) >= 192) return TILE_128x64;
+    // A fragment that is split in registers costs 24 vector instructions whatever it is multiplied with, so the
+    // tile a wavefront holds decides how many MFMAs share that cost -- but the problems this kind meets here are
+    // short of tiles first.  Measured: configs[1] fp32 (n = 64) 137 us with 64x64, 146 with 128x64 as 32x64 per
+    // wavefront, 155 with 128x64 as 64x32; 1024^3 25-27 us with 64x64 (either form), 34-47 with larger tiles.
+    if (n > 64 && tiles(128, 128) >= 512) return TILE_128x128;
+    if (tiles(64, 64) <= 512 && k_bytes >= 2048) return TILE_64x64_W8_K2;
     return TILE_64x64;
   }
   if (n <= 64) return TILE_64x64;  // (the 7x7 stem of ResNet-50 over 2x2 pixel blocks: 191 us against 207 us with 128x64w8)
@@ -390,7 +395,9 @@ hipError_t pack_conv_filter(Plan* p, const void* filter, hipStream_t s) {
     a.gt = p->bt;
     return s2d_filter_launch(es, a, s);
   }
-  return transpose_pack(es, filter, p->bt, d.kh * d.kw * d.ci, d.co, d.co, p->bt_ld, s);
+  if (hipError_t e = transpose_pack(es, filter, p->bt, d.kh * d.kw * d.ci, d.co, d.co, p->bt_ld, s); e != hipSuccess) return e;
+  if (p->b_split) return split_rows_launch(p->bt, d.co, p->bt_ld, d.kh * d.kw * d.ci, s);
+  return hipSuccess;
 }
 
 }  // namespace
@@ -556,6 +563,7 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
+  p->b_split = kind == KIND_F32X3 && !d->b_layout && d->k % 32 == 0;
   if (!d->b_layout && hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
     delete p;
     fail("gemm: cannot allocate the packed right-hand side");
@@ -588,7 +596,10 @@ struct SecondProduct {
 
 static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* bt, int64_t bt_ld, bool packed,
                     const void* a, const void* b, void* c, const void* init, const void* const* operands,
-                    void* const* outs, pml_hip_stream s, const SecondProduct* second = nullptr) {
+                    void* const* outs, pml_hip_stream s, const SecondProduct* second = nullptr, bool bt_is_split = false) {
+  // (a right-hand side that arrives with the call is transposed per run and split in the kernel's registers: a
+  // second small launch costs more than it saves; one packed once is kept split)
+  const bool b_split = bt_is_split && !b;
   if (!a || !c) return fail("gemm_invoke: null operand");
   if (!b && (!packed || d.b_layout)) return fail("gemm_invoke: b is null and no packed right-hand side exists");
   if (d.b_layout && ((uintptr_t)b & 15) != 0) return fail("gemm_invoke: an [N][K] right-hand side must be 16-byte aligned");
@@ -660,14 +671,16 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("gemm_invoke: missing extra output");
-  return check(igemm_launch(mfma_kind, tile, false, g, (hipStream_t)s), "igemm_launch");
+  return check(igemm_launch(b_split ? KIND_F32X3P : mfma_kind, tile, false, g, (hipStream_t)s), "igemm_launch");
 }
 
 int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, const void* init,
                         const void* const* operands, void* const* outs, pml_hip_stream s) {
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
-  return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s);
+  const bool split = p->bt_is_split;
+  if (b && !p->gemm.b_layout) p->bt_is_split = false;  // this run's transposition overwrites the packed copy
+  return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s, nullptr, split);
 }
 
 int pml_hip_gemm_invoke2(int64_t plan, const void* a, const void* b, void* c, const void* init, const void* a2, const void* b2,
@@ -786,6 +799,8 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
       return 0;
     }
   }
+  // (whole 128-byte chunks per filter tap, so that no chunk of heads + remainders straddles two taps)
+  p->b_split = kind == KIND_F32X3 && !via_s2d && !via_patches && d->ci % 32 == 0;
   p->bt_bytes = (size_t)d->co * p->bt_ld * es;
   if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess || hipMemset(p->bt, 0, p->bt_bytes) != hipSuccess) {
     delete p;
@@ -892,7 +907,7 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   }
   if (p->halo_lds)
     return check(conv_halo_launch(p->mfma_kind, g, p->halo_lds, p->n_cus, (hipStream_t)s), "conv_halo_launch");
-  return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
+  return check(igemm_launch(p->b_split ? KIND_F32X3P : p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
 }
 
 int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s) {
@@ -902,6 +917,8 @@ int pml_hip_gemm_pack_b(int64_t plan, const void* b, pml_hip_stream s) {
   if (d.b_layout) return fail("gemm_pack_b: an [N][K] right-hand side needs no packing");
   if (check(transpose_pack(dt_size(d.in_dtype), b, p->bt, d.k, d.n, d.ldb, p->bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
+  if (p->b_split && check(split_rows_launch(p->bt, d.n, p->bt_ld, d.k, (hipStream_t)s), "split_rows_launch")) return 1;
+  p->bt_is_split = p->b_split;
   p->packed = true;
   return 0;
 }

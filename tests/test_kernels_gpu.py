@@ -86,7 +86,7 @@ def test_gemm_f32_matches_oracle_contraction():
     np.testing.assert_allclose(run_gemm(Av, Bv, hk.F32, hk.F32), ref, rtol=FP32_RTOL, atol=1e-5)
 
 
-TILE_NAMES = ['64x64', '128x64', '128x128', '128x64w8', '128x128w8', '128x128w8s2', '256x128w16', '64x64w8k2', '256x256w8']
+TILE_NAMES = ['64x64', '128x64', '128x128', '128x64w8', '128x128w8', '128x128w8s2', '256x128w16', '64x64w8k2', '256x256w8', '128x64n2']
 
 
 @pytest.mark.parametrize('tile', TILE_NAMES)
