@@ -529,7 +529,8 @@ def _stem_case(kind, shape, k, co, stride, pad, seed):
         ref = oracle_conv(Iv, Fv, D.BFLOAT16, stride, op.SAME_UPPER, bias, True, pad=pad)
         np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2)
     else:
-        out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, pad=pad, bias=bias, relu=True)
+        out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, pad=pad, bias=bias, relu=True,
+                       flags=hk.FP32_AS_BF16X3 if kind == 'f32x3' else 0)
         ref = oracle_conv(Iv, Fv, D.FLOAT32, stride, op.SAME_UPPER, bias, True, pad=pad)
         np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4)
 
@@ -540,14 +541,14 @@ STEM_CASES = [((2, 30, 34, 3), 7, 64, None), ((2, 32, 32, 3), 7, 64, 3), ((2, 31
               ((3, 17, 23, 1), 3, 32, 1), ((1, 20, 18, 5), 5, 48, 0), ((2, 16, 16, 3), 2, 64, 0)]
 
 
-@pytest.mark.parametrize('kind', ['f32', 'bf16'])
+@pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
 @pytest.mark.parametrize('shape,k,co,pad', STEM_CASES)
 def test_conv_few_channel_stride2(kind, shape, k, co, pad, capsys):
     _stem_case(kind, shape, k, co, 2, pad, 41)
     assert '2x2 pixel blocks' in capsys.readouterr().out
 
 
-@pytest.mark.parametrize('kind', ['f32', 'bf16'])
+@pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
 @pytest.mark.parametrize('stride', [1, 2])
 def test_conv_few_channel_patch_matrix(kind, stride, capsys, monkeypatch):
     # other strides (and stride 2 on request) gather a patch matrix [M][K padded] and run a plain GEMM

@@ -54,6 +54,23 @@ def test_program_matches_oracle(name, target):
     check(name, got, ref, tol)
 
 
+@pytest.mark.parametrize('name', sorted(n for n in programs.ALL if programs.ALL[n](OE, Oop)[2] == programs.FP32))
+def test_fp32_program_as_three_bf16_products(name):
+    """Every fp32 program again with `hip{fp32=bf16x3}`: GEMMs and convolutions multiply on the bf16 matrix cores
+    (operands split into head + remainder), everything else is unchanged; the fp32 bar holds."""
+    print('program', name, 'target hip{fp32=bf16x3}', flush=True)
+    oprog, ovals, tol = programs.ALL[name](OE, Oop)
+    ref = OE.run(oprog, ovals)
+    prog, vals, _ = programs.ALL[name](E, op)
+    got = E.run(prog, vals, target='hip{fp32=bf16x3}')
+    assert len(got) == len(ref)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        if r.dtype.kind in 'iub':
+            np.testing.assert_array_equal(g, r, err_msg='%s output %d' % (name, k))
+        else:
+            np.testing.assert_allclose(g, r, rtol=1e-3, atol=1e-4, err_msg='%s output %d' % (name, k))
+
+
 def test_config2_full_size_properties():
     """BASELINE configs[2] at full size through the plaidml API: int8 4096^3 -> int32 (bit-exact by a checksum of
     checksums: row sums of C against A . rowsum(B) in int64) and the per-column requantised int8 output (exact
