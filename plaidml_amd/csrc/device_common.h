@@ -45,6 +45,15 @@ __host__ __device__ inline int dt_size(int dt) {
   return 0;
 }
 
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  A kernel whose neighbouring workgroups
+// read overlapping data (window rows) takes its work in this order instead of blockIdx.x: XCD x then owns one
+// contiguous range of work blocks (ranges differ by at most one when the count is no multiple of 8), and what two
+// neighbours share is fetched into one L2 once instead of into up to eight.
+__device__ inline unsigned xcd_contiguous_block(unsigned bid, unsigned nblocks) {
+  const unsigned per = nblocks / 8, rem = nblocks % 8, x = bid % 8;
+  return x * per + (x < rem ? x : rem) + bid / 8;
+}
+
 __device__ inline float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
 // round-to-nearest-even fp32 -> bf16 storage bits

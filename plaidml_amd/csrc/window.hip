@@ -40,6 +40,21 @@ struct VecIO<4> {
   }
 };
 
+// Eight fp32 values to eight bf16 (hardware conversion: round to nearest even, NaN quieted), one 16-byte vector.
+__device__ __forceinline__ i32x4_t pack_bf16_rne(const float* v) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  i32x4_t o;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const bf16x2 h = __builtin_convertvector(f32x2{v[2 * q], v[2 * q + 1]}, bf16x2);
+    uint32_t w;
+    __builtin_memcpy(&w, &h, 4);
+    o[q] = (int)w;
+  }
+  return o;
+}
+
 template <int ES>
 __global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t total_vecs) {
   constexpr int V = VecIO<ES>::V;
@@ -47,7 +62,7 @@ __global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t tot
   const int dt = d.dtype;
   const int64_t cvecs = d.c / V;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total_vecs; g += stride) {
+  for (int64_t g = (int64_t)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x; g < total_vecs; g += stride) {
     const int64_t cv = g % cvecs;
     const int64_t pix = g / cvecs;
     const int ox = (int)(pix % d.ow);
@@ -121,36 +136,51 @@ __global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t tot
 // it loads serve all of them and the nine filter vectors are loaded once (27 loads for 4 outputs
 // instead of 72).  A tap outside the image takes no part in the sum (it is not multiplied by zero).
 constexpr int kDwPx = 4;
-template <int ES>
+// IT: the integer type of the index arithmetic.  Element counts below 2^31 (checked by the launcher) take
+// 32-bit arithmetic: a thread's three divisions and its address sums are a fifth of the 64-bit cost, and on a
+// 19x19x728 image the kernel is bound by its instruction count, not by memory.
+template <int ES, typename IT>
 __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t total) {
   constexpr int V = VecIO<ES>::V;
   const pml_hip_dwconv2d_desc& d = a.d;
-  const int64_t cvecs = d.c / V;
-  const int64_t xblocks = (d.ow + kDwPx - 1) / kDwPx;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
-    const int64_t cv = g % cvecs;
-    int64_t t = g / cvecs;
+  const IT cvecs = (IT)(d.c / V);
+  const IT xblocks = (IT)((d.ow + kDwPx - 1) / kDwPx);
+  const IT oh = (IT)d.oh, H = (IT)d.h, W = (IT)d.w, C = (IT)d.c;
+  const int pad_h = (int)d.pad_h, pad_w = (int)d.pad_w;
+  const IT stride = (IT)gridDim.x * blockDim.x;
+  for (IT g = (IT)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x; g < (IT)total; g += stride) {
+    const IT cv = g % cvecs;
+    IT t = g / cvecs;
     const int ox0 = (int)(t % xblocks) * kDwPx;
     t /= xblocks;
-    const int oy = (int)(t % d.oh);
-    const int64_t n = t / d.oh;
-    const int64_t c0 = cv * V;
+    const int oy = (int)(t % oh);
+    const IT n = t / oh;
+    const IT c0 = cv * V;
+    const int iy0 = oy - pad_h, ix0 = ox0 - pad_w;
     i32x4_t xr[3][kDwPx + 2], wr[9];
     bool ok[3][kDwPx + 2];
-    bool all_ok = true;
 #pragma unroll
-    for (int k = 0; k < 9; ++k) wr[k] = *(const i32x4_t*)((const unsigned char*)a.filter + ((int64_t)k * d.c + c0) * ES);
+    for (int k = 0; k < 9; ++k) wr[k] = *(const i32x4_t*)((const unsigned char*)a.filter + ((int64_t)((IT)k * C + c0)) * ES);
+    // the whole 3 x (kDwPx + 2) window inside the image: one base offset, constant steps, no per-tap checks
+    const bool all_ok = iy0 >= 0 && iy0 + 2 < (int)H && ix0 >= 0 && ix0 + kDwPx + 1 < (int)W;
+    if (all_ok) {
+      const IT base = ((n * H + (IT)iy0) * W + (IT)ix0) * C + c0;
 #pragma unroll
-    for (int ky = 0; ky < 3; ++ky) {
-      const int64_t iy = (int64_t)oy + ky - d.pad_h;
+      for (int ky = 0; ky < 3; ++ky)
 #pragma unroll
-      for (int c = 0; c < kDwPx + 2; ++c) {
-        const int64_t ix = (int64_t)ox0 + c - d.pad_w;
-        ok[ky][c] = iy >= 0 && iy < d.h && ix >= 0 && ix < d.w;
-        all_ok = all_ok && ok[ky][c];
-        const int64_t off = ok[ky][c] ? ((n * d.h + iy) * d.w + ix) * d.c + c0 : 0;
-        xr[ky][c] = *(const i32x4_t*)((const unsigned char*)a.in + off * ES);
+        for (int c = 0; c < kDwPx + 2; ++c)
+          xr[ky][c] = *(const i32x4_t*)((const unsigned char*)a.in + (int64_t)(base + ((IT)ky * W + (IT)c) * C) * ES);
+    } else {
+#pragma unroll
+      for (int ky = 0; ky < 3; ++ky) {
+        const int iy = iy0 + ky;
+#pragma unroll
+        for (int c = 0; c < kDwPx + 2; ++c) {
+          const int ix = ix0 + c;
+          ok[ky][c] = iy >= 0 && iy < (int)H && ix >= 0 && ix < (int)W;
+          const IT off = ok[ky][c] ? ((n * H + (IT)iy) * W + (IT)ix) * C + c0 : 0;
+          xr[ky][c] = *(const i32x4_t*)((const unsigned char*)a.in + (int64_t)off * ES);
+        }
       }
     }
     auto unpack = [](const i32x4_t& raw, float* f) {
@@ -196,16 +226,13 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t to
       accumulate(std::false_type());
     else
       accumulate(std::true_type());
+    const IT orow = ((n * oh + (IT)oy) * (IT)d.ow + (IT)ox0) * C + c0;
 #pragma unroll
     for (int px = 0; px < kDwPx; ++px) {
-      if (ox0 + px >= d.ow) break;
-      const int64_t o0 = ((n * d.oh + oy) * d.ow + ox0 + px) * d.c + c0;
+      if (ox0 + px >= (int)d.ow) break;
+      const int64_t o0 = (int64_t)(orow + (IT)px * C);
       if constexpr (ES == 2) {
-        i32x4_t o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[px][2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[px][2 * i + 1]) << 16));
-        *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+        *(i32x4_t*)((uint16_t*)a.out + o0) = pack_bf16_rne(acc[px]);
       } else {
         const f32x4_t o = {acc[px][0], acc[px][1], acc[px][2], acc[px][3]};
         *(f32x4_t*)((float*)a.out + o0) = o;
@@ -214,24 +241,26 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t to
   }
 }
 
-template <int ES, bool WITH_INDEX>
+// IT: the integer type of the index arithmetic (32 bits where every element offset stays below 2^31).
+// AGG: the aggregation (PML_HIP_AGG_*), a compile-time constant so that the tap loop is straight-line code.
+template <int ES, bool WITH_INDEX, typename IT, int AGG>
 __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_vecs) {
   constexpr int V = VecIO<ES>::V;
   const pml_hip_pool2d_desc& d = a.d;
   const int dt = d.dtype;
-  const int64_t cvecs = d.c / V;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total_vecs; g += stride) {
-    const int64_t cv = g % cvecs;
-    const int64_t pix = g / cvecs;
-    const int ox = (int)(pix % d.ow);
-    const int64_t t = pix / d.ow;
-    const int oy = (int)(t % d.oh);
-    const int64_t n = t / d.oh;
-    const int64_t c0 = cv * V;
+  const IT cvecs = (IT)(d.c / V), ow = (IT)d.ow, oh = (IT)d.oh, H = (IT)d.h, W = (IT)d.w, C = (IT)d.c;
+  const IT stride = (IT)gridDim.x * blockDim.x;
+  for (IT g = (IT)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x; g < (IT)total_vecs; g += stride) {
+    const IT cv = g % cvecs;
+    const IT pix = g / cvecs;
+    const int ox = (int)(pix % ow);
+    const IT t = pix / ow;
+    const int oy = (int)(t % oh);
+    const IT n = t / oh;
+    const IT c0 = cv * V;
     float acc[V];
     int best[V];  // with_index: largest window index whose (in-range) tap equals the pooled value; 0 if none
-    const float ident = d.agg == PML_HIP_AGG_MAX ? -INFINITY : (d.agg == PML_HIP_AGG_MIN ? INFINITY : 0.f);
+    const float ident = AGG == PML_HIP_AGG_MAX ? -INFINITY : (AGG == PML_HIP_AGG_MIN ? INFINITY : 0.f);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       acc[i] = ident;
@@ -242,48 +271,56 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
     // thread has kGroup loads in flight instead of one.
     constexpr int kGroup = 9;
     const int taps = (int)(d.kh * d.kw);
-    const int64_t iy0 = (int64_t)oy * d.stride_h - d.pad_h, ix0 = (int64_t)ox * d.stride_w - d.pad_w;
+    const int iy0 = oy * (int)d.stride_h - (int)d.pad_h, ix0 = ox * (int)d.stride_w - (int)d.pad_w;
+    // the whole window inside the image: the taps' offsets are the first one's plus steps that are the same for
+    // every thread
+    const bool inside = iy0 >= 0 && iy0 + (int)d.kh <= (int)H && ix0 >= 0 && ix0 + (int)d.kw <= (int)W;
+    const IT base = inside ? ((n * H + (IT)iy0) * W + (IT)ix0) * C + c0 : 0;
     int ky = 0, kx = 0;
     for (int k0 = 0; k0 < taps; k0 += kGroup) {
       float x[kGroup][V];
       bool ok[kGroup];
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
-        const int64_t iy = iy0 + ky, ix = ix0 + kx;
-        ok[u] = k0 + u < taps && iy >= 0 && iy < d.h && ix >= 0 && ix < d.w;
-        VecIO<ES>::load(a.in, ok[u] ? ((n * d.h + iy) * d.w + ix) * d.c + c0 : 0, x[u]);
-        if (++kx == d.kw) {
+        const int iy = iy0 + ky, ix = ix0 + kx;
+        IT off;
+        if (inside) {
+          ok[u] = k0 + u < taps;
+          off = ok[u] ? base + ((IT)ky * W + (IT)kx) * C : 0;
+        } else {
+          ok[u] = k0 + u < taps && iy >= 0 && iy < (int)H && ix >= 0 && ix < (int)W;
+          off = ok[u] ? ((n * H + (IT)iy) * W + (IT)ix) * C + c0 : 0;
+        }
+        VecIO<ES>::load(a.in, (int64_t)off, x[u]);
+        if (++kx == (int)d.kw) {
           kx = 0;
           ++ky;
         }
       }
+      // (a tap outside the image takes no part: its comparisons are masked, not branched around)
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
-        if (!ok[u]) continue;
+        const bool live = ok[u];
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          if (d.agg == PML_HIP_AGG_MAX) {
+          if constexpr (AGG == PML_HIP_AGG_MAX) {
             // taps come in rising window index, so ">=" leaves the largest index among equal values
-            if (WITH_INDEX) best[i] = (x[u][i] >= acc[i]) ? k0 + u : best[i];
-            acc[i] = (x[u][i] > acc[i]) ? x[u][i] : acc[i];
-          } else if (d.agg == PML_HIP_AGG_MIN) {
-            if (WITH_INDEX) best[i] = (x[u][i] <= acc[i]) ? k0 + u : best[i];
-            acc[i] = (x[u][i] < acc[i]) ? x[u][i] : acc[i];
+            if (WITH_INDEX) best[i] = (live & (x[u][i] >= acc[i])) ? k0 + u : best[i];
+            acc[i] = (live & (x[u][i] > acc[i])) ? x[u][i] : acc[i];
+          } else if constexpr (AGG == PML_HIP_AGG_MIN) {
+            if (WITH_INDEX) best[i] = (live & (x[u][i] <= acc[i])) ? k0 + u : best[i];
+            acc[i] = (live & (x[u][i] < acc[i])) ? x[u][i] : acc[i];
           } else {
-            acc[i] += x[u][i];
+            acc[i] += live ? x[u][i] : 0.f;
           }
         }
       }
     }
-    const int64_t o0 = pix * d.c + c0;
+    const int64_t o0 = (int64_t)(pix * C + c0);
     if (dt == PML_HIP_BF16 || dt == PML_HIP_F32) {
       // one 16-byte store of the rounded values
       if constexpr (ES == 2) {
-        i32x4_t o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[2 * i + 1]) << 16));
-        *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+        *(i32x4_t*)((uint16_t*)a.out + o0) = pack_bf16_rne(acc);
       } else {
         const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
         *(f32x4_t*)((float*)a.out + o0) = o;
@@ -404,10 +441,16 @@ hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
   if (d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.dil_h == 1 && d.dil_w == 1 && d.tail.n_ops == 0 &&
       (d.dtype == PML_HIP_BF16 || d.dtype == PML_HIP_F32)) {
     const int64_t total4 = d.n * d.oh * ((d.ow + kDwPx - 1) / kDwPx) * (d.c / V);
-    if (es == 2)
-      hipLaunchKernelGGL((dwconv3x3_kernel<2>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
+    // 32-bit index arithmetic where every element offset (and the rounded-up thread count) stays below 2^31
+    const bool narrow = d.n * d.h * d.w * d.c < ((int64_t)1 << 31) - (1 << 24) && d.n * d.oh * d.ow * d.c < ((int64_t)1 << 31) - (1 << 24);
+    if (es == 2 && narrow)
+      hipLaunchKernelGGL((dwconv3x3_kernel<2, uint32_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
+    else if (es == 2)
+      hipLaunchKernelGGL((dwconv3x3_kernel<2, int64_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
+    else if (narrow)
+      hipLaunchKernelGGL((dwconv3x3_kernel<4, uint32_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
     else
-      hipLaunchKernelGGL((dwconv3x3_kernel<4>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
+      hipLaunchKernelGGL((dwconv3x3_kernel<4, int64_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
     return hipGetLastError();
   }
   if (es == 2)
@@ -510,14 +553,34 @@ hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s) {
       return hipGetLastError();
     }
   }
-  if (es == 2 && d.with_index)
-    hipLaunchKernelGGL((pool2d_kernel<2, true>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
-  else if (es == 2)
-    hipLaunchKernelGGL((pool2d_kernel<2, false>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
-  else if (d.with_index)
-    hipLaunchKernelGGL((pool2d_kernel<4, true>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+  // 32-bit index arithmetic where every element offset (and the rounded-up thread count) stays below 2^31
+  const bool narrow = d.n * d.h * d.w * d.c < ((int64_t)1 << 31) - (1 << 24) && d.n * d.oh * d.ow * d.c < ((int64_t)1 << 31) - (1 << 24);
+  auto launch = [&](auto kern) { hipLaunchKernelGGL(kern, dim3(grid_for(total)), dim3(256), 0, s, a, total); };
+  auto pick_index = [&](auto es_tag, auto it_tag, auto agg_tag) {
+    constexpr int kEs = decltype(es_tag)::value, kAgg = decltype(agg_tag)::value;
+    typedef typename decltype(it_tag)::type it_t;
+    if (d.with_index)
+      launch(pool2d_kernel<kEs, true, it_t, kAgg>);
+    else
+      launch(pool2d_kernel<kEs, false, it_t, kAgg>);
+  };
+  auto pick_agg = [&](auto es_tag, auto it_tag) {
+    switch (d.agg) {
+      case PML_HIP_AGG_MAX: pick_index(es_tag, it_tag, std::integral_constant<int, PML_HIP_AGG_MAX>()); break;
+      case PML_HIP_AGG_MIN: pick_index(es_tag, it_tag, std::integral_constant<int, PML_HIP_AGG_MIN>()); break;
+      default: pick_index(es_tag, it_tag, std::integral_constant<int, PML_HIP_AGG_ADD>()); break;
+    }
+  };
+  auto pick_it = [&](auto es_tag) {
+    if (narrow)
+      pick_agg(es_tag, std::common_type<uint32_t>());
+    else
+      pick_agg(es_tag, std::common_type<int64_t>());
+  };
+  if (es == 2)
+    pick_it(std::integral_constant<int, 2>());
   else
-    hipLaunchKernelGGL((pool2d_kernel<4, false>), dim3(grid_for(total)), dim3(256), 0, s, a, total);
+    pick_it(std::integral_constant<int, 4>());
   return hipGetLastError();
 }
 
