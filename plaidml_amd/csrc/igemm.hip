@@ -350,8 +350,9 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
           const int64_t m = m0 + wm * WM + i * 32 + (lane_t & 31);
-          const int64_t off = (m * rs + n0 + wn * WN + j * 32 + 16 * (lane_t >> 5)) * 2;
-          const unsigned voff = (m < p.M && off < (int64_t)kBufRange) ? (unsigned)off : kOutside;
+          const int64_t col = n0 + wn * WN + j * 32 + 16 * (lane_t >> 5);
+          const int64_t off = (m * rs + col) * 2;
+          const unsigned voff = (m < p.M && col < p.N && off < (int64_t)kBufRange) ? (unsigned)off : kOutside;
           __builtin_amdgcn_raw_ptr_buffer_load_lds(rr, PML_LDS(smem + ring_t::kBytes), 4, (int)voff, 0, 0, 0);
         }
     }

@@ -165,7 +165,8 @@ __device__ __forceinline__ bool direct_tail_ok(const IgemmArgs& p, int64_t n0, i
   if constexpr (KIND != KIND_BF16) return false;
   const bool scale_shift = p.tail_mode == 3 && p.tail_ssr != 0 && p.init2 == nullptr;
   if (p.out_dtype != PML_HIP_BF16 || (p.tail_mode != 1 && p.tail_mode != 2 && !scale_shift)) return false;
-  if (n0 + bn > p.N || (p.ldc & 7) != 0 || ((uintptr_t)p.C & 15) != 0) return false;
+  // (a tile that hangs over the last column is fine as long as N ends on a 16-byte piece: whole pieces are skipped)
+  if ((n0 + bn > p.N && (p.N & 7) != 0) || (p.ldc & 7) != 0 || ((uintptr_t)p.C & 15) != 0) return false;
   if (p.init != nullptr && !(p.init_rs == 0 && p.init_cs == 1 && p.init_dtype == PML_HIP_BF16 && ((uintptr_t)p.init & 15) == 0)) return false;
   if (p.tail_mode == 2 && ((p.tail.operand_row_stride[0] & 7) != 0 || ((uintptr_t)p.operands[0] & 15) != 0)) return false;
   if (p.init2 != nullptr && ((uintptr_t)p.init2 & 15) != 0) return false;
@@ -209,21 +210,25 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
   asm volatile("s_nop 15\n\ts_nop 3");
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
+    // the lane's two 8-column pieces of this block; one past the last column (a ragged last tile) is left out
+    bool col_ok[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) col_ok[q] = nw + j * 32 + 16 * q + 8 * hi < p.N;
     i32x4_t bias_bits[2];  // kept packed: registers are the scarce thing here
 #pragma unroll
     for (int q = 0; q < 2; ++q)
-      bias_bits[q] = p.init != nullptr ? *(const i32x4_t*)((const uint16_t*)p.init + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+      bias_bits[q] = (p.init != nullptr && col_ok[q]) ? *(const i32x4_t*)((const uint16_t*)p.init + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
     // the second product's bias, or the scale vector of a scale / shift chain (which excludes a second product)
     i32x4_t second_bits[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       const uint16_t* src = scale_shift ? scale : (const uint16_t*)p.init2;
-      second_bits[q] = src != nullptr ? *(const i32x4_t*)(src + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+      second_bits[q] = (src != nullptr && col_ok[q]) ? *(const i32x4_t*)(src + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
     }
     i32x4_t shift_bits[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q)
-      shift_bits[q] = scale_shift ? *(const i32x4_t*)(shift + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+      shift_bits[q] = (scale_shift && col_ok[q]) ? *(const i32x4_t*)(shift + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int64_t m = mw + i * 32 + (lane & 31);
@@ -231,7 +236,8 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
       i32x4_t res[2] = {i32x4_t{0, 0, 0, 0}, i32x4_t{0, 0, 0, 0}};
       if (residual && row_ok) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) res[q] = *(const i32x4_t*)((const uint16_t*)p.operands[0] + m * rs + nw + j * 32 + 16 * q + 8 * hi);
+        for (int q = 0; q < 2; ++q)
+          if (col_ok[q]) res[q] = *(const i32x4_t*)((const uint16_t*)p.operands[0] + m * rs + nw + j * 32 + 16 * q + 8 * hi);
       }
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
@@ -277,7 +283,7 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = v[e] < 0.f ? 0.f : v[e];
         }
-        if (row_ok) *(i32x4_t*)((uint16_t*)p.C + m * p.ldc + nw + j * 32 + 16 * q + 8 * hi) = pack_bf16x8(v);
+        if (row_ok && col_ok[q]) *(i32x4_t*)((uint16_t*)p.C + m * p.ldc + nw + j * 32 + 16 * q + 8 * hi) = pack_bf16x8(v);
       }
     }
   }

@@ -139,6 +139,8 @@ constexpr int kDwPx = 4;
 // IT: the integer type of the index arithmetic.  Element counts below 2^31 (checked by the launcher) take
 // 32-bit arithmetic: a thread's three divisions and its address sums are a fifth of the 64-bit cost, and on a
 // 19x19x728 image the kernel is bound by its instruction count, not by memory.
+// (165 registers, three wavefronts per SIMD: capping the registers for four or more made the compiler spill and the
+// kernel two to four times slower.)
 template <int ES, typename IT>
 __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t total) {
   constexpr int V = VecIO<ES>::V;
