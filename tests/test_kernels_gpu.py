@@ -216,6 +216,63 @@ def test_gemm_bf16_step_tails_bit_exact(tile, monkeypatch):
         np.testing.assert_array_equal(C, bf16(want))
 
 
+def test_gemm_random_shapes_all_kinds():
+    """Forty seeded random problems -- ragged M, N, K, every element kind, the tails with a vector path (none, bias + relu,
+    + residual + relu, scale / shift + relu) -- against float64 / exact integer arithmetic; bf16 results additionally
+    bit for bit against the step semantics where the accumulation is exact (small-integer operands)."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        kind = ['f32', 'bf16', 'i8', 'f32x3'][case % 4]
+        M, N = int(rng.integers(1, 700)), int(rng.integers(1, 90)) * 8
+        K = int(rng.integers(1, 60)) * (16 if kind == 'i8' else 8)
+        tail_kind = ['none', 'relu', 'residual', 'scale_shift'][int(rng.integers(0, 4))]
+        print('case', case, kind, (M, N, K), tail_kind, flush=True)
+        if kind == 'i8':
+            A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+            B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+            np.testing.assert_array_equal(run_gemm(A, B, hk.I8, hk.I32), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.int32))
+            continue
+        dt = hk.BF16 if kind == 'bf16' else hk.F32
+        flags = hk.FP32_AS_BF16X3 if kind == 'f32x3' else 0
+        if kind == 'bf16':   # small integers: the fp32 accumulation is exact, every rounding is pinned
+            A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+            B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+        else:
+            A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+            B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        rnd = E.round_bf16 if kind == 'bf16' else (lambda x: np.asarray(x, np.float32))
+        enc = bf16 if kind == 'bf16' else (lambda x: np.asarray(x, np.float32))
+        bias = rnd(rng.standard_normal(N).astype(np.float32) * 4)
+        scale = rnd(rng.uniform(0.5, 1.5, N).astype(np.float32))
+        shift = rnd(rng.standard_normal(N).astype(np.float32) * 8)
+        res = rnd(rng.standard_normal((M, N)).astype(np.float32) * 16)
+        relu = [(hk.EPI_RELU, dt, 0, 0, 0.0)]
+        x64 = A.astype(np.float64) @ B.astype(np.float64)
+        if tail_kind == 'none':
+            C = run_gemm(enc(A), enc(B), dt, dt, flags=flags)
+            want = rnd(x64.astype(np.float32)) if kind == 'bf16' else x64
+        elif tail_kind == 'relu':
+            C = run_gemm(enc(A), enc(B), dt, dt, init=enc(bias), init_strides=(0, 1), init_dt=dt, tail=hk.make_tail(ops=relu), flags=flags)
+            want = np.maximum(rnd((x64 + bias).astype(np.float32)) if kind == 'bf16' else x64 + bias, 0)
+        elif tail_kind == 'residual':
+            tail = hk.make_tail(ops=[(hk.EPI_ADD, dt, hk.OPND_TENSOR, 0, 0.0)] + relu, operands=[(dt, N, 1)])
+            C = run_gemm(enc(A), enc(B), dt, dt, init=enc(bias), init_strides=(0, 1), init_dt=dt, tail=tail, operands=(enc(res),), flags=flags)
+            want = np.maximum(rnd(rnd((x64 + bias).astype(np.float32)) + res) if kind == 'bf16' else x64 + bias + res, 0)
+        else:
+            tail = hk.make_tail(ops=[(hk.EPI_MUL, dt, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_ADD, dt, hk.OPND_TENSOR, 1, 0.0)] + relu,
+                                operands=[(dt, 0, 1), (dt, 0, 1)])
+            C = run_gemm(enc(A), enc(B), dt, dt, init=enc(bias), init_strides=(0, 1), init_dt=dt, tail=tail,
+                         operands=(enc(scale), enc(shift)), flags=flags)
+            if kind == 'bf16':
+                want = np.maximum(rnd(rnd(rnd((x64 + bias).astype(np.float32)) * scale) + shift), 0)
+            else:
+                want = np.maximum((x64 + bias) * scale + shift, 0)
+        if kind == 'bf16':
+            np.testing.assert_array_equal(C, bf16(want), err_msg='case %d' % case)
+        else:
+            np.testing.assert_allclose(C, want, rtol=FP32_RTOL, atol=1e-3, err_msg='case %d' % case)
+
+
 def test_gemm_bf16_4096_sampled():
     """bf16 4096^3 with N(0,1) inputs (the large-tile path): sampled rows and columns against float64."""
     rng = np.random.default_rng(9)
@@ -384,6 +441,32 @@ def test_conv_bf16(shape, k, stride, co):
     out = run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=stride, bias=bf16(bias), relu=True)
     ref = oracle_conv(Iv, Fv, D.BFLOAT16, stride, op.SAME_UPPER, bias, True)
     np.testing.assert_allclose(E.bf16_from_bits(out), ref, rtol=BF16_RTOL, atol=1e-2)
+
+
+def test_conv_random_shapes_all_kinds():
+    """Twenty-four seeded random convolutions (1x1 / 3x3 / 5x5, stride 1 / 2, SAME and VALID windows, channel counts that
+    do and do not fill 128-byte pixels, bias + ReLU) in fp32, bf16 and split fp32 against the oracle."""
+    rng = np.random.default_rng(777)
+    for case in range(24):
+        kind = ['f32', 'bf16', 'f32x3'][case % 3]
+        k = int(rng.choice([1, 3, 3, 5]))
+        stride = int(rng.choice([1, 1, 2]))
+        ci, co = int(rng.choice([8, 16, 32, 64, 72])), int(rng.choice([8, 24, 64, 96]))
+        shape = (int(rng.integers(1, 4)), int(rng.integers(k, 20)), int(rng.integers(k, 24)), ci)
+        autopad = op.SAME_UPPER if rng.integers(0, 2) else op.VALID
+        print('case', case, kind, shape, 'k', k, 'stride', stride, 'co', co, 'autopad', autopad, flush=True)
+        Iv, Fv = _conv_case('bf16' if kind == 'bf16' else 'f32', shape, k, k, co, autopad, 1000 + case)
+        bias = rng.standard_normal(co).astype(np.float32)
+        if kind == 'bf16':
+            bias = E.round_bf16(bias)
+            out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=stride, autopad=autopad, bias=bf16(bias), relu=True))
+            ref = oracle_conv(Iv, Fv, D.BFLOAT16, stride, autopad, bias, True)
+            np.testing.assert_allclose(out, ref, rtol=BF16_RTOL, atol=1e-2, err_msg='case %d' % case)
+        else:
+            out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, autopad=autopad, bias=bias, relu=True,
+                           flags=hk.FP32_AS_BF16X3 if kind == 'f32x3' else 0)
+            ref = oracle_conv(Iv, Fv, D.FLOAT32, stride, autopad, bias, True)
+            np.testing.assert_allclose(out, ref, rtol=FP32_RTOL, atol=1e-4, err_msg='case %d' % case)
 
 
 def test_conv_bf16_full_size_properties():
