@@ -711,24 +711,36 @@ static int64_t floorDiv(int64_t a, int64_t b) {
   return (r != 0 && ((r < 0) != (b < 0))) ? q - 1 : q;
 }
 
-void computeBounds(Op* op) {
-  if (op->kind != Op::Contraction) return;
-  const size_t n = op->idxNames.size();
-  const int64_t INF = static_cast<int64_t>(1) << 60;
-  std::vector<int64_t> lo(n, -INF), hi(n, INF);
-  struct Form {
-    const Affine* a;
-    int64_t size;
-  };
-  std::vector<Form> forms;
-  for (size_t s = 0; s < op->accesses.size(); ++s) {
-    const TensorShape& shape = s == 0 ? op->result->shape : op->operands[s - 1]->shape;
-    for (size_t d = 0; d < op->accesses[s].size(); ++d) forms.push_back({&op->accesses[s][d], shape.sizes[d]});
-  }
-  for (const ConstraintForm& c : op->constraints) forms.push_back({&c.lhs, c.rhs});
-  for (int iter = 0; iter < 64; ++iter) {
+// ---------------------------------------------------------------------------------------------------------------
+// Bounds of a contraction's index variables (reference: Contraction::ComputeBounds and Constraints::ComputeBounds,
+// pmlc/dialect/tile/transforms/contraction.cc:107-149,657-681, which minimise and maximise every variable with an
+// integer linear program, pmlc/util/bilp).  The valid set is
+//     { integer x : for every form f:  (coef_f . x + c0_f) / den_f  is an integer in [0, size_f) }
+// over all accesses (output and inputs) and all constraints.  Three steps, each sound on its own:
+//   1. interval propagation: every form bounds each of its variables from the bounds of the others;
+//   2. where that leaves a variable unbounded (a domain bounded only by combinations of forms, e.g. 0 <= i + j < 10
+//      together with 0 <= i - j < 10), Fourier-Motzkin elimination of the other variables from the linear
+//      relaxation gives its range, and propagation runs again from there;
+//   3. exact tightening: a bound is moved inwards while no integer point of the set takes that value, decided by a
+//      depth-first search over the remaining variables with propagation at every node (the integrality of
+//      fractional forms is checked at the leaves).  The search has a node budget; on exhausting it the bounds stay
+//      as they are -- still a superset, and the kernels check every form at every point anyway.
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int64_t kInfBound = static_cast<int64_t>(1) << 60;
+
+struct BoundForm {
+  const Affine* a;
+  int64_t size;
+};
+
+// One pass structure of step 1; returns false when some variable's range becomes empty.
+bool propagateBounds(const std::vector<BoundForm>& forms, std::vector<int64_t>& lo, std::vector<int64_t>& hi) {
+  const size_t n = lo.size();
+  for (int iter = 0; iter < 256; ++iter) {
     bool changed = false;
-    for (const Form& f : forms) {
+    for (const BoundForm& f : forms) {
       // 0 <= sum coef*idx + c0 <= den*(size-1)
       const int64_t loRhs = -f.a->c0, hiRhs = f.a->den * (f.size - 1) - f.a->c0;
       for (size_t v = 0; v < n; ++v) {
@@ -738,7 +750,7 @@ void computeBounds(Op* op) {
         bool finite = true;
         for (size_t u = 0; u < n && finite; ++u) {
           if (u == v || !f.a->coef[u]) continue;
-          if (lo[u] <= -INF || hi[u] >= INF) {
+          if (lo[u] <= -kInfBound || hi[u] >= kInfBound) {
             finite = false;
             break;
           }
@@ -764,14 +776,226 @@ void computeBounds(Op* op) {
           hi[v] = nhi;
           changed = true;
         }
+        if (lo[v] > hi[v]) return false;
       }
     }
     if (!changed) break;
   }
-  for (size_t v = 0; v < n; ++v) {
-    if (lo[v] <= -INF || hi[v] >= INF)
-      throw std::runtime_error("Unbounded index '" + op->idxNames[v] + "' in contraction '" + op->name + "'");
+  return true;
+}
+
+// Step 2.  Rows are inequalities  sum a[v] * x[v] + a[n] >= 0  with integer coefficients.
+typedef std::vector<__int128> IneqRow;
+
+void normaliseRow(IneqRow& r) {
+  __int128 g = 0;
+  for (size_t i = 0; i + 1 < r.size(); ++i) {
+    __int128 x = r[i] < 0 ? -r[i] : r[i];
+    while (x) {
+      const __int128 t = g % x;
+      g = x;
+      x = t;
+    }
   }
+  if (g > 1) {
+    for (size_t i = 0; i + 1 < r.size(); ++i) r[i] /= g;
+    // floor of the constant: the left-hand side is an integer multiple of g
+    __int128 c = r.back();
+    __int128 q = c / g;
+    if (c % g != 0 && c < 0) --q;
+    r.back() = q;
+  }
+}
+
+// Range of variable `keep` in the linear relaxation; false when unbounded on either side or when the elimination
+// grows past its budget.
+bool fourierMotzkinRange(const std::vector<BoundForm>& forms, size_t n, size_t keep, int64_t* lo, int64_t* hi) {
+  std::set<IneqRow> rows;
+  for (const BoundForm& f : forms) {
+    IneqRow up(n + 1), down(n + 1);
+    for (size_t v = 0; v < n; ++v) {
+      up[v] = f.a->coef[v];
+      down[v] = -f.a->coef[v];
+    }
+    up[n] = f.a->c0;
+    down[n] = static_cast<__int128>(f.a->den) * (f.size - 1) - f.a->c0;
+    normaliseRow(up);
+    normaliseRow(down);
+    rows.insert(up);
+    rows.insert(down);
+  }
+  const size_t kBudget = 4000;
+  std::vector<bool> gone(n, false);
+  for (size_t step = 0; step + 1 < n; ++step) {
+    // the variable whose elimination makes the fewest new rows
+    size_t best = n;
+    size_t bestCost = 0;
+    for (size_t v = 0; v < n; ++v) {
+      if (v == keep || gone[v]) continue;
+      size_t pos = 0, neg = 0;
+      for (const IneqRow& r : rows) {
+        if (r[v] > 0) ++pos;
+        if (r[v] < 0) ++neg;
+      }
+      const size_t cost = pos * neg;
+      if (best == n || cost < bestCost) {
+        best = v;
+        bestCost = cost;
+      }
+    }
+    if (best == n) break;
+    std::set<IneqRow> next;
+    std::vector<const IneqRow*> pos, neg;
+    for (const IneqRow& r : rows) {
+      if (r[best] > 0)
+        pos.push_back(&r);
+      else if (r[best] < 0)
+        neg.push_back(&r);
+      else
+        next.insert(r);
+    }
+    for (const IneqRow* p : pos)
+      for (const IneqRow* q : neg) {
+        IneqRow r(n + 1);
+        const __int128 cp = (*p)[best], cq = -(*q)[best];
+        for (size_t i = 0; i <= n; ++i) r[i] = cq * (*p)[i] + cp * (*q)[i];
+        bool any = false;
+        for (size_t i = 0; i < n; ++i) any = any || r[i] != 0;
+        if (!any) continue;  // a statement about constants only
+        normaliseRow(r);
+        next.insert(r);
+        if (next.size() > kBudget) return false;
+      }
+    rows.swap(next);
+    gone[best] = true;
+  }
+  bool haveLo = false, haveHi = false;
+  __int128 vlo = 0, vhi = 0;
+  for (const IneqRow& r : rows) {
+    bool only = true;
+    for (size_t i = 0; i < n; ++i)
+      if (i != keep && r[i] != 0) only = false;
+    if (!only || r[keep] == 0) continue;
+    // a * x + c >= 0
+    const __int128 a = r[keep], c = r[n];
+    if (a > 0) {  // x >= ceil(-c / a)
+      __int128 q = (-c) / a;
+      if ((-c) % a != 0 && (-c) > 0) ++q;
+      if (!haveLo || q > vlo) vlo = q;
+      haveLo = true;
+    } else {  // x <= floor(c / -a)
+      const __int128 d = -a;
+      __int128 q = c / d;
+      if (c % d != 0 && c < 0) --q;
+      if (!haveHi || q < vhi) vhi = q;
+      haveHi = true;
+    }
+  }
+  if (!haveLo || !haveHi) return false;
+  if (vlo < -kInfBound / 2 || vhi > kInfBound / 2) return false;
+  *lo = static_cast<int64_t>(vlo);
+  *hi = static_cast<int64_t>(vhi);
+  return true;
+}
+
+// Step 3: is there an integer point of the set inside the box?  `budget` counts search nodes; -1 = gave up.
+int feasiblePoint(const std::vector<BoundForm>& forms, std::vector<int64_t> lo, std::vector<int64_t> hi, int64_t* budget) {
+  if (--*budget < 0) return -1;
+  if (!propagateBounds(forms, lo, hi)) return 0;
+  const size_t n = lo.size();
+  // branch on the open variable with the smallest range
+  size_t pick = n;
+  for (size_t v = 0; v < n; ++v) {
+    if (lo[v] == hi[v]) continue;
+    if (pick == n || hi[v] - lo[v] < hi[pick] - lo[pick]) pick = v;
+  }
+  if (pick == n) {
+    for (const BoundForm& f : forms) {
+      __int128 num = f.a->c0;
+      for (size_t v = 0; v < n; ++v) num += static_cast<__int128>(f.a->coef[v]) * lo[v];
+      if (num < 0 || num % f.a->den != 0 || num / f.a->den >= f.size) return 0;
+    }
+    return 1;
+  }
+  // values from the middle outwards: interior points are the likeliest to be valid
+  const int64_t mid = lo[pick] + (hi[pick] - lo[pick]) / 2;
+  for (int64_t d = 0; mid - d >= lo[pick] || mid + d <= hi[pick]; ++d) {
+    for (int side = 0; side < (d ? 2 : 1); ++side) {
+      const int64_t x = side ? mid + d : mid - d;
+      if (x < lo[pick] || x > hi[pick]) continue;
+      std::vector<int64_t> l2 = lo, h2 = hi;
+      l2[pick] = h2[pick] = x;
+      const int r = feasiblePoint(forms, l2, h2, budget);
+      if (r != 0) return r;
+    }
+  }
+  return 0;
+}
+
+}  // namespace
+
+void computeBounds(Op* op) {
+  if (op->kind != Op::Contraction) return;
+  const size_t n = op->idxNames.size();
+  std::vector<int64_t> lo(n, -kInfBound), hi(n, kInfBound);
+  std::vector<BoundForm> forms;
+  for (size_t s = 0; s < op->accesses.size(); ++s) {
+    const TensorShape& shape = s == 0 ? op->result->shape : op->operands[s - 1]->shape;
+    for (size_t d = 0; d < op->accesses[s].size(); ++d) forms.push_back({&op->accesses[s][d], shape.sizes[d]});
+  }
+  for (const ConstraintForm& c : op->constraints) forms.push_back({&c.lhs, c.rhs});
+  auto emptySet = [&]() {
+    // no valid index tuple at all: an empty box (the result is the initial value)
+    for (size_t v = 0; v < n; ++v) {
+      lo[v] = 0;
+      hi[v] = -1;
+    }
+  };
+  bool nonEmpty = propagateBounds(forms, lo, hi);
+  if (nonEmpty) {
+    bool open = false;
+    for (size_t v = 0; v < n; ++v) open = open || lo[v] <= -kInfBound || hi[v] >= kInfBound;
+    if (open) {
+      for (size_t v = 0; v < n; ++v) {
+        if (lo[v] > -kInfBound && hi[v] < kInfBound) continue;
+        int64_t l = 0, h = 0;
+        if (!fourierMotzkinRange(forms, n, v, &l, &h))
+          throw std::runtime_error("Unbounded index '" + op->idxNames[v] + "' in contraction '" + op->name + "'");
+        lo[v] = std::max(lo[v], l);
+        hi[v] = std::min(hi[v], h);
+      }
+      nonEmpty = propagateBounds(forms, lo, hi);
+    }
+  }
+  if (nonEmpty) {
+    // exact tightening (step 3), within a budget of search nodes for the whole contraction
+    int64_t budget = 200000;
+    bool gaveUp = false, empty = false;
+    for (size_t v = 0; v < n && !gaveUp && !empty; ++v) {
+      for (int side = 0; side < 2 && !gaveUp && !empty; ++side) {
+        for (;;) {
+          if (lo[v] > hi[v]) {
+            empty = true;
+            break;
+          }
+          std::vector<int64_t> l2 = lo, h2 = hi;
+          l2[v] = h2[v] = side ? hi[v] : lo[v];
+          const int r = feasiblePoint(forms, l2, h2, &budget);
+          if (r < 0) {
+            gaveUp = true;
+            break;
+          }
+          if (r > 0) break;
+          if (side)
+            --hi[v];
+          else
+            ++lo[v];
+        }
+      }
+    }
+    if (empty) nonEmpty = false;
+  }
+  if (!nonEmpty) emptySet();
   op->lower = lo;
   op->upper = hi;
   op->boundsComputed = true;

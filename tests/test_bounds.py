@@ -1,0 +1,125 @@
+"""Bounds of contraction index variables: exact integer minima / maxima over the valid index set.
+
+The reference minimises and maximises every index variable with an integer linear program
+(pmlc/dialect/tile/transforms/contraction.cc:107-149, pmlc/util/bilp).  Known answers: the cases of
+pmlc/util/bilp/test.cc (Subdivision1D :160-189, TrivialILPTest :125-141, ILPTest2D :143-158); a domain that only
+combinations of constraints bound; fractional forms; and, like MilpTest.RandomConstraintsTest (:191-290), random
+constraint systems against brute force over the box.  Runs on the CPU (compilation only)."""
+import itertools
+import re
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from plaidml_amd import edsl as E
+
+D = E.DType
+
+
+def bounds_of(prog):
+    """{index name: (lower, upper)} of the (only) contraction of a compiled program."""
+    prog.compile()
+    text = dict(prog.passes)['tile-compute-bounds']
+    names = re.search(r'idxs = \[([^\]]*)\]', text).group(1).split(', ')
+    lo = [int(x) for x in re.search(r'lowerBounds = \(([^)]*)\)', text).group(1).split(', ')]
+    hi = [int(x) for x in re.search(r'upperBounds = \(([^)]*)\)', text).group(1).split(', ')]
+    return dict(zip(names, zip(lo, hi)))
+
+
+def program(accesses_out, out_dims, accesses_in, in_dims, constraints, name='bounds'):
+    A = E.Placeholder(D.FLOAT32, in_dims, name='A')
+    c = E.Contraction().outShape(*out_dims).outAccess(*accesses_out).sum(A[tuple(accesses_in)])
+    for con in constraints:
+        c = c.add_constraint(con)
+    return E.Program(name, [A], [c.build()])
+
+
+def test_subdivision_1d():
+    # bilp/test.cc Subdivision1D: i_0 in [0, 1], i_1 in [0, 34], k_0 in [0, 2]
+    i0, i1, k0 = E.TensorIndex('i0'), E.TensorIndex('i1'), E.TensorIndex('k0')
+    prog = program([i0, i1], [100, 100], [i0, i1, k0], [100, 100, 100],
+                   [i0 < 2, i0 + 2 * k0 < 5, i0 + i1 + k0 < 35, i0 + 2 * i1 < 70])
+    assert bounds_of(prog) == {'i0': (0, 1), 'i1': (0, 34), 'k0': (0, 2)}
+
+
+@pytest.mark.parametrize('first', ['x + y + 2 < 4', '2 * x + y + 2 < 6'])
+def test_ilp_2d_objective_as_a_variable(first):
+    # bilp/test.cc TrivialILPTest / ILPTest2D: minimise -3x + 2y subject to the three range constraints; the optimum is
+    # -10 at (x, y) = (2, -2).  The objective becomes an index variable t = -3x + 2y + 10, whose lower bound must be 0.
+    x, y, t = E.TensorIndex('x'), E.TensorIndex('y'), E.TensorIndex('t')
+    cons = [eval(first), x + 1 < 4, y + 2 < 5, t + 3 * x - 2 * y - 10 < 1]
+    prog = program([x + 10, y + 10, t], [100, 100, 100], [x + 10], [100], cons)
+    b = bounds_of(prog)
+    assert b['t'][0] == 0
+    assert b['x'] == (-1, 2) and b['y'] == (-2, 2)
+    # and the maximum of the objective, by brute force over the small box
+    pts = [(a, c) for a in range(-1, 3) for c in range(-2, 3)
+           if 0 <= (a + c + 2 if first.startswith('x') else 2 * a + c + 2) < (4 if first.startswith('x') else 6)]
+    assert b['t'][1] == max(-3 * a + 2 * c + 10 for a, c in pts)
+
+
+def test_domain_bounded_only_by_combinations():
+    # 0 <= i + j < 10 and 0 <= i - j < 10: neither form bounds i or j by itself (interval propagation cannot start),
+    # the pair does: i in [0, 9], j in [-4, 4]
+    i, j = E.TensorIndex('i'), E.TensorIndex('j')
+    prog = program([i + j], [10], [i - j], [10], [])
+    assert bounds_of(prog) == {'i': (0, 9), 'j': (-4, 4)}
+
+
+def test_really_unbounded_index_is_an_error():
+    i, j = E.TensorIndex('i'), E.TensorIndex('j')
+    prog = program([i + j], [10], [i + j], [10], [])
+    with pytest.raises(E.PlaidMLError, match='Unbounded index'):
+        prog.compile()
+
+
+def test_fractional_forms_tighten_to_integer_points():
+    # O[i] += A[(i - j + 1) / 2] (FunkySum's shape) with j pinned to 0: the access is an integer only for odd i, and
+    # (i + 1) / 2 < 3 leaves i in {1, 3}.  Intervals alone give i in [0, 5]; the exact bounds are the extreme odd values.
+    i, j = E.TensorIndex('i'), E.TensorIndex('j')
+    prog = program([i], [6], [(i - j + 1) // 2], [3], [j < 1])
+    assert bounds_of(prog) == {'i': (1, 3), 'j': (0, 0)}
+
+
+def _brute(forms, box):
+    los, his = None, None
+    for pt in itertools.product(*[range(a, b + 1) for a, b in box]):
+        ok = True
+        for coef, c0, den, size in forms:
+            v = Fraction(sum(c * x for c, x in zip(coef, pt)) + c0, den)
+            if v.denominator != 1 or not (0 <= v < size):
+                ok = False
+                break
+        if ok:
+            los = list(pt) if los is None else [min(a, b) for a, b in zip(los, pt)]
+            his = list(pt) if his is None else [max(a, b) for a, b in zip(his, pt)]
+    return los, his
+
+
+def test_random_constraint_systems_against_brute_force():
+    rng = np.random.default_rng(5)
+    names = ['x', 'y', 'z', 'w']
+    checked = 0
+    for case in range(60):
+        idx = [E.TensorIndex(n) for n in names]
+        forms = [([1 if k == v else 0 for k in range(4)], 0, 1, 8) for v in range(4)]   # 0 <= var < 8 (the accesses)
+        cons = []
+        for _ in range(int(rng.integers(2, 6))):
+            coef = [int(rng.integers(-4, 5)) for _ in range(4)]
+            if not any(coef):
+                continue
+            c0, den, size = int(rng.integers(-8, 11)), int(rng.choice([1, 1, 2, 3])), int(rng.integers(10, 30))
+            forms.append((coef, c0, den, size))
+            poly = sum((c * i for c, i in zip(coef, idx) if c), start=c0)
+            cons.append((poly // den if den > 1 else poly) < size)
+        want_lo, want_hi = _brute(forms, [(0, 7)] * 4)
+        prog = program(idx, [8, 8, 8, 8], idx, [8, 8, 8, 8], cons, name='random%d' % case)
+        b = bounds_of(prog)
+        got_lo, got_hi = [b[n][0] for n in names], [b[n][1] for n in names]
+        if want_lo is None:
+            assert all(l > h for l, h in zip(got_lo, got_hi)), (case, got_lo, got_hi)   # empty set: an empty box
+        else:
+            assert (got_lo, got_hi) == (want_lo, want_hi), (case, forms[4:])
+            checked += 1
+    assert checked >= 20
