@@ -71,6 +71,24 @@ def test_fp32_program_as_three_bf16_products(name):
             np.testing.assert_allclose(g, r, rtol=1e-3, atol=1e-4, err_msg='%s output %d' % (name, k))
 
 
+def test_domain_bounded_only_by_combinations_of_accesses():
+    """O[i + j] += A[i - j] over 10-element vectors: neither access bounds i or j by itself (i in [0, 9], j in [-4, 4]
+    follow from the pair), so the index box has a negative corner and most of its points are invalid.  Expected result
+    by direct enumeration."""
+    i, j = E.TensorIndex('i'), E.TensorIndex('j')
+    A = E.Placeholder(E.DType.FLOAT32, [10], name='A')
+    O = E.Contraction().outShape(10).outAccess(i + j).sum(A[i - j]).build()
+    a = np.arange(1, 11, dtype=np.float32)
+    want = np.zeros(10, np.float32)
+    for ii in range(-20, 21):
+        for jj in range(-20, 21):
+            if 0 <= ii + jj < 10 and 0 <= ii - jj < 10:
+                want[ii + jj] += a[ii - jj]
+    for target in ('hip', 'hip{specialise=0,fuse=0}'):
+        got, = E.run(E.Program('skewed', [A], [O]), [a], target=target)
+        np.testing.assert_array_equal(got, want)
+
+
 def test_config2_full_size_properties():
     """BASELINE configs[2] at full size through the plaidml API: int8 4096^3 -> int32 (bit-exact by a checksum of
     checksums: row sums of C against A . rowsum(B) in int64) and the per-column requantised int8 output (exact
