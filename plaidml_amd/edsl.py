@@ -989,16 +989,34 @@ class Runner:
         self.out_shapes = program.outputs
         self.outputs = [Buffer(s) for s in self.out_shapes]
 
-    def run(self, inputs):
-        bufs = []
+    def _converted(self, inputs):
         for shape, a in zip(self.in_shapes, inputs):
             dt = shape.dtype
             a = np.asarray(a)
             if dt == DType.BFLOAT16 and a.dtype != np.uint16:
                 a = to_bf16_bits(a)
-            a = np.ascontiguousarray(a, dtype=dt.into_numpy()).reshape(shape.sizes)
-            bufs.append(Buffer(shape, data=a))
+            yield shape, np.ascontiguousarray(a, dtype=dt.into_numpy()).reshape(shape.sizes)
+
+    def stage(self, inputs):
+        """Converts the inputs once into buffers of the library's own (page-locked where large) memory, for
+        callers that run the same batch many times; returns the list to pass to run_staged."""
+        bufs = []
+        for shape, a in self._converted(inputs):
+            b = Buffer(shape)
+            b.copy_from_ndarray(a)
+            bufs.append(b)
+        return bufs
+
+    def run_staged(self, bufs):
+        """One run over staged inputs; results stay in self.outputs until fetch().  Returns the wall ms."""
         self.ms = self.exe.run(bufs, self.outputs)
+        return self.ms
+
+    def run(self, inputs):
+        self.ms = self.exe.run([Buffer(shape, data=a) for shape, a in self._converted(inputs)], self.outputs)
+        return self.fetch()
+
+    def fetch(self):
         outs = []
         for shape, b in zip(self.out_shapes, self.outputs):
             a = b.as_ndarray()
