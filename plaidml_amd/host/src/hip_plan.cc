@@ -1207,6 +1207,23 @@ class Planner {
     return sp->stride > 0 && sp->dil > 0;
   }
 
+  // The output access of a window kernel: every dimension is its own plain index over the whole extent; a
+  // dimension of size 1 (batch 1, a 1x1 plane) has had its index folded to the constant 0 and gets index -1.
+  bool windowOutput(const Op& op, const Normalised& n, const TensorShape& os, int oi[4], std::vector<bool>* in_out) {
+    for (int k = 0; k < 4; ++k) {
+      if (os.sizes[k] == 1 && n.acc[0][k].isConstant() && n.acc[0][k].c0 == 0) {
+        oi[k] = -1;
+        continue;
+      }
+      oi[k] = n.acc[0][k].plainIndex();
+      if (oi[k] < 0 || (*in_out)[oi[k]] || op.lower[oi[k]] != 0 || op.upper[oi[k]] != os.sizes[k] - 1) return false;
+      (*in_out)[oi[k]] = true;
+    }
+    return true;
+  }
+  // the access form is the index idx, or the constant 0 where that index was folded away (idx < 0)
+  static bool sameIndex(const Affine& a, int idx) { return idx >= 0 ? a.plainIndex() == idx : (a.isConstant() && a.c0 == 0); }
+
   // out[n,y,x,co] += I[n, sy*y + dy*ky - py, sx*x + dx*kx - px, ci] * F[ky,kx,ci,co]
   bool tryConv(size_t i) {
     const Op& op = prog_->ops[i];
@@ -1329,12 +1346,8 @@ class Planner {
       if (!impliedByBox(op, c.lhs, c.rhs)) return false;
     int oi[4];
     std::vector<bool> in_out(n.nIdx, false);
-    for (int d = 0; d < 4; ++d) {
-      oi[d] = n.acc[0][d].plainIndex();
-      if (oi[d] < 0 || in_out[oi[d]] || op.lower[oi[d]] != 0 || op.upper[oi[d]] != os.sizes[d] - 1) return false;
-      in_out[oi[d]] = true;
-    }
-    if (n.acc[1][0].plainIndex() != oi[0] || n.acc[1][3].plainIndex() != oi[3] || n.acc[2][2].plainIndex() != oi[3]) return false;
+    if (!windowOutput(op, n, os, oi, &in_out)) return false;
+    if (!sameIndex(n.acc[1][0], oi[0]) || !sameIndex(n.acc[1][3], oi[3]) || !sameIndex(n.acc[2][2], oi[3])) return false;
     if (!(n.acc[2][3].isConstant() && n.acc[2][3].c0 == 0)) return false;
     if (is.sizes[3] != os.sizes[3] || fs.sizes[2] != os.sizes[3] || is.sizes[0] != os.sizes[0]) return false;
     Spatial sy, sx;
@@ -1391,12 +1404,8 @@ class Planner {
     if (os.getRank() != 4 || is.getRank() != 4) return false;
     int oi[4];
     std::vector<bool> in_out(n.nIdx, false);
-    for (int k = 0; k < 4; ++k) {
-      oi[k] = n.acc[0][k].plainIndex();
-      if (oi[k] < 0 || in_out[oi[k]] || op.lower[oi[k]] != 0 || op.upper[oi[k]] != os.sizes[k] - 1) return false;
-      in_out[oi[k]] = true;
-    }
-    if (n.acc[1][0].plainIndex() != oi[0] || n.acc[1][3].plainIndex() != oi[3]) return false;
+    if (!windowOutput(op, n, os, oi, &in_out)) return false;
+    if (!sameIndex(n.acc[1][0], oi[0]) || !sameIndex(n.acc[1][3], oi[3])) return false;
     if (is.sizes[0] != os.sizes[0] || is.sizes[3] != os.sizes[3]) return false;
     if (!spatialForm(n.acc[1][1], in_out, n.active, sy) || !spatialForm(n.acc[1][2], in_out, n.active, sx)) return false;
     if (sy->out_idx != oi[1] || sx->out_idx != oi[2] || sy->dil != 1 || sx->dil != 1) return false;
@@ -1448,16 +1457,18 @@ class Planner {
     Normalised n = normalise(op);
     for (const auto& c : n.cons)
       if (!impliedByBox(op, c.lhs, c.rhs)) return false;
-    const int on = n.acc[0].front().plainIndex(), oc = n.acc[0].back().plainIndex();
-    if (on < 0 || oc < 0 || on == oc) return false;
+    const bool one_image = is.sizes[0] == 1;  // the batch index of a single image is folded to the constant 0
+    const int on = one_image ? -1 : n.acc[0].front().plainIndex(), oc = n.acc[0].back().plainIndex();
+    if ((!one_image && on < 0) || oc < 0 || on == oc) return false;
+    if (one_image && !sameIndex(n.acc[0].front(), -1)) return false;
     if (keep && !(n.acc[0][1].isConstant() && n.acc[0][1].c0 == 0 && n.acc[0][2].isConstant() && n.acc[0][2].c0 == 0)) return false;
     const int iy = n.acc[1][1].plainIndex(), ix = n.acc[1][2].plainIndex();
-    if (n.acc[1][0].plainIndex() != on || n.acc[1][3].plainIndex() != oc || iy < 0 || ix < 0 || iy == ix || iy == on ||
+    if (!sameIndex(n.acc[1][0], on) || n.acc[1][3].plainIndex() != oc || iy < 0 || ix < 0 || iy == ix || iy == on ||
         iy == oc || ix == on || ix == oc)
       return false;
     const int idx[4] = {on, iy, ix, oc};
     for (int k = 0; k < 4; ++k)
-      if (op.lower[idx[k]] != 0 || op.upper[idx[k]] != is.sizes[k] - 1) return false;
+      if (idx[k] >= 0 && (op.lower[idx[k]] != 0 || op.upper[idx[k]] != is.sizes[k] - 1)) return false;
     for (size_t v = 0; v < n.nIdx; ++v)
       if (n.active[v] && static_cast<int>(v) != on && static_cast<int>(v) != oc && static_cast<int>(v) != iy &&
           static_cast<int>(v) != ix)
@@ -1573,13 +1584,10 @@ class Planner {
       // re-use the spatial matcher by hand
       std::vector<bool> in_out(n.nIdx, false);
       int oi[4];
-      for (int k = 0; k < 4; ++k) {
-        oi[k] = n.acc[0][k].plainIndex();
-        if (oi[k] < 0 || in_out[oi[k]]) return false;
-        in_out[oi[k]] = true;
-        if (n.acc[2][k].plainIndex() != oi[k]) return false;
-      }
-      if (n.acc[1][0].plainIndex() != oi[0] || n.acc[1][3].plainIndex() != oi[3]) return false;
+      if (!windowOutput(u, n, u.result->shape, oi, &in_out)) return false;
+      for (int k = 0; k < 4; ++k)
+        if (!sameIndex(n.acc[2][k], oi[k])) return false;
+      if (!sameIndex(n.acc[1][0], oi[0]) || !sameIndex(n.acc[1][3], oi[3])) return false;
       if (!spatialForm(n.acc[1][1], in_out, n.active, &sy) || !spatialForm(n.acc[1][2], in_out, n.active, &sx)) return false;
       if (sy.out_idx != oi[1] || sx.out_idx != oi[2] || sy.dil != 1 || sx.dil != 1) return false;
       if (sy.tap_idx != ky || sx.tap_idx != kx) return false;

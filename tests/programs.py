@@ -749,6 +749,9 @@ ALL = {
     'config3_xception_block_bf16': config3_xception_block,
     'config3_xception_block_f32': lambda E, op: config3_xception_block(E, op, C=16, dtype_name='FLOAT32'),
     'classifier_tail_f32': classifier_tail,
+    # one image: the batch index has a single value and is folded out of every access before kernels are matched
+    'single_image_xception_block_f32': lambda E, op: config3_xception_block(E, op, N=1, C=16, dtype_name='FLOAT32'),
+    'single_image_classifier_tail_f32': lambda E, op: classifier_tail(E, op, N=1),
     'residual_block_bf16': residual_block,
     'resnet50_tiny_bf16': resnet50_tiny,
 }

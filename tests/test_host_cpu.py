@@ -46,6 +46,15 @@ def test_plan_choices_for_the_workload_configs():
     assert t.count('conv2d bf16') + t.count('gemm bf16') == 2 and 'constant' in t and 'add(t' in t, t
 
 
+def test_one_image_keeps_the_window_kernels():
+    """At batch 1 the batch index is a constant; depthwise, pooling, window argmax and the pooling over the whole
+    image must still be matched (the reference tool benchmarks at batch 1 by default)."""
+    t = plan_of(programs.config3_xception_block(E, op, N=1)[0])
+    assert 'dwconv2d bf16' in t and 'pool2d max' in t and '+window argmax' in t and 'contract (general)' not in t, t
+    t = plan_of(programs.classifier_tail(E, op, N=1, dtype_name='BFLOAT16')[0])
+    assert 'pool2d add bf16 1x7x7x64xbf16 over the whole image' in t, t
+
+
 def test_projection_shortcut_and_main_path_share_one_launch():
     """relu(conv1x1(y) + b + conv1x1(x) + b') of a residual block with a projection shortcut is one GEMM with two
     products (plain rows, or the pixel rows of the stride-2 shortcut); `fuse=0` keeps the contractions apart."""
