@@ -154,10 +154,13 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):  # noqa: C901
     from plaidml_amd import edsl as P
     rng = np.random.default_rng(7)
     dI = hk.DeviceBuffer.from_numpy(P.to_bf16_bits(rng.standard_normal((N, H, W, C)).astype(np.float32)))  # N(0,1) as the config says
-    dD, dP = hk.DeviceBuffer(px * C * 2), hk.DeviceBuffer(px * C * 2)
+    # the depthwise result is a temporary: like the planner, give its rows a pitch of whole 128-byte lines
+    pitch = (C * 2 + 127) // 128 * 128 // 2
+    dD, dP = hk.DeviceBuffer(px * pitch * 2), hk.DeviceBuffer(px * C * 2)
     # depthwise
     d = hk.Dwconv2dDesc()
     d.dtype = hk.BF16
+    d.out_pitch = pitch
     d.n, d.h, d.w, d.c, d.kh, d.kw, d.oh, d.ow = N, H, W, C, 3, 3, H, W
     d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
     d.pad_h = d.pad_w = 1
@@ -169,7 +172,7 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):  # noqa: C901
     # pointwise + scale/shift + relu
     g = hk.GemmDesc()
     g.in_dtype = g.out_dtype = g.c_dtype = hk.BF16
-    g.m, g.n, g.k, g.lda, g.ldb, g.ldc = px, C, C, C, C, C
+    g.m, g.n, g.k, g.lda, g.ldb, g.ldc = px, C, C, pitch, C, C
     g.tail = hk.make_tail(ops=[(hk.EPI_MUL, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 1, 0.0),
                                (hk.EPI_RELU, hk.BF16, 0, 0, 0.0)], operands=[(hk.BF16, 0, 1), (hk.BF16, 0, 1)])
     pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
@@ -196,7 +199,36 @@ def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):  # noqa: C901
     out['maxpool3x3s2_argmax'] = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms / 1e6, 1), 'frac_hbm': round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
     for b in (dI, dD, dP, dF, dW, dS, dT, dM, dX):
         b.free()
+    out['block_through_exec'] = xception_program_leg(N, H, W, C)
     return out
+
+
+def xception_program_leg(N, H, W, C, runs=5):
+    """The same block as one Tile program through libplaidml.so: what the planner makes of it, device time of a run."""
+    from plaidml_amd import edsl as P, op as Pop
+    dt = P.DType.BFLOAT16
+    I, Fdw, Fpw = P.Placeholder(dt, [N, H, W, C]), P.Placeholder(dt, [3, 3, C, 1]), P.Placeholder(dt, [1, 1, C, C])
+    scale, shift = P.Placeholder(dt, [C]), P.Placeholder(dt, [C])
+    R = Pop.relu(Pop.convolution(Pop.convolution(I, Fdw, depthwise=True), Fpw) * scale + shift)
+    M = Pop.pool(R, 'max', [3, 3], [2, 2], autopad=Pop.SAME_UPPER)
+    n, x0, x1, c, k0, k1 = P.TensorIndexes(6)
+    IX = P.index([3, 3], 0) * 3 + P.index([3, 3], 1)
+    AM = P.Contraction().outShape(M.shape).outAccess(n, x0, x1, c).max(
+        P.cond(R[n, 2 * x0 + k0 - 1, 2 * x1 + k1 - 1, c], M[n, x0, x1, c], IX[k0, k1])).build()
+    prog = P.Program('xception_block', [I, Fdw, Fpw, scale, shift], [M, AM])
+    rng = np.random.default_rng(7)
+    vals = [rng.standard_normal((N, H, W, C)).astype(np.float32), (rng.standard_normal((3, 3, C, 1)) * np.sqrt(2.0 / 9)).astype(np.float32),
+            (rng.standard_normal((1, 1, C, C)) * np.sqrt(2.0 / C)).astype(np.float32), rng.uniform(0.5, 1.5, C).astype(np.float32),
+            rng.uniform(-0.5, 0.5, C).astype(np.float32)]
+    runner = P.Runner(prog, target='hip')
+    staged = runner.stage(vals)
+    best = None
+    for _ in range(runs):
+        runner.run_staged(staged)
+        st = P.last_run_stats()
+        best = st if best is None or st['kernel_ms'] < best['kernel_ms'] else best
+    plan = [l.strip() for l in dict(prog.passes)['hip-plan'].splitlines()[1:]]
+    return {'kernel_ms': round(best['kernel_ms'], 4), 'launches': int(best['launches']), 'plan': plan}
 
 
 def resnet50_leg(batch=128, runs=5):

@@ -296,7 +296,10 @@ int pml_hip_conv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream 
  * linalgx-regulate-depthwise (pmlc/dialect/linalgx/transforms/regulate_depthwise.cc:22-60). */
 typedef struct {
   int32_t dtype; /* F32 or BF16 */
-  int32_t reserved;
+  /* Elements between the starts of two output pixels; 0 = c (dense).  A larger pitch (a multiple of 16 bytes, no
+   * tail) lets a consumer that reads the result as GEMM rows see every row start on a 128-byte line; the bytes
+   * between c and the pitch are not written. */
+  int32_t out_pitch;
   int64_t n, h, w, c;
   int64_t kh, kw;
   int64_t oh, ow;

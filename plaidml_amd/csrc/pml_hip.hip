@@ -996,6 +996,12 @@ int64_t pml_hip_dwconv2d_dispatch(const pml_hip_dwconv2d_desc* d) {
     fail("dwconv2d: bad geometry or tail");
     return 0;
   }
+  if (d->out_pitch != 0 && d->out_pitch != d->c &&
+      (d->out_pitch < d->c || d->out_pitch % V != 0 || d->tail.n_ops != 0 ||
+       d->n * d->oh * d->ow * (int64_t)d->out_pitch >= ((int64_t)1 << 40))) {
+    fail("dwconv2d: the output pitch must be at least c, a whole number of 16-byte vectors, and has no tail");
+    return 0;
+  }
   Plan* p = new Plan();
   p->kind = PLAN_DWCONV;
   p->dw = *d;

@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void dwconv2d_kernel(DwconvArgs a, int64_t tot
         for (int i = 0; i < V; ++i) acc[i] += x[u][i] * w[u][i];
       }
     }
-    const int64_t o0 = pix * d.c + c0;
+    const int64_t o0 = pix * (d.out_pitch ? (int64_t)d.out_pitch : d.c) + c0;  // a pitch other than c comes without a tail
     if (d.tail.n_ops == 0 && (dt == PML_HIP_BF16 || dt == PML_HIP_F32)) {
       // no tail: one 16-byte store of the rounded values
       if constexpr (ES == 2) {
@@ -148,6 +148,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t to
   const IT cvecs = (IT)(d.c / V);
   const IT xblocks = (IT)((d.ow + kDwPx - 1) / kDwPx);
   const IT oh = (IT)d.oh, H = (IT)d.h, W = (IT)d.w, C = (IT)d.c;
+  const IT CO = d.out_pitch ? (IT)d.out_pitch : C;  // elements between two output pixels
   const int pad_h = (int)d.pad_h, pad_w = (int)d.pad_w;
   const IT stride = (IT)gridDim.x * blockDim.x;
   for (IT g = (IT)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x; g < (IT)total; g += stride) {
@@ -228,11 +229,11 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t to
       accumulate(std::false_type());
     else
       accumulate(std::true_type());
-    const IT orow = ((n * oh + (IT)oy) * (IT)d.ow + (IT)ox0) * C + c0;
+    const IT orow = ((n * oh + (IT)oy) * (IT)d.ow + (IT)ox0) * CO + c0;
 #pragma unroll
     for (int px = 0; px < kDwPx; ++px) {
       if (ox0 + px >= (int)d.ow) break;
-      const int64_t o0 = (int64_t)(orow + (IT)px * C);
+      const int64_t o0 = (int64_t)(orow + (IT)px * CO);
       if constexpr (ES == 2) {
         *(i32x4_t*)((uint16_t*)a.out + o0) = pack_bf16_rne(acc[px]);
       } else {
@@ -444,7 +445,8 @@ hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
       (d.dtype == PML_HIP_BF16 || d.dtype == PML_HIP_F32)) {
     const int64_t total4 = d.n * d.oh * ((d.ow + kDwPx - 1) / kDwPx) * (d.c / V);
     // 32-bit index arithmetic where every element offset (and the rounded-up thread count) stays below 2^31
-    const bool narrow = d.n * d.h * d.w * d.c < ((int64_t)1 << 31) - (1 << 24) && d.n * d.oh * d.ow * d.c < ((int64_t)1 << 31) - (1 << 24);
+    const int64_t opitch = d.out_pitch ? (int64_t)d.out_pitch : d.c;
+    const bool narrow = d.n * d.h * d.w * d.c < ((int64_t)1 << 31) - (1 << 24) && d.n * d.oh * d.ow * opitch < ((int64_t)1 << 31) - (1 << 24);
     if (es == 2 && narrow)
       hipLaunchKernelGGL((dwconv3x3_kernel<2, uint32_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
     else if (es == 2)

@@ -67,7 +67,7 @@ class Conv2dDesc(ctypes.Structure):
 
 
 class Dwconv2dDesc(ctypes.Structure):
-    _fields_ = [('dtype', i32), ('reserved', i32), ('n', i64), ('h', i64), ('w', i64), ('c', i64), ('kh', i64),
+    _fields_ = [('dtype', i32), ('out_pitch', i32), ('n', i64), ('h', i64), ('w', i64), ('c', i64), ('kh', i64),
                 ('kw', i64), ('oh', i64), ('ow', i64), ('stride_h', i64), ('stride_w', i64), ('dil_h', i64),
                 ('dil_w', i64), ('pad_h', i64), ('pad_w', i64), ('tail', Epilogue)]
 

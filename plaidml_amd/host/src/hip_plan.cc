@@ -187,6 +187,7 @@ class Planner {
       plan_->steps.push_back(s);
     }
     if (opt_.fuse && opt_.specialise) fuseSecondProducts();
+    if (opt_.specialise) padDepthwiseResults();
     pruneDeadSteps();
     return plan_;
   }
@@ -325,6 +326,43 @@ class Planner {
         F.text = ss.str();
       }
       plan_->steps[y] = F;  // X is left without readers and is dropped by pruneDeadSteps
+    }
+  }
+
+  // A depthwise convolution whose result is a temporary that only one matrix product reads as its left-hand rows
+  // (the depthwise-separable block): when a pixel's channels do not fill whole 128-byte lines (728 bf16 = 1456
+  // bytes), the temporary gets a row pitch that does, so every GEMM row starts on a line; the depthwise kernel
+  // writes with that pitch, the GEMM reads with it as its leading dimension.  The layout of a temporary is the
+  // planner's to choose (the reference sizes and places its temporaries itself too, pmlc/target/x86/pipeline.cc:289-360).
+  void padDepthwiseResults() {
+    for (size_t x = 0; x < plan_->steps.size(); ++x) {
+      Step& X = plan_->steps[x];
+      if (X.kind != Step::Dwconv2d || X.dw.tail.n_ops != 0 || !X.outs.empty() || X.c < 0) continue;
+      if (plan_->buffers[X.c].kind != BufferInfo::Temp) continue;
+      const int es = X.dw.dtype == PML_HIP_F32 ? 4 : 2;
+      const int64_t row_bytes = X.dw.c * es;
+      if (row_bytes % 128 == 0 || row_bytes < 512) continue;
+      const int64_t pitch = (row_bytes + 127) / 128 * 128 / es;
+      const int64_t rows = X.dw.n * X.dw.oh * X.dw.ow;
+      if (pitch >= (int64_t{1} << 31)) continue;
+      int readers = 0, writers = 0, y = -1;
+      for (size_t k = 0; k < plan_->steps.size(); ++k) {
+        const Step& s = plan_->steps[k];
+        for (int r : {s.a, s.b, s.init, s.a2, s.b2, s.init2}) readers += r == X.c;
+        for (int r : s.operands) readers += r == X.c;
+        writers += s.c == X.c;
+        writers += s.out2 == X.c;
+        for (int w : s.outs) writers += w == X.c;
+        if (s.a == X.c && k > x) y = static_cast<int>(k);
+      }
+      if (readers != 1 || writers != 1 || y < 0) continue;
+      Step& Y = plan_->steps[y];
+      if (Y.kind != Step::Gemm || Y.a_off != 0 || Y.gemm.m != rows || Y.gemm.k != X.dw.c || Y.gemm.lda != X.dw.c) continue;
+      X.dw.out_pitch = static_cast<int32_t>(pitch);
+      Y.gemm.lda = pitch;
+      plan_->buffers[X.c].bytes = static_cast<size_t>(rows * pitch * es);
+      X.text += " (row pitch " + std::to_string(pitch) + ")";
+      Y.text += " (lda " + std::to_string(pitch) + ")";
     }
   }
 

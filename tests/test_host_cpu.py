@@ -46,6 +46,22 @@ def test_plan_choices_for_the_workload_configs():
     assert t.count('conv2d bf16') + t.count('gemm bf16') == 2 and 'constant' in t and 'add(t' in t, t
 
 
+def test_depthwise_temporary_gets_a_pitch_of_whole_lines():
+    """728 bf16 channels are 1456 bytes: the depthwise result that only the pointwise product reads is laid out with
+    768 elements per pixel; 64 channels (128 bytes) need nothing, and a depthwise result that is a program output
+    keeps its dense layout."""
+    t = plan_of(programs.config3_xception_block(E, op, N=2, C=728)[0])
+    assert '(row pitch 768)' in t and '(lda 768)' in t, t
+    t = plan_of(programs.config3_xception_block(E, op, N=2, C=64)[0])
+    assert 'row pitch' not in t and 'lda' not in t, t
+    dt = E.DType.BFLOAT16
+    I, F = E.Placeholder(dt, [1, 9, 9, 328]), E.Placeholder(dt, [3, 3, 328, 1])
+    t = plan_of(E.Program('dw', [I, F], [op.convolution(I, F, depthwise=True)]))
+    assert 'dwconv2d' in t and 'row pitch' not in t, t
+    t = plan_of(programs.config3_xception_block(E, op, N=2, C=728)[0], 'hip{specialise=0}')
+    assert 'row pitch' not in t
+
+
 def test_one_image_keeps_the_window_kernels():
     """At batch 1 the batch index is a constant; depthwise, pooling, window argmax and the pooling over the whole
     image must still be matched (the reference tool benchmarks at batch 1 by default)."""

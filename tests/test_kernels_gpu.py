@@ -683,6 +683,48 @@ def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad):
     hk.lib().pml_hip_plan_free(plan)
 
 
+@pytest.mark.parametrize('kind,N,H,W,C,k,stride,pad', DW_CASES[:3] + DW_CASES[4:])
+def test_dwconv_output_pitch(kind, N, H, W, C, k, stride, pad):
+    """With an output pitch the same values land `pitch` elements apart, bit for bit, and the bytes between a
+    pixel's channels and the next pixel are left alone; a pitch that is no whole number of 16-byte vectors, or
+    smaller than c, or combined with a tail, is refused."""
+    rng = np.random.default_rng(91)
+    es, npdt = (2, np.uint16) if kind == 'bf16' else (4, np.float32)
+    Iv = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    Fv = (rng.standard_normal((k, k, C, 1)) * 0.3).astype(np.float32)
+    OH, OW = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    pitch = C + 3 * (16 // es)
+    outs = []
+    for op_pitch in (0, pitch):
+        d = hk.Dwconv2dDesc()
+        d.dtype = hk.BF16 if kind == 'bf16' else hk.F32
+        d.out_pitch = op_pitch
+        d.n, d.h, d.w, d.c, d.kh, d.kw, d.oh, d.ow = N, H, W, C, k, k, OH, OW
+        d.stride_h = d.stride_w = stride
+        d.dil_h = d.dil_w = 1
+        d.pad_h = d.pad_w = pad
+        plan = hk.lib().pml_hip_dwconv2d_dispatch(ctypes.byref(d))
+        assert plan, hk.lib().pml_hip_last_error()
+        dI = hk.DeviceBuffer.from_numpy(bf16(Iv) if kind == 'bf16' else Iv)
+        dF = hk.DeviceBuffer.from_numpy(bf16(Fv) if kind == 'bf16' else Fv)
+        width = op_pitch or C
+        dO = hk.DeviceBuffer.from_numpy(np.full((N * OH * OW, width), 0x1234 if kind == 'bf16' else 7.5, npdt))
+        hk.check(hk.lib().pml_hip_dwconv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, hk.ptr_array([]), hk.ptr_array([]), None))
+        hk.check(hk.lib().pml_hip_stream_sync(None))
+        outs.append(dO.to_numpy(npdt, (N * OH * OW, width)))
+        hk.lib().pml_hip_plan_free(plan)
+    dense, pitched = outs
+    np.testing.assert_array_equal(pitched[:, :C].view(np.uint16 if es == 2 else np.uint32), dense.view(np.uint16 if es == 2 else np.uint32))
+    assert (pitched[:, C:] == (0x1234 if kind == 'bf16' else 7.5)).all()
+    for bad in (C - 16 // es, C + 1):
+        d.out_pitch = bad
+        assert hk.lib().pml_hip_dwconv2d_dispatch(ctypes.byref(d)) == 0
+        assert 'output pitch' in hk.lib().pml_hip_last_error().decode()
+    d.out_pitch = pitch
+    d.tail = hk.make_tail(ops=[(hk.EPI_RELU, d.dtype, 0, 0, 0.0)], operands=[])
+    assert hk.lib().pml_hip_dwconv2d_dispatch(ctypes.byref(d)) == 0
+
+
 def test_dwconv_pool_bf16():
     rng = np.random.default_rng(9)
     N, H, W, C = 2, 19, 19, 32
