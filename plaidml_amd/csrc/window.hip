@@ -244,6 +244,155 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(DwconvArgs a, int64_t to
   }
 }
 
+// The same work for tensors below 2 GiB, as one straight line of code for interior and border pixels alike.
+// The input is read through a buffer descriptor: a tap outside the image gets an offset beyond the buffer and
+// arrives as zeros, so no lane branches around it and a wavefront whose lanes sit on both sides of an image border
+// does not run two code paths one after the other.  A zero times a finite weight adds nothing, which is what
+// leaving the tap out means; only a weight that is infinite or NaN would turn such a zero into NaN.  Every lane
+// therefore looks at its nine filter vectors once, and the (rare) lanes that hold such a weight and sit on a border
+// redo their sums from the same registers with the outside taps left out.  Indices come from multiply-and-shift
+// divisions prepared on the host.
+struct DwFlatArgs {
+  unsigned total;      // threads with work: images x rows x pixel blocks x channel vectors
+  unsigned cvecs, xblocks, oh;
+  unsigned cv_magic, xb_magic, oh_magic;
+  int cv_shift, xb_shift, oh_shift;
+  unsigned in_bytes;
+};
+
+template <int ES>
+__global__ __launch_bounds__(256, 3) void dwconv3x3_flat_kernel(DwconvArgs a, DwFlatArgs f) {
+  constexpr int V = VecIO<ES>::V;
+  constexpr int kCols = kDwPx + 2;
+  const pml_hip_dwconv2d_desc& d = a.d;
+  const unsigned g = xcd_contiguous_block(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
+  if (g >= f.total) return;
+  const unsigned t1 = fast_div(g, f.cv_magic, f.cv_shift), cv = g - t1 * f.cvecs;
+  const unsigned t2 = fast_div(t1, f.xb_magic, f.xb_shift), xb = t1 - t2 * f.xblocks;
+  const unsigned n = fast_div(t2, f.oh_magic, f.oh_shift), oy = t2 - n * f.oh;
+  const int H = (int)d.h, W = (int)d.w;
+  const unsigned pix_bytes = (unsigned)d.c * ES, c0b = cv * 16u;
+  const int ox0 = (int)xb * kDwPx, iy0 = (int)oy - (int)d.pad_h, ix0 = ox0 - (int)d.pad_w;
+  constexpr unsigned kOutside = 0x80000000u;  // beyond any buffer this kernel is launched for
+
+  i32x4_t wr[9];
+#pragma unroll
+  for (int k = 0; k < 9; ++k) wr[k] = *(const i32x4_t*)((const unsigned char*)a.filter + (unsigned)k * pix_bytes + c0b);
+
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc((void*)a.in, 0, (int)f.in_bytes, 0x00020000u);
+  bool row_ok[3], col_ok[kCols];
+  unsigned col_off[kCols];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    col_ok[c] = (unsigned)(ix0 + c) < (unsigned)W;
+    col_off[c] = col_ok[c] ? (unsigned)(ix0 + c) * pix_bytes + c0b : kOutside;
+  }
+  i32x4_t xr[3][kCols];
+  auto load_row = [&](int ky) {
+    const unsigned row = row_ok[ky] ? (n * (unsigned)H + (unsigned)(iy0 + ky)) * (unsigned)W * pix_bytes : kOutside;
+#pragma unroll
+    for (int c = 0; c < kCols; ++c)  // an offset with the top bit set lies beyond the buffer
+      xr[ky][c] = __builtin_amdgcn_raw_buffer_load_b128(rin, (int)(row | col_off[c]) < 0 ? (int)kOutside : (int)(row + col_off[c]), 0, 0);
+  };
+#pragma unroll
+  for (int ky = 0; ky < 3; ++ky) row_ok[ky] = (unsigned)(iy0 + ky) < (unsigned)H;
+  // The third window row is requested after the first has been used, into the registers the first leaves free; it
+  // arrives during the second row's arithmetic.  With all three up front the kernel needs more than the 168
+  // registers that let three wavefronts share a SIMD.
+  load_row(0);
+  load_row(1);
+
+  // does this lane hold a weight that is infinite or NaN (all exponent bits set)?
+  unsigned odd = 0;
+#pragma unroll
+  for (int k = 0; k < 9; ++k)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned w = (unsigned)wr[k][i];
+      if constexpr (ES == 2)
+        odd |= ((w & 0x7f807f80u) + 0x00800080u) & 0x80008000u;  // a carry out of either exponent field
+      else
+        odd |= ((w & 0x7f800000u) + 0x00800000u) & 0x80000000u;
+    }
+
+  auto unpack = [](const i32x4_t& raw, float* o) {
+    if constexpr (ES == 2) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        o[2 * i] = __uint_as_float(((uint32_t)raw[i]) << 16);
+        o[2 * i + 1] = __uint_as_float(((uint32_t)raw[i]) & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = __int_as_float(raw[i]);
+    }
+  };
+  float acc[kDwPx][V];
+  // taps in the reference's order (ky outer, kx inner) for every pixel
+  auto accumulate = [&](auto checked) {
+#pragma unroll
+    for (int px = 0; px < kDwPx; ++px)
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[px][i] = 0.f;
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+      // (the second pass reads its operands through an empty asm: shared subexpressions of the two passes would
+      // otherwise keep every unpacked value of the first alive for the second)
+      auto fresh = [](i32x4_t v) {
+        if (decltype(checked)::value) asm volatile("" : "+v"(v));
+        return v;
+      };
+      float w[3][V];
+#pragma unroll
+      for (int kx = 0; kx < 3; ++kx) unpack(fresh(wr[ky * 3 + kx]), w[kx]);
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) {
+        if (decltype(checked)::value && !(row_ok[ky] && col_ok[c])) continue;
+        float x[V];
+        unpack(fresh(xr[ky][c]), x);
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+          const int px = c - kx;
+          if (px < 0 || px >= kDwPx) continue;
+#pragma unroll
+          for (int i = 0; i < V; ++i) acc[px][i] += x[i] * w[kx][i];
+        }
+      }
+      // one filter row at a time: unpacked values of later rows would only take registers
+      __builtin_amdgcn_sched_barrier(0);
+      if (!decltype(checked)::value && ky == 0) {
+        load_row(2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  accumulate(std::false_type());
+  const bool border = !(row_ok[0] && row_ok[2] && col_ok[0] && col_ok[kCols - 1]);
+  if (odd != 0 && border) {
+    // everything again from memory (the registers of the first pass have been given up by now)
+#pragma unroll
+    for (int k = 0; k < 9; ++k) wr[k] = *(const i32x4_t*)((const unsigned char*)a.filter + (unsigned)k * pix_bytes + c0b);
+    load_row(0);
+    load_row(1);
+    load_row(2);
+    accumulate(std::true_type());
+  }
+
+  const unsigned opix_bytes = (d.out_pitch ? (unsigned)d.out_pitch : (unsigned)d.c) * ES;
+  const unsigned orow = ((n * f.oh + oy) * (unsigned)d.ow + (unsigned)ox0) * opix_bytes + c0b;
+#pragma unroll
+  for (int px = 0; px < kDwPx; ++px) {
+    if (ox0 + px >= (int)d.ow) break;
+    unsigned char* o = (unsigned char*)a.out + orow + (unsigned)px * opix_bytes;
+    if constexpr (ES == 2) {
+      *(i32x4_t*)o = pack_bf16_rne(acc[px]);
+    } else {
+      const f32x4_t v = {acc[px][0], acc[px][1], acc[px][2], acc[px][3]};
+      *(f32x4_t*)o = v;
+    }
+  }
+}
+
 // IT: the integer type of the index arithmetic (32 bits where every element offset stays below 2^31).
 // AGG: the aggregation (PML_HIP_AGG_*), a compile-time constant so that the tap loop is straight-line code.
 template <int ES, bool WITH_INDEX, typename IT, int AGG>
@@ -447,7 +596,21 @@ hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
     // 32-bit index arithmetic where every element offset (and the rounded-up thread count) stays below 2^31
     const int64_t opitch = d.out_pitch ? (int64_t)d.out_pitch : d.c;
     const bool narrow = d.n * d.h * d.w * d.c < ((int64_t)1 << 31) - (1 << 24) && d.n * d.oh * d.ow * opitch < ((int64_t)1 << 31) - (1 << 24);
-    if (es == 2 && narrow)
+    const bool small = d.n * d.h * d.w * d.c * es < ((int64_t)1 << 31) && d.n * d.oh * d.ow * opitch * es < ((int64_t)1 << 31);
+    if (small) {
+      DwFlatArgs f;
+      f.total = (unsigned)total4;
+      f.cvecs = (unsigned)(d.c / V), f.xblocks = (unsigned)((d.ow + kDwPx - 1) / kDwPx), f.oh = (unsigned)d.oh;
+      fast_div_magic(f.cvecs, &f.cv_magic, &f.cv_shift);
+      fast_div_magic(f.xblocks, &f.xb_magic, &f.xb_shift);
+      fast_div_magic(f.oh, &f.oh_magic, &f.oh_shift);
+      f.in_bytes = (unsigned)(d.n * d.h * d.w * d.c * es);
+      const unsigned blocks = (unsigned)((total4 + 255) / 256);
+      if (es == 2)
+        hipLaunchKernelGGL((dwconv3x3_flat_kernel<2>), dim3(blocks), dim3(256), 0, s, a, f);
+      else
+        hipLaunchKernelGGL((dwconv3x3_flat_kernel<4>), dim3(blocks), dim3(256), 0, s, a, f);
+    } else if (es == 2 && narrow)
       hipLaunchKernelGGL((dwconv3x3_kernel<2, uint32_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
     else if (es == 2)
       hipLaunchKernelGGL((dwconv3x3_kernel<2, int64_t>), dim3(grid_for(total4)), dim3(256), 0, s, a, total4);
