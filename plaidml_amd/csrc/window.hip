@@ -497,6 +497,104 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
   }
 }
 
+// Pooling windows of up to 3 x 3 taps over tensors below 2 GiB as one straight line of code: indices from
+// multiply-and-shift divisions, the taps read through a buffer descriptor (a tap outside the image gets an offset
+// beyond the buffer; what arrives for it is never looked at: its comparisons are masked), no loop over the window
+// and no second code path for windows that cross the image border.
+struct PoolFlatArgs {
+  unsigned total;  // output pixels x channel vectors
+  unsigned cvecs, ow, oh;
+  unsigned cv_magic, ow_magic, oh_magic;
+  int cv_shift, ow_shift, oh_shift;
+  unsigned in_bytes;
+};
+
+template <int ES, bool WITH_INDEX, int AGG, int KH, int KW>
+__global__ __launch_bounds__(256) void pool_flat_kernel(PoolArgs a, PoolFlatArgs f) {
+  constexpr int V = VecIO<ES>::V;
+  const pml_hip_pool2d_desc& d = a.d;
+  const unsigned g = xcd_contiguous_block(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
+  if (g >= f.total) return;
+  const unsigned pix = fast_div(g, f.cv_magic, f.cv_shift), cv = g - pix * f.cvecs;
+  const unsigned t = fast_div(pix, f.ow_magic, f.ow_shift), ox = pix - t * f.ow;
+  const unsigned n = fast_div(t, f.oh_magic, f.oh_shift), oy = t - n * f.oh;
+  const int H = (int)d.h, W = (int)d.w;
+  const unsigned pix_bytes = (unsigned)d.c * ES, c0b = cv * 16u;
+  const int iy0 = (int)oy * (int)d.stride_h - (int)d.pad_h, ix0 = (int)ox * (int)d.stride_w - (int)d.pad_w;
+  constexpr unsigned kOutside = 0x80000000u;
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc((void*)a.in, 0, (int)f.in_bytes, 0x00020000u);
+  bool row_ok[KH], col_ok[KW];
+  unsigned col_off[KW];
+#pragma unroll
+  for (int kx = 0; kx < KW; ++kx) {
+    col_ok[kx] = (unsigned)(ix0 + kx) < (unsigned)W;
+    col_off[kx] = col_ok[kx] ? (unsigned)(ix0 + kx) * pix_bytes + c0b : kOutside;
+  }
+  i32x4_t xr[KH][KW];
+#pragma unroll
+  for (int ky = 0; ky < KH; ++ky) {
+    row_ok[ky] = (unsigned)(iy0 + ky) < (unsigned)H;
+    const unsigned row = row_ok[ky] ? (n * (unsigned)H + (unsigned)(iy0 + ky)) * (unsigned)W * pix_bytes : kOutside;
+#pragma unroll
+    for (int kx = 0; kx < KW; ++kx)
+      xr[ky][kx] = __builtin_amdgcn_raw_buffer_load_b128(rin, (int)(row | col_off[kx]) < 0 ? (int)kOutside : (int)(row + col_off[kx]), 0, 0);
+  }
+  float acc[V];
+  int best[V];  // with_index: largest window index whose (in-range) tap equals the pooled value; 0 if none
+  const float ident = AGG == PML_HIP_AGG_MAX ? -INFINITY : (AGG == PML_HIP_AGG_MIN ? INFINITY : 0.f);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    acc[i] = ident;
+    best[i] = 0;
+  }
+#pragma unroll
+  for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+    for (int kx = 0; kx < KW; ++kx) {
+      const bool live = row_ok[ky] && col_ok[kx];
+      const int k = ky * KW + kx;
+      float x[V];
+      if constexpr (ES == 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          x[2 * i] = __uint_as_float(((uint32_t)xr[ky][kx][i]) << 16);
+          x[2 * i + 1] = __uint_as_float(((uint32_t)xr[ky][kx][i]) & 0xffff0000u);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = __int_as_float(xr[ky][kx][i]);
+      }
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        if constexpr (AGG == PML_HIP_AGG_MAX) {
+          // taps come in rising window index, so ">=" leaves the largest index among equal values
+          if (WITH_INDEX) best[i] = (live & (x[i] >= acc[i])) ? k : best[i];
+          acc[i] = (live & (x[i] > acc[i])) ? x[i] : acc[i];
+        } else if constexpr (AGG == PML_HIP_AGG_MIN) {
+          if (WITH_INDEX) best[i] = (live & (x[i] <= acc[i])) ? k : best[i];
+          acc[i] = (live & (x[i] < acc[i])) ? x[i] : acc[i];
+        } else {
+          acc[i] += live ? x[i] : 0.f;
+        }
+      }
+    }
+  const unsigned o0 = pix * (unsigned)d.c + cv * V;  // in elements
+  if constexpr (ES == 2) {
+    *(i32x4_t*)((uint16_t*)a.out + o0) = pack_bf16_rne(acc);
+  } else {
+    const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
+    *(f32x4_t*)((float*)a.out + o0) = o;
+  }
+  if (WITH_INDEX) {
+    int32_t* ip = (int32_t*)a.idx + o0;
+#pragma unroll
+    for (int i = 0; i < V; i += 4) {
+      const i32x4_t w = {best[i], best[i + 1], best[i + 2], best[i + 3]};
+      *(i32x4_t*)(ip + i) = w;
+    }
+  }
+}
+
 inline unsigned grid_for(int64_t items) {
   int64_t blocks = (items + 255) / 256;
   if (blocks < 1) blocks = 1;
@@ -719,6 +817,45 @@ hipError_t pool2d_launch(const PoolArgs& a, hipStream_t s) {
         hipLaunchKernelGGL((pool_whole_kernel<4>), dim3((unsigned)(d.n * chunks)), dim3(256), 0, s, a, chunks);
       return hipGetLastError();
     }
+  }
+  // windows of 3x3 or 2x2 taps over small tensors: the straight-line kernel
+  const bool small = d.n * d.h * d.w * d.c * es < ((int64_t)1 << 31) && d.n * d.oh * d.ow * d.c * 4 < ((int64_t)1 << 31) &&
+                     (d.dtype == PML_HIP_BF16 || d.dtype == PML_HIP_F32);
+  if (small && d.kh == d.kw && (d.kh == 3 || d.kh == 2)) {
+    PoolFlatArgs f;
+    f.total = (unsigned)total;
+    f.cvecs = (unsigned)(d.c / V), f.ow = (unsigned)d.ow, f.oh = (unsigned)d.oh;
+    fast_div_magic(f.cvecs, &f.cv_magic, &f.cv_shift);
+    fast_div_magic(f.ow, &f.ow_magic, &f.ow_shift);
+    fast_div_magic(f.oh, &f.oh_magic, &f.oh_shift);
+    f.in_bytes = (unsigned)(d.n * d.h * d.w * d.c * es);
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    auto go = [&](auto es_tag, auto idx_tag, auto agg_tag) {
+      constexpr int kEs = decltype(es_tag)::value, kAgg = decltype(agg_tag)::value;
+      constexpr bool kIdx = decltype(idx_tag)::value;
+      if (d.kh == 3)
+        hipLaunchKernelGGL((pool_flat_kernel<kEs, kIdx, kAgg, 3, 3>), dim3(blocks), dim3(256), 0, s, a, f);
+      else
+        hipLaunchKernelGGL((pool_flat_kernel<kEs, kIdx, kAgg, 2, 2>), dim3(blocks), dim3(256), 0, s, a, f);
+    };
+    auto with_agg = [&](auto es_tag, auto idx_tag) {
+      switch (d.agg) {
+        case PML_HIP_AGG_MAX: go(es_tag, idx_tag, std::integral_constant<int, PML_HIP_AGG_MAX>()); break;
+        case PML_HIP_AGG_MIN: go(es_tag, idx_tag, std::integral_constant<int, PML_HIP_AGG_MIN>()); break;
+        default: go(es_tag, idx_tag, std::integral_constant<int, PML_HIP_AGG_ADD>()); break;
+      }
+    };
+    auto with_index = [&](auto es_tag) {
+      if (d.with_index)
+        with_agg(es_tag, std::true_type());
+      else
+        with_agg(es_tag, std::false_type());
+    };
+    if (es == 2)
+      with_index(std::integral_constant<int, 2>());
+    else
+      with_index(std::integral_constant<int, 4>());
+    return hipGetLastError();
   }
   // 32-bit index arithmetic where every element offset (and the rounded-up thread count) stays below 2^31
   const bool narrow = d.n * d.h * d.w * d.c < ((int64_t)1 << 31) - (1 << 24) && d.n * d.oh * d.ow * d.c < ((int64_t)1 << 31) - (1 << 24);
