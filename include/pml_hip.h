@@ -245,6 +245,11 @@ int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s);
  * Random values make the chip lower its clock: the second figure is the ceiling a GEMM on N(0,1) data can reach. */
 int pml_hip_probe_mfma(int random_data, int iters, double* tflops, double* core_mhz);
 
+/* Test aid (host arithmetic only, no device call; no counterpart in the reference): the tile (row block, column block)
+ * that workgroup `workgroup` of a tiles_m x tiles_n GEMM grid works on.  The order keeps the tiles an XCD holds at any
+ * time a compact block of the grid; the tests check that it visits every tile exactly once. */
+int pml_hip_tile_of_workgroup(int tiles_m, int tiles_n, int workgroup, int* tile_m, int* tile_n);
+
 /* The GEMM above in one call that allocates nothing, neither on the host heap of the device runtime nor in
  * device memory: dispatch + invoke without a plan object.  It has no counterpart in the reference; it is for
  * callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid

@@ -54,48 +54,6 @@ constexpr unsigned kOutside = 0x80000000u;     // ... and this one reads as zero
 // Sum of two byte offsets, each of which may be the "outside" mark.
 __device__ inline unsigned join_offsets(unsigned x, unsigned y) { return ((x | y) & kOutside) ? kOutside : x + y; }
 
-// XCD-aware tile order.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its
-// own L2, and a CU takes the next id of its XCD when it falls free: the workgroups resident on an XCD at any
-// time are a run of about 32 consecutive "local" numbers bid / 8.  What such a run costs the L2 is the
-// number of distinct A rows plus Bt rows under its tiles, so a run should be a compact block, not a strip,
-// and above all the tiles that share an A row block must not be dealt to eight different L2s (a 181 x 6
-// grid in workgroup-id order fetched A 6.5 times from memory).  XCD x therefore owns a contiguous range of
-// tile numbers t (the ranges differ by at most one tile when the count is no multiple of 8), and t walks
-// the grid in blocks of TH x TW tiles (32 tiles, as square as the grid allows).  When the grid divides into
-// whole blocks, blocks are numbered row-major and walked row-major; otherwise t walks groups of TH tile rows
-// column by column, the last group being as short as the grid leaves it.  (4096^2 with 256x256 tiles: 2 x 16
-// strips fetch 576 KB per K-slab and XCD, 4 x 8 blocks 384 KB; what misses L2 comes over the fabric from the
-// last-level cache, whose bandwidth is the scarce one.)
-__device__ inline void xcd_tile(int bid, int tiles_m, int tiles_n, int* tm, int* tn) {
-  constexpr int kXcds = 8, kRun = 32;
-  const int nblocks = tiles_m * tiles_n;
-  const int per = nblocks / kXcds, rem = nblocks % kXcds;
-  const int x = bid % kXcds;
-  const int t = x * per + (x < rem ? x : rem) + bid / kXcds;  // contiguous range per XCD
-  if (rem == 0 && per % kRun == 0) {
-    int th = 0, tw = 0;
-    if (tiles_m % 4 == 0 && tiles_n % 8 == 0) { th = 4; tw = 8; }
-    else if (tiles_m % 8 == 0 && tiles_n % 4 == 0) { th = 8; tw = 4; }
-    else if (tiles_m % 16 == 0 && tiles_n % 2 == 0) { th = 16; tw = 2; }
-    else if (tiles_m % 2 == 0 && tiles_n % 16 == 0) { th = 2; tw = 16; }
-    if (th) {
-      const int blk = t / kRun, in = t % kRun;
-      const int blocks_n = tiles_n / tw;
-      *tm = (blk / blocks_n) * th + in / tw;
-      *tn = (blk % blocks_n) * tw + in % tw;
-      return;
-    }
-  }
-  const int tw = tiles_n < 8 ? tiles_n : 8;
-  const int th = kRun / tw;
-  const int group = th * tiles_n;                      // tiles in a group of th tile rows
-  const int first_m = (t / group) * th;
-  const int rows = tiles_m - first_m < th ? tiles_m - first_m : th;
-  const int in = t % group;
-  *tm = first_m + in % rows;
-  *tn = in / rows;
-}
-
 // STAGES = 0: as many as pay for the tile; 2: two, and LDS rounded up to what staging the whole result
 // tile needs (a short-K, bandwidth-bound GEMM gains more from a second workgroup on the CU than from a
 // third slab in flight)
@@ -169,10 +127,8 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   const int wk = wave / (WAVES_M * WAVES_N);  // which part of every slab's K-blocks
   const int wm = (wave % (WAVES_M * WAVES_N)) / WAVES_N, wn = wave % WAVES_N;
 
-  const int tiles_n = (int)((p.N + BN - 1) / BN);
-  const int tiles_m = (int)((p.M + BM - 1) / BM);
   int tile_m, tile_n;
-  xcd_tile(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
+  tile_of(p.order, blockIdx.x, &tile_m, &tile_n);
   const int64_t m0 = (int64_t)tile_m * BM;
   const int64_t n0 = (int64_t)tile_n * BN;
 
@@ -657,12 +613,16 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
 
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
-  const int64_t tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  const int64_t tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int64_t tiles = tiles_m * tiles_n;
+  if (tiles <= 0 || tiles >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
   const size_t lds = Ring<BM, BN, STAGES, SLAB>::kAlloc;
   auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB>;
   static DynamicLdsLimit limit;
   if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), lds, s, a);
+  IgemmArgs b = a;
+  b.order = make_tile_order((int)tiles_m, (int)tiles_n);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), lds, s, b);
   return hipGetLastError();
 }
 

@@ -58,7 +58,83 @@ __device__ inline unsigned fast_div(unsigned n, unsigned magic, int shift) {
 }
 #endif
 
+// XCD-aware tile order of the GEMM grid, prepared on the host so that a workgroup finds its tile with a few
+// scalar multiplies (the divisions by run-time grid sizes took about 150 vector instructions per wavefront).
+// Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own L2, and a CU takes the next
+// id of its XCD when it falls free: the workgroups resident on an XCD at any time are a run of about 32 consecutive
+// "local" numbers bid / 8.  What such a run costs the L2 is the number of distinct A rows plus Bt rows under its
+// tiles, so a run should be a compact block, not a strip, and above all the tiles that share an A row block must
+// not be dealt to eight different L2s (a 181 x 6 grid in workgroup-id order fetched A 6.5 times from memory).
+// XCD x therefore owns a contiguous range of tile numbers t (the ranges differ by at most one tile when the count
+// is no multiple of 8), and t walks the grid in blocks of th x tw tiles (32 tiles, as square as the grid allows).
+// When the grid divides into whole blocks, blocks are numbered row-major and walked row-major; otherwise t walks
+// groups of th tile rows column by column, the last group being as short as the grid leaves it.  (4096^2 with
+// 256x256 tiles: 2 x 16 strips fetch 576 KB per K-slab and XCD, 4 x 8 blocks 384 KB; what misses L2 comes over the
+// fabric from the last-level cache, whose bandwidth is the scarce one.)
+struct TileOrder {
+  int per, rem;                    // tiles per XCD; the first `rem` XCDs take one more
+  int blocked;                     // 1: whole th x tw blocks (tw a power of two), 0: groups of th tile rows
+  int th, tw_shift, blocks_n;      // blocked
+  int group, last_rows, tiles_m;   // grouped: tiles in a full group, tile rows of the last group
+  unsigned bn_magic, group_magic, th_magic, last_magic;
+  int bn_shift, group_shift, th_shift, last_shift;
+};
+inline TileOrder make_tile_order(int tiles_m, int tiles_n) {
+  constexpr int kXcds = 8, kRun = 32;
+  TileOrder o{};
+  const int nblocks = tiles_m * tiles_n;
+  o.per = nblocks / kXcds;
+  o.rem = nblocks % kXcds;
+  o.tiles_m = tiles_m;
+  int th = 0, tw = 0;
+  if (o.rem == 0 && o.per % kRun == 0) {
+    if (tiles_m % 4 == 0 && tiles_n % 8 == 0) { th = 4; tw = 8; }
+    else if (tiles_m % 8 == 0 && tiles_n % 4 == 0) { th = 8; tw = 4; }
+    else if (tiles_m % 16 == 0 && tiles_n % 2 == 0) { th = 16; tw = 2; }
+    else if (tiles_m % 2 == 0 && tiles_n % 16 == 0) { th = 2; tw = 16; }
+  }
+  if (th) {
+    o.blocked = 1;
+    o.th = th;
+    while ((1 << o.tw_shift) < tw) ++o.tw_shift;
+    o.blocks_n = tiles_n / tw;
+    fast_div_magic((unsigned)o.blocks_n, &o.bn_magic, &o.bn_shift);
+    return o;
+  }
+  tw = tiles_n < 8 ? tiles_n : 8;
+  o.th = kRun / tw;
+  o.group = o.th * tiles_n;
+  o.last_rows = tiles_m % o.th ? tiles_m % o.th : o.th;
+  fast_div_magic((unsigned)o.group, &o.group_magic, &o.group_shift);
+  fast_div_magic((unsigned)o.th, &o.th_magic, &o.th_shift);
+  fast_div_magic((unsigned)o.last_rows, &o.last_magic, &o.last_shift);
+  return o;
+}
+#if defined(__HIPCC__)
+__host__ __device__
+#endif
+inline void tile_of(const TileOrder& o, unsigned bid, int* tm, int* tn) {
+  const unsigned x = bid & 7u;
+  const unsigned t = x * (unsigned)o.per + (x < (unsigned)o.rem ? x : (unsigned)o.rem) + (bid >> 3);
+  auto div = [](unsigned n, unsigned magic, int shift) { return (unsigned)(((unsigned long long)n * magic) >> shift); };
+  if (o.blocked) {
+    const unsigned blk = t >> 5, in = t & 31u;
+    const unsigned q = div(blk, o.bn_magic, o.bn_shift), r = blk - q * (unsigned)o.blocks_n;
+    *tm = (int)(q * (unsigned)o.th + (in >> o.tw_shift));
+    *tn = (int)((r << o.tw_shift) + (in & ((1u << o.tw_shift) - 1u)));
+    return;
+  }
+  const unsigned gi = div(t, o.group_magic, o.group_shift), in = t - gi * (unsigned)o.group;
+  const unsigned first_m = gi * (unsigned)o.th;
+  const bool last = (unsigned)o.tiles_m - first_m < (unsigned)o.th;
+  const unsigned rows = last ? (unsigned)o.last_rows : (unsigned)o.th;
+  const unsigned q = last ? div(in, o.last_magic, o.last_shift) : div(in, o.th_magic, o.th_shift);
+  *tm = (int)(first_m + in - q * rows);
+  *tn = (int)q;
+}
+
 struct IgemmArgs {
+  TileOrder order;  // filled in by the launcher for the tile grid of the configuration it launches
   int64_t M, N, K;
   const void* A;
   int64_t lda;

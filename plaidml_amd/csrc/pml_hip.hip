@@ -953,6 +953,15 @@ int pml_hip_probe_mfma(int random_data, int iters, double* tflops, double* core_
   return rc;
 }
 
+int pml_hip_tile_of_workgroup(int tiles_m, int tiles_n, int workgroup, int* tile_m, int* tile_n) {
+  if (tiles_m <= 0 || tiles_n <= 0 || (int64_t)tiles_m * tiles_n >= ((int64_t)1 << 31) || workgroup < 0 ||
+      workgroup >= tiles_m * tiles_n || !tile_m || !tile_n)
+    return fail("tile_of_workgroup: bad argument");
+  const TileOrder o = make_tile_order(tiles_m, tiles_n);
+  tile_of(o, (unsigned)workgroup, tile_m, tile_n);
+  return 0;
+}
+
 int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s) {
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_GEMM || !b2 || p->gemm.k2 <= 0) return fail("gemm_pack_b2: bad argument");
