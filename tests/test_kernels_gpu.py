@@ -807,3 +807,71 @@ def test_pool_whole_image(kind, agg, N, H, W, C):
     else:
         np.testing.assert_array_equal(out, flat.max(1) if agg == 'max' else flat.min(1))
     hk.lib().pml_hip_plan_free(plan)
+
+
+# (kind, agg, N, H, W, C, kh, kw, stride, pad, with_index): the straight-line kernels (3x3, 2x2) and the window loop
+# (5x5, 3x2), windows that cross every border, one image and several, values quantised so that ties occur
+POOL_WINDOW_CASES = [
+    ('bf16', 'max', 2, 19, 19, 24, 3, 3, 2, 1, 1), ('bf16', 'max', 1, 8, 11, 16, 2, 2, 2, 0, 1), ('f32', 'max', 2, 9, 7, 8, 3, 3, 1, 1, 1),
+    ('bf16', 'min', 2, 10, 10, 16, 3, 3, 2, 1, 1), ('f32', 'min', 1, 6, 6, 12, 2, 2, 1, 0, 0), ('bf16', 'add', 2, 12, 9, 16, 3, 3, 2, 1, 0),
+    ('f32', 'add', 3, 7, 7, 4, 2, 2, 2, 1, 0), ('bf16', 'max', 2, 14, 14, 8, 5, 5, 2, 2, 1), ('f32', 'max', 1, 9, 9, 4, 3, 2, 1, 1, 0),
+    ('bf16', 'max', 1, 112, 112, 64, 3, 3, 2, 1, 0)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('kind,agg,N,H,W,C,kh,kw,stride,pad,with_index', POOL_WINDOW_CASES)
+def test_pool_windows_against_enumeration(kind, agg, N, H, W, C, kh, kw, stride, pad, with_index):
+    """Every output against a direct enumeration of its window: taps outside the image take no part; the index output
+    is the largest tap number kh_i * KW + kw_i whose value equals the pooled one (bit-exact, ties included)."""
+    print('pool window', kind, agg, N, H, W, C, kh, kw, stride, pad, with_index, flush=True)
+    rng = np.random.default_rng(H * 100 + W + C)
+    Iv = (np.round(rng.standard_normal((N, H, W, C)) * 4) / 4).astype(np.float32)
+    OH, OW = (H + 2 * pad - kh) // stride + 1, (W + 2 * pad - kw) // stride + 1
+    p = hk.Pool2dDesc()
+    p.dtype = hk.BF16 if kind == 'bf16' else hk.F32
+    p.agg = {'add': hk.AGG_ADD, 'max': hk.AGG_MAX, 'min': hk.AGG_MIN}[agg]
+    p.n, p.h, p.w, p.c, p.kh, p.kw, p.oh, p.ow = N, H, W, C, kh, kw, OH, OW
+    p.stride_h = p.stride_w = stride
+    p.pad_h = p.pad_w = pad
+    p.with_index = with_index
+    plan = hk.lib().pml_hip_pool2d_dispatch(ctypes.byref(p))
+    assert plan, hk.lib().pml_hip_last_error()
+    es = 2 if kind == 'bf16' else 4
+    dI = hk.DeviceBuffer.from_numpy(bf16(Iv) if kind == 'bf16' else Iv)
+    dO = hk.DeviceBuffer(N * OH * OW * C * es)
+    dX = hk.DeviceBuffer(N * OH * OW * C * 4) if with_index else None
+    hk.check(hk.lib().pml_hip_pool2d_invoke(plan, dI.ptr, dO.ptr, dX.ptr if dX else None, None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    out = E.bf16_from_bits(dO.to_numpy(np.uint16, (N, OH, OW, C))) if kind == 'bf16' else dO.to_numpy(np.float32, (N, OH, OW, C))
+    ident = {'add': 0.0, 'max': -np.inf, 'min': np.inf}[agg]
+    ref = np.full((N, OH, OW, C), ident, np.float64)
+    best = np.zeros((N, OH, OW, C), np.int32)
+    taps = []
+    for ky in range(kh):
+        for kx in range(kw):
+            tap = np.full((N, OH, OW, C), np.nan)
+            for oy in range(OH):
+                iy = oy * stride + ky - pad
+                if not 0 <= iy < H:
+                    continue
+                for ox in range(OW):
+                    ix = ox * stride + kx - pad
+                    if 0 <= ix < W:
+                        tap[:, oy, ox] = Iv[:, iy, ix]
+            taps.append(tap)
+            live = ~np.isnan(tap)
+            if agg == 'add':
+                ref = np.where(live, ref + np.nan_to_num(tap), ref)
+            elif agg == 'max':
+                ref = np.where(live & (tap > ref), tap, ref)
+            else:
+                ref = np.where(live & (tap < ref), tap, ref)
+    for k, tap in enumerate(taps):
+        best = np.where(tap == ref, np.int32(k), best)  # NaN (outside) never equals
+    if agg == 'add':
+        np.testing.assert_allclose(out, ref, rtol=BF16_RTOL if kind == 'bf16' else 1e-6, atol=1e-6)
+    else:
+        np.testing.assert_array_equal(out, ref.astype(np.float32))
+    if with_index:
+        np.testing.assert_array_equal(dX.to_numpy(np.int32, (N, OH, OW, C)), best)
+    hk.lib().pml_hip_plan_free(plan)
