@@ -875,3 +875,37 @@ def test_pool_windows_against_enumeration(kind, agg, N, H, W, C, kh, kw, stride,
     if with_index:
         np.testing.assert_array_equal(dX.to_numpy(np.int32, (N, OH, OW, C)), best)
     hk.lib().pml_hip_plan_free(plan)
+
+
+# (M, N, K): many rows, whole 128-column tiles, K of one slab, of three with a 16-byte tail, of four
+MANY_ROWS_CASES = [(140837, 128, 64), (70000, 256, 136), (140800, 128, 256)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('M,N,K', MANY_ROWS_CASES)
+def test_gemm_many_rows_short_k(M, N, K):
+    """The shape class of a residual network's 1x1 convolutions -- a hundred thousand rows and more, K of one to
+    four slabs, thousands of tiles: small-integer operands make every sum exact, so all four vector tails are pinned
+    bit for bit by the step semantics, on a ragged last row tile as well."""
+    print('many rows, short K', (M, N, K), flush=True)
+    rng = np.random.default_rng(M + K)
+    A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    bias = E.round_bf16(rng.standard_normal(N).astype(np.float32) * 8)
+    scale = E.round_bf16(rng.uniform(0.5, 1.5, N).astype(np.float32))
+    shift = E.round_bf16(rng.standard_normal(N).astype(np.float32) * 20)
+    res = E.round_bf16(rng.standard_normal((M, N)).astype(np.float32) * 30)
+    prod = A @ B
+    np.testing.assert_array_equal(run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16), bf16(E.round_bf16(prod)))
+    x = E.round_bf16(prod + bias)
+    tail = hk.make_tail(ops=[(hk.EPI_RELU, hk.BF16, 0, 0, 0.0)], operands=[])
+    C = run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16, tail=tail)
+    np.testing.assert_array_equal(C, bf16(np.maximum(x, 0)))
+    tail = hk.make_tail(ops=[(hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_RELU, hk.BF16, 0, 0, 0.0)], operands=[(hk.BF16, N, 1)])
+    C = run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16, tail=tail, operands=(bf16(res),))
+    np.testing.assert_array_equal(C, bf16(np.maximum(E.round_bf16(x + res), 0)))
+    tail = hk.make_tail(ops=[(hk.EPI_MUL, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 1, 0.0)],
+                        operands=[(hk.BF16, 0, 1), (hk.BF16, 0, 1)])
+    C = run_gemm(bf16(A), bf16(B), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16, tail=tail,
+                 operands=(bf16(scale), bf16(shift)))
+    np.testing.assert_array_equal(C, bf16(E.round_bf16(E.round_bf16(x * scale) + shift)))
