@@ -32,7 +32,7 @@ TRAINING_PRECISION = 2e-03    # plaidbench/core.py Precision.TRAINING
 
 class Golden:
     """The expected value of output 0 (after `select`, which cuts the part of the output the file holds),
-    the relative precision, and the absolute tolerance of the verdict (the reference's is 1e-6)."""
+    the relative precision, and the absolute tolerance of the PASS / FAIL result (the reference's is 1e-6)."""
 
     def __init__(self, expected, precision=INFERENCE_PRECISION, atol=1e-06, select=None):
         self.expected, self.precision, self.atol, self.select = expected, precision, atol, select or (lambda out: out)
@@ -172,7 +172,7 @@ def _toy_golden(batch_size):
     pos = fx['positions']
     # The file holds the output at `positions` x `positions` of the 56x56 plane.  Its values come from another fp32
     # implementation with its own summation order: a float64 evaluation of the definition differs from them by up to
-    # 5e-5 (activations reach 128), so the verdict uses atol 2e-4; fail_ratio keeps the reference's definition.
+    # 5e-5 (activations reach 128), so PASS / FAIL uses atol 2e-4; fail_ratio keeps the reference's definition.
     return Golden(fx['expected'], INFERENCE_PRECISION, atol=2e-04, select=lambda out: np.asarray(out)[0][np.ix_(pos, pos)])
 
 

@@ -20,7 +20,7 @@ def test_correctness_arithmetic_by_hand():
     assert not correct
     assert max_error == pytest.approx(5e-4 * 1e-4 / 1e-6, rel=1e-9)
     assert fail_ratio == 0.5
-    # the same under a wider absolute tolerance: verdict changes, fail_ratio keeps the reference's definition
+    # the same under a wider absolute tolerance: `correct` changes, fail_ratio keeps the reference's definition
     correct, _, _, fail_ratio = pb.check_correctness(np.array([1e-4, 1.0]), np.array([0.0, 1.0]), 5e-4, atol=2e-4)
     assert correct and fail_ratio == 0.5
 
