@@ -8,7 +8,8 @@ computed as `Runner._check_correctness` computes them (:395-416).  A network is 
 program.  Registered here: `resnet50` (v1.5, bf16, synthetic weights: no golden, so "untested" as in the reference
 when the golden file is missing; the softmax rows are checked to sum to one) and `toy_parallel_conv` (fp32, the
 reference tool's own weights, input and golden output at batch size 1, from the fixture file named by
-PLAIDBENCH_GOLDEN or found beside the tests); `register` adds others.
+PLAIDBENCH_GOLDEN or found beside the tests), `toy_gemms` and `toy_xcp` (the reference tool's two other toy
+networks, randomly initialised there as here); `register` adds others.
 
     python -m plaidml_amd.plaidbench resnet50 --batch-size 128 --examples 1024
 """
@@ -177,6 +178,43 @@ def _toy_golden(batch_size):
 
 
 register(Network('toy_parallel_conv', _toy_parallel_conv, golden=_toy_golden))
+
+
+def _finite(outputs):
+    if not all(np.isfinite(np.asarray(o, np.float64)).all() for o in outputs):
+        raise RuntimeError('the output holds values that are not finite')
+
+
+def _toy_gemms(batch_size):
+    """plaidbench/plaidbench/networks/keras/toy_gemms.py:22-38 -- four dense layers 256 -> 512 -> 1024 -> 2048 -> 1000,
+    each followed by ReLU, fp32; randomly initialised as there (Glorot-uniform weights, zero biases), so no golden."""
+    rng = np.random.default_rng(5)
+    f32 = P.DType.FLOAT32
+    X = P.Placeholder(f32, [batch_size, 256])
+    x, width = X, 256
+    for units in (512, 1024, 2048, 1000):
+        limit = np.sqrt(6.0 / (width + units))
+        W = P.Constant(rng.uniform(-limit, limit, (width, units)).astype(np.float32), f32)
+        b = P.Constant(np.zeros(units, np.float32), f32)
+        x, width = Pop.relu(Pop.dot(x, W) + b), units
+    return P.Program('toy_gemms', [X], [x]), [rng.uniform(0, 1, (batch_size, 256)).astype(np.float32)]
+
+
+def _toy_xcp(batch_size):
+    """plaidbench/plaidbench/networks/keras/toy_xcp.py:25-50 (the internal form): ReLU of a 149x149x64 input, a 3x3
+    convolution to 128 channels (SAME, no bias), max-pool 3x3 / 2 (SAME); fp32, random initialisation, no golden."""
+    rng = np.random.default_rng(6)
+    f32 = P.DType.FLOAT32
+    X = P.Placeholder(f32, [batch_size, 149, 149, 64])
+    limit = np.sqrt(6.0 / (9 * 64 + 9 * 128))
+    W = P.Constant(rng.uniform(-limit, limit, (3, 3, 64, 128)).astype(np.float32), f32)
+    y = Pop.convolution(Pop.relu(X), W, autopad=Pop.SAME_UPPER)
+    y = Pop.pool(y, 'max', [3, 3], [2, 2], autopad=Pop.SAME_UPPER)
+    return P.Program('toy_xcp', [X], [y]), [rng.uniform(0, 1, (batch_size, 149, 149, 64)).astype(np.float32)]
+
+
+register(Network('toy_gemms', _toy_gemms, sanity=_finite))
+register(Network('toy_xcp', _toy_xcp, sanity=_finite))
 
 
 def main(argv=None):

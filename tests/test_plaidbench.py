@@ -87,3 +87,66 @@ def test_resnet50_through_the_harness():
     assert r['correct'] == 'untested'       # synthetic weights; the harness has checked the softmax rows
     assert 0 < r['tile_duration_per_example'] <= r['duration_per_example']
     assert pb.main(['resnet50', '--batch-size', '2', '--examples', '2', '--warmups', '0', '--json']) == 0
+
+
+@pytest.mark.gpu
+def test_toy_gemms_through_the_harness_and_against_float64():
+    """Four dense layers with ReLU: the harness runs and reports; the output equals a float64 evaluation with the same
+    weights (the builder's random streams, restated here) to the fp32 bar."""
+    from plaidml_amd import edsl as P
+    r = pb.run('toy_gemms', batch_size=8, examples=16, warmups=8)
+    assert r['correct'] == 'untested' and 0 < r['tile_duration_per_example'] <= r['duration_per_example']
+    program, inputs = pb._NETWORKS['toy_gemms'].build(8)
+    got, = P.run(program, inputs, target='hip')
+    rng = np.random.default_rng(5)
+    weights, width = [], 256
+    for units in (512, 1024, 2048, 1000):
+        limit = np.sqrt(6.0 / (width + units))
+        weights.append(rng.uniform(-limit, limit, (width, units)).astype(np.float32))
+        width = units
+    x = rng.uniform(0, 1, (8, 256)).astype(np.float32)
+    np.testing.assert_array_equal(x, inputs[0])
+    ref = x.astype(np.float64)
+    for W in weights:
+        ref = np.maximum(ref @ W.astype(np.float64), 0)
+    np.testing.assert_allclose(got, ref, rtol=1e-3, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_toy_xcp_through_the_harness_and_against_float64_samples():
+    """ReLU -> 3x3 convolution 64 -> 128 (SAME) -> max-pool 3x3 / 2 (SAME) on 149x149: 400 sampled outputs against a
+    float64 evaluation of their windows."""
+    from plaidml_amd import edsl as P
+    r = pb.run('toy_xcp', batch_size=2, examples=4, warmups=2)
+    assert r['correct'] == 'untested' and 0 < r['tile_duration_per_example'] <= r['duration_per_example']
+    program, inputs = pb._NETWORKS['toy_xcp'].build(2)
+    got, = P.run(program, inputs, target='hip')
+    assert got.shape == (2, 75, 75, 128)
+    rng = np.random.default_rng(6)
+    limit = np.sqrt(6.0 / (9 * 64 + 9 * 128))
+    W = rng.uniform(-limit, limit, (3, 3, 64, 128)).astype(np.float32).astype(np.float64)
+    x = rng.uniform(0, 1, (2, 149, 149, 64)).astype(np.float32)
+    np.testing.assert_array_equal(x, inputs[0])
+    xr = np.maximum(x, 0).astype(np.float64)
+
+    def conv_at(n, y, xx, c):  # SAME, stride 1: pad 1
+        acc = 0.0
+        for ky in range(3):
+            for kx in range(3):
+                iy, ix = y + ky - 1, xx + kx - 1
+                if 0 <= iy < 149 and 0 <= ix < 149:
+                    acc += float(xr[n, iy, ix] @ W[ky, kx, :, c])
+        return acc
+
+    pick = np.random.default_rng(1)
+    for _ in range(400):
+        n, oy, ox, c = int(pick.integers(2)), int(pick.integers(75)), int(pick.integers(75)), int(pick.integers(128))
+        if _ < 8:
+            oy, ox = (0, 74)[_ & 1], (0, 74)[(_ >> 1) & 1]  # corners
+        best = -np.inf
+        for ky in range(3):          # SAME_UPPER with stride 2 on 149 -> 75: pad_before 0... (75 - 1) * 2 + 3 - 149 = 2 -> 1 before
+            for kx in range(3):
+                y, xx = 2 * oy + ky - 1, 2 * ox + kx - 1
+                if 0 <= y < 149 and 0 <= xx < 149:
+                    best = max(best, conv_at(n, y, xx, c))
+        np.testing.assert_allclose(got[n, oy, ox, c], best, rtol=1e-3, atol=1e-5)
