@@ -752,6 +752,9 @@ ALL = {
     # one image: the batch index has a single value and is folded out of every access before kernels are matched
     'single_image_xception_block_f32': lambda E, op: config3_xception_block(E, op, N=1, C=16, dtype_name='FLOAT32'),
     'single_image_classifier_tail_f32': lambda E, op: classifier_tail(E, op, N=1),
+    # 136 fp32 channels are 544 bytes per pixel: the depthwise result feeding the pointwise product is laid out at a
+    # pitch of whole 128-byte lines (640 bytes)
+    'xception_block_f32_pitched_temporary': lambda E, op: config3_xception_block(E, op, N=1, C=136, dtype_name='FLOAT32'),
     'residual_block_bf16': residual_block,
     'resnet50_tiny_bf16': resnet50_tiny,
 }
