@@ -55,10 +55,22 @@ def conv_plan(hk, in_dt, N, H, W, CI, CO, KH, KW, relu=True, flags=0):
     return plan
 
 
-def time_loop(hk, fn, steps, warmup):
+# A device that has been idle runs its first tens of milliseconds of work at a lower clock than it then settles at
+# (a 1024^3 fp32 GEMM: 28.0 us per launch over the first 2 ms, 24.9 us once half a second has passed).  Every timed
+# loop is therefore preceded, after its warm-up steps, by further untimed steps of the same call until this much
+# wall time has passed since the loop began: the figure is the one a device under sustained load shows.
+SETTLE_MS = 100.0
+
+
+def time_loop(hk, fn, steps, warmup, settle_ms=SETTLE_MS):
+    began = time.perf_counter()
     for _ in range(warmup):
         fn()
     hk.check(hk.lib().pml_hip_stream_sync(None))
+    while (time.perf_counter() - began) * 1e3 < settle_ms:
+        for _ in range(32):
+            fn()
+        hk.check(hk.lib().pml_hip_stream_sync(None))
     t = hk.Timer()
     wall0 = time.perf_counter()
     t.start()
@@ -222,11 +234,11 @@ def xception_program_leg(N, H, W, C, runs=5):
             rng.uniform(-0.5, 0.5, C).astype(np.float32)]
     runner = P.Runner(prog, target='hip')
     staged = runner.stage(vals)
-    best = None
-    for _ in range(runs):
+    best, n, began = None, 0, time.perf_counter()
+    while n < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
         runner.run_staged(staged)
         st = P.last_run_stats()
-        best = st if best is None or st['kernel_ms'] < best['kernel_ms'] else best
+        best, n = (st if best is None or st['kernel_ms'] < best['kernel_ms'] else best), n + 1
     plan = [l.strip() for l in dict(prog.passes)['hip-plan'].splitlines()[1:]]
     return {'kernel_ms': round(best['kernel_ms'], 4), 'launches': int(best['launches']), 'plan': plan}
 
@@ -237,13 +249,19 @@ def resnet50_leg(batch=128, runs=5):
     prog, _, flops_full_box = resnet50.build(P, Pop, batch=batch, round_fn=P.round_bf16)
     runner = P.Runner(prog, target='hip')
     x = np.random.default_rng(11).uniform(0, 1, (batch, 224, 224, 3)).astype(np.float32)
-    times = []
-    for _ in range(runs):
-        out, = runner.run([x])
-        times.append(P.last_run_stats())
+    out, = runner.run([x])
+    first = P.last_run_stats()
     if not (np.isfinite(out).all() and np.allclose(out.sum(axis=1), 1.0, atol=2e-2)):
         raise SystemExit('bench: ResNet-50 output is not a probability distribution')
+    # the timed runs follow one another without the 77 MB upload between them (during which the device idles and
+    # its clock falls back): the input is staged once
+    staged = runner.stage([x])
+    times, began = [], time.perf_counter()
+    while len(times) < runs or (time.perf_counter() - began) * 1e3 < 2 * SETTLE_MS:
+        runner.run_staged(staged)
+        times.append(P.last_run_stats())
     best = min(times[1:], key=lambda t: t['kernel_ms'])
+    best = dict(best, h2d_ms=first['h2d_ms'], d2h_ms=first['d2h_ms'])
     return {'img_per_s': round(batch / (best['kernel_ms'] * 1e-3), 1), 'kernel_ms': round(best['kernel_ms'], 3),
             'h2d_ms': round(best['h2d_ms'], 3), 'd2h_ms': round(best['d2h_ms'], 3), 'launches': int(best['launches']),
             'device_MB': round(best['device_bytes'] / 1e6, 1), 'arena_MB': round(best['arena_bytes'] / 1e6, 1),
@@ -391,7 +409,7 @@ def main():
         'config': {'workload': 'configs[1]: conv2d NHWC N128 56x56x64 (*) 3x3x64x64 stride 1 SAME + bias + ReLU, bf16, fp32 accumulate',
                    'plan': hk.describe(plan), 'device': hk.device_name(),
                    'input_output_pairs_in_turn': n_pairs, 'algorithmic_gflop': round(flops / 1e9, 3), 'full_box_gflop': round(flops_full_box / 1e9, 3),
-                   'host_wall_ms_per_step': round(wall_step, 5)},
+                   'host_wall_ms_per_step': round(wall_step, 5), 'settle_ms_before_timing': SETTLE_MS},
         'roofline': {'bound': 'mfma', 'achieved': round(flops / (ms_kernel * 1e-3) / 1e12, 3), 'peak': PEAK['bf16'],
                      'unit': 'TFLOP/s', 'frac': round(flops / (ms_kernel * 1e-3) / 1e12 / PEAK['bf16'], 4),
                      'traffic': committed_traffic(), 'kernel': hk.describe(plan).split('tile=')[-1], 'kernel_ms': round(ms_kernel, 5),

@@ -256,7 +256,9 @@ int pml_hip_tile_of_workgroup(int tiles_m, int tiles_n, int workgroup, int* tile
  * hipMalloc).  The transposed copy of a [K][N] right-hand side (b_layout 0), which a plan keeps in memory of its
  * own, lives in a fixed array in the library's device image instead: n * k * element size must not exceed
  * PML_HIP_STATIC_SCRATCH_BYTES, larger right-hand sides are rejected with an error text that says so
- * (b_layout 1 needs no copy and has no such limit).  Each GPU holds one such array for the life of the process and
+ * (b_layout 1 needs no copy and has no such limit; an fp32 right-hand side that the kernels read where it lies --
+ * n and ldb multiples of four, 16-byte aligned -- leaves the array untouched, the limit applies all the same).
+ * Each GPU holds one such array for the life of the process and
  * every call on that GPU uses it: calls that overlap on one GPU (two streams, two threads) race on it.  The
  * result equals pml_hip_gemm_dispatch + pml_hip_gemm_invoke bit for bit (same tile choice, same kernels). */
 #define PML_HIP_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)

@@ -83,7 +83,12 @@ constexpr int igemm_waves_per_simd() {
   return (NT / 256) * (2 * Ring<BM, BN, STAGES, SLAB>::kAlloc <= kLdsBytes ? 2 : 1);
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
+// BKN: the right-hand side is the caller's row-major B[K][N] of 4-byte elements (p.Bt, p.ldbt its row length): a slab
+// is then 32 rows of B as they lie in memory, [k][n] in LDS, and a lane gathers the four K-values of its fragment
+// with four 4-byte reads (32 consecutive columns per half wavefront: no bank conflicts).  The fp32 MFMA takes one
+// K-value per lane anyway, so nothing has to be transposed -- neither by a launch of its own nor in registers.
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128,
+          bool BKN = false>
 __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>())) void igemm_kernel(IgemmArgs p_by_value) {
   // The argument block is read where the dispatcher put it (the kernel-argument segment, scalar loads),
   // through a reference: taking the by-value parameter's address instead makes the compiler copy all of
@@ -99,6 +104,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
   constexpr bool kSplit = KIND == KIND_F32X3 || KIND == KIND_F32X3P;  // fp32 operands as three bf16 products
   constexpr bool kSplitB = KIND == KIND_F32X3P;                       // ... the right-hand side split when it was packed
+  static_assert(!BKN || ((KIND == KIND_F32 || KIND == KIND_F32X3) && !CONV && SLAB == 128), "a [K][N] right-hand side: fp32 GEMMs only");
   constexpr int kWaves = NT / 64;
   constexpr int kRowsPerPass = NT / CPR;  // operand rows one load of all threads covers
   constexpr int WAVES_N = kWaves / WAVES_M / WAVES_K;
@@ -188,10 +194,19 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
     }
   }
   unsigned b_off[B_VECS];
+  int b_krow[BKN ? B_VECS : 1];  // BKN: the row of the slab (0..31) this thread's chunk belongs to
 #pragma unroll
   for (int i = 0; i < B_VECS; ++i) {
-    const int64_t n = n0 + lr + kRowsPerPass * i;
-    b_off[i] = n < p.N ? (unsigned)(n * p.ldbt * ES) : kOutside;
+    if constexpr (BKN) {
+      constexpr int kChunksPerRow = BN / 4;  // 16-byte chunks of one K-row of the tile
+      const int c = tid + i * NT;
+      const int64_t n = n0 + (c % kChunksPerRow) * 4;
+      b_krow[i] = c / kChunksPerRow;
+      b_off[i] = n < p.N ? (unsigned)(((int64_t)b_krow[i] * p.ldbt + n) * ES) : kOutside;
+    } else {
+      const int64_t n = n0 + lr + kRowsPerPass * i;
+      b_off[i] = n < p.N ? (unsigned)(n * p.ldbt * ES) : kOutside;
+    }
   }
   unsigned a2_off[CONV ? 1 : A_VECS], b2_off[CONV ? 1 : B_VECS];
   if constexpr (!CONV) {
@@ -228,6 +243,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   // the vmcnt arithmetic below relies on.
   unsigned char* req_base = smem;
   unsigned req_a = 0, req_b = 0;  // slab-dependent part of the A / Bt offsets
+  int req_k0 = 0;                 // BKN: first K-index of the slab
   int req_dh = 0, req_dw = 0;     // CONV: the tap's displacement in input rows / columns (columns: plus the chunk's pixel)
   bool req_ok = false;
   bool req_second = false;        // GEMM: the slab belongs to the second product
@@ -258,6 +274,10 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       req_second = nx_kbo >= first_bytes;
       const int kbo = (req_second ? nx_kbo - first_bytes : nx_kbo) + lc * 16;
       req_a = req_b = kbo < (req_second ? k2_bytes : kbytes_row) ? (unsigned)kbo : kOutside;
+      if constexpr (BKN) {
+        req_k0 = nx_kbo / ES;
+        req_b = (unsigned)((int64_t)req_k0 * p.ldbt * ES);  // the slab's first row of B
+      }
       nx_kbo += kSlabBytes;
     }
   };
@@ -277,6 +297,9 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       if (CONV) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16,
                                                  (int)join_offsets(b_off[i], req_b), 0, 0, 0);
+      } else if constexpr (BKN) {
+        const unsigned off = (b_off[i] != kOutside && req_k0 + b_krow[i] < (int)p.K) ? b_off[i] + req_b : kOutside;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16, (int)off, 0, 0, 0);
       } else {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(req_second ? rb2 : rb, PML_LDS(req_base + (BM + i * kRowsPerPass) * kSlabBytes), 16,
                                                  (int)join_offsets(req_second ? b2_off[i] : b_off[i], req_b), 0, 0, 0);
@@ -348,7 +371,21 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       fslot[kb] = ((gb * 2 + h) ^ key) * 16;
       fslot_b[kb] = fslot[kb];
     }
+    // BKN: chunk c of a row holds K-values 4c .. 4c + 3, which in [k][n] order are four rows of BN * 4 bytes
+    if constexpr (BKN) fslot_b[kb] = (kSplit ? ((gb & ~1) * 2 + 2 * h + (gb & 1)) : (gb * 2 + h)) * 4 * (BN * 4);
   }
+  // the Bt fragment of 32-column block j for the K-block whose slot is `slot`, out of the stage whose Bt part `bb`
+  // points into (at the wavefront's first column and the lane's row or column)
+  auto read_b = [&](const unsigned char* bb, int j, int slot) {
+    if constexpr (BKN) {
+      i32x4_t v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = *(const int*)(bb + slot + e * (BN * 4) + j * 32 * 4);
+      return v;
+    } else {
+      return *(const i32x4_t*)(bb + j * 32 * kSlabBytes + slot);
+    }
+  };
 
   // The loop is rotated by one K-block: the one synchronisation point of a slab sits before its LAST
   // K-block, whose fragments are in registers by then.  Past it every wavefront is done reading this
@@ -363,20 +400,20 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   i32x4_t xa_head[kSplit ? MI : 1], xa_rem[kSplit ? MI : 1];
   i32x4_t xb_head[kSplit && !kSplitB ? NI : 1], xb_rem[kSplit && !kSplitB ? NI : 1];
   const unsigned char* a_base = smem + (wm * WM + frow) * kSlabBytes;
-  const unsigned char* b_base = smem + (BM + wn * WN + frow) * kSlabBytes;
+  const unsigned char* b_base = BKN ? smem + BM * kSlabBytes + (wn * WN + frow) * 4 : smem + (BM + wn * WN + frow) * kSlabBytes;
   __builtin_amdgcn_s_waitcnt(0x0F70 | (((kStages - 1) * kLoads) & 15) | ((((kStages - 1) * kLoads) >> 4) << 14));
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int i = 0; i < MI; ++i) fa[0][i] = *(const i32x4_t*)(a_base + i * 32 * kSlabBytes + fslot[0]);
 #pragma unroll
-  for (int j = 0; j < NI; ++j) fb[0][j] = *(const i32x4_t*)(b_base + j * 32 * kSlabBytes + fslot_b[0]);
+  for (int j = 0; j < NI; ++j) fb[0][j] = read_b(b_base, j, fslot_b[0]);
 
   int stage = 0;  // ring stage of slab s
   for (int s = 0; s < n_slabs; ++s) {
     int next_stage = stage + 1;
     if (next_stage == kStages) next_stage = 0;
     const unsigned char* a_next = smem + next_stage * kStage + (wm * WM + frow) * kSlabBytes;
-    const unsigned char* b_next = smem + next_stage * kStage + (BM + wn * WN + frow) * kSlabBytes;
+    const unsigned char* b_next = smem + next_stage * kStage + (BKN ? BM * kSlabBytes + (wn * WN + frow) * 4 : (BM + wn * WN + frow) * kSlabBytes);
 #pragma unroll
     for (int kb = 0; kb < kBlocks; ++kb) {
       const int cur = kb & 1, nxt = cur ^ 1;
@@ -442,7 +479,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
           if (d < MI)
             fa[nxt][d] = *(const i32x4_t*)(ra_ + d * 32 * kSlabBytes + fs);
           else
-            fb[nxt][d - MI] = *(const i32x4_t*)(rb_ + (d - MI) * 32 * kSlabBytes + fs_b);
+            fb[nxt][d - MI] = read_b(rb_, d - MI, fs_b);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -613,6 +650,23 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
 
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
+  if constexpr ((KIND == KIND_F32 || KIND == KIND_F32X3) && !CONV && SLAB == 128) {
+    if (a.b_kn) {
+      const int64_t tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+      const int64_t tiles = tiles_m * tiles_n;
+      if (tiles <= 0 || tiles >= ((int64_t)1 << 31) || a.K2 > 0) return hipErrorInvalidValue;
+      const size_t lds = Ring<BM, BN, STAGES, SLAB>::kAlloc;
+      auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB, true>;
+      static DynamicLdsLimit limit;
+      if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
+      IgemmArgs b = a;
+      b.order = make_tile_order((int)tiles_m, (int)tiles_n);
+      hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), lds, s, b);
+      return hipGetLastError();
+    }
+  } else {
+    if (a.b_kn) return hipErrorInvalidValue;
+  }
   const int64_t tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
   const int64_t tiles = tiles_m * tiles_n;
   if (tiles <= 0 || tiles >= ((int64_t)1 << 31)) return hipErrorInvalidValue;

@@ -135,6 +135,7 @@ inline void tile_of(const TileOrder& o, unsigned bid, int* tm, int* tn) {
 
 struct IgemmArgs {
   TileOrder order;  // filled in by the launcher for the tile grid of the configuration it launches
+  int b_kn;         // 1: Bt / ldbt are the caller's row-major B[K][N] and its row length (fp32 GEMMs only)
   int64_t M, N, K;
   const void* A;
   int64_t lda;

@@ -594,6 +594,13 @@ struct SecondProduct {
   bool packed2 = false;
 };
 
+// An fp32 right-hand side that arrives with the call in its row-major [K][N] form is read as it is (the fp32 kinds
+// gather their K-values from [k][n] slabs); everything else is transposed into Bt[N][K] first.
+static bool reads_b_as_given(const pml_hip_gemm_desc& d, int mfma_kind, const void* b) {
+  return b && !d.b_layout && (mfma_kind == KIND_F32 || mfma_kind == KIND_F32X3) && d.k2 == 0 && d.n % 4 == 0 && d.ldb % 4 == 0 &&
+         ((uintptr_t)b & 15) == 0 && d.k * d.ldb * 4 < ((int64_t)1 << 31);
+}
+
 static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* bt, int64_t bt_ld, bool packed,
                     const void* a, const void* b, void* c, const void* init, const void* const* operands,
                     void* const* outs, pml_hip_stream s, const SecondProduct* second = nullptr, bool bt_is_split = false) {
@@ -606,7 +613,8 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   if (((uintptr_t)a & 15) != 0) return fail("gemm_invoke: A must be 16-byte aligned");
   if (d.init_kind && !init) return fail("gemm_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
-  if (b && !d.b_layout && check(transpose_pack(es, b, bt, d.k, d.n, d.ldb, bt_ld, (hipStream_t)s), "transpose_pack"))
+  const bool b_as_given = reads_b_as_given(d, mfma_kind, b);
+  if (b && !d.b_layout && !b_as_given && check(transpose_pack(es, b, bt, d.k, d.n, d.ldb, bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   if (d.k2 > 0) {
     if (!second || !second->a2) return fail("gemm_invoke: the plan has a second product: use pml_hip_gemm_invoke2");
@@ -641,8 +649,9 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   g.K = d.k;
   g.A = a;
   g.lda = d.lda;
-  g.Bt = d.b_layout ? b : bt;
-  g.ldbt = d.b_layout ? d.ldb : bt_ld;
+  g.Bt = (d.b_layout || b_as_given) ? b : bt;
+  g.ldbt = (d.b_layout || b_as_given) ? d.ldb : bt_ld;
+  g.b_kn = b_as_given ? 1 : 0;
   g.C = c;
   g.ldc = d.ldc;
   g.out_dtype = d.out_dtype;
@@ -679,7 +688,8 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
   const bool split = p->bt_is_split;
-  if (b && !p->gemm.b_layout) p->bt_is_split = false;  // this run's transposition overwrites the packed copy
+  // a right-hand side that this run transposes overwrites the packed copy
+  if (b && !p->gemm.b_layout && !reads_b_as_given(p->gemm, p->mfma_kind, b)) p->bt_is_split = false;
   return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s, nullptr, split);
 }
 

@@ -878,6 +878,68 @@ def test_pool_windows_against_enumeration(kind, agg, N, H, W, C, kh, kw, stride,
 
 
 # (M, N, K): many rows, whole 128-column tiles, K of one slab, of three with a 16-byte tail, of four
+def _gemm_f32_layouts(A, B_kn, ldb, flags, packed_first=False):
+    """A . B for an fp32 right-hand side handed over as [K][N] at leading dimension ldb, and for the same values as
+    [N][K] (K contiguous): both results."""
+    M, K = A.shape
+    N = B_kn.shape[1]
+    out = []
+    for layout in (0, 1):
+        d = hk.GemmDesc()
+        d.in_dtype = d.out_dtype = d.c_dtype = hk.F32
+        d.flags = flags
+        d.m, d.n, d.k = M, N, K
+        d.lda, d.ldc = K, N
+        d.b_layout = layout
+        if layout == 0:
+            Bh = np.zeros((K, ldb), np.float32)
+            Bh[:, :N] = B_kn
+            Bh[:, N:] = np.nan  # what lies between the rows must never be read into a product
+            d.ldb = ldb
+        else:
+            Bh = np.ascontiguousarray(B_kn.T)
+            d.ldb = K
+        plan = hk.lib().pml_hip_gemm_dispatch(ctypes.byref(d))
+        assert plan, hk.lib().pml_hip_last_error()
+        dA, dB, dC = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(Bh), hk.DeviceBuffer(M * N * 4)
+        none = hk.ptr_array([])
+        if packed_first and layout == 0:
+            # a packed copy of OTHER values first: the run below hands its own B over and must use that one, and a
+            # run without B afterwards must still find the packed values
+            other = hk.DeviceBuffer.from_numpy(np.ones_like(Bh))
+            hk.check(hk.lib().pml_hip_gemm_pack_b(plan, other.ptr, None))
+        hk.check(hk.lib().pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, None, none, none, None))
+        hk.check(hk.lib().pml_hip_stream_sync(None))
+        out.append(dC.to_numpy(np.float32, (M, N)))
+        if packed_first and layout == 0:
+            hk.check(hk.lib().pml_hip_gemm_invoke(plan, dA.ptr, None, dC.ptr, None, none, none, None))
+            hk.check(hk.lib().pml_hip_stream_sync(None))
+            ones = dC.to_numpy(np.float32, (M, N))
+            np.testing.assert_allclose(ones, np.repeat(A.astype(np.float64).sum(axis=1)[:, None], N, axis=1), rtol=1e-3, atol=1e-3)
+        hk.lib().pml_hip_plan_free(plan)
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('flags', [0, hk.FP32_AS_BF16X3])
+@pytest.mark.parametrize('M,N,K,ldb', [(1024, 1024, 1024, 1024), (100, 68, 72, 72), (64, 64, 36, 64), (200, 260, 132, 300),
+                                       (130, 4, 8, 4), (96, 512, 2048, 516), (77, 66, 40, 66)])
+def test_gemm_f32_right_hand_side_as_given(M, N, K, ldb, flags):
+    """An fp32 [K][N] right-hand side that arrives with the call is read where it lies (no transposed copy): the
+    result has the same bits as the one from the same values in [N][K] layout -- the two differ only in how the
+    fragments reach the registers, not in what is multiplied or in which order it is summed -- and agrees with
+    float64.  Ragged last tiles in N and K, a leading dimension wider than N with NaNs in the gap, a K
+    of one short slab, and (N = 66) a shape that falls back to the transposed copy."""
+    print('fp32 right-hand side as given', (M, N, K, ldb, flags), flush=True)
+    rng = np.random.default_rng(M * 7 + N + K)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    as_given, n_major = _gemm_f32_layouts(A, B, ldb, flags, packed_first=(M == 100))
+    np.testing.assert_array_equal(as_given.view(np.uint32), n_major.view(np.uint32))
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_allclose(as_given, ref, rtol=FP32_RTOL if not flags else 1e-3, atol=1e-4 if not flags else 2e-3)
+
+
 MANY_ROWS_CASES = [(140837, 128, 64), (70000, 256, 136), (140800, 128, 256)]
 
 
