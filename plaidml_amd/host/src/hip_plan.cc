@@ -1639,6 +1639,33 @@ class Planner {
 
   // ----- the general contraction kernel ---------------------------------------------------
 
+  // Per output dimension the index to solve the output access for, or -1: integer forms only; an index that
+  // appears in one output dimension only; among those the widest range (what a thread no longer walks), the
+  // smaller coefficient on a tie.  A dimension whose access is a constant keeps -1; if a dimension with indices
+  // has no candidate, nothing is solved for (every dimension -1) and the kernel enumerates the whole box.
+  static std::vector<int> choosePivots(const Op& op) {
+    const size_t nIdx = op.idxNames.size(), rank = op.accesses[0].size();
+    std::vector<int> pivot(rank, -1);
+    std::vector<int> uses(nIdx, 0);
+    for (const Affine& a : op.accesses[0]) {
+      if (a.den != 1) return pivot;
+      for (size_t v = 0; v < nIdx; ++v) uses[v] += a.coef[v] != 0;
+    }
+    for (size_t k = 0; k < rank; ++k) {
+      const Affine& a = op.accesses[0][k];
+      if (a.isConstant()) continue;
+      int best = -1;
+      for (size_t v = 0; v < nIdx; ++v) {
+        if (!a.coef[v] || uses[v] != 1 || std::llabs(a.coef[v]) > (1 << 20)) continue;
+        const int64_t range = op.upper[v] - op.lower[v], best_range = best < 0 ? -1 : op.upper[best] - op.lower[best];
+        if (best < 0 || range > best_range || (range == best_range && std::llabs(a.coef[v]) < std::llabs(a.coef[best]))) best = static_cast<int>(v);
+      }
+      if (best < 0) return std::vector<int>(rank, -1);
+      pivot[k] = best;
+    }
+    return pivot;
+  }
+
   void emitGeneral(size_t i) {
     const Op& op = prog_->ops[i];
     const size_t nIdx = op.idxNames.size();
@@ -1672,18 +1699,30 @@ class Planner {
     std::vector<int> order;  // new position -> old index
     std::vector<std::array<int64_t, 2>> extra_box;
     size_t n_fresh = 0;
+    // Output accesses that are sums of indices (a transposed convolution's O[n, 2x + i - 1, ...]): the output
+    // coordinates o_k become the variables, as in the reference's change of variables
+    // (pmlc/dialect/tile/transforms/contraction.cc:340-416, ReduceOutputPolynomials), but one index at a time:
+    // in each output dimension one index v -- the one with the widest range among those no other output
+    // dimension uses -- is solved for, v = (o_k - the form's other terms) / c, and substituted in every form.
+    // Forms then carry the denominator c, and the kernel's "must be an integer" test does what the reference's
+    // Defractionalize (:418-561) arranges by a further change of variables; v's own range becomes a constraint.
+    // A thread then walks the remaining indices only (the taps and input channels), not the whole box.
+    std::vector<int> pivot;  // per output dimension: the index solved for, or -1
     if (injective) {
       order = out_idx;
       d.n_out_idx = static_cast<int>(out_idx.size());
       for (size_t v = 0; v < nIdx; ++v)
         if (std::find(out_idx.begin(), out_idx.end(), static_cast<int>(v)) == out_idx.end()) order.push_back(static_cast<int>(v));
     } else {
-      // one fresh index per output dimension, tied to the sink polynomial by an equality form
+      // one fresh index per output dimension, tied to the sink polynomial by an equality form or by solving
       n_fresh = os.getRank();
       d.n_out_idx = static_cast<int>(n_fresh);
-      for (size_t v = 0; v < nIdx; ++v) order.push_back(static_cast<int>(v));
+      pivot = choosePivots(op);
+      for (size_t v = 0; v < nIdx; ++v)
+        if (std::find(pivot.begin(), pivot.end(), static_cast<int>(v)) == pivot.end()) order.push_back(static_cast<int>(v));
     }
-    const size_t total_idx = n_fresh + nIdx;
+    const size_t n_solved = pivot.size() - static_cast<size_t>(std::count(pivot.begin(), pivot.end(), -1));
+    const size_t total_idx = n_fresh + nIdx - n_solved;
     if (total_idx > PML_HIP_MAX_IDX) throw std::runtime_error("contraction has too many indices for the hip target");
     d.n_idx = static_cast<int>(total_idx);
     d.dtype = hipType(os.elementType);
@@ -1702,22 +1741,43 @@ class Planner {
       d.hi[k] = os.sizes[k] - 1;
     }
     for (size_t v = 0; v < nIdx; ++v) {
+      if (pos[v] < 0) continue;  // solved for
       d.lo[pos[v]] = op.lower[v];
       d.hi[pos[v]] = op.upper[v];
     }
     d.out_elems = 1;
     for (int k = 0; k < d.n_out_idx; ++k) d.out_elems *= std::max<int64_t>(0, d.hi[k] - d.lo[k] + 1);
     int nf = 0;
+    // a form over the program's indices -> one over the kernel's (solved indices substituted)
     auto addForm = [&](const Affine& a, int operand, int64_t size, int64_t stride) {
       if (nf >= PML_HIP_MAX_FORMS) throw std::runtime_error("contraction has too many access dimensions for the hip target");
       pml_hip_form& f = d.forms[nf++];
       std::memset(&f, 0, sizeof f);
-      for (size_t v = 0; v < nIdx; ++v) {
-        if (a.coef[v] > INT32_MAX || a.coef[v] < INT32_MIN) throw std::runtime_error("index coefficient too large");
-        f.coef[pos[v]] = static_cast<int32_t>(a.coef[v]);
+      // common multiple of the solved indices' coefficients that this form touches
+      int64_t scale = 1;
+      for (size_t k = 0; k < pivot.size(); ++k)
+        if (pivot[k] >= 0 && a.coef[pivot[k]] != 0) scale = std::lcm(scale, std::llabs(op.accesses[0][k].coef[pivot[k]]));
+      std::vector<int64_t> coef(total_idx, 0);
+      int64_t c0 = a.c0 * scale;
+      for (size_t v = 0; v < nIdx; ++v)
+        if (pos[v] >= 0) coef[pos[v]] += a.coef[v] * scale;
+      for (size_t k = 0; k < pivot.size(); ++k) {
+        if (pivot[k] < 0 || a.coef[pivot[k]] == 0) continue;
+        const Affine& o = op.accesses[0][k];
+        const int64_t m = a.coef[pivot[k]] * (scale / o.coef[pivot[k]]);  // times (o_k - the other terms of o)
+        coef[k] += m;
+        c0 -= m * o.c0;
+        for (size_t w = 0; w < nIdx; ++w)
+          if (static_cast<int>(w) != pivot[k] && o.coef[w] != 0) coef[pos[w]] -= m * o.coef[w];
       }
-      f.c0 = static_cast<int32_t>(a.c0);
-      f.den = static_cast<int32_t>(a.den);
+      const int64_t den = a.den * scale;
+      for (size_t v = 0; v < total_idx; ++v) {
+        if (coef[v] > INT32_MAX || coef[v] < INT32_MIN) throw std::runtime_error("index coefficient too large");
+        f.coef[v] = static_cast<int32_t>(coef[v]);
+      }
+      if (c0 > INT32_MAX || c0 < INT32_MIN || den > INT32_MAX || den <= 0) throw std::runtime_error("index coefficient too large");
+      f.c0 = static_cast<int32_t>(c0);
+      f.den = static_cast<int32_t>(den);
       f.operand = operand;
       f.size = size;
       f.stride = stride;
@@ -1734,8 +1794,17 @@ class Planner {
         pml_hip_form* fo = addForm(plain, 0, os.sizes[k], ostr[k]);
         fo->coef[k] = 1;
         const Affine& a = op.accesses[0][k];
-        pml_hip_form* fe = addForm(a, -1, 1, 0);
-        fe->coef[k] = static_cast<int32_t>(-a.den);  // (sink_num - den*o_k) / den
+        if (pivot[k] >= 0) {
+          // the solved index must be an integer of its range: 0 <= v - lower < extent
+          Affine v;
+          v.coef.assign(nIdx, 0);
+          v.coef[pivot[k]] = 1;
+          v.c0 = -op.lower[pivot[k]];
+          addForm(v, -1, op.upper[pivot[k]] - op.lower[pivot[k]] + 1, 0);
+        } else {
+          pml_hip_form* fe = addForm(a, -1, 1, 0);
+          fe->coef[k] -= static_cast<int32_t>(fe->den);  // (sink_num - den*o_k) / den
+        }
       }
     }
     for (size_t sidx = 1; sidx < op.accesses.size(); ++sidx) {
@@ -1789,7 +1858,17 @@ class Planner {
     for (const ValuePtr& v : op.operands) s.operands.push_back(bufferFor(v));
     std::stringstream ss;
     ss << "contract (general) " << tile::toString(op.agg) << "/" << tile::toString(op.combo) << " idx=" << d.n_idx
-       << " out_idx=" << d.n_out_idx << (injective ? "" : " (output enumerated per element)") << " -> " << os.str();
+       << " out_idx=" << d.n_out_idx;
+    if (!injective) {
+      ss << " (output enumerated per element";
+      if (n_solved) {
+        ss << "; solved for";
+        for (int v : pivot)
+          if (v >= 0) ss << " " << op.idxNames[v];
+      }
+      ss << ")";
+    }
+    ss << " -> " << os.str();
     s.text = ss.str();
     plan_->steps.push_back(s);
   }

@@ -90,6 +90,58 @@ def defract_long(E, op):
         np.array([[[[2], [3], [4]], [[6], [-3], [-1]], [[-1], [-2], [1]]]], np.float32)], EXACT
 
 
+def flatten_by_contraction(E, op):
+    """`no_reduce` of pmlc/dialect/tile/tests/compute-bounds.mlir:34-45: O[d1 + 10 d0] = I[d0, d1], an output access
+    that is a sum of two indices."""
+    I = E.Placeholder(E.DType.FLOAT32, [10, 10])
+    d0, d1 = E.TensorIndexes(2)
+    O = E.Contraction().outShape(100).outAccess(d1 + d0 * 10).assign(I[d0, d1]).build()
+    return E.Program('no_reduce', [I], [O]), [_rng(3).standard_normal((10, 10)).astype(np.float32)], EXACT
+
+
+def scatter_form_transposed_conv(E, op, N=2, H=6, CI=3, CO=4, dtype_name='FLOAT32'):
+    """A stride-2 transposed convolution written from the input's point of view: every input pixel (x, y) adds its
+    3x3 footprint to O[n, 2x + i - 1, 2y + j - 1, co].  Two output coordinates are sums of indices, many index
+    tuples meet in one output element, footprints hang over the border, and the odd output row / column 2H - 1
+    ... 2H is reached by one tap only."""
+    dt = getattr(E.DType, dtype_name)
+    I = E.Placeholder(dt, [N, H, H, CI])
+    K = E.Placeholder(dt, [3, 3, CI, CO])
+    n, x, y, i, j, ci, co = E.TensorIndexes(7)
+    O = E.Contraction().outShape(N, 2 * H, 2 * H, CO).outAccess(n, 2 * x + i - 1, 2 * y + j - 1, co).sum(
+        I[n, x, y, ci] * K[i, j, ci, co]).build()
+    r = _rng(21)
+    vals = [r.integers(-3, 4, (N, H, H, CI)).astype(np.float32), r.integers(-3, 4, (3, 3, CI, CO)).astype(np.float32)]
+    return E.Program('scatter_form_transposed_conv', [I, K], [O]), vals, EXACT
+
+
+def scatter_form_transposed_conv_answer(I, K):
+    """The same by explicit loops over the input pixels (float64; the test data are small integers, so exact)."""
+    N, H, _, CI = I.shape
+    CO = K.shape[3]
+    O = np.zeros((N, 2 * H, 2 * H, CO))
+    for x in range(H):
+        for y in range(H):
+            for i in range(3):
+                for j in range(3):
+                    ox, oy = 2 * x + i - 1, 2 * y + j - 1
+                    if 0 <= ox < 2 * H and 0 <= oy < 2 * H:
+                        O[:, ox, oy, :] += I[:, x, y, :].astype(np.float64) @ K[i, j].astype(np.float64)
+    return O
+
+
+def mirrored_sum_of_indices(E, op):
+    """O[7 - i + 2 j, c] += A[i, c] * B[j, c]: a negative and a non-unit coefficient in one output coordinate (i in
+    0..5, j in 0..3), another coordinate plain."""
+    A = E.Placeholder(E.DType.INT32, [6, 5])
+    B = E.Placeholder(E.DType.INT32, [4, 5])
+    i, j, c = E.TensorIndexes(3)
+    O = E.Contraction().outShape(14, 5).outAccess(7 - i + 2 * j, c).sum(A[i, c] * B[j, c]).build()
+    r = _rng(22)
+    return E.Program('mirrored_sum_of_indices', [A, B], [O]), [r.integers(-9, 10, (6, 5)).astype(np.int32),
+                                                               r.integers(-9, 10, (4, 5)).astype(np.int32)], EXACT
+
+
 def max_rows(E, op):
     """CppEdsl.Max, plaidml/edsl/tests/edsl_test.cc:576-590."""
     A = E.Placeholder(E.DType.FLOAT32, [3, 3])
@@ -713,6 +765,9 @@ ALL = {
     'gemv_float32': lambda E, op: gemv(E, op, 'FLOAT32'),
     'funky_sum': funky_sum,
     'defract_long': defract_long,
+    'flatten_by_contraction': flatten_by_contraction,
+    'scatter_form_transposed_conv': scatter_form_transposed_conv,
+    'mirrored_sum_of_indices': mirrored_sum_of_indices,
     'max_rows': max_rows,
     'use_default': use_default,
     'eltwise_mix': eltwise_mix,

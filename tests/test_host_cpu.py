@@ -62,6 +62,25 @@ def test_depthwise_temporary_gets_a_pitch_of_whole_lines():
     assert 'row pitch' not in t
 
 
+def test_output_coordinates_that_are_sums_are_solved_for_one_index():
+    """O[n, 2x + i - 1, 2y + j - 1, co]: the planner solves each such coordinate for its widest index (x, y), so the
+    kernel's threads walk the taps and input channels only -- 7 indices (4 output coordinates + i, j, ci), not 11;
+    an output access with a fraction keeps the full enumeration."""
+    t = plan_of(programs.scatter_form_transposed_conv(E, op)[0])
+    assert 'contract (general) add/mul idx=7 out_idx=4 (output enumerated per element; solved for' in t, t
+    solved = t.split('solved for ')[1].split(')')[0].split()
+    assert len(solved) == 4, t  # n and co trivially, x and y from the sums
+    t = plan_of(programs.flatten_by_contraction(E, op)[0])
+    assert 'idx=2 out_idx=1 (output enumerated per element; solved for' in t, t
+    t = plan_of(programs.mirrored_sum_of_indices(E, op)[0])
+    assert 'idx=3 out_idx=2 (output enumerated per element; solved for' in t, t
+    A = E.Placeholder(D.FLOAT32, [8])
+    i, j = E.TensorIndexes(2)
+    O = E.Contraction().outShape(8).outAccess((i + j) // 2).sum(A[i] * A[j]).build()
+    t = plan_of(E.Program('halved', [A], [O]))
+    assert 'idx=3 out_idx=1 (output enumerated per element)' in t, t
+
+
 def test_one_image_keeps_the_window_kernels():
     """At batch 1 the batch index is a constant; depthwise, pooling, window argmax and the pooling over the whole
     image must still be matched (the reference tool benchmarks at batch 1 by default)."""

@@ -379,3 +379,25 @@ def test_eq_combination_closed_forms():
         assert g.dtype == np.bool_ and g.shape == w.shape, k
         np.testing.assert_array_equal(g, w, err_msg=str(k))
     assert outs[0].any() and not outs[1].all() and outs[2].any() and not outs[2].all()  # the case is telling
+
+
+def test_output_accesses_that_are_sums_of_indices():
+    """The oracle on output coordinates that are sums of indices, against closed forms: the flattening contraction of
+    compute-bounds.mlir:34-45 is a reshape; a transposed convolution written from the input's side equals explicit
+    loops over the input pixels; a mirrored, strided coordinate equals a direct double loop."""
+    import programs
+    from oracle import tile_oplib as Oop
+    prog, vals, _ = programs.flatten_by_contraction(E, Oop)
+    np.testing.assert_array_equal(E.run(prog, vals)[0], vals[0].reshape(100))
+    prog, vals, _ = programs.scatter_form_transposed_conv(E, Oop)
+    want = programs.scatter_form_transposed_conv_answer(*vals)
+    got, = E.run(prog, vals)
+    np.testing.assert_array_equal(got, want.astype(np.float32))
+    assert np.count_nonzero(want[:, -1]) and np.count_nonzero(want[:, :, -1])  # the last row / column is reached
+    prog, vals, _ = programs.mirrored_sum_of_indices(E, Oop)
+    A, B = vals
+    want = np.zeros((14, 5), np.int64)
+    for i in range(6):
+        for j in range(4):
+            want[7 - i + 2 * j] += A[i].astype(np.int64) * B[j]
+    np.testing.assert_array_equal(E.run(prog, vals)[0], want.astype(np.int32))

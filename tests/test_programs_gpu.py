@@ -219,6 +219,18 @@ def test_config4_full_size_image_against_golden():
     print('configs[4] run stats', E.last_run_stats(), flush=True)
 
 
+def test_transposed_convolution_from_the_input_side_at_size():
+    """O[n, 2x + i - 1, 2y + j - 1, co] += I[n, x, y, ci] K[i, j, ci, co] on 2 x 32 x 32 x 16 -> 64 x 64 x 16: 131072
+    output elements over a box of 4.7 million index tuples.  Each thread walks the 144 (tap, channel) tuples of its
+    element, the two sums being solved for x and y; exact on small-integer data against loops over the input."""
+    print('transposed convolution, input side, 32x32x16', flush=True)
+    prog, vals, _ = programs.scatter_form_transposed_conv(E, op, N=2, H=32, CI=16, CO=16)
+    want = programs.scatter_form_transposed_conv_answer(*vals)
+    got, = E.run(prog, vals, target='hip')
+    np.testing.assert_array_equal(got, want.astype(np.float32))
+    assert E.last_run_stats()['kernel_ms'] < 50.0
+
+
 def test_run_checks_arity_and_shapes():
     prog, vals, _ = programs.dot_f32(E, op)
     prog.compile()
