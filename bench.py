@@ -219,21 +219,23 @@ def xception_program_leg(N, H, W, C, runs=5):
     """The same block as one Tile program through libplaidml.so: what the planner makes of it, device time of a run."""
     from plaidml_amd import edsl as P, op as Pop
     dt = P.DType.BFLOAT16
-    I, Fdw, Fpw = P.Placeholder(dt, [N, H, W, C]), P.Placeholder(dt, [3, 3, C, 1]), P.Placeholder(dt, [1, 1, C, C])
-    scale, shift = P.Placeholder(dt, [C]), P.Placeholder(dt, [C])
+    rng = np.random.default_rng(7)
+    image = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    # the block's weights are program constants, as a network's are (uploaded and re-laid-out once)
+    I = P.Placeholder(dt, [N, H, W, C])
+    Fdw = P.Constant(P.round_bf16((rng.standard_normal((3, 3, C, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)), dt)
+    Fpw = P.Constant(P.round_bf16((rng.standard_normal((1, 1, C, C)) * np.sqrt(2.0 / C)).astype(np.float32)), dt)
+    scale = P.Constant(P.round_bf16(rng.uniform(0.5, 1.5, C).astype(np.float32)), dt)
+    shift = P.Constant(P.round_bf16(rng.uniform(-0.5, 0.5, C).astype(np.float32)), dt)
     R = Pop.relu(Pop.convolution(Pop.convolution(I, Fdw, depthwise=True), Fpw) * scale + shift)
     M = Pop.pool(R, 'max', [3, 3], [2, 2], autopad=Pop.SAME_UPPER)
     n, x0, x1, c, k0, k1 = P.TensorIndexes(6)
     IX = P.index([3, 3], 0) * 3 + P.index([3, 3], 1)
     AM = P.Contraction().outShape(M.shape).outAccess(n, x0, x1, c).max(
         P.cond(R[n, 2 * x0 + k0 - 1, 2 * x1 + k1 - 1, c], M[n, x0, x1, c], IX[k0, k1])).build()
-    prog = P.Program('xception_block', [I, Fdw, Fpw, scale, shift], [M, AM])
-    rng = np.random.default_rng(7)
-    vals = [rng.standard_normal((N, H, W, C)).astype(np.float32), (rng.standard_normal((3, 3, C, 1)) * np.sqrt(2.0 / 9)).astype(np.float32),
-            (rng.standard_normal((1, 1, C, C)) * np.sqrt(2.0 / C)).astype(np.float32), rng.uniform(0.5, 1.5, C).astype(np.float32),
-            rng.uniform(-0.5, 0.5, C).astype(np.float32)]
+    prog = P.Program('xception_block', [I], [M, AM])
     runner = P.Runner(prog, target='hip')
-    staged = runner.stage(vals)
+    staged = runner.stage([image])
     best, n, began = None, 0, time.perf_counter()
     while n < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
         runner.run_staged(staged)
