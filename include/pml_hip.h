@@ -245,6 +245,13 @@ int pml_hip_gemm_pack_b2(int64_t plan, const void* b2, pml_hip_stream s);
  * Random values make the chip lower its clock: the second figure is the ceiling a GEMM on N(0,1) data can reach. */
 int pml_hip_probe_mfma(int random_data, int iters, double* tflops, double* core_mhz);
 
+/* 1 when this GEMM runs faster with its tail left to a separate element-wise launch than with the tail fused, 0
+ * otherwise (also for a malformed descriptor).  Today: int8 GEMMs large enough for the 256x256 tile, which a tail that
+ * runs in steps (a requantisation chain) cannot use -- 4096^3 with that tail fused takes 108 us, the plain GEMM 72 us
+ * and the chain over its int32 result 16 us.  A planner asks before it fuses (the reference decides fusion per nest
+ * in pmlc/target/x86/pipeline.cc:304-322 without a cost model).  Makes no device call. */
+int pml_hip_gemm_tail_cheaper_apart(const pml_hip_gemm_desc* desc);
+
 /* Test aid (host arithmetic only, no device call; no counterpart in the reference): the tile (row block, column block)
  * that workgroup `workgroup` of a tiles_m x tiles_n GEMM grid works on.  The order keeps the tiles an XCD holds at any
  * time a compact block of the grid; the tests check that it visits every tile exactly once. */

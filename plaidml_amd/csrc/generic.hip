@@ -437,11 +437,15 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltwiseArgs a) {
 
 // Contiguous fast path: the first input has the output's shape, every operand is
 // either output-shaped, a vector along the last dimension, or a single element,
-// and all element types are 2 bytes wide or all 4 bytes wide.  Each thread
-// moves 16 bytes per tensor.
-template <int ES>
+// and the input's and the output's elements are ES and OES bytes wide: both 2, both 4, or a narrower output
+// (the int32 -> int8 end of a requantisation chain).  Each thread reads 16 bytes of the input at a time and
+// writes the 16 / ES results (16, 8 or 4 bytes).
+typedef int i32x2_t __attribute__((ext_vector_type(2)));
+
+template <int ES, int OES = ES>
 __global__ __launch_bounds__(256) void eltwise_vec_kernel(EltwiseArgs a, int64_t inner, unsigned opnd_full_mask,
                                                           unsigned opnd_vec_mask) {
+  static_assert(OES <= ES && (16 / ES) * OES >= 4, "a thread stores at least one 32-bit word");
   constexpr int V = 16 / ES;
   const pml_hip_eltwise_desc& d = a.d;
   const int64_t n_vec = a.total / V;
@@ -472,7 +476,13 @@ __global__ __launch_bounds__(256) void eltwise_vec_kernel(EltwiseArgs a, int64_t
         v = run_tail<float, int>(d.tail, v, &cur, a.operands, off, a.outs, e0 + e);
         store_scalar<float, int>(&res, e, cur, v);
       }
-      *(i32x4_t*)((unsigned char*)a.out + e0 * ES) = res;
+      if constexpr (OES == ES) {
+        *(i32x4_t*)((unsigned char*)a.out + e0 * ES) = res;
+      } else if constexpr (V * OES == 8) {
+        *(i32x2_t*)((unsigned char*)a.out + e0 * OES) = i32x2_t{res[0], res[1]};
+      } else {
+        *(int*)((unsigned char*)a.out + e0 * OES) = res[0];
+      }
     }
   }
 }
@@ -563,6 +573,100 @@ __global__ __launch_bounds__(256) void eltwise_short_kernel(EltwiseArgs a, int64
       store_scalar<float, int>(&res, e, DT, v);
     }
     *(i32x4_t*)((unsigned char*)a.out + e0 * ES) = res;
+  }
+}
+
+// The end of a quantised layer as a launch of its own: int32 sums -> cast to fp32 -> a chain of plain fp32
+// arithmetic (scale per column, clamps, rounding) -> cast to an 8- or 16-bit integer.  Like the short-chain
+// kernel the steps are decoded once per thread and pass, not per element; a thread turns V = 16 / OES int32
+// values (V / 4 loads of 16 bytes) into one 16-byte store.  Each step is the interpreter's expression for
+// that step on the same fp32 values (steps stay separate loop iterations, so none is contracted with its
+// neighbour), which keeps the two bit-identical.
+__host__ __device__ inline bool requant_chain_op(int opcode) {
+  return short_chain_op(opcode) || opcode == PML_HIP_EPI_ROUND || opcode == PML_HIP_EPI_FLOOR || opcode == PML_HIP_EPI_CEIL;
+}
+
+template <int OES>
+__global__ __launch_bounds__(256) void eltwise_requant_kernel(EltwiseArgs a, int64_t inner, unsigned opnd_full_mask,
+                                                              unsigned opnd_vec_mask) {
+  constexpr int V = 16 / OES, L = V / 4;
+  const pml_hip_eltwise_desc& d = a.d;
+  const int64_t n_vec = a.total / V;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const bool to_unsigned = dt_is_unsigned(d.out_dtype);
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_vec; g += stride) {
+    const int64_t e0 = g * V;
+    const int64_t c0 = e0 % inner;
+    float x[V], y[V];
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+      const i32x4_t raw = *(const i32x4_t*)((const unsigned char*)a.in + (e0 + 4 * l) * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[4 * l + e] = (float)raw[e];  // the chain's leading cast
+    }
+    for (int s = 1; s + 1 < d.tail.n_ops; ++s) {
+      const pml_hip_epi_op& op = d.tail.ops[s];
+      if (op.operand_kind == PML_HIP_OPND_TENSOR) {
+        const int q = op.operand;
+        const unsigned char* base = (const unsigned char*)a.operands[q];
+        if (((opnd_full_mask | opnd_vec_mask) >> q) & 1) {
+          const int64_t at = ((opnd_full_mask >> q) & 1) ? e0 : c0;
+#pragma unroll
+          for (int l = 0; l < L; ++l) {
+            const f32x4_t w = *(const f32x4_t*)(base + (at + 4 * l) * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[4 * l + e] = w[e];
+          }
+        } else {
+          const float b = *(const float*)base;
+#pragma unroll
+          for (int e = 0; e < V; ++e) y[e] = b;
+        }
+      } else {
+        const float b = op.operand_kind == PML_HIP_OPND_IMM ? (float)op.imm : 0.0f;
+#pragma unroll
+        for (int e = 0; e < V; ++e) y[e] = b;
+      }
+#define PML_EACH(EXPR)                            \
+  _Pragma("unroll") for (int e = 0; e < V; ++e) { \
+    const float p = x[e], q = y[e];               \
+    x[e] = EXPR;                                  \
+  }                                               \
+  break;
+      switch (op.opcode) {
+        case PML_HIP_EPI_ADD: PML_EACH(p + q)
+        case PML_HIP_EPI_SUB: PML_EACH(p - q)
+        case PML_HIP_EPI_RSUB: PML_EACH(q - p)
+        case PML_HIP_EPI_MUL: PML_EACH(p * q)
+        case PML_HIP_EPI_DIV: PML_EACH(p / q)
+        case PML_HIP_EPI_RDIV: PML_EACH(q / p)
+        case PML_HIP_EPI_MAX: PML_EACH((p < q) ? q : p)
+        case PML_HIP_EPI_MIN: PML_EACH((p < q) ? p : q)
+        case PML_HIP_EPI_RELU: PML_EACH((p < 0.0f) ? 0.0f : p)
+        case PML_HIP_EPI_NEG: PML_EACH(-p)
+        case PML_HIP_EPI_EXP: PML_EACH(expf(p))
+        case PML_HIP_EPI_LOG: PML_EACH(logf(p))
+        case PML_HIP_EPI_SQRT: PML_EACH(sqrtf(p))
+        case PML_HIP_EPI_TANH: PML_EACH(tanhf(p))
+        case PML_HIP_EPI_MAX_GT: PML_EACH((p > q) ? p : q)
+        case PML_HIP_EPI_ROUND: PML_EACH(c_round<float>(p))
+        case PML_HIP_EPI_FLOOR: PML_EACH(floorf(p))
+        case PML_HIP_EPI_CEIL: PML_EACH(ceilf(p))
+        default: break;
+      }
+#undef PML_EACH
+    }
+    // the closing cast: toward zero into 32 bits (by the target's signedness), then the low OES bytes
+    i32x4_t res = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const unsigned v = to_unsigned ? (unsigned)x[e] : (unsigned)(int)x[e];
+      if constexpr (OES == 1)
+        res[e / 4] |= (int)((v & 0xffu) << (8 * (e % 4)));
+      else
+        res[e / 2] |= (int)((v & 0xffffu) << (16 * (e % 2)));
+    }
+    *(i32x4_t*)((unsigned char*)a.out + e0 * OES) = res;
   }
 }
 
@@ -664,9 +768,54 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
     hipLaunchKernelGGL((eltwise_kernel<double, int64_t>), dim3(grid_for(a.total)), dim3(256), 0, s, a);
     return hipGetLastError();
   }
+  // int32 -> fp32 chain -> narrow integer
+  if (d.in_dtype == PML_HIP_I32 && d.tail.n_ops >= 2 && d.rank >= 1 && d.tail.ops[0].opcode == PML_HIP_EPI_CAST &&
+      d.tail.ops[0].dtype == PML_HIP_F32 && d.tail.ops[d.tail.n_ops - 1].opcode == PML_HIP_EPI_CAST &&
+      d.tail.ops[d.tail.n_ops - 1].dtype == d.out_dtype && !dt_is_float(d.out_dtype) && d.out_dtype != PML_HIP_BOOL &&
+      (dt_size(d.out_dtype) == 1 || dt_size(d.out_dtype) == 2)) {
+    const int V = 16 / dt_size(d.out_dtype);
+    const int64_t inner = d.sizes[d.rank - 1];
+    bool ok = a.total % V == 0 && inner % V == 0 && ((((uintptr_t)a.in | (uintptr_t)a.out) & 15) == 0);
+    int64_t st = 1;
+    for (int r = d.rank - 1; r >= 0; --r) {
+      if (d.sizes[r] != 1 && d.in_strides[r] != st) ok = false;
+      st *= d.sizes[r];
+    }
+    unsigned full_mask = 0, vec_mask = 0;
+    for (int q = 0; q < d.tail.n_operands && ok; ++q) {
+      bool full = true, vec = true, scal = true;
+      int64_t st2 = 1;
+      for (int r = d.rank - 1; r >= 0; --r) {
+        const int64_t os = d.operand_strides[q][r];
+        if (d.sizes[r] != 1) {
+          if (os != st2) full = false;
+          if (os != ((r == d.rank - 1) ? 1 : 0)) vec = false;
+          if (os != 0) scal = false;
+        }
+        st2 *= d.sizes[r];
+      }
+      if (d.tail.operand_dtype[q] != PML_HIP_F32 || !(full || vec || scal)) ok = false;
+      if (full)
+        full_mask |= 1u << q;
+      else if (vec)
+        vec_mask |= 1u << q;
+      if ((full || vec) && ((uintptr_t)a.operands[q] & 15)) ok = false;
+    }
+    for (int k = 1; k + 1 < d.tail.n_ops && ok; ++k)
+      ok = requant_chain_op(d.tail.ops[k].opcode) && d.tail.ops[k].dtype == PML_HIP_F32;
+    if (ok) {
+      const unsigned g = grid_for(a.total / V);
+      if (dt_size(d.out_dtype) == 1)
+        hipLaunchKernelGGL((eltwise_requant_kernel<1>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
+      else
+        hipLaunchKernelGGL((eltwise_requant_kernel<2>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
+      return hipGetLastError();
+    }
+  }
   // try the 16-byte path
   const int es = dt_size(d.in_dtype);
-  bool vec_ok = (es == 2 || es == 4) && dt_size(d.out_dtype) == es && d.rank >= 1;
+  const int oes = dt_size(d.out_dtype);
+  bool vec_ok = (es == 2 || es == 4) && (oes == es || (es == 4 && (oes == 1 || oes == 2))) && d.rank >= 1;
   int64_t inner = d.rank >= 1 ? d.sizes[d.rank - 1] : 1;
   unsigned full_mask = 0, vec_mask = 0, row_mask = 0;
   if (vec_ok) {
@@ -702,7 +851,7 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
     for (int k = 0; k < d.tail.n_ops; ++k) {
       const pml_hip_epi_op& op = d.tail.ops[k];
       if (op.opcode == PML_HIP_EPI_STORE) vec_ok = false;
-      if (op.opcode == PML_HIP_EPI_CAST && dt_size(op.dtype) != es && k == d.tail.n_ops - 1) vec_ok = false;
+      if (op.opcode == PML_HIP_EPI_CAST && dt_size(op.dtype) != oes && k == d.tail.n_ops - 1) vec_ok = false;
     }
     const int V = 16 / es;
     if (a.total % V != 0 || inner % V != 0) vec_ok = false;
@@ -731,6 +880,10 @@ hipError_t eltwise_launch(const EltwiseArgs& a, hipStream_t s) {
     if (row_mask == 0) {
       if (es == 2)
         hipLaunchKernelGGL((eltwise_vec_kernel<2>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
+      else if (oes == 2)
+        hipLaunchKernelGGL((eltwise_vec_kernel<4, 2>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
+      else if (oes == 1)
+        hipLaunchKernelGGL((eltwise_vec_kernel<4, 1>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
       else
         hipLaunchKernelGGL((eltwise_vec_kernel<4>), dim3(g), dim3(256), 0, s, a, inner, full_mask, vec_mask);
       return hipGetLastError();

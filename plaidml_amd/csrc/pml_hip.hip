@@ -548,6 +548,17 @@ static int gemm_desc_kind(const pml_hip_gemm_desc* d) {
   return kind;
 }
 
+int pml_hip_gemm_tail_cheaper_apart(const pml_hip_gemm_desc* d) {
+  if (!d || d->tail.n_ops == 0 || d->k2 != 0) return 0;
+  const int kind = gemm_desc_kind(d);
+  if (kind != KIND_I8) return 0;
+  int mode = 0, relu = 0;
+  classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
+  if (mode == 1 || mode == 2) return 0;
+  const int64_t k_bytes = d->k * dt_size(d->in_dtype);
+  return choose_tile(d->m, d->n, k_bytes, kind, true) == TILE_256x256_W8 && choose_tile(d->m, d->n, k_bytes, kind, false) != TILE_256x256_W8;
+}
+
 int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   const int kind = gemm_desc_kind(d);
   if (kind < 0) return 0;

@@ -29,7 +29,7 @@ EXPORTS = [
     'pml_hip_memcpy_d2d', 'pml_hip_fill_u32', 'pml_hip_stream_create', 'pml_hip_stream_destroy',
     'pml_hip_stream_sync', 'pml_hip_event_create', 'pml_hip_event_destroy', 'pml_hip_event_record',
     'pml_hip_event_sync', 'pml_hip_event_elapsed_ms', 'pml_hip_gemm_dispatch', 'pml_hip_gemm_invoke',
-    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_tile_of_workgroup',
+    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_tile_of_workgroup', 'pml_hip_gemm_tail_cheaper_apart',
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
@@ -154,6 +154,7 @@ def lib():
         L.pml_hip_gemm_pack_b2.argtypes = [ctypes.c_int64, vp, vp]
         L.pml_hip_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
         L.pml_hip_tile_of_workgroup.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+        L.pml_hip_gemm_tail_cheaper_apart.argtypes = [ctypes.POINTER(GemmDesc)]
         L.pml_hip_conv2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp, pp, pp, vp]
         L.pml_hip_dwconv2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, pp, pp, vp]
         L.pml_hip_pool2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp]

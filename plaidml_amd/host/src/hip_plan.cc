@@ -1196,6 +1196,16 @@ class Planner {
     if (d.init_kind && !dense_out && !(d.init_row_stride == 0 && d.init_col_stride <= 1)) return unconsume(tb), false;
     d.tail = tb.tail;
     d.c_dtype = hipType(tb.final_dtype);
+    if (tb.tail.n_ops && pml_hip_gemm_tail_cheaper_apart(&d)) {
+      // the kernel library multiplies this shape faster under a plain tail: the chain stays with the
+      // element-wise operations that follow (which fuse among themselves)
+      unconsume(tb);
+      tb = TailBuild();
+      tb.final_value = op.result;
+      tb.final_dtype = op.result->shape.elementType;
+      d.tail = tb.tail;
+      d.c_dtype = hipType(tb.final_dtype);
+    }
     s.a = bufferFor(A);
     s.b = bufferFor(B);
     s.c = bufferFor(tb.final_value);

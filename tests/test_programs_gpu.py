@@ -231,6 +231,43 @@ def test_transposed_convolution_from_the_input_side_at_size():
     assert E.last_run_stats()['kernel_ms'] < 50.0
 
 
+@pytest.mark.parametrize('out_name', ['INT8', 'UINT8', 'INT16'])
+@pytest.mark.parametrize('R,C', [(64, 48), (33, 40), (5, 37), (256, 1024)])
+def test_requantisation_chain_as_its_own_launch(R, C, out_name):
+    """int32 -> fp32 -> scale per column -> clamp -> round -> narrow integer as an element-wise launch of its own
+    (what a large int8 GEMM leaves to a second launch): the typed-chain kernel (rows of whole 16-byte output
+    vectors), the vector kernel with a narrower output (rows of whole 16-byte input vectors) and the interpreter
+    (anything else) must give the bits of the same fp32 arithmetic in numpy; values beyond the clamp included."""
+    print('requantisation chain', (R, C, out_name), flush=True)
+    lo, hi = {'INT8': (-127.0, 127.0), 'UINT8': (0.0, 255.0), 'INT16': (-32767.0, 32767.0)}[out_name]
+    X = E.Placeholder(E.DType.INT32, [R, C])
+    S = E.Placeholder(E.DType.FLOAT32, [C])
+    Q = E.cast(E.round(op.clip(E.cast(X, E.DType.FLOAT32) * S, lo, hi)), getattr(E.DType, out_name))
+    prog = E.Program('requant', [X, S], [Q])
+    rng = np.random.default_rng(R * 131 + C)
+    x = rng.integers(-60000, 60001, (R, C)).astype(np.int32)
+    x[0, :4] = [0, 1, -1, 2 ** 31 - 1]
+    sc = rng.uniform(0.001, 0.01, C).astype(np.float32) * (100.0 if out_name == 'INT16' else 1.0)
+    got, = E.run(prog, [x, sc], target='hip')
+    y = np.minimum(np.maximum(x.astype(np.float32) * sc, np.float32(lo)), np.float32(hi)).astype(np.float32)
+    want = np.where(y >= 0, np.floor(y + np.float32(0.5)), np.ceil(y - np.float32(0.5))).astype(np.float32)
+    np.testing.assert_array_equal(got, want.astype(got.dtype))
+    assert got.min() == lo and got.max() == hi  # both clamps bite
+
+
+def test_large_int8_gemm_leaves_its_requantisation_to_a_second_launch():
+    """4096^3 int8 with the requantisation chain: the planner asks the kernel library, which multiplies this shape
+    faster under a plain tail, and plans two launches; a small problem keeps the chain fused."""
+    prog = programs.config2_int8_gemm(E, op, M=4096, N=4096, K=4096)[0]
+    prog.compile('hip')
+    plan = dict(prog.passes)['hip-plan']
+    assert '2 launches' in plan and 'gemm si8 m=4096 n=4096 k=4096 B=[k][n] -> 4096x4096xsi32' in plan, plan
+    assert 'eltwise cast tail=[cast:f32 mul(t0)' in plan, plan
+    prog = programs.config2_int8_gemm(E, op)[0]
+    prog.compile('hip')
+    assert '1 launches' in dict(prog.passes)['hip-plan']
+
+
 def test_run_checks_arity_and_shapes():
     prog, vals, _ = programs.dot_f32(E, op)
     prog.compile()
