@@ -148,15 +148,18 @@ def int8_program_leg(n=4096, runs=5):
     a = np.random.default_rng(4).integers(-127, 128, (n, n), dtype=np.int8)
     b = np.random.default_rng(5).integers(-127, 128, (n, n), dtype=np.int8)
     sc = np.random.default_rng(6).uniform(0.001, 0.01, n).astype(np.float32)
-    times = []
-    for _ in range(runs):
-        runner.run([a, b, sc])
-        times.append(P.last_run_stats())
-    best = min(times[1:], key=lambda t: t['kernel_ms'])
+    runner.run([a, b, sc])  # one whole run for the transfer times
+    first = P.last_run_stats()
+    staged = runner.stage([a, b, sc])  # then back to back on staged inputs (B is still transposed in every run)
+    best, k, began = None, 0, time.perf_counter()
+    while k < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
+        runner.run_staged(staged)
+        st = P.last_run_stats()
+        best, k = (st if best is None or st['kernel_ms'] < best['kernel_ms'] else best), k + 1
     ops = 2.0 * n ** 3
     return {'kernel_ms': round(best['kernel_ms'], 4), 'launches': int(best['launches']), 'TOP/s': round(ops / best['kernel_ms'] / 1e9, 1),
-            'frac_mfma_i8': round(ops / best['kernel_ms'] / 1e9 / PEAK['i8'], 4), 'h2d_ms': round(best['h2d_ms'], 3),
-            'd2h_ms': round(best['d2h_ms'], 3)}
+            'frac_mfma_i8': round(ops / best['kernel_ms'] / 1e9 / PEAK['i8'], 4), 'h2d_ms': round(first['h2d_ms'], 3),
+            'd2h_ms': round(first['d2h_ms'], 3)}
 
 
 def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):  # noqa: C901
@@ -331,13 +334,20 @@ def conv_through_exec(N, H, W, CI, CO, Iv, Fv, runs=6):
     runner = P.Runner(prog, target='hip')
     bias = np.zeros(CO, np.float32)
     times = []
-    for _ in range(runs):
+    for _ in range(runs):  # whole runs: upload, launch, download (the launch finds an idle device)
         runner.run([Iv, Fv, bias])
         times.append(P.last_run_stats())
-    best = min(times[1:], key=lambda t: t['kernel_ms'])
+    cold = min(times[1:], key=lambda t: t['kernel_ms'])
+    staged = runner.stage([Iv, Fv, bias])  # and back to back on staged inputs, as a stream of batches arrives
+    warm, n, began = None, 0, time.perf_counter()
+    while n < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
+        runner.run_staged(staged)
+        st = P.last_run_stats()
+        warm, n = (st if warm is None or st['kernel_ms'] < warm['kernel_ms'] else warm), n + 1
     plan = [v for k, v in prog.passes if k == 'hip-plan']
-    return {'kernel_ms': round(best['kernel_ms'], 5), 'launches': int(best['launches']), 'h2d_ms': round(best['h2d_ms'], 3),
-            'd2h_ms': round(best['d2h_ms'], 3), 'plan': plan[0].splitlines()[1].strip() if plan else ''}
+    return {'kernel_ms': round(warm['kernel_ms'], 5), 'kernel_ms_after_an_upload': round(cold['kernel_ms'], 5),
+            'launches': int(warm['launches']), 'h2d_ms': round(cold['h2d_ms'], 3), 'd2h_ms': round(cold['d2h_ms'], 3),
+            'plan': plan[0].splitlines()[1].strip() if plan else ''}
 
 
 def main():
