@@ -83,10 +83,14 @@ constexpr int igemm_waves_per_simd() {
   return (NT / 256) * (2 * Ring<BM, BN, STAGES, SLAB>::kAlloc <= kLdsBytes ? 2 : 1);
 }
 
-// BKN: the right-hand side is the caller's row-major B[K][N] of 4-byte elements (p.Bt, p.ldbt its row length): a slab
-// is then 32 rows of B as they lie in memory, [k][n] in LDS, and a lane gathers the four K-values of its fragment
-// with four 4-byte reads (32 consecutive columns per half wavefront: no bank conflicts).  The fp32 MFMA takes one
-// K-value per lane anyway, so nothing has to be transposed -- neither by a launch of its own nor in registers.
+// BKN: the right-hand side is the caller's row-major B[K][N] (p.Bt, p.ldbt its row length): a slab is then the
+// rows of B as they lie in memory, [k][n] in LDS, and nothing is transposed by a launch of its own.
+// fp32 kinds: a lane gathers the four K-values of its fragment with four 4-byte reads (32 consecutive columns per
+// half wavefront: no bank conflicts); the fp32 MFMA takes one K-value per lane anyway.
+// int8: the 16 K-values of a lane's fragment come from two transposing LDS reads (ds_read_b64_tr_b8: the 16 lanes
+// of a group each name 8 bytes -- here 8 columns of one K-row -- and lane i receives byte i % 8 of the data named
+// by lanes i / 8, i / 8 + 2, ..., i.e. 8 K-values of column i).  The 16-byte chunks of K-row k are stored at
+// positions XORed with k % 8 so that the 8 rows of such a read fall into different banks.
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128,
           bool BKN = false>
 __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>())) void igemm_kernel(IgemmArgs p_by_value) {
@@ -104,7 +108,11 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   constexpr int ES = KIND == KIND_BF16 ? 2 : (KIND == KIND_I8 ? 1 : 4);
   constexpr bool kSplit = KIND == KIND_F32X3 || KIND == KIND_F32X3P;  // fp32 operands as three bf16 products
   constexpr bool kSplitB = KIND == KIND_F32X3P;                       // ... the right-hand side split when it was packed
-  static_assert(!BKN || ((KIND == KIND_F32 || KIND == KIND_F32X3) && !CONV && SLAB == 128), "a [K][N] right-hand side: fp32 GEMMs only");
+  static_assert(!BKN || ((KIND == KIND_F32 || KIND == KIND_F32X3 || KIND == KIND_I8) && !CONV && SLAB == 128),
+                "a [K][N] right-hand side: fp32 and int8 GEMMs only");
+  constexpr int kRowChunks = BN * ES / 16;                       // BKN: 16-byte chunks of one K-row of the tile
+  constexpr int kRowKey = kRowChunks >= 8 ? 7 : kRowChunks - 1;  // int8: chunk positions are XORed with (k & kRowKey) * kRowKeyMul
+  constexpr int kRowKeyMul = kRowChunks >= 16 ? 2 : 1;
   constexpr int kWaves = NT / 64;
   constexpr int kRowsPerPass = NT / CPR;  // operand rows one load of all threads covers
   constexpr int WAVES_N = kWaves / WAVES_M / WAVES_K;
@@ -198,10 +206,10 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
 #pragma unroll
   for (int i = 0; i < B_VECS; ++i) {
     if constexpr (BKN) {
-      constexpr int kChunksPerRow = BN / 4;  // 16-byte chunks of one K-row of the tile
       const int c = tid + i * NT;
-      const int64_t n = n0 + (c % kChunksPerRow) * 4;
-      b_krow[i] = c / kChunksPerRow;
+      b_krow[i] = c / kRowChunks;
+      const int chunk = KIND == KIND_I8 ? (c % kRowChunks) ^ ((b_krow[i] & kRowKey) * kRowKeyMul) : c % kRowChunks;  // what this LDS position holds
+      const int64_t n = n0 + chunk * (16 / ES);
       b_off[i] = n < p.N ? (unsigned)(((int64_t)b_krow[i] * p.ldbt + n) * ES) : kOutside;
     } else {
       const int64_t n = n0 + lr + kRowsPerPass * i;
@@ -371,13 +379,31 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       fslot[kb] = ((gb * 2 + h) ^ key) * 16;
       fslot_b[kb] = fslot[kb];
     }
-    // BKN: chunk c of a row holds K-values 4c .. 4c + 3, which in [k][n] order are four rows of BN * 4 bytes
-    if constexpr (BKN) fslot_b[kb] = (kSplit ? ((gb & ~1) * 2 + 2 * h + (gb & 1)) : (gb * 2 + h)) * 4 * (BN * 4);
+    // BKN: chunk c of a row holds K-values 4c .. 4c + 3 (int8: 16c .. 16c + 15), which in [k][n] order are that
+    // many rows of BN elements
+    if constexpr (BKN) fslot_b[kb] = (kSplit ? ((gb & ~1) * 2 + 2 * h + (gb & 1)) : (gb * 2 + h)) * (16 / ES) * (BN * ES);
+  }
+  // BKN, int8: what a lane names in a transposing read of 32-column block j -- K-row (lane % 16) / 2 of the 8, the
+  // 8 columns (lane % 2) of the 16 its group of lanes covers -- as a byte offset into the stage's [k][n] part
+  int bcol[(BKN && KIND == KIND_I8) ? NI : 1];
+  if constexpr (BKN && KIND == KIND_I8) {
+    const int jrow = (lane & 15) >> 1;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int chunk = (wn * WN + j * 32) / 16 + ((lane >> 4) & 1);
+      bcol[j] = jrow * BN + ((chunk ^ ((jrow & kRowKey) * kRowKeyMul)) * 16) + (lane & 1) * 8;
+    }
   }
   // the Bt fragment of 32-column block j for the K-block whose slot is `slot`, out of the stage whose Bt part `bb`
   // points into (at the wavefront's first column and the lane's row or column)
   auto read_b = [&](const unsigned char* bb, int j, int slot) {
-    if constexpr (BKN) {
+    if constexpr (BKN && KIND == KIND_I8) {
+      typedef int v2i_t __attribute__((ext_vector_type(2)));
+      typedef __attribute__((address_space(3))) v2i_t* lds_v2i_ptr;
+      const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)PML_LDS(bb + slot + bcol[j]));
+      const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)PML_LDS(bb + slot + bcol[j] + 8 * BN));
+      return i32x4_t{lo[0], lo[1], hi[0], hi[1]};
+    } else if constexpr (BKN) {
       i32x4_t v;
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = *(const int*)(bb + slot + e * (BN * 4) + j * 32 * 4);
@@ -400,7 +426,8 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   i32x4_t xa_head[kSplit ? MI : 1], xa_rem[kSplit ? MI : 1];
   i32x4_t xb_head[kSplit && !kSplitB ? NI : 1], xb_rem[kSplit && !kSplitB ? NI : 1];
   const unsigned char* a_base = smem + (wm * WM + frow) * kSlabBytes;
-  const unsigned char* b_base = BKN ? smem + BM * kSlabBytes + (wn * WN + frow) * 4 : smem + (BM + wn * WN + frow) * kSlabBytes;
+  const unsigned char* b_base = !BKN ? smem + (BM + wn * WN + frow) * kSlabBytes
+                                     : smem + BM * kSlabBytes + (KIND == KIND_I8 ? 0 : (wn * WN + frow) * 4);
   __builtin_amdgcn_s_waitcnt(0x0F70 | (((kStages - 1) * kLoads) & 15) | ((((kStages - 1) * kLoads) >> 4) << 14));
   __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -413,7 +440,9 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
     int next_stage = stage + 1;
     if (next_stage == kStages) next_stage = 0;
     const unsigned char* a_next = smem + next_stage * kStage + (wm * WM + frow) * kSlabBytes;
-    const unsigned char* b_next = smem + next_stage * kStage + (BKN ? BM * kSlabBytes + (wn * WN + frow) * 4 : (BM + wn * WN + frow) * kSlabBytes);
+    const unsigned char* b_next = smem + next_stage * kStage +
+                                  (!BKN ? (BM + wn * WN + frow) * kSlabBytes
+                                        : BM * kSlabBytes + (KIND == KIND_I8 ? 0 : (wn * WN + frow) * 4));
 #pragma unroll
     for (int kb = 0; kb < kBlocks; ++kb) {
       const int cur = kb & 1, nxt = cur ^ 1;
@@ -650,7 +679,7 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
 
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
-  if constexpr ((KIND == KIND_F32 || KIND == KIND_F32X3) && !CONV && SLAB == 128) {
+  if constexpr ((KIND == KIND_F32 || KIND == KIND_F32X3 || KIND == KIND_I8) && !CONV && SLAB == 128) {
     if (a.b_kn) {
       const int64_t tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
       const int64_t tiles = tiles_m * tiles_n;

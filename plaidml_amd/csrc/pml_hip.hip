@@ -605,11 +605,25 @@ struct SecondProduct {
   bool packed2 = false;
 };
 
-// An fp32 right-hand side that arrives with the call in its row-major [K][N] form is read as it is (the fp32 kinds
-// gather their K-values from [k][n] slabs); everything else is transposed into Bt[N][K] first.
+// An fp32 or int8 right-hand side that arrives with the call in its row-major [K][N] form is read as it is (the
+// fp32 kinds gather their K-values from [k][n] slabs, int8 reads them with transposing LDS reads); everything else
+// is transposed into Bt[N][K] first.  Rows must be whole 16-byte vectors.
 static bool reads_b_as_given(const pml_hip_gemm_desc& d, int mfma_kind, const void* b) {
-  return b && !d.b_layout && (mfma_kind == KIND_F32 || mfma_kind == KIND_F32X3) && d.k2 == 0 && d.n % 4 == 0 && d.ldb % 4 == 0 &&
-         ((uintptr_t)b & 15) == 0 && d.k * d.ldb * 4 < ((int64_t)1 << 31);
+  if (mfma_kind != KIND_F32 && mfma_kind != KIND_F32X3 && mfma_kind != KIND_I8) return false;
+  const int64_t es = mfma_kind == KIND_I8 ? 1 : 4, v = 16 / es;
+  if (!(b && !d.b_layout && d.k2 == 0 && d.n % v == 0 && d.ldb % v == 0 && ((uintptr_t)b & 15) == 0 &&
+        d.k * d.ldb * es < ((int64_t)1 << 31)))
+    return false;
+  if (mfma_kind == KIND_I8) {
+    // The transposing reads make the int8 kernel about 15 % slower (4096^3: 86 us against 74 + 10 for the copy), so
+    // they pay while the transposed copy -- a launch of at least 5 us, 3.2 TB/s beyond that -- costs more than
+    // that share of the multiplication (priced at the 1.8 POP/s the kernel reaches): up to about 3500 rows at
+    // K = N = 4096, always for small problems.
+    const double t_gemm = 2.0 * (double)d.m * (double)d.n * (double)d.k / 1.8e15;
+    const double t_copy = std::max(5e-6, 2.0 * (double)d.k * (double)d.n / 3.2e12);
+    return 0.15 * t_gemm < t_copy;
+  }
+  return true;
 }
 
 static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* bt, int64_t bt_ld, bool packed,

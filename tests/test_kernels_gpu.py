@@ -101,6 +101,9 @@ def test_every_tile_configuration(tile, monkeypatch):
     A = rng.integers(-127, 128, (M, K), dtype=np.int8)
     B = rng.integers(-127, 128, (K, N), dtype=np.int8)
     np.testing.assert_array_equal(run_gemm(A, B, hk.I8, hk.I32), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.int32))
+    # rows of whole 16-byte vectors: the int8 right-hand side is read where it lies, through transposing LDS reads
+    B16 = rng.integers(-127, 128, (K, 528), dtype=np.int8)
+    np.testing.assert_array_equal(run_gemm(A, B16, hk.I8, hk.I32), (A.astype(np.int64) @ B16.astype(np.int64)).astype(np.int32))
     Af = E.round_bf16(rng.standard_normal((M, K)).astype(np.float32))
     Bf = E.round_bf16(rng.standard_normal((K, N)).astype(np.float32))
     bias = E.round_bf16(rng.standard_normal(N).astype(np.float32))
@@ -938,6 +941,34 @@ def test_gemm_f32_right_hand_side_as_given(M, N, K, ldb, flags):
     np.testing.assert_array_equal(as_given.view(np.uint32), n_major.view(np.uint32))
     ref = A.astype(np.float64) @ B.astype(np.float64)
     np.testing.assert_allclose(as_given, ref, rtol=FP32_RTOL if not flags else 1e-3, atol=1e-4 if not flags else 2e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('M,N,K,ldb', [(512, 4096, 4096, 4096), (100, 64, 48, 80), (257, 144, 1040, 160), (64, 16, 16, 16),
+                                       (4096, 1024, 2048, 1024)])
+def test_gemm_int8_right_hand_side_as_given(M, N, K, ldb):
+    """An int8 [K][N] right-hand side whose rows are whole 16-byte vectors is read where it lies (K-values gathered by
+    transposing LDS reads) as long as a transposed copy would cost more than the slower reads: bit for bit the int64
+    product, with a leading dimension wider than N whose gap holds values that must not be read, ragged tiles in
+    M, N and K, and (the last case) a problem large enough to take the transposed copy instead."""
+    print('int8 right-hand side as given', (M, N, K, ldb), flush=True)
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    Bh = rng.integers(-127, 128, (K, ldb), dtype=np.int8)
+    d = hk.GemmDesc()
+    d.in_dtype, d.out_dtype, d.c_dtype = hk.I8, hk.I32, hk.I32
+    d.m, d.n, d.k, d.lda, d.ldb, d.ldc = M, N, K, K, ldb, N
+    plan = hk.lib().pml_hip_gemm_dispatch(ctypes.byref(d))
+    assert plan, hk.lib().pml_hip_last_error()
+    dA, dB, dC = hk.DeviceBuffer.from_numpy(A), hk.DeviceBuffer.from_numpy(Bh), hk.DeviceBuffer(M * N * 4)
+    none = hk.ptr_array([])
+    hk.check(hk.lib().pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, None, none, none, None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    got = dC.to_numpy(np.int32, (M, N))
+    hk.lib().pml_hip_plan_free(plan)
+    # (float64 holds these sums exactly -- |sum| <= 127^2 K < 2^53 -- and multiplies through BLAS)
+    want = (A.astype(np.float64) @ Bh[:, :N].astype(np.float64)).astype(np.int64).astype(np.int32)
+    np.testing.assert_array_equal(got, want)
 
 
 MANY_ROWS_CASES = [(140837, 128, 64), (70000, 256, 136), (140800, 128, 256)]
