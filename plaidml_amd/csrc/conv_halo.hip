@@ -1097,7 +1097,197 @@ hipError_t launch(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// The few-channel, stride-2 convolution at the head of an image network (7x7x3 -> 64), after its input has been
+// re-blocked into 2x2 pixel blocks of 16 channels (32 bytes): a unit-stride convolution with 4x4 block taps, K = 256.
+// As an implicit GEMM it has 4 slabs per tile and 25 thousand tiles, each of which fetches the same 32 KB filter
+// and pays its own start-up and tail.  Here a workgroup walks down the output rows of one image:
+//   - the filter lives in registers for the kernel's life (a wavefront holds all 64 channels: 16 taps x 2 blocks
+//     of 32 channels x 16 bytes per lane);
+//   - LDS holds a ring of five re-blocked input rows (one row of padding slots included); each output row needs
+//     four of them, so every step fetches ONE new row (a 16-byte chunk per thread), which arrives in registers
+//     while the current row is multiplied and is written into the slot the oldest row has left;
+//   - a wavefront takes 32 neighbouring pixels: a tap's operand is one 16-byte LDS read per lane at consecutive
+//     32-byte pixels (the two half-wavefronts read the two channel halves: 1 KB contiguous, no bank conflicts);
+//   - MFMA row 8q + 4h + e is given output channel 32j + 16h + 4q + e, so a lane ends up with 16 consecutive
+//     channels of its pixel and stores 32 bytes.
+// One barrier per output row.  bf16, 64 output channels, plain tail (bias, optional ReLU).
+// ---------------------------------------------------------------------------
+constexpr int kBlkPixBytes = 32;
+constexpr int kBlkRing = 5;
+
+__global__ __launch_bounds__(256, 2) void conv_blocks4x4_kernel(IgemmArgs p, int rows_per_wg, int wgs_per_image) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), h = lane >> 5;
+  const int n = (int)blockIdx.x / wgs_per_image, blk = (int)blockIdx.x % wgs_per_image;
+  const int oy0 = blk * rows_per_wg;
+  const int oy1 = oy0 + rows_per_wg < p.OH ? oy0 + rows_per_wg : p.OH;
+  if (oy0 >= oy1) return;
+  const int Wp = p.OW + 3;                      // pixel slots of an LDS row: source columns -PW .. OW + 2 - PW
+  const int row_bytes = Wp * kBlkPixBytes;
+  const int n_chunks = Wp * 2;                  // 16-byte chunks of a row (at most 2 per thread: OW <= 128)
+  float* const bias = (float*)(smem + kBlkRing * row_bytes);
+  unsigned char* const staging = smem + kBlkRing * row_bytes + 256;  // 4 KB per wavefront
+
+  // the filter: MFMA row i of block j holds output channel 32j + 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3)
+  i32x4_t breg[16][2];
+  {
+    const int i = lane & 31;
+    const int c = 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const unsigned char* src = (const unsigned char*)p.Bt + (int64_t)(32 * j + c) * p.ldbt * 2 + h * 16;
+#pragma unroll
+      for (int t = 0; t < 16; ++t) breg[t][j] = *(const i32x4_t*)(src + t * kBlkPixBytes);
+    }
+  }
+  if (tid < 64) bias[tid] = p.init != nullptr ? load_scalar<float, int>(p.init, (int64_t)tid * p.init_cs, p.init_dtype).f : 0.f;
+
+  // one re-blocked input row (or zeros where it lies outside the image) -> registers -> its ring slot
+  auto fetch_row = [&](int sy, i32x4_t (&regs)[2]) {
+    const bool row_ok = (unsigned)sy < (unsigned)p.H;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int c = tid + 256 * k, col = (c >> 1) - p.PW;
+      regs[k] = i32x4_t{0, 0, 0, 0};
+      if (!(c < n_chunks && row_ok && (unsigned)col < (unsigned)p.W)) continue;
+      if (p.raw_in == nullptr) {
+        regs[k] = *(const i32x4_t*)((const unsigned char*)p.A + (((int64_t)n * p.H + sy) * p.W + col) * kBlkPixBytes + (c & 1) * 16);
+      } else {
+        // block (sy, col) of a 3-channel image: pixels (2 sy, 2 col), (2 sy, 2 col + 1) -- 12 contiguous bytes --
+        // then the same two of row 2 sy + 1, then 8 bytes of zeros; the width is even, so both runs start on
+        // 4-byte boundaries
+        const int* top = (const int*)((const unsigned char*)p.raw_in + (((int64_t)n * p.raw_h + 2 * sy) * p.raw_w + 2 * col) * 6);
+        const int* bot = top + p.raw_w * 6 / 4;
+        const bool bot_ok = 2 * sy + 1 < p.raw_h;
+        if ((c & 1) == 0)
+          regs[k] = i32x4_t{top[0], top[1], top[2], bot_ok ? bot[0] : 0};
+        else if (bot_ok)
+          regs[k] = i32x4_t{bot[1], bot[2], 0, 0};
+      }
+    }
+  };
+  auto put_row = [&](int ring_slot, const i32x4_t (&regs)[2]) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int c = tid + 256 * k;
+      if (c < n_chunks) *(i32x4_t*)(smem + ring_slot * row_bytes + c * 16) = regs[k];
+    }
+  };
+  // output row oy reads source rows oy - PH .. oy - PH + 3, kept in ring slots oy % 5 .. (oy + 3) % 5
+  {
+    i32x4_t regs[2];
+    for (int t = 0; t < 4; ++t) {
+      fetch_row(oy0 - p.PH + t, regs);
+      put_row((oy0 + t) % kBlkRing, regs);
+    }
+  }
+  __syncthreads();
+
+  const float lo = p.tail_relu ? 0.f : -__builtin_inff();
+  // Two fetches are in flight: the row the next step needs (`due`, requested one step ago and written to its slot at
+  // the end of this step) and the row the step after that needs (`later`, requested now).  One step's arithmetic is
+  // shorter than a trip to memory; two steps' worth of it covers more of one.
+  auto step = [&](int oy, i32x4_t (&due)[2], i32x4_t (&later)[2]) {
+    const bool more = oy + 1 < oy1;
+    if (oy + 2 < oy1) fetch_row(oy + 5 - p.PH, later);
+    for (int b = wave; b * 32 < p.OW; b += 4) {
+      const int ox = b * 32 + (lane & 31);
+      const int oxc = ox < p.OW ? ox : p.OW - 1;  // lanes past the row's end multiply its last pixel and store nothing
+      f32x16_t acc[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4_t v = *(const f32x4_t*)(bias + 32 * j + 16 * h + 4 * q);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[j][4 * q + e] = v[e];
+        }
+#pragma unroll
+      for (int ty = 0; ty < 4; ++ty) {
+        const unsigned char* base = smem + ((oy + ty) % kBlkRing) * row_bytes + oxc * kBlkPixBytes + h * 16;
+#pragma unroll
+        for (int tx = 0; tx < 4; ++tx) {
+          const i32x4_t fa = *(const i32x4_t*)(base + tx * kBlkPixBytes);
+#pragma unroll
+          for (int j = 0; j < 2; ++j) mma_block<KIND_BF16>(acc[j], breg[ty * 4 + tx][j], fa);
+        }
+      }
+      // The wavefront's 32 pixels x 128 bytes go through its own 4 KB of LDS, so that a store instruction writes
+      // whole 128-byte lines (8 lanes per pixel) instead of 16 bytes in each of 64 lines.  The 16-byte chunks of a
+      // pixel sit at positions XORed with the pixel number (bank conflicts of the writes: 4-way instead of 32-way).
+      unsigned char* const stage = staging + wave * 4096;
+      {
+        const int px = lane & 31;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            unsigned w[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              float v0 = acc[j][8 * half + 2 * k], v1 = acc[j][8 * half + 2 * k + 1];
+              v0 = v0 < lo ? lo : v0;
+              v1 = v1 < lo ? lo : v1;
+              const f32x2_t pair = {v0, v1};
+              const bf16x2_t hh = __builtin_convertvector(pair, bf16x2_t);
+              __builtin_memcpy(&w[k], &hh, 4);
+            }
+            const int chunk = 4 * j + 2 * h + half;  // channels 32 j + 16 h + 8 half .. + 7
+            *(u32x4_t*)(stage + px * 128 + ((chunk ^ (px & 7)) << 4)) = u32x4_t{w[0], w[1], w[2], w[3]};
+          }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      {
+        const int chunk = lane & 7;
+        unsigned char* const out_row = (unsigned char*)p.C + (((int64_t)n * p.OH + oy) * p.OW + b * 32) * p.ldc * 2 + chunk * 16;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int px = it * 8 + (lane >> 3);
+          const u32x4_t v = *(const u32x4_t*)(stage + px * 128 + ((chunk ^ (px & 7)) << 4));
+          if (b * 32 + px < p.OW) *(u32x4_t*)(out_row + (int64_t)px * p.ldc * 2) = v;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (more) put_row((oy + 4) % kBlkRing, due);  // the slot of row oy - 1, which nothing reads any more
+    __syncthreads();
+  };
+  i32x4_t ra[2], rb[2];
+  if (oy0 + 1 < oy1) fetch_row(oy0 + 4 - p.PH, ra);
+  for (int oy = oy0; oy < oy1; oy += 2) {
+    step(oy, ra, rb);
+    if (oy + 1 < oy1) step(oy + 1, rb, ra);
+  }
+}
+
 }  // namespace
+
+// Does the re-blocked convolution `a` (as conv_args describes it: H x W blocks of pix_pitch bytes, KH block rows of
+// CI = 4 blocks x 16 channels) fit conv_blocks4x4_kernel?  Returns the LDS bytes it needs, or 0.
+size_t conv_blocks4x4_prepare(int kind, const IgemmArgs& a) {
+  if (kind != KIND_BF16 || a.KH != 4 || a.KW != 1 || a.CI != 64 || a.pix_pitch != kBlkPixBytes || a.K != 256) return 0;
+  if (a.N != 64 || a.ldbt != 256 || a.OW > 128 || a.OW < 1 || a.SH != 1 || a.SW != 1 || a.DH != 1 || a.DW != 1) return 0;
+  if (a.PH < 0 || a.PH > 3 || a.PW < 0 || a.PW > 3) return 0;
+  if (a.tail_mode != 1 || a.out_dtype != PML_HIP_BF16 || a.c_dtype != PML_HIP_BF16 || a.init_rs != 0) return 0;
+  if ((a.ldc * 2) % 16 != 0 || (((uintptr_t)a.C | (uintptr_t)a.Bt) & 15) != 0) return 0;
+  return (size_t)kBlkRing * (a.OW + 3) * kBlkPixBytes + 64 * 4 + 4 * 4096;
+}
+
+hipError_t conv_blocks4x4_launch(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
+  // two workgroups per CU, each a run of consecutive output rows of one image
+  int per_image = (2 * n_cus + a.NB - 1) / a.NB;
+  per_image = per_image < 1 ? 1 : (per_image > a.OH ? a.OH : per_image);
+  const int rows = (a.OH + per_image - 1) / per_image;
+  per_image = (a.OH + rows - 1) / rows;
+  static DynamicLdsLimit limit;
+  if (hipError_t e = limit.ensure((const void*)conv_blocks4x4_kernel, lds); e != hipSuccess) return e;
+  hipLaunchKernelGGL(conv_blocks4x4_kernel, dim3((unsigned)(a.NB * per_image)), dim3(256), lds, s, a, rows, per_image);
+  return hipGetLastError();
+}
 
 size_t conv_halo_prepare(int kind, IgemmArgs* a) {
   const int es = kind == KIND_BF16 ? 2 : (kind == KIND_I8 ? 1 : 4);

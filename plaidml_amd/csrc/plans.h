@@ -135,7 +135,11 @@ inline void tile_of(const TileOrder& o, unsigned bid, int* tm, int* tn) {
 
 struct IgemmArgs {
   TileOrder order;  // filled in by the launcher for the tile grid of the configuration it launches
-  int b_kn;         // 1: Bt / ldbt are the caller's row-major B[K][N] and its row length (fp32 GEMMs only)
+  int b_kn;         // 1: Bt / ldbt are the caller's row-major B[K][N] and its row length (fp32 and int8 GEMMs)
+  // conv_blocks4x4_kernel only: the caller's NHWC image of 3 bf16 channels (raw_h x raw_w pixels, raw_w even), from
+  // which the kernel builds the rows of 2x2 pixel blocks itself; null: A already holds the re-blocked image
+  const void* raw_in;
+  int raw_h, raw_w;
   int64_t M, N, K;
   const void* A;
   int64_t lda;
@@ -187,6 +191,10 @@ hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStr
 // shape does not qualify; `a.halo_rows` and `a.n_tiles` are filled in by conv_halo_prepare.
 size_t conv_halo_prepare(int kind, IgemmArgs* a);
 hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s);
+// The re-blocked few-channel convolution with 4x4 block taps of 16 channels and 64 output channels: LDS bytes of the
+// row-walking kernel, or 0 when `a` (already pointing at the re-blocked input) does not qualify.
+size_t conv_blocks4x4_prepare(int kind, const IgemmArgs& a);
+hipError_t conv_blocks4x4_launch(const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s);
 hipError_t mfma_probe_launch(int blocks, int iters, int random, float* sink, unsigned long long* clk, hipStream_t s);
 // splits a packed fp32 Bt[rows][ld] in place (k values per row, a multiple of 32) into the heads / remainders form
 hipError_t split_rows_launch(void* bt, int64_t rows, int64_t ld, int64_t k, hipStream_t s);

@@ -869,9 +869,14 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   p->text = buf;
   if (kind == KIND_F32X3) p->text += " mfma=3 x f32_32x32x16_bf16 (fp32 split into bf16 head + remainder)";
   if (via_patches) p->text += " via patch matrix (k padded to " + std::to_string(p->kpad) + ")";
-  if (via_s2d)
+  if (via_s2d) {
     p->text += " over 2x2 pixel blocks (" + std::to_string(p->s2d_ka) + "x" + std::to_string(p->s2d_kaw) + " block taps of " +
                std::to_string(p->s2d_ch) + " channels, k=" + std::to_string(p->bt_ld) + ")";
+    IgemmArgs g;
+    conv_args(p, g);
+    const char* e = std::getenv("PML_HIP_CONV");
+    if (!(e && std::string(e) == "igemm") && conv_blocks4x4_prepare(kind, g)) p->text += ", row by row with the filter in registers";
+  }
   return (int64_t)(intptr_t)p;
 }
 
@@ -932,12 +937,25 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     return check(igemm_launch(p->mfma_kind, p->tile, false, g, (hipStream_t)s), "igemm_launch");
   }
   if (p->s2d) {
-    S2dArgs sa;
-    s2d_args(p, sa);
-    sa.in = input;
-    sa.out = p->s2d;
-    if (check(s2d_input_launch(es, sa, (hipStream_t)s), "s2d_input_launch")) return 1;
     g.A = p->s2d;
+    // 4x4 block taps onto 64 channels (the 7x7x3 stride-2 head of an image network): the kernel that walks down
+    // the rows with the filter in registers (PML_HIP_CONV=igemm keeps the implicit GEMM).  From a 3-channel bf16
+    // image of even width it builds the 2x2 pixel blocks itself, row by row, and the re-blocking launch is skipped.
+    const char* e = std::getenv("PML_HIP_CONV");
+    const size_t lds = (e && std::string(e) == "igemm") ? 0 : conv_blocks4x4_prepare(p->mfma_kind, g);
+    const bool from_image = lds && d.ci == 3 && d.w % 2 == 0 && ((uintptr_t)input & 3) == 0 && !(e && std::string(e) == "blocks");
+    if (!from_image) {
+      S2dArgs sa;
+      s2d_args(p, sa);
+      sa.in = input;
+      sa.out = p->s2d;
+      if (check(s2d_input_launch(es, sa, (hipStream_t)s), "s2d_input_launch")) return 1;
+    } else {
+      g.raw_in = input;
+      g.raw_h = (int)d.h;
+      g.raw_w = (int)d.w;
+    }
+    if (lds) return check(conv_blocks4x4_launch(g, lds, device_cus(), (hipStream_t)s), "conv_blocks4x4_launch");
     return check(igemm_launch(p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
   }
   if (p->halo_lds)

@@ -624,7 +624,10 @@ def _stem_case(kind, shape, k, co, stride, pad, seed):
 # stride 2 over channels that do not fill 16-byte vectors: unit-stride convolution over 2x2 pixel blocks.
 # (shape, k, co, pad): even and odd padding, odd image sides, 1- and 5-channel images, a 3x3 and a 2x2 filter
 STEM_CASES = [((2, 30, 34, 3), 7, 64, None), ((2, 32, 32, 3), 7, 64, 3), ((2, 31, 29, 3), 7, 64, 3),
-              ((3, 17, 23, 1), 3, 32, 1), ((1, 20, 18, 5), 5, 48, 0), ((2, 16, 16, 3), 2, 64, 0)]
+              ((3, 17, 23, 1), 3, 32, 1), ((1, 20, 18, 5), 5, 48, 0), ((2, 16, 16, 3), 2, 64, 0),
+              # many images (a workgroup of the row-walking bf16 kernel takes several output rows, the last run ragged)
+              # and a wide one (four 32-pixel blocks per row, the last ragged)
+              ((40, 30, 34, 3), 7, 64, None), ((1, 64, 200, 3), 7, 64, 3)]
 
 
 @pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
