@@ -627,7 +627,10 @@ STEM_CASES = [((2, 30, 34, 3), 7, 64, None), ((2, 32, 32, 3), 7, 64, 3), ((2, 31
               ((3, 17, 23, 1), 3, 32, 1), ((1, 20, 18, 5), 5, 48, 0), ((2, 16, 16, 3), 2, 64, 0),
               # many images (a workgroup of the row-walking bf16 kernel takes several output rows, the last run ragged)
               # and a wide one (four 32-pixel blocks per row, the last ragged)
-              ((40, 30, 34, 3), 7, 64, None), ((1, 64, 200, 3), 7, 64, 3)]
+              ((40, 30, 34, 3), 7, 64, None), ((1, 64, 200, 3), 7, 64, 3),
+              # an odd height with an even width: the kernel builds the pixel blocks itself and the last block row
+              # has no second image row
+              ((2, 31, 30, 3), 7, 64, 3), ((1, 9, 8, 3), 7, 64, None)]
 
 
 @pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
