@@ -82,12 +82,34 @@ def time_loop(hk, fn, steps, warmup, settle_ms=SETTLE_MS):
     return ms / steps, wall / steps
 
 
+def fp32_fraction(tflops, flags):
+    """fp32 work against the pipe it runs on: fp32 MFMAs against their own peak; as three bf16 products per term against
+    a third of the bf16 peak (that pipe does three multiplications per useful one)."""
+    if flags:
+        return {'frac_of_bf16_peak_over_3': round(tflops / (PEAK['bf16'] / 3), 4), 'peak_TFLOP/s': round(PEAK['bf16'] / 3, 1)}
+    return {'frac_mfma_f32': round(tflops / PEAK['f32'], 4)}
+
+
 def valid_taps(size, k, pad):
     return sum(1 for x in range(size) for t in range(k) if 0 <= x + t - pad < size)
 
 
+def cpu_model():
+    try:
+        for line in open('/proc/cpuinfo'):
+            if line.startswith('model name'):
+                return line.split(':', 1)[1].strip()
+    except OSError:
+        pass
+    return 'unknown'
+
+
 def cpu_baseline_conv(N_sample, H, W, CI, CO, seed_i, seed_f, flops_per_image):
-    """The only leg that touches oracle/: the OpenMP restatement, timed on a bounded sample."""
+    """The only leg that touches oracle/: the OpenMP restatement, timed on a bounded sample (threads pinned to cores,
+    median of the timed runs)."""
+    # the OpenMP runtime reads its placement when the library is loaded
+    os.environ.setdefault('OMP_PROC_BIND', 'close')
+    os.environ.setdefault('OMP_PLACES', 'cores')
     from oracle import tile_oracle as E  # checker (test infrastructure), never the thing measured
     lib = ctypes.CDLL(os.path.join(ROOT, 'oracle', 'libcpu_baseline.so'))
     lib.cpu_baseline_threads.restype = ctypes.c_int
@@ -104,18 +126,32 @@ def cpu_baseline_conv(N_sample, H, W, CI, CO, seed_i, seed_f, flops_per_image):
                                 out.ctypes.data_as(fp), N_sample, H, W, CI, 3, 3, CO, H, W, 1, 1, 1)
 
     run()  # warm-up
-    reps, total = 0, 0.0
-    while total < 10.0 and reps < 50:
+    times, total = [], 0.0
+    while (total < 10.0 and len(times) < 50) or len(times) < 5:
         t0 = time.perf_counter()
         run()
-        total += time.perf_counter() - t0
-        reps += 1
-    sec = total / reps
+        times.append(time.perf_counter() - t0)
+        total += times[-1]
+    sec = float(np.median(times))
     return {
         'value': round(flops_per_image * N_sample / sec / 1e12, 5), 'unit': 'TFLOP/s', 'cores': threads, 'kind': 'port',
-        'sample': '%d of 128 images of the same conv (fp32 arithmetic on bf16-valued inputs), %d runs, OMP_NUM_THREADS=%s'
-                  % (N_sample, reps, os.environ.get('OMP_NUM_THREADS', 'unset')),
+        'sample': '%d of 128 images of the same conv (fp32 arithmetic on bf16-valued inputs), median of %d runs (fastest %.1f ms, '
+                  'slowest %.1f ms), OMP_NUM_THREADS=%s OMP_PROC_BIND=%s OMP_PLACES=%s'
+                  % (N_sample, len(times), min(times) * 1e3, max(times) * 1e3, os.environ.get('OMP_NUM_THREADS', 'unset'),
+                     os.environ.get('OMP_PROC_BIND'), os.environ.get('OMP_PLACES')),
+        'cpu': cpu_model(),
     }, E.round_bf16(out), Iv, Fv
+
+
+def staged_runs(runner, staged, P, runs, settle_ms):
+    """Runs a staged program back to back -- at least `runs` times and until `settle_ms` have passed -- and returns the
+    statistics of the run whose device time is the median of those after the first, with the fastest beside it."""
+    stats, began = [], time.perf_counter()
+    while len(stats) < runs + 1 or (time.perf_counter() - began) * 1e3 < settle_ms:
+        runner.run_staged(staged)
+        stats.append(P.last_run_stats())
+    timed = sorted(stats[1:], key=lambda t: t['kernel_ms'])
+    return dict(timed[len(timed) // 2], kernel_ms_min=timed[0]['kernel_ms'], runs=len(timed))
 
 
 def copy_calibration(hk, steps):
@@ -151,15 +187,13 @@ def int8_program_leg(n=4096, runs=5):
     runner.run([a, b, sc])  # one whole run for the transfer times
     first = P.last_run_stats()
     staged = runner.stage([a, b, sc])  # then back to back on staged inputs (B is still transposed in every run)
-    best, k, began = None, 0, time.perf_counter()
-    while k < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
-        runner.run_staged(staged)
-        st = P.last_run_stats()
-        best, k = (st if best is None or st['kernel_ms'] < best['kernel_ms'] else best), k + 1
+    mid = staged_runs(runner, staged, P, runs, SETTLE_MS)
     ops = 2.0 * n ** 3
-    return {'kernel_ms': round(best['kernel_ms'], 4), 'launches': int(best['launches']), 'TOP/s': round(ops / best['kernel_ms'] / 1e9, 1),
-            'frac_mfma_i8': round(ops / best['kernel_ms'] / 1e9 / PEAK['i8'], 4), 'h2d_ms': round(first['h2d_ms'], 3),
-            'd2h_ms': round(first['d2h_ms'], 3)}
+    plan = [l.strip() for l in dict(runner.program.passes)['hip-plan'].splitlines()[1:]]
+    return {'kernel_ms': round(mid['kernel_ms'], 4), 'kernel_ms_min': round(mid['kernel_ms_min'], 4), 'runs': mid['runs'],
+            'launches': int(mid['launches']), 'TOP/s': round(ops / mid['kernel_ms'] / 1e9, 1),
+            'frac_mfma_i8': round(ops / mid['kernel_ms'] / 1e9 / PEAK['i8'], 4), 'h2d_ms': round(first['h2d_ms'], 3),
+            'd2h_ms': round(first['d2h_ms'], 3), 'b_layout': '[K][N] as the config states it (program input, re-laid per run)', 'plan': plan}
 
 
 def xception_leg(hk, L, none, N=64, H=19, W=19, C=728):  # noqa: C901
@@ -239,13 +273,10 @@ def xception_program_leg(N, H, W, C, runs=5):
     prog = P.Program('xception_block', [I], [M, AM])
     runner = P.Runner(prog, target='hip')
     staged = runner.stage([image])
-    best, n, began = None, 0, time.perf_counter()
-    while n < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
-        runner.run_staged(staged)
-        st = P.last_run_stats()
-        best, n = (st if best is None or st['kernel_ms'] < best['kernel_ms'] else best), n + 1
+    mid = staged_runs(runner, staged, P, runs, SETTLE_MS)
     plan = [l.strip() for l in dict(prog.passes)['hip-plan'].splitlines()[1:]]
-    return {'kernel_ms': round(best['kernel_ms'], 4), 'launches': int(best['launches']), 'plan': plan}
+    return {'kernel_ms': round(mid['kernel_ms'], 4), 'kernel_ms_min': round(mid['kernel_ms_min'], 4), 'runs': mid['runs'],
+            'launches': int(mid['launches']), 'plan': plan}
 
 
 def resnet50_leg(batch=128, runs=5):
@@ -261,13 +292,11 @@ def resnet50_leg(batch=128, runs=5):
     # the timed runs follow one another without the 77 MB upload between them (during which the device idles and
     # its clock falls back): the input is staged once
     staged = runner.stage([x])
-    times, began = [], time.perf_counter()
-    while len(times) < runs or (time.perf_counter() - began) * 1e3 < 2 * SETTLE_MS:
-        runner.run_staged(staged)
-        times.append(P.last_run_stats())
-    best = min(times[1:], key=lambda t: t['kernel_ms'])
+    best = staged_runs(runner, staged, P, runs, 2 * SETTLE_MS)   # the median run
     best = dict(best, h2d_ms=first['h2d_ms'], d2h_ms=first['d2h_ms'])
     return {'img_per_s': round(batch / (best['kernel_ms'] * 1e-3), 1), 'kernel_ms': round(best['kernel_ms'], 3),
+            'kernel_ms_min': round(best['kernel_ms_min'], 3), 'img_per_s_fastest_run': round(batch / (best['kernel_ms_min'] * 1e-3), 1),
+            'runs': best['runs'],
             'h2d_ms': round(best['h2d_ms'], 3), 'd2h_ms': round(best['d2h_ms'], 3), 'launches': int(best['launches']),
             'device_MB': round(best['device_bytes'] / 1e6, 1), 'arena_MB': round(best['arena_bytes'] / 1e6, 1),
             'temporaries_unshared_MB': round(best['unshared_temp_bytes'] / 1e6, 1),
@@ -287,8 +316,10 @@ def committed_traffic():
     return None
 
 
-def gemm_leg(hk, kind, n=4096):
-    """A square GEMM on the data its config names: int8 uniform in [-127, 127], bf16 N(0,1); B given as [N][K]."""
+def gemm_leg(hk, kind, n=4096, b_nk=True):
+    """A square GEMM on the data its config names: int8 uniform in [-127, 127], bf16 N(0,1).  b_nk: B is handed over as
+    [N][K] (K contiguous, what the matrix instructions read); otherwise as the row-major [K][N] the configs describe,
+    which every run first re-lays (or reads through transposing LDS reads, where the library finds that cheaper)."""
     from plaidml_amd import edsl as P
     L, none = hk.lib(), hk.ptr_array([])
     g = hk.GemmDesc()
@@ -302,12 +333,13 @@ def gemm_leg(hk, kind, n=4096):
         a, b = (P.to_bf16_bits(rng.standard_normal((n, n)).astype(np.float32)) for _ in range(2))
         out_bytes, peak, unit = 2, PEAK['bf16'], 'TFLOP/s'
     g.m = g.n = g.k = g.lda = g.ldb = g.ldc = n
-    g.b_layout = 1
+    g.b_layout = 1 if b_nk else 0
     plan = L.pml_hip_gemm_dispatch(ctypes.byref(g))
     dA, dB, dC = hk.DeviceBuffer.from_numpy(a), hk.DeviceBuffer.from_numpy(b), hk.DeviceBuffer(n * n * out_bytes)
     ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, None, none, none, None)), 20, 5)
     res = {'ms': round(ms, 4), unit: round(2.0 * n ** 3 / ms / 1e9, 2), 'frac_mfma': round(2.0 * n ** 3 / ms / 1e9 / peak, 4),
-           'plan': hk.describe(plan), 'data': 'uniform int8 [-127, 127]' if kind == 'i8' else 'N(0,1) bf16'}
+           'plan': hk.describe(plan), 'data': 'uniform int8 [-127, 127]' if kind == 'i8' else 'N(0,1) bf16',
+           'b_layout': '[N][K], K contiguous (pre-transposed by the caller)' if b_nk else '[K][N] row-major as the config states it (re-laid by every run)'}
     for buf in (dA, dB, dC):
         buf.free()
     L.pml_hip_plan_free(plan)
@@ -337,15 +369,12 @@ def conv_through_exec(N, H, W, CI, CO, Iv, Fv, runs=6):
     for _ in range(runs):  # whole runs: upload, launch, download (the launch finds an idle device)
         runner.run([Iv, Fv, bias])
         times.append(P.last_run_stats())
-    cold = min(times[1:], key=lambda t: t['kernel_ms'])
+    cold = sorted(times[1:], key=lambda t: t['kernel_ms'])[(len(times) - 1) // 2]
     staged = runner.stage([Iv, Fv, bias])  # and back to back on staged inputs, as a stream of batches arrives
-    warm, n, began = None, 0, time.perf_counter()
-    while n < runs or (time.perf_counter() - began) * 1e3 < SETTLE_MS:
-        runner.run_staged(staged)
-        st = P.last_run_stats()
-        warm, n = (st if warm is None or st['kernel_ms'] < warm['kernel_ms'] else warm), n + 1
+    warm = staged_runs(runner, staged, P, runs, SETTLE_MS)
     plan = [v for k, v in prog.passes if k == 'hip-plan']
-    return {'kernel_ms': round(warm['kernel_ms'], 5), 'kernel_ms_after_an_upload': round(cold['kernel_ms'], 5),
+    return {'kernel_ms': round(warm['kernel_ms'], 5), 'kernel_ms_min': round(warm['kernel_ms_min'], 5), 'runs': warm['runs'],
+            'kernel_ms_after_an_upload': round(cold['kernel_ms'], 5),
             'launches': int(warm['launches']), 'h2d_ms': round(cold['h2d_ms'], 3), 'd2h_ms': round(cold['d2h_ms'], 3),
             'plan': plan[0].splitlines()[1].strip() if plan else ''}
 
@@ -429,6 +458,14 @@ def main():
                      'hbm_frac': round(bytes_alg / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }
 
+    # what the matrix cores of this device sustain on random bf16 operands that never leave LDS (the clock the chip holds
+    # under real data): the same achieved figure against that ceiling, beside the fraction of the published peak
+    probe = mfma_ceiling_leg(hk)
+    sustained = probe['random_operands']['TFLOP/s']
+    result['roofline']['frac_of_sustained'] = round(result['roofline']['achieved'] / sustained, 4)
+    result['roofline']['sustained_peak'] = {'TFLOP/s': sustained, 'core_clock_MHz': probe['random_operands']['core_clock_MHz'],
+                                            'what': 'pml_hip_probe_mfma, random bf16 operands resident in LDS'}
+
     # spot check of the timed output against the CPU baseline on the sampled images
     if not args.no_cpu:
         n_s = 4
@@ -465,8 +502,8 @@ def main():
                 p32 = conv_plan(hk, hk.F32, N, H, W, CI, CO, 3, 3, flags=flags)
                 ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_conv2d_invoke(p32, dI32.ptr, dF32.ptr, dO32.ptr, dB32.ptr, none, none, None)),
                                   max(5, args.steps // 5), 3)
-                extra[name] = {'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2),
-                               'frac_mfma_f32': round(flops / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(p32)}
+                extra[name] = dict({'ms': round(ms, 4), 'TFLOP/s': round(flops / ms / 1e9, 2)}, **fp32_fraction(flops / ms / 1e9, flags),
+                                   plan=hk.describe(p32))
                 L.pml_hip_plan_free(p32)
             for b in (dI32, dF32, dB32, dO32):
                 b.free()
@@ -481,17 +518,19 @@ def main():
                 g.flags = flags
                 pg = L.pml_hip_gemm_dispatch(ctypes.byref(g))
                 ms, _ = time_loop(hk, lambda: hk.check(L.pml_hip_gemm_invoke(pg, dA.ptr, dBm.ptr, dC.ptr, None, none, none, None)), 50, 10)
-                extra[name] = {'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2),
-                               'frac_mfma_f32': round(2 * 1024 ** 3 / ms / 1e9 / PEAK['f32'], 4), 'plan': hk.describe(pg)}
+                extra[name] = dict({'ms': round(ms, 4), 'TFLOP/s': round(2 * 1024 ** 3 / ms / 1e9, 2)},
+                                   **fp32_fraction(2 * 1024 ** 3 / ms / 1e9, flags), plan=hk.describe(pg))
                 L.pml_hip_plan_free(pg)
             for b in (dA, dBm, dC):
                 b.free()
         if want('gemm_i8'):
-            extra['gemm_i8_4096_configs2'] = gemm_leg(hk, 'i8')
+            extra['gemm_i8_4096_b_as_nk'] = gemm_leg(hk, 'i8')
+            extra['gemm_i8_4096_configs2_b_as_kn'] = gemm_leg(hk, 'i8', b_nk=False)
         if want('gemm_bf16'):
-            extra['gemm_bf16_4096'] = gemm_leg(hk, 'bf16')
+            extra['gemm_bf16_4096_b_as_nk'] = gemm_leg(hk, 'bf16')
+            extra['gemm_bf16_4096_b_as_kn'] = gemm_leg(hk, 'bf16', b_nk=False)
         if want('mfma_ceiling'):
-            extra['mfma_ceiling_bf16'] = mfma_ceiling_leg(hk)
+            extra['mfma_ceiling_bf16'] = probe
         if want('int8_program'):
             # configs[2] as a Tile program through the plaidml API: cast -> contraction (si32, first output) with the
             # fused per-column requantisation tail (si8, second output); B is a program input, so it is re-laid per run

@@ -160,6 +160,43 @@ enum {
 /* descriptor flag of gemm and conv2d (in_dtype F32 only): multiply fp32 operands as three bf16 products */
 #define PML_HIP_FP32_AS_BF16X3 1
 
+/* Schedule overrides, carried in `flags` of the gemm and conv2d descriptors beside the flag above (all zero: the
+ * library's own choice per shape class).  They play the part of the per-contraction schedule the reference loads from
+ * PLAIDML_SCHEDULE_PATH (pmlc/target/x86/pipeline.cc:267-272): a planner or a tuning run names the tiling of one
+ * contraction without touching any process-wide state.
+ *   bits 8..15  PML_HIP_FLAG_TILE(t): the output tile of the MFMA kernel, t one of PML_HIP_TILE_*
+ *   bits 16..19 PML_HIP_FLAG_CONV(c): the convolution path, c one of PML_HIP_CONV_* (ignored by gemm)
+ * A tile the element kind is not built for falls back to the nearest one that is; a convolution path the shape
+ * does not qualify for is ignored. */
+enum {
+  PML_HIP_TILE_64x64 = 0,      /* 4 wavefronts */
+  PML_HIP_TILE_128x64,         /* 4 wavefronts of 64x32 */
+  PML_HIP_TILE_128x128,        /* 4 wavefronts */
+  PML_HIP_TILE_128x64_W8,      /* 8 wavefronts */
+  PML_HIP_TILE_128x128_W8,     /* 8 wavefronts, three ring stages */
+  PML_HIP_TILE_256x128_W16,    /* 16 wavefronts */
+  PML_HIP_TILE_128x128_W8_S2,  /* 8 wavefronts, two ring stages (two workgroups per CU) */
+  PML_HIP_TILE_64x64_W8_K2,    /* 8 wavefronts as two grids that split every slab's K-blocks */
+  PML_HIP_TILE_256x256_W8,     /* 8 wavefronts of 128x64 */
+  PML_HIP_TILE_128x64_N2,      /* 4 wavefronts of 32x64 (split fp32 kind only) */
+  PML_HIP_TILE_COUNT_
+};
+enum {
+  PML_HIP_CONV_AUTO = 0,
+  PML_HIP_CONV_IGEMM = 1,     /* implicit GEMM, never a resident-filter or row-walking kernel */
+  PML_HIP_CONV_PATCHES = 2,   /* few-channel inputs through a patch matrix even where 2x2 pixel blocks would do */
+  PML_HIP_CONV_LDSFILTER = 3, /* resident filter kept in LDS rather than in registers */
+  PML_HIP_CONV_BLOCKS = 4     /* the row-walking stem kernel behind a separate re-blocking launch */
+};
+#define PML_HIP_FLAG_TILE(t) ((((t) + 1) & 0xff) << 8)
+#define PML_HIP_FLAG_CONV(c) (((c) & 0xf) << 16)
+#define PML_HIP_FLAG_TILE_OF(flags) ((((flags) >> 8) & 0xff) - 1) /* -1: none */
+#define PML_HIP_FLAG_CONV_OF(flags) (((flags) >> 16) & 0xf)
+/* Name of a tile as the plan dump and the `hip{tile=...}` target option spell it ("128x128w8s2"), NULL when out of range;
+ * and the inverse (-1 for an unknown name).  Host arithmetic only. */
+const char* pml_hip_tile_name(int tile);
+int pml_hip_tile_by_name(const char* name);
+
 typedef struct {
   int32_t opcode;
   int32_t dtype;        /* result element type of this step */
@@ -222,7 +259,7 @@ typedef struct {
   int32_t a2_stride;
   int32_t init2_kind;
   int64_t a2_h, a2_w, a2_oh, a2_ow;
-  int32_t flags; /* PML_HIP_FP32_AS_BF16X3 or 0 */
+  int32_t flags; /* PML_HIP_FP32_AS_BF16X3, PML_HIP_FLAG_TILE(t), or 0 */
   int32_t reserved;
 } pml_hip_gemm_desc;
 
@@ -263,8 +300,9 @@ int pml_hip_tile_of_workgroup(int tiles_m, int tiles_n, int workgroup, int* tile
  * hipMalloc).  The transposed copy of a [K][N] right-hand side (b_layout 0), which a plan keeps in memory of its
  * own, lives in a fixed array in the library's device image instead: n * k * element size must not exceed
  * PML_HIP_STATIC_SCRATCH_BYTES, larger right-hand sides are rejected with an error text that says so
- * (b_layout 1 needs no copy and has no such limit; an fp32 right-hand side that the kernels read where it lies --
- * n and ldb multiples of four, 16-byte aligned -- leaves the array untouched, the limit applies all the same).
+ * (b_layout 1 needs no copy and has no such limit; a right-hand side that the kernels read where it lies leaves the
+ * array untouched -- fp32 with n and ldb multiples of four and 16-byte aligned, int8 with rows of whole 16-byte
+ * vectors on problems where transposing reads cost less than the copy -- and the limit applies all the same).
  * Each GPU holds one such array for the life of the process and
  * every call on that GPU uses it: calls that overlap on one GPU (two streams, two threads) race on it.  The
  * result equals pml_hip_gemm_dispatch + pml_hip_gemm_invoke bit for bit (same tile choice, same kernels). */
@@ -293,7 +331,7 @@ typedef struct {
   int32_t init_dtype;
   int64_t init_row_stride, init_col_stride;
   int32_t c_dtype;
-  int32_t flags; /* PML_HIP_FP32_AS_BF16X3 or 0 (see the GEMM descriptor) */
+  int32_t flags; /* PML_HIP_FP32_AS_BF16X3, PML_HIP_FLAG_TILE(t), PML_HIP_FLAG_CONV(c), or 0 */
   pml_hip_epilogue tail;
 } pml_hip_conv2d_desc;
 

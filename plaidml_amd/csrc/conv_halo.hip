@@ -416,9 +416,7 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
 #define PML_LDS(p) ((__attribute__((address_space(3))) void*)(p))
-#ifndef PML_CONV_AHEAD
-#define PML_CONV_AHEAD 2
-#endif
+constexpr int kConvAhead = 2;                 // K-blocks (pairs of them in the register-filter kernel) operand fragments are fetched ahead
 constexpr int kFar = 0x40000000;              // beyond any input this kernel accepts (<= 2^30 bytes); two of them still are
 
 template <int KIND, int NCH>
@@ -625,7 +623,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
     // operand fragments are fetched kAhead K-blocks ahead (kAhead + 1 register sets)
-    constexpr int kAhead = PML_CONV_AHEAD;
+    constexpr int kAhead = kConvAhead;
     i32x4_t fa[kAhead + 1][MI], fb[kAhead + 1][NI];
     auto frag_offsets = [&](int s1, int& ao, int& bo) {
       const int tap = s1 >> 2, ks = s1 & 3;
@@ -839,8 +837,20 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
                                              0);
   };
 
+  // b_raw == 2: the filter was packed once into the order this kernel keeps it in registers (regfilter_image_kernel
+  // below): fragment (channel block cb, K-block s) of lane l is the 16 bytes at ((cb * 36 + s) * 64 + l) * 16, so every
+  // request of a wavefront is 1 KB of consecutive bytes and nothing passes through LDS or is turned in registers.
+  const bool image = p.b_raw == 2;
+  i32x4_t breg[kBlocks][NI];
+  if (image) {
+    const i32x4_t* img = (const i32x4_t*)p.Bt + lane;
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int s = 0; s < kBlocks; ++s) breg[s][j] = img[((cb0 + j) * kBlocks + s) * 64];
+  }
   FilterStager<KIND, kNT> filter;
-  filter.load(p, tid);
+  if (!image) filter.load(p, tid);
   int t = first_tile(blockIdx.x, gridDim.x);
   TileGeom g = tile_geom(p, t, Hv);
   unsigned char* const win0 = smem;
@@ -859,7 +869,7 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
   auto filter_row = [&](int row) {
     return smem + (row < rows_low ? row * kRegBrow : 2 * win_bytes + (row - rows_low) * kRegBrow);
   };
-  filter.store(p, tid, filter_row);
+  if (!image) filter.store(p, tid, filter_row);
   if (tid < kBN) {
     accs_t b = 0;
     if (p.init != nullptr) {
@@ -872,13 +882,14 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
   // MFMA row 8q + 4h + e of channel block cb is given output channel 32cb + 16h + 4q + e, so that
   // a lane (pixel, h) ends up owning the 16 consecutive channels 32cb + 16h .. + 15 in register order;
   // the staged filter keeps that channel in row 32h + 8q + 4cb + e
-  i32x4_t breg[kBlocks][NI];
+  if (!image) {
 #pragma unroll
-  for (int j = 0; j < NI; ++j) {
-    const int row = lane & 31;
-    const unsigned char* src = filter_row(((row >> 2) & 1) * 32 + (row >> 3) * 8 + 4 * (cb0 + j) + (row & 3)) + half * 16;
+    for (int j = 0; j < NI; ++j) {
+      const int row = lane & 31;
+      const unsigned char* src = filter_row(((row >> 2) & 1) * 32 + (row >> 3) * 8 + 4 * (cb0 + j) + (row & 3)) + half * 16;
 #pragma unroll
-    for (int s = 0; s < kBlocks; ++s) breg[s][j] = *(const i32x4_t*)(src + s * 32);
+      for (int s = 0; s < kBlocks; ++s) breg[s][j] = *(const i32x4_t*)(src + s * 32);
+    }
   }
   const int co0 = 32 * cb0 + 16 * half;  // first of the lane's 16 output channels in its first block
   const unsigned char* const bias_src = smem + bias_off + co0 * 4;
@@ -960,7 +971,7 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
         for (int e = 0; e < 4; ++e) acc[j][4 * q + e] = v[e];
       }
     // Operand fragments are fetched kAhead K-blocks ahead.
-    constexpr int kAhead = 2 * PML_CONV_AHEAD;
+    constexpr int kAhead = 2 * kConvAhead;
     i32x4_t fa[kAhead + 1];
     // K-blocks run filter column by filter column (kw outermost): the four permuted vector offsets of
     // a column serve its three taps, which differ by a uniform row offset only
@@ -1064,6 +1075,19 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
   } else {
     flush(accY, m_last);
   }
+}
+
+// The packed filter Bt[64][9 * 128 bytes] in the order conv_regfilter3x3_kernel holds it in registers: for channel
+// block cb (32 channels), K-block s (32 bytes of a row) and lane l, the 16 bytes l >> 5 of that K-block in the row of
+// channel 32 cb + 16 ((l >> 2) & 1) + 4 ((l & 31) >> 3) + (l & 3) -- the channel MFMA row l & 31 is given.
+__global__ __launch_bounds__(256) void regfilter_image_kernel(const unsigned char* __restrict__ bt, int64_t ldbt_bytes,
+                                                              i32x4_t* __restrict__ image) {
+  const int q = blockIdx.x * 256 + threadIdx.x;  // (cb * 36 + s) * 64 + lane
+  if (q >= 2 * 36 * 64) return;
+  const int lane = q & 63, s = (q >> 6) % 36, cb = q / (64 * 36);
+  const int row = lane & 31;
+  const int co = 32 * cb + 16 * ((row >> 2) & 1) + 4 * (row >> 3) + (row & 3);
+  image[q] = *(const i32x4_t*)(bt + co * ldbt_bytes + s * 32 + (lane >> 5) * 16);
 }
 
 template <int KIND, int WV>
@@ -1289,7 +1313,7 @@ hipError_t conv_blocks4x4_launch(const IgemmArgs& a, size_t lds, int n_cus, hipS
   return hipGetLastError();
 }
 
-size_t conv_halo_prepare(int kind, IgemmArgs* a) {
+size_t conv_halo_prepare(int kind, IgemmArgs* a, bool filter_in_lds) {
   const int es = kind == KIND_BF16 ? 2 : (kind == KIND_I8 ? 1 : 4);
   if (a->SH != 1 || a->SW != 1 || a->DH != 1 || a->DW != 1) return 0;
   if ((int64_t)a->CI * es != kPixBytes) return 0;
@@ -1332,14 +1356,19 @@ size_t conv_halo_prepare(int kind, IgemmArgs* a) {
                         ? nchunks
                         : 0;
   // filter in registers: 16- and 8-bit elements, two windows of at most kRegRows rows of 32 .. 64 pixels in LDS
-  // (PML_HIP_CONV=ldsfilter keeps the filter in LDS)
-  const char* e = std::getenv("PML_HIP_CONV");
+  // (filter_in_lds: the caller's schedule keeps the filter in LDS)
   if (a->halo_variant && kind != KIND_F32 && max_rows <= kRegRows && Wv >= 32 && Wv <= 64 &&
-      reg_lds_bytes(Wv) <= 160 * 1024 && !(e && std::string(e) == "ldsfilter")) {
+      reg_lds_bytes(Wv) <= 160 * 1024 && !filter_in_lds) {
     a->halo_variant = 3;
     return (size_t)reg_lds_bytes(Wv);
   }
   return total;
+}
+
+hipError_t regfilter_image_launch(const void* bt, int64_t ldbt_bytes, void* image, hipStream_t s) {
+  if ((((uintptr_t)bt | (uintptr_t)image) & 15) != 0 || ldbt_bytes % 16 != 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(regfilter_image_kernel, dim3(2 * 36 * 64 / 256), dim3(256), 0, s, (const unsigned char*)bt, ldbt_bytes, (i32x4_t*)image);
+  return hipGetLastError();
 }
 
 hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s) {

@@ -91,7 +91,7 @@ constexpr int igemm_waves_per_simd() {
 // of a group each name 8 bytes -- here 8 columns of one K-row -- and lane i receives byte i % 8 of the data named
 // by lanes i / 8, i / 8 + 2, ..., i.e. 8 K-values of column i).  The 16-byte chunks of K-row k are stored at
 // positions XORed with k % 8 so that the 8 rows of such a read fall into different banks.
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128,
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int SLAB = 128,
           bool BKN = false>
 __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>())) void igemm_kernel(IgemmArgs p_by_value) {
   // The argument block is read where the dispatcher put it (the kernel-argument segment, scalar loads),
@@ -449,23 +449,8 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       const bool last = kb + 1 == kBlocks;
       if (last) {
         // fragments of this K-block are in registers (lgkmcnt 0), slab s + 1 has landed
-#ifdef PML_TRACE
-        const uint64_t t0 = __builtin_amdgcn_s_memtime();
-        __builtin_amdgcn_s_waitcnt(0x0F7F & ~0x0F00);  // lgkmcnt(0) only
-        const uint64_t t1 = __builtin_amdgcn_s_memtime();
-#endif
         __builtin_amdgcn_s_waitcnt(0x0070 | (kOutstanding & 15) | ((kOutstanding >> 4) << 14));
-#ifdef PML_TRACE
-        const uint64_t t2 = __builtin_amdgcn_s_memtime();
-#endif
-        if constexpr (!(ABL & 8)) __builtin_amdgcn_s_barrier();
-#ifdef PML_TRACE
-        if (p.outs[5] && blockIdx.x == 37 && lane == 0 && s < 60) {
-          uint64_t* tr = (uint64_t*)p.outs[5] + (wave * 64 + s) * 4;
-          tr[0] = t0; tr[1] = t1; tr[2] = t2; tr[3] = __builtin_amdgcn_s_memtime();
-          if (wave == 15 || (wave == 7 && NT == 512)) tr[1] = __builtin_amdgcn_s_memrealtime();  // the 100 MHz clock, to calibrate
-        }
-#endif
+        __builtin_amdgcn_s_barrier();
         prepare_slab(stage);
       }
       const unsigned char* ra_ = last ? a_next : a_base;
@@ -484,9 +469,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       }
 #pragma unroll
       for (int m = 0; m < kSlots; ++m) {
-        if constexpr (ABL & 4) {
-          asm volatile("" ::"v"(fb[cur][m % NI]), "v"(fa[cur][m / NI]));
-        } else if constexpr (kSplit) {
+        if constexpr (kSplit) {
           // (Bt's fragment is the row operand, as in mma_block; a packed right-hand side's two reads of the pair are
           // its heads and its remainders)
           if (cur == 1) {
@@ -499,12 +482,12 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
         } else {
           mma_block<KIND>(acc[m / NI][m % NI], fb[cur][m % NI], fa[cur][m / NI]);
         }
-        if (last && !(ABL & 1)) {
+        if (last) {
 #pragma unroll
           for (int l = m; l < kLoads; l += kSlots) issue_load(l);
         }
 #pragma unroll
-        for (int d = m; d < ((ABL & 2) ? 0 : MI + NI); d += kSlots) {
+        for (int d = m; d < MI + NI; d += kSlots) {
           if (d < MI)
             fa[nxt][d] = *(const i32x4_t*)(ra_ + d * 32 * kSlabBytes + fs);
           else
@@ -677,7 +660,7 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
   }
 }
 
-template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int ABL = 0, int SLAB = 128>
+template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   if constexpr ((KIND == KIND_F32 || KIND == KIND_F32X3 || KIND == KIND_I8) && !CONV && SLAB == 128) {
     if (a.b_kn) {
@@ -685,7 +668,7 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
       const int64_t tiles = tiles_m * tiles_n;
       if (tiles <= 0 || tiles >= ((int64_t)1 << 31) || a.K2 > 0) return hipErrorInvalidValue;
       const size_t lds = Ring<BM, BN, STAGES, SLAB>::kAlloc;
-      auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB, true>;
+      auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, SLAB, true>;
       static DynamicLdsLimit limit;
       if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
       IgemmArgs b = a;
@@ -700,7 +683,7 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int64_t tiles = tiles_m * tiles_n;
   if (tiles <= 0 || tiles >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
   const size_t lds = Ring<BM, BN, STAGES, SLAB>::kAlloc;
-  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, ABL, SLAB>;
+  auto kern = igemm_kernel<KIND, BM, BN, WAVES_M, CONV, NT, STAGES, WAVES_K, SLAB>;
   static DynamicLdsLimit limit;
   if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
   IgemmArgs b = a;
@@ -711,10 +694,6 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
 
 template <int KIND, bool CONV>
 hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
-#ifdef PML_DEV_CFG  // development builds: one configuration, given as the template arguments after KIND
-  if constexpr (CONV == PML_DEV_CONV && KIND == PML_KIND) return launch_cfg<KIND, PML_DEV_CFG>(a, s);
-  return hipErrorInvalidValue;
-#else
   switch (cfg) {
     case TILE_64x64: return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);
     case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
@@ -749,7 +728,6 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
       }
   }
   return hipErrorInvalidValue;
-#endif
 }
 
 }  // namespace
@@ -829,12 +807,8 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(int iters, int random, 
 
 // MFMAs (32x32x16 bf16) issued by one launch of `iters` rounds on `blocks` workgroups.
 hipError_t mfma_probe_launch(int blocks, int iters, int random, float* sink, unsigned long long* clk, hipStream_t s) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)mfma_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static DynamicLdsLimit limit;
+  if (hipError_t e = limit.ensure((const void*)mfma_probe_kernel, 128 * 1024); e != hipSuccess) return e;
   hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)blocks), dim3(512), 128 * 1024, s, iters, random, sink, clk);
   return hipGetLastError();
 }

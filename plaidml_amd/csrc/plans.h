@@ -37,7 +37,9 @@ struct DynamicLdsLimit {
 // their 32 bf16 heads, then their 32 bf16 remainders), so that only the left-hand fragments are split in registers
 enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2, KIND_F32X3 = 3, KIND_F32X3P = 4 };
 // _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages; _K2: two wavefront grids share the K-blocks of every slab
-enum { TILE_64x64 = 0, TILE_128x64, TILE_128x128, TILE_128x64_W8, TILE_128x128_W8, TILE_256x128_W16, TILE_128x128_W8_S2, TILE_64x64_W8_K2, TILE_256x256_W8, TILE_128x64_N2 };
+enum { TILE_64x64 = PML_HIP_TILE_64x64, TILE_128x64 = PML_HIP_TILE_128x64, TILE_128x128 = PML_HIP_TILE_128x128, TILE_128x64_W8 = PML_HIP_TILE_128x64_W8,
+       TILE_128x128_W8 = PML_HIP_TILE_128x128_W8, TILE_256x128_W16 = PML_HIP_TILE_256x128_W16, TILE_128x128_W8_S2 = PML_HIP_TILE_128x128_W8_S2,
+       TILE_64x64_W8_K2 = PML_HIP_TILE_64x64_W8_K2, TILE_256x256_W8 = PML_HIP_TILE_256x256_W8, TILE_128x64_N2 = PML_HIP_TILE_128x64_N2 };
 
 struct TailPtrs {
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
@@ -154,7 +156,8 @@ struct IgemmArgs {
   int pix_pitch;
   // resident-filter convolution only: image count, LDS rows of the input window, number of 256-pixel tiles
   // halo_variant: 0 = general resident kernel, 1 / 2 = pipelined 3x3 kernel with that many 32-pixel chunks per row
-  // b_raw: Bt points at the caller's [K][N] matrix instead of the packed [N][K] one (pipelined kernel only)
+  // b_raw: 1 = Bt points at the caller's [K][N] matrix instead of the packed [N][K] one (pipelined kernels only);
+  //        2 = Bt points at the filter in register order (the register-filter kernel only; regfilter_image_launch)
   int NB, halo_rows, n_tiles, halo_variant, b_raw;
   int n_cus;  // compute units of the device (persistent grids)
   // n / (OH*OW) and n / OW as multiply-and-shift (see fast_div); set for every convolution
@@ -189,8 +192,12 @@ struct IgemmArgs {
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 // Resident-filter convolution (conv_halo.hip): LDS bytes a shape needs, or 0 when the
 // shape does not qualify; `a.halo_rows` and `a.n_tiles` are filled in by conv_halo_prepare.
-size_t conv_halo_prepare(int kind, IgemmArgs* a);
+size_t conv_halo_prepare(int kind, IgemmArgs* a, bool filter_in_lds = false);
 hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int n_cus, hipStream_t s);
+// The packed 3x3 filter Bt[64][ldbt] of the register-filter kernel (halo_variant 3) re-laid into the order that kernel
+// keeps it in registers: kRegfilterImageBytes bytes at `image`.
+constexpr size_t kRegfilterImageBytes = 2 * 36 * 64 * 16;
+hipError_t regfilter_image_launch(const void* bt, int64_t ldbt_bytes, void* image, hipStream_t s);
 // The re-blocked few-channel convolution with 4x4 block taps of 16 channels and 64 output channels: LDS bytes of the
 // row-walking kernel, or 0 when `a` (already pointing at the re-blocked input) does not qualify.
 size_t conv_blocks4x4_prepare(int kind, const IgemmArgs& a);

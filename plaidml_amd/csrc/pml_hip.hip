@@ -3,6 +3,7 @@
 // it many times.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -45,7 +46,7 @@ struct Plan {
   size_t bt_bytes = 0;
   bool packed = false;
   bool b_split = false;  // split fp32 kind: a right-hand side packed once is kept as bf16 heads + remainders
-  bool bt_is_split = false;  // ... and `bt` holds that form now
+  std::atomic<bool> bt_is_split{false};  // ... and `bt` holds that form now (invokes that bring their own right-hand side clear it)
   // second product of a GEMM: its packed right-hand side Bt2[N][K2]
   void* bt2 = nullptr;
   bool packed2 = false;
@@ -54,8 +55,13 @@ struct Plan {
   int64_t kpad = 0;
   // stride-2 convolution over few channels, run as a unit-stride one over 2x2 pixel blocks: the
   // re-blocked input [N][s2d_h][s2d_w][s2d_ch]; filter taps s2d_ka x s2d_kaw blocks
+  // (allocated by the first invoke that needs it: the row-walking stem kernel builds its blocks from the image)
+  bool via_s2d = false;
   void* s2d = nullptr;
+  std::mutex s2d_mutex;
   int s2d_h = 0, s2d_w = 0, s2d_ch = 0, s2d_ka = 0, s2d_kaw = 0;
+  // register-filter convolution: a filter packed once, in the order the kernel holds it in registers
+  void* reg_image = nullptr;
   // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
   size_t halo_lds = 0;
   int halo_rows = 0, halo_tiles = 0, halo_variant = 0, n_cus = 0;
@@ -65,6 +71,7 @@ struct Plan {
     if (bt2) (void)hipFree(bt2);
     if (patches) (void)hipFree(patches);
     if (s2d) (void)hipFree(s2d);
+    if (reg_image) (void)hipFree(reg_image);
   }
 };
 
@@ -93,6 +100,12 @@ const char* tile_name(int t) {
   return "?";
 }
 
+constexpr int kScheduleBits = 0xff << 8 | 0xf << 16;
+bool schedule_bits_ok(int flags) {
+  return PML_HIP_FLAG_TILE_OF(flags) < PML_HIP_TILE_COUNT_ && PML_HIP_FLAG_CONV_OF(flags) <= PML_HIP_CONV_BLOCKS;
+}
+const char* const kTileShort[PML_HIP_TILE_COUNT_] = {"64x64", "128x64", "128x128", "128x64w8", "128x128w8", "256x128w16", "128x128w8s2", "64x64w8k2", "256x256w8", "128x64n2"};
+
 // Stated tiling choice per shape class.  Measured on MI355X, bf16 unless said otherwise (us; w8 / w16 =
 // 8 / 16 wavefronts per workgroup; s2 = two ring stages and LDS cut to what the result tile needs, so that two
 // workgroups share a CU; the 4-wavefront 256x128 and 256x256 tiles that were tried as well are slower than
@@ -111,6 +124,7 @@ const char* tile_name(int t) {
 //   gemm 23104x728x728                  72      67       78         65           57          58
 //   gemm 128x1000x2048                  14       -        -         19           19          25
 //   gemm 1024^3 (fp32)                  33      45       77         71            -         127
+// A descriptor may name its tile (PML_HIP_FLAG_TILE); every tile is tested on a ragged problem that way.
 // One tile per workgroup and a serial load / multiply / store life per tile: latency is hidden by the
 // other wavefronts of a SIMD -- 8 or 16 per workgroup instead of 4 -- and, for the bandwidth-bound shapes
 // with a short K, by a second workgroup on the CU whose loads run under the first one's tail.  So: long K
@@ -118,21 +132,9 @@ const char* tile_name(int t) {
 // wavefronts, two to a CU if that still gives every CU a workgroup, one to a CU (three stages) below
 // that; and for small problems the smaller of 64x64 and 128x64 by (rounds of resident workgroups) x
 // (tile area), the larger tile on a tie.
-int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, bool plain_tail = true) {
-  // PML_HIP_TILE=64x64|64x64w8k2|128x64|128x128|128x64w8|128x128w8|128x128w8s2|256x128w16|256x256w8|128x64n2 overrides the table (for tuning runs)
-  if (const char* e = std::getenv("PML_HIP_TILE")) {
-    const std::string v(e);
-    if (v == "64x64") return TILE_64x64;
-    if (v == "128x64") return TILE_128x64;
-    if (v == "128x128") return TILE_128x128;
-    if (v == "128x64w8") return TILE_128x64_W8;
-    if (v == "128x128w8") return TILE_128x128_W8;
-    if (v == "128x128w8s2") return TILE_128x128_W8_S2;
-    if (v == "256x128w16") return TILE_256x128_W16;
-    if (v == "64x64w8k2") return TILE_64x64_W8_K2;
-    if (v == "256x256w8") return TILE_256x256_W8;
-    if (v == "128x64n2" && kind == KIND_F32X3) return TILE_128x64_N2;
-  }
+// forced: a tile named by the descriptor's schedule bits (PML_HIP_FLAG_TILE), -1 = none
+int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, bool plain_tail = true, int forced = -1) {
+  if (forced >= 0 && forced < PML_HIP_TILE_COUNT_ && (forced != TILE_128x64_N2 || kind == KIND_F32X3)) return forced;
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (kind == KIND_F32X3) {
     // A fragment that is split in registers costs 24 vector instructions whatever it is multiplied with, so the
@@ -357,7 +359,7 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.halo_variant = p->halo_variant;
   fast_div_magic((unsigned)(d.oh * d.ow), &g.div_per_magic, &g.div_per_shift);
   fast_div_magic((unsigned)d.ow, &g.div_ow_magic, &g.div_ow_shift);
-  if (p->s2d) {
+  if (p->via_s2d) {
     // unit-stride convolution over the re-blocked input: one "tap" per block row, whose K-run covers
     // s2d_kaw neighbouring blocks of s2d_ch channels
     const int es = dt_size(d.in_dtype);
@@ -388,7 +390,7 @@ void s2d_args(const Plan* p, S2dArgs& a) {
 hipError_t pack_conv_filter(Plan* p, const void* filter, hipStream_t s) {
   const pml_hip_conv2d_desc& d = p->conv;
   const int es = dt_size(d.in_dtype);
-  if (p->s2d) {
+  if (p->via_s2d) {
     S2dArgs a;
     s2d_args(p, a);
     a.filter = filter;
@@ -508,8 +510,9 @@ static int gemm_desc_kind(const pml_hip_gemm_desc* d) {
     fail("gemm: out_dtype does not fit in_dtype");
     return -1;
   }
-  if ((d->flags & ~PML_HIP_FP32_AS_BF16X3) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32)) {
-    fail("gemm: flags may only hold PML_HIP_FP32_AS_BF16X3, and only with in_dtype F32");
+  if ((d->flags & ~(PML_HIP_FP32_AS_BF16X3 | kScheduleBits)) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32) ||
+      !schedule_bits_ok(d->flags)) {
+    fail("gemm: flags may only hold PML_HIP_FP32_AS_BF16X3 (with in_dtype F32) and schedule overrides that name an existing tile");
     return -1;
   }
   if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->lda < d->k || d->ldb < (d->b_layout ? d->k : d->n) || d->ldc < d->n ||
@@ -556,6 +559,7 @@ int pml_hip_gemm_tail_cheaper_apart(const pml_hip_gemm_desc* d) {
   classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
   if (mode == 1 || mode == 2) return 0;
   const int64_t k_bytes = d->k * dt_size(d->in_dtype);
+  if (PML_HIP_FLAG_TILE_OF(d->flags) >= 0) return 0;  // a named tile is taken whatever the tail
   return choose_tile(d->m, d->n, k_bytes, kind, true) == TILE_256x256_W8 && choose_tile(d->m, d->n, k_bytes, kind, false) != TILE_256x256_W8;
 }
 
@@ -570,7 +574,7 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   {
     int mode = 0, relu = 0;
     classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
-    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, mode == 1 || mode == 2);
+    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, mode == 1 || mode == 2, PML_HIP_FLAG_TILE_OF(d->flags));
   }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
@@ -749,7 +753,7 @@ int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const voi
   }
   int mode = 0, relu = 0;
   classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
-  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, mode == 1 || mode == 2);
+  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, mode == 1 || mode == 2, PML_HIP_FLAG_TILE_OF(d->flags));
   return gemm_run(*d, kind, tile, bt, d->k, false, a, b, c, init, operands, outs, s);
 }
 
@@ -773,8 +777,9 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     fail("conv2d: out_dtype does not fit in_dtype");
     return 0;
   }
-  if ((d->flags & ~PML_HIP_FP32_AS_BF16X3) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32)) {
-    fail("conv2d: flags may only hold PML_HIP_FP32_AS_BF16X3, and only with in_dtype F32");
+  if ((d->flags & ~(PML_HIP_FP32_AS_BF16X3 | kScheduleBits)) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32) ||
+      !schedule_bits_ok(d->flags)) {
+    fail("conv2d: flags may only hold PML_HIP_FP32_AS_BF16X3 (with in_dtype F32) and schedule overrides that name an existing tile and path");
     return 0;
   }
   if (d->n <= 0 || d->h <= 0 || d->w <= 0 || d->ci <= 0 || d->co <= 0 || d->kh <= 0 || d->kw <= 0 || d->oh <= 0 ||
@@ -785,9 +790,9 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   const int es = dt_size(d->in_dtype);
   // channels that do not fill 16-byte vectors: stride 2 runs over 2x2 pixel blocks, anything else over a patch matrix
   const bool odd_channels = (d->ci * es) % 16 != 0;
-  const char* conv_env = std::getenv("PML_HIP_CONV");
+  const int path = PML_HIP_FLAG_CONV_OF(d->flags);
   const bool via_s2d = odd_channels && d->stride_h == 2 && d->stride_w == 2 && d->dil_h == 1 && d->dil_w == 1 &&
-                       es >= 2 && d->ci <= 16 && !(conv_env && std::string(conv_env) == "patches");
+                       es >= 2 && d->ci <= 16 && path != PML_HIP_CONV_PATCHES;
   const bool via_patches = odd_channels && !via_s2d;
   if (d->n * d->h * d->w * d->ci >= ((int64_t)1 << 40) || d->h * d->w * d->ci * es >= ((int64_t)1 << 31) ||
       d->kh * d->kw * d->ci * es >= ((int64_t)1 << 31)) {
@@ -804,7 +809,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   p->conv = *d;
   const int64_t M = d->n * d->oh * d->ow;
   const int64_t K = d->kh * d->kw * d->ci;
-  p->tile = choose_tile(M, d->co, K * es, kind, false);
+  p->tile = choose_tile(M, d->co, K * es, kind, false, PML_HIP_FLAG_TILE_OF(d->flags));
   p->bt_ld = K;
   if (via_s2d) {
     const int v = 16 / es;
@@ -814,14 +819,9 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     p->s2d_ka = (int)(d->kh + (d->pad_h & 1) + 1) / 2;
     p->s2d_kaw = (int)(d->kw + (d->pad_w & 1) + 1) / 2;
     const int64_t k2 = (int64_t)p->s2d_ka * p->s2d_kaw * p->s2d_ch;
-    p->tile = choose_tile(M, d->co, k2 * es, kind, false);
+    p->tile = choose_tile(M, d->co, k2 * es, kind, false, PML_HIP_FLAG_TILE_OF(d->flags));
     p->bt_ld = k2;
-    // 256 spare bytes: a K-run that starts left of the image is addressed (never read) below the buffer's end only
-    if (hipMalloc(&p->s2d, (size_t)d->n * p->s2d_h * p->s2d_w * p->s2d_ch * es + 256) != hipSuccess) {
-      delete p;
-      fail("conv2d: cannot allocate the re-blocked input");
-      return 0;
-    }
+    p->via_s2d = true;
   }
   if (via_patches) {
     // rows padded with zeros to whole 16-byte vectors on both GEMM operands
@@ -843,15 +843,14 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     return 0;
   }
   {
-    // Filter small enough to stay in LDS: persistent resident-filter kernel (PML_HIP_CONV=igemm keeps the generic one).
-    const char* e = std::getenv("PML_HIP_CONV");
+    // Filter small enough to stay in LDS: persistent resident-filter kernel (PML_HIP_CONV_IGEMM keeps the generic one).
     int dev = 0;
     hipDeviceProp_t prop;
-    if (!odd_channels && kind != KIND_F32X3 && !(e && std::string(e) == "igemm") && hipGetDevice(&dev) == hipSuccess &&
+    if (!odd_channels && kind != KIND_F32X3 && path != PML_HIP_CONV_IGEMM && hipGetDevice(&dev) == hipSuccess &&
         hipGetDeviceProperties(&prop, dev) == hipSuccess) {
       IgemmArgs g;
       conv_args(p, g);
-      const size_t lds = conv_halo_prepare(kind, &g);
+      const size_t lds = conv_halo_prepare(kind, &g, path == PML_HIP_CONV_LDSFILTER);
       if (lds && lds <= prop.sharedMemPerBlock) {
         p->halo_lds = lds;
         p->halo_rows = g.halo_rows;
@@ -874,8 +873,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
                std::to_string(p->s2d_ch) + " channels, k=" + std::to_string(p->bt_ld) + ")";
     IgemmArgs g;
     conv_args(p, g);
-    const char* e = std::getenv("PML_HIP_CONV");
-    if (!(e && std::string(e) == "igemm") && conv_blocks4x4_prepare(kind, g)) p->text += ", row by row with the filter in registers";
+    if (path != PML_HIP_CONV_IGEMM && conv_blocks4x4_prepare(kind, g)) p->text += ", row by row with the filter in registers";
   }
   return (int64_t)(intptr_t)p;
 }
@@ -887,13 +885,17 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   const pml_hip_conv2d_desc& d = p->conv;
   if (!input || !output) return fail("conv2d_invoke: null operand");
   if (!filter && !p->packed) return fail("conv2d_invoke: filter is null and no packed filter exists");
-  if (!p->patches && !p->s2d && ((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
+  if (!p->patches && !p->via_s2d && ((uintptr_t)input & 15) != 0) return fail("conv2d_invoke: input must be 16-byte aligned");
   if (d.init_kind && !init) return fail("conv2d_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
   const int64_t K = d.kh * d.kw * d.ci;
   // the HWCK filter is a row-major [K][CO] matrix; the pipelined resident-filter kernel transposes it itself
   const bool raw_filter = filter && p->halo_lds && p->halo_variant && p->mfma_kind != KIND_I8;
   if (filter && !raw_filter && check(pack_conv_filter(p, filter, (hipStream_t)s), "pack_conv_filter")) return 1;
+  // (a filter that arrives with the call replaces the packed one; its register-order copy follows it)
+  if (filter && !raw_filter && p->reg_image &&
+      check(regfilter_image_launch(p->bt, p->bt_ld * es, p->reg_image, (hipStream_t)s), "regfilter_image_launch"))
+    return 1;
   IgemmArgs g;
   conv_args(p, g);
   if (raw_filter) {
@@ -901,6 +903,9 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     g.Bt = filter;
     g.ldbt = d.co;
     g.b_raw = 1;
+  } else if (!filter && p->reg_image && p->halo_lds && p->halo_variant == 3) {
+    g.Bt = p->reg_image;
+    g.b_raw = 2;
   }
   g.A = input;
   g.C = output;
@@ -936,15 +941,23 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
     g.K = p->kpad;
     return check(igemm_launch(p->mfma_kind, p->tile, false, g, (hipStream_t)s), "igemm_launch");
   }
-  if (p->s2d) {
-    g.A = p->s2d;
+  if (p->via_s2d) {
     // 4x4 block taps onto 64 channels (the 7x7x3 stride-2 head of an image network): the kernel that walks down
-    // the rows with the filter in registers (PML_HIP_CONV=igemm keeps the implicit GEMM).  From a 3-channel bf16
+    // the rows with the filter in registers (PML_HIP_CONV_IGEMM keeps the implicit GEMM).  From a 3-channel bf16
     // image of even width it builds the 2x2 pixel blocks itself, row by row, and the re-blocking launch is skipped.
-    const char* e = std::getenv("PML_HIP_CONV");
-    const size_t lds = (e && std::string(e) == "igemm") ? 0 : conv_blocks4x4_prepare(p->mfma_kind, g);
-    const bool from_image = lds && d.ci == 3 && d.w % 2 == 0 && ((uintptr_t)input & 3) == 0 && !(e && std::string(e) == "blocks");
+    const int path = PML_HIP_FLAG_CONV_OF(d.flags);
+    const size_t lds = path == PML_HIP_CONV_IGEMM ? 0 : conv_blocks4x4_prepare(p->mfma_kind, g);
+    const bool from_image = lds && d.ci == 3 && d.w % 2 == 0 && ((uintptr_t)input & 3) == 0 && path != PML_HIP_CONV_BLOCKS;
     if (!from_image) {
+      {
+        std::lock_guard<std::mutex> lock(p->s2d_mutex);
+        // 256 spare bytes: a K-run that starts left of the image is addressed (never read) below the buffer's end only
+        if (!p->s2d && hipMalloc(&p->s2d, (size_t)d.n * p->s2d_h * p->s2d_w * p->s2d_ch * es + 256) != hipSuccess) {
+          p->s2d = nullptr;
+          return fail("conv2d_invoke: cannot allocate the re-blocked input");
+        }
+      }
+      g.A = p->s2d;
       S2dArgs sa;
       s2d_args(p, sa);
       sa.in = input;
@@ -1006,6 +1019,14 @@ int pml_hip_probe_mfma(int random_data, int iters, double* tflops, double* core_
   return rc;
 }
 
+const char* pml_hip_tile_name(int tile) { return tile >= 0 && tile < PML_HIP_TILE_COUNT_ ? kTileShort[tile] : nullptr; }
+int pml_hip_tile_by_name(const char* name) {
+  if (!name) return -1;
+  for (int t = 0; t < PML_HIP_TILE_COUNT_; ++t)
+    if (std::strcmp(name, kTileShort[t]) == 0) return t;
+  return -1;
+}
+
 int pml_hip_tile_of_workgroup(int tiles_m, int tiles_n, int workgroup, int* tile_m, int* tile_n) {
   if (tiles_m <= 0 || tiles_n <= 0 || (int64_t)tiles_m * tiles_n >= ((int64_t)1 << 31) || workgroup < 0 ||
       workgroup >= tiles_m * tiles_n || !tile_m || !tile_n)
@@ -1031,6 +1052,11 @@ int pml_hip_conv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream 
   const pml_hip_conv2d_desc& d = p->conv;
   (void)d;
   if (check(pack_conv_filter(p, filter, (hipStream_t)s), "pack_conv_filter")) return 1;
+  if (p->halo_lds && p->halo_variant == 3) {
+    // the register-filter kernel takes a constant filter in its own register order: no trip through LDS per launch
+    if (!p->reg_image && check(hipMalloc(&p->reg_image, kRegfilterImageBytes), "hipMalloc")) return 1;
+    if (check(regfilter_image_launch(p->bt, p->bt_ld * dt_size(d.in_dtype), p->reg_image, (hipStream_t)s), "regfilter_image_launch")) return 1;
+  }
   p->packed = true;
   return 0;
 }

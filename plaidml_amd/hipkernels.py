@@ -15,6 +15,20 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libpml_hip.so')
 # element types (values of plaidml_datatype, bfloat16 appended)
 BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, F32, F64, BF16 = 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16
 FP32_AS_BF16X3 = 1  # descriptor flag of gemm / conv2d: fp32 operands multiplied as three bf16 products
+# schedule overrides in the same `flags` field (PML_HIP_FLAG_TILE / PML_HIP_FLAG_CONV of include/pml_hip.h)
+TILE_NAMES = ('64x64', '128x64', '128x128', '128x64w8', '128x128w8', '256x128w16', '128x128w8s2', '64x64w8k2', '256x256w8', '128x64n2')
+CONV_AUTO, CONV_IGEMM, CONV_PATCHES, CONV_LDSFILTER, CONV_BLOCKS = 0, 1, 2, 3, 4
+
+
+def flag_tile(name):
+    """The descriptor bits that name output tile `name` (one of TILE_NAMES)."""
+    return (TILE_NAMES.index(name) + 1) << 8
+
+
+def flag_conv(path):
+    """The descriptor bits that name a convolution path (CONV_*)."""
+    return path << 16
+
 AGG_ASSIGN, AGG_ADD, AGG_MAX, AGG_MIN, AGG_MUL = 0, 1, 2, 3, 4
 COMBO_NONE, COMBO_ADD, COMBO_COND, COMBO_EQ, COMBO_MUL = 0, 1, 2, 3, 4
 (EPI_ADD, EPI_SUB, EPI_RSUB, EPI_MUL, EPI_DIV, EPI_RDIV, EPI_MAX, EPI_MIN, EPI_RELU, EPI_NEG, EPI_EXP, EPI_LOG,
@@ -29,7 +43,7 @@ EXPORTS = [
     'pml_hip_memcpy_d2d', 'pml_hip_fill_u32', 'pml_hip_stream_create', 'pml_hip_stream_destroy',
     'pml_hip_stream_sync', 'pml_hip_event_create', 'pml_hip_event_destroy', 'pml_hip_event_record',
     'pml_hip_event_sync', 'pml_hip_event_elapsed_ms', 'pml_hip_gemm_dispatch', 'pml_hip_gemm_invoke',
-    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_tile_of_workgroup', 'pml_hip_gemm_tail_cheaper_apart',
+    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_tile_of_workgroup', 'pml_hip_tile_name', 'pml_hip_tile_by_name', 'pml_hip_gemm_tail_cheaper_apart',
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
@@ -153,6 +167,9 @@ def lib():
         L.pml_hip_gemm_invoke2.argtypes = [ctypes.c_int64, vp, vp, vp, vp, vp, vp, vp, pp, pp, vp]
         L.pml_hip_gemm_pack_b2.argtypes = [ctypes.c_int64, vp, vp]
         L.pml_hip_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+        L.pml_hip_tile_name.restype = ctypes.c_char_p
+        L.pml_hip_tile_name.argtypes = [ctypes.c_int]
+        L.pml_hip_tile_by_name.argtypes = [ctypes.c_char_p]
         L.pml_hip_tile_of_workgroup.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.pml_hip_gemm_tail_cheaper_apart.argtypes = [ctypes.POINTER(GemmDesc)]
         L.pml_hip_conv2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp, pp, pp, vp]

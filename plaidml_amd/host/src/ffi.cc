@@ -178,6 +178,9 @@ void compileProgram(tile::Program* program, const std::string& requested, bool /
     else if (opts["fp32"] != "mfma")
       throw std::runtime_error("Invalid target option fp32=" + opts["fp32"] + " (mfma or bf16x3)");
   }
+  if (opts.count("tile")) options.tile = opts["tile"];
+  if (opts.count("conv")) options.conv = opts["conv"];
+  options.schedule_path = util::Settings::Instance()->get("PLAIDML_SCHEDULE_PATH");
   program->passes.resize(1);  // keep only the "tile" text when compiling again
   tile::foldAddIntoInit(program);
   program->passes.emplace_back("tile-algebraic-opt", program->str());

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <array>
 #include <cstring>
+#include <fstream>
 #include <map>
 #include <numeric>
 #include <set>
@@ -189,7 +190,77 @@ class Planner {
     if (opt_.fuse && opt_.specialise) fuseSecondProducts();
     if (opt_.specialise) padDepthwiseResults();
     pruneDeadSteps();
+    applySchedule();
     return plan_;
+  }
+
+  // Tiling overrides, per program (target options) and per step (schedule file): they travel to the kernel library in
+  // the descriptors' schedule bits.  Runs last, so that a step is keyed by the text the plan dump shows for it.
+  static int convPathByName(const std::string& name) {
+    static const char* const names[] = {"auto", "igemm", "patches", "ldsfilter", "blocks"};
+    for (int i = 0; i < 5; ++i)
+      if (name == names[i]) return i;
+    throw std::runtime_error("Invalid convolution path '" + name + "' (igemm, patches, ldsfilter or blocks)");
+  }
+  static int tileByName(const std::string& name) {
+    const int t = pml_hip_tile_by_name(name.c_str());
+    if (t < 0) throw std::runtime_error("Invalid tile '" + name + "' (64x64, 128x64, 128x128, 128x64w8, 128x128w8, 128x128w8s2, 256x128w16, 64x64w8k2, 256x256w8, 128x64n2)");
+    return t;
+  }
+  struct Rule {
+    int tile = -1, conv = 0;
+  };
+  static Rule parseRule(const std::string& text) {  // "tile=...,conv=..."
+    Rule r;
+    std::stringstream ss(text);
+    for (std::string item; std::getline(ss, item, ',');) {
+      const auto eq = item.find('=');
+      const std::string key = item.substr(0, eq), value = eq == std::string::npos ? "" : item.substr(eq + 1);
+      if (key == "tile")
+        r.tile = tileByName(value);
+      else if (key == "conv")
+        r.conv = convPathByName(value);
+      else
+        throw std::runtime_error("Invalid schedule entry '" + item + "' (tile=... or conv=...)");
+    }
+    return r;
+  }
+  void applySchedule() {
+    Rule all;
+    if (!opt_.tile.empty()) all.tile = tileByName(opt_.tile);
+    if (!opt_.conv.empty()) all.conv = convPathByName(opt_.conv);
+    std::map<std::string, Rule> rules;
+    if (!opt_.schedule_path.empty()) {
+      std::ifstream f(opt_.schedule_path);
+      if (!f) throw std::runtime_error("Cannot read the schedule file " + opt_.schedule_path);
+      for (std::string line; std::getline(f, line);) {
+        const auto open = line.rfind(" {"), lead = line.find("] ");
+        if (line.empty() || line.back() != '}' || open == std::string::npos || lead == std::string::npos || lead > open) continue;
+        rules[line.substr(lead + 2, open - lead - 2)] = parseRule(line.substr(open + 2, line.size() - open - 3));
+      }
+    }
+    for (Step& s : plan_->steps) {
+      if (s.kind != Step::Gemm && s.kind != Step::Conv2d) continue;
+      Rule r = all;
+      const auto it = rules.find(s.text);
+      if (it != rules.end()) {
+        if (it->second.tile >= 0) r.tile = it->second.tile;
+        if (it->second.conv > 0) r.conv = it->second.conv;
+      }
+      if (s.kind == Step::Gemm) r.conv = 0;
+      int32_t& flags = s.kind == Step::Gemm ? s.gemm.flags : s.conv.flags;
+      std::string text;
+      if (r.tile >= 0) {
+        flags |= PML_HIP_FLAG_TILE(r.tile);
+        text += std::string("tile=") + pml_hip_tile_name(r.tile);
+      }
+      if (r.conv > 0) {
+        static const char* const names[] = {"auto", "igemm", "patches", "ldsfilter", "blocks"};
+        flags |= PML_HIP_FLAG_CONV(r.conv);
+        text += std::string(text.empty() ? "" : ",") + "conv=" + names[r.conv];
+      }
+      if (!text.empty()) s.schedule = " {" + text + "}";
+    }
   }
 
   // Two matrix products that are added -- a residual block's projection shortcut and the last 1x1 convolution
@@ -344,7 +415,8 @@ class Planner {
       if (row_bytes % 128 == 0 || row_bytes < 512) continue;
       const int64_t pitch = (row_bytes + 127) / 128 * 128 / es;
       const int64_t rows = X.dw.n * X.dw.oh * X.dw.ow;
-      if (pitch >= (int64_t{1} << 31)) continue;
+      // (the matrix-core kernels address their left-hand side with 32-bit byte offsets below 2 GiB)
+      if (pitch >= (int64_t{1} << 31) || rows * pitch * es >= (int64_t{1} << 31)) continue;
       int readers = 0, writers = 0, y = -1;
       for (size_t k = 0; k < plan_->steps.size(); ++k) {
         const Step& s = plan_->steps[k];
@@ -1889,7 +1961,7 @@ class Planner {
 std::string Plan::dump() const {
   std::stringstream ss;
   ss << "hip plan: " << steps.size() << " launches, " << buffers.size() << " buffers\n";
-  for (size_t i = 0; i < steps.size(); ++i) ss << "  [" << i << "] " << steps[i].text << "\n";
+  for (size_t i = 0; i < steps.size(); ++i) ss << "  [" << i << "] " << steps[i].text << steps[i].schedule << "\n";
   return ss.str();
 }
 

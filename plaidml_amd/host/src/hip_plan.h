@@ -28,6 +28,7 @@ struct BufferInfo {
 struct Step {
   enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy, Gather, Scatter, ArgSort, Prng } kind = Copy;
   std::string text;  // one line for the plan dump
+  std::string schedule;  // "{tile=...,conv=...}" when the target options or a schedule file named this step's tiling
   // descriptors (only the one matching `kind` is meaningful)
   pml_hip_gemm_desc gemm{};
   pml_hip_conv2d_desc conv{};
@@ -75,6 +76,11 @@ struct Options {
   // fp32 GEMMs and convolutions on the bf16 matrix cores, every operand value split into a bf16 head and a bf16
   // remainder (three products per term, about 2^-16 relative error per product): `hip{fp32=bf16x3}`
   bool fp32_as_bf16x3 = false;
+  // Schedule overrides (the reference: PLAIDML_SCHEDULE_PATH, pmlc/target/x86/pipeline.cc:267-272).  `tile` / `conv`
+  // (`hip{tile=128x128w8,conv=igemm}`) apply to every matrix product / convolution of the program; `schedule_path` names
+  // a file of plan-dump lines, "[n] <step text> {tile=...,conv=...}", that apply to the steps whose text they repeat --
+  // a plan dump edited by hand is such a file.  Names: pml_hip_tile_name, and igemm / patches / ldsfilter / blocks.
+  std::string tile, conv, schedule_path;
 };
 
 // Runs the pipeline on a copy of the program's op list and returns the plan.

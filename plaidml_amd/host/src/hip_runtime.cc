@@ -6,6 +6,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <regex>
 #include <sstream>
 
@@ -390,17 +391,48 @@ void registerRuntime(const std::string& id, std::shared_ptr<Runtime> runtime) {
   registry()[id] = std::move(runtime);
 }
 
+// Page-locked host memory for buffers the library allocates itself.  Asking for it initialises the GPU runtime as a
+// side effect, so a process that must not touch the GPU (one that only builds programs, or that will exec another
+// program) sets PLAIDML_PINNED=0; the total is capped (PLAIDML_PINNED_MAX_MB, default 4096) because page-locked
+// memory is taken from what the host can page.  Beyond the cap, and on any failure, the caller falls back to
+// ordinary memory (nullptr here).
+namespace {
+std::mutex g_pinned_mutex;
+std::map<void*, size_t> g_pinned_sizes;
+size_t g_pinned_total = 0;
+}  // namespace
+
 void* pinnedAlloc(size_t bytes) {
+  const std::string enabled = util::Settings::Instance()->get("PLAIDML_PINNED");
+  if (enabled == "0" || enabled == "false" || enabled == "off") return nullptr;
+  const std::string cap_text = util::Settings::Instance()->get("PLAIDML_PINNED_MAX_MB");
+  const size_t cap = (cap_text.empty() ? size_t{4096} : static_cast<size_t>(std::strtoull(cap_text.c_str(), nullptr, 10))) << 20;
+  {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    if (bytes > cap || g_pinned_total > cap - bytes) return nullptr;
+  }
   initRuntimes();
   if (listDevices().empty()) return nullptr;
   void* p = nullptr;
   if (pml_hip_host_alloc(&p, bytes) != 0 || !p) return nullptr;
   std::memset(p, 0, bytes);
+  std::lock_guard<std::mutex> lock(g_pinned_mutex);
+  g_pinned_sizes[p] = bytes;
+  g_pinned_total += bytes;
   return p;
 }
 
 void pinnedFree(void* p) {
-  if (p) pml_hip_host_free(p);
+  if (!p) return;
+  {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    const auto it = g_pinned_sizes.find(p);
+    if (it != g_pinned_sizes.end()) {
+      g_pinned_total -= it->second;
+      g_pinned_sizes.erase(it);
+    }
+  }
+  pml_hip_host_free(p);
 }
 
 void initRuntimes() {

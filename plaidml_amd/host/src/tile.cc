@@ -807,9 +807,13 @@ void normaliseRow(IneqRow& r) {
   }
 }
 
-// Range of variable `keep` in the linear relaxation; false when unbounded on either side or when the elimination
-// grows past its budget.
-bool fourierMotzkinRange(const std::vector<BoundForm>& forms, size_t n, size_t keep, int64_t* lo, int64_t* hi) {
+// Range of variable `keep` in the linear relaxation: 1 = found, 0 = unbounded on either side, -1 = no range found after
+// the elimination grew past its budget of rows.  Past the budget the rows with the most variables are dropped: fewer
+// constraints describe a larger set, so a range found then still contains the true one (the integer search that
+// follows tightens it), it is only no longer the relaxation's own.  `order` picks the elimination order: 0 = the variable that makes the fewest new rows
+// first, 1 = by index, 2 = by index from the back, 3 = no elimination chain at all, only pairs of forms over the kept variable and one other
+// (further tries when the first runs out of budget).
+int fourierMotzkinRange(const std::vector<BoundForm>& forms, size_t n, size_t keep, int64_t* lo, int64_t* hi, int order = 0) {
   std::set<IneqRow> rows;
   for (const BoundForm& f : forms) {
     IneqRow up(n + 1), down(n + 1);
@@ -824,14 +828,52 @@ bool fourierMotzkinRange(const std::vector<BoundForm>& forms, size_t n, size_t k
     rows.insert(up);
     rows.insert(down);
   }
-  const size_t kBudget = 4000;
+  const size_t kBudget = 1500;
+  int prunings = 0;
+  bool pruned = false;
+  if (order == 3) {
+    // last try, a relaxation that stays small: for every other variable u, only the rows over {keep, u}, and only u
+    // eliminated -- pairs of forms such as a x + b u and a x - b u bound x whatever else the system holds
+    pruned = true;
+    std::set<IneqRow> single;
+    auto support_in = [&](const IneqRow& r, size_t u) {
+      for (size_t i = 0; i < n; ++i)
+        if (i != keep && i != u && r[i] != 0) return false;
+      return true;
+    };
+    for (size_t u = 0; u < n; ++u) {
+      if (u == keep) continue;
+      std::vector<const IneqRow*> pos, neg;
+      for (const IneqRow& r : rows) {
+        if (!support_in(r, u)) continue;
+        if (r[u] > 0) pos.push_back(&r);
+        else if (r[u] < 0) neg.push_back(&r);
+        else if (r[keep] != 0) single.insert(r);
+      }
+      for (const IneqRow* p : pos)
+        for (const IneqRow* q : neg) {
+          IneqRow r(n + 1);
+          const __int128 cp = (*p)[u], cq = -(*q)[u];
+          for (size_t i = 0; i <= n; ++i) r[i] = cq * (*p)[i] + cp * (*q)[i];
+          if (r[keep] == 0) continue;
+          normaliseRow(r);
+          single.insert(r);
+        }
+    }
+    rows.swap(single);
+  }
   std::vector<bool> gone(n, false);
-  for (size_t step = 0; step + 1 < n; ++step) {
+  for (size_t step = 0; step + 1 < n && order != 3; ++step) {
     // the variable whose elimination makes the fewest new rows
     size_t best = n;
     size_t bestCost = 0;
-    for (size_t v = 0; v < n; ++v) {
+    for (size_t k = 0; k < n; ++k) {
+      const size_t v = order == 2 ? n - 1 - k : k;
       if (v == keep || gone[v]) continue;
+      if (order == 1 || order == 2) {
+        best = v;
+        break;
+      }
       size_t pos = 0, neg = 0;
       for (const IneqRow& r : rows) {
         if (r[v] > 0) ++pos;
@@ -864,7 +906,19 @@ bool fourierMotzkinRange(const std::vector<BoundForm>& forms, size_t n, size_t k
         if (!any) continue;  // a statement about constants only
         normaliseRow(r);
         next.insert(r);
-        if (next.size() > kBudget) return false;
+        if (next.size() > 2 * kBudget) {
+          if (++prunings > 4) return -1;
+          pruned = true;
+          std::vector<std::pair<size_t, IneqRow>> ranked;
+          for (const IneqRow& row : next) {
+            size_t vars = 0;
+            for (size_t i = 0; i < n; ++i) vars += row[i] != 0;
+            ranked.emplace_back(vars, row);
+          }
+          std::stable_sort(ranked.begin(), ranked.end(), [](const auto& x, const auto& y) { return x.first < y.first; });
+          next.clear();
+          for (size_t i = 0; i < kBudget; ++i) next.insert(ranked[i].second);
+        }
       }
     rows.swap(next);
     gone[best] = true;
@@ -891,11 +945,11 @@ bool fourierMotzkinRange(const std::vector<BoundForm>& forms, size_t n, size_t k
       haveHi = true;
     }
   }
-  if (!haveLo || !haveHi) return false;
-  if (vlo < -kInfBound / 2 || vhi > kInfBound / 2) return false;
+  if (!haveLo || !haveHi) return pruned ? -1 : 0;
+  if (vlo < -kInfBound / 2 || vhi > kInfBound / 2) return pruned ? -1 : 0;
   *lo = static_cast<int64_t>(vlo);
   *hi = static_cast<int64_t>(vhi);
-  return true;
+  return 1;
 }
 
 // Step 3: is there an integer point of the set inside the box?  `budget` counts search nodes; -1 = gave up.
@@ -959,7 +1013,12 @@ void computeBounds(Op* op) {
       for (size_t v = 0; v < n; ++v) {
         if (lo[v] > -kInfBound && hi[v] < kInfBound) continue;
         int64_t l = 0, h = 0;
-        if (!fourierMotzkinRange(forms, n, v, &l, &h))
+        int found = -1;
+        for (int order = 0; order < 4 && found < 0; ++order) found = fourierMotzkinRange(forms, n, v, &l, &h, order);
+        if (found < 0)
+          throw std::runtime_error("Bounds too complex: eliminating the other indices around '" + op->idxNames[v] + "' of contraction '" +
+                                   op->name + "' outgrows the budget of inequalities in every order tried");
+        if (found == 0)
           throw std::runtime_error("Unbounded index '" + op->idxNames[v] + "' in contraction '" + op->name + "'");
         lo[v] = std::max(lo[v], l);
         hi[v] = std::min(hi[v], h);

@@ -196,9 +196,15 @@ class ForeignBuffer : public Buffer {
   char* data() final { return data_; }
   size_t size() const final { return size_; }
   BufferPtr clone() final {
-    auto copy = std::make_shared<ForeignBuffer>(shape_, alloc_, release_);
-    std::memcpy(copy->data_, data_, size_);
-    return copy;
+    try {
+      auto copy = std::make_shared<ForeignBuffer>(shape_, alloc_, release_);
+      std::memcpy(copy->data_, data_, size_);
+      return copy;
+    } catch (const std::bad_alloc&) {  // the allocator has no more to give (a cap on page-locked memory): ordinary memory
+      auto copy = std::make_shared<SimpleBuffer>(shape_);
+      std::memcpy(copy->data(), data_, size_);
+      return copy;
+    }
   }
 
  private:

@@ -67,6 +67,26 @@ def test_domain_bounded_only_by_combinations():
     assert bounds_of(prog) == {'i': (0, 9), 'j': (-4, 4)}
 
 
+def test_many_coupled_forms():
+    """Systems in which no index has a range of its own and many forms couple the indices: eight indices whose every
+    pairwise sum lies in [0, 10) (x_i >= -4 because x_i + x_j >= 0, x_i + x_k >= 0 and x_j + x_k <= 9 give 2 x_i >= -9;
+    x_i = 9 with all others 0 is feasible), and six indices bound only by sums and differences of pairs, whose exact
+    ranges an integer linear program (scipy.optimize.milp) gave as written below."""
+    xs = [E.TensorIndex('x%d' % i) for i in range(8)]
+    cons = [xs[i] + xs[j] < 10 for i in range(8) for j in range(i + 1, 8)]
+    prog = program([xs[0] + xs[1]], [100], [xs[0] + xs[1]], [100], cons)
+    assert bounds_of(prog) == {'x%d' % i: (-4, 9) for i in range(8)}
+    rng = np.random.default_rng(0)
+    xs = [E.TensorIndex('x%d' % i) for i in range(6)]
+    cons = []
+    for i in range(6):
+        for j in range(i + 1, 6):
+            a, b = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+            cons += [a * xs[i] + b * xs[j] < 10, a * xs[i] - b * xs[j] + 20 < 40]
+    prog = program([xs[0] + 50], [100], [xs[0] + 50], [100], cons)
+    assert bounds_of(prog) == {'x0': (0, 3), 'x1': (-1, 3), 'x2': (0, 3), 'x3': (-1, 3), 'x4': (0, 3), 'x5': (0, 3)}
+
+
 def test_really_unbounded_index_is_an_error():
     i, j = E.TensorIndex('i'), E.TensorIndex('j')
     prog = program([i + j], [10], [i + j], [10], [])

@@ -126,6 +126,45 @@ def test_target_option_fp32_as_three_bf16_products():
         programs.config0_gemm_f32(E, op)[0].compile('hip{fp32=tf32}')
 
 
+def test_schedule_overrides_by_option_and_by_file(tmp_path, monkeypatch):
+    """Tiling overrides: `hip{tile=...,conv=...}` for a whole program, a schedule file for single steps (the reference
+    loads one from PLAIDML_SCHEDULE_PATH, pmlc/target/x86/pipeline.cc:267-272).  The plan dump shows the override and
+    an edited dump is itself a schedule file."""
+    from plaidml_amd import hipkernels as hk
+    L = hk.lib()
+    for t, name in enumerate(hk.TILE_NAMES):  # the Python names are the library's
+        assert L.pml_hip_tile_name(t) == name.encode() and L.pml_hip_tile_by_name(name.encode()) == t
+    assert L.pml_hip_tile_name(len(hk.TILE_NAMES)) is None and L.pml_hip_tile_by_name(b'1x1') == -1
+    plain = plan_of(programs.residual_block(E, op)[0])
+    assert '{' not in plain
+    t = plan_of(programs.residual_block(E, op)[0], 'hip{tile=128x128w8,conv=igemm}')
+    for a, b in zip(plain.splitlines()[1:], t.splitlines()[1:]):
+        if 'conv2d' in a:
+            assert b == a + ' {tile=128x128w8,conv=igemm}'
+        elif 'gemm' in a:
+            assert b == a + ' {tile=128x128w8}'
+        else:
+            assert b == a
+    with pytest.raises(E.PlaidMLError, match="Invalid tile '3x3'"):
+        programs.residual_block(E, op)[0].compile('hip{tile=3x3}')
+    with pytest.raises(E.PlaidMLError, match="Invalid convolution path"):
+        programs.residual_block(E, op)[0].compile('hip{conv=winograd}')
+    # a schedule file: the plain dump with one step's line marked
+    lines = plain.splitlines()
+    k = next(i for i, l in enumerate(lines) if 'gemm' in l or 'conv2d' in l)
+    lines[k] += ' {tile=64x64}'
+    sched = tmp_path / 'schedule.txt'
+    sched.write_text('\n'.join(lines) + '\n')
+    monkeypatch.setenv('PLAIDML_SCHEDULE_PATH', str(sched))
+    t = plan_of(programs.residual_block(E, op)[0])
+    assert t.splitlines() == lines          # only that step changed, and the dump reproduces the file
+    t2 = plan_of(programs.residual_block(E, op)[0], 'hip{tile=128x64}')   # the file's entry wins over the program-wide option
+    assert t2.splitlines()[k] == lines[k] and t2.count('{tile=128x64}') >= 1
+    monkeypatch.setenv('PLAIDML_SCHEDULE_PATH', str(tmp_path / 'missing.txt'))
+    with pytest.raises(E.PlaidMLError, match='Cannot read the schedule file'):
+        programs.residual_block(E, op)[0].compile('')
+
+
 def test_target_options_switch_specialisation_off():
     prog = programs.config1_conv(E, op, 'BFLOAT16')[0]
     t = plan_of(prog, 'hip{specialise=0,fuse=0}')

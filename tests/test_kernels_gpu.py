@@ -28,13 +28,17 @@ def bf16(a):
     return E.bf16_bits(np.asarray(a, np.float32))
 
 
+# schedule bits (hk.flag_tile / hk.flag_conv) that a test adds to every descriptor run_gemm / run_conv build
+FORCED = {'flags': 0}
+
+
 def run_gemm(A, B, in_dt, out_dt, init=None, init_strides=(0, 0), init_dt=0, tail=None, operands=(), c_dt=None,
              extra_out=None, flags=0):
     M, K = A.shape
     _, N = B.shape
     d = hk.GemmDesc()
     d.in_dtype, d.out_dtype = in_dt, out_dt
-    d.flags = flags
+    d.flags = flags | FORCED['flags']
     d.m, d.n, d.k = M, N, K
     d.lda, d.ldb, d.ldc = K, N, N
     d.c_dtype = c_dt if c_dt is not None else out_dt
@@ -91,10 +95,10 @@ TILE_NAMES = ['64x64', '128x64', '128x128', '128x64w8', '128x128w8', '128x128w8s
 
 @pytest.mark.parametrize('tile', TILE_NAMES)
 def test_every_tile_configuration(tile, monkeypatch):
-    """Every tiling the library holds (selected with the tuning override PML_HIP_TILE), on a problem that is ragged
+    """Every tiling the library holds (named in the descriptor's schedule bits), on a problem that is ragged
     in M, N and K and spans several tiles: int8 bit for bit, bf16 (+ bias + relu, the direct tail where the tile is
     interior) and fp32 against float64."""
-    monkeypatch.setenv('PML_HIP_TILE', tile)
+    monkeypatch.setitem(FORCED, 'flags', hk.flag_tile(tile))
     print('tile', tile, flush=True)
     rng = np.random.default_rng(7)
     M, N, K = 600, 520, 336
@@ -360,7 +364,7 @@ def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bia
         OH, OW = (H + 2 * pad - KH) // stride + 1, (W + 2 * pad - KW) // stride + 1
     d = hk.Conv2dDesc()
     d.in_dtype, d.out_dtype, d.c_dtype = in_dt, out_dt, out_dt
-    d.flags = flags
+    d.flags = flags | FORCED['flags']
     d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, KH, KW, CO, OH, OW
     d.stride_h = d.stride_w = stride
     d.dil_h = d.dil_w = 1
@@ -569,7 +573,7 @@ def test_conv_register_filter_matches_lds_filter(batch, monkeypatch):
     Iv, Fv = _conv_case('bf16', (batch, 56, 56, 64), 3, 3, 64, op.SAME_UPPER, 29)
     bias = bf16(E.round_bf16(np.random.default_rng(30).standard_normal(64).astype(np.float32)))
     a = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
-    monkeypatch.setenv('PML_HIP_CONV', 'ldsfilter')
+    monkeypatch.setitem(FORCED, 'flags', hk.flag_conv(hk.CONV_LDSFILTER))
     b = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
     np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
     # the last image (part of the halved tiles when batch = 24) against a float64 evaluation of the definition
@@ -600,7 +604,7 @@ def test_conv_resident_filter_matches_generic_kernel(monkeypatch):
     Iv, Fv = _conv_case('bf16', (4, 28, 28, 64), 3, 3, 64, op.SAME_UPPER, 25)
     bias = bf16(E.round_bf16(np.random.default_rng(26).standard_normal(64).astype(np.float32)))
     a = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
-    monkeypatch.setenv('PML_HIP_CONV', 'igemm')
+    monkeypatch.setitem(FORCED, 'flags', hk.flag_conv(hk.CONV_IGEMM))
     b = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True))
     np.testing.assert_allclose(a, b, rtol=BF16_RTOL, atol=1e-2)
 
@@ -637,14 +641,18 @@ STEM_CASES = [((2, 30, 34, 3), 7, 64, None), ((2, 32, 32, 3), 7, 64, 3), ((2, 31
 @pytest.mark.parametrize('shape,k,co,pad', STEM_CASES)
 def test_conv_few_channel_stride2(kind, shape, k, co, pad, capsys):
     _stem_case(kind, shape, k, co, 2, pad, 41)
-    assert '2x2 pixel blocks' in capsys.readouterr().out
+    text = capsys.readouterr().out
+    assert '2x2 pixel blocks' in text
+    # 7x7 (4x4 block taps) onto 64 channels in bf16 is the row-walking kernel's case: no silent fall-back to the implicit GEMM
+    if kind == 'bf16' and k == 7 and co == 64:
+        assert 'row by row with the filter in registers' in text
 
 
 @pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
 @pytest.mark.parametrize('stride', [1, 2])
 def test_conv_few_channel_patch_matrix(kind, stride, capsys, monkeypatch):
     # other strides (and stride 2 on request) gather a patch matrix [M][K padded] and run a plain GEMM
-    monkeypatch.setenv('PML_HIP_CONV', 'patches')
+    monkeypatch.setitem(FORCED, 'flags', hk.flag_conv(hk.CONV_PATCHES))
     _stem_case(kind, (2, 30, 34, 3), 7, 64, stride, None, 43)
     assert 'patch matrix' in capsys.readouterr().out
 
@@ -896,7 +904,7 @@ def _gemm_f32_layouts(A, B_kn, ldb, flags, packed_first=False):
     for layout in (0, 1):
         d = hk.GemmDesc()
         d.in_dtype = d.out_dtype = d.c_dtype = hk.F32
-        d.flags = flags
+        d.flags = flags | FORCED['flags']
         d.m, d.n, d.k = M, N, K
         d.lda, d.ldc = K, N
         d.b_layout = layout
