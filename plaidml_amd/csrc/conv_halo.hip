@@ -414,6 +414,11 @@ typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
+// relu as a lower clamp in one instruction (v_maximum3_f32: the IEEE 754-2019 maximum, which keeps a NaN like
+// "x < lo ? lo : x" does; it orders -0 below +0, so a result of exactly -0 under relu is stored as +0).
+// lo = 0 with relu, -infinity without.
+__device__ __forceinline__ float relu_clamp(float x, float lo) { return __builtin_elementwise_maximum(x, lo); }
+
 constexpr unsigned kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
 #define PML_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 constexpr int kConvAhead = 2;                 // K-blocks (pairs of them in the register-filter kernel) operand fragments are fetched ahead
@@ -583,7 +588,7 @@ __global__ __launch_bounds__(kThreads) void conv_halo3x3_kernel(IgemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         v[e] = (float)acc[i][j][4 * q + e] + (float)cinit[j][q][e];
-        v[e] = v[e] < lo_f ? lo_f : v[e];
+        v[e] = relu_clamp(v[e], lo_f);
       }
       if (KIND == KIND_BF16) {
         const f32x2_t a01 = {v[0], v[1]}, a23 = {v[2], v[3]};
@@ -838,16 +843,20 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
   };
 
   // b_raw == 2: the filter was packed once into the order this kernel keeps it in registers (regfilter_image_kernel
-  // below): fragment (channel block cb, K-block s) of lane l is the 16 bytes at ((cb * 36 + s) * 64 + l) * 16, so every
-  // request of a wavefront is 1 KB of consecutive bytes and nothing passes through LDS or is turned in registers.
+  // below): fragment (channel block cb, K-block s) of lane l is the 16 bytes at ((cb * 36 + s) * 64 + l) * 16.  The
+  // 72 KB go to LDS as they lie (requests that write LDS directly, no registers, nothing turned) and every fragment
+  // read of a wavefront is 1 KB of consecutive bytes.  (Loading the fragments from memory straight into registers was
+  // measured: 36 KB per wavefront through the vector memory path take longer than the whole trip through LDS.)
   const bool image = p.b_raw == 2;
   i32x4_t breg[kBlocks][NI];
   if (image) {
-    const i32x4_t* img = (const i32x4_t*)p.Bt + lane;
+    // 72 requests of 1 KB into the first window buffer, nine per wavefront
+    const __amdgpu_buffer_rsrc_t rimg = __builtin_amdgcn_make_buffer_rsrc((void*)p.Bt, 0, 2 * kBlocks * 1024, kRsrcFlags);
 #pragma unroll
-    for (int j = 0; j < NI; ++j)
-#pragma unroll
-      for (int s = 0; s < kBlocks; ++s) breg[s][j] = img[((cb0 + j) * kBlocks + s) * 64];
+    for (int r = 0; r < 2 * kBlocks / (kNT / 64); ++r) {
+      const int req = wave + (kNT / 64) * r;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rimg, PML_LDS(smem + req * 1024), 16, req * 1024 + lane * 16, 0, 0, 0);
+    }
   }
   FilterStager<KIND, kNT> filter;
   if (!image) filter.load(p, tid);
@@ -882,6 +891,12 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
   // MFMA row 8q + 4h + e of channel block cb is given output channel 32cb + 16h + 4q + e, so that
   // a lane (pixel, h) ends up owning the 16 consecutive channels 32cb + 16h .. + 15 in register order;
   // the staged filter keeps that channel in row 32h + 8q + 4cb + e
+  if (image) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int s = 0; s < kBlocks; ++s) breg[s][j] = *(const i32x4_t*)(smem + (((cb0 + j) * kBlocks + s) * 64 + lane) * 16);
+  }
   if (!image) {
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
@@ -931,7 +946,7 @@ __global__ __launch_bounds__(512 / NI) void conv_regfilter3x3_kernel(IgemmArgs p
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         v[e] = (float)acc[j][4 * q + e];
-        v[e] = v[e] < lo_f ? lo_f : v[e];
+        v[e] = relu_clamp(v[e], lo_f);
       }
       const f32x2_t a01 = {v[0], v[1]}, a23 = {v[2], v[3]};
       const bf16x2_t h01 = __builtin_convertvector(a01, bf16x2_t), h23 = __builtin_convertvector(a23, bf16x2_t);
@@ -1251,8 +1266,8 @@ __global__ __launch_bounds__(256, 2) void conv_blocks4x4_kernel(IgemmArgs p, int
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
               float v0 = acc[j][8 * half + 2 * k], v1 = acc[j][8 * half + 2 * k + 1];
-              v0 = v0 < lo ? lo : v0;
-              v1 = v1 < lo ? lo : v1;
+              v0 = relu_clamp(v0, lo);
+              v1 = relu_clamp(v1, lo);
               const f32x2_t pair = {v0, v1};
               const bf16x2_t hh = __builtin_convertvector(pair, bf16x2_t);
               __builtin_memcpy(&w[k], &hh, 4);
@@ -1364,6 +1379,9 @@ size_t conv_halo_prepare(int kind, IgemmArgs* a, bool filter_in_lds) {
   }
   return total;
 }
+
+// The image passes through the first window buffer while the first window arrives in the second: it must fit there.
+bool regfilter_takes_image(int ow) { return (size_t)reg_win_bytes(ow + 2) >= kRegfilterImageBytes; }
 
 hipError_t regfilter_image_launch(const void* bt, int64_t ldbt_bytes, void* image, hipStream_t s) {
   if ((((uintptr_t)bt | (uintptr_t)image) & 15) != 0 || ldbt_bytes % 16 != 0) return hipErrorInvalidValue;

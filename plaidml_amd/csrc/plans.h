@@ -198,6 +198,7 @@ hipError_t conv_halo_launch(int kind, const IgemmArgs& a, size_t lds_bytes, int 
 // keeps it in registers: kRegfilterImageBytes bytes at `image`.
 constexpr size_t kRegfilterImageBytes = 2 * 36 * 64 * 16;
 hipError_t regfilter_image_launch(const void* bt, int64_t ldbt_bytes, void* image, hipStream_t s);
+bool regfilter_takes_image(int ow);  // rows of `ow` output pixels leave the image room in LDS (otherwise the packed Bt is used)
 // The re-blocked few-channel convolution with 4x4 block taps of 16 channels and 64 output channels: LDS bytes of the
 // row-walking kernel, or 0 when `a` (already pointing at the re-blocked input) does not qualify.
 size_t conv_blocks4x4_prepare(int kind, const IgemmArgs& a);

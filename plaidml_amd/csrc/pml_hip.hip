@@ -1050,9 +1050,8 @@ int pml_hip_conv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream 
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_CONV || !filter) return fail("conv2d_pack_filter: bad argument");
   const pml_hip_conv2d_desc& d = p->conv;
-  (void)d;
   if (check(pack_conv_filter(p, filter, (hipStream_t)s), "pack_conv_filter")) return 1;
-  if (p->halo_lds && p->halo_variant == 3) {
+  if (p->halo_lds && p->halo_variant == 3 && regfilter_takes_image((int)d.ow)) {
     // the register-filter kernel takes a constant filter in its own register order: no trip through LDS per launch
     if (!p->reg_image && check(hipMalloc(&p->reg_image, kRegfilterImageBytes), "hipMalloc")) return 1;
     if (check(regfilter_image_launch(p->bt, p->bt_ld * dt_size(d.in_dtype), p->reg_image, (hipStream_t)s), "regfilter_image_launch")) return 1;

@@ -354,7 +354,7 @@ def test_gemm_bf16(M, N, K):
 
 
 def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bias=None, relu=False, tail=None,
-             operands=(), flags=0):
+             operands=(), flags=0, packed=False):
     N, H, W, CI = I.shape
     KH, KW, _, CO = F.shape
     ph, OH = op.compute_padding_and_output_size(H, KH, stride, autopad)
@@ -384,7 +384,9 @@ def run_conv(I, F, in_dt, out_dt, stride=1, pad=None, autopad=op.SAME_UPPER, bia
     dO = hk.DeviceBuffer(N * OH * OW * CO * np.dtype(np_c).itemsize)
     dB = hk.DeviceBuffer.from_numpy(bias) if bias is not None else None
     dops = [hk.DeviceBuffer.from_numpy(o) for o in operands]
-    hk.check(hk.lib().pml_hip_conv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, dB.ptr if dB else None,
+    if packed:  # a constant filter: re-laid once, the invoke is given none
+        hk.check(hk.lib().pml_hip_conv2d_pack_filter(plan, dF.ptr, None))
+    hk.check(hk.lib().pml_hip_conv2d_invoke(plan, dI.ptr, None if packed else dF.ptr, dO.ptr, dB.ptr if dB else None,
                                             hk.ptr_array([o.ptr for o in dops]), hk.ptr_array([]), None))
     hk.check(hk.lib().pml_hip_stream_sync(None))
     out = dO.to_numpy(np_c, (N, OH, OW, CO))
@@ -582,6 +584,32 @@ def test_conv_register_filter_matches_lds_filter(batch, monkeypatch):
               for ky in range(3) for kx in range(3))
     ref = np.maximum(ref + E.bf16_from_bits(bias).astype(np.float64), 0)
     np.testing.assert_allclose(a[-1], ref, rtol=BF16_RTOL, atol=2e-2)
+
+
+@pytest.mark.parametrize('kind,shape', [('bf16', (5, 56, 56, 64)), ('bf16', (3, 20, 40, 64)), ('i8', (5, 56, 56, 128)),
+                                        ('i8', (2, 30, 33, 128))])
+def test_conv_filter_packed_once_equals_filter_per_call(kind, shape, capsys):
+    """A constant 3x3 filter re-laid once (rows of 56 pixels: into the order the register-filter kernel holds it in
+    registers; other shapes: as Bt, for whichever resident-filter kernel takes them) against the same filter handed over with every call, bit for bit; with a NaN, an
+    infinity and a -0 product in the data, which relu must keep / keep / may store as +0."""
+    rng = np.random.default_rng(61)
+    if kind == 'bf16':
+        Iv = E.round_bf16(rng.standard_normal(shape).astype(np.float32))
+        Iv[0, 3, 3, 5], Iv[1, 0, 0, 0], Iv[2, 7, 9, :] = np.nan, np.inf, 0.0
+        Fv = E.round_bf16((rng.standard_normal((3, 3, 64, 64)) * 0.06).astype(np.float32))
+        bias = bf16(E.round_bf16(rng.standard_normal(64).astype(np.float32)))
+        a = run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True)
+        assert shape[2] != 56 or 'in registers' in capsys.readouterr().out
+        b = run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, bias=bias, relu=True, packed=True)
+        af = E.bf16_from_bits(a)
+        assert np.isnan(af[0, 2:5, 2:5]).all() and np.isinf(af[1, 0, 0]).any()
+    else:
+        Iv = rng.integers(-127, 128, shape, dtype=np.int8)
+        Fv = rng.integers(-127, 128, (3, 3, 128, 64), dtype=np.int8)
+        a = run_conv(Iv, Fv, hk.I8, hk.I32, relu=True)
+        assert shape[2] != 56 or 'in registers' in capsys.readouterr().out
+        b = run_conv(Iv, Fv, hk.I8, hk.I32, relu=True, packed=True)
+    np.testing.assert_array_equal(a, b)
 
 
 def test_conv_resident_filter_general_tail(capsys):
