@@ -173,6 +173,8 @@ __device__ __forceinline__ bool direct_tail_ok(const IgemmArgs& p, int64_t n0, i
   return true;
 }
 
+typedef unsigned int u32x4_tail_t __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ void unpack_bf16x8(const i32x4_t& w, float* f) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -570,6 +572,75 @@ __device__ __forceinline__ void tile_tail(const IgemmArgs& p, const typename Acc
   // output, cast between si32 / f32 / si8, or are f32 arithmetic on immediates, scalars and per-column
   // vectors -- the requantisation chain  store, cast f32, * scale[col], clamp, round, cast si8.
   // Four columns at a time, 4 / 16-byte stores; the step semantics are the interpreter's.
+  if constexpr (KIND == KIND_I8) {
+    // (both outputs are addressed with 32-bit byte offsets into buffer descriptors of their exact size: a store past
+    // the last row has an offset beyond the buffer and is dropped, so the row loop has no branches)
+    if (p.tail_mode == 4 && p.tail_rq && full4 && (p.ldc & 3) == 0 && (p.init == nullptr || col_init) &&
+        p.M * p.ldc * 4 < ((int64_t)1 << 31)) {
+      // the requantisation chain as straight code: si32 sum (stored to the extra output as it is) -> f32 -> * scale
+      // -> clamp -> round half away from zero -> si8.  Rounding and the cast are one step here: for x >= 0
+      // floor(x + 0.5) and for x < 0 ceil(x - 0.5) both equal trunc(x + copysign(0.5, x)) -- the sum is the same
+      // floating-point addition and floor / ceil of a value of that sign is truncation -- and the conversion to
+      // an integer truncates by itself.  The clamps (v > lo ? v : lo, v < hi ? v : hi: a NaN goes to the bound) are
+      // the hardware's max / min, which agree with them except in the sign of a zero, and a zero of either sign
+      // becomes the same integer; the product they follow is never a signalling NaN.
+      const float* const scale = (const float*)p.operands[p.rq_scale];
+      f32x4_t sc;
+      if (p.tail.operand_col_stride[p.rq_scale] == 0) {
+        sc = f32x4_t{scale[0], scale[0], scale[0], scale[0]};
+      } else {
+        sc = *(const f32x4_t*)(scale + n);
+      }
+      auto pinned = [](int v) {
+        v = __builtin_amdgcn_readfirstlane(v);
+        asm volatile("" : "+s"(v));
+        return v;
+      };
+      const float lo = __int_as_float(pinned(__float_as_int(p.rq_lo))), hi = __int_as_float(pinned(__float_as_int(p.rq_hi)));
+      const int ldc = pinned((int)p.ldc);
+      const unsigned bytes32 = (unsigned)pinned((int)(p.M * p.ldc * 4));
+      constexpr unsigned kFlags = 0x00020000u;  // raw buffer, 32-bit data format
+      const bool with_sums = p.rq_store >= 0;
+      const __amdgpu_buffer_rsrc_t rsum = __builtin_amdgcn_make_buffer_rsrc(with_sums ? p.outs[with_sums ? p.rq_store : 0] : p.C, 0,
+                                                                            with_sums ? (int)bytes32 : 0, kFlags);
+      const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.C, 0, (int)(bytes32 >> 2), kFlags);
+      // element offset of this thread's first row; rows past M are pushed beyond either buffer
+      const unsigned first = (unsigned)((m0 + row0) * ldc + n);
+      const int rows_left = (int)(p.M - m0) - row0;  // rows of this thread's column group that exist, counted from its first
+      constexpr int kIters = (BM + RPP - 1) / RPP;
+      constexpr int kRows = kIters < 8 ? kIters : 8;
+#pragma unroll
+      for (int it0 = 0; it0 < kIters; it0 += kRows) {
+        i32x4_t acc4[kRows];
+#pragma unroll
+        for (int c = 0; c < kRows; ++c) {
+          const int row = row0 + (it0 + c) * RPP;
+          acc4[c] = *(const i32x4_t*)&ctile[(row < BM ? row : row0) * CS + c4];
+        }
+#pragma unroll
+        for (int c = 0; c < kRows; ++c) {
+          const int step = (it0 + c) * RPP;
+          const bool live = row0 + step < BM && step < rows_left;
+          const unsigned o = live ? first + (unsigned)(step * ldc) : 0x20000000u;  // past the si8 buffer; x 4 bytes = 2 GiB: past the si32 one
+          i32x4_t a = acc4[c];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) a[q] = (int)((unsigned)a[q] + (unsigned)(int)cinit[q]);  // (zeros when there is none)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_tail_t, a), rsum, (int)(o << 2), 0, 0);
+          uint32_t w = 0;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float v = (float)a[q] * sc[q];
+            v = __builtin_fmaxf(v, lo);
+            v = __builtin_fminf(v, hi);
+            const int t = (int)(v + __builtin_copysignf(0.5f, v));
+            w |= (uint32_t)(t & 255) << (8 * q);
+          }
+          __builtin_amdgcn_raw_buffer_store_b32(w, rq, (int)o, 0, 0);
+        }
+      }
+      return;
+    }
+  }
   if (KIND == KIND_I8 && p.tail_mode == 4 && full4 && (p.ldc & 3) == 0) {
     float xs[8][4];
 #pragma unroll

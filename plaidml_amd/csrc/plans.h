@@ -172,6 +172,11 @@ struct IgemmArgs {
   int tail_mode;
   int tail_relu;
   int tail_ssr;  // tail_mode 3 only: 1 = result * column vector + column vector, 2 = the same and relu (all in the bf16 result type)
+  // tail_mode 4 only: 1 = the chain is exactly a requantisation -- (store the si32 sum to outs[rq_store])? cast f32,
+  // * operands[rq_scale] (one f32 per column, or a single one), lower clamp rq_lo (v > lo ? v : lo), upper clamp rq_hi
+  // (v < hi ? v : hi), round half away from zero, cast si8 -- which the tail then runs as straight code
+  int tail_rq, rq_store, rq_scale;
+  float rq_lo, rq_hi;
   int c_dtype;
   pml_hip_epilogue tail;
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];

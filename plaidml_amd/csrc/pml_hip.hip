@@ -265,6 +265,30 @@ int tail_scale_shift(const pml_hip_epilogue& t, int out_dtype, int mode) {
   return t.n_ops - 1;
 }
 
+// The requantisation chain of an int8 contraction: store? cast f32, mul by a per-column (or single) f32 tensor operand,
+// maxgt immediate, min immediate, round, cast si8.  Fills the kernel arguments that describe it; false: something else.
+bool tail_requant(const pml_hip_epilogue& t, int out_dtype, int c_dtype, int mode, IgemmArgs* g) {
+  if (g) g->tail_rq = 0;
+  if (mode != 4 || out_dtype != PML_HIP_I32 || c_dtype != PML_HIP_I8) return false;
+  const int first = (t.n_ops > 0 && t.ops[0].opcode == PML_HIP_EPI_STORE) ? 1 : 0;
+  if (t.n_ops != first + 6) return false;
+  const pml_hip_epi_op* o = t.ops + first;
+  const bool shape = o[0].opcode == PML_HIP_EPI_CAST && o[0].dtype == PML_HIP_F32 && o[1].opcode == PML_HIP_EPI_MUL &&
+                     o[1].dtype == PML_HIP_F32 && o[1].operand_kind == PML_HIP_OPND_TENSOR && o[2].opcode == PML_HIP_EPI_MAX_GT &&
+                     o[2].dtype == PML_HIP_F32 && o[2].operand_kind == PML_HIP_OPND_IMM && o[3].opcode == PML_HIP_EPI_MIN &&
+                     o[3].dtype == PML_HIP_F32 && o[3].operand_kind == PML_HIP_OPND_IMM && o[4].opcode == PML_HIP_EPI_ROUND &&
+                     o[4].dtype == PML_HIP_F32 && o[5].opcode == PML_HIP_EPI_CAST && o[5].dtype == PML_HIP_I8;
+  if (!shape) return false;
+  if (g) {
+    g->tail_rq = 1;
+    g->rq_store = first ? t.ops[0].operand : -1;
+    g->rq_scale = o[1].operand;
+    g->rq_lo = (float)o[2].imm;
+    g->rq_hi = (float)o[3].imm;
+  }
+  return true;
+}
+
 // allow64: the standalone elementwise kernel also runs 64-bit steps; the tails of the contraction kernels do not
 bool valid_tail(const pml_hip_epilogue& t, bool allow64 = false) {
   if (t.n_ops < 0 || t.n_ops > PML_HIP_MAX_EPI_OPS) return false;
@@ -351,6 +375,7 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.c_dtype = d.c_dtype;
   classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
   g.tail_ssr = tail_scale_shift(d.tail, d.out_dtype, g.tail_mode);
+  tail_requant(d.tail, d.out_dtype, d.c_dtype, g.tail_mode, &g);
   g.tail = d.tail;
   g.NB = (int)d.n;
   g.n_cus = device_cus();
@@ -557,7 +582,7 @@ int pml_hip_gemm_tail_cheaper_apart(const pml_hip_gemm_desc* d) {
   if (kind != KIND_I8) return 0;
   int mode = 0, relu = 0;
   classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
-  if (mode == 1 || mode == 2) return 0;
+  if (mode == 1 || mode == 2 || tail_requant(d->tail, d->out_dtype, d->c_dtype, mode, nullptr)) return 0;
   const int64_t k_bytes = d->k * dt_size(d->in_dtype);
   if (PML_HIP_FLAG_TILE_OF(d->flags) >= 0) return 0;  // a named tile is taken whatever the tail
   return choose_tile(d->m, d->n, k_bytes, kind, true) == TILE_256x256_W8 && choose_tile(d->m, d->n, k_bytes, kind, false) != TILE_256x256_W8;
@@ -574,7 +599,8 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
   {
     int mode = 0, relu = 0;
     classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
-    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, mode == 1 || mode == 2, PML_HIP_FLAG_TILE_OF(d->flags));
+    const bool plain = mode == 1 || mode == 2 || tail_requant(d->tail, d->out_dtype, d->c_dtype, mode, nullptr);
+    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags));
   }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
@@ -692,6 +718,7 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   g.n_cus = device_cus();
   classify_tail(d.tail, d.out_dtype, d.c_dtype, &g.tail_mode, &g.tail_relu);
   g.tail_ssr = tail_scale_shift(d.tail, d.out_dtype, g.tail_mode);
+  tail_requant(d.tail, d.out_dtype, d.c_dtype, g.tail_mode, &g);
   g.tail = d.tail;
   for (int i = 0; i < d.tail.n_operands; ++i) {
     if (!operands || !operands[i]) return fail("gemm_invoke: missing tail operand");
@@ -753,7 +780,8 @@ int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const voi
   }
   int mode = 0, relu = 0;
   classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
-  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, mode == 1 || mode == 2, PML_HIP_FLAG_TILE_OF(d->flags));
+  const bool plain = mode == 1 || mode == 2 || tail_requant(d->tail, d->out_dtype, d->c_dtype, mode, nullptr);
+  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags));
   return gemm_run(*d, kind, tile, bt, d->k, false, a, b, c, init, operands, outs, s);
 }
 

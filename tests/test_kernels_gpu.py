@@ -343,6 +343,52 @@ def test_gemm_i8_requantize_tail():
     np.testing.assert_array_equal(Q, Qo)
 
 
+def _requant_reference(C32, S, lo, hi):
+    """The chain step by step in float32, as the steps are defined: cast, multiply, v > lo ? v : lo, v < hi ? v : hi,
+    round half away from zero, truncate to si32, wrap to si8."""
+    with np.errstate(invalid='ignore', over='ignore'):
+        v = C32.astype(np.float32) * S.astype(np.float32)
+        v = np.where(v > np.float32(lo), v, np.float32(lo))
+        v = np.where(v < np.float32(hi), v, np.float32(hi))
+        r = np.where(v >= 0, np.floor(v + np.float32(0.5)), np.ceil(v - np.float32(0.5)))
+        return r.astype(np.int32).astype(np.int8)
+
+
+@pytest.mark.parametrize('tile', ['64x64', '128x128', '128x128w8s2', '256x128w16', '256x256w8'])
+@pytest.mark.parametrize('store,vector_scale', [(True, True), (False, True), (True, False)])
+def test_gemm_i8_requantisation_chain_as_straight_code(tile, store, vector_scale, monkeypatch, capsys):
+    """The chain a clip-and-round requantisation compiles to -- (store si32)? cast f32, * scale, maxgt lo, min hi, round,
+    cast si8 -- runs as straight code behind the int8 GEMM on every tile, the 256x256 one included: both outputs bit for
+    bit against the steps evaluated one by one in float32.  Scales of 0.5 / 0.25 put many products exactly half way
+    between integers (both signs); one column scale is NaN, one infinite, one negative; a bias is added to the sums."""
+    monkeypatch.setitem(FORCED, 'flags', hk.flag_tile(tile))
+    rng = np.random.default_rng(77)
+    M, N, K = 600, 520, 336
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    A[:40] = rng.integers(-3, 4, (40, K), dtype=np.int8)  # small sums: the clamps do not hide the rounding
+    bias = rng.integers(-50, 50, N, dtype=np.int32)
+    if vector_scale:
+        S = rng.uniform(0.001, 0.01, N).astype(np.float32)
+        S[::7], S[1::7] = 0.5, 0.25
+        S[3], S[11], S[19] = np.nan, np.inf, -0.004
+    else:
+        S = np.array([0.5], np.float32)
+    ops = ([(hk.EPI_STORE, hk.I32, 0, 0, 0.0)] if store else []) + [
+        (hk.EPI_CAST, hk.F32, 0, 0, 0.0), (hk.EPI_MUL, hk.F32, hk.OPND_TENSOR, 0, 0.0),
+        (hk.EPI_MAX_GT, hk.F32, hk.OPND_IMM, 0, -127.0), (hk.EPI_MIN, hk.F32, hk.OPND_IMM, 0, 127.0),
+        (hk.EPI_ROUND, hk.F32, 0, 0, 0.0), (hk.EPI_CAST, hk.I8, 0, 0, 0.0)]
+    tail = hk.make_tail(ops=ops, operands=[(hk.F32, 0, 1 if vector_scale else 0)])
+    got = run_gemm(A, B, hk.I8, hk.I32, init=bias, init_strides=(0, 1), init_dt=hk.I32, tail=tail, operands=[S], c_dt=hk.I8,
+                   extra_out=np.int32 if store else None)
+    assert tile.split('w')[0] in capsys.readouterr().out
+    Q, C = got if store else (got, None)
+    ref = (A.astype(np.int64) @ B.astype(np.int64) + bias).astype(np.int32)
+    if store:
+        np.testing.assert_array_equal(C, ref)
+    np.testing.assert_array_equal(Q, _requant_reference(ref, S if vector_scale else np.full(N, S[0], np.float32), -127.0, 127.0))
+
+
 @pytest.mark.parametrize('M,N,K', [(256, 256, 256), (72, 200, 136)])
 def test_gemm_bf16(M, N, K):
     rng = np.random.default_rng(6)
