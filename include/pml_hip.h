@@ -179,6 +179,8 @@ enum {
   PML_HIP_TILE_64x64_W8_K2,    /* 8 wavefronts as two grids that split every slab's K-blocks */
   PML_HIP_TILE_256x256_W8,     /* 8 wavefronts of 128x64 */
   PML_HIP_TILE_128x64_N2,      /* 4 wavefronts of 32x64 (split fp32 kind only) */
+  PML_HIP_TILE_192x384_W8,     /* 8 wavefronts of 96x96 (bf16 and int8) */
+  PML_HIP_TILE_64x64_KSPLIT,   /* 64x64 tiles whose K loop is shared out among several workgroups, partial tiles added up by a second launch */
   PML_HIP_TILE_COUNT_
 };
 enum {
@@ -364,6 +366,11 @@ typedef struct {
 int64_t pml_hip_dwconv2d_dispatch(const pml_hip_dwconv2d_desc* desc);
 int pml_hip_dwconv2d_invoke(int64_t plan, const void* input, const void* filter, void* output,
                             const void* const* operands, void* const* outs, pml_hip_stream s);
+/* Same as pml_hip_conv2d_pack_filter for a constant depthwise filter: the plan keeps a copy, and invoke may afterwards
+ * be given filter == NULL.  A 3x3 bf16 filter whose weights are all finite is also re-laid for a kernel that multiplies
+ * the taps of two filter rows in one instruction; the weights are looked at here, once, instead of in every launch.
+ * Waits for the stream (the filter is read back to the host). */
+int pml_hip_dwconv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream s);
 
 /* ---- window reduction: 2-D pooling, NHWC --------------------------------------
  * O[n,y,x,c] = agg_{ky<kh,kx<kw} I[n, sy*y + ky - py, sx*x + kx - px, c] over in-range taps

@@ -91,8 +91,13 @@ constexpr int igemm_waves_per_simd() {
 // of a group each name 8 bytes -- here 8 columns of one K-row -- and lane i receives byte i % 8 of the data named
 // by lanes i / 8, i / 8 + 2, ..., i.e. 8 K-values of column i).  The 16-byte chunks of K-row k are stored at
 // positions XORed with k % 8 so that the 8 rows of such a read fall into different banks.
+// SPLITK: the K loop of a tile is shared out among p.sk_splits workgroups (workgroup id = split x tiles + tile), each
+// of which multiplies p.sk_per consecutive slabs and leaves its partial tile, untouched by any tail, in the workspace
+// p.ws[split][M][sk_pitch]; splitk_reduce_kernel below adds the parts up and runs the tail.  For problems with few
+// tiles and a long K (the 3x3 convolutions of a network's last stages at batch 1: 8 tiles of 72 slabs), which would
+// otherwise leave most of the chip idle for the length of one long serial loop.
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int SLAB = 128,
-          bool BKN = false>
+          bool BKN = false, bool SPLITK = false>
 __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>())) void igemm_kernel(IgemmArgs p_by_value) {
   // The argument block is read where the dispatcher put it (the kernel-argument segment, scalar loads),
   // through a reference: taking the by-value parameter's address instead makes the compiler copy all of
@@ -142,7 +147,14 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   const int wm = (wave % (WAVES_M * WAVES_N)) / WAVES_N, wn = wave % WAVES_N;
 
   int tile_m, tile_n;
-  tile_of(p.order, blockIdx.x, &tile_m, &tile_n);
+  unsigned tile_id = blockIdx.x;
+  int split = 0;
+  if constexpr (SPLITK) {
+    static_assert(WAVES_K == 1 && !BKN, "the split over workgroups stands alone");
+    split = (int)(tile_id / (unsigned)p.sk_tiles);
+    tile_id -= (unsigned)split * (unsigned)p.sk_tiles;
+  }
+  tile_of(p.order, tile_id, &tile_m, &tile_n);
   const int64_t m0 = (int64_t)tile_m * BM;
   const int64_t n0 = (int64_t)tile_n * BN;
 
@@ -257,6 +269,23 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   bool req_second = false;        // GEMM: the slab belongs to the second product
   int nx_kh = 0, nx_kw = 0, nx_cs = 0, nx_dh = 0, nx_dw = 0, nx_tap = 0;  // CONV: tap and slab-in-tap of the next slab
   int nx_kbo = 0;                                                          // GEMM: its first byte of K
+  int slab_count = n_slabs;  // slabs this workgroup multiplies
+  if constexpr (SPLITK) {
+    // this workgroup's run of slabs: the counters start where slab `first` begins
+    const int first = split * p.sk_per;
+    slab_count = n_slabs - first < p.sk_per ? n_slabs - first : p.sk_per;
+    if (CONV) {
+      const int tap = first / slabs_per_tap;
+      nx_cs = first - tap * slabs_per_tap;
+      nx_kh = tap / cKW;
+      nx_kw = tap - nx_kh * cKW;
+      nx_tap = tap * pix_bytes;
+      nx_dh = nx_kh * cDH;
+      nx_dw = nx_kw * cDW;
+    } else {
+      nx_kbo = first * kSlabBytes;
+    }
+  }
   auto prepare_slab = [&](int stage) {
     req_base = smem + stage * kStage + wave * 1024;  // one request of a wavefront fills 1 KB
     if (CONV) {
@@ -317,10 +346,10 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
 
   // a residual tensor of the tail is requested now, so that it arrives under the K loop
   TailPrefetch<KIND, BM, BN, NT> pre;
-  const bool direct = WAVES_K == 1 && direct_tail_ok<KIND>(p, n0, BN);
+  const bool direct = !SPLITK && WAVES_K == 1 && direct_tail_ok<KIND>(p, n0, BN);
 
   pre.valid = false;
-  if (!direct) tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
+  if (!direct && !SPLITK) tail_prefetch<KIND, BM, BN, NT>(p, m0, n0, tid, pre);
   // The direct tail reads its residual rows only after the K loop.  One 4-byte load per lane and 32x32 block,
   // issued here and landing in the dump area of LDS, brings the 64 bytes a row contributes to the block into the
   // caches: a short-K GEMM then waits for operands and residual together instead of one after the other.
@@ -436,7 +465,7 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
   for (int j = 0; j < NI; ++j) fb[0][j] = read_b(b_base, j, fslot_b[0]);
 
   int stage = 0;  // ring stage of slab s
-  for (int s = 0; s < n_slabs; ++s) {
+  for (int s = 0; s < slab_count; ++s) {
     int next_stage = stage + 1;
     if (next_stage == kStages) next_stage = 0;
     const unsigned char* a_next = smem + next_stage * kStage + (wm * WM + frow) * kSlabBytes;
@@ -544,6 +573,18 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
             }
       }
       __syncthreads();
+    }
+    if constexpr (SPLITK) {
+      // the partial tile as it is: four columns per thread, rows of the workspace are whole 16-byte vectors
+      constexpr int TPR = BN / 4, RPP = NT / TPR;
+      const int c4 = (tid % TPR) * 4;
+      accs_t* const ws = (accs_t*)p.ws + (int64_t)split * p.M * p.sk_pitch;
+      if (n0 + c4 < p.sk_pitch) {
+#pragma unroll
+        for (int row = tid / TPR; row < BM; row += RPP)
+          if (m0 + row < p.M) *(acc4_t*)&ws[(m0 + row) * p.sk_pitch + n0 + c4] = *(const acc4_t*)&ctile[row * CS + c4];
+      }
+      return;
     }
     tile_tail<KIND, BM, BN, NT>(p, ctile, m0, n0, tid, &pre);
   } else {
@@ -660,9 +701,62 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
   }
 }
 
+// Second pass of a K split over workgroups: a workgroup per 64 x 64 result tile adds the partial tiles in split order
+// (int32: exact whatever the order) into the same LDS layout the one-pass kernel stages its accumulators in, and runs
+// the same tail code over it.
+template <int KIND>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(IgemmArgs p_by_value) {
+  const IgemmArgs& p = *(const IgemmArgs*)(const __attribute__((address_space(4))) void*)__builtin_amdgcn_kernarg_segment_ptr();
+  typedef typename Acc<KIND>::scalar accs_t;
+  typedef accs_t acc4_t __attribute__((ext_vector_type(4)));
+  constexpr int CS = 64 + 4;
+  __shared__ __attribute__((aligned(16))) accs_t ctile[64 * CS];
+  const int tid = threadIdx.x;
+  int tile_m, tile_n;
+  tile_of(p.order, blockIdx.x, &tile_m, &tile_n);
+  const int64_t m0 = (int64_t)tile_m * 64, n0 = (int64_t)tile_n * 64;
+  const int c4 = (tid & 15) * 4;
+  const accs_t* const ws = (const accs_t*)p.ws;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = (tid >> 4) + 16 * i;
+    acc4_t sum = {0, 0, 0, 0};
+    if (m0 + row < p.M && n0 + c4 < p.sk_pitch) {
+      const accs_t* at = ws + (m0 + row) * p.sk_pitch + n0 + c4;
+      for (int sp = 0; sp < p.sk_splits; ++sp) sum += *(const acc4_t*)(at + (int64_t)sp * p.M * p.sk_pitch);
+    }
+    *(acc4_t*)&ctile[row * CS + c4] = sum;
+  }
+  __syncthreads();
+  tile_tail<KIND, 64, 64, 256>(p, ctile, m0, n0, tid);
+}
+
+// The two launches of a 64 x 64 tiling whose K loop is split over workgroups (a.ws, a.sk_* prepared by the caller).
+template <int KIND, bool CONV>
+hipError_t launch_splitk(const IgemmArgs& a, hipStream_t s) {
+  if constexpr (KIND == KIND_F32X3P) {
+    return hipErrorInvalidValue;
+  } else {
+    const int64_t tiles_m = (a.M + 63) / 64, tiles_n = (a.N + 63) / 64;
+    const int64_t tiles = tiles_m * tiles_n;
+    if (tiles <= 0 || tiles * a.sk_splits >= ((int64_t)1 << 31) || a.K2 > 0 || a.b_kn || !a.ws || a.sk_splits < 2) return hipErrorInvalidValue;
+    const size_t lds = Ring<64, 64, 0, 128>::kAlloc;
+    auto kern = igemm_kernel<KIND, 64, 64, 2, CONV, kThreads, 0, 1, 128, false, true>;
+    static DynamicLdsLimit limit;
+    if (hipError_t e = limit.ensure((const void*)kern, lds); e != hipSuccess) return e;
+    IgemmArgs b = a;
+    b.order = make_tile_order((int)tiles_m, (int)tiles_n);
+    b.sk_tiles = (int)tiles;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * a.sk_splits)), dim3(kThreads), lds, s, b);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)tiles), dim3(256), 0, s, b);
+    return hipGetLastError();
+  }
+}
+
 template <int KIND, int BM, int BN, int WAVES_M, bool CONV, int NT = kThreads, int STAGES = 0, int WAVES_K = 1, int SLAB = 128>
 hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
-  if constexpr ((KIND == KIND_F32 || KIND == KIND_F32X3 || KIND == KIND_I8) && !CONV && SLAB == 128) {
+  if constexpr ((KIND == KIND_F32 || KIND == KIND_F32X3 || KIND == KIND_I8) && !CONV && SLAB == 128 && (BN & (BN - 1)) == 0) {
     if (a.b_kn) {
       const int64_t tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
       const int64_t tiles = tiles_m * tiles_n;
@@ -695,6 +789,9 @@ hipError_t launch_cfg(const IgemmArgs& a, hipStream_t s) {
 template <int KIND, bool CONV>
 hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
   switch (cfg) {
+    case TILE_64x64_KSPLIT:
+      if (a.ws && a.sk_splits >= 2) return launch_splitk<KIND, CONV>(a, s);
+      return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);  // (nothing to split, or no workspace: the plain tile)
     case TILE_64x64: return launch_cfg<KIND, 64, 64, 2, CONV>(a, s);
     case TILE_128x64: return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
     case TILE_128x128: return launch_cfg<KIND, 128, 128, 2, CONV>(a, s);
@@ -715,6 +812,14 @@ hipError_t launch_kind(int cfg, const IgemmArgs& a, hipStream_t s) {
         return launch_cfg<KIND, 128, 64, 4, CONV>(a, s);
       } else {
         return launch_cfg<KIND, 128, 64, 2, CONV>(a, s);
+      }
+    case TILE_192x384_W8:
+      // eight wavefronts of 96 x 96 (2 x 4): per MFMA half the global -> LDS bytes of a 128 x 128 tile and 0.67 KB of
+      // fragment reads; 144 accumulation registers per lane, so 16- and 8-bit elements only
+      if constexpr (KIND == KIND_BF16 || KIND == KIND_I8) {
+        return launch_cfg<KIND, 192, 384, 2, CONV, 512, 2>(a, s);
+      } else {
+        return launch_cfg<KIND, 128, 128, 2, CONV, 512>(a, s);
       }
     case TILE_256x128_W16:
     case TILE_256x256_W8:

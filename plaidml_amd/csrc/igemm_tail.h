@@ -197,7 +197,22 @@ __device__ __forceinline__ i32x4_t pack_bf16x8(const float* v) {
   return o;
 }
 
+// The value of a float after it has been rounded to bf16 (round to nearest even) -- two at a time.
+__device__ __forceinline__ void round_pair_to_bf16(float& x, float& y) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 h = __builtin_convertvector(f32x2{x, y}, bf16x2);
+  uint32_t w;
+  __builtin_memcpy(&w, &h, 4);
+  x = __uint_as_float(w << 16);
+  y = __uint_as_float(w & 0xffff0000u);
+}
+
 // mw, nw: first row / column of the wavefront's MI x NI blocks.
+// What a result costs here is vector instructions (a 96 x 96 wavefront tile holds 144 results per lane), so: the
+// per-column vectors (bias, scale, shift) are unpacked once per column block, not once per row block; a step whose
+// operand is absent is not computed at all (uniform branches); relu is one NaN-keeping maximum; and the eight lane
+// exchanges of a 32 x 32 block sit in one run with one pair of idle cycles around it instead of one pair each.
 template <int MI, int NI>
 __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&acc)[MI][NI], int64_t mw, int64_t nw, int lane) {
   const int hi = lane >> 5;
@@ -207,6 +222,8 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
   const uint16_t* const scale = scale_shift ? (const uint16_t*)p.operands[p.tail.ops[0].operand] : nullptr;
   const uint16_t* const shift = scale_shift ? (const uint16_t*)p.operands[p.tail.ops[1].operand] : nullptr;
   const bool relu = scale_shift ? p.tail_ssr == 2 : p.tail_relu != 0;
+  const float lo = relu ? 0.f : -__builtin_inff();  // relu as a lower clamp (the IEEE maximum keeps a NaN)
+  const bool has_bias = p.init != nullptr || p.init2 != nullptr;
   // the last MFMAs must have written the accumulators before the lane exchange below reads them: the compiler
   // cannot see that read (it is assembler text), so the longest MFMA's passes are waited out here, once
   asm volatile("s_nop 15\n\ts_nop 3");
@@ -216,21 +233,28 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
     bool col_ok[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) col_ok[q] = nw + j * 32 + 16 * q + 8 * hi < p.N;
-    i32x4_t bias_bits[2];  // kept packed: registers are the scarce thing here
+    auto column_vector = [&](const uint16_t* src, int q, float* out) {
+      const i32x4_t bits = (src != nullptr && col_ok[q]) ? *(const i32x4_t*)(src + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+      unpack_bf16x8(bits, out);
+    };
+    float bias[2][8], mul[2][8], add[2][8];
+    if (has_bias) {
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
-      bias_bits[q] = (p.init != nullptr && col_ok[q]) ? *(const i32x4_t*)((const uint16_t*)p.init + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
-    // the second product's bias, or the scale vector of a scale / shift chain (which excludes a second product)
-    i32x4_t second_bits[2];
+      for (int q = 0; q < 2; ++q) {
+        float second[8];
+        column_vector((const uint16_t*)p.init, q, bias[q]);
+        column_vector((const uint16_t*)p.init2, q, second);
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const uint16_t* src = scale_shift ? scale : (const uint16_t*)p.init2;
-      second_bits[q] = (src != nullptr && col_ok[q]) ? *(const i32x4_t*)(src + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+        for (int e = 0; e < 8; ++e) bias[q][e] += second[e];
+      }
     }
-    i32x4_t shift_bits[2];
+    if (scale_shift) {
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
-      shift_bits[q] = (scale_shift && col_ok[q]) ? *(const i32x4_t*)(shift + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
+      for (int q = 0; q < 2; ++q) {
+        column_vector(scale, q, mul[q]);
+        column_vector(shift, q, add[q]);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int64_t m = mw + i * 32 + (lane & 31);
@@ -241,50 +265,51 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
         for (int q = 0; q < 2; ++q)
           if (col_ok[q]) res[q] = *(const i32x4_t*)((const uint16_t*)p.operands[0] + m * rs + nw + j * 32 + 16 * q + 8 * hi);
       }
+      // The lane holds columns 8 g + 4 hi + e (g = 0..3, e = 0..3) of its row.  Exchanging group 2 q + 1 of the lower
+      // half wavefront with group 2 q of the upper one leaves lanes 0..31 with group 2 q whole (8 columns) and lanes
+      // 32..63 with group 2 q + 1.  The exchange works on the accumulator registers themselves (the builtin made the
+      // compiler copy all accumulators first), as one piece of assembler text: the compiler does not see through it,
+      // so the idle cycles the instruction needs after a vector write of its operands and before a vector read of its
+      // results are spelled out, once for the eight exchanges.
+      f32x16_t& c = acc[i][j];
+      asm volatile(
+          "s_nop 1\n\t"
+          "v_permlane32_swap_b32 %0, %4\n\tv_permlane32_swap_b32 %1, %5\n\tv_permlane32_swap_b32 %2, %6\n\tv_permlane32_swap_b32 %3, %7\n\t"
+          "v_permlane32_swap_b32 %8, %12\n\tv_permlane32_swap_b32 %9, %13\n\tv_permlane32_swap_b32 %10, %14\n\tv_permlane32_swap_b32 %11, %15\n\t"
+          "s_nop 1"
+          : "+v"(c[0]), "+v"(c[1]), "+v"(c[2]), "+v"(c[3]), "+v"(c[4]), "+v"(c[5]), "+v"(c[6]), "+v"(c[7]), "+v"(c[8]), "+v"(c[9]),
+            "+v"(c[10]), "+v"(c[11]), "+v"(c[12]), "+v"(c[13]), "+v"(c[14]), "+v"(c[15]));
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        float v[8], bias[8], second[8];
-        unpack_bf16x8(bias_bits[q], bias);
-        unpack_bf16x8(second_bits[q], second);
-        if (!scale_shift) {
+        float v[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) bias[e] += second[e];
-        }
+        for (int e = 0; e < 8; ++e) v[e] = c[8 * q + e];
+        if (has_bias) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // x: group 2q, y: group 2q + 1; afterwards lanes 0..31 hold group 2q whole, lanes 32..63 group 2q + 1.
-          // (As an instruction on the accumulator registers themselves: the builtin made the compiler copy all
-          // accumulators first, which cost the second workgroup of a CU its registers.)
-          float x = acc[i][j][4 * (2 * q) + e], y = acc[i][j][4 * (2 * q + 1) + e];
-          // (the waits: the compiler does not see through the text, so it cannot insert the idle cycles this
-          // instruction needs after a vector write of its operands and before a vector read of its results)
-          asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-          v[e] = x + bias[e];
-          v[4 + e] = y + bias[4 + e];
+          for (int e = 0; e < 8; ++e) v[e] += bias[q][e];
         }
         if (residual) {
           // the contraction result is rounded first, then the bf16 addition rounds again
-          float c[8], r[8];
-          unpack_bf16x8(pack_bf16x8(v), c);
+          float r[8];
           unpack_bf16x8(res[q], r);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = c[e] + r[e];
+          for (int e = 0; e < 8; e += 2) round_pair_to_bf16(v[e], v[e + 1]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += r[e];
         }
         if (scale_shift) {
           // three roundings: the contraction result, the product, the sum
-          float c[8], sh[8];
-          unpack_bf16x8(pack_bf16x8(v), c);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = c[e] * second[e];
-          unpack_bf16x8(pack_bf16x8(v), c);
-          unpack_bf16x8(shift_bits[q], sh);
+          for (int e = 0; e < 8; e += 2) round_pair_to_bf16(v[e], v[e + 1]);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = c[e] + sh[e];
+          for (int e = 0; e < 8; ++e) v[e] *= mul[q][e];
+#pragma unroll
+          for (int e = 0; e < 8; e += 2) round_pair_to_bf16(v[e], v[e + 1]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += add[q][e];
         }
-        if (relu) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = v[e] < 0.f ? 0.f : v[e];
-        }
+        for (int e = 0; e < 8; ++e) v[e] = __builtin_elementwise_maximum(v[e], lo);
         if (row_ok && col_ok[q]) *(i32x4_t*)((uint16_t*)p.C + m * p.ldc + nw + j * 32 + 16 * q + 8 * hi) = pack_bf16x8(v);
       }
     }

@@ -39,7 +39,8 @@ enum { KIND_F32 = 0, KIND_BF16 = 1, KIND_I8 = 2, KIND_F32X3 = 3, KIND_F32X3P = 4
 // _W8 / _W16: eight / sixteen wavefronts per workgroup (two / four per SIMD) instead of four; _S2: two ring stages; _K2: two wavefront grids share the K-blocks of every slab
 enum { TILE_64x64 = PML_HIP_TILE_64x64, TILE_128x64 = PML_HIP_TILE_128x64, TILE_128x128 = PML_HIP_TILE_128x128, TILE_128x64_W8 = PML_HIP_TILE_128x64_W8,
        TILE_128x128_W8 = PML_HIP_TILE_128x128_W8, TILE_256x128_W16 = PML_HIP_TILE_256x128_W16, TILE_128x128_W8_S2 = PML_HIP_TILE_128x128_W8_S2,
-       TILE_64x64_W8_K2 = PML_HIP_TILE_64x64_W8_K2, TILE_256x256_W8 = PML_HIP_TILE_256x256_W8, TILE_128x64_N2 = PML_HIP_TILE_128x64_N2 };
+       TILE_64x64_W8_K2 = PML_HIP_TILE_64x64_W8_K2, TILE_256x256_W8 = PML_HIP_TILE_256x256_W8, TILE_128x64_N2 = PML_HIP_TILE_128x64_N2,
+       TILE_192x384_W8 = PML_HIP_TILE_192x384_W8, TILE_64x64_KSPLIT = PML_HIP_TILE_64x64_KSPLIT };
 
 struct TailPtrs {
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
@@ -177,6 +178,10 @@ struct IgemmArgs {
   // (v < hi ? v : hi), round half away from zero, cast si8 -- which the tail then runs as straight code
   int tail_rq, rq_store, rq_scale;
   float rq_lo, rq_hi;
+  // K split over workgroups (TILE_64x64_KSPLIT): the workspace of partial tiles [sk_splits][M][sk_pitch] (accumulator
+  // type), slabs per split, and -- filled in by the launcher -- the number of result tiles
+  void* ws;
+  int sk_splits, sk_per, sk_pitch, sk_tiles;
   int c_dtype;
   pml_hip_epilogue tail;
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
@@ -195,6 +200,25 @@ struct IgemmArgs {
 };
 
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
+// How TILE_64x64_KSPLIT shares the K loop out: slabs of 128 bytes of K in all, and for a device of n_cus compute units
+// the number of splits (1: not worth splitting) with the slabs each takes -- about two workgroups per CU, at least two
+// slabs per split, at most 32 splits.
+inline int64_t igemm_slabs(const IgemmArgs& a, bool conv, int es) {
+  return conv ? (int64_t)a.KH * a.KW * (((int64_t)a.CI * es + 127) / 128) : (a.K * es + 127) / 128;
+}
+inline void igemm_split_plan(int64_t m, int64_t n, int64_t slabs, int n_cus, int* splits, int* per) {
+  const int64_t tiles = ((m + 63) / 64) * ((n + 63) / 64);
+  int64_t want = tiles > 0 ? (2 * (int64_t)n_cus + tiles - 1) / tiles : 1;
+  if (want > 32) want = 32;
+  if (want > slabs / 2) want = slabs / 2;
+  if (want < 2) {
+    *splits = 1;
+    *per = (int)slabs;
+    return;
+  }
+  *per = (int)((slabs + want - 1) / want);
+  *splits = (int)((slabs + *per - 1) / *per);  // every split has work
+}
 // Resident-filter convolution (conv_halo.hip): LDS bytes a shape needs, or 0 when the
 // shape does not qualify; `a.halo_rows` and `a.n_tiles` are filled in by conv_halo_prepare.
 size_t conv_halo_prepare(int kind, IgemmArgs* a, bool filter_in_lds = false);
@@ -252,8 +276,13 @@ struct DwconvArgs {
   void* out;
   const void* operands[PML_HIP_MAX_EPI_OPERANDS];
   void* outs[PML_HIP_MAX_EPI_OPERANDS];
+  // a 3x3 bf16 filter of finite weights packed once with the taps of rows 0 and 1 paired (dwconv2d_pair_filter), or null
+  const void* paired_filter;
+  int n_cus;  // compute units of the device (the paired kernel sizes its grid by it)
 };
 hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s);
+bool dwconv2d_takes_paired_filter(const pml_hip_dwconv2d_desc& d);
+bool dwconv2d_pair_filter(const uint16_t* filter, int64_t c, uint32_t* packed);
 struct Im2colArgs {
   const void* in;
   void* out;

@@ -9,6 +9,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "device_common.h"
 #include "plans.h"
@@ -60,6 +61,13 @@ struct Plan {
   void* s2d = nullptr;
   std::mutex s2d_mutex;
   int s2d_h = 0, s2d_w = 0, s2d_ch = 0, s2d_ka = 0, s2d_kaw = 0;
+  // depthwise convolution: a constant filter kept by the plan ([kh][kw][c] as the caller holds it), and its paired
+  // form for the 3x3 bf16 kernel when every weight is finite
+  void* dw_filter = nullptr;
+  void* dw_paired = nullptr;
+  // K split over workgroups: workspace of partial tiles and how the slabs are shared out (splits < 2: no split)
+  void* ws = nullptr;
+  int sk_splits = 0, sk_per = 0, sk_pitch = 0;
   // register-filter convolution: a filter packed once, in the order the kernel holds it in registers
   void* reg_image = nullptr;
   // resident-filter convolution: LDS bytes (0 = not used), window rows, tile count, CUs of the device
@@ -72,6 +80,9 @@ struct Plan {
     if (patches) (void)hipFree(patches);
     if (s2d) (void)hipFree(s2d);
     if (reg_image) (void)hipFree(reg_image);
+    if (ws) (void)hipFree(ws);
+    if (dw_filter) (void)hipFree(dw_filter);
+    if (dw_paired) (void)hipFree(dw_paired);
   }
 };
 
@@ -96,6 +107,8 @@ const char* tile_name(int t) {
     case TILE_256x256_W8: return "256x256 (8 wavefronts of 128x64)";
     case TILE_128x64_N2: return "128x64 (4 wavefronts of 32x64)";
     case TILE_128x128_W8_S2: return "128x128 (8 wavefronts, 2 stages)";
+    case TILE_192x384_W8: return "192x384 (8 wavefronts of 96x96)";
+    case TILE_64x64_KSPLIT: return "64x64, K split over workgroups";
   }
   return "?";
 }
@@ -104,7 +117,7 @@ constexpr int kScheduleBits = 0xff << 8 | 0xf << 16;
 bool schedule_bits_ok(int flags) {
   return PML_HIP_FLAG_TILE_OF(flags) < PML_HIP_TILE_COUNT_ && PML_HIP_FLAG_CONV_OF(flags) <= PML_HIP_CONV_BLOCKS;
 }
-const char* const kTileShort[PML_HIP_TILE_COUNT_] = {"64x64", "128x64", "128x128", "128x64w8", "128x128w8", "256x128w16", "128x128w8s2", "64x64w8k2", "256x256w8", "128x64n2"};
+const char* const kTileShort[PML_HIP_TILE_COUNT_] = {"64x64", "128x64", "128x128", "128x64w8", "128x128w8", "256x128w16", "128x128w8s2", "64x64w8k2", "256x256w8", "128x64n2", "192x384w8", "64x64ks"};
 
 // Stated tiling choice per shape class.  Measured on MI355X, bf16 unless said otherwise (us; w8 / w16 =
 // 8 / 16 wavefronts per workgroup; s2 = two ring stages and LDS cut to what the result tile needs, so that two
@@ -133,9 +146,14 @@ const char* const kTileShort[PML_HIP_TILE_COUNT_] = {"64x64", "128x64", "128x128
 // that; and for small problems the smaller of 64x64 and 128x64 by (rounds of resident workgroups) x
 // (tile area), the larger tile on a tie.
 // forced: a tile named by the descriptor's schedule bits (PML_HIP_FLAG_TILE), -1 = none
-int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, bool plain_tail = true, int forced = -1) {
-  if (forced >= 0 && forced < PML_HIP_TILE_COUNT_ && (forced != TILE_128x64_N2 || kind == KIND_F32X3)) return forced;
+int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, bool plain_tail = true, int forced = -1, bool allow_split = true) {
+  if (forced >= 0 && forced < PML_HIP_TILE_COUNT_ && (forced != TILE_128x64_N2 || kind == KIND_F32X3) &&
+      (forced != TILE_192x384_W8 || kind == KIND_BF16 || kind == KIND_I8))
+    return forced;
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+  // Few tiles and a long K (a network's last stages at batch 1: 49 x 512 x 4608 is 8 tiles of 72 slabs): the K loop is
+  // shared out among workgroups and a second launch adds the partial tiles up.  Measured inside ResNet-50 at batch 1.
+  if (allow_split && tiles(64, 64) <= 64 && k_bytes >= 1024) return TILE_64x64_KSPLIT;
   if (kind == KIND_F32X3) {
     // A fragment that is split in registers costs 24 vector instructions whatever it is multiplied with, so the
     // tile a wavefront holds decides how many MFMAs share that cost -- but the problems this kind meets here are
@@ -153,6 +171,14 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, boo
   // 16 KB share of LDS in four rounds, 4096^3 int8 with that tail 132 us against 106 with 256x128.)
   if (kind != KIND_F32 && plain_tail && k_bytes >= 2048 && tiles(256, 256) >= 192 && tiles(256, 256) * 65536 * 10 <= m * n * 11)
     return TILE_256x256_W8;
+  // Eight wavefronts of 96 x 96 on a 192 x 384 tile: per MFMA half the global -> LDS bytes of a 128 x 128 tile (the vector
+  // memory path moves 64 bytes per clock and CU, which 128 x 128 tiles use up entirely) and 0.67 KB of fragment reads.
+  // One workgroup per CU, so its tail is not hidden by a neighbour: it pays where the K loop is most of the work, the
+  // columns fill whole tiles and the tiles fill a round of the chip -- 23104 x 728 x 728 (242 tiles) 39 us against 48.
+  if (kind != KIND_F32 && kind != KIND_F32X3 && k_bytes >= 1024) {
+    const int64_t tn = (n + 383) / 384, t = tiles(192, 384);
+    if (tn * 384 * 100 <= n * 108 && ((t >= 200 && t <= 256) || t >= 640)) return TILE_192x384_W8;
+  }
   if (k_bytes >= 4096 && tiles(256, 128) >= 512) return TILE_256x128_W16;
   if (tiles(128, 128) >= 256) return TILE_128x128_W8_S2;
   if (tiles(128, 128) >= 128) return TILE_128x128_W8;
@@ -339,6 +365,29 @@ void* scratch_of_current_device() {
     g_scratch_ptr[dev] = ptr;
   }
   return g_scratch_ptr[dev];
+}
+
+// A plan whose tile is TILE_64x64_KSPLIT: decides the split for m x n results over `slabs` slabs of K and allocates the
+// workspace.  Leaves the plan unsplit (the plain 64 x 64 tile runs) when a split is not worth it or memory is short.
+void prepare_split(Plan* p, int64_t m, int64_t n, int64_t slabs) {
+  if (p->tile != TILE_64x64_KSPLIT) return;
+  int splits = 1, per = 0;
+  igemm_split_plan(m, n, slabs, device_cus(), &splits, &per);
+  if (splits < 2) return;
+  const int64_t pitch = (n + 3) / 4 * 4;
+  if (pitch >= ((int64_t)1 << 31) || hipMalloc(&p->ws, (size_t)splits * m * pitch * 4) != hipSuccess) {
+    p->ws = nullptr;
+    return;
+  }
+  p->sk_splits = splits;
+  p->sk_per = per;
+  p->sk_pitch = (int)pitch;
+}
+void split_args(const Plan* p, IgemmArgs& g) {
+  g.ws = p->ws;
+  g.sk_splits = p->ws ? p->sk_splits : 0;
+  g.sk_per = p->sk_per;
+  g.sk_pitch = p->sk_pitch;
 }
 
 // Everything of the kernel arguments that the descriptor fixes (no operand pointers).
@@ -600,11 +649,13 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
     int mode = 0, relu = 0;
     classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
     const bool plain = mode == 1 || mode == 2 || tail_requant(d->tail, d->out_dtype, d->c_dtype, mode, nullptr);
-    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags));
+    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags), /*allow_split=*/d->k2 == 0);
+    if (d->k2 == 0) prepare_split(p, d->m, d->n, (d->k * dt_size(d->in_dtype) + 127) / 128);
   }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;
-  p->b_split = kind == KIND_F32X3 && !d->b_layout && d->k % 32 == 0;
+  if (p->tile == TILE_64x64_KSPLIT && !p->ws) p->tile = TILE_64x64;  // (not worth splitting, or no memory for the workspace)
+  p->b_split = kind == KIND_F32X3 && !d->b_layout && d->k % 32 == 0 && !p->ws;
   if (!d->b_layout && hipMalloc(&p->bt, p->bt_bytes) != hipSuccess) {
     delete p;
     fail("gemm: cannot allocate the packed right-hand side");
@@ -638,8 +689,10 @@ struct SecondProduct {
 // An fp32 or int8 right-hand side that arrives with the call in its row-major [K][N] form is read as it is (the
 // fp32 kinds gather their K-values from [k][n] slabs, int8 reads them with transposing LDS reads); everything else
 // is transposed into Bt[N][K] first.  Rows must be whole 16-byte vectors.
-static bool reads_b_as_given(const pml_hip_gemm_desc& d, int mfma_kind, const void* b) {
+static bool reads_b_as_given(const pml_hip_gemm_desc& d, int mfma_kind, const void* b, int tile) {
   if (mfma_kind != KIND_F32 && mfma_kind != KIND_F32X3 && mfma_kind != KIND_I8) return false;
+  if (tile == TILE_64x64_KSPLIT) return false;  // (the split kernel reads Bt)
+  if (tile == TILE_192x384_W8) return false;  // (24 chunks per row: the position swizzle of the [k][n] form needs a power of two)
   const int64_t es = mfma_kind == KIND_I8 ? 1 : 4, v = 16 / es;
   if (!(b && !d.b_layout && d.k2 == 0 && d.n % v == 0 && d.ldb % v == 0 && ((uintptr_t)b & 15) == 0 &&
         d.k * d.ldb * es < ((int64_t)1 << 31)))
@@ -658,7 +711,8 @@ static bool reads_b_as_given(const pml_hip_gemm_desc& d, int mfma_kind, const vo
 
 static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* bt, int64_t bt_ld, bool packed,
                     const void* a, const void* b, void* c, const void* init, const void* const* operands,
-                    void* const* outs, pml_hip_stream s, const SecondProduct* second = nullptr, bool bt_is_split = false) {
+                    void* const* outs, pml_hip_stream s, const SecondProduct* second = nullptr, bool bt_is_split = false,
+                    const Plan* split_plan = nullptr) {
   // (a right-hand side that arrives with the call is transposed per run and split in the kernel's registers: a
   // second small launch costs more than it saves; one packed once is kept split)
   const bool b_split = bt_is_split && !b;
@@ -668,7 +722,7 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   if (((uintptr_t)a & 15) != 0) return fail("gemm_invoke: A must be 16-byte aligned");
   if (d.init_kind && !init) return fail("gemm_invoke: the plan expects an initial value");
   const int es = dt_size(d.in_dtype);
-  const bool b_as_given = reads_b_as_given(d, mfma_kind, b);
+  const bool b_as_given = reads_b_as_given(d, mfma_kind, b, tile);
   if (b && !d.b_layout && !b_as_given && check(transpose_pack(es, b, bt, d.k, d.n, d.ldb, bt_ld, (hipStream_t)s), "transpose_pack"))
     return 1;
   if (d.k2 > 0) {
@@ -736,6 +790,7 @@ static int gemm_run(const pml_hip_gemm_desc& d, int mfma_kind, int tile, void* b
   for (int i = 0; i < d.tail.n_ops; ++i)
     if (d.tail.ops[i].opcode == PML_HIP_EPI_STORE && !g.outs[d.tail.ops[i].operand])
       return fail("gemm_invoke: missing extra output");
+  if (split_plan && !b_split) split_args(split_plan, g);  // (the K split over workgroups is not built for a right-hand side packed split)
   return check(igemm_launch(b_split ? KIND_F32X3P : mfma_kind, tile, false, g, (hipStream_t)s), "igemm_launch");
 }
 
@@ -745,8 +800,8 @@ int pml_hip_gemm_invoke(int64_t plan, const void* a, const void* b, void* c, con
   if (!p || p->kind != PLAN_GEMM) return fail("gemm_invoke: not a gemm plan");
   const bool split = p->bt_is_split;
   // a right-hand side that this run transposes overwrites the packed copy
-  if (b && !p->gemm.b_layout && !reads_b_as_given(p->gemm, p->mfma_kind, b)) p->bt_is_split = false;
-  return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s, nullptr, split);
+  if (b && !p->gemm.b_layout && !reads_b_as_given(p->gemm, p->mfma_kind, b, p->tile)) p->bt_is_split = false;
+  return gemm_run(p->gemm, p->mfma_kind, p->tile, p->bt, p->bt_ld, p->packed, a, b, c, init, operands, outs, s, nullptr, split, p);
 }
 
 int pml_hip_gemm_invoke2(int64_t plan, const void* a, const void* b, void* c, const void* init, const void* a2, const void* b2,
@@ -781,7 +836,8 @@ int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const voi
   int mode = 0, relu = 0;
   classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
   const bool plain = mode == 1 || mode == 2 || tail_requant(d->tail, d->out_dtype, d->c_dtype, mode, nullptr);
-  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags));
+  // (no workspace may be allocated here: the K loop is never split over workgroups)
+  const int tile = choose_tile(d->m, d->n, d->k * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags), /*allow_split=*/false);
   return gemm_run(*d, kind, tile, bt, d->k, false, a, b, c, init, operands, outs, s);
 }
 
@@ -847,7 +903,7 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     p->s2d_ka = (int)(d->kh + (d->pad_h & 1) + 1) / 2;
     p->s2d_kaw = (int)(d->kw + (d->pad_w & 1) + 1) / 2;
     const int64_t k2 = (int64_t)p->s2d_ka * p->s2d_kaw * p->s2d_ch;
-    p->tile = choose_tile(M, d->co, k2 * es, kind, false, PML_HIP_FLAG_TILE_OF(d->flags));
+    p->tile = choose_tile(M, d->co, k2 * es, kind, false, PML_HIP_FLAG_TILE_OF(d->flags), /*allow_split=*/false);
     p->bt_ld = k2;
     p->via_s2d = true;
   }
@@ -862,8 +918,10 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
       return 0;
     }
   }
+  if (!via_s2d && !via_patches) prepare_split(p, M, d->co, d->kh * d->kw * ((d->ci * es + 127) / 128));
+  if (p->tile == TILE_64x64_KSPLIT && !p->ws) p->tile = TILE_64x64;
   // (whole 128-byte chunks per filter tap, so that no chunk of heads + remainders straddles two taps)
-  p->b_split = kind == KIND_F32X3 && !via_s2d && !via_patches && d->ci % 32 == 0;
+  p->b_split = kind == KIND_F32X3 && !via_s2d && !via_patches && d->ci % 32 == 0 && !p->ws;
   p->bt_bytes = (size_t)d->co * p->bt_ld * es;
   if (hipMalloc(&p->bt, p->bt_bytes) != hipSuccess || hipMemset(p->bt, 0, p->bt_bytes) != hipSuccess) {
     delete p;
@@ -1001,6 +1059,7 @@ int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, v
   }
   if (p->halo_lds)
     return check(conv_halo_launch(p->mfma_kind, g, p->halo_lds, p->n_cus, (hipStream_t)s), "conv_halo_launch");
+  split_args(p, g);
   return check(igemm_launch(p->b_split ? KIND_F32X3P : p->mfma_kind, p->tile, true, g, (hipStream_t)s), "igemm_launch");
 }
 
@@ -1132,14 +1191,17 @@ int pml_hip_dwconv2d_invoke(int64_t plan, const void* input, const void* filter,
                             const void* const* operands, void* const* outs, pml_hip_stream s) {
   Plan* p = (Plan*)(intptr_t)plan;
   if (!p || p->kind != PLAN_DWCONV) return fail("dwconv2d_invoke: not a dwconv2d plan");
-  if (!input || !filter || !output) return fail("dwconv2d_invoke: null operand");
+  if (!input || !output) return fail("dwconv2d_invoke: null operand");
+  if (!filter && !p->dw_filter) return fail("dwconv2d_invoke: filter is null and no packed filter exists");
   if ((((uintptr_t)input | (uintptr_t)filter | (uintptr_t)output) & 15) != 0)
     return fail("dwconv2d_invoke: buffers must be 16-byte aligned");
   DwconvArgs a;
   std::memset(&a, 0, sizeof a);
   a.d = p->dw;
   a.in = input;
-  a.filter = filter;
+  a.filter = filter ? filter : p->dw_filter;
+  a.paired_filter = filter ? nullptr : p->dw_paired;
+  a.n_cus = device_cus();
   a.out = output;
   for (int i = 0; i < a.d.tail.n_operands; ++i) {
     if (!operands || !operands[i]) return fail("dwconv2d_invoke: missing tail operand");
@@ -1147,6 +1209,34 @@ int pml_hip_dwconv2d_invoke(int64_t plan, const void* input, const void* filter,
   }
   for (int i = 0; i < PML_HIP_MAX_EPI_OPERANDS; ++i) a.outs[i] = outs ? outs[i] : nullptr;
   return check(dwconv2d_launch(a, (hipStream_t)s), "dwconv2d_launch");
+}
+
+int pml_hip_dwconv2d_pack_filter(int64_t plan, const void* filter, pml_hip_stream s) {
+  Plan* p = (Plan*)(intptr_t)plan;
+  if (!p || p->kind != PLAN_DWCONV || !filter) return fail("dwconv2d_pack_filter: bad argument");
+  const pml_hip_dwconv2d_desc& d = p->dw;
+  const size_t bytes = (size_t)d.kh * d.kw * d.c * dt_size(d.dtype);
+  if (!p->dw_filter && check(hipMalloc(&p->dw_filter, bytes), "hipMalloc")) return 1;
+  if (check(hipMemcpyAsync(p->dw_filter, filter, bytes, hipMemcpyDeviceToDevice, (hipStream_t)s), "hipMemcpyAsync")) return 1;
+  if (p->dw_paired) {
+    (void)hipFree(p->dw_paired);
+    p->dw_paired = nullptr;
+  }
+  if (!dwconv2d_takes_paired_filter(d)) return 0;
+  // once per filter: its weights are looked at on the host (the paired kernel is for finite weights only) and re-laid there
+  std::vector<uint16_t> host(bytes / 2);
+  if (check(hipMemcpyAsync(host.data(), p->dw_filter, bytes, hipMemcpyDeviceToHost, (hipStream_t)s), "hipMemcpyAsync") ||
+      check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize"))
+    return 1;
+  std::vector<uint32_t> packed((size_t)12 * (d.c / 8) * 4);
+  if (!dwconv2d_pair_filter(host.data(), d.c, packed.data())) return 0;  // an infinite or NaN weight: the general kernel
+  if (check(hipMalloc(&p->dw_paired, packed.size() * 4), "hipMalloc")) return 1;
+  if (check(hipMemcpy(p->dw_paired, packed.data(), packed.size() * 4, hipMemcpyHostToDevice), "hipMemcpy")) {
+    (void)hipFree(p->dw_paired);
+    p->dw_paired = nullptr;
+    return 1;
+  }
+  return 0;
 }
 
 int64_t pml_hip_pool2d_dispatch(const pml_hip_pool2d_desc* d) {

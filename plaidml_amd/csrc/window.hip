@@ -393,6 +393,126 @@ __global__ __launch_bounds__(256, 3) void dwconv3x3_flat_kernel(DwconvArgs a, Dw
   }
 }
 
+// The bf16 case with a filter packed once (dw_pack_filter below), all of whose weights are finite.  Two things go
+// away: the look at the weights for infinities (made once, when the filter is packed: a filter that has one keeps the
+// kernel above), and most of the bf16 -> fp32 unpacking, which was half of the arithmetic.  The taps of filter rows 0
+// and 1 that lie above each other are multiplied as a pair: one byte-permute puts a channel's two input values (row
+// y, row y + 1, same column) side by side in a register, the packed filter holds that channel's two weights the same
+// way, and v_dot2_f32_bf16 adds both products to the fp32 sum in one instruction.  Filter row 2 is kept as fp32
+// weights and multiplied the plain way.  Per thread (8 channels x 4 pixels): 48 permutes + 96 paired multiply-adds +
+// 48 unpacks + 96 multiply-adds, against 216 unpacks + 288 multiply-adds + 108 for the weight check before.
+// Packed filter: 12 vectors of 16 bytes per channel vector cv, vector j at (j * cvecs + cv) * 16 --
+//   j = 2 kx + h      (kx = 0..2, h = 0..1): words {w[0][kx][c], w[1][kx][c]} as bf16 pairs, channels 8 cv + 4 h .. + 3
+//   j = 6 + 2 kx + h: w[2][kx][c] as fp32, the same channels.
+// WLDS: the workgroups stay (the grid is what the device holds at once) and walk over their share of the work
+// blocks; the packed filter is copied into LDS once per workgroup and every thread takes its twelve vectors from
+// there.  The vector memory path, which moves 64 bytes per clock and CU, then carries the 18 input vectors of a
+// thread only, not 30; it is what this kernel waits for once the arithmetic is halved.
+template <bool WLDS>
+__global__ __launch_bounds__(256, 3) void dwconv3x3_flat_paired_kernel(DwconvArgs a, DwFlatArgs f, const i32x4_t* __restrict__ pw_global,
+                                                                       unsigned nblocks) {
+  constexpr int V = 8, ES = 2;
+  constexpr int kCols = kDwPx + 2;
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const pml_hip_dwconv2d_desc& d = a.d;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dw_smem[];
+  const i32x4_t* pw = pw_global;
+  if constexpr (WLDS) {
+    for (unsigned q = threadIdx.x; q < 12u * f.cvecs; q += 256u) ((i32x4_t*)dw_smem)[q] = pw_global[q];
+    __syncthreads();
+    pw = (const i32x4_t*)dw_smem;
+  }
+  for (unsigned vb = blockIdx.x; vb < nblocks; vb += gridDim.x) {
+  const unsigned g = xcd_contiguous_block(vb, nblocks) * 256u + threadIdx.x;
+  if (g >= f.total) continue;
+  const unsigned t1 = fast_div(g, f.cv_magic, f.cv_shift), cv = g - t1 * f.cvecs;
+  const unsigned t2 = fast_div(t1, f.xb_magic, f.xb_shift), xb = t1 - t2 * f.xblocks;
+  const unsigned n = fast_div(t2, f.oh_magic, f.oh_shift), oy = t2 - n * f.oh;
+  const int H = (int)d.h, W = (int)d.w;
+  const unsigned pix_bytes = (unsigned)d.c * ES, c0b = cv * 16u;
+  const int ox0 = (int)xb * kDwPx, iy0 = (int)oy - (int)d.pad_h, ix0 = ox0 - (int)d.pad_w;
+  // A tap outside the image must read zeros: its offset is made to lie beyond the buffer.  Rows and columns carry
+  // different marks, so that their plain sum is beyond the buffer whenever either is marked and never wraps around
+  // (the input is smaller than 1 GiB here): no select per load.
+  constexpr unsigned kRowOutside = 0x80000000u, kColOutside = 0x40000000u;
+
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc((void*)a.in, 0, (int)f.in_bytes, 0x00020000u);
+  unsigned col_off[kCols];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) col_off[c] = (unsigned)(ix0 + c) < (unsigned)W ? (unsigned)(ix0 + c) * pix_bytes + c0b : kColOutside;
+  i32x4_t xr[3][kCols];
+#pragma unroll
+  for (int ky = 0; ky < 3; ++ky) {
+    const unsigned row = (unsigned)(iy0 + ky) < (unsigned)H ? (n * (unsigned)H + (unsigned)(iy0 + ky)) * (unsigned)W * pix_bytes : kRowOutside;
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) xr[ky][c] = __builtin_amdgcn_raw_buffer_load_b128(rin, (int)(row + col_off[c]), 0, 0);
+  }
+  i32x4_t wp[3][2];
+#pragma unroll
+  for (int j = 0; j < 6; ++j) wp[j >> 1][j & 1] = pw[(unsigned)j * f.cvecs + cv];
+
+  float acc[kDwPx][V];
+#pragma unroll
+  for (int px = 0; px < kDwPx; ++px)
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[px][i] = 0.f;
+  // filter rows 0 and 1, a column of the window at a time
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    unsigned pair[V];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pair[2 * i] = __builtin_amdgcn_perm((unsigned)xr[1][c][i], (unsigned)xr[0][c][i], 0x05040100u);      // the even channel of both rows
+      pair[2 * i + 1] = __builtin_amdgcn_perm((unsigned)xr[1][c][i], (unsigned)xr[0][c][i], 0x07060302u);  // the odd one
+    }
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx) {
+      const int px = c - kx;
+      if (px < 0 || px >= kDwPx) continue;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        bf16x2 x2, w2;
+        const unsigned wbits = (unsigned)wp[kx][i >> 2][i & 3];
+        __builtin_memcpy(&x2, &pair[i], 4);
+        __builtin_memcpy(&w2, &wbits, 4);
+        acc[px][i] = __builtin_amdgcn_fdot2_f32_bf16(x2, w2, acc[px][i], false);
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);  // the fp32 weights of row 2 are fetched only now: they would only take registers before
+  f32x4_t w2[3][2];
+#pragma unroll
+  for (int j = 0; j < 6; ++j) {
+    const i32x4_t raw = pw[(unsigned)(6 + j) * f.cvecs + cv];
+    w2[j >> 1][j & 1] = __builtin_bit_cast(f32x4_t, raw);
+  }
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    float x[V];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __uint_as_float(((uint32_t)xr[2][c][i]) << 16);
+      x[2 * i + 1] = __uint_as_float(((uint32_t)xr[2][c][i]) & 0xffff0000u);
+    }
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx) {
+      const int px = c - kx;
+      if (px < 0 || px >= kDwPx) continue;
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[px][i] += x[i] * w2[kx][i >> 2][i & 3];
+    }
+  }
+
+  const unsigned opix_bytes = (d.out_pitch ? (unsigned)d.out_pitch : (unsigned)d.c) * ES;
+  const unsigned orow = ((n * f.oh + oy) * (unsigned)d.ow + (unsigned)ox0) * opix_bytes + c0b;
+#pragma unroll
+  for (int px = 0; px < kDwPx; ++px) {
+    if (ox0 + px >= (int)d.ow) break;
+    *(i32x4_t*)((unsigned char*)a.out + orow + (unsigned)px * opix_bytes) = pack_bf16_rne(acc[px]);
+  }
+  }
+}
+
 // IT: the integer type of the index arithmetic (32 bits where every element offset stays below 2^31).
 // AGG: the aggregation (PML_HIP_AGG_*), a compile-time constant so that the tap loop is straight-line code.
 template <int ES, bool WITH_INDEX, typename IT, int AGG>
@@ -682,6 +802,30 @@ __global__ __launch_bounds__(256) void s2d_filter_kernel(S2dArgs a) {
 
 }  // namespace
 
+bool dwconv2d_takes_paired_filter(const pml_hip_dwconv2d_desc& d) {
+  const int64_t opitch = d.out_pitch ? (int64_t)d.out_pitch : d.c;
+  return d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.dil_h == 1 && d.dil_w == 1 && d.tail.n_ops == 0 &&
+         d.dtype == PML_HIP_BF16 && d.n * d.h * d.w * d.c * 2 < ((int64_t)1 << 30) && d.n * d.oh * d.ow * opitch * 2 < ((int64_t)1 << 31);
+}
+
+// The paired layout of a 3x3 bf16 filter [3][3][c] (host arrays: `filter` 9 * c bf16 values, `packed` 12 * c / 8 vectors
+// of 16 bytes).  Returns false, leaving `packed` unfinished, when a weight is infinite or NaN.
+bool dwconv2d_pair_filter(const uint16_t* filter, int64_t c, uint32_t* packed) {
+  const int64_t cvecs = c / 8;
+  for (int64_t i = 0; i < 9 * c; ++i)
+    if ((filter[i] & 0x7f80u) == 0x7f80u) return false;
+  for (int64_t cv = 0; cv < cvecs; ++cv)
+    for (int kx = 0; kx < 3; ++kx)
+      for (int h = 0; h < 2; ++h)
+        for (int e = 0; e < 4; ++e) {
+          const int64_t ch = cv * 8 + h * 4 + e;
+          const uint32_t w0 = filter[(0 * 3 + kx) * c + ch], w1 = filter[(1 * 3 + kx) * c + ch], w2 = filter[(2 * 3 + kx) * c + ch];
+          packed[((2 * kx + h) * cvecs + cv) * 4 + e] = w0 | (w1 << 16);
+          packed[((6 + 2 * kx + h) * cvecs + cv) * 4 + e] = w2 << 16;  // the bf16 value as fp32
+        }
+  return true;
+}
+
 hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
   const pml_hip_dwconv2d_desc& d = a.d;
   const int es = dt_size(d.dtype);
@@ -704,7 +848,16 @@ hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s) {
       fast_div_magic(f.oh, &f.oh_magic, &f.oh_shift);
       f.in_bytes = (unsigned)(d.n * d.h * d.w * d.c * es);
       const unsigned blocks = (unsigned)((total4 + 255) / 256);
-      if (es == 2)
+      const size_t filter_lds = (size_t)12 * f.cvecs * 16;
+      if (es == 2 && a.paired_filter != nullptr && filter_lds <= 48 * 1024) {
+        // three workgroups per CU stay and share the blocks out among them (a multiple of 8, so that a workgroup's blocks
+        // all belong to its XCD's range)
+        const unsigned resident = (unsigned)(3 * a.n_cus + 7) / 8 * 8;
+        const unsigned grid = blocks < resident ? blocks : resident;
+        hipLaunchKernelGGL(dwconv3x3_flat_paired_kernel<true>, dim3(grid), dim3(256), filter_lds, s, a, f, (const i32x4_t*)a.paired_filter, blocks);
+      } else if (es == 2 && a.paired_filter != nullptr)
+        hipLaunchKernelGGL(dwconv3x3_flat_paired_kernel<false>, dim3(blocks), dim3(256), 0, s, a, f, (const i32x4_t*)a.paired_filter, blocks);
+      else if (es == 2)
         hipLaunchKernelGGL((dwconv3x3_flat_kernel<2>), dim3(blocks), dim3(256), 0, s, a, f);
       else
         hipLaunchKernelGGL((dwconv3x3_flat_kernel<4>), dim3(blocks), dim3(256), 0, s, a, f);

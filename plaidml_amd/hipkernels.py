@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libpml_hip.so')
 BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, F32, F64, BF16 = 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16
 FP32_AS_BF16X3 = 1  # descriptor flag of gemm / conv2d: fp32 operands multiplied as three bf16 products
 # schedule overrides in the same `flags` field (PML_HIP_FLAG_TILE / PML_HIP_FLAG_CONV of include/pml_hip.h)
-TILE_NAMES = ('64x64', '128x64', '128x128', '128x64w8', '128x128w8', '256x128w16', '128x128w8s2', '64x64w8k2', '256x256w8', '128x64n2')
+TILE_NAMES = ('64x64', '128x64', '128x128', '128x64w8', '128x128w8', '256x128w16', '128x128w8s2', '64x64w8k2', '256x256w8', '128x64n2', '192x384w8', '64x64ks')
 CONV_AUTO, CONV_IGEMM, CONV_PATCHES, CONV_LDSFILTER, CONV_BLOCKS = 0, 1, 2, 3, 4
 
 
@@ -43,7 +43,7 @@ EXPORTS = [
     'pml_hip_memcpy_d2d', 'pml_hip_fill_u32', 'pml_hip_stream_create', 'pml_hip_stream_destroy',
     'pml_hip_stream_sync', 'pml_hip_event_create', 'pml_hip_event_destroy', 'pml_hip_event_record',
     'pml_hip_event_sync', 'pml_hip_event_elapsed_ms', 'pml_hip_gemm_dispatch', 'pml_hip_gemm_invoke',
-    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_tile_of_workgroup', 'pml_hip_tile_name', 'pml_hip_tile_by_name', 'pml_hip_gemm_tail_cheaper_apart',
+    'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_dwconv2d_pack_filter', 'pml_hip_tile_of_workgroup', 'pml_hip_tile_name', 'pml_hip_tile_by_name', 'pml_hip_gemm_tail_cheaper_apart',
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
@@ -188,6 +188,7 @@ def lib():
         L.pml_hip_argsort.argtypes = [ctypes.POINTER(ArgsortDesc), vp, vp, vp]
         L.pml_hip_prng.argtypes = [vp, ctypes.c_int64, vp, vp, vp]
         L.pml_hip_conv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
+        L.pml_hip_dwconv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
         _lib = L
     return _lib
 

@@ -204,7 +204,7 @@ class Planner {
   }
   static int tileByName(const std::string& name) {
     const int t = pml_hip_tile_by_name(name.c_str());
-    if (t < 0) throw std::runtime_error("Invalid tile '" + name + "' (64x64, 128x64, 128x128, 128x64w8, 128x128w8, 128x128w8s2, 256x128w16, 64x64w8k2, 256x256w8, 128x64n2)");
+    if (t < 0) throw std::runtime_error("Invalid tile '" + name + "' (64x64, 128x64, 128x128, 128x64w8, 128x128w8, 128x128w8s2, 256x128w16, 64x64w8k2, 256x256w8, 128x64n2, 192x384w8, 64x64ks)");
     return t;
   }
   struct Rule {
@@ -1509,11 +1509,13 @@ class Planner {
     s.a = bufferFor(op.operands[0]);
     s.b = bufferFor(op.operands[1]);
     s.c = bufferFor(tb.final_value);
+    s.b_constant = op.operands[1]->kind == Value::Constant;
     attachTail(&s, tb);
     s.flops = 2.0 * os.elements() * d.kh * d.kw;
     s.bytes = static_cast<double>(is.elements() + os.elements() + fs.elements()) * util::byteSize(dt);
     s.text = "dwconv2d " + std::string(util::mnemonic(dt)) + " " + is.str() + " k=" + std::to_string(d.kh) + "x" + std::to_string(d.kw) +
-             " stride=" + std::to_string(d.stride_h) + tailText(tb) + " -> " + tb.final_value->shape.str();
+             " stride=" + std::to_string(d.stride_h) + (s.b_constant ? " (constant filter, packed once)" : "") + tailText(tb) + " -> " +
+             tb.final_value->shape.str();
     plan_->steps.push_back(s);
     return true;
   }

@@ -55,7 +55,7 @@ struct Step {
   std::vector<int64_t> operand_off;
   std::vector<int> outs;           // extra outputs of STORE steps (index = STORE's operand field)
   bool b_is_nk = false;            // Gemm: right-hand side is already [N][K]
-  bool b_constant = false;         // Gemm / Conv2d: right-hand side is a program constant (pack once)
+  bool b_constant = false;         // Gemm / Conv2d / Dwconv2d: right-hand side / filter is a program constant (pack once)
   size_t copy_bytes = 0;           // Copy
   // roofline bookkeeping for reports
   double flops = 0;

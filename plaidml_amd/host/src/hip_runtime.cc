@@ -277,6 +277,7 @@ class HipExecutable final : public Executable {
     if (s.kind == Step::Gemm && s.gemm.k2 > 0 && s.b2_constant && !s.b_is_nk)
       hipCheck(pml_hip_gemm_pack_b2(h, ptr(s.b2, s.b2_off, elemSize(s.gemm.in_dtype)), nullptr), "pack_b2");
     if (s.kind == Step::Conv2d && s.b_constant) hipCheck(pml_hip_conv2d_pack_filter(h, ptr(s.b), nullptr), "pack_filter");
+    if (s.kind == Step::Dwconv2d && s.b_constant) hipCheck(pml_hip_dwconv2d_pack_filter(h, ptr(s.b), nullptr), "pack_filter");
   }
 
   void launch(size_t i) {
@@ -309,7 +310,8 @@ class HipExecutable final : public Executable {
                  s.text.c_str());
         break;
       case Step::Dwconv2d:
-        hipCheck(pml_hip_dwconv2d_invoke(handles_[i], ptr(s.a), ptr(s.b), ptr(s.c), operands, outs, nullptr), s.text.c_str());
+        hipCheck(pml_hip_dwconv2d_invoke(handles_[i], ptr(s.a), s.b_constant ? nullptr : ptr(s.b), ptr(s.c), operands, outs, nullptr),
+                 s.text.c_str());
         break;
       case Step::Pool2d:
         hipCheck(pml_hip_pool2d_invoke(handles_[i], ptr(s.a), ptr(s.c), ptr(s.out2), nullptr), s.text.c_str());

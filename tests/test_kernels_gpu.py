@@ -90,7 +90,7 @@ def test_gemm_f32_matches_oracle_contraction():
     np.testing.assert_allclose(run_gemm(Av, Bv, hk.F32, hk.F32), ref, rtol=FP32_RTOL, atol=1e-5)
 
 
-TILE_NAMES = ['64x64', '128x64', '128x128', '128x64w8', '128x128w8', '128x128w8s2', '256x128w16', '64x64w8k2', '256x256w8', '128x64n2']
+TILE_NAMES = ['64x64', '128x64', '128x128', '128x64w8', '128x128w8', '128x128w8s2', '256x128w16', '64x64w8k2', '256x256w8', '128x64n2', '192x384w8', '64x64ks']
 
 
 @pytest.mark.parametrize('tile', TILE_NAMES)
@@ -738,12 +738,17 @@ DW_CASES = [('bf16', 2, 19, 19, 32, 3, 1, 1), ('bf16', 1, 9, 24, 16, 3, 1, 0), (
             ('bf16', 1, 12, 15, 16, 5, 1, 2), ('f32', 1, 14, 14, 8, 3, 2, 1)]
 
 
+@pytest.mark.parametrize('packed', [False, True, 'finite'])
 @pytest.mark.parametrize('kind,N,H,W,C,k,stride,pad', DW_CASES)
-def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad):
+def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad, packed):
+    """packed: the filter is handed over once (pml_hip_dwconv2d_pack_filter) and the invoke is given none -- with the
+    infinite weight, which keeps the general kernel, and ('finite') without it, which lets the 3x3 bf16 case take the
+    kernel that multiplies the taps of two filter rows in one instruction."""
     rng = np.random.default_rng(90)
     Iv = rng.standard_normal((N, H, W, C)).astype(np.float32)
     Fv = (rng.standard_normal((k, k, C, 1)) * 0.3).astype(np.float32)
-    if k == 3 and stride == 1 and pad == 1:
+    with_inf = k == 3 and stride == 1 and pad == 1 and packed != 'finite'
+    if with_inf:
         Fv[0, 0, 0, 0] = np.inf  # only pixels whose top-left tap lies inside the image see it
     if kind == 'bf16':
         Iv, Fv = E.round_bf16(Iv), E.round_bf16(Fv)
@@ -760,7 +765,10 @@ def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad):
     dI = hk.DeviceBuffer.from_numpy(bf16(Iv) if kind == 'bf16' else Iv)
     dF = hk.DeviceBuffer.from_numpy(bf16(Fv) if kind == 'bf16' else Fv)
     dO = hk.DeviceBuffer(N * OH * OW * C * es)
-    hk.check(hk.lib().pml_hip_dwconv2d_invoke(plan, dI.ptr, dF.ptr, dO.ptr, hk.ptr_array([]), hk.ptr_array([]), None))
+    if packed:
+        hk.check(hk.lib().pml_hip_dwconv2d_pack_filter(plan, dF.ptr, None))
+        hk.check(hk.lib().pml_hip_fill_u32(dF.ptr, 0x7fc07fc0, k * k * C * es // 4, None))  # the plan keeps its own copy
+    hk.check(hk.lib().pml_hip_dwconv2d_invoke(plan, dI.ptr, None if packed else dF.ptr, dO.ptr, hk.ptr_array([]), hk.ptr_array([]), None))
     hk.check(hk.lib().pml_hip_stream_sync(None))
     out = dO.to_numpy(np.uint16 if kind == 'bf16' else np.float32, (N, OH, OW, C))
     if kind == 'bf16':
@@ -769,7 +777,7 @@ def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad):
     I, F = E.Placeholder(dt, Iv.shape), E.Placeholder(dt, Fv.shape)
     O = op.convolution(I, F, strides=[stride, stride], autopad=op.EXPLICIT, manual_padding=[pad, pad], depthwise=True)
     ref, = E.run(E.Program('dw', [I, F], [O]), [Iv, Fv])
-    assert np.isinf(ref).any() == (k == 3 and stride == 1 and pad == 1) and not np.isnan(ref).any()
+    assert np.isinf(ref).any() == with_inf and not np.isnan(ref).any()
     np.testing.assert_allclose(out, ref, rtol=BF16_RTOL if kind == 'bf16' else FP32_RTOL, atol=1e-2 if kind == 'bf16' else 1e-4)
     hk.lib().pml_hip_plan_free(plan)
 

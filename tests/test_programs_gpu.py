@@ -255,14 +255,24 @@ def test_requantisation_chain_as_its_own_launch(R, C, out_name):
     assert got.min() == lo and got.max() == hi  # both clamps bite
 
 
-def test_large_int8_gemm_leaves_its_requantisation_to_a_second_launch():
-    """4096^3 int8 with the requantisation chain: the planner asks the kernel library, which multiplies this shape
-    faster under a plain tail, and plans two launches; a small problem keeps the chain fused."""
+def test_large_int8_gemm_keeps_its_requantisation_and_leaves_other_chains_to_a_second_launch():
+    """4096^3 int8: the clip-and-round requantisation chain runs as straight code behind the large tile and stays fused
+    (one launch); a chain that only the step-wise tail can run (here floor instead of clip and round) would cost
+    that tile, so the planner, having asked the kernel library, leaves it to an element-wise launch of its own."""
     prog = programs.config2_int8_gemm(E, op, M=4096, N=4096, K=4096)[0]
     prog.compile('hip')
     plan = dict(prog.passes)['hip-plan']
+    assert '1 launches' in plan and 'tail=[store cast:f32 mul(t0) maxgt(-127) min(127) round cast:si8]' in plan, plan
+    M = N = K = 4096
+    A, B, S = E.Placeholder(E.DType.INT8, [M, K]), E.Placeholder(E.DType.INT8, [K, N]), E.Placeholder(E.DType.FLOAT32, [N])
+    i, j, k = E.TensorIndexes(3)
+    C = E.Contraction().outShape(M, N).outAccess(i, j).sum(E.cast(A, E.DType.INT32)[i, k] * E.cast(B, E.DType.INT32)[k, j]).build()
+    Q = E.cast(E.floor(E.cast(C, E.DType.FLOAT32) * S), E.DType.INT8)
+    prog = E.Program('int8_gemm_floor', [A, B, S], [C, Q])
+    prog.compile('hip')
+    plan = dict(prog.passes)['hip-plan']
     assert '2 launches' in plan and 'gemm si8 m=4096 n=4096 k=4096 B=[k][n] -> 4096x4096xsi32' in plan, plan
-    assert 'eltwise cast tail=[cast:f32 mul(t0)' in plan, plan
+    assert 'eltwise cast tail=[cast:f32 mul(t0) floor' in plan, plan
     prog = programs.config2_int8_gemm(E, op)[0]
     prog.compile('hip')
     assert '1 launches' in dict(prog.passes)['hip-plan']
