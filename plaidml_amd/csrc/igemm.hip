@@ -578,11 +578,11 @@ __global__ __launch_bounds__(NT, (igemm_waves_per_simd<BM, BN, STAGES, SLAB, NT>
       // the partial tile as it is: four columns per thread, rows of the workspace are whole 16-byte vectors
       constexpr int TPR = BN / 4, RPP = NT / TPR;
       const int c4 = (tid % TPR) * 4;
-      accs_t* const ws = (accs_t*)p.ws + (int64_t)split * p.M * p.sk_pitch;
       if (n0 + c4 < p.sk_pitch) {
+        accs_t* const mine = (accs_t*)p.ws + (int64_t)split * p.M * p.sk_pitch;
 #pragma unroll
         for (int row = tid / TPR; row < BM; row += RPP)
-          if (m0 + row < p.M) *(acc4_t*)&ws[(m0 + row) * p.sk_pitch + n0 + c4] = *(const acc4_t*)&ctile[row * CS + c4];
+          if (m0 + row < p.M) *(acc4_t*)&mine[(m0 + row) * p.sk_pitch + n0 + c4] = *(const acc4_t*)&ctile[row * CS + c4];
       }
       return;
     }
@@ -701,34 +701,38 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t* __
   }
 }
 
-// Second pass of a K split over workgroups: a workgroup per 64 x 64 result tile adds the partial tiles in split order
-// (int32: exact whatever the order) into the same LDS layout the one-pass kernel stages its accumulators in, and runs
-// the same tail code over it.
+// Second pass of a K split over workgroups: a workgroup per 16 rows x 64 columns of the result, a thread per four
+// columns, adds the partial tiles in split order (int32: exact whatever the order; eight loads in flight per thread)
+// into the LDS layout the one-pass kernel stages its accumulators in, and runs the same tail code over it.  (The two
+// passes are two launches on purpose: the partial tiles then pass from one to the other across a kernel boundary;
+// handing them over inside one launch -- an arrival count per tile, the last workgroup adds up -- needs a device-wide
+// release and acquire in every workgroup, and those cost more than the second launch: 25-40 us a layer against 12.)
 template <int KIND>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(IgemmArgs p_by_value) {
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(IgemmArgs p_by_value, int strips_n) {
   const IgemmArgs& p = *(const IgemmArgs*)(const __attribute__((address_space(4))) void*)__builtin_amdgcn_kernarg_segment_ptr();
   typedef typename Acc<KIND>::scalar accs_t;
   typedef accs_t acc4_t __attribute__((ext_vector_type(4)));
   constexpr int CS = 64 + 4;
-  __shared__ __attribute__((aligned(16))) accs_t ctile[64 * CS];
+  __shared__ __attribute__((aligned(16))) accs_t ctile[16 * CS];
   const int tid = threadIdx.x;
-  int tile_m, tile_n;
-  tile_of(p.order, blockIdx.x, &tile_m, &tile_n);
-  const int64_t m0 = (int64_t)tile_m * 64, n0 = (int64_t)tile_n * 64;
-  const int c4 = (tid & 15) * 4;
-  const accs_t* const ws = (const accs_t*)p.ws;
+  const int strip_m = (int)(blockIdx.x / (unsigned)strips_n), strip_n = (int)(blockIdx.x % (unsigned)strips_n);
+  const int64_t m0 = (int64_t)strip_m * 16, n0 = (int64_t)strip_n * 64;
+  const int row = tid >> 4, c4 = (tid & 15) * 4;
+  acc4_t sum = {0, 0, 0, 0};
+  if (m0 + row < p.M && n0 + c4 < p.sk_pitch) {
+    const int64_t part = (int64_t)p.M * p.sk_pitch;
+    const accs_t* const at = (const accs_t*)p.ws + (m0 + row) * p.sk_pitch + n0 + c4;
+    for (int sp = 0; sp < p.sk_splits; sp += 8) {
+      acc4_t got[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = (tid >> 4) + 16 * i;
-    acc4_t sum = {0, 0, 0, 0};
-    if (m0 + row < p.M && n0 + c4 < p.sk_pitch) {
-      const accs_t* at = ws + (m0 + row) * p.sk_pitch + n0 + c4;
-      for (int sp = 0; sp < p.sk_splits; ++sp) sum += *(const acc4_t*)(at + (int64_t)sp * p.M * p.sk_pitch);
+      for (int u = 0; u < 8; ++u) got[u] = sp + u < p.sk_splits ? *(const acc4_t*)(at + (sp + u) * part) : acc4_t{0, 0, 0, 0};
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sum += got[u];
     }
-    *(acc4_t*)&ctile[row * CS + c4] = sum;
   }
+  *(acc4_t*)&ctile[row * CS + c4] = sum;
   __syncthreads();
-  tile_tail<KIND, 64, 64, 256>(p, ctile, m0, n0, tid);
+  tile_tail<KIND, 16, 64, 256>(p, ctile, m0, n0, tid);
 }
 
 // The two launches of a 64 x 64 tiling whose K loop is split over workgroups (a.ws, a.sk_* prepared by the caller).
@@ -749,7 +753,9 @@ hipError_t launch_splitk(const IgemmArgs& a, hipStream_t s) {
     b.sk_tiles = (int)tiles;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * a.sk_splits)), dim3(kThreads), lds, s, b);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-    hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)tiles), dim3(256), 0, s, b);
+    const int64_t strips = ((a.M + 15) / 16) * tiles_n;
+    if (strips >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)strips), dim3(256), 0, s, b, (int)tiles_n);
     return hipGetLastError();
   }
 }

@@ -201,15 +201,15 @@ struct IgemmArgs {
 
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);
 // How TILE_64x64_KSPLIT shares the K loop out: slabs of 128 bytes of K in all, and for a device of n_cus compute units
-// the number of splits (1: not worth splitting) with the slabs each takes -- about two workgroups per CU, at least two
-// slabs per split, at most 32 splits.
+// the number of splits (1: not worth splitting) with the slabs each takes -- about one workgroup per CU, at least two
+// slabs per split, at most 16 splits.
 inline int64_t igemm_slabs(const IgemmArgs& a, bool conv, int es) {
   return conv ? (int64_t)a.KH * a.KW * (((int64_t)a.CI * es + 127) / 128) : (a.K * es + 127) / 128;
 }
 inline void igemm_split_plan(int64_t m, int64_t n, int64_t slabs, int n_cus, int* splits, int* per) {
   const int64_t tiles = ((m + 63) / 64) * ((n + 63) / 64);
-  int64_t want = tiles > 0 ? (2 * (int64_t)n_cus + tiles - 1) / tiles : 1;
-  if (want > 32) want = 32;
+  int64_t want = tiles > 0 ? ((int64_t)n_cus + tiles - 1) / tiles : 1;
+  if (want > 16) want = 16;
   if (want > slabs / 2) want = slabs / 2;
   if (want < 2) {
     *splits = 1;

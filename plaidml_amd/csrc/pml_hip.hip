@@ -153,7 +153,7 @@ int choose_tile(int64_t m, int64_t n, int64_t k_bytes, int kind = KIND_BF16, boo
   auto tiles = [&](int64_t bm, int64_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   // Few tiles and a long K (a network's last stages at batch 1: 49 x 512 x 4608 is 8 tiles of 72 slabs): the K loop is
   // shared out among workgroups and a second launch adds the partial tiles up.  Measured inside ResNet-50 at batch 1.
-  if (allow_split && tiles(64, 64) <= 64 && k_bytes >= 1024) return TILE_64x64_KSPLIT;
+  if (allow_split && tiles(64, 64) <= 64 && k_bytes >= 2048) return TILE_64x64_KSPLIT;
   if (kind == KIND_F32X3) {
     // A fragment that is split in registers costs 24 vector instructions whatever it is multiplied with, so the
     // tile a wavefront holds decides how many MFMAs share that cost -- but the problems this kind meets here are

@@ -33,7 +33,7 @@ FORCED = {'flags': 0}
 
 
 def run_gemm(A, B, in_dt, out_dt, init=None, init_strides=(0, 0), init_dt=0, tail=None, operands=(), c_dt=None,
-             extra_out=None, flags=0):
+             extra_out=None, flags=0, invokes=1):
     M, K = A.shape
     _, N = B.shape
     d = hk.GemmDesc()
@@ -60,8 +60,10 @@ def run_gemm(A, B, in_dt, out_dt, init=None, init_strides=(0, 0), init_dt=0, tai
     if extra_out is not None:
         dX = hk.DeviceBuffer(M * N * np.dtype(extra_out).itemsize)
         outs = [dX.ptr]
-    hk.check(hk.lib().pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, dI.ptr if dI else None,
-                                          hk.ptr_array([o.ptr for o in dops]), hk.ptr_array(outs), None))
+    for _ in range(invokes):  # (the last run's result is the one returned: what a run leaves behind must not show in the next)
+        hk.check(hk.lib().pml_hip_fill_u32(dC.ptr, 0xdeadbeef, M * N * np.dtype(np_c).itemsize // 4, None))
+        hk.check(hk.lib().pml_hip_gemm_invoke(plan, dA.ptr, dB.ptr, dC.ptr, dI.ptr if dI else None,
+                                              hk.ptr_array([o.ptr for o in dops]), hk.ptr_array(outs), None))
     hk.check(hk.lib().pml_hip_stream_sync(None))
     C = dC.to_numpy(np_c, (M, N))
     X = dX.to_numpy(extra_out, (M, N)) if dX else None
@@ -341,6 +343,57 @@ def test_gemm_i8_requantize_tail():
     x = E.select(x < 127.0, x, E.cast(E.Constant(127.0), D.FLOAT32))
     Qo, = E.run(E.Program('q', [Cp, Sp], [E.cast(E.round(x), D.INT8)]), [ref, S])
     np.testing.assert_array_equal(Q, Qo)
+
+
+@pytest.mark.parametrize('M,N,K', [(49, 512, 2048), (196, 256, 2048), (100, 130, 4096), (1, 1000, 2048), (300, 72, 2064)])
+def test_gemm_k_split_over_workgroups(M, N, K, capsys):
+    """Few result tiles and a long K: the library shares the K loop out among workgroups (partial tiles in a workspace,
+    added up by a second launch that runs the tail; three runs of one plan over the same workspace).  int8 bit for bit -- the sum of the parts is the sum; bf16 with
+    bias + residual + relu, fp32 and the split fp32 kind against float64; ragged M, N (a workspace pitch of whole
+    vectors) and a K that leaves the last split short."""
+    rng = np.random.default_rng(123)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    bias_i = rng.integers(-1000, 1000, N, dtype=np.int32)
+    C = run_gemm(A, B, hk.I8, hk.I32, init=bias_i, init_strides=(0, 1), init_dt=hk.I32, invokes=3)
+    assert 'K split over workgroups' in capsys.readouterr().out
+    np.testing.assert_array_equal(C, (A.astype(np.int64) @ B.astype(np.int64) + bias_i).astype(np.int32))
+    Af = E.round_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    Bf = E.round_bf16((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32))
+    bias = E.round_bf16(rng.standard_normal(N).astype(np.float32))
+    R = E.round_bf16(rng.standard_normal((M, N)).astype(np.float32))
+    tail = hk.make_tail(ops=[(hk.EPI_ADD, hk.BF16, hk.OPND_TENSOR, 0, 0.0), (hk.EPI_RELU, hk.BF16, 0, 0, 0.0)], operands=[(hk.BF16, N, 1)])
+    got = E.bf16_from_bits(run_gemm(bf16(Af), bf16(Bf), hk.BF16, hk.BF16, init=bf16(bias), init_strides=(0, 1), init_dt=hk.BF16,
+                                    tail=tail, operands=[bf16(R)]))
+    assert 'K split over workgroups' in capsys.readouterr().out
+    ref = np.maximum(E.round_bf16((Af.astype(np.float64) @ Bf.astype(np.float64) + bias).astype(np.float32)).astype(np.float64) + R, 0)
+    np.testing.assert_allclose(got, ref, rtol=BF16_RTOL, atol=2e-2)
+    A32 = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B32 = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    for flags in (0, hk.FP32_AS_BF16X3):
+        got = run_gemm(A32, B32, hk.F32, hk.F32, flags=flags)
+        assert 'K split over workgroups' in capsys.readouterr().out
+        np.testing.assert_allclose(got, A32.astype(np.float64) @ B32.astype(np.float64), rtol=FP32_RTOL, atol=2e-3)
+
+
+@pytest.mark.parametrize('kind', ['bf16', 'f32'])
+@pytest.mark.parametrize('shape,k,co,stride', [((1, 7, 7, 512), 3, 512, 1), ((1, 14, 14, 256), 3, 256, 2), ((2, 9, 11, 96), 5, 40, 1)])
+def test_conv_k_split_over_workgroups(kind, shape, k, co, stride, capsys):
+    """The same for convolutions (the 3x3 layers of a network's last stages at batch 1): a split begins in the middle
+    of the tap sequence, also in the middle of a tap's channels (96 channels: one and a half slabs per tap in bf16)."""
+    Iv, Fv = _conv_case(kind, shape, k, k, co, op.SAME_UPPER, 57)
+    bias = np.random.default_rng(58).standard_normal(co).astype(np.float32)
+    if kind == 'bf16':
+        bias = E.round_bf16(bias)
+        out = E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=stride, bias=bf16(bias), relu=True))
+        ref = oracle_conv(Iv, Fv, D.BFLOAT16, stride, op.SAME_UPPER, bias, True)
+        tol = dict(rtol=BF16_RTOL, atol=2e-2)
+    else:
+        out = run_conv(Iv, Fv, hk.F32, hk.F32, stride=stride, bias=bias, relu=True)
+        ref = oracle_conv(Iv, Fv, D.FLOAT32, stride, op.SAME_UPPER, bias, True)
+        tol = dict(rtol=FP32_RTOL, atol=1e-3)
+    assert 'K split over workgroups' in capsys.readouterr().out
+    np.testing.assert_allclose(out, ref, **tol)
 
 
 def _requant_reference(C32, S, lo, hi):
