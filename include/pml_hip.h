@@ -76,6 +76,18 @@ int pml_hip_event_record(pml_hip_event e, pml_hip_stream s);
 int pml_hip_event_sync(pml_hip_event e);
 int pml_hip_event_elapsed_ms(pml_hip_event start, pml_hip_event stop, float* ms);
 
+/* Replay of a fixed sequence of launches as one HIP graph: what the reference gets from jitting a whole program into
+ * one function (pmlc/rt/jit_executable.cc:484-490 calls it once per run) -- here a run is many launches, and at small
+ * batch the launches cost more than the kernels.  Between _begin and _end every launch on `s` (a stream made by
+ * pml_hip_stream_create, never NULL) is recorded instead of run; every *_invoke of this library may be recorded once
+ * it has run at least once on the same plan (first runs may allocate).  _end returns the replayable graph, or fails
+ * (and leaves `s` usable) if something could not be recorded.  Pointers are baked in: replay with the same buffers. */
+typedef void* pml_hip_graph;
+int pml_hip_capture_begin(pml_hip_stream s);
+int pml_hip_capture_end(pml_hip_stream s, pml_hip_graph* graph);
+int pml_hip_graph_launch(pml_hip_graph graph, pml_hip_stream s);
+int pml_hip_graph_destroy(pml_hip_graph graph);
+
 /* ---- fused elementwise tail ------------------------------------------------
  * A chain of scalar operations applied to one running value per output
  * element.  It plays the role of the bias / ReLU variants of the reference

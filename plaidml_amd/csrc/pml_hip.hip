@@ -554,6 +554,35 @@ int pml_hip_event_create(pml_hip_event* e) {
   *e = (pml_hip_event)ev;
   return 0;
 }
+int pml_hip_capture_begin(pml_hip_stream s) {
+  if (!s) return fail("pml_hip_capture_begin: the default stream cannot be captured");
+  // (thread-local mode: other threads of the process may go on allocating while this one records)
+  return check(hipStreamBeginCapture((hipStream_t)s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+int pml_hip_capture_end(pml_hip_stream s, pml_hip_graph* graph) {
+  if (!s || !graph) return fail("pml_hip_capture_end: null argument");
+  *graph = nullptr;
+  hipGraph_t g = nullptr;
+  // (always called, also after a failed recording: it is what takes the stream out of capture mode)
+  const hipError_t e = hipStreamEndCapture((hipStream_t)s, &g);
+  if (e != hipSuccess || !g) {
+    (void)hipGetLastError();
+    return fail(std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+  }
+  hipGraphExec_t exec = nullptr;
+  const hipError_t ei = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (check(ei, "hipGraphInstantiate")) return 1;
+  *graph = (pml_hip_graph)exec;
+  return 0;
+}
+int pml_hip_graph_launch(pml_hip_graph graph, pml_hip_stream s) {
+  if (!graph) return fail("pml_hip_graph_launch: null graph");
+  return check(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)s), "hipGraphLaunch");
+}
+int pml_hip_graph_destroy(pml_hip_graph graph) {
+  return graph ? check(hipGraphExecDestroy((hipGraphExec_t)graph), "hipGraphExecDestroy") : 0;
+}
 int pml_hip_event_destroy(pml_hip_event e) { return check(hipEventDestroy((hipEvent_t)e), "hipEventDestroy"); }
 int pml_hip_event_record(pml_hip_event e, pml_hip_stream s) {
   return check(hipEventRecord((hipEvent_t)e, (hipStream_t)s), "hipEventRecord");

@@ -97,7 +97,8 @@ _SIGS = {
 }
 # the two functions that take no plaidml_error, and the statistics helper
 EXPORTS = sorted(list(_SIGS) + ['plaidml_string_ptr', 'plaidml_string_free', 'plaidml_hip_last_run_stats',
-                               'plaidml_hip_last_run_memory', 'plaidml_hip_last_run_step_ms'])
+                               'plaidml_hip_last_run_memory', 'plaidml_hip_last_run_step_ms', 'plaidml_hip_last_run_replayed',
+                               'plaidml_hip_last_run_graph_note'])
 
 _lib = None
 
@@ -122,6 +123,10 @@ def lib():
         L.plaidml_hip_last_run_memory.restype = None
         L.plaidml_hip_last_run_memory.argtypes = [ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]
         L.plaidml_hip_last_run_step_ms.restype = sz
+        L.plaidml_hip_last_run_replayed.restype = ctypes.c_int
+        L.plaidml_hip_last_run_replayed.argtypes = []
+        L.plaidml_hip_last_run_graph_note.restype = ctypes.c_char_p
+        L.plaidml_hip_last_run_graph_note.argtypes = []
         L.plaidml_hip_last_run_step_ms.argtypes = [sz, ctypes.POINTER(f64)]
         _lib = L
         call('plaidml_init')
@@ -956,7 +961,8 @@ def last_run_stats():
     steps = (f64 * (n.value or 1))()
     got = lib().plaidml_hip_last_run_step_ms(n.value, steps)  # per launch; empty unless PLAIDML_PROFILE=1 was set
     return {'kernel_ms': k.value, 'h2d_ms': h.value, 'd2h_ms': d.value, 'launches': n.value, 'arena_bytes': a.value,
-            'unshared_temp_bytes': u.value, 'device_bytes': t.value, 'step_ms': [steps[i] for i in range(got if got < n.value else n.value)]}
+            'unshared_temp_bytes': u.value, 'device_bytes': t.value, 'graph': bool(lib().plaidml_hip_last_run_replayed()),
+            'graph_note': lib().plaidml_hip_last_run_graph_note().decode(), 'step_ms': [steps[i] for i in range(got if got < n.value else n.value)]}
 
 
 def to_bf16_bits(a):

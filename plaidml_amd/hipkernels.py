@@ -42,7 +42,8 @@ EXPORTS = [
     'pml_hip_free', 'pml_hip_host_alloc', 'pml_hip_host_free', 'pml_hip_memcpy_h2d', 'pml_hip_memcpy_d2h',
     'pml_hip_memcpy_d2d', 'pml_hip_fill_u32', 'pml_hip_stream_create', 'pml_hip_stream_destroy',
     'pml_hip_stream_sync', 'pml_hip_event_create', 'pml_hip_event_destroy', 'pml_hip_event_record',
-    'pml_hip_event_sync', 'pml_hip_event_elapsed_ms', 'pml_hip_gemm_dispatch', 'pml_hip_gemm_invoke',
+    'pml_hip_event_sync', 'pml_hip_event_elapsed_ms', 'pml_hip_capture_begin', 'pml_hip_capture_end',
+    'pml_hip_graph_launch', 'pml_hip_graph_destroy', 'pml_hip_gemm_dispatch', 'pml_hip_gemm_invoke',
     'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_dwconv2d_pack_filter', 'pml_hip_tile_of_workgroup', 'pml_hip_tile_name', 'pml_hip_tile_by_name', 'pml_hip_gemm_tail_cheaper_apart',
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
@@ -161,6 +162,10 @@ def lib():
         L.pml_hip_event_record.argtypes = [vp, vp]
         L.pml_hip_event_sync.argtypes = [vp]
         L.pml_hip_event_elapsed_ms.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
+        L.pml_hip_capture_begin.argtypes = [vp]
+        L.pml_hip_capture_end.argtypes = [vp, ctypes.POINTER(vp)]
+        L.pml_hip_graph_launch.argtypes = [vp, vp]
+        L.pml_hip_graph_destroy.argtypes = [vp]
         pp = ctypes.POINTER(vp)
         L.pml_hip_gemm_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp, pp, pp, vp]
         L.pml_hip_gemm_run_static.argtypes = [ctypes.POINTER(GemmDesc), vp, vp, vp, vp, pp, pp, vp]

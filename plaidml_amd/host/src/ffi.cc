@@ -180,6 +180,7 @@ void compileProgram(tile::Program* program, const std::string& requested, bool /
   }
   if (opts.count("tile")) options.tile = opts["tile"];
   if (opts.count("conv")) options.conv = opts["conv"];
+  if (opts.count("graph")) options.graph = truthy(opts["graph"]);
   options.schedule_path = util::Settings::Instance()->get("PLAIDML_SCHEDULE_PATH");
   program->passes.resize(1);  // keep only the "tile" text when compiling again
   tile::foldAddIntoInit(program);
@@ -849,6 +850,15 @@ void plaidml_hip_last_run_memory(size_t* arena_bytes, size_t* unshared_temp_byte
   if (arena_bytes) *arena_bytes = s.arena_bytes;
   if (unshared_temp_bytes) *unshared_temp_bytes = s.unshared_temp_bytes;
   if (device_bytes) *device_bytes = s.device_bytes;
+}
+
+// 1 when that run replayed its launches as one recorded HIP graph, 0 when it launched them one by one.
+int plaidml_hip_last_run_replayed(void) { return rt::lastInvokeStats().replayed ? 1 : 0; }
+// Why not, when recording was tried and failed ("" otherwise); valid until the calling thread's next run.
+const char* plaidml_hip_last_run_graph_note(void) {
+  thread_local std::string note;
+  note = rt::lastInvokeStats().graph_note;
+  return note.c_str();
 }
 
 // Per-launch device milliseconds of that run (filled only when PLAIDML_PROFILE=1 was set during it): copies up

@@ -140,7 +140,9 @@ struct TailBuild {
 
 class Planner {
  public:
-  Planner(Program* program, const Options& options) : prog_(program), opt_(options), plan_(std::make_shared<Plan>()) {}
+  Planner(Program* program, const Options& options) : prog_(program), opt_(options), plan_(std::make_shared<Plan>()) {
+    plan_->graph = options.graph;
+  }
 
   std::shared_ptr<Plan> run() {
     rewriteSelectMinMax();

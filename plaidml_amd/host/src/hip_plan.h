@@ -67,6 +67,7 @@ struct Plan {
   std::vector<Step> steps;
   std::vector<int> input_buffers;   // buffer id per program input
   std::vector<int> output_buffers;  // buffer id per program output
+  bool graph = true;                // the runtime may replay the launches of a run as one recorded graph
   std::string dump() const;
 };
 
@@ -81,6 +82,9 @@ struct Options {
   // a file of plan-dump lines, "[n] <step text> {tile=...,conv=...}", that apply to the steps whose text they repeat --
   // a plan dump edited by hand is such a file.  Names: pml_hip_tile_name, and igemm / patches / ldsfilter / blocks.
   std::string tile, conv, schedule_path;
+  // `hip{graph=0}`: every run launches its kernels one by one (the default records the launches of the third run of an
+  // executable into a HIP graph and replays that from then on: at batch 1 the launches cost more than the kernels)
+  bool graph = true;
 };
 
 // Runs the pipeline on a copy of the program's op list and returns the plan.

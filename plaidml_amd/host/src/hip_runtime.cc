@@ -68,7 +68,15 @@ class HipExecutable final : public Executable {
       for (size_t i = 0; i < plan_->steps.size(); ++i) dispatch(i);
       hipCheck(pml_hip_event_create(&ev0_), "event");
       hipCheck(pml_hip_event_create(&ev1_), "event");
+      hipCheck(pml_hip_stream_create(&stream_), "stream");
       hipCheck(pml_hip_stream_sync(nullptr), "sync");
+      // Recording is for runs of plain kernel launches and device-to-device copies: the sort, scatter, gather, index and random-number steps keep
+      // state or sizes on the host side of their entry points and stay with one-by-one launches.
+      graphable_ = plan_->graph && plan_->steps.size() > 1;
+      for (const Step& s : plan_->steps)
+        if (s.kind != Step::Gemm && s.kind != Step::Conv2d && s.kind != Step::Dwconv2d && s.kind != Step::Pool2d &&
+            s.kind != Step::Eltwise && s.kind != Step::Contract && s.kind != Step::Select && s.kind != Step::Copy)
+          graphable_ = false;
     } catch (...) {
       release();
       throw;
@@ -88,25 +96,36 @@ class HipExecutable final : public Executable {
     for (size_t i = 0; i < inputs.size(); ++i) {
       const BufferInfo& b = plan_->buffers[plan_->input_buffers[i]];
       if (inputs[i]->size() < b.bytes) throw std::runtime_error("input buffer #" + std::to_string(i) + " is too small");
-      hipCheck(pml_hip_memcpy_h2d(device_[plan_->input_buffers[i]], inputs[i]->data(), b.bytes, nullptr), "h2d");
+      hipCheck(pml_hip_memcpy_h2d(device_[plan_->input_buffers[i]], inputs[i]->data(), b.bytes, stream_), "h2d");
     }
     st.h2d_ms = nowMs() - t0;
     if (profile && step_events_.size() != plan_->steps.size() + 1) {
       step_events_.assign(plan_->steps.size() + 1, nullptr);
       for (auto& e : step_events_) hipCheck(pml_hip_event_create(&e), "event");
     }
-    hipCheck(pml_hip_event_record(ev0_, nullptr), "event record");
-    for (size_t i = 0; i < plan_->steps.size(); ++i) {
-      if (profile) hipCheck(pml_hip_event_record(step_events_[i], nullptr), "event record");
-      launch(i);
+    // The launches of a run never change (same plans, same device buffers), so from the third run on they are
+    // replayed as one graph recorded during that run; the first two run one by one (first runs of a kernel plan may
+    // allocate, which cannot be recorded).  A recording that fails leaves the executable with one-by-one launches.
+    if (graphable_ && !profile && !graph_ && runs_ >= 2) record();
+    ++runs_;
+    hipCheck(pml_hip_event_record(ev0_, stream_), "event record");
+    if (graph_ && !profile) {
+      hipCheck(pml_hip_graph_launch(graph_, stream_), "graph launch");
+      st.replayed = true;
+    } else {
+      for (size_t i = 0; i < plan_->steps.size(); ++i) {
+        if (profile) hipCheck(pml_hip_event_record(step_events_[i], stream_), "event record");
+        launch(i);
+      }
     }
-    if (profile) hipCheck(pml_hip_event_record(step_events_.back(), nullptr), "event record");
-    hipCheck(pml_hip_event_record(ev1_, nullptr), "event record");
+    if (profile) hipCheck(pml_hip_event_record(step_events_.back(), stream_), "event record");
+    hipCheck(pml_hip_event_record(ev1_, stream_), "event record");
     hipCheck(pml_hip_event_sync(ev1_), "event sync");
     float ms = 0;
     hipCheck(pml_hip_event_elapsed_ms(ev0_, ev1_, &ms), "event elapsed");
     st.kernel_ms = ms;
     st.launches = plan_->steps.size();
+    st.graph_note = graph_note_;
     st.arena_bytes = arena_bytes_;
     st.unshared_temp_bytes = unshared_temp_bytes_;
     st.device_bytes = arena_bytes_ + fixed_bytes_;
@@ -131,7 +150,7 @@ class HipExecutable final : public Executable {
     for (size_t i = 0; i < outputs.size(); ++i) {
       const BufferInfo& b = plan_->buffers[plan_->output_buffers[i]];
       if (outputs[i]->size() < b.bytes) throw std::runtime_error("output buffer #" + std::to_string(i) + " is too small");
-      hipCheck(pml_hip_memcpy_d2h(outputs[i]->data(), device_[plan_->output_buffers[i]], b.bytes, nullptr), "d2h");
+      hipCheck(pml_hip_memcpy_d2h(outputs[i]->data(), device_[plan_->output_buffers[i]], b.bytes, stream_), "d2h");
     }
     st.d2h_ms = nowMs() - t0;
     st.wall_ms = nowMs() - start;
@@ -152,6 +171,34 @@ class HipExecutable final : public Executable {
   std::vector<int64_t> handles_;
   pml_hip_event ev0_ = nullptr, ev1_ = nullptr;
   std::vector<pml_hip_event> step_events_;
+  pml_hip_stream stream_ = nullptr;  // every copy and launch of this executable
+  pml_hip_graph graph_ = nullptr;    // the launches of one run, recorded
+  bool graphable_ = false;
+  int runs_ = 0;
+  std::string graph_note_;
+
+  void record() {
+    if (pml_hip_capture_begin(stream_) != 0) {
+      graph_note_ = pml_hip_last_error();
+      graphable_ = false;
+      return;
+    }
+    bool ok = true;
+    try {
+      for (size_t i = 0; i < plan_->steps.size(); ++i) launch(i);
+    } catch (const std::exception& e) {
+      graph_note_ = e.what();
+      ok = false;
+    }
+    pml_hip_graph g = nullptr;
+    if (pml_hip_capture_end(stream_, &g) != 0 || !ok) {
+      if (ok) graph_note_ = pml_hip_last_error();
+      if (g) pml_hip_graph_destroy(g);
+      graphable_ = false;
+      return;
+    }
+    graph_ = g;
+  }
 
   // Offsets of the temporaries in the arena.  A temporary is live from the first to the last step that names
   // it; steps run in order on one stream, so two temporaries whose spans do not overlap may share bytes.  A
@@ -239,6 +286,10 @@ class HipExecutable final : public Executable {
     if (ev0_) pml_hip_event_destroy(ev0_);
     if (ev1_) pml_hip_event_destroy(ev1_);
     ev0_ = ev1_ = nullptr;
+    if (graph_) pml_hip_graph_destroy(graph_);
+    graph_ = nullptr;
+    if (stream_) pml_hip_stream_destroy(stream_);
+    stream_ = nullptr;
   }
 
   char* ptr(int buf, int64_t elem_off = 0, size_t elem_size = 1) const {
@@ -295,54 +346,54 @@ class HipExecutable final : public Executable {
           const void* b2 = ptr(s.b2, s.b2_off, es);
           if (s.b2_constant && !s.b_is_nk) b2 = nullptr;
           hipCheck(pml_hip_gemm_invoke2(handles_[i], ptr(s.a, s.a_off, es), b, ptr(s.c, s.c_off, elemSize(s.gemm.c_dtype)), ptr(s.init),
-                                        ptr(s.a2, s.a2_off, es), b2, ptr(s.init2), operands, outs, nullptr),
+                                        ptr(s.a2, s.a2_off, es), b2, ptr(s.init2), operands, outs, stream_),
                    s.text.c_str());
           break;
         }
         hipCheck(pml_hip_gemm_invoke(handles_[i], ptr(s.a, s.a_off, es), b, ptr(s.c, s.c_off, elemSize(s.gemm.c_dtype)),
-                                     ptr(s.init), operands, outs, nullptr),
+                                     ptr(s.init), operands, outs, stream_),
                  s.text.c_str());
         break;
       }
       case Step::Conv2d:
         hipCheck(pml_hip_conv2d_invoke(handles_[i], ptr(s.a), s.b_constant ? nullptr : ptr(s.b), ptr(s.c), ptr(s.init), operands,
-                                       outs, nullptr),
+                                       outs, stream_),
                  s.text.c_str());
         break;
       case Step::Dwconv2d:
-        hipCheck(pml_hip_dwconv2d_invoke(handles_[i], ptr(s.a), s.b_constant ? nullptr : ptr(s.b), ptr(s.c), operands, outs, nullptr),
+        hipCheck(pml_hip_dwconv2d_invoke(handles_[i], ptr(s.a), s.b_constant ? nullptr : ptr(s.b), ptr(s.c), operands, outs, stream_),
                  s.text.c_str());
         break;
       case Step::Pool2d:
-        hipCheck(pml_hip_pool2d_invoke(handles_[i], ptr(s.a), ptr(s.c), ptr(s.out2), nullptr), s.text.c_str());
+        hipCheck(pml_hip_pool2d_invoke(handles_[i], ptr(s.a), ptr(s.c), ptr(s.out2), stream_), s.text.c_str());
         break;
       case Step::Eltwise:
-        hipCheck(pml_hip_eltwise_invoke(handles_[i], ptr(s.a), ptr(s.c), operands, outs, nullptr), s.text.c_str());
+        hipCheck(pml_hip_eltwise_invoke(handles_[i], ptr(s.a), ptr(s.c), operands, outs, stream_), s.text.c_str());
         break;
       case Step::Select:
-        hipCheck(pml_hip_select(&s.sel, operands[0], operands[1], operands[2], ptr(s.c), nullptr), s.text.c_str());
+        hipCheck(pml_hip_select(&s.sel, operands[0], operands[1], operands[2], ptr(s.c), stream_), s.text.c_str());
         break;
       case Step::Index:
-        hipCheck(pml_hip_index(ptr(s.c), static_cast<int32_t>(s.index_sizes.size()), s.index_sizes.data(), s.index_axis, nullptr),
+        hipCheck(pml_hip_index(ptr(s.c), static_cast<int32_t>(s.index_sizes.size()), s.index_sizes.data(), s.index_axis, stream_),
                  s.text.c_str());
         break;
       case Step::Contract:
-        hipCheck(pml_hip_contract_invoke(handles_[i], operands, ptr(s.c), nullptr), s.text.c_str());
+        hipCheck(pml_hip_contract_invoke(handles_[i], operands, ptr(s.c), stream_), s.text.c_str());
         break;
       case Step::Copy:
-        hipCheck(pml_hip_memcpy_d2d(ptr(s.c), ptr(s.a), s.copy_bytes, nullptr), s.text.c_str());
+        hipCheck(pml_hip_memcpy_d2d(ptr(s.c), ptr(s.a), s.copy_bytes, stream_), s.text.c_str());
         break;
       case Step::Gather:
-        hipCheck(pml_hip_gather(&s.gat, operands[0], operands[1], ptr(s.c), nullptr), s.text.c_str());
+        hipCheck(pml_hip_gather(&s.gat, operands[0], operands[1], ptr(s.c), stream_), s.text.c_str());
         break;
       case Step::Scatter:
-        hipCheck(pml_hip_scatter(&s.sca, operands[0], operands[1], operands[2], ptr(s.c), nullptr), s.text.c_str());
+        hipCheck(pml_hip_scatter(&s.sca, operands[0], operands[1], operands[2], ptr(s.c), stream_), s.text.c_str());
         break;
       case Step::ArgSort:
-        hipCheck(pml_hip_argsort(&s.srt, operands[0], ptr(s.c), nullptr), s.text.c_str());
+        hipCheck(pml_hip_argsort(&s.srt, operands[0], ptr(s.c), stream_), s.text.c_str());
         break;
       case Step::Prng:
-        hipCheck(pml_hip_prng(operands[0], s.prng_count, s.prng_state ? nullptr : ptr(s.c), s.prng_state ? ptr(s.c) : nullptr, nullptr),
+        hipCheck(pml_hip_prng(operands[0], s.prng_count, s.prng_state ? nullptr : ptr(s.c), s.prng_state ? ptr(s.c) : nullptr, stream_),
                  s.text.c_str());
         break;
     }

@@ -62,6 +62,8 @@ struct InvokeStats {
   size_t unshared_temp_bytes = 0;  // what the temporaries would take with memory of their own
   size_t device_bytes = 0;         // arena + inputs + outputs + constants
   std::vector<double> step_ms;     // per launch, only with PLAIDML_PROFILE=1
+  bool replayed = false;           // the launches ran as one recorded graph
+  std::string graph_note;          // why they did not, when recording was tried and failed
 };
 InvokeStats lastInvokeStats();
 
