@@ -547,6 +547,7 @@ def main():
             # configs[4]: ResNet-50 v1.5, batch 128, bf16, through the plaidml API (weights are program constants)
             extra['resnet50_v1_5_b128_bf16'] = resnet50_leg()
             result['resnet50_b128_img_per_s'] = extra['resnet50_v1_5_b128_bf16']['img_per_s']
+        if want('resnet50_b1'):
             # the same network on one image: latency (few tiles per layer: the K loops of the long-K layers are split
             # over workgroups, the launches replayed as one graph)
             extra['resnet50_v1_5_b1_bf16'] = resnet50_leg(batch=1, runs=20)
