@@ -12,6 +12,13 @@
  * Every function returns 0 on success and a non-zero status on failure unless
  * stated otherwise; pml_hip_last_error() gives the message for the calling
  * thread.  Plain C types only.
+ *
+ * A plan may own device memory that its invokes write: a right-hand side or filter
+ * re-laid per invoke, a re-blocked input or patch matrix of a few-channel
+ * convolution, the partial tiles of a K loop split over workgroups.  Invokes of ONE
+ * plan must therefore not overlap (one stream, or streams ordered by events);
+ * different plans are independent, and dispatching, packing and freeing plans is
+ * safe from several threads.
  */
 #ifndef PML_HIP_H_
 #define PML_HIP_H_
