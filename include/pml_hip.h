@@ -406,7 +406,10 @@ typedef struct {
   int64_t stride_h, stride_w;
   int64_t pad_h, pad_w;
   int32_t with_index;
-  int32_t reserved;
+  /* 0: none.  Otherwise the aggregate, rounded to `dtype`, is divided by this value and rounded again -- a mean written
+   * as sum / count (plaidml/op/lib/ops.cc:1970-2003) in one launch.  ADD over the whole image only (kh = h, kw = w,
+   * no padding, no index); any other descriptor with a divisor is rejected. */
+  float divisor;
 } pml_hip_pool2d_desc;
 
 int64_t pml_hip_pool2d_dispatch(const pml_hip_pool2d_desc* desc);

@@ -1287,6 +1287,16 @@ int64_t pml_hip_pool2d_dispatch(const pml_hip_pool2d_desc* d) {
     fail("pool2d: bad geometry (channels must cover whole 16-byte vectors)");
     return 0;
   }
+  if (d->divisor != 0.f) {
+    // (what pool_whole_kernel takes: pool2d_launch's own test)
+    const int64_t chunks = (d->c / V + 31) / 32;
+    const bool whole = d->agg == PML_HIP_AGG_ADD && d->oh == 1 && d->ow == 1 && d->kh == d->h && d->kw == d->w && d->pad_h == 0 &&
+                       d->pad_w == 0 && !d->with_index && d->h * d->w >= 16 && d->n * chunks <= 0x7fffffff;
+    if (!whole || !(d->divisor == d->divisor)) {
+      fail("pool2d: a divisor goes with the sum over a whole image of at least 16 pixels only");
+      return 0;
+    }
+  }
   Plan* p = new Plan();
   p->kind = PLAN_POOL;
   p->pool = *d;

@@ -938,6 +938,11 @@ __global__ __launch_bounds__(256) void pool_whole_kernel(PoolArgs a, int64_t chu
         acc[i] += y;
     }
   }
+  if (d.divisor != 0.f) {
+    // a mean: the sum is rounded to the element type first, as the separate division would have found it
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = (ES == 2 ? __uint_as_float((uint32_t)f32_to_bf16_bits(acc[i]) << 16) : acc[i]) / d.divisor;
+  }
   const int64_t o0 = n * d.c + cv * V;
   if constexpr (ES == 2) {
     i32x4_t o;

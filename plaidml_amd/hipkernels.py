@@ -90,7 +90,7 @@ class Dwconv2dDesc(ctypes.Structure):
 class Pool2dDesc(ctypes.Structure):
     _fields_ = [('dtype', i32), ('agg', i32), ('n', i64), ('h', i64), ('w', i64), ('c', i64), ('kh', i64), ('kw', i64),
                 ('oh', i64), ('ow', i64), ('stride_h', i64), ('stride_w', i64), ('pad_h', i64), ('pad_w', i64),
-                ('with_index', i32), ('reserved', i32)]
+                ('with_index', i32), ('divisor', ctypes.c_float)]
 
 
 class EltwiseDesc(ctypes.Structure):

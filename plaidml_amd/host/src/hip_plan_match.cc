@@ -494,10 +494,29 @@ bool Planner::tryGlobalPool(size_t i) {
   d.stride_h = d.stride_w = 1;
   d.pad_h = d.pad_w = 0;
   s.a = bufferFor(op.operands[0]);
-  s.c = bufferFor(op.result);
+  // A mean is written as sum / count: the division by a literal, when it is all that follows and the kernel that
+  // sums whole images will run (at least 16 pixels), rides in the same launch.
+  ValuePtr result = op.result;
+  std::string divided;
+  if (op.agg == AggKind::add && d.h * d.w >= 16) {
+    TailBuild tb;
+    extendTail(&tb, op.result, i, /*two_d=*/true, /*allow64=*/false);
+    const bool one_division = tb.tail.n_ops == 1 && tb.tail.ops[0].opcode == PML_HIP_EPI_DIV &&
+                              tb.tail.ops[0].operand_kind == PML_HIP_OPND_IMM && tb.tail.ops[0].dtype == hipType(dt) &&
+                              tb.final_dtype == dt && tb.outs.empty() && tb.tail.ops[0].imm != 0 &&
+                              static_cast<double>(static_cast<float>(tb.tail.ops[0].imm)) == tb.tail.ops[0].imm;
+    if (one_division) {
+      d.divisor = static_cast<float>(tb.tail.ops[0].imm);
+      result = tb.final_value;
+      divided = tailText(tb);
+    } else {
+      unconsume(tb);
+    }
+  }
+  s.c = bufferFor(result);
   s.bytes = static_cast<double>(is.elements() + os.elements()) * util::byteSize(dt);
   s.text = "pool2d " + tile::toString(op.agg) + " " + std::string(util::mnemonic(dt)) + " " + is.str() +
-           " over the whole image -> " + os.str();
+           " over the whole image" + divided + " -> " + os.str();
   plan_->steps.push_back(s);
   return true;
 }

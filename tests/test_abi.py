@@ -56,3 +56,19 @@ def test_dispatch_rejects_bad_descriptors_without_a_gpu():
     e.tail = hk.make_tail(ops=[(hk.EPI_ADD, hk.F32, hk.OPND_TENSOR, 3, 0.0)], operands=[(hk.F32, 0, 1)])
     assert L.pml_hip_eltwise_dispatch(ctypes.byref(e)) == 0
     assert b'outside the operand list' in L.pml_hip_last_error()
+    # a pooling divisor goes with the sum over a whole image only
+    p = hk.Pool2dDesc()
+    p.dtype, p.agg = hk.BF16, hk.AGG_ADD
+    p.n, p.h, p.w, p.c, p.kh, p.kw, p.oh, p.ow = 1, 8, 8, 16, 2, 2, 4, 4
+    p.stride_h = p.stride_w = 2
+    p.divisor = 4.0
+    assert L.pml_hip_pool2d_dispatch(ctypes.byref(p)) == 0
+    assert b'divisor' in L.pml_hip_last_error()
+    p.kh = p.kw = 8
+    p.oh = p.ow = p.stride_h = p.stride_w = 1
+    p.agg = hk.AGG_MAX
+    assert L.pml_hip_pool2d_dispatch(ctypes.byref(p)) == 0
+    p.agg = hk.AGG_ADD
+    plan = L.pml_hip_pool2d_dispatch(ctypes.byref(p))
+    assert plan, L.pml_hip_last_error()
+    L.pml_hip_plan_free(plan)

@@ -90,6 +90,23 @@ def test_one_image_keeps_the_window_kernels():
     assert 'pool2d add bf16 1x7x7x64xbf16 over the whole image' in t, t
 
 
+def test_mean_over_the_image_is_one_launch():
+    """mean = sum / count: the division by the literal rides in the launch that sums whole images (49 pixels: the
+    kernel that shares an image's taps among threads); a 3x3 image (the plain window kernel) keeps it apart, and so
+    does `fuse=0`."""
+    def program(h):
+        X = E.Placeholder(E.DType.BFLOAT16, [2, h, h, 64])
+        return E.Program('mean', [X], [op.mean(X, axes=[1, 2])])
+    t = plan_of(program(7))
+    assert 'over the whole image tail=[div(49)]' in t and 'hip plan: 1 launches' in t, t
+    t = plan_of(program(3))
+    assert 'hip plan: 2 launches' in t and 'eltwise div' in t, t
+    prog = program(7)
+    prog.compile('hip{fuse=0}')
+    t = dict(prog.passes)['hip-plan']
+    assert 'hip plan: 2 launches' in t, t
+
+
 def test_projection_shortcut_and_main_path_share_one_launch():
     """relu(conv1x1(y) + b + conv1x1(x) + b') of a residual block with a projection shortcut is one GEMM with two
     products (plain rows, or the pixel rows of the stride-2 shortcut); `fuse=0` keeps the contractions apart."""

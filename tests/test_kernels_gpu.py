@@ -928,13 +928,15 @@ def test_dwconv_pool_bf16():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('kind,agg,N,H,W,C', [
-    ('bf16', 'add', 3, 7, 7, 2048), ('bf16', 'max', 2, 7, 7, 264), ('bf16', 'min', 2, 10, 13, 64),
-    ('f32', 'add', 2, 7, 7, 516), ('f32', 'max', 1, 9, 8, 128), ('f32', 'add', 2, 4, 4, 36), ('bf16', 'add', 2, 3, 3, 64)])
-def test_pool_whole_image(kind, agg, N, H, W, C):
+@pytest.mark.parametrize('kind,agg,N,H,W,C,divisor', [
+    ('bf16', 'add', 3, 7, 7, 2048, 0), ('bf16', 'max', 2, 7, 7, 264, 0), ('bf16', 'min', 2, 10, 13, 64, 0),
+    ('f32', 'add', 2, 7, 7, 516, 0), ('f32', 'max', 1, 9, 8, 128, 0), ('f32', 'add', 2, 4, 4, 36, 0), ('bf16', 'add', 2, 3, 3, 64, 0),
+    ('bf16', 'add', 3, 7, 7, 2048, 49), ('f32', 'add', 2, 7, 7, 516, 49), ('bf16', 'add', 1, 5, 4, 72, 20)])
+def test_pool_whole_image(kind, agg, N, H, W, C, divisor):
     """Pooling over the whole image (taps shared by eight threads when there are at least 16; the plain window
-    kernel below that) against numpy: max / min exactly, sums to the accumulation tolerance."""
-    print('whole-image pool', kind, agg, N, H, W, C, flush=True)
+    kernel below that) against numpy: max / min exactly, sums to the accumulation tolerance.  With a divisor (a mean
+    as sum / count in one launch) the sum is rounded to the element type before the division, as two launches would."""
+    print('whole-image pool', kind, agg, N, H, W, C, divisor, flush=True)
     rng = np.random.default_rng(N * 1000 + C)
     Iv = rng.standard_normal((N, H, W, C)).astype(np.float32)
     if kind == 'bf16':
@@ -944,6 +946,7 @@ def test_pool_whole_image(kind, agg, N, H, W, C):
     p.agg = {'add': hk.AGG_ADD, 'max': hk.AGG_MAX, 'min': hk.AGG_MIN}[agg]
     p.n, p.h, p.w, p.c, p.kh, p.kw, p.oh, p.ow = N, H, W, C, H, W, 1, 1
     p.stride_h = p.stride_w = 1
+    p.divisor = divisor
     plan = hk.lib().pml_hip_pool2d_dispatch(ctypes.byref(p))
     assert plan, hk.lib().pml_hip_last_error()
     es = 2 if kind == 'bf16' else 4
@@ -953,7 +956,20 @@ def test_pool_whole_image(kind, agg, N, H, W, C):
     hk.check(hk.lib().pml_hip_stream_sync(None))
     out = E.bf16_from_bits(dO.to_numpy(np.uint16, (N, C))) if kind == 'bf16' else dO.to_numpy(np.float32, (N, C))
     flat = Iv.reshape(N, H * W, C)
-    if agg == 'add':
+    if agg == 'add' and divisor:
+        # the two-launch form on the same device: sum, then the division as an elementwise launch of its own
+        p.divisor = 0
+        plan0 = hk.lib().pml_hip_pool2d_dispatch(ctypes.byref(p))
+        dS = hk.DeviceBuffer(N * C * es)
+        hk.check(hk.lib().pml_hip_pool2d_invoke(plan0, dI.ptr, dS.ptr, None, None))
+        hk.check(hk.lib().pml_hip_stream_sync(None))
+        sums = E.bf16_from_bits(dS.to_numpy(np.uint16, (N, C))) if kind == 'bf16' else dS.to_numpy(np.float32, (N, C))
+        apart = (sums.astype(np.float32) / np.float32(divisor)).astype(np.float32)
+        np.testing.assert_array_equal(out, E.round_bf16(apart) if kind == 'bf16' else apart)
+        np.testing.assert_allclose(out, flat.astype(np.float64).sum(1) / divisor, rtol=BF16_RTOL if kind == 'bf16' else 1e-5,
+                                   atol=2e-2 if kind == 'bf16' else 1e-5)
+        hk.lib().pml_hip_plan_free(plan0)
+    elif agg == 'add':
         ref = flat.astype(np.float64).sum(1)
         np.testing.assert_allclose(out, ref, rtol=BF16_RTOL if kind == 'bf16' else 1e-5, atol=2e-2 if kind == 'bf16' else 1e-5)
     else:
