@@ -435,6 +435,18 @@ int64_t pml_hip_eltwise_dispatch(const pml_hip_eltwise_desc* desc);
 int pml_hip_eltwise_invoke(int64_t plan, const void* input, void* output, const void* const* operands,
                            void* const* outs, pml_hip_stream s);
 
+/* ---- softmax over the last axis -------------------------------------------------
+ * y[r, c] = e[r, c] / sum_c e[r, c] with e[r, c] = exp(x[r, c] - max_c x[r, c]): the five operations the op library
+ * composes a softmax from (plaidml/op/lib/ops.cc:3049-3098: contraction max, sub, exp, contraction add, div) in one
+ * launch instead of four, every intermediate rounded to `dtype` as those operations round it (the maximum by
+ * `v > acc ? v : acc` from -inf, the sum accumulated in fp32 and rounded once).  x and y are dense [rows][cols]. */
+typedef struct {
+  int32_t dtype; /* F32 or BF16 */
+  int32_t reserved;
+  int64_t rows, cols;
+} pml_hip_softmax_desc;
+int pml_hip_softmax(const pml_hip_softmax_desc* desc, const void* x, void* y, pml_hip_stream s);
+
 /* three-input select(cond, t, f) with broadcasting (tile.select, SelectOp of
  * pmlc/conversion/tile_to_linalg/tile_to_linalg.cc:262-273) */
 typedef struct {
@@ -569,7 +581,7 @@ int pml_hip_contract_invoke(int64_t plan, const void* const* srcs, void* out, pm
 
 /* sizeof() of a descriptor struct as this library was compiled, so that a foreign-language
  * binding can verify its own layout: 0 epilogue, 1 gemm, 2 conv2d, 3 dwconv2d, 4 pool2d,
- * 5 eltwise, 6 select, 7 contract, 8 form, 9 gather, 10 scatter, 11 argsort.  Returns 0 for an unknown id. */
+ * 5 eltwise, 6 select, 7 contract, 8 form, 9 gather, 10 scatter, 11 argsort, 12 softmax.  Returns 0 for an unknown id. */
 size_t pml_hip_struct_size(int which);
 
 /* Releases a plan returned by any *_dispatch. */

@@ -915,6 +915,55 @@ hipError_t index_launch(void* out, int rank, const int64_t* sizes, int axis, hip
   return hipGetLastError();
 }
 
+// Softmax over the last axis: a workgroup per row, three walks over the row (maximum, sum of exponentials, quotients;
+// rows are short and stay in the caches), each reduction folded through the wavefronts' lanes and then through LDS in
+// a fixed order.  BF: every intermediate is rounded to bf16 where the separate operations would have stored it.
+template <bool BF>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const void* x_, void* y_, int64_t cols) {
+  __shared__ float part[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = blockIdx.x;
+  auto load = [&](int64_t c) {
+    if constexpr (BF) return bf16_bits_to_f32(((const uint16_t*)x_)[row * cols + c]);
+    return ((const float*)x_)[row * cols + c];
+  };
+  auto rounded = [](float v) { return BF ? round_to_bf16(v) : v; };
+  auto across = [&](float v, auto fold) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v = fold(v, __shfl_xor(v, d, 64));
+    __syncthreads();  // (the previous reduction's readers are done with `part`)
+    if (lane == 0) part[wave] = v;
+    __syncthreads();
+    return fold(fold(part[0], part[1]), fold(part[2], part[3]));
+  };
+  float m = -INFINITY;
+  for (int64_t c = tid; c < cols; c += 256) {
+    const float v = load(c);
+    m = v > m ? v : m;
+  }
+  m = across(m, [](float a, float b) { return b > a ? b : a; });
+  float sum = 0.f;
+  for (int64_t c = tid; c < cols; c += 256) sum += rounded(expf(rounded(load(c) - m)));
+  sum = rounded(across(sum, [](float a, float b) { return a + b; }));
+  for (int64_t c = tid; c < cols; c += 256) {
+    const float q = rounded(rounded(expf(rounded(load(c) - m))) / sum);
+    if constexpr (BF)
+      ((uint16_t*)y_)[row * cols + c] = f32_to_bf16_bits(q);
+    else
+      ((float*)y_)[row * cols + c] = q;
+  }
+}
+
+hipError_t softmax_launch(const pml_hip_softmax_desc& d, const void* x, void* y, hipStream_t s) {
+  if (d.rows == 0 || d.cols == 0) return hipSuccess;
+  if (d.rows > 0x7fffffff) return hipErrorInvalidValue;
+  if (d.dtype == PML_HIP_BF16)
+    hipLaunchKernelGGL(softmax_rows_kernel<true>, dim3((unsigned)d.rows), dim3(256), 0, s, x, y, d.cols);
+  else
+    hipLaunchKernelGGL(softmax_rows_kernel<false>, dim3((unsigned)d.rows), dim3(256), 0, s, x, y, d.cols);
+  return hipGetLastError();
+}
+
 hipError_t fill_u32_launch(void* p, uint32_t pattern, size_t n_words, hipStream_t s) {
   if (n_words == 0) return hipSuccess;
   hipLaunchKernelGGL(fill_kernel, dim3(grid_for((int64_t)n_words)), dim3(256), 0, s, (uint32_t*)p, pattern, n_words);

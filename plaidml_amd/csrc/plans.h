@@ -260,6 +260,7 @@ hipError_t select_launch(const pml_hip_select_desc& d, const void* c, const void
                          hipStream_t s);
 hipError_t index_launch(void* out, int rank, const int64_t* sizes, int axis, hipStream_t s);
 hipError_t fill_u32_launch(void* p, uint32_t pattern, size_t n_words, hipStream_t s);
+hipError_t softmax_launch(const pml_hip_softmax_desc& d, const void* x, void* y, hipStream_t s);
 
 // special operations (special.hip)
 hipError_t gather_launch(const pml_hip_gather_desc& d, const void* tensor, const void* indices, void* out, hipStream_t s);

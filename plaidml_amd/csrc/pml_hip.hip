@@ -1384,6 +1384,13 @@ int pml_hip_select(const pml_hip_select_desc* d, const void* cond, const void* t
   return check(select_launch(*d, cond, t, f, out, (hipStream_t)s), "select_launch");
 }
 
+int pml_hip_softmax(const pml_hip_softmax_desc* d, const void* x, void* y, pml_hip_stream s) {
+  if (!d || !x || !y) return fail("softmax: null argument");
+  if (d->dtype != PML_HIP_F32 && d->dtype != PML_HIP_BF16) return fail("softmax: dtype must be F32 or BF16");
+  if (d->rows < 0 || d->cols < 0 || d->rows > 0x7fffffff) return fail("softmax: rows or cols out of range");
+  return check(softmax_launch(*d, x, y, (hipStream_t)s), "softmax_launch");
+}
+
 int pml_hip_index(void* out, int32_t rank, const int64_t* sizes, int32_t axis, pml_hip_stream s) {
   if (!out || !sizes || rank <= 0 || axis < 0 || axis >= rank) return fail("index: bad argument");
   return check(index_launch(out, rank, sizes, axis, (hipStream_t)s), "index_launch");
@@ -1572,6 +1579,7 @@ size_t pml_hip_struct_size(int which) {
     case 9: return sizeof(pml_hip_gather_desc);
     case 10: return sizeof(pml_hip_scatter_desc);
     case 11: return sizeof(pml_hip_argsort_desc);
+    case 12: return sizeof(pml_hip_softmax_desc);
   }
   return 0;
 }

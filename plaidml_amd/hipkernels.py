@@ -47,7 +47,7 @@ EXPORTS = [
     'pml_hip_gemm_run_static', 'pml_hip_gemm_invoke2', 'pml_hip_gemm_pack_b2', 'pml_hip_probe_mfma', 'pml_hip_dwconv2d_pack_filter', 'pml_hip_tile_of_workgroup', 'pml_hip_tile_name', 'pml_hip_tile_by_name', 'pml_hip_gemm_tail_cheaper_apart',
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
-    'pml_hip_select', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
+    'pml_hip_select', 'pml_hip_softmax', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
     'pml_hip_plan_describe', 'pml_hip_struct_size', 'pml_hip_gemm_pack_b', 'pml_hip_conv2d_pack_filter',
     'pml_hip_gather', 'pml_hip_scatter', 'pml_hip_argsort', 'pml_hip_prng',
 ]
@@ -135,6 +135,10 @@ class ArgsortDesc(ctypes.Structure):
     _fields_ = [('dtype', i32), ('rank', i32), ('axis', i32), ('direction', i32), ('sizes', i64 * MAX_SPECIAL_RANK)]
 
 
+class SoftmaxDesc(ctypes.Structure):
+    _fields_ = [('dtype', i32), ('reserved', i32), ('rows', i64), ('cols', i64)]
+
+
 _lib = None
 
 
@@ -182,6 +186,7 @@ def lib():
         L.pml_hip_pool2d_invoke.argtypes = [ctypes.c_int64, vp, vp, vp, vp]
         L.pml_hip_eltwise_invoke.argtypes = [ctypes.c_int64, vp, vp, pp, pp, vp]
         L.pml_hip_select.argtypes = [ctypes.POINTER(SelectDesc), vp, vp, vp, vp, vp]
+        L.pml_hip_softmax.argtypes = [ctypes.POINTER(SoftmaxDesc), vp, vp, vp]
         L.pml_hip_index.argtypes = [vp, i32, ctypes.POINTER(i64), i32, vp]
         L.pml_hip_contract_invoke.argtypes = [ctypes.c_int64, pp, vp, vp]
         L.pml_hip_plan_free.argtypes = [ctypes.c_int64]

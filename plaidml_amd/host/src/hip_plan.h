@@ -26,7 +26,7 @@ struct BufferInfo {
 };
 
 struct Step {
-  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy, Gather, Scatter, ArgSort, Prng } kind = Copy;
+  enum Kind { Gemm, Conv2d, Dwconv2d, Pool2d, Eltwise, Select, Index, Contract, Copy, Gather, Scatter, ArgSort, Prng, Softmax } kind = Copy;
   std::string text;  // one line for the plan dump
   std::string schedule;  // "{tile=...,conv=...}" when the target options or a schedule file named this step's tiling
   // descriptors (only the one matching `kind` is meaningful)
@@ -40,6 +40,7 @@ struct Step {
   pml_hip_gather_desc gat{};
   pml_hip_scatter_desc sca{};
   pml_hip_argsort_desc srt{};
+  pml_hip_softmax_desc sm{};
   int64_t prng_count = 0;   // Prng: values drawn
   bool prng_state = false;  //       the step yields the advanced state instead of the values
   int index_axis = 0;

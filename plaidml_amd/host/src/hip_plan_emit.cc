@@ -268,6 +268,7 @@ void Planner::emitContraction(size_t i) {
     if (tryDepthwise(i)) return;
     if (tryPool(i)) return;
     if (tryGlobalPool(i)) return;
+    if (opt_.fuse && trySoftmax(i)) return;
   }
   emitGeneral(i);
 }

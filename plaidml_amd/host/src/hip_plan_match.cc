@@ -622,4 +622,94 @@ bool Planner::matchWindowArgmax(size_t ui, const Op& pool, const pml_hip_pool2d_
   return isWindowIota(u.operands[2], pd.kh, pd.kw);
 }
 
+// agg over the last axis of one dense operand, nothing else: O[x0, .., 0] = agg_{x_last} I[x0, .., x_last]
+bool Planner::reducesLastAxis(const Op& op, AggKind agg) {
+  if (op.kind != Op::Contraction || op.agg != agg || op.combo != ComboKind::none || op.operands.size() != 1 || op.init) return false;
+  if (!op.constraints.empty() || op.accesses.size() != 2) return false;
+  const TensorShape &is = op.operands[0]->shape, &os = op.result->shape;
+  const size_t r = is.getRank();
+  if (r < 1 || os.getRank() != r || op.idxNames.size() != r || op.accesses[0].size() != r || op.accesses[1].size() != r) return false;
+  if (os.elementType != is.elementType || os.sizes[r - 1] != 1) return false;
+  std::vector<bool> seen(r, false);
+  for (size_t d = 0; d < r; ++d) {
+    const int v = op.accesses[1][d].plainIndex();
+    if (v < 0 || seen[v]) return false;
+    seen[v] = true;
+    if (op.lower[v] != 0 || op.upper[v] != is.sizes[d] - 1) return false;  // the whole tensor
+    if (d + 1 < r) {
+      if (os.sizes[d] != is.sizes[d] || op.accesses[0][d].plainIndex() != v) return false;
+    } else if (!(op.accesses[0][d].isConstant() && op.accesses[0][d].c0 == 0)) {
+      return false;
+    }
+  }
+  return true;
+}
+
+// The op library's softmax (plaidml/op/lib/ops.cc:3049-3098) -- M = max over the last axis, E = exp(X - M), S = sum of
+// E over the last axis, E / S -- with every intermediate value used by nothing else: one launch of the softmax kernel
+// in place of two reductions and two elementwise launches.  `i` is the max contraction.
+bool Planner::trySoftmax(size_t i) {
+  Op& mx = prog_->ops[i];
+  if (!reducesLastAxis(mx, AggKind::max)) return false;
+  const ValuePtr X = mx.operands[0];
+  const DataType dt = X->shape.elementType;
+  if (dt != DataType::f32 && dt != DataType::bf16) return false;
+  // the only user of a value that is no program output, or npos
+  auto only_user = [&](const ValuePtr& v) -> size_t {
+    if (outputs_.count(v.get())) return std::string::npos;
+    const auto it = users_.find(v.get());
+    if (it == users_.end() || it->second.empty()) return std::string::npos;
+    for (size_t u : it->second)
+      if (u != it->second.front() || consumed_.count(u)) return std::string::npos;
+    return it->second.front();
+  };
+  auto same_shape = [&](const ValuePtr& v) { return v->shape.sizes == X->shape.sizes && v->shape.elementType == dt; };
+  const size_t si = only_user(mx.result);
+  if (si == std::string::npos) return false;
+  const Op& sub = prog_->ops[si];
+  if (sub.kind != Op::Eltwise || sub.fn != "sub" || sub.operands.size() != 2 || sub.operands[0] != X || sub.operands[1] != mx.result ||
+      !same_shape(sub.result))
+    return false;
+  const size_t ei = only_user(sub.result);
+  if (ei == std::string::npos) return false;
+  const Op& ex = prog_->ops[ei];
+  if (ex.kind != Op::Eltwise || ex.fn != "exp" || ex.operands.size() != 1 || !same_shape(ex.result)) return false;
+  const ValuePtr E = ex.result;
+  if (outputs_.count(E.get())) return false;
+  const auto eu = users_.find(E.get());
+  if (eu == users_.end()) return false;
+  std::set<size_t> e_users(eu->second.begin(), eu->second.end());
+  if (e_users.size() != 2) return false;
+  size_t sum_i = std::string::npos, div_i = std::string::npos;
+  for (size_t u : e_users) {
+    if (consumed_.count(u)) return false;
+    if (prog_->ops[u].kind == Op::Contraction)
+      sum_i = u;
+    else
+      div_i = u;
+  }
+  if (sum_i == std::string::npos || div_i == std::string::npos) return false;
+  Op& sm = prog_->ops[sum_i];
+  if (!sm.boundsComputed) tile::computeBounds(&sm);
+  if (!reducesLastAxis(sm, AggKind::add) || sm.operands[0] != E) return false;
+  const Op& dv = prog_->ops[div_i];
+  if (dv.kind != Op::Eltwise || dv.fn != "div" || dv.operands.size() != 2 || dv.operands[0] != E || dv.operands[1] != sm.result ||
+      !same_shape(dv.result))
+    return false;
+  if (only_user(sm.result) != div_i) return false;
+  const size_t r = X->shape.getRank();
+  Step s;
+  s.kind = Step::Softmax;
+  s.sm.dtype = hipType(dt);
+  s.sm.cols = X->shape.sizes[r - 1];
+  s.sm.rows = X->shape.sizes[r - 1] ? static_cast<int64_t>(X->shape.elements()) / X->shape.sizes[r - 1] : 0;
+  s.a = bufferFor(X);
+  s.c = bufferFor(dv.result);
+  for (size_t k : {si, ei, sum_i, div_i}) consumed_.insert(k);
+  s.bytes = 2.0 * static_cast<double>(X->shape.elements()) * util::byteSize(dt);
+  s.text = "softmax " + std::string(util::mnemonic(dt)) + " over the last axis of " + X->shape.str() + " -> " + dv.result->shape.str();
+  plan_->steps.push_back(s);
+  return true;
+}
+
 }  // namespace pmlc::target::hip

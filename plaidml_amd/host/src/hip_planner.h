@@ -219,6 +219,8 @@ class Planner {
   bool tryPool(size_t i);
   bool isWindowIota(const ValuePtr& ix, int64_t kh, int64_t kw);
   bool matchWindowArgmax(size_t ui, const Op& pool, const pml_hip_pool2d_desc& pd);
+  static bool reducesLastAxis(const Op& op, AggKind agg);
+  bool trySoftmax(size_t i);
 
   // ----- the general contraction kernel ---------------------------------------------------
 

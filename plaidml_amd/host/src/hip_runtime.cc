@@ -75,7 +75,8 @@ class HipExecutable final : public Executable {
       graphable_ = plan_->graph && plan_->steps.size() > 1;
       for (const Step& s : plan_->steps)
         if (s.kind != Step::Gemm && s.kind != Step::Conv2d && s.kind != Step::Dwconv2d && s.kind != Step::Pool2d &&
-            s.kind != Step::Eltwise && s.kind != Step::Contract && s.kind != Step::Select && s.kind != Step::Copy)
+            s.kind != Step::Eltwise && s.kind != Step::Contract && s.kind != Step::Select && s.kind != Step::Copy &&
+            s.kind != Step::Softmax)
           graphable_ = false;
     } catch (...) {
       release();
@@ -318,6 +319,7 @@ class HipExecutable final : public Executable {
       case Step::Scatter:
       case Step::ArgSort:
       case Step::Prng:
+      case Step::Softmax:
       case Step::Copy: return;
     }
     if (!h) throw std::runtime_error("hip dispatch failed for '" + s.text + "': " + pml_hip_last_error());
@@ -372,6 +374,9 @@ class HipExecutable final : public Executable {
         break;
       case Step::Select:
         hipCheck(pml_hip_select(&s.sel, operands[0], operands[1], operands[2], ptr(s.c), stream_), s.text.c_str());
+        break;
+      case Step::Softmax:
+        hipCheck(pml_hip_softmax(&s.sm, ptr(s.a), ptr(s.c), stream_), s.text.c_str());
         break;
       case Step::Index:
         hipCheck(pml_hip_index(ptr(s.c), static_cast<int32_t>(s.index_sizes.size()), s.index_sizes.data(), s.index_axis, stream_),

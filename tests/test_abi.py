@@ -27,7 +27,7 @@ def test_descriptor_layouts_match():
     L = hk.lib()
     for which, cls in enumerate([hk.Epilogue, hk.GemmDesc, hk.Conv2dDesc, hk.Dwconv2dDesc, hk.Pool2dDesc,
                                  hk.EltwiseDesc, hk.SelectDesc, hk.ContractDesc, hk.Form, hk.GatherDesc, hk.ScatterDesc,
-                                 hk.ArgsortDesc]):
+                                 hk.ArgsortDesc, hk.SoftmaxDesc]):
         assert L.pml_hip_struct_size(which) == ctypes.sizeof(cls), cls.__name__
 
 

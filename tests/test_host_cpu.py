@@ -90,6 +90,28 @@ def test_one_image_keeps_the_window_kernels():
     assert 'pool2d add bf16 1x7x7x64xbf16 over the whole image' in t, t
 
 
+def test_softmax_is_one_launch():
+    """The op library's softmax (max, sub, exp, sum, div) is recognised as a whole when nothing else reads its
+    intermediate values; an intermediate that is also a program output keeps the five operations apart."""
+    X = E.Placeholder(E.DType.BFLOAT16, [4, 1000])
+    t = plan_of(E.Program('sm', [X], [op.softmax(X, axis=1)]))
+    assert 'hip plan: 1 launches' in t and 'softmax bf16 over the last axis of 4x1000xbf16' in t, t
+    X = E.Placeholder(E.DType.FLOAT32, [2, 3, 10])
+    t = plan_of(E.Program('sm3', [X], [op.softmax(X, axis=2)]))
+    assert 'hip plan: 1 launches' in t and 'softmax f32' in t, t
+    X = E.Placeholder(E.DType.FLOAT32, [4, 10])
+    i, j = E.TensorIndexes(2)
+    M = E.Contraction().outShape(4, 1).outAccess(i, 0).max(X[i, j]).build()
+    Ex = E.exp(X - M)
+    S = E.Contraction().outShape(4, 1).outAccess(i, 0).sum(Ex[i, j]).build()
+    t = plan_of(E.Program('sm_visible', [X], [Ex / S, Ex]))
+    assert 'softmax' not in t and 'hip plan: 4 launches' in t, t
+    X = E.Placeholder(E.DType.BFLOAT16, [4, 1000])
+    prog = E.Program('sm', [X], [op.softmax(X, axis=1)])
+    prog.compile('hip{fuse=0}')
+    assert 'softmax' not in dict(prog.passes)['hip-plan']
+
+
 def test_mean_over_the_image_is_one_launch():
     """mean = sum / count: the division by the literal rides in the launch that sums whole images (49 pixels: the
     kernel that shares an image's taps among threads); a 3x3 image (the plain window kernel) keeps it apart, and so

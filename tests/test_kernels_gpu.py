@@ -977,6 +977,33 @@ def test_pool_whole_image(kind, agg, N, H, W, C, divisor):
     hk.lib().pml_hip_plan_free(plan)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize('kind,rows,cols', [('bf16', 1, 1000), ('bf16', 128, 1000), ('f32', 3, 5), ('f32', 2, 4097), ('bf16', 5, 257)])
+def test_softmax_rows(kind, rows, cols):
+    """pml_hip_softmax against the five operations it stands for, evaluated in numpy with the roundings they would make
+    (bf16: after the subtraction, the exponential, the sum and the quotient).  The fp32 sum is accumulated in another
+    order than numpy's, so sums and quotients are compared to a few units in the last place of the result type."""
+    print('softmax', kind, rows, cols, flush=True)
+    rng = np.random.default_rng(rows * 31 + cols)
+    X = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    rnd = E.round_bf16 if kind == 'bf16' else (lambda a: a.astype(np.float32))
+    X = rnd(X)
+    d = hk.SoftmaxDesc()
+    d.dtype, d.rows, d.cols = (hk.BF16 if kind == 'bf16' else hk.F32), rows, cols
+    dX = hk.DeviceBuffer.from_numpy(bf16(X) if kind == 'bf16' else X)
+    dY = hk.DeviceBuffer(rows * cols * (2 if kind == 'bf16' else 4))
+    hk.check(hk.lib().pml_hip_softmax(ctypes.byref(d), dX.ptr, dY.ptr, None))
+    hk.check(hk.lib().pml_hip_stream_sync(None))
+    Y = E.bf16_from_bits(dY.to_numpy(np.uint16, (rows, cols))) if kind == 'bf16' else dY.to_numpy(np.float32, (rows, cols))
+    m = X.max(axis=1, keepdims=True)
+    e = rnd(np.exp(rnd(X - m).astype(np.float64)).astype(np.float32))
+    ssum = rnd(e.astype(np.float64).sum(axis=1, keepdims=True).astype(np.float32))
+    ref = rnd((e / ssum).astype(np.float32))
+    tol = 2.0 ** -7 if kind == 'bf16' else 1e-5   # one bf16 step of the sum moves every quotient of its row by one step
+    np.testing.assert_allclose(Y, ref, rtol=tol, atol=1e-30)
+    np.testing.assert_allclose(Y.astype(np.float64).sum(axis=1), 1.0, rtol=0, atol=2e-2 if kind == 'bf16' else 1e-5)
+
+
 # (kind, agg, N, H, W, C, kh, kw, stride, pad, with_index): the straight-line kernels (3x3, 2x2) and the window loop
 # (5x5, 3x2), windows that cross every border, one image and several, values quantised so that ties occur
 POOL_WINDOW_CASES = [
