@@ -227,17 +227,27 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
   // the last MFMAs must have written the accumulators before the lane exchange below reads them: the compiler
   // cannot see that read (it is assembler text), so the longest MFMA's passes are waited out here, once
   asm volatile("s_nop 15\n\ts_nop 3");
+  // Order of the wavefront's 32x32 blocks.  With several block columns the blocks of a block row follow one another
+  // (and the column vectors, hot in L1, are fetched again for every block): the 64-byte pieces that share a 128-byte
+  // line of a result row are then stored within a few instructions of each other and leave L2 as one line.  With the
+  // column blocks outermost a 192x384 tile wrote 1.86 x its result to memory (WRITE_SIZE 61.0 MB for 33.6 MB at
+  // 23104 x 728 x 728: lines left L2 half-written and were written again), a 256x256 tile 1.50 x.
+  constexpr bool kRowsOuter = NI > 1;
+  bool col_ok[2];
+  float bias[2][8], mul[2][8], add[2][8];
 #pragma unroll
-  for (int j = 0; j < NI; ++j) {
+  for (int outer = 0; outer < (kRowsOuter ? MI : NI); ++outer) {
+#pragma unroll
+    for (int inner = 0; inner < (kRowsOuter ? NI : MI); ++inner) {
+    const int i = kRowsOuter ? outer : inner, j = kRowsOuter ? inner : outer;
+    if (kRowsOuter || inner == 0) {
     // the lane's two 8-column pieces of this block; one past the last column (a ragged last tile) is left out
-    bool col_ok[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) col_ok[q] = nw + j * 32 + 16 * q + 8 * hi < p.N;
     auto column_vector = [&](const uint16_t* src, int q, float* out) {
       const i32x4_t bits = (src != nullptr && col_ok[q]) ? *(const i32x4_t*)(src + nw + j * 32 + 16 * q + 8 * hi) : i32x4_t{0, 0, 0, 0};
       unpack_bf16x8(bits, out);
     };
-    float bias[2][8], mul[2][8], add[2][8];
     if (has_bias) {
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
@@ -255,8 +265,8 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
         column_vector(shift, q, add[q]);
       }
     }
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
+    }
+    {
       // Memory is touched 64 bytes of a row at a time: access t (0, 1) of the block covers rows 16 t .. 16 t + 15, lane l
       // the eight columns from mcol = 16 ((l / 16) % 2) + 8 (l / 32) of row 16 t + l % 16 -- four lanes per row.  The
       // values are worked on in the accumulators' arrangement (lane l: row l % 32, pieces q = 0, 1 at columns
@@ -338,6 +348,7 @@ __device__ __forceinline__ void direct_tail_bf16(const IgemmArgs& p, f32x16_t (&
         const int64_t m = mw + i * 32 + 16 * t + (lane & 15);
         if (m < p.M && mcol_ok) *(i32x4_t*)((uint16_t*)p.C + m * p.ldc + nw + j * 32 + mcol) = packed[t];
       }
+    }
     }
   }
 }
