@@ -745,7 +745,7 @@ hipError_t launch_splitk(const IgemmArgs& a, hipStream_t s) {
   } else {
     const int64_t tiles_m = (a.M + 63) / 64, tiles_n = (a.N + 63) / 64;
     const int64_t tiles = tiles_m * tiles_n;
-    if (tiles <= 0 || tiles * a.sk_splits >= ((int64_t)1 << 31) || a.K2 > 0 || a.b_kn || !a.ws || a.sk_splits < 2) return hipErrorInvalidValue;
+    if (tiles <= 0 || tiles * a.sk_splits >= ((int64_t)1 << 31) || a.b_kn || !a.ws || a.sk_splits < 2) return hipErrorInvalidValue;
     const size_t lds = Ring<64, 64, 0, 128>::kAlloc;
     auto kern = igemm_kernel<KIND, 64, 64, 2, CONV, kThreads, 0, 1, 128, false, true>;
     static DynamicLdsLimit limit;

@@ -683,8 +683,9 @@ int64_t pml_hip_gemm_dispatch(const pml_hip_gemm_desc* d) {
     int mode = 0, relu = 0;
     classify_tail(d->tail, d->out_dtype, d->c_dtype, &mode, &relu);
     const bool plain = mode == 1 || mode == 2 || tail_requant(d->tail, d->out_dtype, d->c_dtype, mode, nullptr);
-    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags), /*allow_split=*/d->k2 == 0);
-    if (d->k2 == 0) prepare_split(p, d->m, d->n, (d->k * dt_size(d->in_dtype) + 127) / 128);
+    p->tile = choose_tile(d->m, d->n, (d->k + d->k2) * dt_size(d->in_dtype), kind, plain, PML_HIP_FLAG_TILE_OF(d->flags));
+    // (a second product's slabs follow the first one's on the slab axis the splits share out)
+    prepare_split(p, d->m, d->n, (d->k * dt_size(d->in_dtype) + 127) / 128 + (d->k2 * dt_size(d->in_dtype) + 127) / 128);
   }
   p->bt_ld = d->k;
   p->bt_bytes = (size_t)d->n * d->k * es;

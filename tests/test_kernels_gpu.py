@@ -146,16 +146,19 @@ def test_gemm_f32_as_three_bf16_products(M, N, K):
     np.testing.assert_array_equal(run_gemm(Ai, Bi, hk.F32, hk.F32, flags=hk.FP32_AS_BF16X3), Ai @ Bi)
 
 
+@pytest.mark.parametrize('long_k', [False, True])
 @pytest.mark.parametrize('stride', [0, 2])
-def test_gemm_two_products(stride):
+def test_gemm_two_products(stride, long_k):
     """C = relu(A.B + b + A2.B2 + b2) in one launch: the second left-hand side as plain rows, and as the pixel rows a
-    1x1 convolution with stride 2 reads from an NHWC image (a residual block's projection shortcut)."""
+    1x1 convolution with stride 2 reads from an NHWC image (a residual block's projection shortcut).  With few tiles and
+    long K's (the shortcut of a network's last stage at batch 1) the slabs of both products are shared out among
+    workgroups; a split then begins in the middle of the first product or in the second."""
     rng = np.random.default_rng(21)
-    NB, OH, OW, K1, K2, N = 3, 7, 9, 72, 40, 136
+    NB, OH, OW, K1, K2, N = (1, 7, 7, 520, 1024, 136) if long_k else (3, 7, 9, 72, 40, 136)
     M = NB * OH * OW
     A = E.round_bf16(rng.standard_normal((M, K1)).astype(np.float32))
-    B = E.round_bf16(rng.standard_normal((K1, N)).astype(np.float32) * 0.2)
-    B2 = E.round_bf16(rng.standard_normal((K2, N)).astype(np.float32) * 0.2)
+    B = E.round_bf16(rng.standard_normal((K1, N)).astype(np.float32) * (0.2 if not long_k else 0.05))
+    B2 = E.round_bf16(rng.standard_normal((K2, N)).astype(np.float32) * (0.2 if not long_k else 0.05))
     b1 = E.round_bf16(rng.standard_normal(N).astype(np.float32))
     b2 = E.round_bf16(rng.standard_normal(N).astype(np.float32))
     if stride:
@@ -178,6 +181,7 @@ def test_gemm_two_products(stride):
     plan = L.pml_hip_gemm_dispatch(ctypes.byref(d))
     assert plan, L.pml_hip_last_error()
     print('plan:', hk.describe(plan), flush=True)
+    assert ('K split over workgroups' in hk.describe(plan)) == long_k
     bufs = [hk.DeviceBuffer.from_numpy(bf16(x)) for x in (A, B, b1, a2_dev, B2, b2)]
     dC = hk.DeviceBuffer(M * N * 2)
     none = hk.ptr_array([])
@@ -188,7 +192,7 @@ def test_gemm_two_products(stride):
     hk.check(L.pml_hip_stream_sync(None))
     C = E.bf16_from_bits(dC.to_numpy(np.uint16, (M, N)))
     ref = np.maximum(A.astype(np.float64) @ B + A2.astype(np.float64) @ B2 + b1 + b2, 0)
-    np.testing.assert_allclose(C, ref, rtol=BF16_RTOL, atol=BF16_RTOL)
+    np.testing.assert_allclose(C, ref, rtol=BF16_RTOL, atol=BF16_RTOL if not long_k else 4e-2)
     L.pml_hip_plan_free(plan)
 
 
