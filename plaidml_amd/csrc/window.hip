@@ -592,10 +592,10 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
     if (dt == PML_HIP_BF16 || dt == PML_HIP_F32) {
       // one 16-byte store of the rounded values
       if constexpr (ES == 2) {
-        *(i32x4_t*)((uint16_t*)a.out + o0) = pack_bf16_rne(acc);
+        store_streaming((i32x4_t*)((uint16_t*)a.out + o0), pack_bf16_rne(acc));
       } else {
         const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
-        *(f32x4_t*)((float*)a.out + o0) = o;
+        store_streaming((f32x4_t*)((float*)a.out + o0), o);
       }
     } else {
 #pragma unroll
@@ -611,7 +611,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a, int64_t total_v
 #pragma unroll
       for (int i = 0; i < V; i += 4) {
         i32x4_t w = {best[i], best[i + 1], best[i + 2], best[i + 3]};
-        *(i32x4_t*)(ip + i) = w;
+        store_streaming((i32x4_t*)(ip + i), w);
       }
     }
   }
@@ -700,17 +700,17 @@ __global__ __launch_bounds__(256) void pool_flat_kernel(PoolArgs a, PoolFlatArgs
     }
   const unsigned o0 = pix * (unsigned)d.c + cv * V;  // in elements
   if constexpr (ES == 2) {
-    *(i32x4_t*)((uint16_t*)a.out + o0) = pack_bf16_rne(acc);
+    store_streaming((i32x4_t*)((uint16_t*)a.out + o0), pack_bf16_rne(acc));
   } else {
     const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
-    *(f32x4_t*)((float*)a.out + o0) = o;
+    store_streaming((f32x4_t*)((float*)a.out + o0), o);
   }
   if (WITH_INDEX) {
     int32_t* ip = (int32_t*)a.idx + o0;
 #pragma unroll
     for (int i = 0; i < V; i += 4) {
       const i32x4_t w = {best[i], best[i + 1], best[i + 2], best[i + 3]};
-      *(i32x4_t*)(ip + i) = w;
+      store_streaming((i32x4_t*)(ip + i), w);
     }
   }
 }
@@ -949,10 +949,10 @@ __global__ __launch_bounds__(256) void pool_whole_kernel(PoolArgs a, int64_t chu
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       o[i] = (int)((uint32_t)f32_to_bf16_bits(acc[2 * i]) | ((uint32_t)f32_to_bf16_bits(acc[2 * i + 1]) << 16));
-    *(i32x4_t*)((uint16_t*)a.out + o0) = o;
+    store_streaming((i32x4_t*)((uint16_t*)a.out + o0), o);
   } else {
     const f32x4_t o = {acc[0], acc[1], acc[2], acc[3]};
-    *(f32x4_t*)((float*)a.out + o0) = o;
+    store_streaming((f32x4_t*)((float*)a.out + o0), o);
   }
 }
 
