@@ -283,6 +283,7 @@ struct DwconvArgs {
 };
 hipError_t dwconv2d_launch(const DwconvArgs& a, hipStream_t s);
 bool dwconv2d_takes_paired_filter(const pml_hip_dwconv2d_desc& d);
+bool dwconv2d_walks_rows(const pml_hip_dwconv2d_desc& d, int n_cus, int64_t* ysegs, int64_t* seg_rows);
 bool dwconv2d_pair_filter(const uint16_t* filter, int64_t c, uint32_t* packed);
 struct Im2colArgs {
   const void* in;

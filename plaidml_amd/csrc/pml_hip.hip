@@ -1219,6 +1219,11 @@ int64_t pml_hip_dwconv2d_dispatch(const pml_hip_dwconv2d_desc* d) {
                 d->dtype == PML_HIP_F32 ? "f32" : "bf16", (long long)d->n, (long long)d->h, (long long)d->w,
                 (long long)d->c, (long long)d->kh, (long long)d->kw, (long long)d->oh, (long long)d->ow);
   p->text = buf;
+  int64_t ysegs, seg_rows;
+  if (dwconv2d_walks_rows(*d, device_cus(), &ysegs, &seg_rows)) {
+    std::snprintf(buf, sizeof buf, ", window rows walked in registers (%lld runs of %lld rows)", (long long)ysegs, (long long)seg_rows);
+    p->text += buf;
+  }
   return (int64_t)(intptr_t)p;
 }
 

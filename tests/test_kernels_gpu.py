@@ -839,6 +839,61 @@ def test_dwconv_shapes(kind, N, H, W, C, k, stride, pad, packed):
     hk.lib().pml_hip_plan_free(plan)
 
 
+# (dtype, N, H, W, C, pad, with an infinite weight): 3x3 unit-stride cases with enough threads for the kernel that walks
+# down the image with the window rows in registers -- runs of rows with a ragged last one, an odd width (the last
+# pixel pair is half empty), SAME, VALID and a wider padding, lanes with an infinite weight next to lanes without
+DW_WALK_CASES = [('bf16', 16, 19, 19, 728, 1, True), ('bf16', 16, 19, 19, 728, 1, False), ('bf16', 64, 12, 40, 256, 0, False),
+                 ('f32', 24, 20, 21, 512, 2, True), ('f32', 12, 33, 18, 512, 1, False)]
+
+
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('kind,N,H,W,C,pad,with_inf', DW_WALK_CASES)
+def test_dwconv_rows_walked_in_registers(kind, N, H, W, C, pad, with_inf, packed):
+    rng = np.random.default_rng(92)
+    Iv = rng.standard_normal((N, H, W, C)).astype(np.float32)
+    Fv = (rng.standard_normal((3, 3, C, 1)) * 0.3).astype(np.float32)
+    if with_inf:
+        Fv[0, 0, 0, 0] = np.inf   # a corner tap: padded for the first row and column only
+        Fv[2, 1, C - 1, 0] = -np.inf
+    if kind == 'bf16':
+        Iv, Fv = E.round_bf16(Iv), E.round_bf16(Fv)
+    OH, OW = H + 2 * pad - 2, W + 2 * pad - 2
+    es = 2 if kind == 'bf16' else 4
+    outs = []
+    for pitch in (0, C + 2 * (16 // es)):
+        d = hk.Dwconv2dDesc()
+        d.dtype = hk.BF16 if kind == 'bf16' else hk.F32
+        d.out_pitch = pitch
+        d.n, d.h, d.w, d.c, d.kh, d.kw, d.oh, d.ow = N, H, W, C, 3, 3, OH, OW
+        d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
+        d.pad_h = d.pad_w = pad
+        plan = hk.lib().pml_hip_dwconv2d_dispatch(ctypes.byref(d))
+        assert plan, hk.lib().pml_hip_last_error()
+        assert 'window rows walked in registers' in hk.describe(plan)
+        dI = hk.DeviceBuffer.from_numpy(bf16(Iv) if kind == 'bf16' else Iv)
+        dF = hk.DeviceBuffer.from_numpy(bf16(Fv) if kind == 'bf16' else Fv)
+        width = pitch or C
+        dO = hk.DeviceBuffer(N * OH * OW * width * es)
+        dO.fill_u32(0x12341234)
+        if packed:
+            hk.check(hk.lib().pml_hip_dwconv2d_pack_filter(plan, dF.ptr, None))
+        hk.check(hk.lib().pml_hip_dwconv2d_invoke(plan, dI.ptr, None if packed else dF.ptr, dO.ptr, hk.ptr_array([]), hk.ptr_array([]), None))
+        hk.check(hk.lib().pml_hip_stream_sync(None))
+        outs.append(dO.to_numpy(np.uint16 if es == 2 else np.uint32, (N * OH * OW, width)))
+        hk.lib().pml_hip_plan_free(plan)
+    dense, pitched = outs
+    # the pitched result: the same bits, the bytes between a pixel's channels and the next pixel left alone
+    np.testing.assert_array_equal(pitched[:, :C], dense)
+    assert (pitched[:, C:] == (0x1234 if es == 2 else 0x12341234)).all()
+    out = E.bf16_from_bits(dense.reshape(N, OH, OW, C)) if es == 2 else dense.view(np.float32).reshape(N, OH, OW, C)
+    dt = D.BFLOAT16 if kind == 'bf16' else D.FLOAT32
+    I, F = E.Placeholder(dt, Iv.shape), E.Placeholder(dt, Fv.shape)
+    O = op.convolution(I, F, strides=[1, 1], autopad=op.EXPLICIT, manual_padding=[pad, pad], depthwise=True)
+    ref, = E.run(E.Program('dw', [I, F], [O]), [Iv, Fv])
+    assert np.isinf(ref).any() == with_inf and not np.isnan(ref).any()
+    np.testing.assert_allclose(out, ref, rtol=BF16_RTOL if kind == 'bf16' else FP32_RTOL, atol=1e-2 if kind == 'bf16' else 1e-4)
+
+
 @pytest.mark.parametrize('kind,N,H,W,C,k,stride,pad', DW_CASES[:3] + DW_CASES[4:])
 def test_dwconv_output_pitch(kind, N, H, W, C, k, stride, pad):
     """With an output pitch the same values land `pitch` elements apart, bit for bit, and the bytes between a
