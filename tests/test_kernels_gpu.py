@@ -779,6 +779,29 @@ def test_conv_few_channel_stride2(kind, shape, k, co, pad, capsys):
         assert 'row by row with the filter in registers' in text
 
 
+# Runs of four and more output rows per workgroup take the row-walking kernel's eight-wavefront form (a pixel's 128
+# bytes then come from two wavefronts, through LDS, one row late): ragged last runs, a second pixel block that is half
+# empty with two idle wavefront pairs, four pixel blocks with a ragged last one.  The first case against the oracle;
+# the larger ones, which the oracle would take minutes over, against the implicit-GEMM path of the same library
+# (itself held to the oracle by the cases above).
+@pytest.mark.parametrize('shape,pad,against_oracle', [((256, 14, 34, 3), None, True), ((96, 62, 70, 3), 3, False),
+                                                      ((128, 26, 250, 3), 3, False)])
+def test_conv_stem_long_runs(shape, pad, against_oracle, capsys):
+    if against_oracle:
+        _stem_case('bf16', shape, 7, 64, 2, pad, 47)
+        assert 'row by row with the filter in registers' in capsys.readouterr().out
+        return
+    Iv, Fv = _conv_case('bf16', shape, 7, 7, 64, op.SAME_UPPER, 47)
+    bias = E.round_bf16(np.random.default_rng(48).standard_normal(64).astype(np.float32))
+    outs = []
+    for flags in (0, hk.flag_conv(hk.CONV_IGEMM)):
+        outs.append(E.bf16_from_bits(run_conv(bf16(Iv), bf16(Fv), hk.BF16, hk.BF16, stride=2, pad=pad, bias=bf16(bias), relu=True,
+                                              flags=flags)))
+    text = capsys.readouterr().out
+    assert text.count('row by row with the filter in registers') == 1
+    np.testing.assert_allclose(outs[0], outs[1], rtol=BF16_RTOL, atol=1e-2)
+
+
 @pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
 @pytest.mark.parametrize('stride', [1, 2])
 def test_conv_few_channel_patch_matrix(kind, stride, capsys, monkeypatch):
