@@ -1442,9 +1442,11 @@ hipError_t conv_blocks4x4_launch(const IgemmArgs& a, size_t lds, int n_cus, hipS
   per_image = per_image < 1 ? 1 : (per_image > a.OH ? a.OH : per_image);
   const int rows = (a.OH + per_image - 1) / per_image;
   per_image = (a.OH + rows - 1) / rows;
-  // Runs of at least four rows take the eight-wavefront form (128 x 224 x 224 x 3: 76 us against 98-104 on one device);
-  // below that -- one image -- a workgroup is all prologue, and the smaller one starts faster (12.4 against 13.6 us).
-  if (rows >= 4) {
+  // Runs of two rows and more take the eight-wavefront form (128 x 224 x 224 x 3: 76 us against 98-104 on one device; 8 and
+  // 12 images, runs of two and three rows: 14.4 against 15.2 and 16.6 against 17.5).  One row per workgroup -- up to four
+  // images -- is all prologue; there the two forms are within a microsecond of each other, the smaller one ahead as the
+  // first kernel of a network (12.4 against 13.6 us), the larger one in a loop of its own (7.4 against 8.0).
+  if (rows >= 2) {
     const size_t lds8 = (size_t)kBlkRing * (a.OW + 3) * kBlkPixBytes + 64 * 4 + 8 * 4096;
     static DynamicLdsLimit limit8;
     if (hipError_t e = limit8.ensure((const void*)conv_blocks4x4_w8_kernel, lds8); e != hipSuccess) return e;

@@ -779,7 +779,7 @@ def test_conv_few_channel_stride2(kind, shape, k, co, pad, capsys):
         assert 'row by row with the filter in registers' in text
 
 
-# Runs of four and more output rows per workgroup take the row-walking kernel's eight-wavefront form (a pixel's 128
+# Runs of two and more output rows per workgroup take the row-walking kernel's eight-wavefront form (a pixel's 128
 # bytes then come from two wavefronts, through LDS, one row late): ragged last runs, a second pixel block that is half
 # empty with two idle wavefront pairs, four pixel blocks with a ragged last one.  The first case against the oracle;
 # the larger ones, which the oracle would take minutes over, against the implicit-GEMM path of the same library
