@@ -186,7 +186,15 @@ enum {
  *   bits 8..15  PML_HIP_FLAG_TILE(t): the output tile of the MFMA kernel, t one of PML_HIP_TILE_*
  *   bits 16..19 PML_HIP_FLAG_CONV(c): the convolution path, c one of PML_HIP_CONV_* (ignored by gemm)
  * A tile the element kind is not built for falls back to the nearest one that is; a convolution path the shape
- * does not qualify for is ignored. */
+ * does not qualify for is ignored.
+ *   bits 20..24 PML_HIP_FLAG_MAXPOOL3x3S2(pt, pb, pl, pr) (conv2d only): a 3x3 stride-2 max-pool with 0 or 1 rows /
+ *               columns of padding on each side runs over the convolution's result inside the launch, and `output`
+ *               is the pooled tensor [n][(oh + pt + pb - 3) / 2 + 1][(ow + pl + pr - 3) / 2 + 1][co] -- bit for bit
+ *               what pml_hip_pool2d (max) makes of the convolution's own output.  oh / ow stay the convolution's.
+ *               Only where pml_hip_conv2d_takes_maxpool says so (the row-walking kernel of a few-channel stride-2
+ *               bf16 convolution onto 64 channels with a plain tail: an image network's head); dispatch fails
+ *               elsewhere.  Counterpart of the reference's producer / consumer fusion of such nests
+ *               (pmlc/target/x86/pipeline.cc:304-322). */
 enum {
   PML_HIP_TILE_64x64 = 0,      /* 4 wavefronts */
   PML_HIP_TILE_128x64,         /* 4 wavefronts of 64x32 */
@@ -213,6 +221,9 @@ enum {
 #define PML_HIP_FLAG_CONV(c) (((c) & 0xf) << 16)
 #define PML_HIP_FLAG_TILE_OF(flags) ((((flags) >> 8) & 0xff) - 1) /* -1: none */
 #define PML_HIP_FLAG_CONV_OF(flags) (((flags) >> 16) & 0xf)
+#define PML_HIP_FLAG_MAXPOOL3x3S2(pt, pb, pl, pr) \
+  ((1 << 20) | (((pt) & 1) << 21) | (((pb) & 1) << 22) | (((pl) & 1) << 23) | (((pr) & 1) << 24))
+#define PML_HIP_FLAG_MAXPOOL_OF(flags) (((flags) >> 20) & 0x1f) /* 0: none; bit 0 set: fused, bits 1..4 = pt, pb, pl, pr */
 /* Name of a tile as the plan dump and the `hip{tile=...}` target option spell it ("128x128w8s2"), NULL when out of range;
  * and the inverse (-1 for an unknown name).  Host arithmetic only. */
 const char* pml_hip_tile_name(int tile);
@@ -357,6 +368,9 @@ typedef struct {
 } pml_hip_conv2d_desc;
 
 int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* desc);
+/* 1 when a descriptor carrying PML_HIP_FLAG_MAXPOOL3x3S2 would be accepted by pml_hip_conv2d_dispatch (host arithmetic
+ * only: a planner asks before it folds a pooling step into the convolution in front of it). */
+int pml_hip_conv2d_takes_maxpool(const pml_hip_conv2d_desc* desc);
 int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, void* output, const void* init,
                           const void* const* operands, void* const* outs, pml_hip_stream s);
 /* Same as pml_hip_gemm_pack_b for a constant filter: afterwards invoke may be given filter == NULL. */

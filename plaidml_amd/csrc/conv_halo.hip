@@ -1310,19 +1310,37 @@ __global__ __launch_bounds__(256, 2) void conv_blocks4x4_kernel(IgemmArgs p, int
 // A pixel's 128 bytes now come from two wavefronts: a finished row is staged in LDS (one 4 KB area per pixel block,
 // two sets taking turns by row parity) and goes to memory at the start of the next step, after the step's barrier,
 // every wavefront storing 16 pixels of its pixel block as whole 128-byte lines.
+// POOL: the rows are not stored; the last four stay in LDS (the staging areas, taking turns by row number) and a 3x3
+// stride-2 max-pool over them leaves instead (p.pool_*): rows_per_wg then counts pooled rows, and a workgroup computes
+// the convolution rows its pooled rows cover (one more than twice as many: neighbouring workgroups both compute the row
+// between them).  The values pooled are the stored bf16 values and the comparisons those of pool_flat_kernel, so the
+// result is, bit for bit, that of the two launches.
+template <bool POOL>
 __global__ __launch_bounds__(512, 4) void conv_blocks4x4_w8_kernel(IgemmArgs p, int rows_per_wg, int wgs_per_image) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), h = lane >> 5;
   const int pb = wave & 3, j = wave >> 2;
   const int n = (int)blockIdx.x / wgs_per_image, blk = (int)blockIdx.x % wgs_per_image;
-  const int oy0 = blk * rows_per_wg;
-  const int oy1 = oy0 + rows_per_wg < p.OH ? oy0 + rows_per_wg : p.OH;
+  int oy0 = blk * rows_per_wg;
+  int oy1 = oy0 + rows_per_wg < p.OH ? oy0 + rows_per_wg : p.OH;
+  int py0 = 0, py1 = 0;  // POOL: the workgroup's pooled rows
+  if (POOL) {
+    py0 = blk * rows_per_wg;
+    py1 = py0 + rows_per_wg < p.pool_oh ? py0 + rows_per_wg : p.pool_oh;
+    oy0 = 2 * py0 - p.pool_pt < 0 ? 0 : 2 * py0 - p.pool_pt;
+    oy1 = 2 * (py1 - 1) - p.pool_pt + 3 < p.OH ? 2 * (py1 - 1) - p.pool_pt + 3 : p.OH;
+    if (py0 >= py1) return;
+  }
   if (oy0 >= oy1) return;
   const int Wp = p.OW + 3;                      // pixel slots of an LDS row: source columns -PW .. OW + 2 - PW
   const int row_bytes = Wp * kBlkPixBytes;
   const int n_chunks = Wp * 2;                  // 16-byte chunks of a row (at most one per thread: OW <= 128)
   float* const bias = (float*)(smem + kBlkRing * row_bytes);
-  unsigned char* const staging = smem + kBlkRing * row_bytes + 256;  // 2 sets x 4 pixel blocks x 4 KB
+  // staged result rows: two sets of four pixel blocks of 4 KB; POOL: four sets of OW pixels of 128 bytes (a row being
+  // staged then never takes the place of one of the three a pooled row may still be reading)
+  unsigned char* const staging = smem + kBlkRing * row_bytes + 256;
+  constexpr int kSets = POOL ? 4 : 2;
+  const int set_bytes = POOL ? p.OW * 128 : 4 * 4096;
 
   // the filter of the wavefront's 32 channels: MFMA row i holds output channel 32j + 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3)
   i32x4_t breg[16];
@@ -1360,7 +1378,7 @@ __global__ __launch_bounds__(512, 4) void conv_blocks4x4_w8_kernel(IgemmArgs p, 
   const float lo = p.tail_relu ? 0.f : -__builtin_inff();
   // the staged row oy leaves for memory: the wavefront's 16 pixels of its pixel block, eight lanes per pixel
   auto store_row = [&](int oy) {
-    const unsigned char* const stage = staging + ((oy & 1) * 4 + pb) * 4096;
+    const unsigned char* const stage = staging + (oy % kSets) * set_bytes + pb * 4096;
     const int chunk = lane & 7;
     unsigned char* const out_row = (unsigned char*)p.C + (((int64_t)n * p.OH + oy) * p.OW + pb * 32) * p.ldc * 2 + chunk * 16;
 #pragma unroll
@@ -1370,15 +1388,92 @@ __global__ __launch_bounds__(512, 4) void conv_blocks4x4_w8_kernel(IgemmArgs p, 
       if (pb * 32 + px < p.OW) *(u32x4_t*)(out_row + (int64_t)px * p.ldc * 2) = v;
     }
   };
+  // POOL: pooled row py out of the staged rows 2 py - pool_pt .. + 2 (those that exist): a thread per pooled pixel and
+  // 16-byte chunk of channels, taps in rising window index, a tap replacing the running value when it is greater (a NaN
+  // never is).  Behind a ReLU the staged values are +0 and above, or -infinity where the convolution gave NaN (see the
+  // staging below): bf16 values of that kind compare like the 16-bit integers they are, two per instruction.
+  // (a thread's three window columns are the same for every pooled row: their offsets inside a staged row, once)
+  int pool_col[3] = {0, 0, 0};
+  if (POOL) {
+    const int ppx = tid >> 3, chunk = tid & 7;
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx) {
+      int c = 2 * ppx - p.pool_pl + kx;
+      c = c < 0 ? 0 : (c > p.OW - 1 ? p.OW - 1 : c);
+      const int px = c & 31;
+      pool_col[kx] = c * 128 + ((chunk ^ (px & 7)) << 4);
+    }
+  }
+  auto pool_row = [&](int py) {
+    const int ppx = tid >> 3, chunk = tid & 7;
+    if (ppx >= p.pool_ow) return;
+    typedef short i16x2_t __attribute__((ext_vector_type(2)));
+    auto max_i16x2 = [](unsigned a, unsigned b) {
+      return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(i16x2_t, a), __builtin_bit_cast(i16x2_t, b)));
+    };
+    float best[8];
+    unsigned best2[4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) best[e] = -__builtin_inff();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) best2[q] = 0xff80ff80u;  // -infinity twice
+    // A tap outside the image is replaced by the nearest one inside, which belongs to the same window: the maximum is
+    // the same and no lane branches.  A window row's three reads are under way together (all nine would not fit the
+    // registers beside the filter).
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+      int r = 2 * py - p.pool_pt + ky;
+      r = r < 0 ? 0 : (r > p.OH - 1 ? p.OH - 1 : r);
+      u32x4_t v[3];
+      const unsigned char* const row = staging + (r % kSets) * set_bytes;
+#pragma unroll
+      for (int kx = 0; kx < 3; ++kx) v[kx] = *(const u32x4_t*)(row + pool_col[kx]);
+      if (p.tail_relu) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) best2[q] = max_i16x2(best2[q], v[k][q]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float lo_half = __uint_as_float(v[k][q] << 16), hi_half = __uint_as_float(v[k][q] & 0xffff0000u);
+            best[2 * q] = lo_half > best[2 * q] ? lo_half : best[2 * q];
+            best[2 * q + 1] = hi_half > best[2 * q + 1] ? hi_half : best[2 * q + 1];
+          }
+      }
+    }
+    u32x4_t o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      o[q] = p.tail_relu ? best2[q] : (__float_as_uint(best[2 * q]) >> 16) | (__float_as_uint(best[2 * q + 1]) & 0xffff0000u);
+    *(u32x4_t*)((unsigned char*)p.C + ((((int64_t)n * p.pool_oh + py) * p.pool_ow + ppx) * p.ldc + chunk * 8) * 2) = o;
+  };
+  // the pooled rows whose last existing window row is `oy` (at most two: a whole window, and one cut off by the image's
+  // end); true if there was one
+  auto pool_after = [&](int oy) {
+    bool any = false;
+    for (int py = py0; py < py1; ++py) {
+      const int last = 2 * py - p.pool_pt + 2 < p.OH - 1 ? 2 * py - p.pool_pt + 2 : p.OH - 1;
+      if (last != oy) continue;
+      pool_row(py);
+      any = true;
+    }
+    return any;
+  };
   // Two fetches are in flight: the row the next step needs (`due`) and the row the step after that needs (`later`).
   auto step = [&](int oy, i32x4_t& due, i32x4_t& later) {
     const bool more = oy + 1 < oy1;
     if (oy + 2 < oy1) later = fetch_row(oy + 5 - p.PH);
-    if (oy > oy0) store_row(oy - 1);
-    if (pb * 32 < p.OW) {
+    if (!POOL && oy > oy0) store_row(oy - 1);
+    // POOL: the pooled rows that row oy - 1 completed go first, at every wavefront's own pace beside the others' MFMAs
+    if (POOL && oy > oy0) pool_after(oy - 1);
+    const bool active = pb * 32 < p.OW;  // (a row of at most 96 pixels leaves pixel blocks, and their wavefronts, without work)
+    f32x16_t acc;
+    if (active) {
       const int ox = pb * 32 + (lane & 31);
       const int oxc = ox < p.OW ? ox : p.OW - 1;  // lanes past the row's end multiply its last pixel; their values are staged and never stored
-      f32x16_t acc;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const f32x4_t v = *(const f32x4_t*)(bias + 32 * j + 16 * h + 4 * q);
@@ -1391,10 +1486,13 @@ __global__ __launch_bounds__(512, 4) void conv_blocks4x4_w8_kernel(IgemmArgs p, 
 #pragma unroll
         for (int tx = 0; tx < 4; ++tx) mma_block<KIND_BF16>(acc, breg[ty * 4 + tx], *(const i32x4_t*)(base + tx * kBlkPixBytes));
       }
+    }
+    if (active) {
       // the lane's 16 channels 32 j + 16 h .. of pixel lane % 32: two 16-byte chunks of the pixel's 128 bytes, at positions
       // XORed with the pixel number
-      unsigned char* const stage = staging + ((oy & 1) * 4 + pb) * 4096;
+      unsigned char* const stage = staging + (oy % kSets) * set_bytes + pb * 4096;
       const int px = lane & 31;
+      const bool staged = !POOL || pb * 32 + px < p.OW;  // (POOL: a set ends with the row's last pixel)
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         unsigned w[4];
@@ -1403,12 +1501,16 @@ __global__ __launch_bounds__(512, 4) void conv_blocks4x4_w8_kernel(IgemmArgs p, 
           float v0 = acc[8 * half + 2 * k], v1 = acc[8 * half + 2 * k + 1];
           v0 = relu_clamp(v0, lo);
           v1 = relu_clamp(v1, lo);
+          if (POOL && p.tail_relu) {  // a NaN is never the maximum of a window: it is staged as the value every other one beats
+            v0 = v0 != v0 ? -__builtin_inff() : v0;
+            v1 = v1 != v1 ? -__builtin_inff() : v1;
+          }
           const f32x2_t pair = {v0, v1};
           const bf16x2_t hh = __builtin_convertvector(pair, bf16x2_t);
           __builtin_memcpy(&w[k], &hh, 4);
         }
         const int chunk = 4 * j + 2 * h + half;  // channels 32 j + 16 h + 8 half .. + 7
-        *(u32x4_t*)(stage + px * 128 + ((chunk ^ (px & 7)) << 4)) = u32x4_t{w[0], w[1], w[2], w[3]};
+        if (staged) *(u32x4_t*)(stage + px * 128 + ((chunk ^ (px & 7)) << 4)) = u32x4_t{w[0], w[1], w[2], w[3]};
       }
     }
     if (more) put_row((oy + 4) % kBlkRing, due);  // the slot of row oy - 1, which nothing reads any more
@@ -1420,7 +1522,8 @@ __global__ __launch_bounds__(512, 4) void conv_blocks4x4_w8_kernel(IgemmArgs p, 
     step(oy, ra, rb);
     if (oy + 1 < oy1) step(oy + 1, rb, ra);
   }
-  store_row(oy1 - 1);
+  if (!POOL) store_row(oy1 - 1);
+  if (POOL) pool_after(oy1 - 1);
 }
 
 }  // namespace
@@ -1437,20 +1540,23 @@ size_t conv_blocks4x4_prepare(int kind, const IgemmArgs& a) {
 }
 
 hipError_t conv_blocks4x4_launch(const IgemmArgs& a, size_t lds, int n_cus, hipStream_t s) {
-  // two workgroups per CU, each a run of consecutive output rows of one image
+  // two workgroups per CU, each a run of consecutive output rows (with a fused pool: pooled rows) of one image
+  const int out_rows = a.pool ? a.pool_oh : a.OH;
   int per_image = (2 * n_cus + a.NB - 1) / a.NB;
-  per_image = per_image < 1 ? 1 : (per_image > a.OH ? a.OH : per_image);
-  const int rows = (a.OH + per_image - 1) / per_image;
-  per_image = (a.OH + rows - 1) / rows;
+  per_image = per_image < 1 ? 1 : (per_image > out_rows ? out_rows : per_image);
+  const int rows = (out_rows + per_image - 1) / per_image;
+  per_image = (out_rows + rows - 1) / rows;
   // Runs of two rows and more take the eight-wavefront form (128 x 224 x 224 x 3: 76 us against 98-104 on one device; 8 and
   // 12 images, runs of two and three rows: 14.4 against 15.2 and 16.6 against 17.5).  One row per workgroup -- up to four
   // images -- is all prologue; there the two forms are within a microsecond of each other, the smaller one ahead as the
-  // first kernel of a network (12.4 against 13.6 us), the larger one in a loop of its own (7.4 against 8.0).
-  if (rows >= 2) {
-    const size_t lds8 = (size_t)kBlkRing * (a.OW + 3) * kBlkPixBytes + 64 * 4 + 8 * 4096;
-    static DynamicLdsLimit limit8;
-    if (hipError_t e = limit8.ensure((const void*)conv_blocks4x4_w8_kernel, lds8); e != hipSuccess) return e;
-    hipLaunchKernelGGL(conv_blocks4x4_w8_kernel, dim3((unsigned)(a.NB * per_image)), dim3(512), lds8, s, a, rows, per_image);
+  // first kernel of a network (12.4 against 13.6 us), the larger one in a loop of its own (7.4 against 8.0).  The fused
+  // pool exists in the eight-wavefront form only.
+  if (rows >= 2 || a.pool) {
+    const size_t lds8 = (size_t)kBlkRing * (a.OW + 3) * kBlkPixBytes + 64 * 4 + (a.pool ? (size_t)4 * a.OW * 128 : (size_t)8 * 4096);
+    auto kern = a.pool ? conv_blocks4x4_w8_kernel<true> : conv_blocks4x4_w8_kernel<false>;
+    static DynamicLdsLimit limit8[2];
+    if (hipError_t e = limit8[a.pool ? 1 : 0].ensure((const void*)kern, lds8); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(a.NB * per_image)), dim3(512), lds8, s, a, rows, per_image);
     return hipGetLastError();
   }
   static DynamicLdsLimit limit;

@@ -197,6 +197,10 @@ struct IgemmArgs {
   int g2_stride, g2_h, g2_w, g2_ohw, g2_ow;
   unsigned g2_ohw_magic, g2_ow_magic;
   int g2_ohw_shift, g2_ow_shift;
+  // conv_blocks4x4_w8_kernel only: pool = 1 applies a 3x3 stride-2 max-pool to the convolution's rows before they leave the
+  // chip -- C is then the pooled tensor [NB][pool_oh][pool_ow][N], pooled pixel (y, x) covering result rows 2y - pool_pt ..
+  // + 2 and columns 2x - pool_pl .. + 2 as far as they exist
+  int pool, pool_oh, pool_ow, pool_pt, pool_pl;
 };
 
 hipError_t igemm_launch(int kind, int cfg, bool conv, const IgemmArgs& a, hipStream_t s);

@@ -114,6 +114,7 @@ const char* tile_name(int t) {
 }
 
 constexpr int kScheduleBits = 0xff << 8 | 0xf << 16;
+constexpr int kMaxpoolBits = 0x1f << 20;
 bool schedule_bits_ok(int flags) {
   return PML_HIP_FLAG_TILE_OF(flags) < PML_HIP_TILE_COUNT_ && PML_HIP_FLAG_CONV_OF(flags) <= PML_HIP_CONV_BLOCKS;
 }
@@ -438,6 +439,13 @@ void conv_args(const Plan* p, IgemmArgs& g) {
   g.halo_variant = p->halo_variant;
   fast_div_magic((unsigned)(d.oh * d.ow), &g.div_per_magic, &g.div_per_shift);
   fast_div_magic((unsigned)d.ow, &g.div_ow_magic, &g.div_ow_shift);
+  if (const int mp = PML_HIP_FLAG_MAXPOOL_OF(d.flags)) {
+    g.pool = 1;
+    g.pool_pt = (mp >> 1) & 1;
+    g.pool_pl = (mp >> 3) & 1;
+    g.pool_oh = (int)((d.oh + ((mp >> 1) & 1) + ((mp >> 2) & 1) - 3) / 2 + 1);
+    g.pool_ow = (int)((d.ow + ((mp >> 3) & 1) + ((mp >> 4) & 1) - 3) / 2 + 1);
+  }
   if (p->via_s2d) {
     // unit-stride convolution over the re-blocked input: one "tap" per block row, whose K-run covers
     // s2d_kaw neighbouring blocks of s2d_ch channels
@@ -880,6 +888,20 @@ int pml_hip_gemm_run_static(const pml_hip_gemm_desc* d, const void* a, const voi
 // conv2d
 // ---------------------------------------------------------------------------
 
+// A plan (its descriptor, element kind and 2x2-block geometry filled in) whose convolution the row-walking kernel takes,
+// with a result the fused 3x3 stride-2 max-pool can walk: a pooled row per thread group of 512 threads, eight per pixel.
+static bool conv2d_takes_maxpool(const Plan* p) {
+  const pml_hip_conv2d_desc& d = p->conv;
+  const int path = PML_HIP_FLAG_CONV_OF(d.flags);
+  if (!p->via_s2d || path == PML_HIP_CONV_IGEMM || path == PML_HIP_CONV_PATCHES) return false;
+  IgemmArgs g;
+  conv_args(p, g);
+  // (the filter pointer's alignment is the allocator's: not part of the question)
+  g.Bt = nullptr;
+  if (!conv_blocks4x4_prepare(p->mfma_kind, g)) return false;
+  return d.oh >= 3 && d.ow >= 3 && g.pool_oh >= 1 && g.pool_ow >= 1 && g.pool_ow <= 64 && d.tail.n_operands == 0;
+}
+
 int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
   if (!d) {
     fail("null descriptor");
@@ -896,8 +918,8 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     fail("conv2d: out_dtype does not fit in_dtype");
     return 0;
   }
-  if ((d->flags & ~(PML_HIP_FP32_AS_BF16X3 | kScheduleBits)) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32) ||
-      !schedule_bits_ok(d->flags)) {
+  if ((d->flags & ~(PML_HIP_FP32_AS_BF16X3 | kScheduleBits | kMaxpoolBits)) != 0 || ((d->flags & PML_HIP_FP32_AS_BF16X3) && d->in_dtype != PML_HIP_F32) ||
+      !schedule_bits_ok(d->flags) || (PML_HIP_FLAG_MAXPOOL_OF(d->flags) != 0 && (PML_HIP_FLAG_MAXPOOL_OF(d->flags) & 1) == 0)) {
     fail("conv2d: flags may only hold PML_HIP_FP32_AS_BF16X3 (with in_dtype F32) and schedule overrides that name an existing tile and path");
     return 0;
   }
@@ -996,7 +1018,42 @@ int64_t pml_hip_conv2d_dispatch(const pml_hip_conv2d_desc* d) {
     conv_args(p, g);
     if (path != PML_HIP_CONV_IGEMM && conv_blocks4x4_prepare(kind, g)) p->text += ", row by row with the filter in registers";
   }
+  if (PML_HIP_FLAG_MAXPOOL_OF(d->flags)) {
+    if (!conv2d_takes_maxpool(p)) {
+      delete p;
+      fail("conv2d: the fused max-pool needs the row-walking kernel (see pml_hip_conv2d_takes_maxpool) and a convolution result of at least 3 x 3 and at most 128 pixels a row");
+      return 0;
+    }
+    IgemmArgs g;
+    conv_args(p, g);
+    p->text += " + max-pool 3x3 stride 2 -> " + std::to_string(g.pool_oh) + "x" + std::to_string(g.pool_ow);
+  }
   return (int64_t)(intptr_t)p;
+}
+
+int pml_hip_conv2d_takes_maxpool(const pml_hip_conv2d_desc* d) {
+  if (!d || !PML_HIP_FLAG_MAXPOOL_OF(d->flags)) return 0;
+  const int kind = mfma_kind_of(d->in_dtype, d->flags);
+  if (kind != KIND_BF16 || d->n <= 0 || d->h <= 0 || d->w <= 0 || d->ci <= 0 || d->co <= 0 || d->kh <= 0 || d->kw <= 0 || d->oh <= 0 ||
+      d->ow <= 0 || !valid_tail(d->tail))
+    return 0;
+  // the plan's fields that conv_args reads, without any of its allocations
+  Plan p;
+  p.kind = PLAN_CONV;
+  p.mfma_kind = kind;
+  p.conv = *d;
+  const int es = 2, v = 8;
+  const bool via_s2d = (d->ci * es) % 16 != 0 && d->stride_h == 2 && d->stride_w == 2 && d->dil_h == 1 && d->dil_w == 1 && d->ci <= 16 &&
+                       PML_HIP_FLAG_CONV_OF(d->flags) != PML_HIP_CONV_PATCHES;
+  if (!via_s2d) return 0;
+  p.s2d_h = (int)(d->h + 1) / 2;
+  p.s2d_w = (int)(d->w + 1) / 2;
+  p.s2d_ch = (int)(4 * d->ci + v - 1) / v * v;
+  p.s2d_ka = (int)(d->kh + (d->pad_h & 1) + 1) / 2;
+  p.s2d_kaw = (int)(d->kw + (d->pad_w & 1) + 1) / 2;
+  p.bt_ld = (int64_t)p.s2d_ka * p.s2d_kaw * p.s2d_ch;
+  p.via_s2d = true;
+  return conv2d_takes_maxpool(&p) ? 1 : 0;
 }
 
 int pml_hip_conv2d_invoke(int64_t plan, const void* input, const void* filter, void* output, const void* init,

@@ -29,6 +29,12 @@ def flag_conv(path):
     """The descriptor bits that name a convolution path (CONV_*)."""
     return path << 16
 
+
+def flag_maxpool3x3s2(pad_top, pad_bottom, pad_left, pad_right):
+    """The conv2d descriptor bits that ask for a 3x3 stride-2 max-pool over the convolution's result inside the launch
+    (padding 0 or 1 per side; PML_HIP_FLAG_MAXPOOL3x3S2)."""
+    return (1 << 20) | (pad_top & 1) << 21 | (pad_bottom & 1) << 22 | (pad_left & 1) << 23 | (pad_right & 1) << 24
+
 AGG_ASSIGN, AGG_ADD, AGG_MAX, AGG_MIN, AGG_MUL = 0, 1, 2, 3, 4
 COMBO_NONE, COMBO_ADD, COMBO_COND, COMBO_EQ, COMBO_MUL = 0, 1, 2, 3, 4
 (EPI_ADD, EPI_SUB, EPI_RSUB, EPI_MUL, EPI_DIV, EPI_RDIV, EPI_MAX, EPI_MIN, EPI_RELU, EPI_NEG, EPI_EXP, EPI_LOG,
@@ -48,7 +54,7 @@ EXPORTS = [
     'pml_hip_conv2d_dispatch', 'pml_hip_conv2d_invoke', 'pml_hip_dwconv2d_dispatch', 'pml_hip_dwconv2d_invoke',
     'pml_hip_pool2d_dispatch', 'pml_hip_pool2d_invoke', 'pml_hip_eltwise_dispatch', 'pml_hip_eltwise_invoke',
     'pml_hip_select', 'pml_hip_softmax', 'pml_hip_index', 'pml_hip_contract_dispatch', 'pml_hip_contract_invoke', 'pml_hip_plan_free',
-    'pml_hip_plan_describe', 'pml_hip_struct_size', 'pml_hip_gemm_pack_b', 'pml_hip_conv2d_pack_filter',
+    'pml_hip_plan_describe', 'pml_hip_struct_size', 'pml_hip_gemm_pack_b', 'pml_hip_conv2d_pack_filter', 'pml_hip_conv2d_takes_maxpool',
     'pml_hip_gather', 'pml_hip_scatter', 'pml_hip_argsort', 'pml_hip_prng',
 ]
 
@@ -198,6 +204,8 @@ def lib():
         L.pml_hip_argsort.argtypes = [ctypes.POINTER(ArgsortDesc), vp, vp, vp]
         L.pml_hip_prng.argtypes = [vp, ctypes.c_int64, vp, vp, vp]
         L.pml_hip_conv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
+        L.pml_hip_conv2d_takes_maxpool.argtypes = [vp]
+        L.pml_hip_conv2d_takes_maxpool.restype = ctypes.c_int
         L.pml_hip_dwconv2d_pack_filter.argtypes = [ctypes.c_int64, vp, vp]
         _lib = L
     return _lib

@@ -49,6 +49,7 @@ std::shared_ptr<Plan> Planner::run() {
   }
   if (opt_.fuse && opt_.specialise) fuseSecondProducts();
   if (opt_.specialise) padDepthwiseResults();
+  if (opt_.fuse && opt_.specialise) fusePoolIntoConv();
   pruneDeadSteps();
   applySchedule();
   return plan_;
@@ -109,6 +110,12 @@ void Planner::applySchedule() {
     }
     if (s.kind == Step::Gemm) r.conv = 0;
     int32_t& flags = s.kind == Step::Gemm ? s.gemm.flags : s.conv.flags;
+    if (r.conv > 0 && s.kind == Step::Conv2d && PML_HIP_FLAG_MAXPOOL_OF(flags)) {
+      // (a convolution that pools its result inside the launch keeps the path that can)
+      pml_hip_conv2d_desc probe = s.conv;
+      probe.flags |= PML_HIP_FLAG_CONV(r.conv);
+      if (!pml_hip_conv2d_takes_maxpool(&probe)) r.conv = 0;
+    }
     std::string text;
     if (r.tile >= 0) {
       flags |= PML_HIP_FLAG_TILE(r.tile);

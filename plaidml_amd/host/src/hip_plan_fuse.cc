@@ -177,6 +177,55 @@ void Planner::padDepthwiseResults() {
   }
 }
 
+// A 3x3 stride-2 max-pool that is the only reader of a convolution's result, where the kernel library's convolution can
+// pool its rows before they leave the chip (pml_hip_conv2d_takes_maxpool: the few-channel stride-2 head of an image
+// network): the pooling step goes, the convolution writes the pooled tensor, and the full-size result -- 205 MB at
+// 128 x 112 x 112 x 64 -- is neither written nor read.  The reference fuses such producer / consumer nests in its own
+// way (pmlc/target/x86/pipeline.cc:304-322).  Not under a program-wide convolution path (`hip{conv=...}`).
+void Planner::fusePoolIntoConv() {
+  if (!opt_.conv.empty()) return;
+  for (size_t x = 0; x < plan_->steps.size(); ++x) {
+    Step& X = plan_->steps[x];
+    if (X.kind != Step::Conv2d || X.c < 0 || X.c_off != 0 || !X.outs.empty() || X.out2 >= 0) continue;
+    if (plan_->buffers[X.c].kind != BufferInfo::Temp || PML_HIP_FLAG_MAXPOOL_OF(X.conv.flags)) continue;
+    int readers = 0, writers = 0, y = -1;
+    for (size_t k = 0; k < plan_->steps.size(); ++k) {
+      const Step& s = plan_->steps[k];
+      for (int r : {s.a, s.b, s.init, s.a2, s.b2, s.init2}) readers += r == X.c;
+      for (int r : s.operands) readers += r == X.c;
+      writers += s.c == X.c;
+      writers += s.out2 == X.c;
+      for (int w : s.outs) writers += w == X.c;
+      if (s.a == X.c && k > x) y = static_cast<int>(k);
+    }
+    if (readers != 1 || writers != 1 || y < 0) continue;
+    const Step& Y = plan_->steps[y];
+    const pml_hip_pool2d_desc& q = Y.pool;
+    if (Y.kind != Step::Pool2d || Y.a_off != 0 || Y.c < 0 || Y.out2 >= 0 || !Y.outs.empty() || !Y.operands.empty()) continue;
+    if (q.agg != PML_HIP_AGG_MAX || q.with_index || q.divisor != 0.f || q.kh != 3 || q.kw != 3 || q.stride_h != 2 || q.stride_w != 2 ||
+        q.dtype != PML_HIP_BF16 || q.pad_h < 0 || q.pad_h > 1 || q.pad_w < 0 || q.pad_w > 1)
+      continue;
+    if (q.n != X.conv.n || q.h != X.conv.oh || q.w != X.conv.ow || q.c != X.conv.co) continue;
+    // the padding behind is whatever makes the pooled size come out (taps past the image's end are left out either way)
+    int pb = -1, pr = -1;
+    for (int e = 1; e >= 0; --e) {
+      if ((q.h + q.pad_h + e - 3) / 2 + 1 == q.oh && q.h + q.pad_h + e >= 3) pb = e;
+      if ((q.w + q.pad_w + e - 3) / 2 + 1 == q.ow && q.w + q.pad_w + e >= 3) pr = e;
+    }
+    if (pb < 0 || pr < 0) continue;
+    pml_hip_conv2d_desc probe = X.conv;
+    probe.flags |= PML_HIP_FLAG_MAXPOOL3x3S2(static_cast<int>(q.pad_h), pb, static_cast<int>(q.pad_w), pr);
+    if (!pml_hip_conv2d_takes_maxpool(&probe)) continue;
+    X.conv = probe;
+    X.c = Y.c;
+    X.c_off = Y.c_off;
+    const auto arrow = X.text.rfind(" -> ");
+    X.text = (arrow == std::string::npos ? X.text : X.text.substr(0, arrow)) + " + max-pool 3x3 stride 2" + Y.text.substr(Y.text.rfind(" -> "));
+    X.bytes += Y.bytes - 2.0 * static_cast<double>(q.n * q.h * q.w * q.c) * 2.0;
+    plan_->steps.erase(plan_->steps.begin() + y);
+  }
+}
+
 // A kernel that took over the work of earlier operations (the int8 GEMM reads the un-cast operands, a pool
 // kernel also writes the window argmax) can leave launches whose results nobody reads: drop them.
 void Planner::pruneDeadSteps() {

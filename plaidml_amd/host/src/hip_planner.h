@@ -160,6 +160,7 @@ class Planner {
   void applySchedule();
   void fuseSecondProducts();
   void padDepthwiseResults();
+  void fusePoolIntoConv();
   void pruneDeadSteps();
 
  private:

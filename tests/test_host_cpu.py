@@ -129,6 +129,29 @@ def test_mean_over_the_image_is_one_launch():
     assert 'hip plan: 2 launches' in t, t
 
 
+def test_stem_convolution_pools_inside_its_launch():
+    """relu(conv 7x7x3 stride 2 + b) followed by a 3x3 stride-2 max-pool that alone reads it: the pooling step goes and
+    the convolution writes the pooled tensor (the kernel library is asked first).  Not when the convolution's result is
+    also a program output, not with a window argmax beside the pool, not under `fuse=0` or a program-wide `conv=`."""
+    bf = E.DType.BFLOAT16
+    def program(also_output=False):
+        X = E.Placeholder(bf, [2, 64, 64, 3])
+        F = E.Constant(np.zeros((7, 7, 3, 64), np.float32), bf)
+        B = E.Constant(np.zeros(64, np.float32), bf)
+        C = op.relu(op.convolution(X, F, strides=[2, 2], autopad=op.SAME_UPPER) + B)
+        M = op.pool(C, 'max', [3, 3], [2, 2], autopad=op.SAME_UPPER)
+        return E.Program('stem', [X], [M, C] if also_output else [M])
+    t = plan_of(program())
+    assert 'hip plan: 1 launches' in t and '+ max-pool 3x3 stride 2 -> 2x16x16x64xbf16' in t, t
+    t = plan_of(program(also_output=True))
+    assert 'hip plan: 2 launches' in t and 'max-pool 3x3 stride 2' not in t, t
+    for target in ('hip{fuse=0}', 'hip{conv=igemm}'):
+        prog = program()
+        prog.compile(target)
+        t = dict(prog.passes)['hip-plan']
+        assert 'max-pool 3x3 stride 2' not in t and 'pool2d max' in t, t
+
+
 def test_projection_shortcut_and_main_path_share_one_launch():
     """relu(conv1x1(y) + b + conv1x1(x) + b') of a residual block with a projection shortcut is one GEMM with two
     products (plain rows, or the pixel rows of the stride-2 shortcut); `fuse=0` keeps the contractions apart."""

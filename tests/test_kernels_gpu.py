@@ -802,6 +802,99 @@ def test_conv_stem_long_runs(shape, pad, against_oracle, capsys):
     np.testing.assert_allclose(outs[0], outs[1], rtol=BF16_RTOL, atol=1e-2)
 
 
+# The stem convolution with its 3x3 stride-2 max-pool inside the launch (PML_HIP_FLAG_MAXPOOL3x3S2) against the same
+# convolution followed by pml_hip_pool2d, bit for bit.  (shape, conv pad, pool pads top / bottom / left / right): the
+# network shape in small (SAME_UPPER pooling of an even side: one row and column of padding behind), padding in front,
+# on both sides and none, odd sides, a last window cut off by the image's end, rows of more than one pixel block with a
+# ragged last block, many images (several pooled rows per workgroup) and one (a pooled row per workgroup)
+MAXPOOL_CASES = [((8, 64, 64, 3), 3, (0, 1, 0, 1)), ((3, 30, 34, 3), None, (1, 1, 1, 1)), ((2, 31, 29, 3), 3, (1, 0, 1, 0)),
+                 ((5, 40, 140, 3), 3, (0, 0, 0, 0)), ((160, 24, 70, 3), 3, (0, 1, 1, 1)), ((1, 64, 200, 3), 3, (0, 1, 0, 1)),
+                 ((2, 14, 16, 3), 3, (1, 1, 0, 0))]
+
+
+@pytest.mark.parametrize('shape,pad,pp', MAXPOOL_CASES)
+def test_conv_stem_with_maxpool_inside(shape, pad, pp):
+    L = hk.lib()
+    Iv, Fv = _conv_case('bf16', shape, 7, 7, 64, op.SAME_UPPER, 51)
+    bias = bf16(E.round_bf16(np.random.default_rng(52).standard_normal(64).astype(np.float32)))
+    N, H, W, CI = shape
+    # infinities of both signs in the image: convolution results that are +infinity, and NaN (which no window may pick;
+    # a window of nothing but NaN pools to -infinity)
+    Iv = Iv.copy()
+    Iv[0, H // 2, W // 2, :] = np.inf
+    Iv[0, H // 2 + 1, W // 2 + 1, 0] = -np.inf
+    Iv[N - 1, 2:12, 2:12, 1] = np.inf
+    Iv[N - 1, 3:11, 3:11, 2] = -np.inf
+    ph, OH = op.compute_padding_and_output_size(H, 7, 2, op.SAME_UPPER)
+    pw, OW = op.compute_padding_and_output_size(W, 7, 2, op.SAME_UPPER)
+    if pad is not None:
+        ph = pw = pad
+        OH, OW = (H + 2 * pad - 7) // 2 + 1, (W + 2 * pad - 7) // 2 + 1
+    pt, pb, pl, pr = pp
+    POH, POW = (OH + pt + pb - 3) // 2 + 1, (OW + pl + pr - 3) // 2 + 1
+
+    def conv_desc(flags):
+        d = hk.Conv2dDesc()
+        d.in_dtype = d.out_dtype = d.c_dtype = hk.BF16
+        d.flags = flags
+        d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = N, H, W, CI, 7, 7, 64, OH, OW
+        d.stride_h = d.stride_w = 2
+        d.dil_h = d.dil_w = 1
+        d.pad_h, d.pad_w = ph, pw
+        d.init_kind, d.init_dtype = 1, hk.BF16
+        d.init_row_stride, d.init_col_stride = 0, 1
+        d.tail = hk.make_tail(ops=[(hk.EPI_RELU, hk.BF16, 0, 0, 0.0)])
+        return d
+    dI, dF, dB = hk.DeviceBuffer.from_numpy(bf16(Iv)), hk.DeviceBuffer.from_numpy(bf16(Fv)), hk.DeviceBuffer.from_numpy(bias)
+    none = hk.ptr_array([])
+    # the two launches
+    d = conv_desc(0)
+    plan = L.pml_hip_conv2d_dispatch(ctypes.byref(d))
+    assert plan, L.pml_hip_last_error()
+    dC = hk.DeviceBuffer(N * OH * OW * 64 * 2)
+    hk.check(L.pml_hip_conv2d_invoke(plan, dI.ptr, dF.ptr, dC.ptr, dB.ptr, none, none, None))
+    q = hk.Pool2dDesc()
+    q.dtype, q.agg = hk.BF16, hk.AGG_MAX
+    q.n, q.h, q.w, q.c, q.kh, q.kw, q.oh, q.ow = N, OH, OW, 64, 3, 3, POH, POW
+    q.stride_h = q.stride_w = 2
+    q.pad_h, q.pad_w = pt, pl
+    plan2 = L.pml_hip_pool2d_dispatch(ctypes.byref(q))
+    assert plan2, L.pml_hip_last_error()
+    dP = hk.DeviceBuffer(N * POH * POW * 64 * 2)
+    hk.check(L.pml_hip_pool2d_invoke(plan2, dC.ptr, dP.ptr, None, None))
+    hk.check(L.pml_hip_stream_sync(None))
+    apart = dP.to_numpy(np.uint16, (N, POH, POW, 64))
+    # one launch
+    f = conv_desc(hk.flag_maxpool3x3s2(pt, pb, pl, pr))
+    assert L.pml_hip_conv2d_takes_maxpool(ctypes.byref(f)) == 1
+    plan3 = L.pml_hip_conv2d_dispatch(ctypes.byref(f))
+    assert plan3, L.pml_hip_last_error()
+    assert 'max-pool 3x3 stride 2 -> %dx%d' % (POH, POW) in hk.describe(plan3)
+    dQ = hk.DeviceBuffer(N * POH * POW * 64 * 2)
+    dQ.fill_u32(0x7fc07fc0)
+    hk.check(L.pml_hip_conv2d_invoke(plan3, dI.ptr, dF.ptr, dQ.ptr, dB.ptr, none, none, None))
+    hk.check(L.pml_hip_stream_sync(None))
+    fused = dQ.to_numpy(np.uint16, (N, POH, POW, 64))
+    np.testing.assert_array_equal(fused, apart)
+    assert not np.isnan(E.bf16_from_bits(fused)).any()
+    for pl_ in (plan, plan2, plan3):
+        L.pml_hip_plan_free(pl_)
+
+
+def test_conv_maxpool_inside_is_refused_elsewhere():
+    """Only the row-walking stem kernel has the pool: other convolutions refuse the flag at dispatch, and say so."""
+    L = hk.lib()
+    d = hk.Conv2dDesc()
+    d.in_dtype = d.out_dtype = d.c_dtype = hk.BF16
+    d.flags = hk.flag_maxpool3x3s2(0, 1, 0, 1)
+    d.n, d.h, d.w, d.ci, d.kh, d.kw, d.co, d.oh, d.ow = 2, 16, 16, 64, 3, 3, 64, 16, 16
+    d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
+    d.pad_h = d.pad_w = 1
+    assert L.pml_hip_conv2d_takes_maxpool(ctypes.byref(d)) == 0
+    assert L.pml_hip_conv2d_dispatch(ctypes.byref(d)) == 0
+    assert 'fused max-pool' in L.pml_hip_last_error().decode()
+
+
 @pytest.mark.parametrize('kind', ['f32', 'bf16', 'f32x3'])
 @pytest.mark.parametrize('stride', [1, 2])
 def test_conv_few_channel_patch_matrix(kind, stride, capsys, monkeypatch):
